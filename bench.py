@@ -1,0 +1,216 @@
+#!/usr/bin/env python3
+"""Benchmark of the batch-1 fused trellis decode + mat-vec on one MI355X.
+
+One step = one call of decompress_matvec_16_8_1 (hashed-codebook stream, 2 bits/weight, 16-bit
+window) on the Llama-2-7B down-projection shape m=4096, n=11008, batch 1, through the C ABI.
+Steps rotate over distinct weight copies (default 32 x 11.27 MB > the 256 MB Infinity Cache) so
+every launch streams its weights from HBM.  The metric is GB/s of compressed weight bytes.
+
+The line printed at the end also carries
+  roofline      compressed bytes per launch / average launch duration (HIP events on the launch
+                stream over the timed region) against the 8 TB/s HBM peak;
+  cpu_baseline  the CPU oracle's fused decode+mat-vec (the checker, timed here only as a
+                baseline) on the host cores of the same box.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for p in (ROOT, os.path.join(ROOT, "let-it-slide_amd")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+HBM_PEAK_GBS = 8000.0
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=1000)
+    ap.add_argument("--warmup", type=int, default=100)
+    ap.add_argument("--copies", type=int, default=32, help="distinct weight copies to rotate over")
+    ap.add_argument("--m", type=int, default=4096)
+    ap.add_argument("--n", type=int, default=11008)
+    ap.add_argument("--S", type=int, default=8, choices=(6, 8))
+    ap.add_argument("--launch", choices=("graph", "direct"), default="graph",
+                    help="graph: the timed steps are one captured HIP graph; direct: one host call per step")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--extra-shapes", action="store_true", help="also time the other layer shapes")
+    return ap.parse_args()
+
+
+class Runner:
+    """Launches the op through the C ABI with pre-bound arguments (no timing, asynchronous)."""
+
+    def __init__(self, m, n, S, copies, seed=42):
+        import torch
+        import rptc_kernels
+        self.torch = torch
+        self.m, self.n, self.S = m, n, S
+        self.lib = rptc_kernels.library()
+        rc = self.lib.rptc_init()
+        if rc:
+            raise RuntimeError(self.lib.rptc_status_string(rc).decode())
+        self.fn = getattr(self.lib, f"rptc_decompress_matvec_16_{S}_1")
+        g = torch.Generator(device="cuda")
+        g.manual_seed(seed)
+        words = m * n // 16
+        self.weights = [torch.randint(-(1 << 31), 1 << 31, (words,), generator=g, dtype=torch.int64,
+                                      device="cuda").to(torch.int32) for _ in range(copies)]
+        self.codebook = torch.randn(2 << S, generator=g, device="cuda").to(torch.float16)
+        self.x = torch.randn(n, generator=g, device="cuda").to(torch.float16)
+        self.out = torch.zeros(m, dtype=torch.float16, device="cuda")
+        self.bytes = m * n * 2 // 8
+        torch.cuda.synchronize()
+
+    def launch(self, k, stream):
+        w = self.weights[k % len(self.weights)]
+        rc = self.fn(w.data_ptr(), self.codebook.data_ptr(), self.x.data_ptr(), self.out.data_ptr(),
+                     self.m, self.n, 0, ctypes.c_void_p(stream), None)
+        if rc:
+            raise RuntimeError(self.lib.rptc_status_string(rc).decode())
+
+    def run(self, steps, warmup, mode):
+        """Returns (wall seconds, event milliseconds) for exactly `steps` launches."""
+        torch = self.torch
+        stream = torch.cuda.current_stream()
+        for k in range(warmup):
+            self.launch(k, stream.cuda_stream)
+        torch.cuda.synchronize()
+        ev0 = torch.cuda.Event(enable_timing=True)
+        ev1 = torch.cuda.Event(enable_timing=True)
+        if mode == "graph":
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                cs = torch.cuda.current_stream().cuda_stream
+                for k in range(steps):
+                    self.launch(k, cs)
+            graph.replay()                      # untimed: first replay uploads the graph
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            ev0.record()
+            graph.replay()
+            ev1.record()
+            torch.cuda.synchronize()
+            t1 = time.perf_counter()
+        else:
+            t0 = time.perf_counter()
+            ev0.record()
+            for k in range(steps):
+                self.launch(k, stream.cuda_stream)
+            ev1.record()
+            torch.cuda.synchronize()
+            t1 = time.perf_counter()
+        return t1 - t0, ev0.elapsed_time(ev1)
+
+    def check(self):
+        """Guard against timing a kernel that computes nothing: the output must equal the dense
+        product of the exported matrix (full parity lives in tests/)."""
+        torch = self.torch
+        import rptc_kernels
+        W = torch.zeros((self.m, self.n), dtype=torch.float16, device="cuda")
+        rptc_kernels.matvec_dense(self.weights[0], self.codebook, W, self.S)
+        self.launch(0, torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        want = W.double() @ self.x.double()
+        err = ((self.out.double() - want).norm() / want.norm()).item()
+        if not err < 1e-3:
+            raise RuntimeError(f"kernel output is wrong: rel-L2 {err}")
+        return err
+
+
+def cpu_baseline(runner, min_seconds=8.0):
+    """The oracle's fused decode + mat-vec (fp32 accumulate, threads over rows) on the same
+    layer, repeated until it has run for min_seconds."""
+    import numpy as np
+    from oracle import rptc_oracle
+    comp = runner.weights[0].cpu().numpy().view(np.uint32)
+    cb = runner.codebook.cpu().numpy()
+    x = runner.x.cpu().numpy()
+    threads = rptc_oracle.num_threads()
+    rptc_oracle.matvec_f32(comp, cb, x, runner.m, runner.S)           # warm the caches and the thread pool
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        rptc_oracle.matvec_f32(comp, cb, x, runner.m, runner.S)
+        reps += 1
+        dt = time.perf_counter() - t0
+        if dt >= min_seconds and reps >= 3:
+            break
+    gbs = runner.bytes * reps / dt / 1e9
+    return {"value": round(gbs, 4), "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": f"{reps} full passes of the same {runner.m}x{runner.n} layer, {dt:.1f} s of CPU work",
+            "ms_per_pass": round(dt / reps * 1e3, 3)}
+
+
+def main():
+    a = parse()
+    if a.gpus != 1:
+        print("bench.py: this build runs on one GPU; --gpus must be 1 (no multi-GPU path exists)", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    torch.cuda.set_device(0)
+    runner = Runner(a.m, a.n, a.S, a.copies)
+    err = runner.check()
+    wall, ev_ms = runner.run(a.steps, a.warmup, a.launch)
+    ms_per_step = wall * 1e3 / a.steps
+    launch_ms = ev_ms / a.steps
+    value = runner.bytes / (ms_per_step * 1e-3) / 1e9
+    achieved = runner.bytes / (launch_ms * 1e-3) / 1e9
+    line = {
+        "metric": "fused decode+GEMV GB/s (compressed)",
+        "value": round(value, 2),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": a.steps,
+        "warmup": a.warmup,
+        "ms_per_step": round(ms_per_step, 6),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {
+            "workload": f"decompress_matvec_16_{a.S}_1 m={a.m} n={a.n} 2 bits/weight batch 1 "
+                        f"(Llama-2-7B down_proj shape), {a.copies} rotating weight copies (cold cache)",
+            "launch": a.launch,
+            "accumulate": "f32",
+            "carry_mode": "as_written",
+            "compressed_bytes": runner.bytes,
+            "rel_l2_vs_dense": float(f"{err:.3e}"),
+        },
+        "roofline": {
+            "bound": "hbm",
+            "achieved": round(achieved, 2),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBS, 4),
+            "traffic": None,
+            "launch_us": round(launch_ms * 1e3, 3),
+        },
+    }
+    if a.extra_shapes:
+        extra = {}
+        for (m, n) in ((4096, 4096), (11008, 4096), (8192, 8192), (28672, 8192), (8192, 28672)):
+            r = Runner(m, n, a.S, max(2, min(a.copies, (512 << 20) // (m * n // 4) + 1)))
+            r.check()
+            _, ms = r.run(a.steps, a.warmup, a.launch)
+            us = ms / a.steps * 1e3
+            extra[f"{m}x{n}"] = {"launch_us": round(us, 3), "GBps": round(r.bytes / us / 1e3, 1),
+                                 "frac": round(r.bytes / us / 1e3 / HBM_PEAK_GBS, 4)}
+            del r
+            torch.cuda.empty_cache()
+        line["other_shapes"] = extra
+    if not a.no_cpu:
+        line["cpu_baseline"] = cpu_baseline(runner)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,128 @@
+/*
+ * rptc_hip.h -- C ABI of librptc_hip.so: gfx950 (MI355X) kernels for the trellis-coded
+ * linear layer's inference path.
+ *
+ * Every entry point takes plain device pointers and sizes, launches on the HIP stream the
+ * caller passes (NULL = the legacy default stream), allocates no device memory, keeps no
+ * reference to the caller's buffers and returns a status instead of exiting:
+ *     0   success
+ *   < 0   an RPTC_E* argument error (nothing was launched)
+ *   > 0   a hipError_t reported by the runtime
+ * rptc_status_string() turns either into text.  When `ms` is not NULL the call brackets its
+ * kernels with two events on `stream`, waits for the second and stores the elapsed
+ * milliseconds (the reference ops return this figure: wrapper.cpp:4-56); when it is NULL the
+ * call is asynchronous.
+ *
+ * fp16 values travel as uint16_t bit patterns.  `carry_mode` selects how a decoder treats the
+ * places where the reference CUDA source departs from one unbroken shift register per row
+ * (rptc.py:74-85): RPTC_AS_WRITTEN reproduces the CUDA arithmetic, RPTC_CONTINUOUS the
+ * unbroken register.
+ *
+ * Reference paths below are relative to rptc_kernels/csrc/rptc_kernels/ in the reference tree.
+ */
+#ifndef RPTC_HIP_H
+#define RPTC_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define RPTC_AS_WRITTEN 0
+#define RPTC_CONTINUOUS 1
+
+#define RPTC_OK 0
+#define RPTC_ENULL (-1)      /* a required pointer is NULL */
+#define RPTC_ESHAPE (-2)     /* a size breaks the op's shape rule */
+#define RPTC_EALIGN (-3)     /* a pointer is not 16-byte aligned */
+#define RPTC_EMODE (-4)      /* carry_mode is not one of the two modes */
+#define RPTC_ELIMIT (-5)     /* a size exceeds what the kernel's LDS staging can hold */
+#define RPTC_EDEVICE (-6)    /* the current device is not gfx950 */
+
+/* Library version, major*10000 + minor*100 + patch. */
+int rptc_version(void);
+
+/* Text for a status returned by any entry point (static storage, never NULL). */
+const char *rptc_status_string(int status);
+
+/*
+ * Optional.  Prepares the calling thread's current device (queries its properties, creates the
+ * two timing events, raises the kernels' dynamic-LDS limits) so that the first op call does not
+ * pay for it.  Every op does the same lazily.  Returns RPTC_EDEVICE on anything but gfx950.
+ */
+int rptc_init(void);
+
+/*
+ * Decode only.  Replaces `float decompress(Tensor& compressed, Tensor& codebook, Tensor& out)`
+ * (inference.cu:99-160, kernel inference.cu:42-96; bound at wrapper.cpp:60).
+ *   compressed  int32 [m][words_per_row], words_per_row % 128 == 0 (inference.cu:106)
+ *   codebook    fp16 [65536]                                      (inference.cu:116)
+ *   out         fp16 [m][16 * words_per_row], overwritten         (inference.cu:120-123)
+ */
+int rptc_decompress(const int32_t *compressed, const uint16_t *codebook, uint16_t *out,
+                    int64_t m, int64_t words_per_row, int carry_mode, void *stream, float *ms);
+
+/*
+ * Fused decode + mat-vec on the [slab][row][lane] stream with the hashed pair codebook.
+ * Replace `float decompress_matvec_{L}_{S}_1(Tensor& compressed, Tensor& codebook, Tensor& x,
+ * Tensor& out)` (inference.cu:280-380, kernel inference.cu:189-277; bound at
+ * wrapper.cpp:61-64).  L names the variant only: the reference kernel never reads it, every
+ * variant slides a 16-bit window.
+ *   compressed  int32, m*n/16 words: [n/2048][m][32][4]; when n % 2048 != 0 one more slab
+ *               [m][(n % 2048)/64][4] follows (an extension of this library; the reference
+ *               requires n % 2048 == 0, inference.cu:295-300)
+ *   codebook    fp16 [2^(S+1)]: 2^S pairs                         (inference.cu:303-305)
+ *   x           fp16 [n], n % 64 == 0
+ *   out         fp16 [m], overwritten.  The reference needs m % 32 == 0 (inference.cu:320);
+ *               any m >= 1 is accepted here.
+ * Products are accumulated in fp32 and rounded once (the reference accumulates in fp16).
+ */
+int rptc_decompress_matvec_16_6_1(const int32_t *compressed, const uint16_t *codebook,
+                                  const uint16_t *x, uint16_t *out, int64_t m, int64_t n,
+                                  int carry_mode, void *stream, float *ms);
+int rptc_decompress_matvec_20_6_1(const int32_t *compressed, const uint16_t *codebook,
+                                  const uint16_t *x, uint16_t *out, int64_t m, int64_t n,
+                                  int carry_mode, void *stream, float *ms);
+int rptc_decompress_matvec_16_8_1(const int32_t *compressed, const uint16_t *codebook,
+                                  const uint16_t *x, uint16_t *out, int64_t m, int64_t n,
+                                  int carry_mode, void *stream, float *ms);
+int rptc_decompress_matvec_20_8_1(const int32_t *compressed, const uint16_t *codebook,
+                                  const uint16_t *x, uint16_t *out, int64_t m, int64_t n,
+                                  int carry_mode, void *stream, float *ms);
+
+/*
+ * Fused decode + mat-vec on the column-interleaved stream with a scalar 2^L codebook.
+ * Replace `float decompress_matvec_t_{16,14}(Tensor& compressed, Tensor& codebook, Tensor& x,
+ * Tensor& out)` (inference_t.cu:178-268, kernel inference_t.cu:68-175; bound at
+ * wrapper.cpp:65-66).
+ *   compressed  int32, at least m*n/16 words, read as uint4 [n/64][m]   (inference_t.cu:116)
+ *   codebook    fp16 [2^L]                                              (inference_t.cu:206)
+ *   x           fp16 [n], n % 64 == 0, n <= 32768 (the reference's constant-memory bound,
+ *               inference_t.cu:49,216)
+ *   out         fp16 [m]; the product is ADDED to it                    (inference_t.cu:170-171)
+ */
+int rptc_decompress_matvec_t_16(const int32_t *compressed, const uint16_t *codebook,
+                                const uint16_t *x, uint16_t *out, int64_t m, int64_t n,
+                                int carry_mode, void *stream, float *ms);
+int rptc_decompress_matvec_t_14(const int32_t *compressed, const uint16_t *codebook,
+                                const uint16_t *x, uint16_t *out, int64_t m, int64_t n,
+                                int carry_mode, void *stream, float *ms);
+
+/*
+ * The dense fp16 matrix a stream stands for, W [m][n] row-major, so that decoded weights can be
+ * compared bit for bit.  No counterpart in the reference (its fused kernels never materialise
+ * W); the column each decoded pair lands in is fixed by the activation pairing of
+ * inference.cu:215-221,249 and inference_t.cu:141-146.
+ *   S in {6, 8};  L in {14, 16}.
+ */
+int rptc_matvec_dense(const int32_t *compressed, const uint16_t *codebook, uint16_t *W,
+                      int64_t m, int64_t n, int S, int carry_mode, void *stream, float *ms);
+int rptc_matvec_t_dense(const int32_t *compressed, const uint16_t *codebook, uint16_t *W,
+                        int64_t m, int64_t n, int L, int carry_mode, void *stream, float *ms);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* RPTC_HIP_H */

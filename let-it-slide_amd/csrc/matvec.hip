@@ -1,0 +1,345 @@
+// Fused decode + mat-vec on the [slab][row][lane] stream with the hashed pair codebook.
+//
+// Semantics: rptc_kernels/csrc/rptc_kernels/inference.cu:189-277 (kernel) and :280-356
+// (launcher) of the reference.  One stream element (16 bytes, one lane of one row of one slab)
+// is 32 steps; step s reads the 16-bit window that ends 4(s+1) bits into the element, hashes
+// it with h*(h+1), takes hash byte 1 as the codebook entry (bit 7 of that byte replaces the
+// sign of the pair's first value) and multiplies the pair with two activations.
+//
+// gfx950 design (not the reference's):
+//   * one workgroup of 16 waves per CU, each owning a block of rows and every slab of those
+//     rows, so the sum over slabs stays inside the workgroup and is added in a fixed order;
+//   * a half-wave (32 lanes) is one row of one slab, exactly one 512-byte line of the stream;
+//     a wave keeps a slab's 32 activation pairs per lane in registers and walks row pairs, so
+//     activations cost one LDS read per 2*R rows instead of one per step;
+//   * two adjacent windows come out of one v_alignbit_b32, both hashes out of one
+//     v_pk_mad_u16, the LDS address out of one v_and_or_b32 / v_perm_b32 (hash byte 1 is the
+//     row of a 256-entry table whose sign is already applied, replicated once per lane so the
+//     gather has no bank conflicts), and the pair product out of one v_dot2_f32_f16 with fp32
+//     accumulation: three vector ops per decoded pair;
+//   * every wave issues its stream loads before the table is built.
+#include "rptc_common.hpp"
+
+namespace rptc {
+
+constexpr int kMatvecThreads = 1024;
+constexpr int kMatvecWaves = kMatvecThreads / kWave;
+constexpr int kTableBytes = 256 * 256;     // 256 rows of 64 lane copies of one half2
+constexpr int kBatch = 4;                  // stream elements in flight per lane
+
+struct Geometry {
+    int m, n, T, Lt, slabs;
+    __host__ __device__ Geometry(int m_, int n_) : m(m_), n(n_), T(n_ >> 11), Lt((n_ & 2047) >> 6), slabs((n_ >> 11) + (((n_ & 2047) >> 6) ? 1 : 0)) {}
+    __host__ __device__ int lanes(int slab) const { return slab < T ? 32 : Lt; }
+    // index of the uint4 element (slab, row, lane)
+    __host__ __device__ size_t elem(int slab, int row, int lane) const
+    {
+        return slab < T ? ((size_t)slab * m + row) * 32 + lane
+                        : (size_t)T * m * 32 + (size_t)row * Lt + lane;
+    }
+    // half2 slot of step q = 4k + j of lane l (inference.cu:249 for the full slabs)
+    __host__ __device__ int slot(int slab, int q, int lane) const
+    {
+        return slab < T ? 1024 * slab + 32 * q + lane : 1024 * T + q * Lt + lane;
+    }
+};
+
+// The 256-row table: row b holds entry b & (2^S - 1) with sign bit b >> 7 in the first value.
+template <int S>
+__device__ __forceinline__ uint32_t table_value(const uint32_t *__restrict__ codebook, int b)
+{
+    const uint32_t pair = codebook[b & ((1 << S) - 1)];
+    return (pair & 0xFFFF7FFFu) | ((uint32_t)(b >> 7) << 15);
+}
+
+// One window register g = two windows 16 bits (4 steps) apart: hi half first in the stream.
+// lane4 = LDS address of the table + 4 * lane; the table starts on a 64 KiB boundary, so OR-ing
+// the row offset in equals adding it.
+__device__ __forceinline__ void two_steps(uint32_t g, uint32_t lane4, uint32_t x_hi, uint32_t x_lo,
+                                          float &acc_a, float &acc_b)
+{
+    const uint32_t h = pk_hash16(g);
+    const uint32_t a_lo = and_or(h, 0xFF00u, lane4);           // (byte 1 of h) << 8 | lane4
+    const uint32_t a_hi = perm(h, lane4, 0x0C0C0700u);         // (byte 3 of h) << 8 | lane4
+    acc_a = dot2(lds_read_abs(a_hi), x_hi, acc_a);
+    acc_b = dot2(lds_read_abs(a_lo), x_lo, acc_b);
+}
+
+// All 32 steps of one element.  xr[q], q = 4k + j, is the activation pair of step (k, j).
+__device__ __forceinline__ float decode_element(const uint4 e, const uint32_t carry, const uint32_t lane4,
+                                                const uint32_t (&xr)[32])
+{
+    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const uint32_t sh = 12 - 4 * j;
+        // {carry,x}: hi = step (k=7, j), lo = (k=0, j);  {x,y}: (4, j), (1, j);
+        // {y,z}: (5, j), (2, j);  {z,w}: (6, j), (3, j)        (inference.cu:237-250)
+        const uint32_t gc = j == 3 ? e.x : alignbit(carry, e.x, sh);
+        const uint32_t gx = j == 3 ? e.y : alignbit(e.x, e.y, sh);
+        const uint32_t gy = j == 3 ? e.z : alignbit(e.y, e.z, sh);
+        const uint32_t gz = j == 3 ? e.w : alignbit(e.z, e.w, sh);
+        two_steps(gc, lane4, xr[28 + j], xr[0 + j], a0, a1);
+        two_steps(gx, lane4, xr[16 + j], xr[4 + j], a2, a3);
+        two_steps(gy, lane4, xr[20 + j], xr[8 + j], a0, a1);
+        two_steps(gz, lane4, xr[24 + j], xr[12 + j], a2, a3);
+    }
+    return (a0 + a1) + (a2 + a3);
+}
+
+template <int S, int MODE>
+__global__ __launch_bounds__(kMatvecThreads) void matvec_kernel(
+    const uint4 *__restrict__ comp, const uint32_t *__restrict__ codebook,
+    const uint4 *__restrict__ x, uint16_t *__restrict__ out, int m, int n, int rows_per_block)
+{
+    extern __shared__ uint32_t lds[];
+    uint32_t *sx = lds + kTableBytes / 4;             // activation pairs, slot order
+    float *part = reinterpret_cast<float *>(sx + n / 2);   // [slab][row in block]
+
+    const Geometry g(m, n);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l = lane & 31, hw = lane >> 5;
+    // the table is the first thing in LDS; its address is 0 when the kernel has no static LDS
+    // (the low 32 bits of a flat pointer into LDS are the LDS address)
+    const uint32_t lane4 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds)) + lane * 4;
+    const int row0 = blockIdx.x * rows_per_block;
+    const int rows = min(rows_per_block, m - row0);
+    const int pairs = (rows + 1) >> 1;
+    const int items = g.slabs * pairs;                // item = slab * pairs + pair
+    const int per_wave = (items + kMatvecWaves - 1) / kMatvecWaves;
+    const int it_begin = wave * per_wave;
+    const int it_end = min(items, it_begin + per_wave);
+
+    uint4 buf[kBatch];
+    uint32_t cw[kBatch];
+    auto load_batch = [&](int base) {
+#pragma unroll
+        for (int u = 0; u < kBatch; u++) {
+            const int it = base + u;
+            buf[u] = make_uint4(0, 0, 0, 0);
+            cw[u] = 0;
+            if (it < it_end) {
+                const int slab = it / pairs, row = 2 * (it - slab * pairs) + hw;
+                if (row < rows && l < g.lanes(slab)) {
+                    buf[u] = comp[g.elem(slab, row0 + row, l)];
+                    if (MODE == RPTC_CONTINUOUS && l == 0 && slab > 0)
+                        cw[u] = comp[g.elem(slab - 1, row0 + row, 31)].w;
+                }
+            }
+        }
+    };
+    load_batch(it_begin);
+
+    // table and activations into LDS while the stream loads are in flight
+    for (int d = tid; d < kTableBytes / 4; d += kMatvecThreads) lds[d] = table_value<S>(codebook, d >> 6);
+    const int n8 = n >> 3;
+    for (int idx = tid; idx < n8; idx += kMatvecThreads) {
+        const uint4 v = x[idx];                       // halves 8idx .. 8idx+7 (inference.cu:215-221)
+        sx[idx] = v.x;
+        sx[idx + n8] = v.y;
+        sx[idx + 2 * n8] = v.z;
+        sx[idx + 3 * n8] = v.w;
+    }
+    __syncthreads();
+
+    uint32_t xr[32];
+    int cur_slab = -1;
+    for (int base = it_begin; base < it_end; base += kBatch) {
+        uint4 cur[kBatch];
+        uint32_t ccw[kBatch];
+#pragma unroll
+        for (int u = 0; u < kBatch; u++) {
+            cur[u] = buf[u];
+            ccw[u] = cw[u];
+        }
+        if (base + kBatch < it_end) load_batch(base + kBatch);
+#pragma unroll
+        for (int u = 0; u < kBatch; u++) {
+            const int it = base + u;
+            if (it >= it_end) break;
+            const int slab = it / pairs, pair = it - slab * pairs, row = 2 * pair + hw;
+            const bool active = row < rows && l < g.lanes(slab);
+            if (slab != cur_slab) {
+                cur_slab = slab;
+                const bool has = l < g.lanes(slab);
+#pragma unroll
+                for (int q = 0; q < 32; q++) xr[q] = has ? sx[g.slot(slab, q, l)] : 0u;
+            }
+            // previous lane's last word; lane 0 of a row keeps its own as written
+            // (inference.cu:232: the shuffle returns the caller's value to lane 0)
+            uint32_t carry = __shfl_up(cur[u].w, 1, 32);
+            if (MODE == RPTC_CONTINUOUS && l == 0) carry = ccw[u];
+            float acc = decode_element(cur[u], carry, lane4, xr);
+            acc = active ? acc : 0.f;
+            acc += __shfl_xor(acc, 16, 32);
+            acc += __shfl_xor(acc, 8, 32);
+            acc += __shfl_xor(acc, 4, 32);
+            acc += __shfl_xor(acc, 2, 32);
+            acc += __shfl_xor(acc, 1, 32);
+            if (l == 0 && row < rows) part[slab * rows_per_block + row] = acc;
+        }
+    }
+    __syncthreads();
+    for (int r = tid; r < rows; r += kMatvecThreads) {
+        float y = 0.f;
+        for (int t = 0; t < g.slabs; t++) y += part[t * rows_per_block + r];
+        out[row0 + r] = float_to_half_bits(y);
+    }
+}
+
+// Dense export: one thread per stream element, 32 pairs scattered to their columns.
+template <int S, int MODE>
+__global__ __launch_bounds__(256) void matvec_dense_kernel(
+    const uint4 *__restrict__ comp, const uint32_t *__restrict__ codebook, uint32_t *__restrict__ W,
+    int m, int n, int slab, int slab_elems)
+{
+    const Geometry g(m, n);
+    const int lanes = g.lanes(slab);
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= slab_elems) return;
+    const int row = i / lanes, l = i - row * lanes;
+    const uint4 e = comp[g.elem(slab, row, l)];
+    uint32_t carry;
+    if (l > 0) carry = comp[g.elem(slab, row, l - 1)].w;
+    else if (MODE == RPTC_AS_WRITTEN) carry = e.w;
+    else carry = slab > 0 ? comp[g.elem(slab - 1, row, 31)].w : 0u;
+    const uint32_t reg_c[8] = {e.x, e.y, e.z, e.w,
+                               alignbit(e.x, e.y, 16), alignbit(e.y, e.z, 16), alignbit(e.z, e.w, 16),
+                               alignbit(carry, e.x, 16)};
+    const int n8 = n >> 3;
+    uint32_t *wrow = W + (size_t)row * (n >> 1);
+#pragma unroll
+    for (int k = 0; k < 8; k++) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint32_t h = (reg_c[k] >> (12 - 4 * j)) & 0xFFFFu;
+            const uint32_t hash = h * (h + 1u);
+            const uint32_t pair = codebook[(hash >> 8) & ((1u << S) - 1u)];
+            const uint32_t val = (pair & 0xFFFF7FFFu) | (hash & 0x8000u);
+            const int P = g.slot(slab, 4 * k + j, l);
+            const int ii = P / n8, idx = P - ii * n8;
+            wrow[4 * idx + ii] = val;                 // halves 8idx + 2i, 8idx + 2i + 1
+        }
+    }
+}
+
+static int matvec_lds_bytes(int n, int slabs, int rows_per_block)
+{
+    return kTableBytes + 2 * n + 4 * slabs * rows_per_block;
+}
+
+template <int S>
+static int launch_matvec(const int32_t *compressed, const uint16_t *codebook, const uint16_t *x,
+                         uint16_t *out, int64_t m, int64_t n, int carry_mode, void *stream, float *ms)
+{
+    if (!compressed || !codebook || !x || !out) return RPTC_ENULL;
+    if (m < 1 || n < 64 || n % 64 != 0) return RPTC_ESHAPE;
+    if (carry_mode != RPTC_AS_WRITTEN && carry_mode != RPTC_CONTINUOUS) return RPTC_EMODE;
+    if (!aligned16(compressed) || !aligned16(codebook) || !aligned16(x)) return RPTC_EALIGN;
+    if (m >= (1 << 24) || n >= (1 << 20) || m * n >= ((int64_t)1 << 36)) return RPTC_ELIMIT;
+
+    DeviceInfo *dev;
+    int rc = device_info(&dev);
+    if (rc) return rc;
+    const Geometry g((int)m, (int)n);
+    int rows_per_block = 2 * (int)((m + 2 * dev->cus - 1) / (2 * dev->cus));
+    const int lds_bytes = matvec_lds_bytes((int)n, g.slabs, rows_per_block);
+    if (lds_bytes > kMaxLds) return RPTC_ELIMIT;
+    const int grid = (int)((m + rows_per_block - 1) / rows_per_block);
+
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    Timer t;
+    rc = t.begin(dev, s, ms);
+    if (rc) return rc;
+    auto a_comp = reinterpret_cast<const uint4 *>(compressed);
+    auto a_cb = reinterpret_cast<const uint32_t *>(codebook);
+    auto a_x = reinterpret_cast<const uint4 *>(x);
+    if (carry_mode == RPTC_AS_WRITTEN)
+        hipLaunchKernelGGL((matvec_kernel<S, RPTC_AS_WRITTEN>), dim3(grid), dim3(kMatvecThreads), lds_bytes, s,
+                           a_comp, a_cb, a_x, out, (int)m, (int)n, rows_per_block);
+    else
+        hipLaunchKernelGGL((matvec_kernel<S, RPTC_CONTINUOUS>), dim3(grid), dim3(kMatvecThreads), lds_bytes, s,
+                           a_comp, a_cb, a_x, out, (int)m, (int)n, rows_per_block);
+    return t.end();
+}
+
+template <int S, int MODE>
+static void launch_dense_slabs(const uint4 *comp, const uint32_t *cb, uint32_t *W, int m, int n, hipStream_t s)
+{
+    const Geometry g(m, n);
+    for (int slab = 0; slab < g.slabs; slab++) {
+        const int elems = m * g.lanes(slab);
+        hipLaunchKernelGGL((matvec_dense_kernel<S, MODE>), dim3((elems + 255) / 256), dim3(256), 0, s,
+                           comp, cb, W, m, n, slab, elems);
+    }
+}
+
+template <typename F>
+static int set_lds_limit(F *kernel)
+{
+    return (int)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds);
+}
+
+int prepare_matvec()
+{
+    int rc;
+    if ((rc = set_lds_limit(matvec_kernel<6, RPTC_AS_WRITTEN>))) return rc;
+    if ((rc = set_lds_limit(matvec_kernel<6, RPTC_CONTINUOUS>))) return rc;
+    if ((rc = set_lds_limit(matvec_kernel<8, RPTC_AS_WRITTEN>))) return rc;
+    if ((rc = set_lds_limit(matvec_kernel<8, RPTC_CONTINUOUS>))) return rc;
+    return 0;
+}
+
+}  // namespace rptc
+
+using namespace rptc;
+
+extern "C" int rptc_decompress_matvec_16_6_1(const int32_t *c, const uint16_t *cb, const uint16_t *x, uint16_t *out,
+                                             int64_t m, int64_t n, int mode, void *stream, float *ms)
+{
+    return launch_matvec<6>(c, cb, x, out, m, n, mode, stream, ms);
+}
+
+extern "C" int rptc_decompress_matvec_20_6_1(const int32_t *c, const uint16_t *cb, const uint16_t *x, uint16_t *out,
+                                             int64_t m, int64_t n, int mode, void *stream, float *ms)
+{
+    return launch_matvec<6>(c, cb, x, out, m, n, mode, stream, ms);
+}
+
+extern "C" int rptc_decompress_matvec_16_8_1(const int32_t *c, const uint16_t *cb, const uint16_t *x, uint16_t *out,
+                                             int64_t m, int64_t n, int mode, void *stream, float *ms)
+{
+    return launch_matvec<8>(c, cb, x, out, m, n, mode, stream, ms);
+}
+
+extern "C" int rptc_decompress_matvec_20_8_1(const int32_t *c, const uint16_t *cb, const uint16_t *x, uint16_t *out,
+                                             int64_t m, int64_t n, int mode, void *stream, float *ms)
+{
+    return launch_matvec<8>(c, cb, x, out, m, n, mode, stream, ms);
+}
+
+extern "C" int rptc_matvec_dense(const int32_t *compressed, const uint16_t *codebook, uint16_t *W, int64_t m,
+                                 int64_t n, int S, int carry_mode, void *stream, float *ms)
+{
+    if (!compressed || !codebook || !W) return RPTC_ENULL;
+    if (m < 1 || n < 64 || n % 64 != 0 || (S != 6 && S != 8)) return RPTC_ESHAPE;
+    if (carry_mode != RPTC_AS_WRITTEN && carry_mode != RPTC_CONTINUOUS) return RPTC_EMODE;
+    if (!aligned16(compressed) || !aligned16(codebook) || !aligned16(W)) return RPTC_EALIGN;
+    if (m >= (1 << 24) || n >= (1 << 20) || m * 32 >= ((int64_t)1 << 31)) return RPTC_ELIMIT;
+    DeviceInfo *dev;
+    int rc = device_info(&dev);
+    if (rc) return rc;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    Timer t;
+    rc = t.begin(dev, s, ms);
+    if (rc) return rc;
+    auto a_comp = reinterpret_cast<const uint4 *>(compressed);
+    auto a_cb = reinterpret_cast<const uint32_t *>(codebook);
+    auto a_w = reinterpret_cast<uint32_t *>(W);
+    const bool aw = carry_mode == RPTC_AS_WRITTEN;
+    if (S == 6 && aw) launch_dense_slabs<6, RPTC_AS_WRITTEN>(a_comp, a_cb, a_w, (int)m, (int)n, s);
+    else if (S == 6) launch_dense_slabs<6, RPTC_CONTINUOUS>(a_comp, a_cb, a_w, (int)m, (int)n, s);
+    else if (aw) launch_dense_slabs<8, RPTC_AS_WRITTEN>(a_comp, a_cb, a_w, (int)m, (int)n, s);
+    else launch_dense_slabs<8, RPTC_CONTINUOUS>(a_comp, a_cb, a_w, (int)m, (int)n, s);
+    return t.end();
+}

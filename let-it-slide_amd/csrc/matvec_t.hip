@@ -1,0 +1,231 @@
+// Fused decode + mat-vec on the column-interleaved stream with a scalar 2^L codebook.
+//
+// Semantics: rptc_kernels/csrc/rptc_kernels/inference_t.cu:68-175 (kernel) and :178-256
+// (launcher) of the reference.  The stream is uint4 c[col * m + row]: consecutive rows are
+// consecutive in memory, so a lane is a row (coalesced 16-byte loads), the activations are the
+// same for the whole wave and come through the scalar cache, and nothing crosses lanes.
+//
+// gfx950 design: the whole codebook (128 KiB at L = 16) sits in LDS; the reference's
+// one-thread-per-row loop is split over the 8 waves of a workgroup along the columns, which the
+// stream allows because the decoder state after an element depends only on that element
+// (as written: the top nibbles of its four words, inference_t.cu:131-142; continuous: its last
+// L bits), so a wave warms its state up from the element before its range.
+#include "rptc_common.hpp"
+
+namespace rptc {
+
+constexpr int kTThreads = 512;
+constexpr int kTWaves = kTThreads / kWave;
+
+template <int L>
+__device__ __forceinline__ uint32_t warm_state(const uint4 e, int mode)
+{
+    constexpr uint32_t mask = (1u << L) - 1u;
+    if (mode == RPTC_CONTINUOUS) return e.w & mask;
+    uint32_t c = 0;
+    c = mask & ((c << 4) | (e.x >> 28));
+    c = mask & ((c << 4) | (e.y >> 28));
+    c = mask & ((c << 4) | (e.z >> 28));
+    c = mask & ((c << 4) | (e.w >> 28));
+    return c;
+}
+
+template <int L, int MODE>
+__global__ __launch_bounds__(kTThreads) void matvec_t_kernel(
+    const uint4 *__restrict__ comp, const uint4 *__restrict__ codebook, const uint32_t *__restrict__ x,
+    uint16_t *__restrict__ out, int m, int cols)
+{
+    extern __shared__ uint4 lds_u4[];
+    constexpr int lut_u4 = (2 << L) / 16;
+    constexpr uint32_t mask = (1u << L) - 1u;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    for (int i = tid; i < lut_u4; i += kTThreads) lds_u4[i] = codebook[i];
+    __syncthreads();
+    const uint16_t *lut = reinterpret_cast<const uint16_t *>(lds_u4);
+    float *part = reinterpret_cast<float *>(lds_u4 + lut_u4);      // [wave][lane]
+
+    const int row = blockIdx.x * kWave + lane;
+    const bool valid = row < m;
+    const int per = (cols + kTWaves - 1) / kTWaves;
+    const int c0 = wave * per, c1 = min(cols, c0 + per);
+    const uint4 zero = make_uint4(0, 0, 0, 0);
+
+    uint32_t carry = 0;
+    if (c0 > 0 && c0 < c1 && valid) carry = warm_state<L>(comp[(size_t)(c0 - 1) * m + row], MODE);
+    float acc = 0.f;
+    uint4 next = (c0 < c1 && valid) ? comp[(size_t)c0 * m + row] : zero;
+    for (int col = c0; col < c1; col++) {
+        const uint4 e = next;
+        if (col + 1 < c1 && valid) next = comp[(size_t)(col + 1) * m + row];
+        const uint32_t words[4] = {e.x, e.y, e.z, e.w};
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const uint32_t word = words[k];
+            const uint32_t *xp = x + 32 * col + 8 * k;      // wave-uniform
+            if (MODE == RPTC_AS_WRITTEN) {
+                // all eight steps of a word see the carry the word started with
+                // (inference_t.cu:125-134), and the carry becomes the 4-bit-advanced state
+                const uint32_t s2 = mask & ((carry << 2) | (word >> 30));
+                const uint32_t s4 = mask & ((carry << 4) | (word >> 28));
+                carry = s4;
+                const uint32_t w = (uint32_t)lut[s2] | ((uint32_t)lut[s4] << 16);
+#pragma unroll
+                for (int j = 0; j < 8; j++) acc = dot2(w, xp[j], acc);
+            } else {
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    const uint32_t s2 = mask & alignbit(carry, word, 30 - 4 * j);
+                    const uint32_t s4 = mask & alignbit(carry, word, 28 - 4 * j);
+                    const uint32_t w = (uint32_t)lut[s2] | ((uint32_t)lut[s4] << 16);
+                    acc = dot2(w, xp[j], acc);
+                }
+                carry = word & mask;
+            }
+        }
+    }
+    part[wave * kWave + lane] = acc;
+    __syncthreads();
+    if (tid < kWave && valid) {
+        float y = 0.f;
+#pragma unroll
+        for (int w = 0; w < kTWaves; w++) y += part[w * kWave + tid];
+        // the product is added to what out holds (inference_t.cu:170-171)
+        out[row] = float_to_half_bits(half_bits_to_float(out[row]) + y);
+    }
+}
+
+// Dense export: one thread per stream element.
+template <int L, int MODE>
+__global__ __launch_bounds__(256) void matvec_t_dense_kernel(
+    const uint4 *__restrict__ comp, const uint16_t *__restrict__ codebook, uint32_t *__restrict__ W,
+    int m, int cols)
+{
+    constexpr uint32_t mask = (1u << L) - 1u;
+    const int row = blockIdx.x * 256 + threadIdx.x;
+    const int col = blockIdx.y;
+    if (row >= m) return;
+    uint32_t carry = col > 0 ? warm_state<L>(comp[(size_t)(col - 1) * m + row], MODE) : 0u;
+    const uint4 e = comp[(size_t)col * m + row];
+    const uint32_t words[4] = {e.x, e.y, e.z, e.w};
+    uint32_t *wrow = W + (size_t)row * (cols * 32) + col * 32;
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const uint32_t word = words[k];
+        if (MODE == RPTC_AS_WRITTEN) {
+            const uint32_t s2 = mask & ((carry << 2) | (word >> 30));
+            const uint32_t s4 = mask & ((carry << 4) | (word >> 28));
+            carry = s4;
+            const uint32_t w = (uint32_t)codebook[s2] | ((uint32_t)codebook[s4] << 16);
+#pragma unroll
+            for (int j = 0; j < 8; j++) wrow[8 * k + j] = w;
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const uint32_t s2 = mask & alignbit(carry, word, 30 - 4 * j);
+                const uint32_t s4 = mask & alignbit(carry, word, 28 - 4 * j);
+                wrow[8 * k + j] = (uint32_t)codebook[s2] | ((uint32_t)codebook[s4] << 16);
+            }
+            carry = word & mask;
+        }
+    }
+}
+
+template <int L>
+static int lds_bytes_t() { return (2 << L) + kTThreads * 4; }
+
+template <int L>
+static int launch_matvec_t(const int32_t *compressed, const uint16_t *codebook, const uint16_t *x,
+                           uint16_t *out, int64_t m, int64_t n, int carry_mode, void *stream, float *ms)
+{
+    if (!compressed || !codebook || !x || !out) return RPTC_ENULL;
+    if (m < 1 || n < 64 || n % 64 != 0) return RPTC_ESHAPE;
+    if (n > 32768) return RPTC_ELIMIT;      // the reference's 64 KiB of constant memory (inference_t.cu:49)
+    if (carry_mode != RPTC_AS_WRITTEN && carry_mode != RPTC_CONTINUOUS) return RPTC_EMODE;
+    if (!aligned16(compressed) || !aligned16(codebook) || !aligned16(x)) return RPTC_EALIGN;
+    if (m >= (1 << 24)) return RPTC_ELIMIT;
+    DeviceInfo *dev;
+    int rc = device_info(&dev);
+    if (rc) return rc;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    Timer t;
+    rc = t.begin(dev, s, ms);
+    if (rc) return rc;
+    const int grid = (int)((m + kWave - 1) / kWave);
+    auto a_comp = reinterpret_cast<const uint4 *>(compressed);
+    auto a_cb = reinterpret_cast<const uint4 *>(codebook);
+    auto a_x = reinterpret_cast<const uint32_t *>(x);
+    if (carry_mode == RPTC_AS_WRITTEN)
+        hipLaunchKernelGGL((matvec_t_kernel<L, RPTC_AS_WRITTEN>), dim3(grid), dim3(kTThreads), lds_bytes_t<L>(), s,
+                           a_comp, a_cb, a_x, out, (int)m, (int)(n / 64));
+    else
+        hipLaunchKernelGGL((matvec_t_kernel<L, RPTC_CONTINUOUS>), dim3(grid), dim3(kTThreads), lds_bytes_t<L>(), s,
+                           a_comp, a_cb, a_x, out, (int)m, (int)(n / 64));
+    return t.end();
+}
+
+template <int L>
+static int launch_t_dense(const int32_t *compressed, const uint16_t *codebook, uint16_t *W, int64_t m,
+                          int64_t n, int carry_mode, hipStream_t s)
+{
+    auto a_comp = reinterpret_cast<const uint4 *>(compressed);
+    auto a_w = reinterpret_cast<uint32_t *>(W);
+    const dim3 grid((unsigned)((m + 255) / 256), (unsigned)(n / 64));
+    if (carry_mode == RPTC_AS_WRITTEN)
+        hipLaunchKernelGGL((matvec_t_dense_kernel<L, RPTC_AS_WRITTEN>), grid, dim3(256), 0, s, a_comp, codebook, a_w,
+                           (int)m, (int)(n / 64));
+    else
+        hipLaunchKernelGGL((matvec_t_dense_kernel<L, RPTC_CONTINUOUS>), grid, dim3(256), 0, s, a_comp, codebook, a_w,
+                           (int)m, (int)(n / 64));
+    return 0;
+}
+
+int prepare_matvec_t()
+{
+    const void *k[] = {
+        reinterpret_cast<const void *>(matvec_t_kernel<16, RPTC_AS_WRITTEN>),
+        reinterpret_cast<const void *>(matvec_t_kernel<16, RPTC_CONTINUOUS>),
+        reinterpret_cast<const void *>(matvec_t_kernel<14, RPTC_AS_WRITTEN>),
+        reinterpret_cast<const void *>(matvec_t_kernel<14, RPTC_CONTINUOUS>),
+    };
+    for (const void *f : k) {
+        int rc = (int)hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds);
+        if (rc) return rc;
+    }
+    return 0;
+}
+
+}  // namespace rptc
+
+using namespace rptc;
+
+extern "C" int rptc_decompress_matvec_t_16(const int32_t *c, const uint16_t *cb, const uint16_t *x, uint16_t *out,
+                                           int64_t m, int64_t n, int mode, void *stream, float *ms)
+{
+    return launch_matvec_t<16>(c, cb, x, out, m, n, mode, stream, ms);
+}
+
+extern "C" int rptc_decompress_matvec_t_14(const int32_t *c, const uint16_t *cb, const uint16_t *x, uint16_t *out,
+                                           int64_t m, int64_t n, int mode, void *stream, float *ms)
+{
+    return launch_matvec_t<14>(c, cb, x, out, m, n, mode, stream, ms);
+}
+
+extern "C" int rptc_matvec_t_dense(const int32_t *compressed, const uint16_t *codebook, uint16_t *W, int64_t m,
+                                   int64_t n, int L, int carry_mode, void *stream, float *ms)
+{
+    if (!compressed || !codebook || !W) return RPTC_ENULL;
+    if (m < 1 || n < 64 || n % 64 != 0 || (L != 14 && L != 16)) return RPTC_ESHAPE;
+    if (carry_mode != RPTC_AS_WRITTEN && carry_mode != RPTC_CONTINUOUS) return RPTC_EMODE;
+    if (!aligned16(compressed) || !aligned16(codebook) || !aligned16(W)) return RPTC_EALIGN;
+    if (m >= (1 << 24) || n / 64 >= 65536) return RPTC_ELIMIT;
+    DeviceInfo *dev;
+    int rc = device_info(&dev);
+    if (rc) return rc;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    Timer t;
+    rc = t.begin(dev, s, ms);
+    if (rc) return rc;
+    if (L == 16) launch_t_dense<16>(compressed, codebook, W, m, n, carry_mode, s);
+    else launch_t_dense<14>(compressed, codebook, W, m, n, carry_mode, s);
+    return t.end();
+}

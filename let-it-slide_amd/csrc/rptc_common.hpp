@@ -1,0 +1,114 @@
+// Shared host/device helpers of librptc_hip.so (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/rptc_hip.h"
+
+namespace rptc {
+
+constexpr int kWave = 64;              // CDNA4 wavefront
+constexpr int kMaxLds = 160 * 1024;    // LDS per workgroup on gfx950
+
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef unsigned short ushort2_t __attribute__((ext_vector_type(2)));
+
+struct DeviceInfo {
+    int device = -1;
+    int cus = 0;
+    hipEvent_t ev_start = nullptr, ev_stop = nullptr;
+};
+
+// Per-device state, created on first use with that device current.  Returns a status.
+int device_info(DeviceInfo **out);
+
+// Brackets a launch with the two cached events when ms != nullptr.
+struct Timer {
+    hipStream_t stream;
+    float *ms;
+    DeviceInfo *dev;
+    int begin(DeviceInfo *d, hipStream_t s, float *out_ms)
+    {
+        dev = d;
+        stream = s;
+        ms = out_ms;
+        if (!ms) return 0;
+        return (int)hipEventRecord(dev->ev_start, stream);
+    }
+    int end()
+    {
+        int rc = (int)hipGetLastError();
+        if (rc) return rc;
+        if (!ms) return 0;
+        rc = (int)hipEventRecord(dev->ev_stop, stream);
+        if (rc) return rc;
+        rc = (int)hipEventSynchronize(dev->ev_stop);
+        if (rc) return rc;
+        return (int)hipEventElapsedTime(ms, dev->ev_start, dev->ev_stop);
+    }
+};
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+#ifdef __HIPCC__
+// ---------------------------------------------------------------- device helpers
+
+__device__ __forceinline__ uint32_t alignbit(uint32_t hi, uint32_t lo, uint32_t shift)
+{
+    // low 32 bits of ({hi, lo} >> shift), shift in [0, 31]: v_alignbit_b32
+    return __builtin_amdgcn_alignbit(hi, lo, shift);
+}
+
+// both 16-bit halves of g: h*h + h mod 2^16.  Written as asm because the compiler turns the C
+// expression into an add and a multiply.
+__device__ __forceinline__ uint32_t pk_hash16(uint32_t g)
+{
+    uint32_t h;
+    asm("v_pk_mad_u16 %0, %1, %1, %1" : "=v"(h) : "v"(g));
+    return h;
+}
+
+// (a & mask) | c in one op; mask must sit in a scalar register (no literals in VOP3 on gfx9)
+__device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask, uint32_t c)
+{
+    uint32_t d;
+    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(d) : "v"(a), "s"(mask), "v"(c));
+    return d;
+}
+
+// byte permute of {hi, lo}: selector byte i picks the source of result byte i
+// (0-3 = bytes of lo, 4-7 = bytes of hi, 0x0C = zero)
+__device__ __forceinline__ uint32_t perm(uint32_t hi, uint32_t lo, uint32_t sel)
+{
+    uint32_t d;
+    asm("v_perm_b32 %0, %1, %2, %3" : "=v"(d) : "v"(hi), "v"(lo), "s"(sel));
+    return d;
+}
+
+// 32-bit LDS read at an absolute LDS byte address (no base is added)
+__device__ __forceinline__ uint32_t lds_read_abs(uint32_t byte_address)
+{
+    typedef __attribute__((address_space(3))) const uint32_t lds_u32;
+    return *reinterpret_cast<lds_u32 *>(static_cast<uintptr_t>(byte_address));
+}
+
+__device__ __forceinline__ float dot2(uint32_t w, uint32_t a, float acc)
+{
+    // acc + w.lo*a.lo + w.hi*a.hi with the products and the sum in fp32: v_dot2_f32_f16
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, w), __builtin_bit_cast(half2_t, a), acc, false);
+}
+
+__device__ __forceinline__ uint16_t float_to_half_bits(float f)
+{
+    _Float16 h = (_Float16)f;   // v_cvt_f16_f32, round to nearest even
+    return __builtin_bit_cast(uint16_t, h);
+}
+
+__device__ __forceinline__ float half_bits_to_float(uint16_t b)
+{
+    return (float)__builtin_bit_cast(_Float16, b);
+}
+#endif
+
+}  // namespace rptc

@@ -1,0 +1,271 @@
+"""rptc_kernels for MI355X: the reference extension's seven ops over hand-written gfx950 kernels.
+
+Drop-in for the reference's pybind11 module (rptc_kernels/csrc/rptc_kernels/wrapper.cpp:59-67):
+the same seven callables, positional ``torch.Tensor`` arguments, outputs written in place into
+tensors the caller allocates, elapsed milliseconds returned as a ``float``, argument errors
+raised as ``RuntimeError`` (what ``TORCH_CHECK`` raises).  The work is done by
+``librptc_hip.so`` through its C ABI (include/rptc_hip.h); this module only validates tensors
+and passes raw device pointers plus the current HIP stream.  There is no CPU implementation:
+without the library, or with CPU tensors, every op raises.
+
+Differences from the reference, all deliberate:
+* ``carry_mode`` (module-level, see ``set_carry_mode``) chooses between the CUDA source's literal
+  arithmetic (``AS_WRITTEN``, the default) and one unbroken shift register per row
+  (``CONTINUOUS``, the trellis of rptc.py:74-85).
+* the returned milliseconds always time the op's own kernels on the stream they ran on (the
+  reference's ``decompress_matvec_*`` times an idle stream, inference.cu:335-350).  Timing makes
+  a call host-synchronous, as ``decompress`` and ``decompress_matvec_t_*`` are in the reference;
+  ``set_timing(False)`` makes every op asynchronous and return 0.0.
+* ``decompress_matvec_*`` accumulates in fp32 and accepts any row count and any ``n % 64 == 0``
+  (a ragged last slab); ``decompress_matvec_t_*`` accepts any row count.
+"""
+import ctypes
+import os
+
+import torch
+
+AS_WRITTEN = 0
+CONTINUOUS = 1
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(os.path.dirname(_HERE), "librptc_hip.so")
+
+_lib = None
+_carry_mode = AS_WRITTEN
+_timing = True
+
+_VP, _I64, _INT = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
+_FP = ctypes.POINTER(ctypes.c_float)
+
+_MATVEC_ARGS = [_VP, _VP, _VP, _VP, _I64, _I64, _INT, _VP, _FP]
+_SIGNATURES = {
+    "rptc_version": ([], _INT),
+    "rptc_status_string": ([_INT], ctypes.c_char_p),
+    "rptc_init": ([], _INT),
+    "rptc_decompress": ([_VP, _VP, _VP, _I64, _I64, _INT, _VP, _FP], _INT),
+    "rptc_decompress_matvec_16_6_1": (_MATVEC_ARGS, _INT),
+    "rptc_decompress_matvec_20_6_1": (_MATVEC_ARGS, _INT),
+    "rptc_decompress_matvec_16_8_1": (_MATVEC_ARGS, _INT),
+    "rptc_decompress_matvec_20_8_1": (_MATVEC_ARGS, _INT),
+    "rptc_decompress_matvec_t_16": (_MATVEC_ARGS, _INT),
+    "rptc_decompress_matvec_t_14": (_MATVEC_ARGS, _INT),
+    "rptc_matvec_dense": ([_VP, _VP, _VP, _I64, _I64, _INT, _INT, _VP, _FP], _INT),
+    "rptc_matvec_t_dense": ([_VP, _VP, _VP, _I64, _I64, _INT, _INT, _VP, _FP], _INT),
+}
+
+
+def library_path():
+    return _LIB_PATH
+
+
+def exported_symbols():
+    """Names the C header declares; used by the load test."""
+    return sorted(_SIGNATURES)
+
+
+def library():
+    """The loaded C-ABI library.  Raises if it has not been built: there is no fallback."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            raise RuntimeError(
+                f"rptc_kernels: {_LIB_PATH} is missing; build it with "
+                "`python let-it-slide_amd/build.py` (hipcc, gfx950)")
+        lib = ctypes.CDLL(_LIB_PATH)
+        for name, (argtypes, restype) in _SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.argtypes = argtypes
+            fn.restype = restype
+        _lib = lib
+    return _lib
+
+
+def set_carry_mode(mode):
+    """AS_WRITTEN (default) or CONTINUOUS; returns the previous mode."""
+    global _carry_mode
+    if mode not in (AS_WRITTEN, CONTINUOUS):
+        raise ValueError("carry mode must be rptc_kernels.AS_WRITTEN or rptc_kernels.CONTINUOUS")
+    prev, _carry_mode = _carry_mode, mode
+    return prev
+
+
+def get_carry_mode():
+    return _carry_mode
+
+
+def set_timing(enabled):
+    """When False, ops launch asynchronously and return 0.0; returns the previous setting."""
+    global _timing
+    prev, _timing = _timing, bool(enabled)
+    return prev
+
+
+def _check(cond, msg):
+    if not cond:
+        raise RuntimeError(msg)
+
+
+def _check_input(t, name):
+    # CHECK_INPUT of the reference (inference.cu:26-28)
+    _check(isinstance(t, torch.Tensor), f"{name} must be a torch.Tensor")
+    _check(t.is_cuda, f"{name} must be a CUDA tensor")
+    _check(t.is_contiguous(), f"{name} must be contiguous")
+
+
+def _status(rc):
+    if rc != 0:
+        text = library().rptc_status_string(rc).decode()
+        raise RuntimeError(f"rptc_kernels: {text} (status {rc})")
+
+
+def _call(fn, tensors, *args):
+    device = tensors[0].device
+    for t in tensors[1:]:
+        _check(t.device == device, "all tensors must be on the same device")
+    ms = ctypes.c_float(0.0)
+    with torch.cuda.device(device):
+        stream = torch.cuda.current_stream().cuda_stream
+        rc = fn(*[t.data_ptr() for t in tensors], *args, _carry_mode, ctypes.c_void_p(stream),
+                ctypes.byref(ms) if _timing else None)
+    _status(rc)
+    return float(ms.value)
+
+
+def decompress(compressed, codebook, out):
+    """Decode the row-major stream: out[r, t] = codebook[16 stream bits ending at bit 2t+2].
+
+    compressed int32 [m, 4c] with 4c % 128 == 0; codebook fp16 [65536]; out fp16 [m, 64c]
+    (inference.cu:99-160).  Returns elapsed ms."""
+    _check_input(compressed, "compressed")
+    _check(compressed.dim() == 2, "compressed.dim() == 2")
+    _check(compressed.size(1) % (4 * 32) == 0, "compressed.size(1) % (4 * 32) == 0")
+    _check(compressed.dtype == torch.int32, "compressed.scalar_type() == torch::kInt32")
+    m = compressed.size(0)
+    n = compressed.size(1) // 4 * 64
+    _check(m >= 1 and compressed.size(1) >= 128, "compressed must not be empty")
+    _check_input(codebook, "codebook")
+    _check(codebook.dim() == 1, "codebook.dim() == 1")
+    _check(codebook.size(0) == 1 << 16, "codebook.size(0) == 1<<16")
+    _check(codebook.dtype == torch.float16, "codebook.scalar_type() == torch::kFloat16")
+    _check_input(out, "out")
+    _check(out.dim() == 2, "out.dim() == 2")
+    _check(out.size(0) == m, "out.size(0) == m")
+    _check(out.size(1) == n, "out.size(1) == n")
+    _check(out.dtype == torch.float16, "out.scalar_type() == torch::kFloat16")
+    return _call(library().rptc_decompress, (compressed, codebook, out), m, compressed.size(1))
+
+
+def _matvec(symbol, S, compressed, codebook, x, out):
+    # checks of inference.cu:293-316, relaxed where the library accepts more
+    _check_input(compressed, "compressed")
+    _check(compressed.dtype == torch.int32, "compressed.scalar_type() == torch::kInt32")
+    _check_input(x, "x")
+    _check(x.dim() == 1, "x.dim() == 1")
+    _check(x.dtype == torch.float16, "x.scalar_type() == torch::kFloat16")
+    _check_input(out, "out")
+    _check(out.dim() == 1, "out.dim() == 1")
+    _check(out.dtype == torch.float16, "out.scalar_type() == torch::kFloat16")
+    n, m = x.size(0), out.size(0)
+    if compressed.dim() == 3:
+        # the reference layout [n/2048, m, 128]
+        _check(compressed.size(2) == 32 * 4, "compressed.size(2) == 32 * 4")
+        _check(compressed.size(1) == m, "out.size(0) == m")
+        _check(compressed.size(0) * 32 * 4 * 16 == n, "x.size(0) == n")
+    else:
+        # flat stream with a ragged last slab (n % 2048 != 0)
+        _check(compressed.dim() == 1, "compressed.dim() == 3 (or 1 for a ragged stream)")
+        _check(n % 64 == 0, "x.size(0) % 64 == 0")
+        _check(compressed.numel() * 16 == m * n, "compressed.numel() * 16 == m * n")
+    _check(m >= 1 and n >= 64, "compressed must not be empty")
+    _check_input(codebook, "codebook")
+    _check(codebook.dim() == 1, "codebook.dim() == 1")
+    _check(codebook.size(0) == 1 << (S + 1), "codebook.size(0) == 1<<(S+V)")
+    _check(codebook.dtype == torch.float16, "codebook.scalar_type() == torch::kFloat16")
+    return _call(getattr(library(), symbol), (compressed, codebook, x, out), m, n)
+
+
+def decompress_matvec_16_6_1(compressed, codebook, x, out):
+    """out = W x for the hashed-codebook stream, 64 codebook pairs (inference.cu:358-362)."""
+    return _matvec("rptc_decompress_matvec_16_6_1", 6, compressed, codebook, x, out)
+
+
+def decompress_matvec_20_6_1(compressed, codebook, x, out):
+    """Same function as decompress_matvec_16_6_1: the reference kernel ignores L (inference.cu:364-368)."""
+    return _matvec("rptc_decompress_matvec_20_6_1", 6, compressed, codebook, x, out)
+
+
+def decompress_matvec_16_8_1(compressed, codebook, x, out):
+    """out = W x for the hashed-codebook stream, 256 codebook pairs (inference.cu:370-374)."""
+    return _matvec("rptc_decompress_matvec_16_8_1", 8, compressed, codebook, x, out)
+
+
+def decompress_matvec_20_8_1(compressed, codebook, x, out):
+    """Same function as decompress_matvec_16_8_1 (inference.cu:376-380)."""
+    return _matvec("rptc_decompress_matvec_20_8_1", 8, compressed, codebook, x, out)
+
+
+def _matvec_t(symbol, L, compressed, codebook, x, out):
+    # checks of inference_t.cu:188-221; m and n come from out and x as in the reference
+    _check_input(compressed, "compressed")
+    _check(compressed.dtype == torch.int32, "compressed.scalar_type() == torch::kInt32")
+    _check_input(out, "out")
+    _check_input(x, "x")
+    m, n = out.size(0), x.size(0)
+    _check_input(codebook, "codebook")
+    _check(codebook.dim() == 1, "codebook.dim() == 1")
+    _check(codebook.size(0) == 1 << L, "codebook.size(0) == 1<<L")
+    _check(codebook.dtype == torch.float16, "codebook.scalar_type() == torch::kFloat16")
+    _check(x.dim() == 1, "x.dim() == 1")
+    _check(x.size(0) % 8 == 0, "x.size(0) % 8 == 0")
+    _check(x.dtype == torch.float16, "x.scalar_type() == torch::kFloat16")
+    _check(n % 64 == 0 and n >= 64, "x.size(0) % 64 == 0 (the kernel reads whole uint4 elements)")
+    _check(n <= 32768, "x must fit the 64 KiB activation buffer (n <= 32768)")
+    _check(out.dim() == 1, "out.dim() == 1")
+    _check(out.dtype == torch.float16, "out.scalar_type() == torch::kFloat16")
+    _check(m >= 1, "out must not be empty")
+    _check(compressed.numel() * 16 >= m * n, "compressed holds fewer than m*n/16 words")
+    return _call(getattr(library(), symbol), (compressed, codebook, x, out), m, n)
+
+
+def decompress_matvec_t_16(compressed, codebook, x, out):
+    """out += W x for the column-interleaved stream, 2^16 scalar codebook (inference_t.cu:258-262)."""
+    return _matvec_t("rptc_decompress_matvec_t_16", 16, compressed, codebook, x, out)
+
+
+def decompress_matvec_t_14(compressed, codebook, x, out):
+    """out += W x for the column-interleaved stream, 2^14 scalar codebook (inference_t.cu:264-268)."""
+    return _matvec_t("rptc_decompress_matvec_t_14", 14, compressed, codebook, x, out)
+
+
+# ---------------------------------------------------------------- additions to the reference API
+
+def matvec_dense(compressed, codebook, out, S):
+    """Write the dense fp16 [m, n] matrix a hashed-codebook stream stands for into ``out``."""
+    _check_input(compressed, "compressed")
+    _check(compressed.dtype == torch.int32, "compressed.scalar_type() == torch::kInt32")
+    _check_input(codebook, "codebook")
+    _check(S in (6, 8), "S must be 6 or 8")
+    _check(codebook.dim() == 1 and codebook.size(0) == 1 << (S + 1), "codebook.size(0) == 1<<(S+V)")
+    _check(codebook.dtype == torch.float16, "codebook.scalar_type() == torch::kFloat16")
+    _check_input(out, "out")
+    _check(out.dim() == 2 and out.dtype == torch.float16, "out must be a 2-D fp16 tensor")
+    m, n = out.shape
+    _check(n % 64 == 0 and m >= 1 and n >= 64, "out.size(1) % 64 == 0")
+    _check(compressed.numel() * 16 == m * n, "compressed.numel() * 16 == m * n")
+    return _call(library().rptc_matvec_dense, (compressed, codebook, out), m, n, S)
+
+
+def matvec_t_dense(compressed, codebook, out, L):
+    """Write the dense fp16 [m, n] matrix a column-interleaved stream stands for into ``out``."""
+    _check_input(compressed, "compressed")
+    _check(compressed.dtype == torch.int32, "compressed.scalar_type() == torch::kInt32")
+    _check_input(codebook, "codebook")
+    _check(L in (14, 16), "L must be 14 or 16")
+    _check(codebook.dim() == 1 and codebook.size(0) == 1 << L, "codebook.size(0) == 1<<L")
+    _check(codebook.dtype == torch.float16, "codebook.scalar_type() == torch::kFloat16")
+    _check_input(out, "out")
+    _check(out.dim() == 2 and out.dtype == torch.float16, "out must be a 2-D fp16 tensor")
+    m, n = out.shape
+    _check(n % 64 == 0 and m >= 1 and n >= 64, "out.size(1) % 64 == 0")
+    _check(compressed.numel() * 16 >= m * n, "compressed holds fewer than m*n/16 words")
+    return _call(library().rptc_matvec_t_dense, (compressed, codebook, out), m, n, L)

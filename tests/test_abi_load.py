@@ -1,0 +1,85 @@
+"""The C-ABI library loads without a GPU and exports every function include/rptc_hip.h declares;
+the Python module validates arguments the way the reference's TORCH_CHECKs do."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "rptc_hip.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(rptc_\w+)\s*\(", text)))
+
+
+def test_header_declares_the_reference_surface():
+    names = declared_functions()
+    for op in ("decompress", "decompress_matvec_16_6_1", "decompress_matvec_20_6_1", "decompress_matvec_16_8_1",
+               "decompress_matvec_20_8_1", "decompress_matvec_t_16", "decompress_matvec_t_14"):
+        assert "rptc_" + op in names
+
+
+def test_library_exports_every_declared_symbol():
+    import rptc_kernels
+    assert os.path.exists(rptc_kernels.library_path()), "build with python let-it-slide_amd/build.py"
+    lib = ctypes.CDLL(rptc_kernels.library_path())
+    for name in declared_functions():
+        assert hasattr(lib, name), name
+    assert sorted(rptc_kernels.exported_symbols()) == declared_functions()
+    assert rptc_kernels.library().rptc_version() >= 100
+    assert b"NULL" in rptc_kernels.library().rptc_status_string(-1)
+
+
+def test_python_module_has_the_reference_names():
+    import rptc_kernels
+    for op in ("decompress", "decompress_matvec_16_6_1", "decompress_matvec_20_6_1", "decompress_matvec_16_8_1",
+               "decompress_matvec_20_8_1", "decompress_matvec_t_16", "decompress_matvec_t_14"):
+        assert callable(getattr(rptc_kernels, op))
+
+
+def test_cpu_tensors_are_rejected_not_computed():
+    import rptc_kernels
+    comp = torch.zeros((2, 128), dtype=torch.int32)
+    cb = torch.zeros(65536, dtype=torch.float16)
+    out = torch.zeros((2, 2048), dtype=torch.float16)
+    with pytest.raises(RuntimeError, match="must be a CUDA tensor"):
+        rptc_kernels.decompress(comp, cb, out)
+    with pytest.raises(RuntimeError, match="must be a CUDA tensor"):
+        rptc_kernels.decompress_matvec_16_8_1(torch.zeros((1, 32, 128), dtype=torch.int32),
+                                              torch.zeros(512, dtype=torch.float16),
+                                              torch.zeros(2048, dtype=torch.float16),
+                                              torch.zeros(32, dtype=torch.float16))
+    with pytest.raises(RuntimeError, match="must be a CUDA tensor"):
+        rptc_kernels.decompress_matvec_t_16(torch.zeros(256 * 64 // 16, dtype=torch.int32), cb,
+                                            torch.zeros(64, dtype=torch.float16),
+                                            torch.zeros(256, dtype=torch.float16))
+
+
+def test_c_abi_rejects_bad_arguments_before_touching_a_device():
+    import rptc_kernels
+    lib = rptc_kernels.library()
+    # NULL pointers and bad shapes are reported as negative statuses; no device is needed for these
+    assert lib.rptc_decompress(None, None, None, 1, 128, 0, None, None) == -1
+    assert lib.rptc_decompress(16, 16, 16, 1, 100, 0, None, None) == -2
+    assert lib.rptc_decompress(16, 16, 16, 1, 128, 7, None, None) == -4
+    assert lib.rptc_decompress(8, 16, 16, 1, 128, 0, None, None) == -3
+    assert lib.rptc_decompress_matvec_16_8_1(16, 16, 16, 16, 32, 100, 0, None, None) == -2
+    assert lib.rptc_decompress_matvec_t_16(16, 16, 16, 16, 256, 65536, 0, None, None) == -5
+    assert lib.rptc_matvec_dense(16, 16, 16, 4, 64, 7, 0, None, None) == -2
+    assert lib.rptc_matvec_t_dense(16, 16, 16, 4, 64, 15, 0, None, None) == -2
+
+
+def test_carry_mode_and_timing_switches():
+    import rptc_kernels
+    prev = rptc_kernels.set_carry_mode(rptc_kernels.CONTINUOUS)
+    assert rptc_kernels.get_carry_mode() == rptc_kernels.CONTINUOUS
+    rptc_kernels.set_carry_mode(prev)
+    with pytest.raises(ValueError):
+        rptc_kernels.set_carry_mode(3)
+    prev = rptc_kernels.set_timing(False)
+    rptc_kernels.set_timing(prev)

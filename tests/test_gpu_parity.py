@@ -1,0 +1,328 @@
+"""GPU parity: the HIP kernels, called through the rptc_kernels module (ctypes -> C ABI), against
+the CPU oracle on the same seeded inputs.  Decoded weights must match bit for bit; layer outputs
+must be within rel-L2 1e-3 of the double-precision product of the decoded fp16 weights."""
+import numpy as np
+import pytest
+import torch
+
+from util import np_f16, np_u32, rand_codes, rand_half, rel_l2
+
+pytestmark = pytest.mark.gpu
+
+REL_L2_TOL = 1e-3          # the tolerance the north star states for layer outputs (fp32 accumulate)
+MODES = [0, 1]
+
+
+@pytest.fixture(scope="module")
+def rk():
+    import rptc_kernels
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    rc = rptc_kernels.library().rptc_init()
+    assert rc == 0, rptc_kernels.library().rptc_status_string(rc)
+    return rptc_kernels
+
+
+@pytest.fixture(autouse=True)
+def _announce(request):
+    print(f"\n[case] {request.node.nodeid}", flush=True)
+    yield
+
+
+def with_mode(rk, mode):
+    class _Ctx:
+        def __enter__(self):
+            self.prev = rk.set_carry_mode(mode)
+
+        def __exit__(self, *a):
+            rk.set_carry_mode(self.prev)
+    return _Ctx()
+
+
+# ------------------------------------------------------------------ decompress (inference.cu:42-160)
+
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("m,cn", [(1, 32), (3, 96), (64, 64), (257, 32)])
+def test_decompress_bit_exact(rk, oracle, mode, m, cn):
+    comp = rand_codes(m * 4 * cn, seed=m + cn).reshape(m, 4 * cn)
+    cb = rand_half(65536, seed=3)
+    out = torch.full((m, 64 * cn), float("nan"), dtype=torch.float16, device="cuda")
+    with with_mode(rk, mode):
+        ms = rk.decompress(comp.cuda(), cb.cuda(), out)
+    assert ms > 0
+    want = oracle.decompress(np_u32(comp), np_f16(cb), mode=mode)
+    assert np.array_equal(np_f16(out).view(np.uint16), want.view(np.uint16))
+
+
+def test_decompress_state_sequence_with_bit_pattern_codebook(rk, oracle):
+    # codebook[s] has raw bits s, so the output IS the decoder state: no float compare involved
+    m, cn = 8, 64
+    comp = rand_codes(m * 4 * cn, seed=99).reshape(m, 4 * cn)
+    cb = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.float16)
+    out = torch.zeros((m, 64 * cn), dtype=torch.float16, device="cuda")
+    for mode in MODES:
+        with with_mode(rk, mode):
+            rk.decompress(comp.cuda(), cb.cuda(), out)
+        want = oracle.decompress(np_u32(comp), np_f16(cb), mode=mode)
+        assert np.array_equal(np_f16(out).view(np.uint16), want.view(np.uint16))
+    # hand-derived: first word of row 0 from state 0
+    word = int(np_u32(comp)[0, 0])
+    states = []
+    s = 0
+    for i in range(16):
+        s = ((s << 2) | ((word >> (30 - 2 * i)) & 3)) & 0xFFFF
+        states.append(s)
+    assert np_f16(out).view(np.uint16)[0, :16].tolist() == states
+
+
+def test_decompress_full_size_4096x4096(rk, oracle):
+    m, cn = 4096, 64
+    comp = rand_codes(m * 4 * cn, seed=42).reshape(m, 4 * cn)
+    cb = rand_half(65536, seed=43)
+    out = torch.zeros((m, 64 * cn), dtype=torch.float16, device="cuda")
+    rk.decompress(comp.cuda(), cb.cuda(), out)
+    want = oracle.decompress(np_u32(comp), np_f16(cb), mode=0)
+    assert np.array_equal(np_f16(out).view(np.uint16), want.view(np.uint16))
+
+
+def test_decompress_rejects_what_the_reference_rejects(rk):
+    cb = torch.zeros(65536, dtype=torch.float16, device="cuda")
+    good = torch.zeros((2, 128), dtype=torch.int32, device="cuda")
+    out = torch.zeros((2, 2048), dtype=torch.float16, device="cuda")
+    with pytest.raises(RuntimeError):
+        rk.decompress(torch.zeros((2, 64), dtype=torch.int32, device="cuda"), cb, out)      # size(1) % 128
+    with pytest.raises(RuntimeError):
+        rk.decompress(good.to(torch.int64), cb, out)                                         # dtype
+    with pytest.raises(RuntimeError):
+        rk.decompress(good, cb[:4096], out)                                                  # codebook size
+    with pytest.raises(RuntimeError):
+        rk.decompress(good, cb, out[:, :1024])                                               # out shape / contiguity
+    with pytest.raises(RuntimeError):
+        rk.decompress(good.t(), cb, out)                                                     # non-contiguous
+
+
+# ------------------------------------------------------------------ decompress_matvec (inference.cu:189-380)
+
+def matvec_fn(rk, L, S):
+    return getattr(rk, f"decompress_matvec_{L}_{S}_1")
+
+
+MATVEC_SHAPES = [(32, 2048), (64, 4096), (33, 2048), (1, 64), (7, 704), (96, 4096 + 768), (512, 6144)]
+
+
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("S", [6, 8])
+@pytest.mark.parametrize("m,n", MATVEC_SHAPES)
+def test_matvec_dense_export_bit_exact(rk, oracle, mode, S, m, n):
+    comp = rand_codes(m * n // 16, seed=m * 7 + n)
+    cb = rand_half(2 << S, seed=S)
+    W = torch.zeros((m, n), dtype=torch.float16, device="cuda")
+    with with_mode(rk, mode):
+        rk.matvec_dense(comp.cuda(), cb.cuda(), W, S)
+    want = oracle.matvec_dense(np_u32(comp), np_f16(cb), m, n, S, mode=mode)
+    assert np.array_equal(np_f16(W).view(np.uint16), want.view(np.uint16))
+
+
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("L,S", [(16, 6), (20, 6), (16, 8), (20, 8)])
+@pytest.mark.parametrize("m,n", MATVEC_SHAPES)
+def test_matvec_output_within_tolerance(rk, oracle, mode, L, S, m, n):
+    comp = rand_codes(m * n // 16, seed=m + n)
+    cb = rand_half(2 << S, seed=S + 10)
+    x = rand_half(n, seed=5)
+    out = torch.full((m,), float("nan"), dtype=torch.float16, device="cuda")
+    c = comp.cuda().reshape(n // 2048, m, 128) if n % 2048 == 0 else comp.cuda()
+    with with_mode(rk, mode):
+        ms = matvec_fn(rk, L, S)(c, cb.cuda(), x.cuda(), out)
+    assert ms > 0
+    want = oracle.matvec(np_u32(comp), np_f16(cb), np_f16(x), m, S, mode=mode)
+    got = np_f16(out).astype(np.float64)
+    assert np.all(np.isfinite(got))
+    # fp16 rounding of the result alone is 2^-11 relative per element
+    assert rel_l2(got, want) < REL_L2_TOL
+
+
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("S", [6, 8])
+def test_matvec_fused_kernel_decodes_bit_exactly(rk, oracle, mode, S):
+    """One-hot activations: y[r] = W[r, p] exactly (a single product 1.0 * w, added to zeros in
+    fp32), so the fused kernel's own decode and column map are checked bit for bit."""
+    m, n = 64, 2048 + 192
+    comp = rand_codes(m * n // 16, seed=123)
+    cb = rand_half(2 << S, seed=S + 20)
+    want = oracle.matvec_dense(np_u32(comp), np_f16(cb), m, n, S, mode=mode)
+    c, cbd = comp.cuda(), cb.cuda()
+    out = torch.zeros((m,), dtype=torch.float16, device="cuda")
+    x = torch.zeros(n, dtype=torch.float16, device="cuda")
+    got = np.zeros((m, n), dtype=np.float16)
+    prev_timing = rk.set_timing(False)
+    try:
+        with with_mode(rk, mode):
+            cols = list(range(0, n, 7)) + list(range(n - 200, n)) + list(range(0, 64))
+            for p in cols:
+                x.zero_()
+                x[p] = 1.0
+                matvec_fn(rk, 16, S)(c, cbd, x, out)
+                got[:, p] = np_f16(out)
+    finally:
+        rk.set_timing(prev_timing)
+    cols = sorted(set(cols))
+    g = got[:, cols].view(np.uint16)
+    w = want[:, cols].view(np.uint16)
+    # -0.0 * 1.0 + 0.0 = +0.0 in the accumulator: compare zeros by value
+    nz = (w & 0x7FFF) != 0
+    assert np.array_equal(g[nz], w[nz])
+    assert np.all((g[~nz] & 0x7FFF) == 0)
+
+
+@pytest.mark.parametrize("m,n", [(4096, 4096), (4096, 11008), (11008, 4096)])
+def test_matvec_full_size(rk, oracle, m, n):
+    S = 8
+    comp = rand_codes(m * n // 16, seed=42)
+    cb = rand_half(2 << S, seed=43)
+    x = rand_half(n, seed=44)
+    out = torch.zeros((m,), dtype=torch.float16, device="cuda")
+    c = comp.cuda().reshape(n // 2048, m, 128) if n % 2048 == 0 else comp.cuda()
+    matvec_fn(rk, 16, S)(c, cb.cuda(), x.cuda(), out)
+    want = oracle.matvec(np_u32(comp), np_f16(cb), np_f16(x), m, S, mode=0)
+    assert rel_l2(np_f16(out), want) < REL_L2_TOL
+    # decoded weights at full size, bit for bit
+    W = torch.zeros((m, n), dtype=torch.float16, device="cuda")
+    rk.matvec_dense(comp.cuda(), cb.cuda(), W, S)
+    wantW = oracle.matvec_dense(np_u32(comp), np_f16(cb), m, n, S, mode=0)
+    assert np.array_equal(np_f16(W).view(np.uint16), wantW.view(np.uint16))
+    # size-independent properties: the fused product equals the dense product of the exported
+    # matrix, and the op is linear in x
+    y_dense = (W.double() @ x.cuda().double()).cpu().numpy()
+    assert rel_l2(np_f16(out), y_dense) < REL_L2_TOL
+    x2 = rand_half(n, seed=45)
+    out2 = torch.zeros_like(out)
+    out12 = torch.zeros_like(out)
+    matvec_fn(rk, 16, S)(c, cb.cuda(), x2.cuda(), out2)
+    xs = (x.float() + x2.float()).to(torch.float16)
+    matvec_fn(rk, 16, S)(c, cb.cuda(), xs.cuda(), out12)
+    lin = (W.double() @ xs.cuda().double()).cpu().numpy()
+    assert rel_l2(np_f16(out12), lin) < REL_L2_TOL
+    assert rel_l2(np_f16(out12).astype(np.float64), np_f16(out).astype(np.float64) + np_f16(out2).astype(np.float64)) < 5e-3
+
+
+def test_matvec_zero_stream_closed_form(rk):
+    m, n, S = 64, 4096, 6
+    cb = rand_half(2 << S, seed=3)
+    x = rand_half(n, seed=4)
+    out = torch.zeros((m,), dtype=torch.float16, device="cuda")
+    rk.decompress_matvec_16_6_1(torch.zeros((2, m, 128), dtype=torch.int32, device="cuda"), cb.cuda(), x.cuda(), out)
+    xe = x.double()[0::2].sum().item()
+    xo = x.double()[1::2].sum().item()
+    want = abs(float(cb[0])) * xe + float(cb[1]) * xo
+    assert np.allclose(np_f16(out).astype(np.float64), want, rtol=2e-3, atol=2e-2)
+
+
+def test_matvec_rejects_what_the_reference_rejects(rk):
+    cb = torch.zeros(512, dtype=torch.float16, device="cuda")
+    comp = torch.zeros((1, 32, 128), dtype=torch.int32, device="cuda")
+    x = torch.zeros(2048, dtype=torch.float16, device="cuda")
+    out = torch.zeros(32, dtype=torch.float16, device="cuda")
+    f = rk.decompress_matvec_16_8_1
+    with pytest.raises(RuntimeError):
+        f(torch.zeros((1, 32, 64), dtype=torch.int32, device="cuda"), cb, x, out)     # size(2) == 128
+    with pytest.raises(RuntimeError):
+        f(comp, cb[:128], x, out)                                                     # codebook size 2^(S+V)
+    with pytest.raises(RuntimeError):
+        f(comp, cb, x[:1024], out)                                                    # x.size(0) == n
+    with pytest.raises(RuntimeError):
+        f(comp, cb, x, out[:16])                                                      # out.size(0) == m
+    with pytest.raises(RuntimeError):
+        f(comp, cb, x.float(), out)                                                   # dtype
+    with pytest.raises(RuntimeError):
+        rk.decompress_matvec_16_6_1(comp, cb, x, out)                                 # S=6 wants 128 values
+    assert f(comp, cb, x, out) >= 0.0
+
+
+# ------------------------------------------------------------------ decompress_matvec_t (inference_t.cu:68-268)
+
+T_SHAPES = [(256, 64), (256, 1024), (300, 4096), (1, 128), (1024, 2048)]
+
+
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("L", [14, 16])
+@pytest.mark.parametrize("m,n", T_SHAPES)
+def test_matvec_t_dense_export_bit_exact(rk, oracle, mode, L, m, n):
+    comp = rand_codes(m * n // 16, seed=m + n + L)
+    cb = rand_half(1 << L, seed=L)
+    W = torch.zeros((m, n), dtype=torch.float16, device="cuda")
+    with with_mode(rk, mode):
+        rk.matvec_t_dense(comp.cuda(), cb.cuda(), W, L)
+    want = oracle.matvec_t_dense(np_u32(comp), np_f16(cb), m, n, L, mode=mode)
+    assert np.array_equal(np_f16(W).view(np.uint16), want.view(np.uint16))
+
+
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("L", [14, 16])
+@pytest.mark.parametrize("m,n", T_SHAPES)
+def test_matvec_t_output_within_tolerance(rk, oracle, mode, L, m, n):
+    comp = rand_codes(m * n // 16, seed=m + n + L)
+    cb = rand_half(1 << L, seed=L)
+    x = rand_half(n, seed=6)
+    out0 = rand_half(m, seed=8)
+    out = out0.cuda()
+    with with_mode(rk, mode):
+        ms = getattr(rk, f"decompress_matvec_t_{L}")(comp.cuda(), cb.cuda(), x.cuda(), out)
+    assert ms > 0
+    want = oracle.matvec_t(np_u32(comp), np_f16(cb), np_f16(x), m, L, mode=mode)
+    want = want + np_f16(out0).astype(np.float64)         # the op accumulates into out
+    assert rel_l2(np_f16(out), want) < REL_L2_TOL
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_matvec_t_fused_kernel_decodes_bit_exactly(rk, oracle, mode):
+    L, m, n = 16, 128, 512
+    comp = rand_codes(m * n // 16, seed=77)
+    cb = rand_half(1 << L, seed=78)
+    want = oracle.matvec_t_dense(np_u32(comp), np_f16(cb), m, n, L, mode=mode)
+    c, cbd = comp.cuda(), cb.cuda()
+    x = torch.zeros(n, dtype=torch.float16, device="cuda")
+    got = np.zeros((m, n), dtype=np.float16)
+    prev_timing = rk.set_timing(False)
+    try:
+        with with_mode(rk, mode):
+            for p in range(n):
+                x.zero_()
+                x[p] = 1.0
+                out = torch.zeros((m,), dtype=torch.float16, device="cuda")
+                rk.decompress_matvec_t_16(c, cbd, x, out)
+                got[:, p] = np_f16(out)
+    finally:
+        rk.set_timing(prev_timing)
+    g, w = got.view(np.uint16), want.view(np.uint16)
+    nz = (w & 0x7FFF) != 0
+    assert np.array_equal(g[nz], w[nz])
+    assert np.all((g[~nz] & 0x7FFF) == 0)
+
+
+def test_matvec_t_full_size_4096(rk, oracle):
+    L, m, n = 16, 4096, 4096
+    comp = rand_codes(m * n // 16, seed=42)
+    cb = rand_half(1 << L, seed=43)
+    x = rand_half(n, seed=44)
+    for mode in MODES:
+        out = torch.zeros((m,), dtype=torch.float16, device="cuda")
+        with with_mode(rk, mode):
+            rk.decompress_matvec_t_16(comp.cuda(), cb.cuda(), x.cuda(), out)
+        want = oracle.matvec_t(np_u32(comp), np_f16(cb), np_f16(x), m, L, mode=mode)
+        assert rel_l2(np_f16(out), want) < REL_L2_TOL
+
+
+def test_matvec_t_rejects_bad_arguments(rk):
+    cb = torch.zeros(65536, dtype=torch.float16, device="cuda")
+    comp = torch.zeros(256 * 64 // 16, dtype=torch.int32, device="cuda")
+    x = torch.zeros(64, dtype=torch.float16, device="cuda")
+    out = torch.zeros(256, dtype=torch.float16, device="cuda")
+    with pytest.raises(RuntimeError):
+        rk.decompress_matvec_t_16(comp, cb[:16384], x, out)          # codebook.size(0) == 1<<L
+    with pytest.raises(RuntimeError):
+        rk.decompress_matvec_t_14(comp, cb, x, out)
+    with pytest.raises(RuntimeError):
+        rk.decompress_matvec_t_16(comp[:16], cb, x, out)             # stream too short
+    with pytest.raises(RuntimeError):
+        rk.decompress_matvec_t_16(comp, cb, torch.zeros(40000, dtype=torch.float16, device="cuda"), out)
+    assert rk.decompress_matvec_t_16(comp, cb, x, out) >= 0.0
