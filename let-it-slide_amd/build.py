@@ -12,6 +12,8 @@ FLAGS = [
     "-O3", "-std=c++17", "--offload-arch=gfx950", "-shared", "-fPIC",
     # hipcc must not form packed-fp32 instructions on this hardware pool
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # kernel arguments arrive in SGPRs at wave start instead of through a scalar load
+    "-mllvm", "-amdgpu-kernarg-preload-count=8",
     "-Wall", "-Wno-unused-function",
 ]
 

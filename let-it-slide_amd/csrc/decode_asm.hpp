@@ -1,0 +1,102 @@
+// The 32 steps of one stream element as one hand-scheduled instruction block.
+//
+// The compiler serialises "LDS gather, wait, multiply" per step; here the gathers of 8 steps are
+// in flight while the products of the previous 8 are formed, with explicit s_waitcnt.
+// Per 8 steps (one shift amount): 4 v_alignbit_b32 (none for shift 0), 4 v_pk_mad_u16 (two
+// window hashes each), 8 address ops (v_perm_b32 for the high window, v_and_or_b32 for the low
+// one), 8 ds_read_b32, 8 v_dot2c_f32_f16.
+#pragma once
+
+#include "rptc_common.hpp"
+
+namespace rptc {
+
+// hash, two addresses, two gathers for window register G (high window -> TH, low window -> TL)
+#define RPTC_RD2(G, TH, TL)                                   \
+    "v_perm_b32 " TH ", " G ", %[lane4], %[sel]\n"            \
+    "v_and_or_b32 " TL ", " G ", %[mask], %[lane4]\n"         \
+    "ds_read_b32 " TH ", " TH "\n"                            \
+    "ds_read_b32 " TL ", " TL "\n"
+
+#define RPTC_WINDOWS(SH)                                      \
+    "v_alignbit_b32 %[g0], %[cy], %[ex], " #SH "\n"           \
+    "v_alignbit_b32 %[g1], %[ex], %[ey], " #SH "\n"           \
+    "v_alignbit_b32 %[g2], %[ey], %[ez], " #SH "\n"           \
+    "v_alignbit_b32 %[g3], %[ez], %[ew], " #SH "\n"           \
+    "v_pk_mad_u16 %[g0], %[g0], %[g0], %[g0]\n"               \
+    "v_pk_mad_u16 %[g1], %[g1], %[g1], %[g1]\n"               \
+    "v_pk_mad_u16 %[g2], %[g2], %[g2], %[g2]\n"               \
+    "v_pk_mad_u16 %[g3], %[g3], %[g3], %[g3]\n"
+
+#define RPTC_WINDOWS_SH0                                      \
+    "v_pk_mad_u16 %[g0], %[ex], %[ex], %[ex]\n"               \
+    "v_pk_mad_u16 %[g1], %[ey], %[ey], %[ey]\n"               \
+    "v_pk_mad_u16 %[g2], %[ez], %[ez], %[ez]\n"               \
+    "v_pk_mad_u16 %[g3], %[ew], %[ew], %[ew]\n"
+
+#define RPTC_READS(T0, T1, T2, T3, T4, T5, T6, T7)            \
+    RPTC_RD2("%[g0]", T0, T1)                                 \
+    RPTC_RD2("%[g1]", T2, T3)                                 \
+    RPTC_RD2("%[g2]", T4, T5)                                 \
+    RPTC_RD2("%[g3]", T6, T7)
+
+// products of block j: {carry,x}: steps 28+j (high), j (low); {x,y}: 16+j, 4+j; {y,z}: 20+j, 8+j;
+// {z,w}: 24+j, 12+j
+#define RPTC_DOTS(T0, T1, T2, T3, T4, T5, T6, T7, XA, XB, XC, XD, XE, XF, XG, XH) \
+    "v_dot2c_f32_f16 %[a0], " T0 ", %[" XA "]\n"              \
+    "v_dot2c_f32_f16 %[a1], " T1 ", %[" XB "]\n"              \
+    "v_dot2c_f32_f16 %[a2], " T2 ", %[" XC "]\n"              \
+    "v_dot2c_f32_f16 %[a3], " T3 ", %[" XD "]\n"              \
+    "v_dot2c_f32_f16 %[a0], " T4 ", %[" XE "]\n"              \
+    "v_dot2c_f32_f16 %[a1], " T5 ", %[" XF "]\n"              \
+    "v_dot2c_f32_f16 %[a2], " T6 ", %[" XG "]\n"              \
+    "v_dot2c_f32_f16 %[a3], " T7 ", %[" XH "]\n"
+
+// one more expansion pass so that a register-list macro can stand for eight arguments
+#define RPTC_READS_X(...) RPTC_READS(__VA_ARGS__)
+#define RPTC_DOTS_X(...) RPTC_DOTS(__VA_ARGS__)
+
+#define RPTC_TA "%[t0]", "%[t1]", "%[t2]", "%[t3]", "%[t4]", "%[t5]", "%[t6]", "%[t7]"
+#define RPTC_TB "%[u0]", "%[u1]", "%[u2]", "%[u3]", "%[u4]", "%[u5]", "%[u6]", "%[u7]"
+
+// lane4: LDS address of this lane's copy of table row 0.  xr[q]: activation pair of step q.
+__device__ __forceinline__ void decode_element_asm(const uint4 e, const uint32_t carry, const uint32_t lane4,
+                                                   const uint32_t (&xr)[32], float &a0, float &a1, float &a2,
+                                                   float &a3)
+{
+    uint32_t g0, g1, g2, g3, t0, t1, t2, t3, t4, t5, t6, t7, u0, u1, u2, u3, u4, u5, u6, u7;
+    asm volatile(
+        RPTC_WINDOWS(12) RPTC_READS_X(RPTC_TA)
+        RPTC_WINDOWS(8) RPTC_READS_X(RPTC_TB)
+        "s_waitcnt lgkmcnt(8)\n"
+        RPTC_DOTS_X(RPTC_TA, "x28", "x0", "x16", "x4", "x20", "x8", "x24", "x12")
+        RPTC_WINDOWS(4) RPTC_READS_X(RPTC_TA)
+        "s_waitcnt lgkmcnt(8)\n"
+        RPTC_DOTS_X(RPTC_TB, "x29", "x1", "x17", "x5", "x21", "x9", "x25", "x13")
+        RPTC_WINDOWS_SH0 RPTC_READS_X(RPTC_TB)
+        "s_waitcnt lgkmcnt(8)\n"
+        RPTC_DOTS_X(RPTC_TA, "x30", "x2", "x18", "x6", "x22", "x10", "x26", "x14")
+        "s_waitcnt lgkmcnt(0)\n"
+        RPTC_DOTS_X(RPTC_TB, "x31", "x3", "x19", "x7", "x23", "x11", "x27", "x15")
+        // a dot product's result must not be read by another kind of VALU op for 3 wait states,
+        // and the compiler cannot see inside this block
+        "s_nop 3\n"
+        : [a0] "+v"(a0), [a1] "+v"(a1), [a2] "+v"(a2), [a3] "+v"(a3),
+          [g0] "=&v"(g0), [g1] "=&v"(g1), [g2] "=&v"(g2), [g3] "=&v"(g3),
+          [t0] "=&v"(t0), [t1] "=&v"(t1), [t2] "=&v"(t2), [t3] "=&v"(t3),
+          [t4] "=&v"(t4), [t5] "=&v"(t5), [t6] "=&v"(t6), [t7] "=&v"(t7),
+          [u0] "=&v"(u0), [u1] "=&v"(u1), [u2] "=&v"(u2), [u3] "=&v"(u3),
+          [u4] "=&v"(u4), [u5] "=&v"(u5), [u6] "=&v"(u6), [u7] "=&v"(u7)
+        : [ex] "v"(e.x), [ey] "v"(e.y), [ez] "v"(e.z), [ew] "v"(e.w), [cy] "v"(carry), [lane4] "v"(lane4),
+          [mask] "s"(0xFF00u), [sel] "s"(0x0C0C0700u),
+          [x0] "v"(xr[0]), [x1] "v"(xr[1]), [x2] "v"(xr[2]), [x3] "v"(xr[3]),
+          [x4] "v"(xr[4]), [x5] "v"(xr[5]), [x6] "v"(xr[6]), [x7] "v"(xr[7]),
+          [x8] "v"(xr[8]), [x9] "v"(xr[9]), [x10] "v"(xr[10]), [x11] "v"(xr[11]),
+          [x12] "v"(xr[12]), [x13] "v"(xr[13]), [x14] "v"(xr[14]), [x15] "v"(xr[15]),
+          [x16] "v"(xr[16]), [x17] "v"(xr[17]), [x18] "v"(xr[18]), [x19] "v"(xr[19]),
+          [x20] "v"(xr[20]), [x21] "v"(xr[21]), [x22] "v"(xr[22]), [x23] "v"(xr[23]),
+          [x24] "v"(xr[24]), [x25] "v"(xr[25]), [x26] "v"(xr[26]), [x27] "v"(xr[27]),
+          [x28] "v"(xr[28]), [x29] "v"(xr[29]), [x30] "v"(xr[30]), [x31] "v"(xr[31]));
+}
+
+}  // namespace rptc

@@ -18,7 +18,13 @@
 //     gather has no bank conflicts), and the pair product out of one v_dot2_f32_f16 with fp32
 //     accumulation: three vector ops per decoded pair;
 //   * every wave issues its stream loads before the table is built.
+#include "decode_asm.hpp"
 #include "rptc_common.hpp"
+
+// Development hook: a probe build defines RPTC_STAMP to record a per-wave timestamp at each phase.
+#ifndef RPTC_STAMP
+#define RPTC_STAMP(slot) ((void)0)
+#endif
 
 namespace rptc {
 
@@ -52,39 +58,12 @@ __device__ __forceinline__ uint32_t table_value(const uint32_t *__restrict__ cod
     return (pair & 0xFFFF7FFFu) | ((uint32_t)(b >> 7) << 15);
 }
 
-// One window register g = two windows 16 bits (4 steps) apart: hi half first in the stream.
-// lane4 = LDS address of the table + 4 * lane; the table starts on a 64 KiB boundary, so OR-ing
-// the row offset in equals adding it.
-__device__ __forceinline__ void two_steps(uint32_t g, uint32_t lane4, uint32_t x_hi, uint32_t x_lo,
-                                          float &acc_a, float &acc_b)
+// A stream element is read exactly once: load it with the non-temporal hint.
+__device__ __forceinline__ uint4 load_stream(const uint4 *p)
 {
-    const uint32_t h = pk_hash16(g);
-    const uint32_t a_lo = and_or(h, 0xFF00u, lane4);           // (byte 1 of h) << 8 | lane4
-    const uint32_t a_hi = perm(h, lane4, 0x0C0C0700u);         // (byte 3 of h) << 8 | lane4
-    acc_a = dot2(lds_read_abs(a_hi), x_hi, acc_a);
-    acc_b = dot2(lds_read_abs(a_lo), x_lo, acc_b);
-}
-
-// All 32 steps of one element.  xr[q], q = 4k + j, is the activation pair of step (k, j).
-__device__ __forceinline__ float decode_element(const uint4 e, const uint32_t carry, const uint32_t lane4,
-                                                const uint32_t (&xr)[32])
-{
-    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-        const uint32_t sh = 12 - 4 * j;
-        // {carry,x}: hi = step (k=7, j), lo = (k=0, j);  {x,y}: (4, j), (1, j);
-        // {y,z}: (5, j), (2, j);  {z,w}: (6, j), (3, j)        (inference.cu:237-250)
-        const uint32_t gc = j == 3 ? e.x : alignbit(carry, e.x, sh);
-        const uint32_t gx = j == 3 ? e.y : alignbit(e.x, e.y, sh);
-        const uint32_t gy = j == 3 ? e.z : alignbit(e.y, e.z, sh);
-        const uint32_t gz = j == 3 ? e.w : alignbit(e.z, e.w, sh);
-        two_steps(gc, lane4, xr[28 + j], xr[0 + j], a0, a1);
-        two_steps(gx, lane4, xr[16 + j], xr[4 + j], a2, a3);
-        two_steps(gy, lane4, xr[20 + j], xr[8 + j], a0, a1);
-        two_steps(gz, lane4, xr[24 + j], xr[12 + j], a2, a3);
-    }
-    return (a0 + a1) + (a2 + a3);
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p));
+    return make_uint4(v.x, v.y, v.z, v.w);
 }
 
 template <int S, int MODE>
@@ -93,53 +72,90 @@ __global__ __launch_bounds__(kMatvecThreads) void matvec_kernel(
     const uint4 *__restrict__ x, uint16_t *__restrict__ out, int m, int n, int rows_per_block)
 {
     extern __shared__ uint32_t lds[];
-    uint32_t *sx = lds + kTableBytes / 4;             // activation pairs, slot order
-    float *part = reinterpret_cast<float *>(sx + n / 2);   // [slab][row in block]
+    RPTC_STAMP(0);
+    uint32_t *sx = lds + kTableBytes / 4;                  // activation pairs, slot order
+    float *part = reinterpret_cast<float *>(sx + n / 2);   // [row in block][slab][32 lanes]
 
     const Geometry g(m, n);
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l = lane & 31, hw = lane >> 5;
-    // the table is the first thing in LDS; its address is 0 when the kernel has no static LDS
-    // (the low 32 bits of a flat pointer into LDS are the LDS address)
+    const int tid = threadIdx.x, lane = tid & 63, l = lane & 31, hw = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: keeps the item loop scalar
+    // The table is the first thing in LDS and the kernel has no static LDS, so it starts at LDS
+    // address 0 (the low 32 bits of a flat pointer into LDS are the LDS address); OR-ing a row
+    // offset into lane4 then equals adding it.
     const uint32_t lane4 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds)) + lane * 4;
     const int row0 = blockIdx.x * rows_per_block;
     const int rows = min(rows_per_block, m - row0);
     const int pairs = (rows + 1) >> 1;
-    const int items = g.slabs * pairs;                // item = slab * pairs + pair
+    const int items = g.slabs * pairs;                     // item = slab * pairs + pair
     const int per_wave = (items + kMatvecWaves - 1) / kMatvecWaves;
-    const int it_begin = wave * per_wave;
+    const int it_begin = min(items, wave * per_wave);
     const int it_end = min(items, it_begin + per_wave);
+
+    // (slab, pair) of the next item to load / to decode, advanced without dividing
+    int ld_slab = it_begin / pairs, ld_pair = it_begin - ld_slab * pairs;
+    int slab = ld_slab, pair = ld_pair;
+
+    // Loads are returned in issue order, so the small loads the table and the activation image
+    // wait for go first and the stream loads, which take longest, are issued right behind them.
+    constexpr int kTableWrites = kTableBytes / 16 / kMatvecThreads;     // 16-byte writes per thread
+    uint32_t cbv[kTableWrites];
+#pragma unroll
+    for (int i = 0; i < kTableWrites; i++) {
+        const int row = (i * kMatvecThreads + tid) >> 4;                // a table row is 16 uint4
+        cbv[i] = table_value<S>(codebook, row);
+    }
+    const int n8 = n >> 3;
+    constexpr int kXRegs = 2;
+    uint4 xv[kXRegs];
+#pragma unroll
+    for (int u = 0; u < kXRegs; u++) {
+        const int idx = tid + u * kMatvecThreads;
+        xv[u] = idx < n8 ? x[idx] : make_uint4(0, 0, 0, 0);
+    }
 
     uint4 buf[kBatch];
     uint32_t cw[kBatch];
     auto load_batch = [&](int base) {
 #pragma unroll
         for (int u = 0; u < kBatch; u++) {
-            const int it = base + u;
             buf[u] = make_uint4(0, 0, 0, 0);
             cw[u] = 0;
-            if (it < it_end) {
-                const int slab = it / pairs, row = 2 * (it - slab * pairs) + hw;
-                if (row < rows && l < g.lanes(slab)) {
-                    buf[u] = comp[g.elem(slab, row0 + row, l)];
-                    if (MODE == RPTC_CONTINUOUS && l == 0 && slab > 0)
-                        cw[u] = comp[g.elem(slab - 1, row0 + row, 31)].w;
+            if (base + u < it_end) {
+                const int row = 2 * ld_pair + hw;
+                if (row < rows && l < g.lanes(ld_slab)) {
+                    buf[u] = load_stream(comp + g.elem(ld_slab, row0 + row, l));
+                    if (MODE == RPTC_CONTINUOUS && l == 0 && ld_slab > 0)
+                        cw[u] = comp[g.elem(ld_slab - 1, row0 + row, 31)].w;
+                }
+                if (++ld_pair == pairs) {
+                    ld_pair = 0;
+                    ld_slab++;
                 }
             }
         }
     };
     load_batch(it_begin);
+    RPTC_STAMP(1);
 
-    // table and activations into LDS while the stream loads are in flight
-    for (int d = tid; d < kTableBytes / 4; d += kMatvecThreads) lds[d] = table_value<S>(codebook, d >> 6);
-    const int n8 = n >> 3;
-    for (int idx = tid; idx < n8; idx += kMatvecThreads) {
-        const uint4 v = x[idx];                       // halves 8idx .. 8idx+7 (inference.cu:215-221)
+    // table (256 rows x 64 lane copies) and activation image into LDS
+    uint4 *lds4 = reinterpret_cast<uint4 *>(lds);
+#pragma unroll
+    for (int i = 0; i < kTableWrites; i++)
+        lds4[i * kMatvecThreads + tid] = make_uint4(cbv[i], cbv[i], cbv[i], cbv[i]);
+    auto stage_x = [&](int idx, const uint4 v) {          // halves 8idx .. 8idx+7 (inference.cu:215-221)
         sx[idx] = v.x;
         sx[idx + n8] = v.y;
         sx[idx + 2 * n8] = v.z;
         sx[idx + 3 * n8] = v.w;
+    };
+#pragma unroll
+    for (int u = 0; u < kXRegs; u++) {
+        const int idx = tid + u * kMatvecThreads;
+        if (idx < n8) stage_x(idx, xv[u]);
     }
+    for (int idx = tid + kXRegs * kMatvecThreads; idx < n8; idx += kMatvecThreads) stage_x(idx, x[idx]);
     __syncthreads();
+    RPTC_STAMP(2);
 
     uint32_t xr[32];
     int cur_slab = -1;
@@ -154,36 +170,43 @@ __global__ __launch_bounds__(kMatvecThreads) void matvec_kernel(
         if (base + kBatch < it_end) load_batch(base + kBatch);
 #pragma unroll
         for (int u = 0; u < kBatch; u++) {
-            const int it = base + u;
-            if (it >= it_end) break;
-            const int slab = it / pairs, pair = it - slab * pairs, row = 2 * pair + hw;
+            if (base + u >= it_end) break;
+            const int row = 2 * pair + hw;
             const bool active = row < rows && l < g.lanes(slab);
             if (slab != cur_slab) {
                 cur_slab = slab;
-                const bool has = l < g.lanes(slab);
+                // lanes past a ragged slab's end read lane 0's pairs; their sums are dropped below
+                const int lx = l < g.lanes(slab) ? l : 0;
 #pragma unroll
-                for (int q = 0; q < 32; q++) xr[q] = has ? sx[g.slot(slab, q, l)] : 0u;
+                for (int q = 0; q < 32; q++) xr[q] = sx[g.slot(slab, q, lx)];
             }
-            // previous lane's last word; lane 0 of a row keeps its own as written
-            // (inference.cu:232: the shuffle returns the caller's value to lane 0)
-            uint32_t carry = __shfl_up(cur[u].w, 1, 32);
-            if (MODE == RPTC_CONTINUOUS && l == 0) carry = ccw[u];
-            float acc = decode_element(cur[u], carry, lane4, xr);
-            acc = active ? acc : 0.f;
-            acc += __shfl_xor(acc, 16, 32);
-            acc += __shfl_xor(acc, 8, 32);
-            acc += __shfl_xor(acc, 4, 32);
-            acc += __shfl_xor(acc, 2, 32);
-            acc += __shfl_xor(acc, 1, 32);
-            if (l == 0 && row < rows) part[slab * rows_per_block + row] = acc;
+            // Previous lane's last word.  Lane 0 of a row keeps its own as written
+            // (inference.cu:232: the shuffle hands lane 0 its own value back).
+            uint32_t carry = __builtin_amdgcn_update_dpp(0u, cur[u].w, 0x138 /* wave_shr:1 */, 0xF, 0xF, false);
+            if (l == 0) carry = MODE == RPTC_CONTINUOUS ? ccw[u] : cur[u].w;
+            float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+            decode_element_asm(cur[u], carry, lane4, xr, a0, a1, a2, a3);
+            const float acc = (a0 + a1) + (a2 + a3);
+            if (row < rows) part[((row * g.slabs) + slab) * 32 + l] = active ? acc : 0.f;
+            if (base + u == it_begin) RPTC_STAMP(3);
+            if (++pair == pairs) {
+                pair = 0;
+                slab++;
+            }
         }
     }
+    RPTC_STAMP(4);
     __syncthreads();
-    for (int r = tid; r < rows; r += kMatvecThreads) {
+    // one wave per row: add the row's slabs * 32 partial sums in a fixed order
+    const int per_row = g.slabs * 32;
+    for (int r = wave; r < rows; r += kMatvecWaves) {
         float y = 0.f;
-        for (int t = 0; t < g.slabs; t++) y += part[t * rows_per_block + r];
-        out[row0 + r] = float_to_half_bits(y);
+        for (int i = lane; i < per_row; i += kWave) y += part[r * per_row + i];
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) y += __shfl_xor(y, off, 64);
+        if (lane == 0) out[row0 + r] = float_to_half_bits(y);
     }
+    RPTC_STAMP(5);
 }
 
 // Dense export: one thread per stream element, 32 pairs scattered to their columns.
@@ -224,7 +247,7 @@ __global__ __launch_bounds__(256) void matvec_dense_kernel(
 
 static int matvec_lds_bytes(int n, int slabs, int rows_per_block)
 {
-    return kTableBytes + 2 * n + 4 * slabs * rows_per_block;
+    return kTableBytes + 2 * n + 4 * slabs * rows_per_block * 32;
 }
 
 template <int S>
@@ -241,9 +264,14 @@ static int launch_matvec(const int32_t *compressed, const uint16_t *codebook, co
     int rc = device_info(&dev);
     if (rc) return rc;
     const Geometry g((int)m, (int)n);
+    // one workgroup per CU when the per-row partial sums fit in LDS beside the table and the
+    // activations, else as many rows per workgroup as do fit
     int rows_per_block = 2 * (int)((m + 2 * dev->cus - 1) / (2 * dev->cus));
+    const int fixed_bytes = matvec_lds_bytes((int)n, g.slabs, 0);
+    if (fixed_bytes + 2 * 128 * g.slabs > kMaxLds) return RPTC_ELIMIT;
+    const int fit_rows = ((kMaxLds - fixed_bytes) / (128 * g.slabs)) & ~1;
+    if (rows_per_block > fit_rows) rows_per_block = fit_rows;
     const int lds_bytes = matvec_lds_bytes((int)n, g.slabs, rows_per_block);
-    if (lds_bytes > kMaxLds) return RPTC_ELIMIT;
     const int grid = (int)((m + rows_per_block - 1) / rows_per_block);
 
     hipStream_t s = static_cast<hipStream_t>(stream);
