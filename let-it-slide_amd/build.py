@@ -13,7 +13,7 @@ FLAGS = [
     # hipcc must not form packed-fp32 instructions on this hardware pool
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     # kernel arguments arrive in SGPRs at wave start instead of through a scalar load
-    "-mllvm", "-amdgpu-kernarg-preload-count=8",
+    "-mllvm", "-amdgpu-kernarg-preload-count=16",
     "-Wall", "-Wno-unused-function",
 ]
 

@@ -7,17 +7,21 @@
 // sign of the pair's first value) and multiplies the pair with two activations.
 //
 // gfx950 design (not the reference's):
-//   * one workgroup of 16 waves per CU, each owning a block of rows and every slab of those
-//     rows, so the sum over slabs stays inside the workgroup and is added in a fixed order;
-//   * a half-wave (32 lanes) is one row of one slab, exactly one 512-byte line of the stream;
-//     a wave keeps a slab's 32 activation pairs per lane in registers and walks row pairs, so
-//     activations cost one LDS read per 2*R rows instead of one per step;
+//   * one workgroup of 16 waves per CU owns a block of rows and every slab of those rows, so the
+//     sum over slabs stays inside the workgroup and is added in a fixed order (deterministic);
+//   * a wave item is 64 consecutive stream elements (1 KiB, one coalesced 16-byte load per lane):
+//     two rows of a full slab, or floor(64 / Lt) rows of the ragged last slab.  Its address is a
+//     wave-uniform base plus 16 bytes per lane, so addressing costs scalar instructions only;
+//   * a wave keeps a slab's 32 activation pairs per lane in registers and walks consecutive
+//     items of that slab, so activations cost one LDS read per slab change, not one per step;
 //   * two adjacent windows come out of one v_alignbit_b32, both hashes out of one
 //     v_pk_mad_u16, the LDS address out of one v_and_or_b32 / v_perm_b32 (hash byte 1 is the
-//     row of a 256-entry table whose sign is already applied, replicated once per lane so the
-//     gather has no bank conflicts), and the pair product out of one v_dot2_f32_f16 with fp32
-//     accumulation: three vector ops per decoded pair;
-//   * every wave issues its stream loads before the table is built.
+//     row of a 256-row table whose sign is already applied, replicated once per lane so the
+//     gather has no bank conflicts), and the pair product out of one v_dot2c_f32_f16 with fp32
+//     accumulation: about three vector ops per decoded pair, hand-scheduled in decode_asm.hpp;
+//   * loads return in issue order, so the small loads that the table and the activation image
+//     wait for are issued first and every wave's stream loads right behind them, before the
+//     table is built; kernel arguments are preloaded into SGPRs.
 #include "decode_asm.hpp"
 #include "rptc_common.hpp"
 
@@ -58,42 +62,56 @@ __device__ __forceinline__ uint32_t table_value(const uint32_t *__restrict__ cod
     return (pair & 0xFFFF7FFFu) | ((uint32_t)(b >> 7) << 15);
 }
 
-// A stream element is read exactly once: load it with the non-temporal hint.
-__device__ __forceinline__ uint4 load_stream(const uint4 *p)
+// A stream element is read exactly once: load it with the non-temporal hint.  The address is a
+// wave-uniform base plus 16 bytes per lane, so no vector address arithmetic is needed.
+__device__ __forceinline__ uint4 load_stream(const uint4 *wave_base, int lane)
 {
     typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-    const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p));
+    const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(wave_base) + lane);
     return make_uint4(v.x, v.y, v.z, v.w);
 }
+
+// What a wave needs to know about the slab it is working on.  A wave item is 64 consecutive
+// stream elements of one slab: rows_per_item whole rows of `lanes` elements each (2 rows of 32
+// in a full slab; floor(64 / Lt) rows in the ragged last slab).
+struct SlabView {
+    int lanes;            // elements per row
+    int rows_per_item;
+    int items;            // items of this slab in a workgroup
+    int part_off;         // where this slab's partial sums start inside a row's run
+    size_t elem0;         // index of element (slab, row 0 of the matrix, lane 0)
+};
+
+struct MatvecArgs {
+    int m, n, rows_per_block;
+    int rw_tail;          // rows per item in the ragged slab
+    int items_full;       // items per full slab per workgroup   = rows_per_block / 2
+    int items_tail;       // items of the ragged slab            = ceil(rows_per_block / rw_tail)
+};
 
 template <int S, int MODE>
 __global__ __launch_bounds__(kMatvecThreads) void matvec_kernel(
     const uint4 *__restrict__ comp, const uint32_t *__restrict__ codebook,
-    const uint4 *__restrict__ x, uint16_t *__restrict__ out, int m, int n, int rows_per_block)
+    const uint4 *__restrict__ x, uint16_t *__restrict__ out, int arg_m, int arg_n, int arg_rows_per_block,
+    int arg_rw_tail, int arg_items_full, int arg_items_tail)
 {
+    // separate scalar arguments (not a struct) so that all of them are preloaded into SGPRs
+    const MatvecArgs a = {arg_m, arg_n, arg_rows_per_block, arg_rw_tail, arg_items_full, arg_items_tail};
     extern __shared__ uint32_t lds[];
     RPTC_STAMP(0);
+    const int m = a.m, n = a.n;
+    const int T = n >> 11, Lt = (n & 2047) >> 6, npr = n >> 6, n8 = n >> 3;
     uint32_t *sx = lds + kTableBytes / 4;                  // activation pairs, slot order
-    float *part = reinterpret_cast<float *>(sx + n / 2);   // [row in block][slab][32 lanes]
+    float *part = reinterpret_cast<float *>(sx + (n >> 1));   // [row in block][n / 64]
 
-    const Geometry g(m, n);
-    const int tid = threadIdx.x, lane = tid & 63, l = lane & 31, hw = lane >> 5;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: keeps the item loop scalar
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: keeps control flow scalar
     // The table is the first thing in LDS and the kernel has no static LDS, so it starts at LDS
     // address 0 (the low 32 bits of a flat pointer into LDS are the LDS address); OR-ing a row
     // offset into lane4 then equals adding it.
     const uint32_t lane4 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds)) + lane * 4;
-    const int row0 = blockIdx.x * rows_per_block;
-    const int rows = min(rows_per_block, m - row0);
-    const int pairs = (rows + 1) >> 1;
-    const int items = g.slabs * pairs;                     // item = slab * pairs + pair
-    const int per_wave = (items + kMatvecWaves - 1) / kMatvecWaves;
-    const int it_begin = min(items, wave * per_wave);
-    const int it_end = min(items, it_begin + per_wave);
-
-    // (slab, pair) of the next item to load / to decode, advanced without dividing
-    int ld_slab = it_begin / pairs, ld_pair = it_begin - ld_slab * pairs;
-    int slab = ld_slab, pair = ld_pair;
+    const int row0 = blockIdx.x * a.rows_per_block;
+    const int rows = min(a.rows_per_block, m - row0);
 
     // Loads are returned in issue order, so the small loads the table and the activation image
     // wait for go first and the stream loads, which take longest, are issued right behind them.
@@ -104,7 +122,6 @@ __global__ __launch_bounds__(kMatvecThreads) void matvec_kernel(
         const int row = (i * kMatvecThreads + tid) >> 4;                // a table row is 16 uint4
         cbv[i] = table_value<S>(codebook, row);
     }
-    const int n8 = n >> 3;
     constexpr int kXRegs = 2;
     uint4 xv[kXRegs];
 #pragma unroll
@@ -113,6 +130,30 @@ __global__ __launch_bounds__(kMatvecThreads) void matvec_kernel(
         xv[u] = idx < n8 ? x[idx] : make_uint4(0, 0, 0, 0);
     }
 
+    // This wave's items: a contiguous piece of [slab 0 items][slab 1 items]...[ragged slab items].
+    const int total = T * a.items_full + a.items_tail;
+    const int per_wave = (total + kMatvecWaves - 1) / kMatvecWaves;
+    const int it_begin = min(total, wave * per_wave);
+    const int it_end = min(total, it_begin + per_wave);
+    auto view = [&](int slab) {
+        SlabView v;
+        const bool full = slab < T;
+        v.lanes = full ? 32 : Lt;
+        v.rows_per_item = full ? 2 : a.rw_tail;
+        v.items = full ? a.items_full : a.items_tail;
+        v.part_off = slab * 32;
+        v.elem0 = full ? (size_t)slab * m * 32 : (size_t)T * m * 32;
+        return v;
+    };
+    int first_slab = 0, first_idx = it_begin;              // no divide: walk the few slabs
+    while (first_slab < T && first_idx >= a.items_full) {
+        first_idx -= a.items_full;
+        first_slab++;
+    }
+
+    // cursor of the loads and cursor of the decode (slab, item index inside the slab)
+    int ld_slab = first_slab, ld_idx = first_idx;
+    SlabView ld = view(ld_slab);
     uint4 buf[kBatch];
     uint32_t cw[kBatch];
     auto load_batch = [&](int base) {
@@ -121,15 +162,23 @@ __global__ __launch_bounds__(kMatvecThreads) void matvec_kernel(
             buf[u] = make_uint4(0, 0, 0, 0);
             cw[u] = 0;
             if (base + u < it_end) {
-                const int row = 2 * ld_pair + hw;
-                if (row < rows && l < g.lanes(ld_slab)) {
-                    buf[u] = load_stream(comp + g.elem(ld_slab, row0 + row, l));
-                    if (MODE == RPTC_CONTINUOUS && l == 0 && ld_slab > 0)
-                        cw[u] = comp[g.elem(ld_slab - 1, row0 + row, 31)].w;
+                const int row_first = ld_idx * ld.rows_per_item;           // row inside the block
+                const int rows_here = min(ld.rows_per_item, rows - row_first);
+                if (lane < rows_here * ld.lanes) {
+                    const uint4 *wave_base = comp + ld.elem0 + (size_t)(row0 + row_first) * ld.lanes;
+                    buf[u] = load_stream(wave_base, lane);
+                    if (MODE == RPTC_CONTINUOUS && ld_slab > 0) {
+                        // the word in front of a row: last word of the row's lane 31 in the slab before
+                        const int sub = ld_slab < T ? lane >> 5 : lane / ld.lanes;
+                        const int l = lane - sub * ld.lanes;
+                        if (l == 0)
+                            cw[u] = comp[((size_t)(ld_slab - 1) * m + row0 + row_first + sub) * 32 + 31].w;
+                    }
                 }
-                if (++ld_pair == pairs) {
-                    ld_pair = 0;
+                if (++ld_idx == ld.items) {
+                    ld_idx = 0;
                     ld_slab++;
+                    ld = view(ld_slab);
                 }
             }
         }
@@ -158,7 +207,10 @@ __global__ __launch_bounds__(kMatvecThreads) void matvec_kernel(
     RPTC_STAMP(2);
 
     uint32_t xr[32];
-    int cur_slab = -1;
+    int slab = first_slab, idx = first_idx, cur_slab = -1;
+    SlabView sv = view(slab);
+    int l = 0, sub = 0;                     // this lane's element inside a row, row inside the item
+    uint32_t part_lane = 0;                 // LDS byte address of this lane's partial for row 0
     for (int base = it_begin; base < it_end; base += kBatch) {
         uint4 cur[kBatch];
         uint32_t ccw[kBatch];
@@ -171,40 +223,59 @@ __global__ __launch_bounds__(kMatvecThreads) void matvec_kernel(
 #pragma unroll
         for (int u = 0; u < kBatch; u++) {
             if (base + u >= it_end) break;
-            const int row = 2 * pair + hw;
-            const bool active = row < rows && l < g.lanes(slab);
             if (slab != cur_slab) {
                 cur_slab = slab;
-                // lanes past a ragged slab's end read lane 0's pairs; their sums are dropped below
-                const int lx = l < g.lanes(slab) ? l : 0;
+                // lane -> (row inside the item, element inside the row); lanes past the last whole
+                // row of a ragged item idle on element 0
+                if (slab < T) {
+                    sub = lane >> 5;
+                    l = lane & 31;
+                } else {
+                    sub = lane / sv.lanes;
+                    l = lane - sub * sv.lanes;
+                    if (sub >= sv.rows_per_item) l = 0;
+                }
+                // step q of element l multiplies pair slot(slab, q, l) (inference.cu:249)
+                const uint32_t *xp = sx + (slab < T ? 1024 * slab : 1024 * T) + l;
+                if (slab < T) {
 #pragma unroll
-                for (int q = 0; q < 32; q++) xr[q] = sx[g.slot(slab, q, lx)];
+                    for (int q = 0; q < 32; q++) xr[q] = xp[32 * q];
+                } else {
+#pragma unroll
+                    for (int q = 0; q < 32; q++) xr[q] = xp[q * sv.lanes];
+                }
+                part_lane = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(part)) +
+                            4u * (uint32_t)(sub * npr + sv.part_off + l);
             }
+            const int row_first = idx * sv.rows_per_item;
+            const bool active = sub < sv.rows_per_item && row_first + sub < rows;
             // Previous lane's last word.  Lane 0 of a row keeps its own as written
             // (inference.cu:232: the shuffle hands lane 0 its own value back).
             uint32_t carry = __builtin_amdgcn_update_dpp(0u, cur[u].w, 0x138 /* wave_shr:1 */, 0xF, 0xF, false);
             if (l == 0) carry = MODE == RPTC_CONTINUOUS ? ccw[u] : cur[u].w;
             float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
             decode_element_asm(cur[u], carry, lane4, xr, a0, a1, a2, a3);
-            const float acc = (a0 + a1) + (a2 + a3);
-            if (row < rows) part[((row * g.slabs) + slab) * 32 + l] = active ? acc : 0.f;
+            if (active) {
+                typedef __attribute__((address_space(3))) float lds_float;
+                *reinterpret_cast<lds_float *>(static_cast<uintptr_t>(part_lane + 4u * (uint32_t)(row_first * npr))) =
+                    (a0 + a1) + (a2 + a3);
+            }
             if (base + u == it_begin) RPTC_STAMP(3);
-            if (++pair == pairs) {
-                pair = 0;
+            if (++idx == sv.items) {
+                idx = 0;
                 slab++;
+                sv = view(slab);
             }
         }
     }
     RPTC_STAMP(4);
     __syncthreads();
-    // one wave per row: add the row's slabs * 32 partial sums in a fixed order
-    const int per_row = g.slabs * 32;
+    // one wave per row: add the row's n / 64 partial sums in a fixed order
     for (int r = wave; r < rows; r += kMatvecWaves) {
         float y = 0.f;
-        for (int i = lane; i < per_row; i += kWave) y += part[r * per_row + i];
-#pragma unroll
-        for (int off = 32; off > 0; off >>= 1) y += __shfl_xor(y, off, 64);
-        if (lane == 0) out[row0 + r] = float_to_half_bits(y);
+        for (int i = lane; i < npr; i += kWave) y += part[r * npr + i];
+        y = wave_sum(y);
+        if (lane == 63) out[row0 + r] = float_to_half_bits(y);
     }
     RPTC_STAMP(5);
 }
@@ -245,9 +316,9 @@ __global__ __launch_bounds__(256) void matvec_dense_kernel(
     }
 }
 
-static int matvec_lds_bytes(int n, int slabs, int rows_per_block)
+static int matvec_lds_bytes(int n, int rows_per_block)
 {
-    return kTableBytes + 2 * n + 4 * slabs * rows_per_block * 32;
+    return kTableBytes + 2 * n + 4 * (n / 64) * rows_per_block;
 }
 
 template <int S>
@@ -263,16 +334,23 @@ static int launch_matvec(const int32_t *compressed, const uint16_t *codebook, co
     DeviceInfo *dev;
     int rc = device_info(&dev);
     if (rc) return rc;
-    const Geometry g((int)m, (int)n);
     // one workgroup per CU when the per-row partial sums fit in LDS beside the table and the
     // activations, else as many rows per workgroup as do fit
-    int rows_per_block = 2 * (int)((m + 2 * dev->cus - 1) / (2 * dev->cus));
-    const int fixed_bytes = matvec_lds_bytes((int)n, g.slabs, 0);
-    if (fixed_bytes + 2 * 128 * g.slabs > kMaxLds) return RPTC_ELIMIT;
-    const int fit_rows = ((kMaxLds - fixed_bytes) / (128 * g.slabs)) & ~1;
-    if (rows_per_block > fit_rows) rows_per_block = fit_rows;
-    const int lds_bytes = matvec_lds_bytes((int)n, g.slabs, rows_per_block);
-    const int grid = (int)((m + rows_per_block - 1) / rows_per_block);
+    MatvecArgs a;
+    a.m = (int)m;
+    a.n = (int)n;
+    a.rows_per_block = 2 * (int)((m + 2 * dev->cus - 1) / (2 * dev->cus));
+    const int fixed_bytes = matvec_lds_bytes(a.n, 0);
+    const int row_bytes = 4 * (a.n / 64);
+    if (fixed_bytes + 2 * row_bytes > kMaxLds) return RPTC_ELIMIT;
+    const int fit_rows = ((kMaxLds - fixed_bytes) / row_bytes) & ~1;
+    if (a.rows_per_block > fit_rows) a.rows_per_block = fit_rows;
+    const int lt = (a.n & 2047) >> 6;
+    a.rw_tail = lt ? 64 / lt : 1;
+    a.items_full = a.rows_per_block / 2;
+    a.items_tail = lt ? (a.rows_per_block + a.rw_tail - 1) / a.rw_tail : 0;
+    const int lds_bytes = matvec_lds_bytes(a.n, a.rows_per_block);
+    const int grid = (int)((m + a.rows_per_block - 1) / a.rows_per_block);
 
     hipStream_t s = static_cast<hipStream_t>(stream);
     Timer t;
@@ -283,10 +361,10 @@ static int launch_matvec(const int32_t *compressed, const uint16_t *codebook, co
     auto a_x = reinterpret_cast<const uint4 *>(x);
     if (carry_mode == RPTC_AS_WRITTEN)
         hipLaunchKernelGGL((matvec_kernel<S, RPTC_AS_WRITTEN>), dim3(grid), dim3(kMatvecThreads), lds_bytes, s,
-                           a_comp, a_cb, a_x, out, (int)m, (int)n, rows_per_block);
+                           a_comp, a_cb, a_x, out, a.m, a.n, a.rows_per_block, a.rw_tail, a.items_full, a.items_tail);
     else
         hipLaunchKernelGGL((matvec_kernel<S, RPTC_CONTINUOUS>), dim3(grid), dim3(kMatvecThreads), lds_bytes, s,
-                           a_comp, a_cb, a_x, out, (int)m, (int)n, rows_per_block);
+                           a_comp, a_cb, a_x, out, a.m, a.n, a.rows_per_block, a.rw_tail, a.items_full, a.items_tail);
     return t.end();
 }
 

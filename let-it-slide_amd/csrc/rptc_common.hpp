@@ -99,6 +99,23 @@ __device__ __forceinline__ float dot2(uint32_t w, uint32_t a, float acc)
     return __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, w), __builtin_bit_cast(half2_t, a), acc, false);
 }
 
+// Sum over the 64 lanes of a wave with DPP adds only (no LDS traffic); the total ends up in
+// lane 63.  Steps: within rows of 16 lanes, then row 0 into 1 and 2 into 3, then rows 0-1 into 2-3.
+__device__ __forceinline__ float wave_sum(float v)
+{
+#define RPTC_DPP_ADD(ctrl, row_mask, bank_mask)                                                      \
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0u, __builtin_bit_cast(uint32_t, v), \
+                                                               ctrl, row_mask, bank_mask, false))
+    RPTC_DPP_ADD(0x111, 0xF, 0xF);   // row_shr:1
+    RPTC_DPP_ADD(0x112, 0xF, 0xF);   // row_shr:2
+    RPTC_DPP_ADD(0x114, 0xF, 0xF);   // row_shr:4
+    RPTC_DPP_ADD(0x118, 0xF, 0xF);   // row_shr:8   -> lane 15 of each row holds the row's sum
+    RPTC_DPP_ADD(0x142, 0xA, 0xF);   // row_bcast:15 into rows 1 and 3
+    RPTC_DPP_ADD(0x143, 0xC, 0xF);   // row_bcast:31 into rows 2 and 3
+#undef RPTC_DPP_ADD
+    return v;
+}
+
 __device__ __forceinline__ uint16_t float_to_half_bits(float f)
 {
     _Float16 h = (_Float16)f;   // v_cvt_f16_f32, round to nearest even
