@@ -26,6 +26,10 @@ for p in (ROOT, os.path.join(ROOT, "let-it-slide_amd")):
 
 HBM_PEAK_GBS = 8000.0
 
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a copy kernel
+# of known size; the runs are summarised under profiles/).  Keyed by (m, n, S); other workloads report null.
+MEASURED_TRAFFIC_BYTES = {(4096, 11008, 8): 11610000}
+
 
 def parse():
     ap = argparse.ArgumentParser()
@@ -39,6 +43,9 @@ def parse():
     ap.add_argument("--launch", choices=("graph", "direct"), default="graph",
                     help="graph: the timed steps are one captured HIP graph; direct: one host call per step")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--pmc-probe", action="store_true",
+                    help="for `rocprofv3 --pmc`: a few direct launches of the kernel plus a plain device copy of "
+                         "known size (the calibration for FETCH_SIZE / WRITE_SIZE); prints no benchmark line")
     ap.add_argument("--extra-shapes", action="store_true", help="also time the other layer shapes")
     return ap.parse_args()
 
@@ -157,6 +164,19 @@ def main():
         sys.exit(1)
     torch.cuda.set_device(0)
     runner = Runner(a.m, a.n, a.S, a.copies)
+    if a.pmc_probe:
+        # calibration: an int32 -> float32 conversion copy is a plain streaming kernel that reads
+        # 64 MiB and writes 64 MiB
+        src = torch.randint(0, 1 << 20, (16 << 20,), dtype=torch.int32, device="cuda")
+        dst = torch.empty(16 << 20, dtype=torch.float32, device="cuda")
+        stream = torch.cuda.current_stream().cuda_stream
+        for k in range(8):
+            dst.copy_(src)
+            runner.launch(k, stream)
+        torch.cuda.synchronize()
+        print(f"pmc-probe: 8 conversion copies of {src.numel() * 4} bytes in / {dst.numel() * 4} bytes out "
+              f"and 8 launches of {runner.bytes} compressed bytes")
+        return
     err = runner.check()
     wall, ev_ms = runner.run(a.steps, a.warmup, a.launch)
     ms_per_step = wall * 1e3 / a.steps
@@ -191,7 +211,7 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4),
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC_BYTES.get((a.m, a.n, a.S)),
             "launch_us": round(launch_ms * 1e3, 3),
         },
     }
