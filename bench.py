@@ -47,6 +47,8 @@ def parse():
                     help="for `rocprofv3 --pmc`: a few direct launches of the kernel plus a plain device copy of "
                          "known size (the calibration for FETCH_SIZE / WRITE_SIZE); prints no benchmark line")
     ap.add_argument("--extra-shapes", action="store_true", help="also time the other layer shapes")
+    ap.add_argument("--matmul", action="store_true",
+                    help="time the batch 8/16/32 fused decode + MFMA mat-mat instead (prints its own JSON line)")
     return ap.parse_args()
 
 
@@ -153,6 +155,77 @@ def cpu_baseline(runner, min_seconds=8.0):
             "ms_per_pass": round(dt / reps * 1e3, 3)}
 
 
+MFMA_F16_PEAK_TFLOPS = 2516.6
+
+
+def bench_matmul(a):
+    """Batch 8/16/32 fused decode + mat-mat on the same layer, next to decode-then-dense-GEMM
+    (dense export kernel + torch.matmul on the decoded fp16 matrix)."""
+    import torch
+    import rptc_kernels
+    lib = rptc_kernels.library()
+    rptc_kernels.set_timing(False)
+    m, n, S = a.m, a.n, a.S
+    g = torch.Generator(device="cuda")
+    g.manual_seed(42)
+    words = m * n // 16
+    copies = max(2, min(a.copies, (512 << 20) // (words * 4) + 1))
+    weights = [torch.randint(-(1 << 31), 1 << 31, (words,), generator=g, dtype=torch.int64, device="cuda").to(torch.int32)
+               for _ in range(copies)]
+    cb = torch.randn(2 << S, generator=g, device="cuda").to(torch.float16)
+    W = torch.zeros((m, n), dtype=torch.float16, device="cuda")
+    results = {}
+    for batch in (8, 16, 32):
+        x = torch.randn((batch, n), generator=g, device="cuda").to(torch.float16)
+        out = torch.zeros((batch, m), dtype=torch.float16, device="cuda")
+        fn = getattr(rptc_kernels, f"decompress_matmul_16_{S}_1")
+
+        def fused(k):
+            fn(weights[k % copies], cb, x, out)
+
+        def baseline(k):
+            rptc_kernels.matvec_dense(weights[k % copies], cb, W, S)
+            torch.matmul(x, W.t(), out=out)
+
+        times = {}
+        for name, step in (("fused", fused), ("decode_then_gemm", baseline)):
+            for k in range(10):
+                step(k)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            steps = min(a.steps, 200)
+            with torch.cuda.graph(graph):
+                for k in range(steps):
+                    step(k)
+            graph.replay()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            graph.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            times[name] = e0.elapsed_time(e1) / steps * 1e3          # us per call
+        fused(0)
+        rptc_kernels.matvec_dense(weights[0], cb, W, S)
+        torch.cuda.synchronize()
+        want = x.double() @ W.double().t()
+        err = ((out.double() - want).norm() / want.norm()).item()
+        flops = 2.0 * m * n * batch
+        us = times["fused"]
+        results[f"batch{batch}"] = {
+            "us": round(us, 2), "TFLOPs": round(flops / us / 1e6, 2),
+            "mfma_util": round(flops / us / 1e6 / MFMA_F16_PEAK_TFLOPS, 5),
+            "hbm_GBps": round(m * n / 4 / us / 1e3, 1), "hbm_frac": round(m * n / 4 / us / 1e3 / HBM_PEAK_GBS, 4),
+            "decode_then_gemm_us": round(times["decode_then_gemm"], 2),
+            "speedup_vs_decode_then_gemm": round(times["decode_then_gemm"] / us, 2),
+            "rel_l2_vs_dense": float(f"{err:.3e}"),
+        }
+    print(json.dumps({"metric": "fused decode+GEMM (MFMA) per call", "unit": "us", "n_gpus": 1,
+                      "config": {"workload": f"decompress_matmul_16_{S}_1 m={m} n={n} 2 bits/weight, {copies} rotating "
+                                             f"weight copies", "launch": "graph"},
+                      "results": results}))
+
+
 def main():
     a = parse()
     if a.gpus != 1:
@@ -163,6 +236,9 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
     torch.cuda.set_device(0)
+    if a.matmul:
+        bench_matmul(a)
+        return
     runner = Runner(a.m, a.n, a.S, a.copies)
     if a.pmc_probe:
         # calibration: an int32 -> float32 conversion copy is a plain streaming kernel that reads

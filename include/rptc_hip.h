@@ -121,6 +121,19 @@ int rptc_matvec_dense(const int32_t *compressed, const uint16_t *codebook, uint1
 int rptc_matvec_t_dense(const int32_t *compressed, const uint16_t *codebook, uint16_t *W,
                         int64_t m, int64_t n, int L, int carry_mode, void *stream, float *ms);
 
+/*
+ * Fused decode + small-batch mat-mat on the hashed pair stream (the stream, codebook and dense
+ * matrix W of rptc_decompress_matvec_*; S in {6, 8}):  out[b][r] = sum_c W[r][c] * x[b][c].
+ * No counterpart in the reference, which only has the batch-1 kernels (inference.cu:189-277).
+ *   x    fp16 [batch][n], batch in [1, 32], n % 64 == 0, n <= 32768
+ *   out  fp16 [batch][m], overwritten
+ * fp16 products accumulated in fp32 on the matrix cores, rounded once.  The call stages the
+ * activations in a static device buffer: calls on different streams of one device must not overlap.
+ */
+int rptc_decompress_matmul(const int32_t *compressed, const uint16_t *codebook, const uint16_t *x,
+                           uint16_t *out, int64_t m, int64_t n, int64_t batch, int S, int carry_mode,
+                           void *stream, float *ms);
+
 #ifdef __cplusplus
 }
 #endif

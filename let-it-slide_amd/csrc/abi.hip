@@ -9,6 +9,7 @@ namespace rptc {
 int prepare_decompress();
 int prepare_matvec();
 int prepare_matvec_t();
+int prepare_matmul(int device);
 
 constexpr int kMaxDevices = 64;
 static DeviceInfo g_devices[kMaxDevices];
@@ -35,6 +36,7 @@ int device_info(DeviceInfo **out)
         if ((rc = prepare_decompress())) return rc;
         if ((rc = prepare_matvec())) return rc;
         if ((rc = prepare_matvec_t())) return rc;
+        if ((rc = prepare_matmul(dev))) return rc;
         g_ready[dev] = true;
     }
     *out = &g_devices[dev];

@@ -51,6 +51,7 @@ _SIGNATURES = {
     "rptc_decompress_matvec_t_14": (_MATVEC_ARGS, _INT),
     "rptc_matvec_dense": ([_VP, _VP, _VP, _I64, _I64, _INT, _INT, _VP, _FP], _INT),
     "rptc_matvec_t_dense": ([_VP, _VP, _VP, _I64, _I64, _INT, _INT, _VP, _FP], _INT),
+    "rptc_decompress_matmul": ([_VP, _VP, _VP, _VP, _I64, _I64, _I64, _INT, _INT, _VP, _FP], _INT),
 }
 
 
@@ -269,3 +270,35 @@ def matvec_t_dense(compressed, codebook, out, L):
     _check(n % 64 == 0 and m >= 1 and n >= 64, "out.size(1) % 64 == 0")
     _check(compressed.numel() * 16 >= m * n, "compressed holds fewer than m*n/16 words")
     return _call(library().rptc_matvec_t_dense, (compressed, codebook, out), m, n, L)
+
+
+def _matmul(S, compressed, codebook, x, out):
+    _check_input(compressed, "compressed")
+    _check(compressed.dtype == torch.int32, "compressed.scalar_type() == torch::kInt32")
+    _check_input(x, "x")
+    _check(x.dim() == 2, "x.dim() == 2 ([batch, n])")
+    _check(x.dtype == torch.float16, "x.scalar_type() == torch::kFloat16")
+    _check_input(out, "out")
+    _check(out.dim() == 2, "out.dim() == 2 ([batch, m])")
+    _check(out.dtype == torch.float16, "out.scalar_type() == torch::kFloat16")
+    batch, n = x.shape
+    _check(out.size(0) == batch, "out.size(0) == x.size(0)")
+    m = out.size(1)
+    _check(1 <= batch <= 32, "1 <= batch <= 32")
+    _check(n % 64 == 0 and n >= 64 and m >= 1, "x.size(1) % 64 == 0")
+    _check(n <= 32768, "x.size(1) <= 32768")
+    _check(compressed.numel() * 16 == m * n, "compressed.numel() * 16 == m * n")
+    _check_input(codebook, "codebook")
+    _check(codebook.dim() == 1 and codebook.size(0) == 1 << (S + 1), "codebook.size(0) == 1<<(S+V)")
+    _check(codebook.dtype == torch.float16, "codebook.scalar_type() == torch::kFloat16")
+    return _call(library().rptc_decompress_matmul, (compressed, codebook, x, out), m, n, batch, S)
+
+
+def decompress_matmul_16_6_1(compressed, codebook, x, out):
+    """out[b] = W x[b] for batch 1..32 on the hashed-codebook stream with 64 pairs; x [batch, n], out [batch, m]."""
+    return _matmul(6, compressed, codebook, x, out)
+
+
+def decompress_matmul_16_8_1(compressed, codebook, x, out):
+    """out[b] = W x[b] for batch 1..32 on the hashed-codebook stream with 256 pairs; x [batch, n], out [batch, m]."""
+    return _matmul(8, compressed, codebook, x, out)

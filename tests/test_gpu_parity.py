@@ -326,3 +326,91 @@ def test_matvec_t_rejects_bad_arguments(rk):
     with pytest.raises(RuntimeError):
         rk.decompress_matvec_t_16(comp, cb, torch.zeros(40000, dtype=torch.float16, device="cuda"), out)
     assert rk.decompress_matvec_t_16(comp, cb, x, out) >= 0.0
+
+
+# ------------------------------------------------------------------ decompress_matmul (batch 1..32, MFMA)
+
+MATMUL_SHAPES = [(16, 2048), (64, 4096), (33, 2048), (5, 704), (96, 4096 + 768), (300, 6144)]
+
+
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("S", [6, 8])
+@pytest.mark.parametrize("batch", [1, 8, 16, 17, 32])
+@pytest.mark.parametrize("m,n", MATMUL_SHAPES)
+def test_matmul_output_within_tolerance(rk, oracle, mode, S, batch, m, n):
+    comp = rand_codes(m * n // 16, seed=m + n + batch)
+    cb = rand_half(2 << S, seed=S + 30)
+    x = rand_half(batch * n, seed=9).reshape(batch, n)
+    out = torch.full((batch, m), float("nan"), dtype=torch.float16, device="cuda")
+    with with_mode(rk, mode):
+        ms = getattr(rk, f"decompress_matmul_16_{S}_1")(comp.cuda(), cb.cuda(), x.cuda(), out)
+    assert ms > 0
+    want = oracle.matvec(np_u32(comp), np_f16(cb), np_f16(x), m, S, mode=mode)      # [batch, m] in double
+    got = np_f16(out).astype(np.float64)
+    assert np.all(np.isfinite(got))
+    assert rel_l2(got, want) < REL_L2_TOL
+    for b in range(batch):
+        assert rel_l2(got[b], want[b]) < 2 * REL_L2_TOL
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_matmul_identity_batch_recovers_weights_bit_exactly(rk, oracle, mode):
+    """x = 32 one-hot rows at a time: out[b][r] = W[r][p_b] exactly, so the MFMA path's decode,
+    operand layout and column map are checked bit for bit."""
+    S, m, n = 8, 48, 2048 + 320
+    comp = rand_codes(m * n // 16, seed=321)
+    cb = rand_half(2 << S, seed=31)
+    want = oracle.matvec_dense(np_u32(comp), np_f16(cb), m, n, S, mode=mode)
+    c, cbd = comp.cuda(), cb.cuda()
+    got = np.zeros((m, n), dtype=np.float16)
+    out = torch.zeros((32, m), dtype=torch.float16, device="cuda")
+    prev_timing = rk.set_timing(False)
+    try:
+        with with_mode(rk, mode):
+            for p0 in range(0, n, 32):
+                x = torch.zeros((32, n), dtype=torch.float16, device="cuda")
+                x[torch.arange(32), torch.arange(p0, p0 + 32)] = 1.0
+                rk.decompress_matmul_16_8_1(c, cbd, x, out)
+                got[:, p0:p0 + 32] = np_f16(out).T
+    finally:
+        rk.set_timing(prev_timing)
+    g, w = got.view(np.uint16), want.view(np.uint16)
+    nz = (w & 0x7FFF) != 0
+    assert np.array_equal(g[nz], w[nz])
+    assert np.all((g[~nz] & 0x7FFF) == 0)
+
+
+@pytest.mark.parametrize("batch", [8, 16, 32])
+def test_matmul_full_size_equals_decode_then_dense_gemm(rk, oracle, batch):
+    S, m, n = 8, 4096, 11008
+    comp = rand_codes(m * n // 16, seed=42)
+    cb = rand_half(2 << S, seed=43)
+    x = rand_half(batch * n, seed=44).reshape(batch, n)
+    out = torch.zeros((batch, m), dtype=torch.float16, device="cuda")
+    rk.decompress_matmul_16_8_1(comp.cuda(), cb.cuda(), x.cuda(), out)
+    W = torch.zeros((m, n), dtype=torch.float16, device="cuda")
+    rk.matvec_dense(comp.cuda(), cb.cuda(), W, S)
+    want = (x.cuda().double() @ W.double().t()).cpu().numpy()
+    assert rel_l2(np_f16(out), want) < REL_L2_TOL
+    # and the batch-1 kernel agrees with row 0
+    y = torch.zeros((m,), dtype=torch.float16, device="cuda")
+    rk.decompress_matvec_16_8_1(comp.cuda(), cb.cuda(), x[0].cuda().contiguous(), y)
+    assert rel_l2(np_f16(y), want[0]) < REL_L2_TOL
+
+
+def test_matmul_rejects_bad_arguments(rk):
+    cb = torch.zeros(512, dtype=torch.float16, device="cuda")
+    comp = torch.zeros(32 * 2048 // 16, dtype=torch.int32, device="cuda")
+    x = torch.zeros((4, 2048), dtype=torch.float16, device="cuda")
+    out = torch.zeros((4, 32), dtype=torch.float16, device="cuda")
+    f = rk.decompress_matmul_16_8_1
+    with pytest.raises(RuntimeError):
+        f(comp, cb, x[0], out)                                  # x must be 2-D
+    with pytest.raises(RuntimeError):
+        f(comp, cb, x, out[:2])                                 # batch mismatch
+    with pytest.raises(RuntimeError):
+        f(comp, cb, torch.zeros((33, 2048), dtype=torch.float16, device="cuda"),
+          torch.zeros((33, 32), dtype=torch.float16, device="cuda"))      # batch > 32
+    with pytest.raises(RuntimeError):
+        f(comp[:100], cb, x, out)                               # stream size
+    assert f(comp, cb, x, out) >= 0.0
