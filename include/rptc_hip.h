@@ -134,6 +134,20 @@ int rptc_decompress_matmul(const int32_t *compressed, const uint16_t *codebook, 
                            uint16_t *out, int64_t m, int64_t n, int64_t batch, int S, int carry_mode,
                            void *stream, float *ms);
 
+/*
+ * Random-sign Hadamard (incoherence) transform on activations, fp16 in and out, fp32 inside.
+ * No counterpart in the reference (quantize_hf.py:77-117 conditions weights by a scale-and-bias
+ * factorisation instead).  Each row of x [batch][n] is cut into blocks of `block` elements
+ * (a power of two dividing n, at most 32768; 0 = the largest such power of two) and each block
+ * is mapped by
+ *     inverse == 0:  y = H (signs .* x) / sqrt(block)
+ *     inverse != 0:  y = signs .* (H x) / sqrt(block)
+ * with H the Sylvester Hadamard matrix in natural order and signs fp16 [n] of +-1; the two
+ * directions undo each other.  out may alias x.
+ */
+int rptc_sign_hadamard(const uint16_t *x, const uint16_t *signs, uint16_t *out, int64_t batch,
+                       int64_t n, int64_t block, int inverse, void *stream, float *ms);
+
 #ifdef __cplusplus
 }
 #endif

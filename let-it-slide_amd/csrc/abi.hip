@@ -10,6 +10,7 @@ int prepare_decompress();
 int prepare_matvec();
 int prepare_matvec_t();
 int prepare_matmul(int device);
+int prepare_hadamard();
 
 constexpr int kMaxDevices = 64;
 static DeviceInfo g_devices[kMaxDevices];
@@ -37,6 +38,7 @@ int device_info(DeviceInfo **out)
         if ((rc = prepare_matvec())) return rc;
         if ((rc = prepare_matvec_t())) return rc;
         if ((rc = prepare_matmul(dev))) return rc;
+        if ((rc = prepare_hadamard())) return rc;
         g_ready[dev] = true;
     }
     *out = &g_devices[dev];

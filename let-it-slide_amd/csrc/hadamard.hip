@@ -1,0 +1,87 @@
+// Random-sign Hadamard (incoherence) transform on activations.
+//
+// No counterpart in the reference (it conditions weights with a row/column scale-and-bias
+// factorisation instead, quantize_hf.py:77-117); this is the transform the north star asks for.
+// Definition: the vector of length n is cut into blocks of P elements, P a power of two dividing
+// n (by default the largest one: 4096 for n = 4096, 256 for n = 11008 = 43 * 256, 4096 for
+// n = 28672 = 7 * 4096), and each block is mapped by
+//     forward   y = H_P (s .* x) / sqrt(P)        inverse   y = s .* (H_P x) / sqrt(P)
+// with H_P the Sylvester Hadamard matrix (natural order) and s a vector of +-1.  H_P is symmetric
+// and H_P H_P = P I, so the two are inverses and both are orthogonal.
+//
+// Kernel: one workgroup per (batch row, block); the block lives in LDS as fp32, log2(P) butterfly
+// stages with P/2 butterflies spread over the threads.  The op moves 4 bytes per element
+// (fp16 in, fp16 out): HBM-bound, LDS traffic is local.
+#include "rptc_common.hpp"
+
+namespace rptc {
+
+constexpr int kHadThreads = 256;
+constexpr int kHadMaxBlock = 32768;       // 128 KiB of fp32 in LDS
+
+__global__ __launch_bounds__(kHadThreads) void sign_hadamard_kernel(
+    const uint16_t *__restrict__ x, const uint16_t *__restrict__ signs, uint16_t *__restrict__ out,
+    int n, int P, int blocks_per_row, int signs_after)
+{
+    extern __shared__ float buf[];
+    const int tid = threadIdx.x;
+    const int row = blockIdx.x / blocks_per_row, blk = blockIdx.x - row * blocks_per_row;
+    const size_t base = (size_t)row * n + (size_t)blk * P;
+    const uint16_t *s = signs + (size_t)blk * P;
+    for (int i = tid; i < P; i += kHadThreads) {
+        float v = half_bits_to_float(x[base + i]);
+        if (!signs_after) v *= half_bits_to_float(s[i]);
+        buf[i] = v;
+    }
+    __syncthreads();
+    for (int h = 1; h < P; h <<= 1) {
+        for (int k = tid; k < P / 2; k += kHadThreads) {
+            const int i = ((k & ~(h - 1)) << 1) | (k & (h - 1));
+            const float a = buf[i], b = buf[i + h];
+            buf[i] = a + b;
+            buf[i + h] = a - b;
+        }
+        __syncthreads();
+    }
+    const float scale = rsqrtf((float)P);
+    for (int i = tid; i < P; i += kHadThreads) {
+        float v = buf[i] * scale;
+        if (signs_after) v *= half_bits_to_float(s[i]);
+        out[base + i] = float_to_half_bits(v);
+    }
+}
+
+int prepare_hadamard()
+{
+    return (int)hipFuncSetAttribute(reinterpret_cast<const void *>(sign_hadamard_kernel),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, kHadMaxBlock * 4);
+}
+
+}  // namespace rptc
+
+using namespace rptc;
+
+extern "C" int rptc_sign_hadamard(const uint16_t *x, const uint16_t *signs, uint16_t *out, int64_t batch,
+                                  int64_t n, int64_t block, int inverse, void *stream, float *ms)
+{
+    if (!x || !signs || !out) return RPTC_ENULL;
+    if (batch < 1 || n < 2) return RPTC_ESHAPE;
+    int64_t P = block;
+    if (P == 0) {
+        P = 1;
+        while (n % (2 * P) == 0 && 2 * P <= kHadMaxBlock) P *= 2;
+    }
+    if (P < 2 || (P & (P - 1)) != 0 || n % P != 0) return RPTC_ESHAPE;
+    if (P > kHadMaxBlock || n >= ((int64_t)1 << 30) || batch * (n / P) >= ((int64_t)1 << 31)) return RPTC_ELIMIT;
+    DeviceInfo *dev;
+    int rc = device_info(&dev);
+    if (rc) return rc;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    Timer t;
+    rc = t.begin(dev, s, ms);
+    if (rc) return rc;
+    const int blocks_per_row = (int)(n / P);
+    hipLaunchKernelGGL(sign_hadamard_kernel, dim3((unsigned)(batch * blocks_per_row)), dim3(kHadThreads),
+                       (size_t)P * 4, s, x, signs, out, (int)n, (int)P, blocks_per_row, inverse ? 1 : 0);
+    return t.end();
+}

@@ -52,6 +52,7 @@ _SIGNATURES = {
     "rptc_matvec_dense": ([_VP, _VP, _VP, _I64, _I64, _INT, _INT, _VP, _FP], _INT),
     "rptc_matvec_t_dense": ([_VP, _VP, _VP, _I64, _I64, _INT, _INT, _VP, _FP], _INT),
     "rptc_decompress_matmul": ([_VP, _VP, _VP, _VP, _I64, _I64, _I64, _INT, _INT, _VP, _FP], _INT),
+    "rptc_sign_hadamard": ([_VP, _VP, _VP, _I64, _I64, _I64, _INT, _VP, _FP], _INT),
 }
 
 
@@ -302,3 +303,39 @@ def decompress_matmul_16_6_1(compressed, codebook, x, out):
 def decompress_matmul_16_8_1(compressed, codebook, x, out):
     """out[b] = W x[b] for batch 1..32 on the hashed-codebook stream with 256 pairs; x [batch, n], out [batch, m]."""
     return _matmul(8, compressed, codebook, x, out)
+
+
+def hadamard_block(n):
+    """The default block length of the sign-Hadamard transform: the largest power of two dividing n (<= 32768)."""
+    p = 1
+    while n % (2 * p) == 0 and 2 * p <= 32768:
+        p *= 2
+    return p
+
+
+def sign_hadamard(x, signs, out, block=0, inverse=False):
+    """Blockwise random-sign Hadamard transform of the rows of x ([n] or [batch, n], fp16).
+
+    forward: out = H (signs * x) / sqrt(block); inverse: out = signs * (H x) / sqrt(block), per block of
+    ``block`` elements (0 = the largest power of two dividing n).  ``out`` may be ``x``.  Returns elapsed ms."""
+    _check_input(x, "x")
+    _check_input(signs, "signs")
+    _check_input(out, "out")
+    _check(x.dtype == torch.float16 and signs.dtype == torch.float16 and out.dtype == torch.float16,
+           "x, signs and out must be fp16")
+    _check(x.dim() in (1, 2), "x.dim() in (1, 2)")
+    _check(out.shape == x.shape, "out.shape == x.shape")
+    n = x.size(-1)
+    batch = x.size(0) if x.dim() == 2 else 1
+    _check(signs.dim() == 1 and signs.size(0) == n, "signs.size(0) == n")
+    p = block or hadamard_block(n)
+    _check(p >= 2 and p & (p - 1) == 0 and n % p == 0 and p <= 32768, "block must be a power of two dividing n")
+    device = x.device
+    ms = ctypes.c_float(0.0)
+    with torch.cuda.device(device):
+        stream = torch.cuda.current_stream().cuda_stream
+        rc = library().rptc_sign_hadamard(x.data_ptr(), signs.data_ptr(), out.data_ptr(), batch, n, p,
+                                          1 if inverse else 0, ctypes.c_void_p(stream),
+                                          ctypes.byref(ms) if _timing else None)
+    _status(rc)
+    return float(ms.value)

@@ -523,6 +523,38 @@ void orc_dense_matvec(const uint16_t *W, const uint16_t *x, double *y,
     free(xf);
 }
 
+/* ------------------------------------------------- sign-Hadamard transform */
+
+/*
+ * No counterpart in the reference.  Blockwise y = H (s .* x) / sqrt(P) (inverse: s .* (H x) /
+ * sqrt(P)), H the Sylvester Hadamard matrix in natural order, computed by the in-place fast
+ * Walsh-Hadamard butterflies in double.  x, signs: fp16 bits; y: double.
+ */
+int orc_sign_hadamard(const uint16_t *x, const uint16_t *signs, double *y, int64_t batch,
+                      int64_t n, int64_t P, int inverse)
+{
+    if (P < 1 || (P & (P - 1)) != 0 || n % P != 0) return -1;
+    for (int64_t b = 0; b < batch; b++) {
+        for (int64_t blk = 0; blk < n / P; blk++) {
+            double *v = y + b * n + blk * P;
+            const uint16_t *xs = x + b * n + blk * P, *ss = signs + blk * P;
+            for (int64_t i = 0; i < P; i++)
+                v[i] = (double)half_to_float(xs[i]) * (inverse ? 1.0 : (double)half_to_float(ss[i]));
+            for (int64_t h = 1; h < P; h <<= 1)
+                for (int64_t i = 0; i < P; i += 2 * h)
+                    for (int64_t j = i; j < i + h; j++) {
+                        double a = v[j], c = v[j + h];
+                        v[j] = a + c;
+                        v[j + h] = a - c;
+                    }
+            double scale = 1.0 / sqrt((double)P);
+            for (int64_t i = 0; i < P; i++)
+                v[i] = v[i] * scale * (inverse ? (double)half_to_float(ss[i]) : 1.0);
+        }
+    }
+    return 0;
+}
+
 /* -------------------------------------------------- timed CPU baseline leg */
 
 /*

@@ -44,6 +44,8 @@ def lib():
         _lib.orc_matvec_f32.restype = i32
         _lib.orc_half_to_float.argtypes = [vp, vp, i64]
         _lib.orc_float_to_half.argtypes = [vp, vp, i64]
+        _lib.orc_sign_hadamard.argtypes = [vp, vp, vp, i64, i64, i64, i32]
+        _lib.orc_sign_hadamard.restype = i32
         _lib.orc_num_threads.restype = i32
         _lib.orc_set_num_threads.argtypes = [i32]
     return _lib
@@ -200,6 +202,19 @@ def matvec_f32(compressed, codebook, x, m, S, mode=AS_WRITTEN):
     rc = lib().orc_matvec_f32(_p(c), _p(cb), _p(xx), _p(y), m, n, S, mode)
     assert rc == 0, rc
     return y
+
+
+def sign_hadamard(x, signs, block, inverse=False):
+    """Blockwise sign-Hadamard transform in double of float16 x [n] or [batch, n]; returns float64."""
+    xx = _u16(x)
+    single = xx.ndim == 1
+    xx = xx.reshape(-1, xx.shape[-1])
+    ss = _u16(signs)
+    batch, n = xx.shape
+    y = np.empty((batch, n), dtype=np.float64)
+    rc = lib().orc_sign_hadamard(_p(xx), _p(ss), _p(y), batch, n, block, 1 if inverse else 0)
+    assert rc == 0, rc
+    return y[0] if single else y
 
 
 def half_to_float(h):

@@ -414,3 +414,35 @@ def test_matmul_rejects_bad_arguments(rk):
     with pytest.raises(RuntimeError):
         f(comp[:100], cb, x, out)                               # stream size
     assert f(comp, cb, x, out) >= 0.0
+
+
+# ------------------------------------------------------------------ sign-Hadamard transform
+
+@pytest.mark.parametrize("batch,n,block", [(1, 4096, 0), (3, 11008, 0), (2, 28672, 0), (1, 64, 0), (4, 8192, 256),
+                                           (1, 32768, 0), (2, 704, 0)])
+@pytest.mark.parametrize("inverse", [False, True])
+def test_sign_hadamard_matches_oracle(rk, oracle, batch, n, block, inverse):
+    x = rand_half(batch * n, seed=n).reshape(batch, n)
+    signs = torch.where(torch.rand(n, generator=torch.Generator().manual_seed(n)) < 0.5, -1.0, 1.0).to(torch.float16)
+    out = torch.zeros_like(x, device="cuda")
+    ms = rk.sign_hadamard(x.cuda(), signs.cuda(), out, block=block, inverse=inverse)
+    assert ms > 0
+    P = block or rk.hadamard_block(n)
+    want = oracle.sign_hadamard(np_f16(x), np_f16(signs), P, inverse=inverse)
+    # fp32 butterflies, one fp16 rounding at the end: 2^-11 relative per element
+    assert rel_l2(np_f16(out), want) < REL_L2_TOL
+
+
+def test_sign_hadamard_round_trip_and_norm(rk):
+    n = 11008
+    x = rand_half(2 * n, seed=3).reshape(2, n).cuda()
+    signs = torch.where(torch.rand(n, generator=torch.Generator().manual_seed(1)) < 0.5, -1.0, 1.0).to(torch.float16).cuda()
+    y = torch.zeros_like(x)
+    z = torch.zeros_like(x)
+    rk.sign_hadamard(x, signs, y)
+    rk.sign_hadamard(y, signs, z, inverse=True)
+    assert rel_l2(z.cpu().numpy(), x.cpu().numpy()) < REL_L2_TOL
+    assert abs(y.double().norm().item() / x.double().norm().item() - 1.0) < 1e-3
+    # in place
+    rk.sign_hadamard(y, signs, y, inverse=True)
+    assert torch.equal(y, z)

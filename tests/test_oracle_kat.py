@@ -348,3 +348,30 @@ def test_lite_dequantize_window(oracle):
     for t, s in enumerate(symbols):
         state = ((state << R) | int(s)) & 0xFFFFFFFF
         assert np.array_equal(got[t], alphabet[_index_fn_python(state, L, S)])
+
+
+# ------------------------------------------------------------------ sign-Hadamard transform (no reference counterpart)
+
+@pytest.mark.parametrize("P", [2, 64, 256, 1024])
+def test_sign_hadamard_equals_dense_sylvester_product(oracle, P):
+    from scipy.linalg import hadamard
+    g = rng(P)
+    n = 3 * P
+    x = g.standard_normal((2, n)).astype(np.float16)
+    s = np.where(g.random(n) < 0.5, -1.0, 1.0).astype(np.float16)
+    H = hadamard(P).astype(np.float64)
+    xs = x.astype(np.float64) * s.astype(np.float64)
+    fwd = np.concatenate([(xs[:, b * P:(b + 1) * P] @ H.T) / np.sqrt(P) for b in range(3)], axis=1)
+    assert np.allclose(oracle.sign_hadamard(x, s, P), fwd, rtol=1e-12, atol=1e-12)
+    xd = x.astype(np.float64)
+    inv = np.concatenate([(xd[:, b * P:(b + 1) * P] @ H.T) / np.sqrt(P) for b in range(3)], axis=1) * s.astype(np.float64)
+    assert np.allclose(oracle.sign_hadamard(x, s, P, inverse=True), inv, rtol=1e-12, atol=1e-12)
+
+
+def test_sign_hadamard_is_orthogonal(oracle):
+    g = rng(5)
+    n, P = 11008, 256
+    x = g.standard_normal(n).astype(np.float16)
+    s = np.where(g.random(n) < 0.5, -1.0, 1.0).astype(np.float16)
+    y = oracle.sign_hadamard(x, s, P)
+    assert np.isclose(np.linalg.norm(y), np.linalg.norm(x.astype(np.float64)), rtol=1e-12)
