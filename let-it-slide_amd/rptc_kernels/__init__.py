@@ -120,14 +120,15 @@ def _status(rc):
         raise RuntimeError(f"rptc_kernels: {text} (status {rc})")
 
 
-def _call(fn, tensors, *args):
+def _call(fn, tensors, *args, carry_mode=None):
     device = tensors[0].device
     for t in tensors[1:]:
         _check(t.device == device, "all tensors must be on the same device")
     ms = ctypes.c_float(0.0)
+    mode = _carry_mode if carry_mode is None else carry_mode
     with torch.cuda.device(device):
         stream = torch.cuda.current_stream().cuda_stream
-        rc = fn(*[t.data_ptr() for t in tensors], *args, _carry_mode, ctypes.c_void_p(stream),
+        rc = fn(*[t.data_ptr() for t in tensors], *args, mode, ctypes.c_void_p(stream),
                 ctypes.byref(ms) if _timing else None)
     _status(rc)
     return float(ms.value)

@@ -1,0 +1,177 @@
+"""QuantizedLinear: a linear layer whose weight lives as a packed trellis stream.
+
+The reference never builds such a module: ``quantize_hf.py:215`` writes the de-quantized matrix
+back into a dense ``nn.Linear`` (``module.weight.copy_(recon)``).  This module keeps the stream and
+runs the fused kernels instead.  It follows the reference's reconstruction formula
+(``quantize_hf.py:167``)
+
+    W = b_out + b_in + s_out * s_in * W_hat            (b_out, s_out per row; b_in, s_in per column)
+
+so  y = s_out * (W_hat (s_in * x)) + b_out * sum(x) + (b_in . x),  with W_hat the matrix the stream
+decodes to, and its list of quantized modules (``quantize_hf.py:189``).
+"""
+import re
+
+import torch
+
+import rptc_kernels as rk
+
+# the modules quantize_hf.py:189 quantizes
+REFERENCE_PATTERN = r"model\.layers\.(\d+)\.(self_attn\.(\w+)_proj|mlp\.(\w+)_proj)"
+
+
+class QuantizedLinear(torch.nn.Module):
+    """y = W x with W held as a hashed-pair trellis stream (2 bits/weight) plus the optional
+    row/column scales and biases of the reference's factorisation and an optional sign-Hadamard
+    transform of the input."""
+
+    def __init__(self, in_features, out_features, S=8, carry_mode=rk.CONTINUOUS, device="cuda"):
+        super().__init__()
+        if in_features % 64 != 0:
+            raise ValueError("in_features must be a multiple of 64 (whole stream elements per row)")
+        if S not in (6, 8):
+            raise ValueError("S must be 6 or 8")
+        self.in_features, self.out_features, self.S, self.carry_mode = in_features, out_features, S, carry_mode
+        words = out_features * in_features // 16
+        self.register_buffer("compressed", torch.zeros(words, dtype=torch.int32, device=device))
+        self.register_buffer("codebook", torch.zeros(2 << S, dtype=torch.float16, device=device))
+        for name in ("scales_out", "scales_in", "biases_out", "biases_in", "signs"):
+            self.register_buffer(name, None)
+
+    # ---------------------------------------------------------------- construction
+
+    @classmethod
+    def from_random(cls, in_features, out_features, S=8, seed=42, weight_std=None, device="cuda", **kw):
+        """Seeded random stream and codebook: decode cost does not depend on the data, so this is
+        what the synthetic benchmarks use.  The codebook is scaled so that W has std weight_std
+        (default 1/sqrt(in_features))."""
+        layer = cls(in_features, out_features, S=S, device=device, **kw)
+        g = torch.Generator(device=device)
+        g.manual_seed(seed)
+        layer.compressed.copy_(torch.randint(-(1 << 31), 1 << 31, layer.compressed.shape, generator=g,
+                                             dtype=torch.int64, device=device).to(torch.int32))
+        std = weight_std if weight_std is not None else in_features ** -0.5
+        layer.codebook.copy_((torch.randn(2 << S, generator=g, device=device) * std).to(torch.float16))
+        return layer
+
+    @classmethod
+    def from_symbols(cls, symbols, codebook, out_features, S=8, device="cuda", **kw):
+        """symbols: 4-bit trellis symbols [out_features, in_features/2] in stream order (numpy or tensor)."""
+        from rptc_kernels import packing
+        import numpy as np
+        sym = symbols.cpu().numpy() if isinstance(symbols, torch.Tensor) else np.asarray(symbols)
+        layer = cls(2 * sym.shape[1], out_features, S=S, device=device, **kw)
+        layer.compressed.copy_(torch.from_numpy(packing.pack_matvec(sym)).to(device))
+        layer.codebook.copy_(torch.as_tensor(codebook, dtype=torch.float16).to(device))
+        return layer
+
+    def set_affine(self, scales_out=None, scales_in=None, biases_out=None, biases_in=None):
+        """The reference's row/column factorisation (quantize_hf.py:77-117,167); any may be None."""
+        def prep(v, n):
+            if v is None:
+                return None
+            v = torch.as_tensor(v, dtype=torch.float16, device=self.compressed.device).reshape(-1).contiguous()
+            if v.numel() != n:
+                raise ValueError("wrong length")
+            return v
+        self.scales_out = prep(scales_out, self.out_features)
+        self.biases_out = prep(biases_out, self.out_features)
+        self.scales_in = prep(scales_in, self.in_features)
+        self.biases_in = prep(biases_in, self.in_features)
+        return self
+
+    def set_signs(self, signs):
+        """+-1 per input feature: the input goes through the sign-Hadamard transform first, i.e. the
+        stream encodes W_hat in the transformed basis."""
+        self.signs = None if signs is None else torch.as_tensor(
+            signs, dtype=torch.float16, device=self.compressed.device).reshape(-1).contiguous()
+        return self
+
+    # ---------------------------------------------------------------- forward
+
+    def _product(self, x2):
+        """x2 fp16 [batch, n] contiguous -> fp16 [batch, m] = W_hat x, through the fused kernels."""
+        batch = x2.size(0)
+        out = torch.empty((batch, self.out_features), dtype=torch.float16, device=x2.device)
+        lib = rk.library()
+        if batch == 1:
+            fn = getattr(lib, f"rptc_decompress_matvec_16_{self.S}_1")
+            rk._call(fn, (self.compressed, self.codebook, x2, out), self.out_features, self.in_features,
+                     carry_mode=self.carry_mode)
+            return out
+        for b0 in range(0, batch, 32):
+            xb = x2[b0:b0 + 32]
+            ob = out[b0:b0 + 32]
+            rk._call(lib.rptc_decompress_matmul, (self.compressed, self.codebook, xb, ob), self.out_features,
+                     self.in_features, xb.size(0), self.S, carry_mode=self.carry_mode)
+        return out
+
+    def forward(self, x):
+        if x.dtype != torch.float16 or not x.is_cuda:
+            raise RuntimeError("QuantizedLinear runs on fp16 CUDA tensors only (there is no CPU path)")
+        shape = x.shape
+        x2 = x.reshape(-1, self.in_features).contiguous()
+        xs = x2 * self.scales_in if self.scales_in is not None else x2
+        if self.signs is not None:
+            t = torch.empty_like(xs)
+            prev = rk.set_timing(False)
+            try:
+                rk.sign_hadamard(xs, self.signs, t)
+            finally:
+                rk.set_timing(prev)
+            xs = t
+        prev = rk.set_timing(False)
+        try:
+            y = self._product(xs)
+        finally:
+            rk.set_timing(prev)
+        if self.scales_out is not None:
+            y = y * self.scales_out
+        if self.biases_out is not None:
+            y = y + self.biases_out * x2.float().sum(dim=1, keepdim=True).to(torch.float16)
+        if self.biases_in is not None:
+            y = y + (x2.float() @ self.biases_in.float()).to(torch.float16).unsqueeze(1)
+        return y.reshape(shape[:-1] + (self.out_features,))
+
+    # ---------------------------------------------------------------- inspection
+
+    def decoded_weight(self):
+        """W_hat, fp16 [m, n], bit-exact decode of the stream."""
+        W = torch.empty((self.out_features, self.in_features), dtype=torch.float16, device=self.compressed.device)
+        prev = rk.set_timing(False)
+        try:
+            rk._call(rk.library().rptc_matvec_dense, (self.compressed, self.codebook, W), self.out_features,
+                     self.in_features, self.S, carry_mode=self.carry_mode)
+        finally:
+            rk.set_timing(prev)
+        return W
+
+    def compressed_bytes(self):
+        return self.compressed.numel() * 4
+
+    def extra_repr(self):
+        return f"in_features={self.in_features}, out_features={self.out_features}, S={self.S}, bits_per_weight=2"
+
+
+def patch_model(model, pattern=REFERENCE_PATTERN, S=8, seed=42, make_layer=None):
+    """Replace every ``nn.Linear`` whose qualified name matches ``pattern`` (default: the modules
+    quantize_hf.py:189 quantizes) by a QuantizedLinear.  ``make_layer(name, linear)`` may build the
+    replacement; by default a seeded random stream of the same shape is used (synthetic weights).
+    Returns the list of replaced names."""
+    rx = re.compile(pattern)
+    replaced = []
+    for i, (name, module) in enumerate(list(model.named_modules())):
+        if not isinstance(module, torch.nn.Linear) or re.fullmatch(rx, name) is None:
+            continue
+        if make_layer is not None:
+            new = make_layer(name, module)
+        else:
+            new = QuantizedLinear.from_random(module.in_features, module.out_features, S=S, seed=seed + i,
+                                              device=module.weight.device)
+        parent = model
+        parts = name.split(".")
+        for p in parts[:-1]:
+            parent = getattr(parent, p)
+        setattr(parent, parts[-1], new)
+        replaced.append(name)
+    return replaced

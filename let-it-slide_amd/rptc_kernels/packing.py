@@ -1,0 +1,84 @@
+"""Host-side packers: trellis symbols -> the three packed streams the kernels read.
+
+The reference has no packer: its quantizers return unpacked symbol arrays (rptc.py:68,
+rptc_lite.py:57) and nothing writes the bitstreams its CUDA kernels consume.  The layouts below
+are read off the decoders (inference.cu:42-96, 189-277; inference_t.cu:68-175): symbols are
+consumed most-significant-bits first inside each 32-bit word, words in memory order.  All
+functions are plain numpy and return int32 arrays ready for ``torch.from_numpy``.
+"""
+import numpy as np
+
+
+def _words_from_symbols(symbols, bits):
+    """[..., k] symbols of `bits` bits (32 % bits == 0) -> [..., k*bits/32] uint32, first symbol on top."""
+    per = 32 // bits
+    s = np.asarray(symbols, dtype=np.uint32)
+    assert s.shape[-1] % per == 0 and (s < (1 << bits)).all()
+    s = s.reshape(s.shape[:-1] + (s.shape[-1] // per, per))
+    shifts = (32 - bits * (np.arange(per, dtype=np.uint32) + 1)).astype(np.uint32)
+    return np.bitwise_or.reduce(s << shifts, axis=-1).astype(np.uint32)
+
+
+def pack_rowmajor(symbols):
+    """2-bit symbols [m, n] -> the stream of ``decompress``: int32 [m, n/16], n % 2048 == 0.
+
+    Row r, output t is decoded from symbols t-7..t of the row (inference.cu:68-94)."""
+    symbols = np.asarray(symbols)
+    m, n = symbols.shape
+    assert n % 2048 == 0, "decompress needs whole groups of 32 stream elements per row"
+    return _words_from_symbols(symbols, 2).view(np.int32)
+
+
+def pack_transposed(symbols):
+    """2-bit symbols [m, n] -> the stream of ``decompress_matvec_t_*``: int32 [n/64, m, 4], n % 64 == 0.
+
+    Element col of row r holds the row's symbols 64*col .. 64*col+63 (inference_t.cu:116)."""
+    symbols = np.asarray(symbols)
+    m, n = symbols.shape
+    assert n % 64 == 0
+    words = _words_from_symbols(symbols, 2).reshape(m, n // 64, 4)
+    return np.ascontiguousarray(words.transpose(1, 0, 2)).view(np.int32)
+
+
+def matvec_stream_columns(n):
+    """Column of the FIRST weight of every step of a row of the hashed pair stream, in stream order.
+
+    Returns int64 [n/2]: entry p is the column 8*idx + 2*i of the pair decoded by the p-th 4-bit
+    symbol of a row, p = (slab*32 + lane)*32 + step for the full slabs and the ragged last slab
+    appended (inference.cu:215-221,249; step s <-> (k, j): k = 7, 0, 4, 1, 5, 2, 6, 3 for
+    s // 4 = 0..7, j = s % 4).  The second weight of the pair is the next column."""
+    assert n % 64 == 0
+    T, Lt, n8 = n // 2048, (n % 2048) // 64, n // 8
+    k_of = np.array([7, 0, 4, 1, 5, 2, 6, 3])
+    s = np.arange(32)
+    q = 4 * k_of[s // 4] + s % 4                       # slot step index 4k + j
+    cols = []
+    for slab in range(T + (1 if Lt else 0)):
+        lanes = 32 if slab < T else Lt
+        lane = np.arange(lanes)[:, None]
+        P = 1024 * slab + (32 * q[None, :] + lane if slab < T else q[None, :] * Lt + lane)
+        i, idx = P // n8, P % n8
+        cols.append((8 * idx + 2 * i).reshape(-1))
+    return np.concatenate(cols).astype(np.int64)
+
+
+def pack_matvec(symbols):
+    """4-bit symbols [m, n/2] in stream order -> the stream of ``decompress_matvec_*``: int32 [m*n/16].
+
+    Row r's p-th symbol is step p % 32 of lane (p // 32) % lanes of slab p // 1024; the flat result
+    is [n/2048][m][32][4] followed by the ragged slab [m][Lt][4] (reshape to [n/2048, m, 128] when
+    n % 2048 == 0).  In CONTINUOUS mode the decoder state before a step is the previous four
+    symbols of the row."""
+    symbols = np.asarray(symbols)
+    m, half = symbols.shape
+    n = 2 * half
+    assert n % 64 == 0
+    T, Lt = n // 2048, (n % 2048) // 64
+    words = _words_from_symbols(symbols, 4)           # [m, n/16]: 4 words per element, elements in stream order
+    parts = []
+    if T:
+        full = words[:, :T * 128].reshape(m, T, 128)
+        parts.append(np.ascontiguousarray(full.transpose(1, 0, 2)).reshape(-1))
+    if Lt:
+        parts.append(np.ascontiguousarray(words[:, T * 128:]).reshape(-1))
+    return np.concatenate(parts).view(np.int32)

@@ -1,0 +1,118 @@
+"""QuantizedLinear and the model patcher on the GPU, against dense reconstructions."""
+import numpy as np
+import pytest
+import torch
+
+from util import rel_l2
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def rk():
+    import rptc_kernels
+    assert torch.cuda.is_available()
+    return rptc_kernels
+
+
+@pytest.mark.parametrize("batch", [1, 5, 32, 70])
+def test_quantized_linear_matches_dense_reconstruction(rk, batch):
+    from rptc_kernels.linear import QuantizedLinear
+    n, m = 4096 + 768, 1024
+    layer = QuantizedLinear.from_random(n, m, S=8, seed=1)
+    g = torch.Generator(device="cuda").manual_seed(2)
+    so = (torch.rand(m, generator=g, device="cuda") + 0.5).half()
+    si = (torch.rand(n, generator=g, device="cuda") + 0.5).half()
+    bo = (torch.randn(m, generator=g, device="cuda") * 0.01).half()
+    bi = (torch.randn(n, generator=g, device="cuda") * 0.01).half()
+    layer.set_affine(so, si, bo, bi)
+    x = torch.randn((batch, n), generator=g, device="cuda").half()
+    y = layer(x)
+    assert y.shape == (batch, m) and y.dtype == torch.float16
+    # quantize_hf.py:167: W = b_out + b_in + s_out * s_in * W_hat
+    W = bo.double()[:, None] + bi.double()[None, :] + so.double()[:, None] * si.double()[None, :] * layer.decoded_weight().double()
+    want = x.double() @ W.t()
+    assert rel_l2(y.cpu().numpy(), want.cpu().numpy()) < 2e-3      # several fp16 roundings in the epilogue
+
+
+def test_quantized_linear_with_sign_hadamard(rk):
+    from rptc_kernels.linear import QuantizedLinear
+    n, m = 11008, 256
+    layer = QuantizedLinear.from_random(n, m, S=6, seed=3)
+    signs = torch.where(torch.rand(n, device="cuda") < 0.5, -1.0, 1.0).half()
+    layer.set_signs(signs)
+    x = torch.randn((3, 2, n), device="cuda").half()
+    y = layer(x)
+    assert y.shape == (3, 2, m)
+    t = torch.empty((6, n), dtype=torch.float16, device="cuda")
+    rk.sign_hadamard(x.reshape(6, n).contiguous(), signs, t)
+    want = t.double() @ layer.decoded_weight().double().t()
+    assert rel_l2(y.reshape(6, m).cpu().numpy(), want.cpu().numpy()) < 1e-3
+
+
+def test_from_symbols_decodes_the_trellis_path(rk):
+    from rptc_kernels.linear import QuantizedLinear
+    from rptc_kernels import packing
+    g = np.random.default_rng(4)
+    m, n, S = 32, 2048 + 128, 8
+    symbols = g.integers(0, 16, (m, n // 2))
+    cb = g.standard_normal(2 << S).astype(np.float16)
+    layer = QuantizedLinear.from_symbols(symbols, cb, m, S=S)
+    W = layer.decoded_weight().cpu().numpy().view(np.uint16)
+    cols = packing.matvec_stream_columns(n)
+    cbb = cb.view(np.uint16)
+    for r in (0, 17, 31):
+        state = 0
+        for p, sym in enumerate(symbols[r]):
+            state = ((state << 4) | int(sym)) & 0xFFFF
+            prod = state * (state + 1)
+            e = (prod >> 8) & 0xFF
+            assert W[r, cols[p]] == (int(cbb[2 * e]) & 0x7FFF) | (prod & 0x8000)
+            assert W[r, cols[p] + 1] == cbb[2 * e + 1]
+
+
+def test_patch_model_replaces_the_reference_module_list(rk):
+    from rptc_kernels.linear import QuantizedLinear, patch_model
+
+    class Attn(torch.nn.Module):
+        def __init__(self, d):
+            super().__init__()
+            self.q_proj, self.k_proj, self.v_proj, self.o_proj = (torch.nn.Linear(d, d, bias=False) for _ in range(4))
+
+    class Mlp(torch.nn.Module):
+        def __init__(self, d, f):
+            super().__init__()
+            self.gate_proj, self.up_proj = torch.nn.Linear(d, f, bias=False), torch.nn.Linear(d, f, bias=False)
+            self.down_proj = torch.nn.Linear(f, d, bias=False)
+
+        def forward(self, x):
+            return self.down_proj(torch.nn.functional.silu(self.gate_proj(x)) * self.up_proj(x))
+
+    class Layer(torch.nn.Module):
+        def __init__(self, d, f):
+            super().__init__()
+            self.self_attn, self.mlp = Attn(d), Mlp(d, f)
+
+    class Inner(torch.nn.Module):
+        def __init__(self, d, f):
+            super().__init__()
+            self.layers = torch.nn.ModuleList([Layer(d, f) for _ in range(2)])
+
+    class Model(torch.nn.Module):
+        def __init__(self, d=256, f=704):
+            super().__init__()
+            self.model = Inner(d, f)
+            self.lm_head = torch.nn.Linear(d, 100, bias=False)
+
+    model = Model().half().cuda()
+    names = patch_model(model)
+    assert len(names) == 14 and "lm_head" not in names        # 7 projections per layer, quantize_hf.py:189
+    assert isinstance(model.model.layers[1].mlp.down_proj, QuantizedLinear)
+    assert isinstance(model.lm_head, torch.nn.Linear)
+    mlp = model.model.layers[0].mlp
+    x = torch.randn((1, 256), device="cuda").half()
+    y = mlp(x)
+    Wg, Wu, Wd = (l.decoded_weight().float() for l in (mlp.gate_proj, mlp.up_proj, mlp.down_proj))
+    h = (torch.nn.functional.silu(x.float() @ Wg.t()).half().float() * (x.float() @ Wu.t()).half().float()).half().float()
+    want = h @ Wd.t()
+    assert rel_l2(y.float().cpu().numpy(), want.cpu().numpy()) < 5e-3
