@@ -47,6 +47,8 @@ def parse():
                     help="for `rocprofv3 --pmc`: a few direct launches of the kernel plus a plain device copy of "
                          "known size (the calibration for FETCH_SIZE / WRITE_SIZE); prints no benchmark line")
     ap.add_argument("--extra-shapes", action="store_true", help="also time the other layer shapes")
+    ap.add_argument("--other-ops", action="store_true",
+                    help="time decompress, decompress_matvec_t_16 and sign_hadamard instead (prints its own JSON line)")
     ap.add_argument("--matmul", action="store_true",
                     help="time the batch 8/16/32 fused decode + MFMA mat-mat instead (prints its own JSON line)")
     return ap.parse_args()
@@ -226,6 +228,75 @@ def bench_matmul(a):
                       "results": results}))
 
 
+def _graph_time_us(step, steps):
+    """Average microseconds per call of step(k) over one HIP-graph replay of `steps` calls."""
+    import torch
+    for k in range(10):
+        step(k)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for k in range(steps):
+            step(k)
+    graph.replay()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    graph.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / steps * 1e3
+
+
+def bench_other_ops(a):
+    """The ops beside the headline kernel, each against the roofline that bounds it:
+    decompress (writes 2mn bytes), decompress_matvec_t_16 (reads mn/4), sign_hadamard (4 bytes/element)."""
+    import torch
+    import rptc_kernels as rk
+    rk.set_timing(False)
+    g = torch.Generator(device="cuda")
+    g.manual_seed(42)
+    steps = min(a.steps, 200)
+    res = {}
+
+    def rand_words(k):
+        return torch.randint(-(1 << 31), 1 << 31, (k,), generator=g, dtype=torch.int64, device="cuda").to(torch.int32)
+
+    # decompress: 4096 x 4096, the reference's CPU-runnable configuration
+    m, n = 4096, 4096
+    comps = [rand_words(m * n // 16).reshape(m, n // 16) for _ in range(8)]
+    cb16 = torch.randn(65536, generator=g, device="cuda").half()
+    outs = [torch.empty((m, n), dtype=torch.float16, device="cuda") for _ in range(8)]
+    us = _graph_time_us(lambda k: rk.decompress(comps[k % 8], cb16, outs[k % 8]), steps)
+    byts = m * n // 4 + 2 * m * n
+    res["decompress 4096x4096"] = {"us": round(us, 2), "bytes": byts, "GBps": round(byts / us / 1e3, 1),
+                                   "frac_hbm": round(byts / us / 1e3 / HBM_PEAK_GBS, 4)}
+    # transposed mat-vec, both carry modes
+    for (m, n) in ((4096, 4096), (11008, 4096)):
+        streams = [rand_words(m * n // 16) for _ in range(16)]
+        x = torch.randn(n, generator=g, device="cuda").half()
+        out = torch.zeros(m, dtype=torch.float16, device="cuda")
+        for mode, name in ((rk.AS_WRITTEN, "as_written"), (rk.CONTINUOUS, "continuous")):
+            rk.set_carry_mode(mode)
+            us = _graph_time_us(lambda k: rk.decompress_matvec_t_16(streams[k % 16], cb16, x, out), steps)
+            byts = m * n // 4
+            res[f"decompress_matvec_t_16 {m}x{n} {name}"] = {
+                "us": round(us, 2), "bytes": byts, "GBps": round(byts / us / 1e3, 1),
+                "frac_hbm": round(byts / us / 1e3 / HBM_PEAK_GBS, 4)}
+        rk.set_carry_mode(rk.AS_WRITTEN)
+    # sign-Hadamard transform
+    for (batch, n) in ((1, 4096), (1, 11008), (32, 11008), (16, 28672)):
+        x = torch.randn((batch, n), generator=g, device="cuda").half()
+        signs = torch.where(torch.rand(n, generator=g, device="cuda") < 0.5, -1.0, 1.0).half()
+        y = torch.empty_like(x)
+        us = _graph_time_us(lambda k: rk.sign_hadamard(x, signs, y), steps)
+        byts = 4 * batch * n
+        res[f"sign_hadamard batch {batch} n {n}"] = {"us": round(us, 2), "bytes": byts,
+                                                     "GBps": round(byts / us / 1e3, 1)}
+    print(json.dumps({"metric": "other ops, microseconds per call", "unit": "us", "n_gpus": 1,
+                      "config": {"launch": "graph", "steps": steps}, "results": res}))
+
+
 def main():
     a = parse()
     if a.gpus != 1:
@@ -238,6 +309,9 @@ def main():
     torch.cuda.set_device(0)
     if a.matmul:
         bench_matmul(a)
+        return
+    if a.other_ops:
+        bench_other_ops(a)
         return
     runner = Runner(a.m, a.n, a.S, a.copies)
     if a.pmc_probe:

@@ -132,9 +132,11 @@ __global__ __launch_bounds__(kMatvecThreads) void matvec_kernel(
 
     // This wave's items: a contiguous piece of [slab 0 items][slab 1 items]...[ragged slab items].
     const int total = T * a.items_full + a.items_tail;
-    const int per_wave = (total + kMatvecWaves - 1) / kMatvecWaves;
-    const int it_begin = min(total, wave * per_wave);
-    const int it_end = min(total, it_begin + per_wave);
+    // The first total % 16 waves take one item more.  Waves w, w+4, w+8, w+12 share a SIMD, so
+    // this also spreads the remainder evenly over the four SIMDs.
+    const int per_wave = total / kMatvecWaves, extra = total % kMatvecWaves;
+    const int it_begin = wave * per_wave + min(wave, extra);
+    const int it_end = it_begin + per_wave + (wave < extra ? 1 : 0);
     auto view = [&](int slab) {
         SlabView v;
         const bool full = slab < T;
