@@ -19,9 +19,13 @@
 namespace rptc {
 
 constexpr int kHadThreads = 256;
-constexpr int kHadMaxBlock = 32768;       // 128 KiB of fp32 in LDS
+constexpr int kHadMaxBlock = 32768;       // 132 KiB of fp32 in LDS (with padding)
 
-// stages s .. s+R_LOG-1 of the transform on buf[0, P)
+// Element i of the block lives at buf[pad(i)]: one unused float after every 32 keeps the 16-point
+// gathers (lane stride 16 floats in the first pass) off the same LDS bank.
+__device__ __forceinline__ int pad(int i) { return i + (i >> 5); }
+
+// stages s .. s+R_LOG-1 of the transform on the block in buf
 template <int R_LOG>
 __device__ __forceinline__ void hadamard_pass(float *buf, int P, int s, int tid)
 {
@@ -31,7 +35,7 @@ __device__ __forceinline__ void hadamard_pass(float *buf, int P, int s, int tid)
         const int base = ((grp >> s) << (s + R_LOG)) | (grp & low_mask);
         float v[R];
 #pragma unroll
-        for (int k = 0; k < R; k++) v[k] = buf[base + (k << s)];
+        for (int k = 0; k < R; k++) v[k] = buf[pad(base + (k << s))];
 #pragma unroll
         for (int h = 1; h < R; h <<= 1) {
 #pragma unroll
@@ -44,7 +48,7 @@ __device__ __forceinline__ void hadamard_pass(float *buf, int P, int s, int tid)
             }
         }
 #pragma unroll
-        for (int k = 0; k < R; k++) buf[base + (k << s)] = v[k];
+        for (int k = 0; k < R; k++) buf[pad(base + (k << s))] = v[k];
     }
 }
 
@@ -60,7 +64,7 @@ __global__ __launch_bounds__(kHadThreads) void sign_hadamard_kernel(
     for (int i = tid; i < P; i += kHadThreads) {
         float v = half_bits_to_float(x[base + i]);
         if (!signs_after) v *= half_bits_to_float(s[i]);
-        buf[i] = v;
+        buf[pad(i)] = v;
     }
     __syncthreads();
     int stage = 0;
@@ -75,7 +79,7 @@ __global__ __launch_bounds__(kHadThreads) void sign_hadamard_kernel(
     if (rest) __syncthreads();
     const float scale = rsqrtf((float)P);
     for (int i = tid; i < P; i += kHadThreads) {
-        float v = buf[i] * scale;
+        float v = buf[pad(i)] * scale;
         if (signs_after) v *= half_bits_to_float(s[i]);
         out[base + i] = float_to_half_bits(v);
     }
@@ -84,7 +88,7 @@ __global__ __launch_bounds__(kHadThreads) void sign_hadamard_kernel(
 int prepare_hadamard()
 {
     return (int)hipFuncSetAttribute(reinterpret_cast<const void *>(sign_hadamard_kernel),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, kHadMaxBlock * 4);
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (kHadMaxBlock + kHadMaxBlock / 32) * 4);
 }
 
 }  // namespace rptc
@@ -114,6 +118,6 @@ extern "C" int rptc_sign_hadamard(const uint16_t *x, const uint16_t *signs, uint
     int log_p = 0;
     while (((int64_t)1 << log_p) < P) log_p++;
     hipLaunchKernelGGL(sign_hadamard_kernel, dim3((unsigned)(batch * blocks_per_row)), dim3(kHadThreads),
-                       (size_t)P * 4, s, x, signs, out, (int)n, (int)P, log_p, blocks_per_row, inverse ? 1 : 0);
+                       (size_t)(P + P / 32) * 4, s, x, signs, out, (int)n, (int)P, log_p, blocks_per_row, inverse ? 1 : 0);
     return t.end();
 }

@@ -65,6 +65,22 @@ class QuantizedLinear(torch.nn.Module):
         layer.codebook.copy_(torch.as_tensor(codebook, dtype=torch.float16).to(device))
         return layer
 
+    @classmethod
+    def from_weight(cls, weight, codebook=None, S=8, importance=None, seed=42, device="cuda"):
+        """Quantize a dense weight [out, in] with the Viterbi search of ``rptc_kernels.quantize`` (run on
+        ``device``) and pack the result.  codebook: fp16 [2^(S+1)] or None for a seeded Gaussian one
+        scaled to the weight's standard deviation."""
+        from rptc_kernels import quantize
+        W = torch.as_tensor(weight).to(device=device, dtype=torch.float32)
+        if codebook is None:
+            g = torch.Generator().manual_seed(seed)
+            codebook = (torch.randn(2 << S, generator=g) * W.std().item()).to(torch.float16)
+        codebook = torch.as_tensor(codebook, dtype=torch.float16)
+        symbols, mse = quantize.quantize_matrix(W, codebook.to(device), S, importance=importance)
+        layer = cls.from_symbols(symbols, codebook, W.size(0), S=S, device=device)
+        layer.quantization_mse = mse
+        return layer
+
     def set_affine(self, scales_out=None, scales_in=None, biases_out=None, biases_in=None):
         """The reference's row/column factorisation (quantize_hf.py:77-117,167); any may be None."""
         def prep(v, n):

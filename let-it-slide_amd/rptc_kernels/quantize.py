@@ -1,0 +1,110 @@
+"""Viterbi trellis quantizer for the hashed pair stream (torch, runs on CPU or GPU).
+
+Semantics follow the reference's quantizer (rptc.py:13-71, diag_only path): the trellis starts in
+state 0 (``rho[0] = 0``, rptc.py:55-56), a step shifts new symbol bits into the state
+(rptc.py:77-79), the path cost is the sum of per-step squared errors, and the best final state is
+traced back (rptc.py:60-65).  What differs is the decoder the path is optimised for: the one the
+inference kernels implement (inference.cu:250-262) — a 16-bit state, 4 bits per step, two weights
+per step looked up through ``hash = s*(s+1)`` — so that the symbols can be packed
+(``packing.pack_matvec``) and run by ``decompress_matvec_*`` in CONTINUOUS mode.  The reference
+itself never connects its quantizer to its kernels.
+
+The search is exact (full Viterbi over all 65 536 states); ties are broken by ``torch.min``'s first
+index, which need not match ``jnp.argmin`` of the reference bit for bit.
+"""
+import torch
+
+from . import packing
+
+STATE_BITS = 16
+STEP_BITS = 4
+
+
+def decode_table(codebook, S):
+    """[65536, 2] float32: the weight pair state s decodes to (inference.cu:250-262)."""
+    cb = torch.as_tensor(codebook).to(torch.float32).reshape(-1)
+    assert cb.numel() == 2 << S
+    s = torch.arange(1 << STATE_BITS, dtype=torch.int64, device=cb.device)
+    prod = s * (s + 1)
+    e = (prod >> 8) & ((1 << S) - 1)
+    sign = ((prod >> 15) & 1).to(torch.float32)
+    w0 = cb[2 * e].abs() * (1.0 - 2.0 * sign)      # the hash bit replaces the sign of the first value
+    w1 = cb[2 * e + 1]
+    return torch.stack([w0, w1], dim=1)
+
+
+def viterbi_pairs(targets, table, weights=None, state_bits=STATE_BITS, step_bits=STEP_BITS):
+    """Exact trellis search.  targets [rows, steps, 2] float; table [2^state_bits, 2]; weights None or
+    [rows, steps, 2] (per-weight importance, the diagonal of rptc.py's ``corrections``).
+    Returns (symbols int64 [rows, steps], cost float [rows])."""
+    rows, steps, _ = targets.shape
+    M, R = 1 << state_bits, 1 << step_bits
+    dev = targets.device
+    table = table.to(dev)
+    rho = torch.full((rows, M), float("inf"), device=dev)
+    rho[:, 0] = 0.0
+    back = torch.empty((steps, rows, M >> step_bits), dtype=torch.uint8, device=dev)
+    t0, t1 = table[:, 0].unsqueeze(0), table[:, 1].unsqueeze(0)
+    for t in range(steps):
+        # state s' = ((s << step_bits) | sym) & (M-1): its predecessors share the low bits s' >> step_bits
+        best, arg = rho.view(rows, R, M >> step_bits).min(dim=1)
+        back[t] = arg.to(torch.uint8)
+        d0 = targets[:, t, 0:1] - t0
+        d1 = targets[:, t, 1:2] - t1
+        if weights is None:
+            loss = d0 * d0 + d1 * d1
+        else:
+            loss = weights[:, t, 0:1] * d0 * d0 + weights[:, t, 1:2] * d1 * d1
+        rho = best.repeat_interleave(R, dim=1) + loss
+    cost, state = rho.min(dim=1)
+    symbols = torch.empty((rows, steps), dtype=torch.int64, device=dev)
+    r = torch.arange(rows, device=dev)
+    for t in range(steps - 1, -1, -1):
+        symbols[:, t] = state & (R - 1)
+        low = state >> step_bits
+        top = back[t, r, low].to(torch.int64)
+        state = (top << (state_bits - step_bits)) | low
+    return symbols, cost
+
+
+def quantize_matrix(W, codebook, S=8, importance=None, rows_per_batch=64):
+    """Quantize W [m, n] (n % 64 == 0) to 4-bit symbols [m, n/2] in stream order, for the decoder of
+    ``decompress_matvec_*`` in CONTINUOUS mode.  importance: optional [n] per-column weight (e.g. the
+    Hessian diagonal, quantize_hf.py:164).  Returns (symbols int64 [m, n/2] on the CPU, mse float)."""
+    W = torch.as_tensor(W)
+    m, n = W.shape
+    dev = W.device
+    table = decode_table(torch.as_tensor(codebook).to(dev), S)
+    cols = torch.from_numpy(packing.matvec_stream_columns(n)).to(dev)     # first column of every step
+    Wf = W.to(torch.float32)
+    targets = torch.stack([Wf[:, cols], Wf[:, cols + 1]], dim=2)          # [m, n/2, 2] in stream order
+    wts = None
+    if importance is not None:
+        imp = torch.as_tensor(importance, dtype=torch.float32, device=dev)
+        wts = torch.stack([imp[cols], imp[cols + 1]], dim=1).unsqueeze(0)
+    out = torch.empty((m, n // 2), dtype=torch.int64)
+    total = 0.0
+    for r0 in range(0, m, rows_per_batch):
+        tg = targets[r0:r0 + rows_per_batch]
+        w = None if wts is None else wts.expand(tg.size(0), -1, -1)
+        sym, cost = viterbi_pairs(tg, table, w)
+        out[r0:r0 + rows_per_batch] = sym.cpu()
+        total += cost.sum().item()
+    return out, total / (m * n)
+
+
+def dequantize_symbols(symbols, codebook, S=8):
+    """The dense matrix [m, n] a symbol array (stream order) decodes to, by walking the shift register
+    (rptc.py:74-85 with 4-bit steps and the hashed pair lookup): the definition the kernels are held to."""
+    symbols = torch.as_tensor(symbols, dtype=torch.int64)
+    m, half = symbols.shape
+    n = 2 * half
+    table = decode_table(torch.as_tensor(codebook), S)
+    cols = torch.from_numpy(packing.matvec_stream_columns(n))
+    state = torch.zeros(m, dtype=torch.int64)
+    W = torch.empty((m, n), dtype=torch.float32)
+    for p in range(half):
+        state = ((state << STEP_BITS) | symbols[:, p]) & ((1 << STATE_BITS) - 1)
+        W[:, cols[p]] = table[state, 0]
+        W[:, cols[p] + 1] = table[state, 1]
+    return W

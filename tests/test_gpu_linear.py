@@ -116,3 +116,22 @@ def test_patch_model_replaces_the_reference_module_list(rk):
     h = (torch.nn.functional.silu(x.float() @ Wg.t()).half().float() * (x.float() @ Wu.t()).half().float()).half().float()
     want = h @ Wd.t()
     assert rel_l2(y.float().cpu().numpy(), want.cpu().numpy()) < 5e-3
+
+
+def test_from_weight_quantizes_and_runs(rk):
+    """A real (small) weight through the Viterbi quantizer, the packer and the fused kernel: the layer
+    output equals the dense product of what the symbols decode to, and the quantization error is the
+    2-bit trellis code's, not a random matrix's."""
+    from rptc_kernels.linear import QuantizedLinear
+    from rptc_kernels import quantize
+    g = torch.Generator().manual_seed(5)
+    m, n = 16, 256
+    W = torch.randn((m, n), generator=g) * 0.02
+    layer = QuantizedLinear.from_weight(W, S=8)
+    What = layer.decoded_weight().float().cpu()
+    rel = ((W - What).norm() / W.norm()).item()
+    assert rel < 0.45, rel                    # ~0.3 for a 2 bit/weight trellis code on Gaussian data
+    x = torch.randn((1, n), generator=g).half().cuda()
+    y = layer(x)
+    want = x.double().cpu() @ What.double().t()
+    assert rel_l2(y.cpu().numpy(), want.numpy()) < 1e-3

@@ -1,0 +1,60 @@
+"""The Viterbi quantizer: optimal on a trellis small enough to enumerate, consistent with the decoder
+the kernels implement, and better than chance on a real-size state space."""
+import itertools
+
+import numpy as np
+import torch
+
+from rptc_kernels import packing, quantize
+
+
+def test_viterbi_is_optimal_on_a_small_trellis():
+    g = torch.Generator().manual_seed(0)
+    state_bits, step_bits, steps, rows = 6, 2, 6, 3
+    table = torch.randn((1 << state_bits, 2), generator=g)
+    targets = torch.randn((rows, steps, 2), generator=g)
+    sym, cost = quantize.viterbi_pairs(targets, table, state_bits=state_bits, step_bits=step_bits)
+    for r in range(rows):
+        best = None
+        for seq in itertools.product(range(1 << step_bits), repeat=steps):
+            state, c = 0, 0.0
+            for t, s in enumerate(seq):
+                state = ((state << step_bits) | s) & ((1 << state_bits) - 1)
+                c += float(((targets[r, t] - table[state]) ** 2).sum())
+            if best is None or c < best[0]:
+                best = (c, seq)
+        assert abs(best[0] - float(cost[r])) < 1e-4
+        # the returned path has the reported cost (ties may pick another optimal path)
+        state, c = 0, 0.0
+        for t in range(steps):
+            state = ((state << step_bits) | int(sym[r, t])) & ((1 << state_bits) - 1)
+            c += float(((targets[r, t] - table[state]) ** 2).sum())
+        assert abs(c - float(cost[r])) < 1e-4
+
+
+def test_decode_table_matches_the_oracle_hash(oracle):
+    cb = np.random.default_rng(1).standard_normal(512).astype(np.float16)
+    table = quantize.decode_table(torch.from_numpy(cb), 8).numpy()
+    for s in (0, 1, 0x00B5, 0x1234, 0xBEEF, 0xFFFF, 40000):
+        _, e, sign = oracle.hash_window(s, 8)
+        w0 = -abs(float(cb[2 * e])) if sign else abs(float(cb[2 * e]))
+        assert table[s, 0] == np.float32(w0) and table[s, 1] == np.float32(cb[2 * e + 1])
+
+
+def test_quantize_matrix_round_trip_through_the_packed_stream(oracle):
+    g = np.random.default_rng(2)
+    m, n, S = 4, 192, 8
+    W = g.standard_normal((m, n)).astype(np.float32)
+    cb = g.standard_normal(2 << S).astype(np.float16)
+    symbols, mse = quantize.quantize_matrix(torch.from_numpy(W), torch.from_numpy(cb), S)
+    assert symbols.shape == (m, n // 2) and int(symbols.max()) < 16
+    # the decoder walk, the packed stream decoded by the oracle, and the reported error all agree
+    What = quantize.dequantize_symbols(symbols, torch.from_numpy(cb), S).numpy()
+    stream = packing.pack_matvec(symbols.numpy())
+    Wor = oracle.matvec_dense(stream, cb, m, n, S, mode=oracle.CONTINUOUS).astype(np.float32)
+    assert np.array_equal(What, Wor)
+    assert abs(((W - What) ** 2).mean() - mse) < 1e-5
+    # a 2-bit/weight trellis code with a 256-pair random codebook is far better than random symbols
+    rand = quantize.dequantize_symbols(torch.from_numpy(g.integers(0, 16, (m, n // 2))), torch.from_numpy(cb), S).numpy()
+    assert mse < 0.25 * ((W - rand) ** 2).mean()
+    assert mse < 0.2          # unit-variance Gaussian at 2 bits/weight: rate-distortion bound 0.0625
