@@ -57,7 +57,7 @@ def parse():
 class Runner:
     """Launches the op through the C ABI with pre-bound arguments (no timing, asynchronous)."""
 
-    def __init__(self, m, n, S, copies, seed=42):
+    def __init__(self, m, n, S, copies, seed=42, bits=2):
         import torch
         import rptc_kernels
         self.torch = torch
@@ -66,22 +66,28 @@ class Runner:
         rc = self.lib.rptc_init()
         if rc:
             raise RuntimeError(self.lib.rptc_status_string(rc).decode())
-        self.fn = getattr(self.lib, f"rptc_decompress_matvec_16_{S}_1")
+        self.bits = bits
+        self.fn = getattr(self.lib, f"rptc_decompress_matvec_16_{S}_1") if bits == 2 else None
         g = torch.Generator(device="cuda")
         g.manual_seed(seed)
-        words = m * n // 16
+        words = m * n * bits // 32
         self.weights = [torch.randint(-(1 << 31), 1 << 31, (words,), generator=g, dtype=torch.int64,
                                       device="cuda").to(torch.int32) for _ in range(copies)]
         self.codebook = torch.randn(2 << S, generator=g, device="cuda").to(torch.float16)
         self.x = torch.randn(n, generator=g, device="cuda").to(torch.float16)
         self.out = torch.zeros(m, dtype=torch.float16, device="cuda")
-        self.bytes = m * n * 2 // 8
+        self.bytes = m * n * bits // 8
         torch.cuda.synchronize()
 
     def launch(self, k, stream):
         w = self.weights[k % len(self.weights)]
-        rc = self.fn(w.data_ptr(), self.codebook.data_ptr(), self.x.data_ptr(), self.out.data_ptr(),
-                     self.m, self.n, 0, ctypes.c_void_p(stream), None)
+        if self.bits == 2:
+            rc = self.fn(w.data_ptr(), self.codebook.data_ptr(), self.x.data_ptr(), self.out.data_ptr(),
+                         self.m, self.n, 0, ctypes.c_void_p(stream), None)
+        else:
+            rc = self.lib.rptc_decompress_matvec_bits(w.data_ptr(), self.codebook.data_ptr(), self.x.data_ptr(),
+                                                      self.out.data_ptr(), self.m, self.n, self.S, self.bits, 0,
+                                                      ctypes.c_void_p(stream), None)
         if rc:
             raise RuntimeError(self.lib.rptc_status_string(rc).decode())
 
@@ -124,7 +130,7 @@ class Runner:
         torch = self.torch
         import rptc_kernels
         W = torch.zeros((self.m, self.n), dtype=torch.float16, device="cuda")
-        rptc_kernels.matvec_dense(self.weights[0], self.codebook, W, self.S)
+        rptc_kernels.matvec_bits_dense(self.weights[0], self.codebook, W, self.bits)
         self.launch(0, torch.cuda.current_stream().cuda_stream)
         torch.cuda.synchronize()
         want = W.double() @ self.x.double()
@@ -376,6 +382,16 @@ def main():
                                  "frac": round(r.bytes / us / 1e3 / HBM_PEAK_GBS, 4)}
             del r
             torch.cuda.empty_cache()
+        for bits in (3, 4):
+            for (m, n) in ((4096, 11008), (11008, 4096)):
+                r = Runner(m, n, a.S, max(2, min(a.copies, (512 << 20) // (m * n * bits // 8) + 1)), bits=bits)
+                r.check()
+                _, ms = r.run(a.steps, a.warmup, a.launch)
+                us = ms / a.steps * 1e3
+                extra[f"{m}x{n} {bits}b"] = {"launch_us": round(us, 3), "GBps": round(r.bytes / us / 1e3, 1),
+                                            "frac": round(r.bytes / us / 1e3 / HBM_PEAK_GBS, 4)}
+                del r
+                torch.cuda.empty_cache()
         line["other_shapes"] = extra
     if not a.no_cpu:
         line["cpu_baseline"] = cpu_baseline(runner)

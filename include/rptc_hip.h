@@ -135,6 +135,21 @@ int rptc_decompress_matmul(const int32_t *compressed, const uint16_t *codebook, 
                            void *stream, float *ms);
 
 /*
+ * The hashed pair stream at `bits` = 2, 3 or 4 bits per weight, S in {6, 8}.  No counterpart in
+ * the reference for 3 and 4 (all its kernels are 2 bits/weight); bits == 2 is exactly
+ * rptc_decompress_matvec_16_{S}_1.  A step still emits two weights through the same hash of a
+ * 16-bit window but consumes 2*bits stream bits; an element still holds 32 steps, so it is
+ * 2*bits words long and the stream is int32 [n/2048][m][32][2*bits] (+ ragged slab
+ * [m][(n % 2048)/64][2*bits]), m*n*bits/32 words.  x, out, accumulation as for the mat-vec.
+ * rptc_matvec_bits_dense writes the dense fp16 matrix W [m][n] such a stream stands for.
+ */
+int rptc_decompress_matvec_bits(const int32_t *compressed, const uint16_t *codebook, const uint16_t *x,
+                                uint16_t *out, int64_t m, int64_t n, int S, int bits, int carry_mode,
+                                void *stream, float *ms);
+int rptc_matvec_bits_dense(const int32_t *compressed, const uint16_t *codebook, uint16_t *W, int64_t m,
+                           int64_t n, int S, int bits, int carry_mode, void *stream, float *ms);
+
+/*
  * Random-sign Hadamard (incoherence) transform on activations, fp16 in and out, fp32 inside.
  * No counterpart in the reference (quantize_hf.py:77-117 conditions weights by a scale-and-bias
  * factorisation instead).  Each row of x [batch][n] is cut into blocks of `block` elements

@@ -35,7 +35,6 @@ namespace rptc {
 constexpr int kMatvecThreads = 1024;
 constexpr int kMatvecWaves = kMatvecThreads / kWave;
 constexpr int kTableBytes = 256 * 256;     // 256 rows of 64 lane copies of one half2
-constexpr int kBatch = 4;                  // stream elements in flight per lane
 
 struct Geometry {
     int m, n, T, Lt, slabs;
@@ -64,11 +63,74 @@ __device__ __forceinline__ uint32_t table_value(const uint32_t *__restrict__ cod
 
 // A stream element is read exactly once: load it with the non-temporal hint.  The address is a
 // wave-uniform base plus 16 bytes per lane, so no vector address arithmetic is needed.
-__device__ __forceinline__ uint4 load_stream(const uint4 *wave_base, int lane)
+// An element is 2 * BITS words: 4 at 2 bits per weight (the reference format), 6 at 3, 8 at 4.
+template <int WORDS>
+struct Elem {
+    uint32_t w[WORDS];
+};
+
+template <int WORDS>
+__device__ __forceinline__ Elem<WORDS> load_stream(const uint32_t *wave_base, int lane)
 {
     typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-    const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(wave_base) + lane);
-    return make_uint4(v.x, v.y, v.z, v.w);
+    typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+    Elem<WORDS> e;
+    const uint32_t *p = wave_base + lane * WORDS;
+    if constexpr (WORDS % 4 == 0) {
+#pragma unroll
+        for (int i = 0; i < WORDS / 4; i++) {
+            const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p) + i);
+            e.w[4 * i] = v.x, e.w[4 * i + 1] = v.y, e.w[4 * i + 2] = v.z, e.w[4 * i + 3] = v.w;
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < WORDS / 2; i++) {
+            const u32x2 v = __builtin_nontemporal_load(reinterpret_cast<const u32x2 *>(p) + i);
+            e.w[2 * i] = v.x, e.w[2 * i + 1] = v.y;
+        }
+    }
+    return e;
+}
+
+// Step s of an element reads slot 4k + j with k = 7, 0, 4, 1, 5, 2, 6, 3 for s / 4 = 0..7, j = s % 4
+// (inference.cu:237-250: which of reg_c[0..7] holds the window that ends 4(s+1) bits in).
+__host__ __device__ constexpr int slot_of_step(int s)
+{
+    constexpr int k_of[8] = {7, 0, 4, 1, 5, 2, 6, 3};
+    return 4 * k_of[s / 4] + s % 4;
+}
+
+// All 32 steps of one element at 3 or 4 bits per weight (a step consumes 2 * BITS stream bits; the
+// window is the 16 bits that end 2 * BITS * (s + 1) bits into the element, the previous lane's last
+// 16 bits in front).  Plain C++: the shifts are compile-time constants.
+template <int BITS>
+__device__ __forceinline__ float decode_element_bits(const Elem<2 * BITS> &e, uint32_t carry, uint32_t lane4,
+                                                     const uint32_t (&xr)[32])
+{
+    constexpr int SB = 2 * BITS;
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s0 = 0; s0 < 32; s0 += 8) {
+        uint32_t wv[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            const int s = s0 + u;
+            const int end = SB * (s + 1), start = end - 16;
+            uint32_t h;
+            if (start < 0) {
+                h = (carry << end) | (e.w[0] >> (32 - end));
+            } else {
+                const int wi = start >> 5, o = start & 31;
+                h = o <= 16 ? e.w[wi] >> (16 - o) : alignbit(e.w[wi], e.w[wi + 1 < 2 * BITS ? wi + 1 : wi], 48 - o);
+            }
+            h &= 0xFFFFu;
+            const uint32_t prod = __umul24(h, h) + h;                 // low 16 bits of h * (h + 1)
+            wv[u] = lds_read_abs(and_or(prod, 0xFF00u, lane4));
+        }
+#pragma unroll
+        for (int u = 0; u < 8; u++) acc[u & 3] = dot2(wv[u], xr[slot_of_step(s0 + u)], acc[u & 3]);
+    }
+    return (acc[0] + acc[1]) + (acc[2] + acc[3]);
 }
 
 // What a wave needs to know about the slab it is working on.  A wave item is 64 consecutive
@@ -89,14 +151,16 @@ struct MatvecArgs {
     int items_tail;       // items of the ragged slab            = ceil(rows_per_block / rw_tail)
 };
 
-template <int S, int MODE>
+template <int S, int MODE, int BITS>
 __global__ __launch_bounds__(kMatvecThreads) void matvec_kernel(
-    const uint4 *__restrict__ comp, const uint32_t *__restrict__ codebook,
+    const uint32_t *__restrict__ comp, const uint32_t *__restrict__ codebook,
     const uint4 *__restrict__ x, uint16_t *__restrict__ out, int arg_m, int arg_n, int arg_rows_per_block,
     int arg_rw_tail, int arg_items_full, int arg_items_tail)
 {
     // separate scalar arguments (not a struct) so that all of them are preloaded into SGPRs
     const MatvecArgs a = {arg_m, arg_n, arg_rows_per_block, arg_rw_tail, arg_items_full, arg_items_tail};
+    constexpr int WORDS = 2 * BITS;                        // words per stream element
+    constexpr int kBatch = BITS == 2 ? 4 : 2;              // stream elements in flight per lane
     extern __shared__ uint32_t lds[];
     RPTC_STAMP(0);
     const int m = a.m, n = a.n;
@@ -156,25 +220,26 @@ __global__ __launch_bounds__(kMatvecThreads) void matvec_kernel(
     // cursor of the loads and cursor of the decode (slab, item index inside the slab)
     int ld_slab = first_slab, ld_idx = first_idx;
     SlabView ld = view(ld_slab);
-    uint4 buf[kBatch];
+    Elem<WORDS> buf[kBatch];
     uint32_t cw[kBatch];
     auto load_batch = [&](int base) {
 #pragma unroll
         for (int u = 0; u < kBatch; u++) {
-            buf[u] = make_uint4(0, 0, 0, 0);
+#pragma unroll
+            for (int i = 0; i < WORDS; i++) buf[u].w[i] = 0;
             cw[u] = 0;
             if (base + u < it_end) {
                 const int row_first = ld_idx * ld.rows_per_item;           // row inside the block
                 const int rows_here = min(ld.rows_per_item, rows - row_first);
                 if (lane < rows_here * ld.lanes) {
-                    const uint4 *wave_base = comp + ld.elem0 + (size_t)(row0 + row_first) * ld.lanes;
-                    buf[u] = load_stream(wave_base, lane);
+                    const uint32_t *wave_base = comp + (ld.elem0 + (size_t)(row0 + row_first) * ld.lanes) * WORDS;
+                    buf[u] = load_stream<WORDS>(wave_base, lane);
                     if (MODE == RPTC_CONTINUOUS && ld_slab > 0) {
                         // the word in front of a row: last word of the row's lane 31 in the slab before
                         const int sub = ld_slab < T ? lane >> 5 : lane / ld.lanes;
                         const int l = lane - sub * ld.lanes;
                         if (l == 0)
-                            cw[u] = comp[((size_t)(ld_slab - 1) * m + row0 + row_first + sub) * 32 + 31].w;
+                            cw[u] = comp[(((size_t)(ld_slab - 1) * m + row0 + row_first + sub) * 32 + 31) * WORDS + WORDS - 1];
                     }
                 }
                 if (++ld_idx == ld.items) {
@@ -214,7 +279,7 @@ __global__ __launch_bounds__(kMatvecThreads) void matvec_kernel(
     int l = 0, sub = 0;                     // this lane's element inside a row, row inside the item
     uint32_t part_lane = 0;                 // LDS byte address of this lane's partial for row 0
     for (int base = it_begin; base < it_end; base += kBatch) {
-        uint4 cur[kBatch];
+        Elem<WORDS> cur[kBatch];
         uint32_t ccw[kBatch];
 #pragma unroll
         for (int u = 0; u < kBatch; u++) {
@@ -253,14 +318,21 @@ __global__ __launch_bounds__(kMatvecThreads) void matvec_kernel(
             const bool active = sub < sv.rows_per_item && row_first + sub < rows;
             // Previous lane's last word.  Lane 0 of a row keeps its own as written
             // (inference.cu:232: the shuffle hands lane 0 its own value back).
-            uint32_t carry = __builtin_amdgcn_update_dpp(0u, cur[u].w, 0x138 /* wave_shr:1 */, 0xF, 0xF, false);
-            if (l == 0) carry = MODE == RPTC_CONTINUOUS ? ccw[u] : cur[u].w;
-            float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
-            decode_element_asm(cur[u], carry, lane4, xr, a0, a1, a2, a3);
+            const uint32_t last = cur[u].w[WORDS - 1];
+            uint32_t carry = __builtin_amdgcn_update_dpp(0u, last, 0x138 /* wave_shr:1 */, 0xF, 0xF, false);
+            if (l == 0) carry = MODE == RPTC_CONTINUOUS ? ccw[u] : last;
+            float sum;
+            if constexpr (BITS == 2) {
+                float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+                decode_element_asm(make_uint4(cur[u].w[0], cur[u].w[1], cur[u].w[2], cur[u].w[3]), carry, lane4, xr,
+                                   a0, a1, a2, a3);
+                sum = (a0 + a1) + (a2 + a3);
+            } else {
+                sum = decode_element_bits<BITS>(cur[u], carry, lane4, xr);
+            }
             if (active) {
                 typedef __attribute__((address_space(3))) float lds_float;
-                *reinterpret_cast<lds_float *>(static_cast<uintptr_t>(part_lane + 4u * (uint32_t)(row_first * npr))) =
-                    (a0 + a1) + (a2 + a3);
+                *reinterpret_cast<lds_float *>(static_cast<uintptr_t>(part_lane + 4u * (uint32_t)(row_first * npr))) = sum;
             }
             if (base + u == it_begin) RPTC_STAMP(3);
             if (++idx == sv.items) {
@@ -323,7 +395,7 @@ static int matvec_lds_bytes(int n, int rows_per_block)
     return kTableBytes + 2 * n + 4 * (n / 64) * rows_per_block;
 }
 
-template <int S>
+template <int S, int BITS = 2>
 static int launch_matvec(const int32_t *compressed, const uint16_t *codebook, const uint16_t *x,
                          uint16_t *out, int64_t m, int64_t n, int carry_mode, void *stream, float *ms)
 {
@@ -358,16 +430,69 @@ static int launch_matvec(const int32_t *compressed, const uint16_t *codebook, co
     Timer t;
     rc = t.begin(dev, s, ms);
     if (rc) return rc;
-    auto a_comp = reinterpret_cast<const uint4 *>(compressed);
+    auto a_comp = reinterpret_cast<const uint32_t *>(compressed);
     auto a_cb = reinterpret_cast<const uint32_t *>(codebook);
     auto a_x = reinterpret_cast<const uint4 *>(x);
     if (carry_mode == RPTC_AS_WRITTEN)
-        hipLaunchKernelGGL((matvec_kernel<S, RPTC_AS_WRITTEN>), dim3(grid), dim3(kMatvecThreads), lds_bytes, s,
+        hipLaunchKernelGGL((matvec_kernel<S, RPTC_AS_WRITTEN, BITS>), dim3(grid), dim3(kMatvecThreads), lds_bytes, s,
                            a_comp, a_cb, a_x, out, a.m, a.n, a.rows_per_block, a.rw_tail, a.items_full, a.items_tail);
     else
-        hipLaunchKernelGGL((matvec_kernel<S, RPTC_CONTINUOUS>), dim3(grid), dim3(kMatvecThreads), lds_bytes, s,
+        hipLaunchKernelGGL((matvec_kernel<S, RPTC_CONTINUOUS, BITS>), dim3(grid), dim3(kMatvecThreads), lds_bytes, s,
                            a_comp, a_cb, a_x, out, a.m, a.n, a.rows_per_block, a.rw_tail, a.items_full, a.items_tail);
     return t.end();
+}
+
+// Dense export at 3 and 4 bits per weight: one thread per stream element.
+template <int S, int MODE, int BITS>
+__global__ __launch_bounds__(256) void bits_dense_kernel(
+    const uint32_t *__restrict__ comp, const uint32_t *__restrict__ codebook, uint32_t *__restrict__ W,
+    int m, int n, int slab, int slab_elems)
+{
+    constexpr int WORDS = 2 * BITS, SB = 2 * BITS;
+    const Geometry g(m, n);
+    const int lanes = g.lanes(slab);
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= slab_elems) return;
+    const int row = i / lanes, l = i - row * lanes;
+    const uint32_t *ep = comp + g.elem(slab, row, l) * WORDS;
+    uint32_t w[WORDS];
+#pragma unroll
+    for (int q = 0; q < WORDS; q++) w[q] = ep[q];
+    uint32_t carry;
+    if (l > 0) carry = ep[-1];
+    else if (MODE == RPTC_AS_WRITTEN) carry = w[WORDS - 1];
+    else carry = slab > 0 ? comp[g.elem(slab - 1, row, 31) * WORDS + WORDS - 1] : 0u;
+    const int n8 = n >> 3;
+    uint32_t *wrow = W + (size_t)row * (n >> 1);
+#pragma unroll
+    for (int s = 0; s < 32; s++) {
+        const int end = SB * (s + 1), start = end - 16;
+        uint32_t h;
+        if (start < 0) {
+            h = (carry << end) | (w[0] >> (32 - end));
+        } else {
+            const int wi = start >> 5, o = start & 31;
+            h = o <= 16 ? w[wi] >> (16 - o) : alignbit(w[wi], w[wi + 1 < WORDS ? wi + 1 : wi], 48 - o);
+        }
+        h &= 0xFFFFu;
+        const uint32_t hash = h * (h + 1u);
+        const uint32_t pair = codebook[(hash >> 8) & ((1u << S) - 1u)];
+        const uint32_t val = (pair & 0xFFFF7FFFu) | (hash & 0x8000u);
+        const int P = g.slot(slab, slot_of_step(s), l);
+        const int ii = P / n8, idx = P - ii * n8;
+        wrow[4 * idx + ii] = val;
+    }
+}
+
+template <int S, int MODE, int BITS>
+static void launch_bits_dense_slabs(const uint32_t *comp, const uint32_t *cb, uint32_t *W, int m, int n, hipStream_t s)
+{
+    const Geometry g(m, n);
+    for (int slab = 0; slab < g.slabs; slab++) {
+        const int elems = m * g.lanes(slab);
+        hipLaunchKernelGGL((bits_dense_kernel<S, MODE, BITS>), dim3((elems + 255) / 256), dim3(256), 0, s,
+                           comp, cb, W, m, n, slab, elems);
+    }
 }
 
 template <int S, int MODE>
@@ -391,10 +516,15 @@ static int set_lds_limit(F *kernel)
 int prepare_matvec()
 {
     int rc;
-    if ((rc = set_lds_limit(matvec_kernel<6, RPTC_AS_WRITTEN>))) return rc;
-    if ((rc = set_lds_limit(matvec_kernel<6, RPTC_CONTINUOUS>))) return rc;
-    if ((rc = set_lds_limit(matvec_kernel<8, RPTC_AS_WRITTEN>))) return rc;
-    if ((rc = set_lds_limit(matvec_kernel<8, RPTC_CONTINUOUS>))) return rc;
+#define RPTC_SET_LIMITS(BITS)                                                               \
+    if ((rc = set_lds_limit(matvec_kernel<6, RPTC_AS_WRITTEN, BITS>))) return rc;              \
+    if ((rc = set_lds_limit(matvec_kernel<6, RPTC_CONTINUOUS, BITS>))) return rc;              \
+    if ((rc = set_lds_limit(matvec_kernel<8, RPTC_AS_WRITTEN, BITS>))) return rc;              \
+    if ((rc = set_lds_limit(matvec_kernel<8, RPTC_CONTINUOUS, BITS>))) return rc;
+    RPTC_SET_LIMITS(2)
+    RPTC_SET_LIMITS(3)
+    RPTC_SET_LIMITS(4)
+#undef RPTC_SET_LIMITS
     return 0;
 }
 
@@ -449,5 +579,47 @@ extern "C" int rptc_matvec_dense(const int32_t *compressed, const uint16_t *code
     else if (S == 6) launch_dense_slabs<6, RPTC_CONTINUOUS>(a_comp, a_cb, a_w, (int)m, (int)n, s);
     else if (aw) launch_dense_slabs<8, RPTC_AS_WRITTEN>(a_comp, a_cb, a_w, (int)m, (int)n, s);
     else launch_dense_slabs<8, RPTC_CONTINUOUS>(a_comp, a_cb, a_w, (int)m, (int)n, s);
+    return t.end();
+}
+
+extern "C" int rptc_decompress_matvec_bits(const int32_t *c, const uint16_t *cb, const uint16_t *x, uint16_t *out,
+                                           int64_t m, int64_t n, int S, int bits, int mode, void *stream, float *ms)
+{
+    if ((S != 6 && S != 8) || bits < 2 || bits > 4) return RPTC_ESHAPE;
+    if (bits == 2) return S == 6 ? launch_matvec<6, 2>(c, cb, x, out, m, n, mode, stream, ms)
+                                 : launch_matvec<8, 2>(c, cb, x, out, m, n, mode, stream, ms);
+    if (bits == 3) return S == 6 ? launch_matvec<6, 3>(c, cb, x, out, m, n, mode, stream, ms)
+                                 : launch_matvec<8, 3>(c, cb, x, out, m, n, mode, stream, ms);
+    return S == 6 ? launch_matvec<6, 4>(c, cb, x, out, m, n, mode, stream, ms)
+                  : launch_matvec<8, 4>(c, cb, x, out, m, n, mode, stream, ms);
+}
+
+extern "C" int rptc_matvec_bits_dense(const int32_t *compressed, const uint16_t *codebook, uint16_t *W, int64_t m,
+                                      int64_t n, int S, int bits, int carry_mode, void *stream, float *ms)
+{
+    if (bits == 2) return rptc_matvec_dense(compressed, codebook, W, m, n, S, carry_mode, stream, ms);
+    if (!compressed || !codebook || !W) return RPTC_ENULL;
+    if (m < 1 || n < 64 || n % 64 != 0 || (S != 6 && S != 8) || (bits != 3 && bits != 4)) return RPTC_ESHAPE;
+    if (carry_mode != RPTC_AS_WRITTEN && carry_mode != RPTC_CONTINUOUS) return RPTC_EMODE;
+    if (!aligned16(compressed) || !aligned16(codebook) || !aligned16(W)) return RPTC_EALIGN;
+    if (m >= (1 << 24) || n >= (1 << 20) || m * 32 >= ((int64_t)1 << 31)) return RPTC_ELIMIT;
+    DeviceInfo *dev;
+    int rc = device_info(&dev);
+    if (rc) return rc;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    Timer t;
+    rc = t.begin(dev, s, ms);
+    if (rc) return rc;
+    auto a_comp = reinterpret_cast<const uint32_t *>(compressed);
+    auto a_cb = reinterpret_cast<const uint32_t *>(codebook);
+    auto a_w = reinterpret_cast<uint32_t *>(W);
+    const bool aw = carry_mode == RPTC_AS_WRITTEN;
+#define RPTC_DENSE(SS, BB)                                                                          \
+    if (S == SS && bits == BB) {                                                                    \
+        if (aw) launch_bits_dense_slabs<SS, RPTC_AS_WRITTEN, BB>(a_comp, a_cb, a_w, (int)m, (int)n, s); \
+        else launch_bits_dense_slabs<SS, RPTC_CONTINUOUS, BB>(a_comp, a_cb, a_w, (int)m, (int)n, s);    \
+    }
+    RPTC_DENSE(6, 3) RPTC_DENSE(6, 4) RPTC_DENSE(8, 3) RPTC_DENSE(8, 4)
+#undef RPTC_DENSE
     return t.end();
 }

@@ -53,6 +53,8 @@ _SIGNATURES = {
     "rptc_matvec_t_dense": ([_VP, _VP, _VP, _I64, _I64, _INT, _INT, _VP, _FP], _INT),
     "rptc_decompress_matmul": ([_VP, _VP, _VP, _VP, _I64, _I64, _I64, _INT, _INT, _VP, _FP], _INT),
     "rptc_sign_hadamard": ([_VP, _VP, _VP, _I64, _I64, _I64, _INT, _VP, _FP], _INT),
+    "rptc_decompress_matvec_bits": ([_VP, _VP, _VP, _VP, _I64, _I64, _INT, _INT, _INT, _VP, _FP], _INT),
+    "rptc_matvec_bits_dense": ([_VP, _VP, _VP, _I64, _I64, _INT, _INT, _INT, _VP, _FP], _INT),
 }
 
 
@@ -340,3 +342,42 @@ def sign_hadamard(x, signs, out, block=0, inverse=False):
                                           ctypes.byref(ms) if _timing else None)
     _status(rc)
     return float(ms.value)
+
+
+def decompress_matvec_bits(compressed, codebook, x, out, bits):
+    """out = W x for the hashed pair stream at ``bits`` (2, 3, 4) bits per weight; S from the codebook length.
+
+    compressed int32 with m*n*bits/32 words ([n/2048, m, 32, 2*bits] + ragged slab); bits == 2 is
+    decompress_matvec_16_{S}_1."""
+    _check(bits in (2, 3, 4), "bits must be 2, 3 or 4")
+    _check_input(compressed, "compressed")
+    _check(compressed.dtype == torch.int32, "compressed.scalar_type() == torch::kInt32")
+    _check_input(codebook, "codebook")
+    _check(codebook.dim() == 1 and codebook.size(0) in (128, 512), "codebook.size(0) == 1<<(S+V), S in {6, 8}")
+    _check(codebook.dtype == torch.float16, "codebook.scalar_type() == torch::kFloat16")
+    S = 6 if codebook.size(0) == 128 else 8
+    _check_input(x, "x")
+    _check(x.dim() == 1 and x.dtype == torch.float16, "x must be a 1-D fp16 tensor")
+    _check_input(out, "out")
+    _check(out.dim() == 1 and out.dtype == torch.float16, "out must be a 1-D fp16 tensor")
+    n, m = x.size(0), out.size(0)
+    _check(n % 64 == 0 and n >= 64 and m >= 1, "x.size(0) % 64 == 0")
+    _check(compressed.numel() * 32 == m * n * bits, "compressed.numel() * 32 == m * n * bits")
+    return _call(library().rptc_decompress_matvec_bits, (compressed, codebook, x, out), m, n, S, bits)
+
+
+def matvec_bits_dense(compressed, codebook, out, bits):
+    """Write the dense fp16 [m, n] matrix of a hashed pair stream at ``bits`` bits per weight into ``out``."""
+    _check(bits in (2, 3, 4), "bits must be 2, 3 or 4")
+    _check_input(compressed, "compressed")
+    _check(compressed.dtype == torch.int32, "compressed.scalar_type() == torch::kInt32")
+    _check_input(codebook, "codebook")
+    _check(codebook.dim() == 1 and codebook.size(0) in (128, 512), "codebook.size(0) == 1<<(S+V), S in {6, 8}")
+    _check(codebook.dtype == torch.float16, "codebook.scalar_type() == torch::kFloat16")
+    S = 6 if codebook.size(0) == 128 else 8
+    _check_input(out, "out")
+    _check(out.dim() == 2 and out.dtype == torch.float16, "out must be a 2-D fp16 tensor")
+    m, n = out.shape
+    _check(n % 64 == 0 and m >= 1 and n >= 64, "out.size(1) % 64 == 0")
+    _check(compressed.numel() * 32 == m * n * bits, "compressed.numel() * 32 == m * n * bits")
+    return _call(library().rptc_matvec_bits_dense, (compressed, codebook, out), m, n, S, bits)

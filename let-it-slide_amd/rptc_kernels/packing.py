@@ -62,8 +62,22 @@ def matvec_stream_columns(n):
     return np.concatenate(cols).astype(np.int64)
 
 
-def pack_matvec(symbols):
-    """4-bit symbols [m, n/2] in stream order -> the stream of ``decompress_matvec_*``: int32 [m*n/16].
+def _element_words(symbols, step_bits):
+    """[..., 32 k] symbols of `step_bits` bits -> [..., k * step_bits] uint32: every 32 symbols become one
+    element of step_bits words, first symbol in the top bits of the first word."""
+    s = np.asarray(symbols, dtype=np.uint32)
+    assert s.shape[-1] % 32 == 0 and (s < (1 << step_bits)).all()
+    shifts = np.arange(step_bits - 1, -1, -1, dtype=np.uint32)
+    bits = ((s[..., None] >> shifts) & 1).astype(np.uint8).reshape(s.shape[:-1] + (s.shape[-1] * step_bits,))
+    packed = np.packbits(bits, axis=-1, bitorder="big")
+    return np.ascontiguousarray(packed).view(">u4").astype(np.uint32)
+
+
+def pack_matvec(symbols, bits=2):
+    """Symbols of 2*bits bits [m, n/2] in stream order -> the hashed pair stream: int32 [m*n*bits/32].
+
+    bits == 2 is the stream of ``decompress_matvec_*`` (4-bit symbols); bits 3 and 4 (6- and 8-bit symbols) are
+    this library's extension, elements of 2*bits words.
 
     Row r's p-th symbol is step p % 32 of lane (p // 32) % lanes of slab p // 1024; the flat result
     is [n/2048][m][32][4] followed by the ragged slab [m][Lt][4] (reshape to [n/2048, m, 128] when
@@ -74,11 +88,12 @@ def pack_matvec(symbols):
     n = 2 * half
     assert n % 64 == 0
     T, Lt = n // 2048, (n % 2048) // 64
-    words = _words_from_symbols(symbols, 4)           # [m, n/16]: 4 words per element, elements in stream order
+    wpe = 2 * bits                                     # words per element
+    words = _element_words(symbols, 2 * bits)          # [m, n/64 * wpe]: elements in stream order
     parts = []
     if T:
-        full = words[:, :T * 128].reshape(m, T, 128)
+        full = words[:, :T * 32 * wpe].reshape(m, T, 32 * wpe)
         parts.append(np.ascontiguousarray(full.transpose(1, 0, 2)).reshape(-1))
     if Lt:
-        parts.append(np.ascontiguousarray(words[:, T * 128:]).reshape(-1))
+        parts.append(np.ascontiguousarray(words[:, T * 32 * wpe:]).reshape(-1))
     return np.concatenate(parts).view(np.int32)

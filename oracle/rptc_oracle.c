@@ -27,7 +27,7 @@
  *   orc_lite_index_fn /   hand-computed known answers; PARITY UNPINNED beyond
  *   orc_lite_dequantize   those (the reference holds no vectors and its
  *                         Python needs jax, which is not installed)
- *   orc_matvec (ragged n), orc_decompress_bits, orc_sign_hadamard: formats and
+ *   orc_matvec (ragged n), orc_bits_dense, orc_sign_hadamard: formats and
  *                         ops of this build with no counterpart in the
  *                         reference; pinned by closed forms only.
  * The reference holds no golden vectors for any of these, so none is pinned by
@@ -371,6 +371,61 @@ int orc_matvec_dense(const uint32_t *compressed, const uint16_t *codebook,
                 for (int s = 0; s < 32; s++) {
                     uint32_t h = 0;
                     for (int b = 0; b < 16; b++) h = (h << 1) | bits[4 * (s + 1) + b];
+                    int k = k_of_s[s / 4], j = s % 4;
+                    int64_t P = (t < g.T) ? (((8 * t + k) * 4 + j) * 32 + l)
+                                          : (1024 * g.T + (4 * k + j) * g.Lt + l);
+                    int64_t i = P / n8, idx = P % n8;
+                    uint16_t w0, w1;
+                    pair_of_window(h, S, codebook, &w0, &w1);
+                    W[r * n + 8 * idx + 2 * i] = w0;
+                    W[r * n + 8 * idx + 2 * i + 1] = w1;
+                }
+            }
+        }
+    }
+    return 0;
+}
+
+/* ------------------------------ hashed pair stream at 3 and 4 bits per weight */
+
+/*
+ * No counterpart in the reference (all its kernels are 2 bits/weight; rptc_lite.py:63-73 has a
+ * general R only as JAX, with another hash).  The 2-bit stream generalised: a step still emits
+ * two weights through the same hash of a 16-bit window, but consumes 2*bits stream bits, and an
+ * element (one lane of one row of one slab) still holds 32 steps = 64 weights, so it is
+ * 4*bits/2 words long: 4 words at 2 bits, 6 at 3 bits, 8 at 4 bits.  Layout
+ * [slab][row][32 lanes][words] + ragged slab [row][Lt][words]; step s reads the window that
+ * ends 2*bits*(s+1) bits into the element, the previous lane's last 16 bits in front; steps map
+ * to (k, j) and to activation slots exactly as at 2 bits.  bits == 2 is the reference format.
+ */
+int orc_bits_dense(const uint32_t *compressed, const uint16_t *codebook, uint16_t *W,
+                   int64_t m, int64_t n, int S, int bits, int mode)
+{
+    geom_t g;
+    if (make_geom(&g, m, n) || bits < 2 || bits > 4) return -1;
+    const int64_t n8 = n / 8, words = 2 * bits, step_bits = 2 * bits;
+    const int64_t slabs = g.T + (g.Lt ? 1 : 0);
+    static const int k_of_s[8] = {7, 0, 4, 1, 5, 2, 6, 3};
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < m; r++) {
+        for (int64_t t = 0; t < slabs; t++) {
+            int64_t lanes = (t < g.T) ? 32 : g.Lt;
+            for (int64_t l = 0; l < lanes; l++) {
+#define ORC_BITS_ELEM(tt, rr, ll) (compressed + (((tt) < g.T) ? (((tt) * g.m + (rr)) * 32 + (ll)) * words \
+                                                             : g.T * g.m * 32 * words + ((rr) * g.Lt + (ll)) * words))
+                const uint32_t *e = ORC_BITS_ELEM(t, r, l);
+                uint32_t carry;
+                if (l > 0) carry = ORC_BITS_ELEM(t, r, l - 1)[words - 1];
+                else if (mode == ORC_AS_WRITTEN) carry = e[words - 1];
+                else carry = t > 0 ? ORC_BITS_ELEM(t - 1, r, 31)[words - 1] : 0;
+#undef ORC_BITS_ELEM
+                uint8_t bitstr[16 + 256];
+                for (int b = 0; b < 16; b++) bitstr[b] = (carry >> (15 - b)) & 1u;
+                for (int q = 0; q < words; q++)
+                    for (int b = 0; b < 32; b++) bitstr[16 + 32 * q + b] = (e[q] >> (31 - b)) & 1u;
+                for (int s = 0; s < 32; s++) {
+                    uint32_t h = 0;
+                    for (int b = 0; b < 16; b++) h = (h << 1) | bitstr[step_bits * (s + 1) + b];
                     int k = k_of_s[s / 4], j = s % 4;
                     int64_t P = (t < g.T) ? (((8 * t + k) * 4 + j) * 32 + l)
                                           : (1024 * g.T + (4 * k + j) * g.Lt + l);

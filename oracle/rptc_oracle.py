@@ -44,6 +44,8 @@ def lib():
         _lib.orc_matvec_f32.restype = i32
         _lib.orc_half_to_float.argtypes = [vp, vp, i64]
         _lib.orc_float_to_half.argtypes = [vp, vp, i64]
+        _lib.orc_bits_dense.argtypes = [vp, vp, vp, i64, i64, i32, i32, i32]
+        _lib.orc_bits_dense.restype = i32
         _lib.orc_sign_hadamard.argtypes = [vp, vp, vp, i64, i64, i64, i32]
         _lib.orc_sign_hadamard.restype = i32
         _lib.orc_num_threads.restype = i32
@@ -202,6 +204,17 @@ def matvec_f32(compressed, codebook, x, m, S, mode=AS_WRITTEN):
     rc = lib().orc_matvec_f32(_p(c), _p(cb), _p(xx), _p(y), m, n, S, mode)
     assert rc == 0, rc
     return y
+
+
+def bits_dense(compressed, codebook, m, n, S, bits, mode=AS_WRITTEN):
+    """The dense float16 [m, n] matrix of a hashed pair stream at `bits` (2, 3, 4) bits per weight."""
+    c = _u32(compressed).reshape(-1)
+    cb = _u16(codebook)
+    assert c.size * 32 == m * n * bits and cb.shape == (2 << S,)
+    W = np.empty((m, n), dtype=np.uint16)
+    rc = lib().orc_bits_dense(_p(c), _p(cb), _p(W), m, n, S, bits, mode)
+    assert rc == 0, rc
+    return W.view(np.float16)
 
 
 def sign_hadamard(x, signs, block, inverse=False):

@@ -446,3 +446,67 @@ def test_sign_hadamard_round_trip_and_norm(rk):
     # in place
     rk.sign_hadamard(y, signs, y, inverse=True)
     assert torch.equal(y, z)
+
+
+# ------------------------------------------------------------------ 3 and 4 bits per weight (no reference counterpart)
+
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("bits", [2, 3, 4])
+@pytest.mark.parametrize("S", [6, 8])
+@pytest.mark.parametrize("m,n", [(32, 2048), (33, 4096 + 768), (7, 704), (512, 6144)])
+def test_matvec_bits_dense_and_output(rk, oracle, mode, bits, S, m, n):
+    comp = rand_codes(m * n * bits // 32, seed=m + n + bits)
+    cb = rand_half(2 << S, seed=S + 40)
+    x = rand_half(n, seed=11)
+    W = torch.zeros((m, n), dtype=torch.float16, device="cuda")
+    out = torch.full((m,), float("nan"), dtype=torch.float16, device="cuda")
+    with with_mode(rk, mode):
+        rk.matvec_bits_dense(comp.cuda(), cb.cuda(), W, bits)
+        ms = rk.decompress_matvec_bits(comp.cuda(), cb.cuda(), x.cuda(), out, bits)
+    assert ms > 0
+    want = oracle.bits_dense(np_u32(comp), np_f16(cb), m, n, S, bits, mode=mode)
+    assert np.array_equal(np_f16(W).view(np.uint16), want.view(np.uint16))
+    y = oracle.dense_matvec(want, np_f16(x))
+    assert rel_l2(np_f16(out), y) < REL_L2_TOL
+
+
+@pytest.mark.parametrize("bits", [3, 4])
+def test_matvec_bits_fused_kernel_decodes_bit_exactly(rk, oracle, bits):
+    S, m, n = 8, 64, 2048 + 192
+    comp = rand_codes(m * n * bits // 32, seed=55 + bits)
+    cb = rand_half(2 << S, seed=56)
+    want = oracle.bits_dense(np_u32(comp), np_f16(cb), m, n, S, bits, mode=1)
+    c, cbd = comp.cuda(), cb.cuda()
+    out = torch.zeros((m,), dtype=torch.float16, device="cuda")
+    x = torch.zeros(n, dtype=torch.float16, device="cuda")
+    got = np.zeros((m, n), dtype=np.float16)
+    prev_timing = rk.set_timing(False)
+    cols = sorted(set(list(range(0, n, 5)) + list(range(n - 200, n))))
+    try:
+        with with_mode(rk, 1):
+            for p in cols:
+                x.zero_()
+                x[p] = 1.0
+                rk.decompress_matvec_bits(c, cbd, x, out, bits)
+                got[:, p] = np_f16(out)
+    finally:
+        rk.set_timing(prev_timing)
+    g, w = got[:, cols].view(np.uint16), want[:, cols].view(np.uint16)
+    nz = (w & 0x7FFF) != 0
+    assert np.array_equal(g[nz], w[nz])
+    assert np.all((g[~nz] & 0x7FFF) == 0)
+
+
+@pytest.mark.parametrize("bits", [3, 4])
+@pytest.mark.parametrize("m,n", [(4096, 11008), (11008, 4096)])
+def test_matvec_bits_full_size(rk, bits, m, n):
+    S = 8
+    comp = rand_codes(m * n * bits // 32, seed=42).cuda()
+    cb = rand_half(2 << S, seed=43).cuda()
+    x = rand_half(n, seed=44).cuda()
+    out = torch.zeros((m,), dtype=torch.float16, device="cuda")
+    W = torch.zeros((m, n), dtype=torch.float16, device="cuda")
+    rk.decompress_matvec_bits(comp, cb, x, out, bits)
+    rk.matvec_bits_dense(comp, cb, W, bits)
+    want = (W.double() @ x.double()).cpu().numpy()
+    assert rel_l2(np_f16(out), want) < REL_L2_TOL

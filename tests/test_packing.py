@@ -56,3 +56,27 @@ def test_pack_matvec_round_trip(oracle, n, S):
             e = (prod >> 8) & ((1 << S) - 1)
             w0 = (int(cbb[2 * e]) & 0x7FFF) | (prod & 0x8000)
             assert got[r, cols[p]] == w0 and got[r, cols[p] + 1] == cbb[2 * e + 1]
+
+
+@pytest.mark.parametrize("bits", [2, 3, 4])
+@pytest.mark.parametrize("n", [2048, 2048 + 320, 64])
+def test_pack_matvec_bits_round_trip(oracle, bits, n):
+    """6- and 8-bit symbols (3 and 4 bits per weight): the packed stream decodes to the shift-register walk."""
+    g = rng(n + bits)
+    m, S = 2, 8
+    sb = 2 * bits
+    symbols = g.integers(0, 1 << sb, (m, n // 2))
+    cb = g.standard_normal(2 << S).astype(np.float16)
+    stream = packing.pack_matvec(symbols, bits=bits)
+    assert stream.shape == (m * n * bits // 32,)
+    got = oracle.bits_dense(stream, cb, m, n, S, bits, mode=oracle.CONTINUOUS).view(np.uint16)
+    cols = packing.matvec_stream_columns(n)
+    cbb = cb.view(np.uint16)
+    for r in range(m):
+        state = 0
+        for p, sym in enumerate(symbols[r]):
+            state = ((state << sb) | int(sym)) & 0xFFFF
+            prod = state * (state + 1)
+            e = (prod >> 8) & ((1 << S) - 1)
+            w0 = (int(cbb[2 * e]) & 0x7FFF) | (prod & 0x8000)
+            assert got[r, cols[p]] == w0 and got[r, cols[p] + 1] == cbb[2 * e + 1]
