@@ -49,6 +49,10 @@ def parse():
     ap.add_argument("--extra-shapes", action="store_true", help="also time the other layer shapes")
     ap.add_argument("--other-ops", action="store_true",
                     help="time decompress, decompress_matvec_t_16 and sign_hadamard instead (prints its own JSON line)")
+    ap.add_argument("--decode", action="store_true",
+                    help="greedy decode with a Llama-2-7B-shaped random-init model whose projections are 2-bit streams "
+                         "(prompt 512, 128 new tokens, batch 1); prints its own JSON line")
+    ap.add_argument("--decode-layers", type=int, default=32)
     ap.add_argument("--matmul", action="store_true",
                     help="time the batch 8/16/32 fused decode + MFMA mat-mat instead (prints its own JSON line)")
     return ap.parse_args()
@@ -318,6 +322,24 @@ def main():
         return
     if a.other_ops:
         bench_other_ops(a)
+        return
+    if a.decode:
+        from rptc_kernels.llama_decode import LlamaShape, QuantizedLlama, greedy_decode
+        shape = LlamaShape(layers=a.decode_layers)
+        model = QuantizedLlama(shape, S=a.S)
+        g = torch.Generator().manual_seed(42)
+        prompt = torch.randint(0, shape.vocab, (512,), generator=g)
+        res = {}
+        for use_graph in (True, False):
+            toks, dt = greedy_decode(model, prompt, 128, use_graph=use_graph)
+            res["graph" if use_graph else "eager"] = {"tok_per_s": round(127 / dt, 1), "ms_per_token": round(dt / 127 * 1e3, 3)}
+        stream_bytes = sum(b.compressed_bytes() for blk in model.blocks for b in blk.children())
+        print(json.dumps({"metric": "decode tok/s Llama-2-7B-shape bs=1", "value": res["graph"]["tok_per_s"], "unit": "tok/s",
+                          "n_gpus": 1, "data": "synthetic",
+                          "config": {"workload": f"{shape.layers} layers d=4096 heads=32 mlp=11008 vocab=32000, random-init, "
+                                                 f"projections as seeded random 2-bit streams ({stream_bytes} bytes), prompt 512 "
+                                                 f"random ids, 128 greedy tokens, one HIP graph per token"},
+                          "results": res}))
         return
     runner = Runner(a.m, a.n, a.S, a.copies)
     if a.pmc_probe:

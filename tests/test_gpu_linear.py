@@ -135,3 +135,38 @@ def test_from_weight_quantizes_and_runs(rk):
     y = layer(x)
     want = x.double().cpu() @ What.double().t()
     assert rel_l2(y.cpu().numpy(), want.numpy()) < 1e-3
+
+
+def test_llama_decode_graph_equals_eager_and_dense_reference(rk):
+    """A 2-layer Llama-shaped model on streams: the captured decode step reproduces eager decoding token
+    for token, and the logits match the same network run on the decoded dense weights."""
+    from rptc_kernels.llama_decode import LlamaShape, QuantizedLlama, greedy_decode
+    from rptc_kernels.linear import QuantizedLinear
+    shape = LlamaShape(layers=2, d_model=256, heads=4, d_ff=704, vocab=1000, max_len=128)
+    model = QuantizedLlama(shape, S=8, seed=7)
+    prompt = torch.randint(0, shape.vocab, (40,), generator=torch.Generator().manual_seed(1))
+    toks_graph, _ = greedy_decode(model, prompt, 12, use_graph=True)
+    model.k_cache.zero_(); model.v_cache.zero_()
+    toks_eager, _ = greedy_decode(model, prompt, 12, use_graph=False)
+    assert toks_graph == toks_eager
+
+    # dense reference: swap every QuantizedLinear for a matmul with its decoded weight
+    class Dense(torch.nn.Module):
+        def __init__(self, w):
+            super().__init__()
+            self.w = w
+
+        def forward(self, x):
+            return (x.float() @ self.w.float().t()).half()
+
+    model.k_cache.zero_(); model.v_cache.zero_()
+    pos = torch.arange(40, device="cuda")
+    with torch.no_grad():
+        logits_q = model.forward_tokens(prompt[:32].cuda(), pos[:32])
+        for blk in model.blocks:
+            for name, child in list(blk.named_children()):
+                if isinstance(child, QuantizedLinear):
+                    setattr(blk, name, Dense(child.decoded_weight()))
+        model.k_cache.zero_(); model.v_cache.zero_()
+        logits_d = model.forward_tokens(prompt[:32].cuda(), pos[:32])
+    assert rel_l2(logits_q.cpu().numpy(), logits_d.cpu().numpy()) < 2e-2
