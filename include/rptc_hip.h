@@ -163,6 +163,26 @@ int rptc_matvec_bits_dense(const int32_t *compressed, const uint16_t *codebook, 
 int rptc_sign_hadamard(const uint16_t *x, const uint16_t *signs, uint16_t *out, int64_t batch,
                        int64_t n, int64_t block, int inverse, void *stream, float *ms);
 
+/*
+ * The small kernels between the quantized projections of a Llama decoder layer, batch 1, one token
+ * per call (no counterpart in the reference, which generates with transformers on dense weights,
+ * quantize_hf.py:229-236).  fp16 in and out, fp32 arithmetic, asynchronous on `stream`; `pos` is a
+ * device pointer to the token's position so that a captured HIP graph can be replayed.
+ *   rptc_add_rmsnorm  x_out = x_in + delta (delta may be NULL); h_out = rmsnorm(x_out) * weight; all [d]
+ *   rptc_rope_cache   qkv = [q|k|v], each heads*hd: rotate the (2i, 2i+1) pairs of q and k by
+ *                     cos/sin [max_len][hd/2] at *pos, write q_out and k, v into caches [heads][max_len][hd]
+ *   rptc_attn_decode  out[h] = softmax(q[h] . K[h]^T / sqrt(hd)) V[h] over cache positions 0..*pos
+ *   rptc_silu_mul     gate_up = [gate|up], each f: out = silu(gate) * up
+ */
+int rptc_add_rmsnorm(const uint16_t *x_in, const uint16_t *delta, const uint16_t *weight, uint16_t *x_out,
+                     uint16_t *h_out, int64_t d, float eps, void *stream);
+int rptc_rope_cache(const uint16_t *qkv, const uint16_t *cos_t, const uint16_t *sin_t, const int64_t *pos,
+                    uint16_t *q_out, uint16_t *k_cache, uint16_t *v_cache, int64_t heads, int64_t hd,
+                    int64_t max_len, void *stream);
+int rptc_attn_decode(const uint16_t *q, const uint16_t *k_cache, const uint16_t *v_cache, const int64_t *pos,
+                     uint16_t *out, int64_t heads, int64_t hd, int64_t max_len, void *stream);
+int rptc_silu_mul(const uint16_t *gate_up, uint16_t *out, int64_t f, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

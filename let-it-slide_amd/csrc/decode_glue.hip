@@ -1,0 +1,219 @@
+// The small kernels between the quantized projections of a Llama decoder layer, batch 1, one
+// token per call: residual add + RMS norm, rotary embedding + KV-cache write, single-query
+// attention over the cache, SiLU gate.  They exist so that a decode step is a handful of launches
+// per layer instead of dozens of framework element-wise kernels; none of them is in the reference
+// (it generates with transformers on dense weights, quantize_hf.py:229-236).
+// fp16 in and out, fp32 arithmetic.  The position is read from device memory so that a captured
+// HIP graph can be replayed for successive tokens.
+#include "rptc_common.hpp"
+
+namespace rptc {
+
+__device__ __forceinline__ float block_sum(float v, float *scratch)
+{
+    // scratch: one float per wave; returns the sum over the workgroup to every thread
+    v = wave_sum(v);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
+    if (lane == 63) scratch[wave] = v;
+    __syncthreads();
+    float t = 0.f;
+    for (int w = 0; w < waves; w++) t += scratch[w];
+    __syncthreads();
+    return t;
+}
+
+__device__ __forceinline__ float block_max(float v, float *scratch)
+{
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
+    if (lane == 0) scratch[wave] = v;
+    __syncthreads();
+    float t = scratch[0];
+    for (int w = 1; w < waves; w++) t = fmaxf(t, scratch[w]);
+    __syncthreads();
+    return t;
+}
+
+// x_out = x_in + delta (delta may be null);  h_out = x_out * rsqrt(mean(x_out^2) + eps) * weight
+__global__ __launch_bounds__(1024) void add_rmsnorm_kernel(const uint16_t *__restrict__ x_in, const uint16_t *delta,
+                                                            const uint16_t *__restrict__ weight, uint16_t *x_out,
+                                                            uint16_t *__restrict__ h_out, int d, float eps)
+{
+    __shared__ float scratch[16];
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < d; i += blockDim.x) {
+        float v = half_bits_to_float(x_in[i]);
+        if (delta) v = half_bits_to_float(float_to_half_bits(v + half_bits_to_float(delta[i])));   // the fp16 residual stream
+        x_out[i] = float_to_half_bits(v);
+        ss += v * v;
+    }
+    const float inv = rsqrtf(block_sum(ss, scratch) / (float)d + eps);
+    for (int i = threadIdx.x; i < d; i += blockDim.x) {
+        const float v = half_bits_to_float(x_out[i]);
+        h_out[i] = float_to_half_bits(half_bits_to_float(float_to_half_bits(v * inv)) * half_bits_to_float(weight[i]));
+    }
+}
+
+// qkv = [q | k | v], each heads*hd.  Rotates the (2i, 2i+1) pairs of q and k by the angle of the
+// position, writes q to q_out and k, v into the caches [heads][max_len][hd] at that position.
+__global__ __launch_bounds__(256) void rope_cache_kernel(const uint16_t *__restrict__ qkv, const uint16_t *__restrict__ cos_t,
+                                                         const uint16_t *__restrict__ sin_t, const int64_t *__restrict__ pos_p,
+                                                         uint16_t *__restrict__ q_out, uint16_t *__restrict__ k_cache,
+                                                         uint16_t *__restrict__ v_cache, int heads, int hd, int max_len)
+{
+    const int pos = (int)*pos_p;
+    const int half = hd >> 1, d = heads * hd;
+    const int t = blockIdx.x * blockDim.x + threadIdx.x;        // one (head, pair) per thread
+    if (t >= heads * half) return;
+    const int h = t / half, i = t - h * half;
+    const float c = half_bits_to_float(cos_t[pos * half + i]), s = half_bits_to_float(sin_t[pos * half + i]);
+    const int e = h * hd + 2 * i;
+    const size_t ce = ((size_t)h * max_len + pos) * hd + 2 * i;
+    const float qa = half_bits_to_float(qkv[e]), qb = half_bits_to_float(qkv[e + 1]);
+    const float ka = half_bits_to_float(qkv[d + e]), kb = half_bits_to_float(qkv[d + e + 1]);
+    // fp16 products and fp16 difference, as the element-wise framework path computes them
+    auto h16 = [](float v) { return half_bits_to_float(float_to_half_bits(v)); };
+    q_out[e] = float_to_half_bits(h16(qa * c) - h16(qb * s));
+    q_out[e + 1] = float_to_half_bits(h16(qa * s) + h16(qb * c));
+    k_cache[ce] = float_to_half_bits(h16(ka * c) - h16(kb * s));
+    k_cache[ce + 1] = float_to_half_bits(h16(ka * s) + h16(kb * c));
+    v_cache[ce] = qkv[2 * d + e];
+    v_cache[ce + 1] = qkv[2 * d + e + 1];
+}
+
+// One workgroup of 1024 threads per head: softmax(q . K^T / sqrt(hd)) V over cache positions 0..pos.
+// Scores: 16 lanes share a key (16 bytes of it each, so a wave reads 1 KiB of four consecutive
+// keys per load) and add their partial dot products with DPP-free shuffles inside the 16.
+// Values: a thread owns one pair of output dimensions, the keys are cut into 1024 / (hd/2)
+// interleaved groups whose sums are added in a fixed order.
+constexpr int kAttnThreads = 1024;
+
+__global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(
+    const uint16_t *__restrict__ q, const uint16_t *__restrict__ k_cache, const uint16_t *__restrict__ v_cache,
+    const int64_t *__restrict__ pos_p, uint16_t *__restrict__ out, int hd, int max_len)
+{
+    extern __shared__ float lds_f[];
+    float *scores = lds_f;                       // [max_len]
+    float *scratch = lds_f + max_len;            // [16]
+    float *acc = scratch + 16;                   // [groups][hd]
+    const int h = blockIdx.x, tid = threadIdx.x;
+    const int len = (int)*pos_p + 1;
+    const uint16_t *kh = k_cache + (size_t)h * max_len * hd, *vh = v_cache + (size_t)h * max_len * hd;
+    const float scale = rsqrtf((float)hd);
+
+    // scores
+    const int lanes_per_key = hd >> 3;           // 16 bytes = 8 values per lane
+    const int sub = tid % lanes_per_key, slot = tid / lanes_per_key, slots = kAttnThreads / lanes_per_key;
+    float qf[8];
+    {
+        const uint4 v = *reinterpret_cast<const uint4 *>(q + h * hd + 8 * sub);
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            qf[2 * u] = half_bits_to_float((uint16_t)(w[u] & 0xFFFFu));
+            qf[2 * u + 1] = half_bits_to_float((uint16_t)(w[u] >> 16));
+        }
+    }
+    for (int s0 = 0; s0 < len; s0 += slots) {
+        const int s = s0 + slot;
+        float dot = 0.f;
+        if (s < len) {
+            const uint4 v = *reinterpret_cast<const uint4 *>(kh + (size_t)s * hd + 8 * sub);
+            const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                dot += half_bits_to_float((uint16_t)(w[u] & 0xFFFFu)) * qf[2 * u];
+                dot += half_bits_to_float((uint16_t)(w[u] >> 16)) * qf[2 * u + 1];
+            }
+        }
+        for (int off = lanes_per_key >> 1; off > 0; off >>= 1) dot += __shfl_xor(dot, off, 64);
+        if (s < len && sub == 0) scores[s] = dot * scale;
+    }
+    __syncthreads();
+    float mx = -INFINITY;
+    for (int s = tid; s < len; s += kAttnThreads) mx = fmaxf(mx, scores[s]);
+    mx = block_max(mx, scratch);
+    float sum = 0.f;
+    for (int s = tid; s < len; s += kAttnThreads) {
+        const float p = __expf(scores[s] - mx);
+        scores[s] = p;
+        sum += p;
+    }
+    const float inv = 1.f / block_sum(sum, scratch);     // (its barriers also publish the new scores)
+
+    // values
+    const int pairs = hd >> 1, groups = kAttnThreads / pairs, grp = tid / pairs, dp = tid - grp * pairs;
+    float a0 = 0.f, a1 = 0.f;
+    for (int s = grp; s < len; s += groups) {
+        const uint32_t v = *reinterpret_cast<const uint32_t *>(vh + (size_t)s * hd + 2 * dp);
+        const float p = scores[s];
+        a0 += p * half_bits_to_float((uint16_t)(v & 0xFFFFu));
+        a1 += p * half_bits_to_float((uint16_t)(v >> 16));
+    }
+    acc[grp * hd + 2 * dp] = a0;
+    acc[grp * hd + 2 * dp + 1] = a1;
+    __syncthreads();
+    for (int i = tid; i < hd; i += kAttnThreads) {
+        float y = 0.f;
+        for (int gidx = 0; gidx < groups; gidx++) y += acc[gidx * hd + i];
+        out[h * hd + i] = float_to_half_bits(y * inv);
+    }
+}
+
+// gu = [gate | up], each f:  out = silu(gate) * up
+__global__ __launch_bounds__(256) void silu_mul_kernel(const uint16_t *__restrict__ gu, uint16_t *__restrict__ out, int f)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= f) return;
+    const float g = half_bits_to_float(gu[i]), u = half_bits_to_float(gu[f + i]);
+    const float sg = half_bits_to_float(float_to_half_bits(g / (1.f + __expf(-g))));
+    out[i] = float_to_half_bits(sg * u);
+}
+
+}  // namespace rptc
+
+using namespace rptc;
+
+extern "C" int rptc_add_rmsnorm(const uint16_t *x_in, const uint16_t *delta, const uint16_t *weight, uint16_t *x_out,
+                                uint16_t *h_out, int64_t d, float eps, void *stream)
+{
+    if (!x_in || !weight || !x_out || !h_out) return RPTC_ENULL;
+    if (d < 1 || d > (1 << 20)) return RPTC_ESHAPE;
+    hipLaunchKernelGGL(add_rmsnorm_kernel, dim3(1), dim3(1024), 0, static_cast<hipStream_t>(stream), x_in, delta, weight,
+                       x_out, h_out, (int)d, eps);
+    return (int)hipGetLastError();
+}
+
+extern "C" int rptc_rope_cache(const uint16_t *qkv, const uint16_t *cos_t, const uint16_t *sin_t, const int64_t *pos,
+                               uint16_t *q_out, uint16_t *k_cache, uint16_t *v_cache, int64_t heads, int64_t hd,
+                               int64_t max_len, void *stream)
+{
+    if (!qkv || !cos_t || !sin_t || !pos || !q_out || !k_cache || !v_cache) return RPTC_ENULL;
+    if (heads < 1 || hd < 2 || hd % 2 != 0 || max_len < 1) return RPTC_ESHAPE;
+    const int threads = (int)(heads * hd / 2);
+    hipLaunchKernelGGL(rope_cache_kernel, dim3((threads + 255) / 256), dim3(256), 0, static_cast<hipStream_t>(stream), qkv,
+                       cos_t, sin_t, pos, q_out, k_cache, v_cache, (int)heads, (int)hd, (int)max_len);
+    return (int)hipGetLastError();
+}
+
+extern "C" int rptc_attn_decode(const uint16_t *q, const uint16_t *k_cache, const uint16_t *v_cache, const int64_t *pos,
+                                uint16_t *out, int64_t heads, int64_t hd, int64_t max_len, void *stream)
+{
+    if (!q || !k_cache || !v_cache || !pos || !out) return RPTC_ENULL;
+    // hd a power of two in [16, 256]: 16 bytes per lane, whole keys per wave, whole groups per workgroup
+    if (heads < 1 || hd < 16 || hd > 256 || (hd & (hd - 1)) != 0 || max_len < 1) return RPTC_ESHAPE;
+    const size_t lds = (size_t)(max_len + 16 + (kAttnThreads / (hd / 2)) * hd) * 4;
+    if (lds > 64 * 1024) return RPTC_ELIMIT;
+    hipLaunchKernelGGL(attn_decode_kernel, dim3((unsigned)heads), dim3(kAttnThreads), lds, static_cast<hipStream_t>(stream),
+                       q, k_cache, v_cache, pos, out, (int)hd, (int)max_len);
+    return (int)hipGetLastError();
+}
+
+extern "C" int rptc_silu_mul(const uint16_t *gate_up, uint16_t *out, int64_t f, void *stream)
+{
+    if (!gate_up || !out) return RPTC_ENULL;
+    if (f < 1 || f > (1 << 24)) return RPTC_ESHAPE;
+    hipLaunchKernelGGL(silu_mul_kernel, dim3((unsigned)((f + 255) / 256)), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       gate_up, out, (int)f);
+    return (int)hipGetLastError();
+}

@@ -55,6 +55,10 @@ _SIGNATURES = {
     "rptc_sign_hadamard": ([_VP, _VP, _VP, _I64, _I64, _I64, _INT, _VP, _FP], _INT),
     "rptc_decompress_matvec_bits": ([_VP, _VP, _VP, _VP, _I64, _I64, _INT, _INT, _INT, _VP, _FP], _INT),
     "rptc_matvec_bits_dense": ([_VP, _VP, _VP, _I64, _I64, _INT, _INT, _INT, _VP, _FP], _INT),
+    "rptc_add_rmsnorm": ([_VP, _VP, _VP, _VP, _VP, _I64, ctypes.c_float, _VP], _INT),
+    "rptc_rope_cache": ([_VP, _VP, _VP, _VP, _VP, _VP, _VP, _I64, _I64, _I64, _VP], _INT),
+    "rptc_attn_decode": ([_VP, _VP, _VP, _VP, _VP, _I64, _I64, _I64, _VP], _INT),
+    "rptc_silu_mul": ([_VP, _VP, _I64, _VP], _INT),
 }
 
 

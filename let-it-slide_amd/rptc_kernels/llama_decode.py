@@ -1,14 +1,23 @@
-"""A Llama-architecture decoder whose seven projections per layer are QuantizedLinear streams.
+"""A Llama-architecture decoder whose projections are QuantizedLinear streams.
 
 The reference quantizes ``model.layers.N.{self_attn.{q,k,v,o}_proj, mlp.{gate,up,down}_proj}`` of a
 HuggingFace Llama-2-7B (quantize_hf.py:189) but writes dense weights back and generates with
-``transformers`` (quantize_hf.py:229-236).  Here the same module list runs on the packed streams.
-The model is built from its shape only (random-init norms, embeddings and lm_head; seeded random
-streams for the projections): nothing is downloaded.  Greedy decode of one sequence; the whole
-per-token step is captured in one HIP graph so that host launch overhead does not set the rate.
+``transformers`` (quantize_hf.py:229-236).  Here the same projections run on the packed streams,
+grouped the way the reference groups them for its Hessians (quantize_hf.py:14-22: q, k, v -> one
+"qkv" matrix, gate and up -> one "up" matrix), which is one kernel launch per group.  The model is
+built from its shape only (random-init norms, embeddings and lm_head; seeded random streams for the
+projections): nothing is downloaded.
+
+Two ways through a token: ``forward_tokens`` (torch ops between the projections; used for the
+prompt, any number of tokens) and ``decode_step`` (this library's fused glue kernels, one token).
+Greedy decoding captures one ``decode_step`` in a HIP graph and replays it per token.
 """
+import ctypes
+import time
+
 import torch
 
+import rptc_kernels as rk
 from .linear import QuantizedLinear
 
 
@@ -20,6 +29,8 @@ class LlamaShape:
 
 
 class QuantizedLlama(torch.nn.Module):
+    EPS = 1e-5
+
     def __init__(self, shape, S=8, seed=42, device="cuda"):
         super().__init__()
         self.shape = shape
@@ -32,8 +43,8 @@ class QuantizedLlama(torch.nn.Module):
         self.blocks = torch.nn.ModuleList()
         for i in range(shape.layers):
             blk = torch.nn.Module()
-            for j, (name, n_in, n_out) in enumerate((("q_proj", d, d), ("k_proj", d, d), ("v_proj", d, d), ("o_proj", d, d),
-                                                     ("gate_proj", d, f), ("up_proj", d, f), ("down_proj", f, d))):
+            for j, (name, n_in, n_out) in enumerate((("qkv_proj", d, 3 * d), ("o_proj", d, d),
+                                                     ("gate_up_proj", d, 2 * f), ("down_proj", f, d))):
                 setattr(blk, name, QuantizedLinear.from_random(n_in, n_out, S=S, seed=seed + 16 * i + j, device=device))
             blk.norm1 = torch.ones(d, dtype=torch.float16, device=device)
             blk.norm2 = torch.ones(d, dtype=torch.float16, device=device)
@@ -41,17 +52,23 @@ class QuantizedLlama(torch.nn.Module):
         hd = shape.head_dim
         inv = 1.0 / (shape.rope_theta ** (torch.arange(0, hd, 2, device=device).float() / hd))
         ang = torch.arange(shape.max_len, device=device).float()[:, None] * inv[None, :]
-        self.cos, self.sin = ang.cos().half(), ang.sin().half()                       # [max_len, hd/2]
+        self.cos, self.sin = ang.cos().half().contiguous(), ang.sin().half().contiguous()    # [max_len, hd/2]
         self.k_cache = torch.zeros((shape.layers, shape.heads, shape.max_len, hd), dtype=torch.float16, device=device)
         self.v_cache = torch.zeros_like(self.k_cache)
+        # work buffers of the one-token path
+        z = lambda k: torch.zeros(k, dtype=torch.float16, device=device)
+        self._x, self._h, self._qkv, self._q, self._att = z(d), z(d), z(3 * d), z(d), z(d)
+        self._o, self._gu, self._act, self._down = z(d), z(2 * f), z(f), z(d)
 
-    @staticmethod
-    def _rms(x, w):
+    # ---------------------------------------------------------------- torch path (any number of tokens)
+
+    @classmethod
+    def _rms(cls, x, w):
         v = x.float()
-        return (v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + 1e-5)).half() * w
+        return (v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + cls.EPS)).half() * w
 
     def _rope(self, t, pos):
-        # t [T, heads, hd]; pos [T] (long)
+        # t [T, heads, hd]; pos [T] (long): rotate the (2i, 2i+1) pairs
         c, s = self.cos[pos][:, None, :], self.sin[pos][:, None, :]
         a, b = t[..., 0::2], t[..., 1::2]
         return torch.stack([a * c - b * s, a * s + b * c], dim=-1).flatten(-2)
@@ -60,61 +77,106 @@ class QuantizedLlama(torch.nn.Module):
         """tokens [T] long, pos [T] long (their positions, contiguous); writes the KV cache at pos and
         returns the logits of the last token.  Attention looks at cache positions <= the token's own."""
         sh = self.shape
-        T = tokens.numel()
+        T, d, f = tokens.numel(), sh.d_model, sh.d_ff
         x = self.embed[tokens]                                                     # [T, d]
         key_pos = torch.arange(sh.max_len, device=x.device)
         mask = key_pos[None, :] <= pos[:, None]                                    # [T, max_len]
         for i, blk in enumerate(self.blocks):
             h = self._rms(x, blk.norm1)
-            q = self._rope(blk.q_proj(h).view(T, sh.heads, sh.head_dim), pos)
-            k = self._rope(blk.k_proj(h).view(T, sh.heads, sh.head_dim), pos)
-            v = blk.v_proj(h).view(T, sh.heads, sh.head_dim)
+            q, k, v = blk.qkv_proj(h).split(d, dim=-1)
+            q = self._rope(q.reshape(T, sh.heads, sh.head_dim), pos)
+            k = self._rope(k.reshape(T, sh.heads, sh.head_dim), pos)
+            v = v.reshape(T, sh.heads, sh.head_dim)
             self.k_cache[i].index_copy_(1, pos, k.transpose(0, 1))
             self.v_cache[i].index_copy_(1, pos, v.transpose(0, 1))
             o = torch.nn.functional.scaled_dot_product_attention(q.transpose(0, 1), self.k_cache[i], self.v_cache[i],
                                                                  attn_mask=mask[None])      # [heads, T, hd]
-            o = o.transpose(0, 1).reshape(T, sh.d_model)
-            x = x + blk.o_proj(o)
+            x = x + blk.o_proj(o.transpose(0, 1).reshape(T, d))
             h = self._rms(x, blk.norm2)
-            x = x + blk.down_proj(torch.nn.functional.silu(blk.gate_proj(h)) * blk.up_proj(h))
+            g, u = blk.gate_up_proj(h).split(f, dim=-1)
+            x = x + blk.down_proj(torch.nn.functional.silu(g) * u)
         h = self._rms(x[-1:], self.final_norm)
         return (h @ self.lm_head.t()).float()                                      # [1, vocab]
 
+    # ---------------------------------------------------------------- fused one-token path
 
-def greedy_decode(model, prompt, new_tokens, use_graph=True):
+    def decode_step(self, token, pos):
+        """token [1] long, pos [1] long, both on the device (read by the kernels, so a captured graph can be
+        replayed with new values).  Returns the logits [1, vocab] (float)."""
+        sh = self.shape
+        lib = rk.library()
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        d, f = sh.d_model, sh.d_ff
+
+        def ok(rc):
+            if rc:
+                raise RuntimeError(lib.rptc_status_string(rc).decode())
+
+        def gemv(layer, x, out):
+            fn = getattr(lib, f"rptc_decompress_matvec_16_{layer.S}_1")
+            ok(fn(layer.compressed.data_ptr(), layer.codebook.data_ptr(), x.data_ptr(), out.data_ptr(),
+                  layer.out_features, layer.in_features, layer.carry_mode, stream, None))
+
+        self._x.copy_(self.embed[token].reshape(-1))
+        delta = None
+        for i, blk in enumerate(self.blocks):
+            ok(lib.rptc_add_rmsnorm(self._x.data_ptr(), delta, blk.norm1.data_ptr(), self._x.data_ptr(),
+                                    self._h.data_ptr(), d, self.EPS, stream))
+            gemv(blk.qkv_proj, self._h, self._qkv)
+            ok(lib.rptc_rope_cache(self._qkv.data_ptr(), self.cos.data_ptr(), self.sin.data_ptr(), pos.data_ptr(),
+                                   self._q.data_ptr(), self.k_cache[i].data_ptr(), self.v_cache[i].data_ptr(),
+                                   sh.heads, sh.head_dim, sh.max_len, stream))
+            ok(lib.rptc_attn_decode(self._q.data_ptr(), self.k_cache[i].data_ptr(), self.v_cache[i].data_ptr(),
+                                    pos.data_ptr(), self._att.data_ptr(), sh.heads, sh.head_dim, sh.max_len, stream))
+            gemv(blk.o_proj, self._att, self._o)
+            ok(lib.rptc_add_rmsnorm(self._x.data_ptr(), self._o.data_ptr(), blk.norm2.data_ptr(), self._x.data_ptr(),
+                                    self._h.data_ptr(), d, self.EPS, stream))
+            gemv(blk.gate_up_proj, self._h, self._gu)
+            ok(lib.rptc_silu_mul(self._gu.data_ptr(), self._act.data_ptr(), f, stream))
+            gemv(blk.down_proj, self._act, self._down)
+            delta = self._down.data_ptr()
+        ok(lib.rptc_add_rmsnorm(self._x.data_ptr(), delta, self.final_norm.data_ptr(), self._x.data_ptr(),
+                                self._h.data_ptr(), d, self.EPS, stream))
+        return (self._h.unsqueeze(0) @ self.lm_head.t()).float()
+
+
+def greedy_decode(model, prompt, new_tokens, mode="fused_graph"):
     """Prefill the prompt (in chunks of 32 tokens: the batch the fused mat-mat kernel takes), then decode
-    ``new_tokens`` greedily one at a time.  Returns (token list, seconds spent in the decode loop)."""
-    import time
+    ``new_tokens`` greedily one at a time.  mode: "fused_graph" (glue kernels, one HIP graph per token),
+    "fused" (glue kernels, direct launches), "torch_graph" / "torch" (framework ops between the projections).
+    Returns (token list, seconds spent in the decode loop)."""
     dev = model.embed.device
     prompt = torch.as_tensor(prompt, dtype=torch.long, device=dev)
     P = prompt.numel()
+    step = model.decode_step if mode.startswith("fused") else model.forward_tokens
     with torch.no_grad():
         logits = None
         for p0 in range(0, P, 32):
             chunk = prompt[p0:p0 + 32]
             logits = model.forward_tokens(chunk, torch.arange(p0, p0 + chunk.numel(), device=dev))
         tok = logits.argmax(-1)                                                    # [1]
-        out = [int(tok)]
+        out = [tok.clone()]
         s_tok = tok.clone()
         s_pos = torch.tensor([P], dtype=torch.long, device=dev)
-        if use_graph:
-            # warm up on a side stream, then capture one decode step with static token/position tensors
+        graph = None
+        if mode.endswith("graph"):
+            # warm up on a side stream, then capture one step with static token/position tensors
             side = torch.cuda.Stream()
             side.wait_stream(torch.cuda.current_stream())
             with torch.cuda.stream(side):
-                model.forward_tokens(s_tok, s_pos)
+                step(s_tok, s_pos)
             torch.cuda.current_stream().wait_stream(side)
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
-                s_next = model.forward_tokens(s_tok, s_pos).argmax(-1)
+                s_next = step(s_tok, s_pos).argmax(-1)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for _ in range(new_tokens - 1):
-            if use_graph:
+            if graph is not None:
                 graph.replay()
                 nxt = s_next
             else:
-                nxt = model.forward_tokens(s_tok, s_pos).argmax(-1)
+                nxt = step(s_tok, s_pos).argmax(-1)
             s_tok.copy_(nxt)
             s_pos.add_(1)
             out.append(nxt.clone())

@@ -137,18 +137,37 @@ def test_from_weight_quantizes_and_runs(rk):
     assert rel_l2(y.cpu().numpy(), want.numpy()) < 1e-3
 
 
-def test_llama_decode_graph_equals_eager_and_dense_reference(rk):
-    """A 2-layer Llama-shaped model on streams: the captured decode step reproduces eager decoding token
-    for token, and the logits match the same network run on the decoded dense weights."""
+def test_llama_decode_paths_agree(rk):
+    """A 2-layer Llama-shaped model on streams: the fused one-token step matches the torch path's logits,
+    graph replay reproduces direct launches token for token, and the logits match the same network run on
+    the decoded dense weights."""
     from rptc_kernels.llama_decode import LlamaShape, QuantizedLlama, greedy_decode
     from rptc_kernels.linear import QuantizedLinear
     shape = LlamaShape(layers=2, d_model=256, heads=4, d_ff=704, vocab=1000, max_len=128)
     model = QuantizedLlama(shape, S=8, seed=7)
     prompt = torch.randint(0, shape.vocab, (40,), generator=torch.Generator().manual_seed(1))
-    toks_graph, _ = greedy_decode(model, prompt, 12, use_graph=True)
-    model.k_cache.zero_(); model.v_cache.zero_()
-    toks_eager, _ = greedy_decode(model, prompt, 12, use_graph=False)
-    assert toks_graph == toks_eager
+    runs = {}
+    for mode in ("fused_graph", "fused", "torch_graph", "torch"):
+        model.k_cache.zero_(); model.v_cache.zero_()
+        runs[mode], _ = greedy_decode(model, prompt, 12, mode=mode)
+    assert runs["fused_graph"] == runs["fused"]
+    assert runs["torch_graph"] == runs["torch"]
+
+    # one decode step after the same prefill: fused glue vs torch glue
+    pos = torch.arange(40, device="cuda")
+    with torch.no_grad():
+        model.k_cache.zero_(); model.v_cache.zero_()
+        for p0 in (0, 32):
+            model.forward_tokens(prompt[p0:p0 + 32].cuda(), pos[p0:p0 + 32])
+        tok = torch.tensor([5], device="cuda")
+        p40 = torch.tensor([40], device="cuda")
+        kc, vc = model.k_cache.clone(), model.v_cache.clone()
+        lt = model.forward_tokens(tok, p40)
+        kt = model.k_cache.clone()
+        model.k_cache.copy_(kc); model.v_cache.copy_(vc)
+        lf = model.decode_step(tok, p40)
+        assert rel_l2(lf.cpu().numpy(), lt.cpu().numpy()) < 1e-2
+        assert rel_l2(model.k_cache.float().cpu().numpy(), kt.float().cpu().numpy()) < 1e-2
 
     # dense reference: swap every QuantizedLinear for a matmul with its decoded weight
     class Dense(torch.nn.Module):
@@ -159,9 +178,8 @@ def test_llama_decode_graph_equals_eager_and_dense_reference(rk):
         def forward(self, x):
             return (x.float() @ self.w.float().t()).half()
 
-    model.k_cache.zero_(); model.v_cache.zero_()
-    pos = torch.arange(40, device="cuda")
     with torch.no_grad():
+        model.k_cache.zero_(); model.v_cache.zero_()
         logits_q = model.forward_tokens(prompt[:32].cuda(), pos[:32])
         for blk in model.blocks:
             for name, child in list(blk.named_children()):
