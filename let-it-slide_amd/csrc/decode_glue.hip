@@ -114,20 +114,27 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(
             qf[2 * u + 1] = half_bits_to_float((uint16_t)(w[u] >> 16));
         }
     }
-    for (int s0 = 0; s0 < len; s0 += slots) {
-        const int s = s0 + slot;
-        float dot = 0.f;
-        if (s < len) {
-            const uint4 v = *reinterpret_cast<const uint4 *>(kh + (size_t)s * hd + 8 * sub);
-            const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    // four keys per thread in flight: the cache is far larger than L2, every load is an HBM round trip
+    for (int s0 = 0; s0 < len; s0 += 4 * slots) {
+        uint4 kv[4];
 #pragma unroll
-            for (int u = 0; u < 4; u++) {
-                dot += half_bits_to_float((uint16_t)(w[u] & 0xFFFFu)) * qf[2 * u];
-                dot += half_bits_to_float((uint16_t)(w[u] >> 16)) * qf[2 * u + 1];
-            }
+        for (int u = 0; u < 4; u++) {
+            const int s = s0 + u * slots + slot;
+            kv[u] = s < len ? *reinterpret_cast<const uint4 *>(kh + (size_t)s * hd + 8 * sub) : make_uint4(0, 0, 0, 0);
         }
-        for (int off = lanes_per_key >> 1; off > 0; off >>= 1) dot += __shfl_xor(dot, off, 64);
-        if (s < len && sub == 0) scores[s] = dot * scale;
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int s = s0 + u * slots + slot;
+            const uint32_t w[4] = {kv[u].x, kv[u].y, kv[u].z, kv[u].w};
+            float dot = 0.f;
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                dot += half_bits_to_float((uint16_t)(w[c] & 0xFFFFu)) * qf[2 * c];
+                dot += half_bits_to_float((uint16_t)(w[c] >> 16)) * qf[2 * c + 1];
+            }
+            for (int off = lanes_per_key >> 1; off > 0; off >>= 1) dot += __shfl_xor(dot, off, 64);
+            if (s < len && sub == 0) scores[s] = dot * scale;
+        }
     }
     __syncthreads();
     float mx = -INFINITY;
@@ -144,11 +151,20 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(
     // values
     const int pairs = hd >> 1, groups = kAttnThreads / pairs, grp = tid / pairs, dp = tid - grp * pairs;
     float a0 = 0.f, a1 = 0.f;
-    for (int s = grp; s < len; s += groups) {
-        const uint32_t v = *reinterpret_cast<const uint32_t *>(vh + (size_t)s * hd + 2 * dp);
-        const float p = scores[s];
-        a0 += p * half_bits_to_float((uint16_t)(v & 0xFFFFu));
-        a1 += p * half_bits_to_float((uint16_t)(v >> 16));
+    for (int s0 = grp; s0 < len; s0 += 8 * groups) {
+        uint32_t vv[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            const int s = s0 + u * groups;
+            vv[u] = s < len ? *reinterpret_cast<const uint32_t *>(vh + (size_t)s * hd + 2 * dp) : 0u;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            const int s = s0 + u * groups;
+            const float p = s < len ? scores[s] : 0.f;
+            a0 += p * half_bits_to_float((uint16_t)(vv[u] & 0xFFFFu));
+            a1 += p * half_bits_to_float((uint16_t)(vv[u] >> 16));
+        }
     }
     acc[grp * hd + 2 * dp] = a0;
     acc[grp * hd + 2 * dp + 1] = a1;
