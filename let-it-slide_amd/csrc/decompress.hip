@@ -23,39 +23,62 @@ __global__ __launch_bounds__(kDecompressThreads) void decompress_kernel(
 {
     extern __shared__ uint4 lds_u4[];
     const int tid = threadIdx.x;
-    for (int i = tid; i < kLutBytes / 16; i += kDecompressThreads) lds_u4[i] = codebook[i];
+    {
+        // all of a thread's share of the table is requested before any of it is stored: one memory
+        // round trip instead of eight
+        constexpr int kPerThread = kLutBytes / 16 / kDecompressThreads;
+        uint4 t[kPerThread];
+#pragma unroll
+        for (int i = 0; i < kPerThread; i++) t[i] = codebook[i * kDecompressThreads + tid];
+#pragma unroll
+        for (int i = 0; i < kPerThread; i++) lds_u4[i * kDecompressThreads + tid] = t[i];
+    }
     __syncthreads();
     const uint16_t *lut = reinterpret_cast<const uint16_t *>(lds_u4);
 
     const uint32_t groups_per_row = words_per_row * 2;   // a word holds 16 outputs = two groups of 8
-    for (uint32_t g = blockIdx.x * kDecompressThreads + tid; g < total_groups;
-         g += gridDim.x * kDecompressThreads) {
-        const uint32_t row = g / groups_per_row;
-        const uint32_t gw = g - row * groups_per_row;
-        const uint32_t w = gw >> 1;
-        const uint32_t *rowp = comp + (size_t)row * words_per_row;
-        const uint32_t cur = rowp[w];
-        uint32_t v;   // 16 bits of history above the 16 new bits
-        if (gw & 1) {
-            v = cur;
-        } else {
-            uint32_t hist = 0;
-            if (w) {
-                const uint32_t prev = rowp[w - 1];
+    const uint32_t stride = gridDim.x * kDecompressThreads;
+    constexpr int kInFlight = 4;   // groups whose stream words are requested before any is decoded
+    for (uint32_t g0 = blockIdx.x * kDecompressThreads + tid; g0 < total_groups; g0 += stride * kInFlight) {
+        uint32_t cur[kInFlight], prev[kInFlight];
+#pragma unroll
+        for (int u = 0; u < kInFlight; u++) {
+            const uint32_t g = g0 + u * stride;
+            cur[u] = prev[u] = 0;
+            if (g < total_groups) {
+                const uint32_t row = g / groups_per_row;
+                const uint32_t w = (g - row * groups_per_row) >> 1;
+                const uint32_t *rowp = comp + (size_t)row * words_per_row;
+                cur[u] = rowp[w];
+                if (w && !(g & 1)) prev[u] = rowp[w - 1];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kInFlight; u++) {
+            const uint32_t g = g0 + u * stride;
+            if (g >= total_groups) break;
+            const uint32_t w = (g % groups_per_row) >> 1;
+            uint32_t v;   // 16 bits of history above the 16 new bits
+            if (g & 1) {  // groups_per_row is even, so the parity of g is the parity within the row
+                v = cur[u];
+            } else {
                 // inference.cu:56-62: lane 0 of a warp reads the uint16 just below its element,
                 // the high half of the previous word; every other lane gets the low half.
-                hist = (MODE == RPTC_AS_WRITTEN && (w & 127u) == 0) ? (prev >> 16) : (prev & 0xFFFFu);
+                const uint32_t hist = (MODE == RPTC_AS_WRITTEN && (w & 127u) == 0) ? (prev[u] >> 16)
+                                                                                   : (prev[u] & 0xFFFFu);
+                v = (hist << 16) | (cur[u] >> 16);
             }
-            v = (hist << 16) | (cur >> 16);
-        }
-        uint32_t o[4];
+            uint32_t o[4];
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const uint32_t s0 = (v >> (14 - 4 * i)) & 0xFFFFu;
-            const uint32_t s1 = (v >> (12 - 4 * i)) & 0xFFFFu;
-            o[i] = (uint32_t)lut[s0] | ((uint32_t)lut[s1] << 16);
+            for (int i = 0; i < 4; i++) {
+                const uint32_t s0 = (v >> (14 - 4 * i)) & 0xFFFFu;
+                const uint32_t s1 = (v >> (12 - 4 * i)) & 0xFFFFu;
+                o[i] = (uint32_t)lut[s0] | ((uint32_t)lut[s1] << 16);
+            }
+            typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+            u32x4 ov = {o[0], o[1], o[2], o[3]};
+            __builtin_nontemporal_store(ov, reinterpret_cast<u32x4 *>(out) + g);
         }
-        out[g] = make_uint4(o[0], o[1], o[2], o[3]);
     }
 }
 

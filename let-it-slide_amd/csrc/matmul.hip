@@ -13,10 +13,11 @@
 //     registers while it walks the row blocks.
 //   * the decode is the mat-vec's (window pair per v_alignbit_b32, two hashes per v_pk_mad_u16,
 //     one address op and one conflict-free LDS gather per pair) minus the per-pair dot product.
-//   * a small pre-kernel writes the activations once in [slot][16 batch columns] order (the order
-//     the B operand and the LDS want); the main kernel copies one slab's slice of it into LDS per
-//     slab.  That scratch image lives in a static device buffer (no allocation per call); calls
-//     on different streams of one device share it and must not overlap.
+//   * a small pre-kernel writes the activations once in [slot][16 batch columns] order, the order
+//     the B operand wants: a wave's read of one step's pairs is 256 consecutive bytes.  The image
+//     (a few hundred KiB) stays in L2 and is read straight into registers one slab ahead; it lives
+//     in a static device buffer (no allocation per call), so calls on different streams of one
+//     device share it and must not overlap.
 //   * a workgroup owns its rows for all slabs, keeps the 16x16 accumulators in registers and
 //     adds the eight waves' tiles in a fixed order at the end: deterministic, no atomics.
 #include "rptc_common.hpp"
@@ -26,7 +27,6 @@ namespace rptc {
 constexpr int kMmThreads = 512;
 constexpr int kMmWaves = kMmThreads / kWave;       // one wave per group of 4 lanes-of-row
 constexpr int kMmTableBytes = 256 * 256;
-constexpr int kMmSliceBytes = 1024 * 16 * 4;       // one slab of activation pairs for 16 batch columns
 constexpr int kMmMaxRowBlocks = 4;                 // 16-row blocks per workgroup
 constexpr int kMmMaxN = 32768;
 constexpr int kMmMaxBatch = 32;
@@ -83,9 +83,7 @@ __global__ __launch_bounds__(kMmThreads) void matmul_kernel(
     uint16_t *__restrict__ out, int m, int n, int batch, int rows_per_block)
 {
     extern __shared__ uint32_t lds[];
-    uint4 *slice4 = reinterpret_cast<uint4 *>(lds + kMmTableBytes / 4);
-    const uint32_t *slice = lds + kMmTableBytes / 4;
-    float *part = reinterpret_cast<float *>(lds + (kMmTableBytes + kMmSliceBytes) / 4);   // [wave][rb][v][lane]
+    float *part = reinterpret_cast<float *>(lds + kMmTableBytes / 4);   // [wave][rb][v][lane]
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int c = __builtin_amdgcn_readfirstlane(tid >> 6);      // this wave's group of four lanes-of-row
@@ -103,22 +101,25 @@ __global__ __launch_bounds__(kMmThreads) void matmul_kernel(
 #pragma unroll
     for (int rb = 0; rb < kMmMaxRowBlocks; rb++) acc[rb] = v4f32{0.f, 0.f, 0.f, 0.f};
 
-    // Everything a slab needs from memory is requested one slab ahead: this lane's stream
-    // elements (one per row block) with their carry words, and this thread's share of the slab's
-    // activation slice, which goes to LDS after the current slab's products are done.
-    constexpr int kSliceRegs = kMmSliceBytes / 16 / kMmThreads;
-    uint4 e_next[kMmMaxRowBlocks], slice_next[kSliceRegs];
-    uint32_t carry_next[kMmMaxRowBlocks];
+    // Everything a slab needs from memory is requested one slab ahead, straight into registers: this
+    // lane's stream elements (one per row block) with their carry words, and the 32 activation pairs
+    // of its batch column (lanes of one group read 64 consecutive bytes of the packed image, a wave
+    // 256: coalesced, and the image stays in L2).  No LDS staging, so no barrier inside the loop.
+    const uint32_t *xp32 = reinterpret_cast<const uint32_t *>(xp);
+    uint4 e_next[kMmMaxRowBlocks];
+    uint32_t carry_next[kMmMaxRowBlocks], xb_next[32];
     auto request = [&](int slab) {
         const int lanes = slab < T ? 32 : Lt;
         const size_t elem0 = slab < T ? (size_t)slab * m * 32 : (size_t)T * m * 32;
         const size_t slot0 = (size_t)(slab < T ? slab : T) * 1024;
         const int l = 4 * c + g;
+        const bool has_l = l < lanes;
+        // Activation pairs of step q for batch column i: slot 32q + l (full) or q*Lt + l (ragged).
+        // Lanes past the end of a ragged row get zeros: whatever their (all-zero) element decodes
+        // to is then multiplied by zero, so the decode needs no per-lane predicate.
+        const uint32_t *xq = xp32 + (slot0 + (has_l ? l : 0)) * 16 + i;
 #pragma unroll
-        for (int u = 0; u < kSliceRegs; u++) {
-            const int idx = u * kMmThreads + tid;
-            slice_next[u] = idx < 32 * lanes * 4 ? xp[slot0 * 4 + idx] : make_uint4(0, 0, 0, 0);
-        }
+        for (int q = 0; q < 32; q++) xb_next[q] = has_l ? xq[(size_t)q * lanes * 16] : 0u;
 #pragma unroll
         for (int rb = 0; rb < kMmMaxRowBlocks; rb++) {
             const int row = row0 + 16 * rb + i;
@@ -134,37 +135,29 @@ __global__ __launch_bounds__(kMmThreads) void matmul_kernel(
         }
     };
     request(0);
+    __syncthreads();                                              // the table is complete
 
     for (int slab = 0; slab < slabs; slab++) {
         const int lanes = slab < T ? 32 : Lt;                     // elements per row in this slab
         uint4 e_cur[kMmMaxRowBlocks];
-        uint32_t carry_cur[kMmMaxRowBlocks];
+        uint32_t carry_cur[kMmMaxRowBlocks], xb[32];
 #pragma unroll
         for (int rb = 0; rb < kMmMaxRowBlocks; rb++) {
             e_cur[rb] = e_next[rb];
             carry_cur[rb] = carry_next[rb];
         }
-        __syncthreads();                                          // the previous slice is no longer read
 #pragma unroll
-        for (int u = 0; u < kSliceRegs; u++) slice4[u * kMmThreads + tid] = slice_next[u];
-        __syncthreads();
+        for (int q = 0; q < 32; q++) xb[q] = xb_next[q];
         if (slab + 1 < slabs) request(slab + 1);
         if (4 * c >= lanes) continue;                             // nothing of this slab for this wave
-        const int l = 4 * c + g;
-        const bool has_l = l < lanes;
-        const int lx = has_l ? l : 0;
-        // activation pairs of step q for batch column i: slot 32q + l (full) or q*Lt + l (ragged)
-        uint32_t xb[32];
-#pragma unroll
-        for (int q = 0; q < 32; q++) xb[q] = slice[(q * lanes + lx) * 16 + i];
 
 #pragma unroll
         for (int rb = 0; rb < kMmMaxRowBlocks; rb++) {
             if (rb >= row_blocks) break;
             const uint4 e = e_cur[rb];
             const uint32_t carry = carry_cur[rb];
-            const bool live = has_l && row0 + 16 * rb + i < m;
-            v4f32 d = acc[rb];
+            // rows past m decode zeros into tile rows that are never stored
+            v4f32 d0 = acc[rb], d1 = v4f32{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int j = 0; j < 4; j++) {
                 const uint32_t sh = 12 - 4 * j;
@@ -177,11 +170,10 @@ __global__ __launch_bounds__(kMmThreads) void matmul_kernel(
                 gather2(gx, lane4, w2, w3);
                 gather2(gy, lane4, w4, w5);
                 gather2(gz, lane4, w6, w7);
-                if (!live) w0 = w1 = w2 = w3 = w4 = w5 = w6 = w7 = 0u;
-                d = mma4(w0, w1, w2, w3, xb[28 + j], xb[j], xb[16 + j], xb[4 + j], d);
-                d = mma4(w4, w5, w6, w7, xb[20 + j], xb[8 + j], xb[24 + j], xb[12 + j], d);
+                d0 = mma4(w0, w1, w2, w3, xb[28 + j], xb[j], xb[16 + j], xb[4 + j], d0);
+                d1 = mma4(w4, w5, w6, w7, xb[20 + j], xb[8 + j], xb[24 + j], xb[12 + j], d1);
             }
-            acc[rb] = d;
+            acc[rb] = d0 + d1;
         }
     }
 
@@ -235,7 +227,7 @@ static void launch_planes(const uint4 *comp, const uint32_t *cb, const uint32_t 
     if (row_blocks > kMmMaxRowBlocks) row_blocks = kMmMaxRowBlocks;
     const int rows_per_block = 16 * row_blocks;
     const int grid = (m + rows_per_block - 1) / rows_per_block;
-    const int lds_bytes = kMmTableBytes + kMmSliceBytes + kMmWaves * row_blocks * 4 * 64 * 4;
+    const int lds_bytes = kMmTableBytes + kMmWaves * row_blocks * 4 * 64 * 4;
     for (int p = 0; p < planes; p++) {
         const uint4 *xp_plane = reinterpret_cast<const uint4 *>(xp + (size_t)p * (n / 2) * 16);
         uint16_t *out_plane = out + (size_t)p * 16 * m;

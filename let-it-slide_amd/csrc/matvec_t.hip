@@ -39,7 +39,15 @@ __global__ __launch_bounds__(kTThreads) void matvec_t_kernel(
     constexpr int lut_u4 = (2 << L) / 16;
     constexpr uint32_t mask = (1u << L) - 1u;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    for (int i = tid; i < lut_u4; i += kTThreads) lds_u4[i] = codebook[i];
+    {
+        // all of a thread's share of the table is requested before any of it is stored
+        constexpr int kPerThread = lut_u4 / kTThreads;
+        uint4 t[kPerThread];
+#pragma unroll
+        for (int i = 0; i < kPerThread; i++) t[i] = codebook[i * kTThreads + tid];
+#pragma unroll
+        for (int i = 0; i < kPerThread; i++) lds_u4[i * kTThreads + tid] = t[i];
+    }
     __syncthreads();
     const uint16_t *lut = reinterpret_cast<const uint16_t *>(lds_u4);
     float *part = reinterpret_cast<float *>(lds_u4 + lut_u4);      // [wave][lane]
