@@ -18,16 +18,29 @@
 //     (a few hundred KiB) stays in L2 and is read straight into registers one slab ahead; it lives
 //     in a static device buffer (no allocation per call), so calls on different streams of one
 //     device share it and must not overlap.
-//   * a workgroup owns its rows for all slabs, keeps the 16x16 accumulators in registers and
-//     adds the eight waves' tiles in a fixed order at the end: deterministic, no atomics.
+//   * a workgroup owns one slab (2048 columns) of a group of up to 128 rows, so the activation pairs
+//     a wave holds serve every row block of the group (a workgroup that owned whole rows would read
+//     the complete activation image for as few as 16 rows: eight times the bytes of its stream).
+//     Its eight waves' 16x16 tiles are added in LDS in a fixed order and go to a static scratch
+//     buffer as fp32; the workgroup that finishes a row group last (a counter per group) adds the
+//     slabs' partial tiles in slab order and writes fp16.  The order of every sum is fixed, so the
+//     output is deterministic whichever workgroup comes last.
+//   * batch 17..32 decodes once and feeds two sets of MFMAs (two planes of 16 batch columns).
 #include "rptc_common.hpp"
+
+// Development hook: a probe build defines RPTC_MM_STAMP to record a per-wave timestamp at each phase.
+#ifndef RPTC_MM_STAMP
+#define RPTC_MM_STAMP(slot) ((void)0)
+#endif
 
 namespace rptc {
 
 constexpr int kMmThreads = 512;
 constexpr int kMmWaves = kMmThreads / kWave;       // one wave per group of 4 lanes-of-row
 constexpr int kMmTableBytes = 256 * 256;
-constexpr int kMmMaxRowBlocks = 4;                 // 16-row blocks per workgroup
+constexpr int kMmMaxRowBlocks = 8;                 // 16-row blocks per workgroup (6 with two planes: registers)
+constexpr int kMmScratchFloats = 8 << 20;          // 32 MiB of partial tiles
+constexpr int kMmMaxGroups = 32768;
 constexpr int kMmMaxN = 32768;
 constexpr int kMmMaxBatch = 32;
 
@@ -37,13 +50,18 @@ typedef uint32_t v4u32 __attribute__((ext_vector_type(4)));
 
 // activations in [plane of 16 batch columns][slot][16] order, written by pack_x_kernel
 static __device__ __align__(256) uint32_t g_xpack[(kMmMaxBatch / 16) * (kMmMaxN / 2) * 16];
+// partial tiles [row group][slab][row block][plane][256] and one arrival counter per row group
+static __device__ __align__(256) float g_partial[kMmScratchFloats];
+static __device__ __align__(256) uint32_t g_arrived[kMmMaxGroups];
 
 // x: fp16 [batch][n] seen as dwords [batch][n/2]; slot P pairs x[8*idx + 2i], x[8*idx + 2i + 1]
 // with i = P / (n/8), idx = P % (n/8) (inference.cu:215-221): dword 4*idx + i of the row.
 __global__ __launch_bounds__(256) void pack_x_kernel(const uint32_t *__restrict__ x, uint32_t *__restrict__ xp,
-                                                     int n, int batch, int planes)
+                                                     uint32_t *__restrict__ arrived, int groups, int n, int batch,
+                                                     int planes)
 {
     const int t = blockIdx.x * 256 + threadIdx.x;
+    if (t < groups) arrived[t] = 0;   // the counters start every call at zero, whatever an earlier call left
     const int slots = n >> 1, n8 = n >> 3;
     if (t >= planes * slots * 16) return;
     const int j = t & 15, slot = (t >> 4) % slots, plane = (t >> 4) / slots;
@@ -77,87 +95,103 @@ __device__ __forceinline__ void gather2(uint32_t g, uint32_t lane4, uint32_t &w_
     w_lo = lds_read_abs(and_or(h, 0xFF00u, lane4));
 }
 
-template <int S, int MODE>
-__global__ __launch_bounds__(kMmThreads) void matmul_kernel(
-    const uint4 *__restrict__ comp, const uint32_t *__restrict__ codebook, const uint4 *__restrict__ xp,
-    uint16_t *__restrict__ out, int m, int n, int batch, int rows_per_block)
+// four waves per SIMD = two workgroups per CU: at most 128 vector registers
+template <int S, int MODE, int PLANES>
+__global__ __launch_bounds__(kMmThreads) __attribute__((amdgpu_waves_per_eu(4, 4))) void matmul_kernel(
+    const uint4 *__restrict__ comp, const uint32_t *__restrict__ codebook, const uint32_t *__restrict__ xp32,
+    float *__restrict__ partial, uint32_t *__restrict__ arrived, uint16_t *__restrict__ out, int m, int n, int batch,
+    int max_rb, int groups_total, int group_base)
 {
     extern __shared__ uint32_t lds[];
-    float *part = reinterpret_cast<float *>(lds + kMmTableBytes / 4);   // [wave][rb][v][lane]
+    // 64 KiB of table + 16 KiB of tiles: two workgroups share a CU's 160 KiB whatever the batch
+    constexpr int kPartBuffers = PLANES == 1 ? 2 : 1;
+    constexpr int kMaxRb = PLANES == 1 ? kMmMaxRowBlocks : 6;
+    RPTC_MM_STAMP(0);
+    float *part = reinterpret_cast<float *>(lds + kMmTableBytes / 4);   // [buffer][wave][plane][v][lane]
+    // the "came last" flag reuses the first word of the tiles once they are no longer read (all LDS
+    // is dynamic, and 64 + 16 KiB lets two workgroups share a CU)
+    uint32_t *s_last = lds + kMmTableBytes / 4;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int c = __builtin_amdgcn_readfirstlane(tid >> 6);      // this wave's group of four lanes-of-row
     const int i = lane & 15, g = lane >> 4;
-    // the table is the first thing in LDS and the kernel has no static LDS: it starts at address 0
     const uint32_t lane4 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds)) + lane * 4;
     const int T = n >> 11, Lt = (n & 2047) >> 6, slabs = T + (Lt ? 1 : 0);
-    const int row0 = blockIdx.x * rows_per_block;
-    const int row_blocks = rows_per_block >> 4;
+    // grp counts the row groups of this launch (a very tall matrix takes several launches)
+    const int grp = blockIdx.x / slabs, slab = blockIdx.x - grp * slabs;
+    // the row blocks (16 rows each) are dealt to the groups as evenly as integers allow
+    const int total_rb = (m + 15) >> 4;
+    const int rb_begin = (int)(((int64_t)(group_base + grp) * total_rb) / groups_total);
+    const int row_blocks = (int)(((int64_t)(group_base + grp + 1) * total_rb) / groups_total) - rb_begin;
+    const int row0 = rb_begin * 16;
     const uint32_t *comp32 = reinterpret_cast<const uint32_t *>(comp);
 
-    for (int d = tid; d < kMmTableBytes / 4; d += kMmThreads) lds[d] = mm_table_value<S>(codebook, d >> 6);
+    const int lanes = slab < T ? 32 : Lt;                        // elements per row in this slab
+    const size_t elem0 = (size_t)(slab < T ? slab : T) * m * 32;
+    const size_t slot0 = (size_t)(slab < T ? slab : T) * 1024;
+    const int l = 4 * c + g;
+    const bool has_l = l < lanes;
+    const int waves_used = (lanes + 3) >> 2;
 
-    v4f32 acc[kMmMaxRowBlocks];
-#pragma unroll
-    for (int rb = 0; rb < kMmMaxRowBlocks; rb++) acc[rb] = v4f32{0.f, 0.f, 0.f, 0.f};
+    // first request: this thread's row of the table (vector loads return in order)
+    const uint32_t table_value = mm_table_value<S>(codebook, tid >> 1);
 
-    // Everything a slab needs from memory is requested one slab ahead, straight into registers: this
-    // lane's stream elements (one per row block) with their carry words, and the 32 activation pairs
-    // of its batch column (lanes of one group read 64 consecutive bytes of the packed image, a wave
-    // 256: coalesced, and the image stays in L2).  No LDS staging, so no barrier inside the loop.
-    const uint32_t *xp32 = reinterpret_cast<const uint32_t *>(xp);
-    uint4 e_next[kMmMaxRowBlocks];
-    uint32_t carry_next[kMmMaxRowBlocks], xb_next[32];
-    auto request = [&](int slab) {
-        const int lanes = slab < T ? 32 : Lt;
-        const size_t elem0 = slab < T ? (size_t)slab * m * 32 : (size_t)T * m * 32;
-        const size_t slot0 = (size_t)(slab < T ? slab : T) * 1024;
-        const int l = 4 * c + g;
-        const bool has_l = l < lanes;
-        // Activation pairs of step q for batch column i: slot 32q + l (full) or q*Lt + l (ragged).
-        // Lanes past the end of a ragged row get zeros: whatever their (all-zero) element decodes
-        // to is then multiplied by zero, so the decode needs no per-lane predicate.
+    // Everything comes straight into registers, all requests before the first use: the activation
+    // pairs of this lane's 32 steps for its batch column(s) (lanes of one group read 64 consecutive
+    // bytes of the packed image, a wave 256), and this lane's element of every row block with its
+    // carry word.  Lanes past the end of a ragged row get zero activations: whatever their all-zero
+    // element decodes to is multiplied by zero, so the decode needs no per-lane predicate.
+    uint32_t xb[PLANES][32];
+    {
         const uint32_t *xq = xp32 + (slot0 + (has_l ? l : 0)) * 16 + i;
 #pragma unroll
-        for (int q = 0; q < 32; q++) xb_next[q] = has_l ? xq[(size_t)q * lanes * 16] : 0u;
+        for (int p = 0; p < PLANES; p++)
 #pragma unroll
-        for (int rb = 0; rb < kMmMaxRowBlocks; rb++) {
-            const int row = row0 + 16 * rb + i;
-            e_next[rb] = make_uint4(0, 0, 0, 0);
-            carry_next[rb] = 0;
-            if (rb < row_blocks && l < lanes && row < m) {
-                const size_t ei = elem0 + (size_t)row * lanes + l;
-                e_next[rb] = comp[ei];
-                if (l > 0) carry_next[rb] = comp32[ei * 4 - 1];              // last word of the previous lane-of-row
-                else if (MODE == RPTC_AS_WRITTEN) carry_next[rb] = e_next[rb].w;   // inference.cu:232: lane 0 keeps its own
-                else if (slab > 0) carry_next[rb] = comp32[(((size_t)(slab - 1) * m + row) * 32 + 31) * 4 + 3];
-            }
-        }
-    };
-    request(0);
+            for (int q = 0; q < 32; q++) xb[p][q] = has_l ? xq[(size_t)p * (n >> 1) * 16 + (size_t)q * lanes * 16] : 0u;
+    }
+    // No branch around these loads and no use of their results before the row-block loop: a lane
+    // with nothing to decode (row past m, lane past a ragged row, row block past the group) reads
+    // element 0 instead, which is harmless: its products are multiplied by zero activations or land
+    // in tile rows that are never stored.  Lane-of-row 0 reads its own last word as the carry
+    // (inference.cu:232, as written) or lane 31 of the previous slab (continuous).
+    uint4 e_all[kMaxRb];
+    uint32_t carry_all[kMaxRb];
+#pragma unroll
+    for (int rb = 0; rb < kMaxRb; rb++) {
+        const int row = row0 + 16 * rb + i;
+        const bool valid = rb < row_blocks && has_l && row < m;
+        const size_t ei = valid ? elem0 + (size_t)row * lanes + l : 0;
+        size_t ci = ei * 4 + 3;
+        if (l > 0 && valid) ci = ei * 4 - 1;                             // last word of the previous lane-of-row
+        else if (MODE == RPTC_CONTINUOUS && slab > 0 && valid) ci = (((size_t)(slab - 1) * m + row) * 32 + 31) * 4 + 3;
+        e_all[rb] = comp[ei];
+        carry_all[rb] = comp32[ci];
+    }
+    const bool no_carry = MODE == RPTC_CONTINUOUS && slab == 0 && l == 0;     // the stream starts here
+
+    {
+        // table row r = tid / 2 (64 lane copies of one pair): each thread writes 32 copies of the value
+        // it asked for before anything else
+        uint4 *dst = reinterpret_cast<uint4 *>(lds) + (tid >> 1) * 16 + (tid & 1) * 8;
+        const uint4 v4 = make_uint4(table_value, table_value, table_value, table_value);
+#pragma unroll
+        for (int k = 0; k < 8; k++) dst[k] = v4;
+    }
+    RPTC_MM_STAMP(1);
     __syncthreads();                                              // the table is complete
+    RPTC_MM_STAMP(2);
 
-    for (int slab = 0; slab < slabs; slab++) {
-        const int lanes = slab < T ? 32 : Lt;                     // elements per row in this slab
-        uint4 e_cur[kMmMaxRowBlocks];
-        uint32_t carry_cur[kMmMaxRowBlocks], xb[32];
+    float *my_partial = partial + ((size_t)blockIdx.x * max_rb) * (PLANES * 256);
 #pragma unroll
-        for (int rb = 0; rb < kMmMaxRowBlocks; rb++) {
-            e_cur[rb] = e_next[rb];
-            carry_cur[rb] = carry_next[rb];
-        }
+    for (int rb = 0; rb < kMaxRb; rb++) {
+        if (rb >= row_blocks) break;
+        float *buf = part + (kPartBuffers == 2 ? (rb & 1) : 0) * (kMmWaves * PLANES * 256);
+        if (c < waves_used) {
+            const uint4 e = e_all[rb];
+            const uint32_t carry = no_carry ? 0u : carry_all[rb];
+            v4f32 d0[PLANES], d1[PLANES];
 #pragma unroll
-        for (int q = 0; q < 32; q++) xb[q] = xb_next[q];
-        if (slab + 1 < slabs) request(slab + 1);
-        if (4 * c >= lanes) continue;                             // nothing of this slab for this wave
-
-#pragma unroll
-        for (int rb = 0; rb < kMmMaxRowBlocks; rb++) {
-            if (rb >= row_blocks) break;
-            const uint4 e = e_cur[rb];
-            const uint32_t carry = carry_cur[rb];
-            // rows past m decode zeros into tile rows that are never stored
-            v4f32 d0 = acc[rb], d1 = v4f32{0.f, 0.f, 0.f, 0.f};
+            for (int p = 0; p < PLANES; p++) d0[p] = d1[p] = v4f32{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int j = 0; j < 4; j++) {
                 const uint32_t sh = 12 - 4 * j;
@@ -170,74 +204,155 @@ __global__ __launch_bounds__(kMmThreads) void matmul_kernel(
                 gather2(gx, lane4, w2, w3);
                 gather2(gy, lane4, w4, w5);
                 gather2(gz, lane4, w6, w7);
-                d0 = mma4(w0, w1, w2, w3, xb[28 + j], xb[j], xb[16 + j], xb[4 + j], d0);
-                d1 = mma4(w4, w5, w6, w7, xb[20 + j], xb[8 + j], xb[24 + j], xb[12 + j], d1);
+#pragma unroll
+                for (int p = 0; p < PLANES; p++) {
+                    d0[p] = mma4(w0, w1, w2, w3, xb[p][28 + j], xb[p][j], xb[p][16 + j], xb[p][4 + j], d0[p]);
+                    d1[p] = mma4(w4, w5, w6, w7, xb[p][20 + j], xb[p][8 + j], xb[p][24 + j], xb[p][12 + j], d1[p]);
+                }
             }
-            acc[rb] = d0 + d1;
+            // tile element (row 4*(lane/16) + v, batch column lane%16) sits in register v of lane `lane`
+#pragma unroll
+            for (int p = 0; p < PLANES; p++) {
+                const v4f32 d = d0[p] + d1[p];
+#pragma unroll
+                for (int v = 0; v < 4; v++) buf[((c * PLANES + p) * 4 + v) * 64 + lane] = d[v];
+            }
         }
+        if (rb == 0) RPTC_MM_STAMP(3);
+        // With two buffers one barrier per row block is enough: the halves of `part` alternate, and a
+        // wave can only reach the write of row block rb+2 after it passed the barrier of rb+1, which
+        // every wave reaches after its sum of rb.
+        __syncthreads();
+        if (tid < PLANES * 256) {
+            float y = 0.f;
+            const int p = tid >> 8, vl = tid & 255;
+            for (int w = 0; w < waves_used; w++) y += buf[(w * PLANES + p) * 256 + vl];
+            // device-coherent store (written through the XCD's L2): visible to the workgroup on
+            // another XCD that adds the slabs, without flushing a whole cache
+            __hip_atomic_store(&my_partial[rb * (PLANES * 256) + tid], y, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        if (kPartBuffers == 1) __syncthreads();                   // the one buffer is free again
     }
 
-    // add the waves' 16x16 tiles in a fixed order.  Tile element (row 4*(lane/16) + v, batch lane%16)
-    // sits in register v of lane `lane`.
+    // The workgroup that arrives last at its row group's counter adds the slabs' tiles, in slab order.
+    // Every partial tile is stored and loaded with device-scope atomic accesses, which bypass the
+    // XCD-private cache levels, so the only ordering needed is that this workgroup's stores have
+    // completed before its arrival is counted (the wait below, then the barrier).
+    RPTC_MM_STAMP(4);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_waitcnt(0);
+    RPTC_MM_STAMP(5);
     __syncthreads();
-#pragma unroll
-    for (int rb = 0; rb < kMmMaxRowBlocks; rb++) {
-        if (rb < row_blocks) {
-#pragma unroll
-            for (int v = 0; v < 4; v++) part[((c * row_blocks + rb) * 4 + v) * 64 + lane] = acc[rb][v];
-        }
+    if (tid == 0) {
+        const uint32_t prev = __hip_atomic_fetch_add(&arrived[grp], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const bool last = prev == (uint32_t)(slabs - 1);
+        if (last) __hip_atomic_store(&arrived[grp], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // for the next launch
+        *s_last = last;
     }
     __syncthreads();
-    for (int t = tid; t < row_blocks * 256; t += kMmThreads) {
-        const int ln = t & 63, v = (t >> 6) & 3, rb = t >> 8;
-        float y = 0.f;
+    RPTC_MM_STAMP(6);
+    if (!*s_last) return;
+    const int tile_floats = row_blocks * PLANES * 256, tile_stride = max_rb * PLANES * 256;
+    const float *grp_partial = partial + (size_t)grp * slabs * tile_stride;
+    // every thread requests its share of four slabs' tiles before it adds any of them: the loads go
+    // to memory, and one at a time they would cost a round trip each
+    constexpr int kPerThread = kMaxRb * PLANES * 256 / kMmThreads;
+    float y[kPerThread];
 #pragma unroll
-        for (int w = 0; w < kMmWaves; w++) y += part[((w * row_blocks + rb) * 4 + v) * 64 + ln];
-        const int b = ln & 15, row = row0 + 16 * rb + 4 * (ln >> 4) + v;
-        if (b < batch && row < m) out[(size_t)b * m + row] = float_to_half_bits(y);
+    for (int k = 0; k < kPerThread; k++) y[k] = 0.f;
+    for (int sl0 = 0; sl0 < slabs; sl0 += 4) {
+        float v[kPerThread][4];
+#pragma unroll
+        for (int k = 0; k < kPerThread; k++)
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int t = tid + k * kMmThreads;
+                v[k][u] = 0.f;
+                if (t < tile_floats && sl0 + u < slabs)
+                    v[k][u] = __hip_atomic_load(&grp_partial[(size_t)(sl0 + u) * tile_stride + t], __ATOMIC_RELAXED,
+                                                __HIP_MEMORY_SCOPE_AGENT);
+            }
+#pragma unroll
+        for (int k = 0; k < kPerThread; k++)
+#pragma unroll
+            for (int u = 0; u < 4; u++) y[k] += v[k][u];          // slab order
     }
+#pragma unroll
+    for (int k = 0; k < kPerThread; k++) {
+        const int t = tid + k * kMmThreads;
+        if (t >= tile_floats) break;
+        const int ln = t & 63, v = (t >> 6) & 3, p = (t >> 8) % PLANES, rb = t / (PLANES * 256);
+        const int b = 16 * p + (ln & 15), row = row0 + 16 * rb + 4 * (ln >> 4) + v;
+        if (b < batch && row < m) out[(size_t)b * m + row] = float_to_half_bits(y[k]);
+    }
+    RPTC_MM_STAMP(7);
 }
 
-static uint32_t *g_xpack_ptr[64];   // per device: address of g_xpack
+struct MmScratch {
+    uint32_t *xpack;
+    float *partial;
+    uint32_t *arrived;
+};
+static MmScratch g_mm[64];   // per device: addresses of the static scratch arrays
+
+template <typename K>
+static int mm_allow_lds(K kernel)
+{
+    return (int)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    kMaxLds);
+}
 
 int prepare_matmul(int device)
 {
-    const void *k[] = {
-        reinterpret_cast<const void *>(matmul_kernel<6, RPTC_AS_WRITTEN>),
-        reinterpret_cast<const void *>(matmul_kernel<6, RPTC_CONTINUOUS>),
-        reinterpret_cast<const void *>(matmul_kernel<8, RPTC_AS_WRITTEN>),
-        reinterpret_cast<const void *>(matmul_kernel<8, RPTC_CONTINUOUS>),
-    };
-    for (const void *f : k) {
-        int rc = (int)hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds);
-        if (rc) return rc;
-    }
-    // the device address of the static scratch image (the symbol itself is not a device address)
-    return (int)hipGetSymbolAddress(reinterpret_cast<void **>(&g_xpack_ptr[device]), HIP_SYMBOL(g_xpack));
+    int rc;
+    if ((rc = mm_allow_lds(matmul_kernel<6, RPTC_AS_WRITTEN, 1>))) return rc;
+    if ((rc = mm_allow_lds(matmul_kernel<6, RPTC_CONTINUOUS, 1>))) return rc;
+    if ((rc = mm_allow_lds(matmul_kernel<8, RPTC_AS_WRITTEN, 1>))) return rc;
+    if ((rc = mm_allow_lds(matmul_kernel<8, RPTC_CONTINUOUS, 1>))) return rc;
+    if ((rc = mm_allow_lds(matmul_kernel<6, RPTC_AS_WRITTEN, 2>))) return rc;
+    if ((rc = mm_allow_lds(matmul_kernel<6, RPTC_CONTINUOUS, 2>))) return rc;
+    if ((rc = mm_allow_lds(matmul_kernel<8, RPTC_AS_WRITTEN, 2>))) return rc;
+    if ((rc = mm_allow_lds(matmul_kernel<8, RPTC_CONTINUOUS, 2>))) return rc;
+    // the device addresses of the static scratch arrays (the symbols themselves are not device addresses)
+    MmScratch &sc = g_mm[device];
+    if ((rc = (int)hipGetSymbolAddress(reinterpret_cast<void **>(&sc.xpack), HIP_SYMBOL(g_xpack)))) return rc;
+    if ((rc = (int)hipGetSymbolAddress(reinterpret_cast<void **>(&sc.partial), HIP_SYMBOL(g_partial)))) return rc;
+    return (int)hipGetSymbolAddress(reinterpret_cast<void **>(&sc.arrived), HIP_SYMBOL(g_arrived));
 }
 
-template <int S>
-static void launch_planes(const uint4 *comp, const uint32_t *cb, const uint32_t *x, uint32_t *xp, uint16_t *out,
-                          int m, int n, int batch, int carry_mode, int cus, hipStream_t s)
+// Number of row groups: as many as keep every workgroup of the launch resident at once (two per
+// CU), but no group larger than kMmMaxRowBlocks row blocks.
+static int mm_groups(int m, int slabs, int cus, int planes)
 {
-    const int planes = (batch + 15) / 16;
-    const int total = planes * (n / 2) * 16;
-    hipLaunchKernelGGL(pack_x_kernel, dim3((total + 255) / 256), dim3(256), 0, s, x, xp, n, batch, planes);
-    int row_blocks = (m + 16 * cus - 1) / (16 * cus);
-    if (row_blocks > kMmMaxRowBlocks) row_blocks = kMmMaxRowBlocks;
-    const int rows_per_block = 16 * row_blocks;
-    const int grid = (m + rows_per_block - 1) / rows_per_block;
-    const int lds_bytes = kMmTableBytes + kMmWaves * row_blocks * 4 * 64 * 4;
-    for (int p = 0; p < planes; p++) {
-        const uint4 *xp_plane = reinterpret_cast<const uint4 *>(xp + (size_t)p * (n / 2) * 16);
-        uint16_t *out_plane = out + (size_t)p * 16 * m;
-        const int b = batch - 16 * p < 16 ? batch - 16 * p : 16;
+    const int max_rb = planes == 1 ? kMmMaxRowBlocks : 6;
+    const int total = (m + 15) / 16;
+    int groups = 2 * cus / slabs;
+    if (groups < 1) groups = 1;
+    if (groups > total) groups = total;
+    const int least = (total + max_rb - 1) / max_rb;
+    return groups < least ? least : groups;
+}
+
+template <int S, int PLANES>
+static void launch_matmul(const uint4 *comp, const uint32_t *cb, const MmScratch &sc, uint16_t *out, int m, int n,
+                          int batch, int carry_mode, int groups, int slabs, hipStream_t s)
+{
+    const int lds_bytes = kMmTableBytes + kMmWaves * 2 * 256 * 4;
+    const int total = (m + 15) / 16;
+    const int max_rb = (total + groups - 1) / groups;
+    // as many row groups per launch as the scratch buffer holds partial tiles for
+    int64_t per_launch = kMmScratchFloats / ((int64_t)slabs * max_rb * PLANES * 256);
+    if (per_launch > kMmMaxGroups) per_launch = kMmMaxGroups;
+    for (int g0 = 0; g0 < groups; g0 += (int)per_launch) {
+        const int g_n = groups - g0 < per_launch ? groups - g0 : (int)per_launch;
         if (carry_mode == RPTC_AS_WRITTEN)
-            hipLaunchKernelGGL((matmul_kernel<S, RPTC_AS_WRITTEN>), dim3(grid), dim3(kMmThreads), lds_bytes, s, comp,
-                               cb, xp_plane, out_plane, m, n, b, rows_per_block);
+            hipLaunchKernelGGL((matmul_kernel<S, RPTC_AS_WRITTEN, PLANES>), dim3(g_n * slabs), dim3(kMmThreads),
+                               lds_bytes, s, comp, cb, sc.xpack, sc.partial, sc.arrived, out, m, n, batch, max_rb,
+                               groups, g0);
         else
-            hipLaunchKernelGGL((matmul_kernel<S, RPTC_CONTINUOUS>), dim3(grid), dim3(kMmThreads), lds_bytes, s, comp,
-                               cb, xp_plane, out_plane, m, n, b, rows_per_block);
+            hipLaunchKernelGGL((matmul_kernel<S, RPTC_CONTINUOUS, PLANES>), dim3(g_n * slabs), dim3(kMmThreads),
+                               lds_bytes, s, comp, cb, sc.xpack, sc.partial, sc.arrived, out, m, n, batch, max_rb,
+                               groups, g0);
     }
 }
 
@@ -258,14 +373,24 @@ extern "C" int rptc_decompress_matmul(const int32_t *compressed, const uint16_t 
     int rc = device_info(&dev);
     if (rc) return rc;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    Timer t;
-    rc = t.begin(dev, s, ms);
-    if (rc) return rc;
     auto a_comp = reinterpret_cast<const uint4 *>(compressed);
     auto a_cb = reinterpret_cast<const uint32_t *>(codebook);
     auto a_x = reinterpret_cast<const uint32_t *>(x);
-    uint32_t *xp = g_xpack_ptr[dev->device];
-    if (S == 6) launch_planes<6>(a_comp, a_cb, a_x, xp, out, (int)m, (int)n, (int)batch, carry_mode, dev->cus, s);
-    else launch_planes<8>(a_comp, a_cb, a_x, xp, out, (int)m, (int)n, (int)batch, carry_mode, dev->cus, s);
+    const MmScratch &sc = g_mm[dev->device];
+    const int planes = batch > 16 ? 2 : 1;
+    const int slabs = (int)(n / 2048) + (n % 2048 ? 1 : 0);
+    const int groups = mm_groups((int)m, slabs, dev->cus, planes);
+    Timer t;
+    rc = t.begin(dev, s, ms);
+    if (rc) return rc;
+    const int counters = groups < kMmMaxGroups ? groups : kMmMaxGroups;
+    const int total = planes * (int)(n / 2) * 16;
+    const int pack_threads = total > counters ? total : counters;
+    hipLaunchKernelGGL(pack_x_kernel, dim3((pack_threads + 255) / 256), dim3(256), 0, s, a_x, sc.xpack, sc.arrived,
+                       counters, (int)n, (int)batch, planes);
+    if (S == 6 && planes == 1) launch_matmul<6, 1>(a_comp, a_cb, sc, out, (int)m, (int)n, (int)batch, carry_mode, groups, slabs, s);
+    else if (S == 6) launch_matmul<6, 2>(a_comp, a_cb, sc, out, (int)m, (int)n, (int)batch, carry_mode, groups, slabs, s);
+    else if (planes == 1) launch_matmul<8, 1>(a_comp, a_cb, sc, out, (int)m, (int)n, (int)batch, carry_mode, groups, slabs, s);
+    else launch_matmul<8, 2>(a_comp, a_cb, sc, out, (int)m, (int)n, (int)batch, carry_mode, groups, slabs, s);
     return t.end();
 }
