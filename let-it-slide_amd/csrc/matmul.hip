@@ -54,20 +54,26 @@ static __device__ __align__(256) uint32_t g_xpack[(kMmMaxBatch / 16) * (kMmMaxN 
 static __device__ __align__(256) float g_partial[kMmScratchFloats];
 static __device__ __align__(256) uint32_t g_arrived[kMmMaxGroups];
 
-// x: fp16 [batch][n] seen as dwords [batch][n/2]; slot P pairs x[8*idx + 2i], x[8*idx + 2i + 1]
-// with i = P / (n/8), idx = P % (n/8) (inference.cu:215-221): dword 4*idx + i of the row.
-__global__ __launch_bounds__(256) void pack_x_kernel(const uint32_t *__restrict__ x, uint32_t *__restrict__ xp,
+// x: fp16 [batch][n]; slot P pairs x[8*idx + 2i], x[8*idx + 2i + 1] with i = P / (n/8), idx = P % (n/8)
+// (inference.cu:215-221).  Thread (plane, idx, j) reads the 16 bytes x[16*plane + j][8*idx .. 8*idx+7]
+// (a wave: 16 rows x 64 contiguous bytes) and writes one dword to each of the slots i*(n/8) + idx,
+// i = 0..3 (a wave: 256 contiguous bytes per i).
+__global__ __launch_bounds__(256) void pack_x_kernel(const uint4 *__restrict__ x, uint32_t *__restrict__ xp,
                                                      uint32_t *__restrict__ arrived, int groups, int n, int batch,
                                                      int planes)
 {
     const int t = blockIdx.x * 256 + threadIdx.x;
     if (t < groups) arrived[t] = 0;   // the counters start every call at zero, whatever an earlier call left
-    const int slots = n >> 1, n8 = n >> 3;
-    if (t >= planes * slots * 16) return;
-    const int j = t & 15, slot = (t >> 4) % slots, plane = (t >> 4) / slots;
+    const int n8 = n >> 3;
+    if (t >= planes * n8 * 16) return;
+    const int j = t & 15, idx = (t >> 4) % n8, plane = (t >> 4) / n8;
     const int b = plane * 16 + j;
-    const int i = slot / n8, idx = slot - i * n8;
-    xp[t] = b < batch ? x[(size_t)b * slots + 4 * idx + i] : 0u;
+    const uint4 v = b < batch ? x[(size_t)b * n8 + idx] : make_uint4(0, 0, 0, 0);
+    uint32_t *dst = xp + (size_t)plane * (n >> 1) * 16 + (size_t)idx * 16 + j;
+    dst[0] = v.x;
+    dst[(size_t)n8 * 16] = v.y;
+    dst[(size_t)n8 * 32] = v.z;
+    dst[(size_t)n8 * 48] = v.w;
 }
 
 template <int S>
@@ -375,7 +381,6 @@ extern "C" int rptc_decompress_matmul(const int32_t *compressed, const uint16_t 
     hipStream_t s = static_cast<hipStream_t>(stream);
     auto a_comp = reinterpret_cast<const uint4 *>(compressed);
     auto a_cb = reinterpret_cast<const uint32_t *>(codebook);
-    auto a_x = reinterpret_cast<const uint32_t *>(x);
     const MmScratch &sc = g_mm[dev->device];
     const int planes = batch > 16 ? 2 : 1;
     const int slabs = (int)(n / 2048) + (n % 2048 ? 1 : 0);
@@ -384,9 +389,9 @@ extern "C" int rptc_decompress_matmul(const int32_t *compressed, const uint16_t 
     rc = t.begin(dev, s, ms);
     if (rc) return rc;
     const int counters = groups < kMmMaxGroups ? groups : kMmMaxGroups;
-    const int total = planes * (int)(n / 2) * 16;
+    const int total = planes * (int)(n / 8) * 16;
     const int pack_threads = total > counters ? total : counters;
-    hipLaunchKernelGGL(pack_x_kernel, dim3((pack_threads + 255) / 256), dim3(256), 0, s, a_x, sc.xpack, sc.arrived,
+    hipLaunchKernelGGL(pack_x_kernel, dim3((pack_threads + 255) / 256), dim3(256), 0, s, reinterpret_cast<const uint4 *>(x), sc.xpack, sc.arrived,
                        counters, (int)n, (int)batch, planes);
     if (S == 6 && planes == 1) launch_matmul<6, 1>(a_comp, a_cb, sc, out, (int)m, (int)n, (int)batch, carry_mode, groups, slabs, s);
     else if (S == 6) launch_matmul<6, 2>(a_comp, a_cb, sc, out, (int)m, (int)n, (int)batch, carry_mode, groups, slabs, s);
