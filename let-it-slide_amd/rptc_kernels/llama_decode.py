@@ -73,9 +73,10 @@ class QuantizedLlama(torch.nn.Module):
         a, b = t[..., 0::2], t[..., 1::2]
         return torch.stack([a * c - b * s, a * s + b * c], dim=-1).flatten(-2)
 
-    def forward_tokens(self, tokens, pos):
+    def forward_tokens(self, tokens, pos, all_logits=False):
         """tokens [T] long, pos [T] long (their positions, contiguous); writes the KV cache at pos and
-        returns the logits of the last token.  Attention looks at cache positions <= the token's own."""
+        returns the logits of the last token ([1, vocab]), or of every token ([T, vocab]) with
+        ``all_logits``.  Attention looks at cache positions <= the token's own."""
         sh = self.shape
         T, d, f = tokens.numel(), sh.d_model, sh.d_ff
         x = self.embed[tokens]                                                     # [T, d]
@@ -95,8 +96,8 @@ class QuantizedLlama(torch.nn.Module):
             h = self._rms(x, blk.norm2)
             g, u = blk.gate_up_proj(h).split(f, dim=-1)
             x = x + blk.down_proj(torch.nn.functional.silu(g) * u)
-        h = self._rms(x[-1:], self.final_norm)
-        return (h @ self.lm_head.t()).float()                                      # [1, vocab]
+        h = self._rms(x if all_logits else x[-1:], self.final_norm)
+        return (h @ self.lm_head.t()).float()                                      # [T or 1, vocab]
 
     # ---------------------------------------------------------------- fused one-token path
 
