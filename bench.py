@@ -330,7 +330,7 @@ def main():
         g = torch.Generator().manual_seed(42)
         prompt = torch.randint(0, shape.vocab, (512,), generator=g)
         res = {}
-        for mode in ("fused_graph", "fused", "torch_graph", "torch"):
+        for mode in ("fused_graph", "fused", "glue_graph", "torch_graph", "torch"):
             model.k_cache.zero_()
             model.v_cache.zero_()
             toks, dt = greedy_decode(model, prompt, 128, mode=mode)
@@ -340,7 +340,7 @@ def main():
                           "n_gpus": 1, "data": "synthetic",
                           "config": {"workload": f"{shape.layers} layers d=4096 heads=32 mlp=11008 vocab=32000, random-init, "
                                                  f"projections as seeded random 2-bit streams ({stream_bytes} bytes), prompt 512 "
-                                                 f"random ids, 128 greedy tokens; fused_graph = glue kernels + one HIP graph per token"},
+                                                 f"random ids, 128 greedy tokens; fused_graph = five launches per layer (element-wise steps inside the projections) in one HIP graph per token; glue_graph = nine launches per layer"},
                           "results": res}))
         return
     runner = Runner(a.m, a.n, a.S, a.copies)

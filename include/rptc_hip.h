@@ -39,6 +39,7 @@ extern "C" {
 #define RPTC_EMODE (-4)      /* carry_mode is not one of the two modes */
 #define RPTC_ELIMIT (-5)     /* a size exceeds what the kernel's LDS staging can hold */
 #define RPTC_EDEVICE (-6)    /* the current device is not gfx950 */
+#define RPTC_EALIAS (-7)     /* an output buffer aliases an input the op still reads */
 
 /* Library version, major*10000 + minor*100 + patch. */
 int rptc_version(void);
@@ -173,6 +174,7 @@ int rptc_sign_hadamard(const uint16_t *x, const uint16_t *signs, uint16_t *out, 
  *                     cos/sin [max_len][hd/2] at *pos, write q_out and k, v into caches [heads][max_len][hd]
  *   rptc_attn_decode  out[h] = softmax(q[h] . K[h]^T / sqrt(hd)) V[h] over cache positions 0..*pos
  *   rptc_silu_mul     gate_up = [gate|up], each f: out = silu(gate) * up
+ *   rptc_rope_attn_decode  rptc_rope_cache followed by rptc_attn_decode in one launch (q stays on chip)
  */
 int rptc_add_rmsnorm(const uint16_t *x_in, const uint16_t *delta, const uint16_t *weight, uint16_t *x_out,
                      uint16_t *h_out, int64_t d, float eps, void *stream);
@@ -182,6 +184,27 @@ int rptc_rope_cache(const uint16_t *qkv, const uint16_t *cos_t, const uint16_t *
 int rptc_attn_decode(const uint16_t *q, const uint16_t *k_cache, const uint16_t *v_cache, const int64_t *pos,
                      uint16_t *out, int64_t heads, int64_t hd, int64_t max_len, void *stream);
 int rptc_silu_mul(const uint16_t *gate_up, uint16_t *out, int64_t f, void *stream);
+int rptc_rope_attn_decode(const uint16_t *qkv, const uint16_t *cos_t, const uint16_t *sin_t, const int64_t *pos,
+                          uint16_t *k_cache, uint16_t *v_cache, uint16_t *out, int64_t heads, int64_t hd,
+                          int64_t max_len, void *stream);
+
+/*
+ * The mat-vec of rptc_decompress_matvec_16_{S}_1 with the element-wise step that precedes it in a
+ * decoder layer done inside the kernel, while the stream is on its way from memory (no counterpart
+ * in the reference).  Same stream, codebook, shape rules, carry modes and fp16 roundings as the
+ * separate calls.
+ *   rptc_decompress_matvec_silu     activations = silu(gate) * up, gate_up = [gate | up], each n
+ *   rptc_decompress_matvec_rmsnorm  r = x_in + delta (delta may be NULL); x_out = r;
+ *                                   activations = r * rsqrt(mean(r^2) + eps) * weight; n <= 16384;
+ *                                   x_out must not be x_in or delta (RPTC_EALIAS)
+ */
+int rptc_decompress_matvec_silu(const int32_t *compressed, const uint16_t *codebook, const uint16_t *gate_up,
+                                uint16_t *out, int64_t m, int64_t n, int S, int carry_mode, void *stream,
+                                float *ms);
+int rptc_decompress_matvec_rmsnorm(const int32_t *compressed, const uint16_t *codebook, const uint16_t *x_in,
+                                   const uint16_t *delta, const uint16_t *weight, uint16_t *x_out, uint16_t *out,
+                                   int64_t m, int64_t n, float eps, int S, int carry_mode, void *stream,
+                                   float *ms);
 
 #ifdef __cplusplus
 }

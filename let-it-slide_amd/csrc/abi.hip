@@ -65,6 +65,7 @@ extern "C" const char *rptc_status_string(int status)
     case RPTC_EMODE: return "carry_mode must be RPTC_AS_WRITTEN (0) or RPTC_CONTINUOUS (1)";
     case RPTC_ELIMIT: return "a size exceeds what the kernel supports";
     case RPTC_EDEVICE: return "the current device is not a gfx950 GPU";
+    case RPTC_EALIAS: return "an output buffer aliases an input the op still reads";
     default: break;
     }
     if (status > 0) return hipGetErrorString(static_cast<hipError_t>(status));

@@ -34,6 +34,20 @@ __device__ __forceinline__ float block_max(float v, float *scratch)
     return t;
 }
 
+// Rotation of the pair (a, b) by the angle with cosine c and sine s: fp16 products and an fp16
+// difference / sum, as the element-wise framework path computes them.  Contraction is off so that
+// every kernel that rotates rounds the same way (a fused multiply-add would skip one rounding, and
+// which product it skips is the compiler's choice).
+__device__ __forceinline__ void rope_pair(float a, float b, float c, float s, uint16_t &ra, uint16_t &rb)
+{
+#pragma clang fp contract(off)
+    const _Float16 ha = (_Float16)a, hb = (_Float16)b, hc = (_Float16)c, hs = (_Float16)s;
+    const _Float16 ac = ha * hc, bs = hb * hs, as = ha * hs, bc = hb * hc;
+    const _Float16 x = ac - bs, y = as + bc;
+    ra = __builtin_bit_cast(uint16_t, x);
+    rb = __builtin_bit_cast(uint16_t, y);
+}
+
 // x_out = x_in + delta (delta may be null);  h_out = x_out * rsqrt(mean(x_out^2) + eps) * weight
 __global__ __launch_bounds__(1024) void add_rmsnorm_kernel(const uint16_t *__restrict__ x_in, const uint16_t *delta,
                                                             const uint16_t *__restrict__ weight, uint16_t *x_out,
@@ -71,12 +85,8 @@ __global__ __launch_bounds__(256) void rope_cache_kernel(const uint16_t *__restr
     const size_t ce = ((size_t)h * max_len + pos) * hd + 2 * i;
     const float qa = half_bits_to_float(qkv[e]), qb = half_bits_to_float(qkv[e + 1]);
     const float ka = half_bits_to_float(qkv[d + e]), kb = half_bits_to_float(qkv[d + e + 1]);
-    // fp16 products and fp16 difference, as the element-wise framework path computes them
-    auto h16 = [](float v) { return half_bits_to_float(float_to_half_bits(v)); };
-    q_out[e] = float_to_half_bits(h16(qa * c) - h16(qb * s));
-    q_out[e + 1] = float_to_half_bits(h16(qa * s) + h16(qb * c));
-    k_cache[ce] = float_to_half_bits(h16(ka * c) - h16(kb * s));
-    k_cache[ce + 1] = float_to_half_bits(h16(ka * s) + h16(kb * c));
+    rope_pair(qa, qb, c, s, q_out[e], q_out[e + 1]);
+    rope_pair(ka, kb, c, s, k_cache[ce], k_cache[ce + 1]);
     v_cache[ce] = qkv[2 * d + e];
     v_cache[ce + 1] = qkv[2 * d + e + 1];
 }
@@ -88,9 +98,14 @@ __global__ __launch_bounds__(256) void rope_cache_kernel(const uint16_t *__restr
 // interleaved groups whose sums are added in a fixed order.
 constexpr int kAttnThreads = 1024;
 
+// ROPE = true: q is the projection output [q | k | v]; the workgroup first rotates its head's q
+// and k (as rope_cache_kernel does), appends k and v to the caches at *pos and keeps q in LDS,
+// then attends.  Its own writes to the caches are ordered before its reads by the barrier.
+template <bool ROPE>
 __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(
-    const uint16_t *__restrict__ q, const uint16_t *__restrict__ k_cache, const uint16_t *__restrict__ v_cache,
-    const int64_t *__restrict__ pos_p, uint16_t *__restrict__ out, int hd, int max_len)
+    const uint16_t *__restrict__ q, uint16_t *k_cache, uint16_t *v_cache, const uint16_t *__restrict__ cos_t,
+    const uint16_t *__restrict__ sin_t, const int64_t *__restrict__ pos_p, uint16_t *__restrict__ out, int heads, int hd,
+    int max_len)
 {
     extern __shared__ float lds_f[];
     float *scores = lds_f;                       // [max_len]
@@ -98,15 +113,35 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(
     float *acc = scratch + 16;                   // [groups][hd]
     const int h = blockIdx.x, tid = threadIdx.x;
     const int len = (int)*pos_p + 1;
-    const uint16_t *kh = k_cache + (size_t)h * max_len * hd, *vh = v_cache + (size_t)h * max_len * hd;
+    uint16_t *kh = k_cache + (size_t)h * max_len * hd, *vh = v_cache + (size_t)h * max_len * hd;
     const float scale = rsqrtf((float)hd);
+    // [hd] halves behind acc, on a 16-byte boundary; ROPE only
+    uint16_t *q_rot = reinterpret_cast<uint16_t *>(lds_f + ((max_len + 16 + (kAttnThreads / (hd >> 1)) * hd + 3) & ~3));
+    if (ROPE) {
+        const int pos = len - 1, half = hd >> 1, d = heads * hd;
+        if (tid < half) {
+            const int i = tid, e = h * hd + 2 * i;
+            const float c = half_bits_to_float(cos_t[pos * half + i]), s = half_bits_to_float(sin_t[pos * half + i]);
+            const float qa = half_bits_to_float(q[e]), qb = half_bits_to_float(q[e + 1]);
+            const float ka = half_bits_to_float(q[d + e]), kb = half_bits_to_float(q[d + e + 1]);
+            uint16_t *kd = kh + (size_t)pos * hd + 2 * i, *vd = vh + (size_t)pos * hd + 2 * i;
+            rope_pair(qa, qb, c, s, q_rot[2 * i], q_rot[2 * i + 1]);
+            rope_pair(ka, kb, c, s, kd[0], kd[1]);
+            vd[0] = q[2 * d + e];
+            vd[1] = q[2 * d + e + 1];
+        }
+        // the new cache row must have reached memory before other waves read it back
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
+    }
 
     // scores
     const int lanes_per_key = hd >> 3;           // 16 bytes = 8 values per lane
     const int sub = tid % lanes_per_key, slot = tid / lanes_per_key, slots = kAttnThreads / lanes_per_key;
     float qf[8];
     {
-        const uint4 v = *reinterpret_cast<const uint4 *>(q + h * hd + 8 * sub);
+        const uint4 v = ROPE ? *reinterpret_cast<const uint4 *>(q_rot + 8 * sub)
+                             : *reinterpret_cast<const uint4 *>(q + h * hd + 8 * sub);
         const uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
         for (int u = 0; u < 4; u++) {
@@ -220,8 +255,24 @@ extern "C" int rptc_attn_decode(const uint16_t *q, const uint16_t *k_cache, cons
     if (heads < 1 || hd < 16 || hd > 256 || (hd & (hd - 1)) != 0 || max_len < 1) return RPTC_ESHAPE;
     const size_t lds = (size_t)(max_len + 16 + (kAttnThreads / (hd / 2)) * hd) * 4;
     if (lds > 64 * 1024) return RPTC_ELIMIT;
-    hipLaunchKernelGGL(attn_decode_kernel, dim3((unsigned)heads), dim3(kAttnThreads), lds, static_cast<hipStream_t>(stream),
-                       q, k_cache, v_cache, pos, out, (int)hd, (int)max_len);
+    hipLaunchKernelGGL(attn_decode_kernel<false>, dim3((unsigned)heads), dim3(kAttnThreads), lds,
+                       static_cast<hipStream_t>(stream), q, const_cast<uint16_t *>(k_cache), const_cast<uint16_t *>(v_cache),
+                       nullptr, nullptr, pos, out, (int)heads, (int)hd, (int)max_len);
+    return (int)hipGetLastError();
+}
+
+extern "C" int rptc_rope_attn_decode(const uint16_t *qkv, const uint16_t *cos_t, const uint16_t *sin_t, const int64_t *pos,
+                                     uint16_t *k_cache, uint16_t *v_cache, uint16_t *out, int64_t heads, int64_t hd,
+                                     int64_t max_len, void *stream)
+{
+    if (!qkv || !cos_t || !sin_t || !pos || !k_cache || !v_cache || !out) return RPTC_ENULL;
+    if (heads < 1 || hd < 16 || hd > 256 || (hd & (hd - 1)) != 0 || max_len < 1) return RPTC_ESHAPE;
+    if (!aligned16(qkv) || !aligned16(k_cache) || !aligned16(v_cache)) return RPTC_EALIGN;
+    const size_t lds = (size_t)(max_len + 16 + (kAttnThreads / (hd / 2)) * hd + 4) * 4 + (size_t)hd * 2;
+    if (lds > 64 * 1024) return RPTC_ELIMIT;
+    hipLaunchKernelGGL(attn_decode_kernel<true>, dim3((unsigned)heads), dim3(kAttnThreads), lds,
+                       static_cast<hipStream_t>(stream), qkv, k_cache, v_cache, cos_t, sin_t, pos, out, (int)heads, (int)hd,
+                       (int)max_len);
     return (int)hipGetLastError();
 }
 

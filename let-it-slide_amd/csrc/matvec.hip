@@ -151,14 +151,61 @@ struct MatvecArgs {
     int items_tail;       // items of the ragged slab            = ceil(rows_per_block / rw_tail)
 };
 
-template <int S, int MODE, int BITS>
-__global__ __launch_bounds__(kMatvecThreads) void matvec_kernel(
-    const uint32_t *__restrict__ comp, const uint32_t *__restrict__ codebook,
-    const uint4 *__restrict__ x, uint16_t *__restrict__ out, int arg_m, int arg_n, int arg_rows_per_block,
-    int arg_rw_tail, int arg_items_full, int arg_items_tail)
+// Where the activations come from.  Plain: x.  SiluMul: x is [gate | up] (n each) and the
+// activations are silu(gate) * up.  AddRmsNorm: r = x (+ x2), activations = r * rsqrt(mean(r^2) +
+// eps) * norm_w, and workgroup 0 writes r to x_out: the element-wise step that precedes a
+// projection in a decoder layer, done while the stream loads are in flight instead of in a
+// kernel of its own.  The fp16 roundings are those of the stand-alone kernels (decode_glue.hip).
+constexpr int kXPlain = 0, kXSiluMul = 1, kXAddRmsNorm = 2;
+
+struct XFuse {
+    const uint4 *x2;       // AddRmsNorm: the residual delta, or null
+    const uint4 *norm_w;   // AddRmsNorm: the norm's weight
+    uint4 *x_out;          // AddRmsNorm: the updated residual stream (must not alias x or x2)
+    float eps;
+};
+
+struct Halves8 {
+    float v[8];
+};
+
+__device__ __forceinline__ Halves8 unpack8(const uint4 q)
 {
-    // separate scalar arguments (not a struct) so that all of them are preloaded into SGPRs
-    const MatvecArgs a = {arg_m, arg_n, arg_rows_per_block, arg_rw_tail, arg_items_full, arg_items_tail};
+    const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+    Halves8 r;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        r.v[2 * i] = half_bits_to_float((uint16_t)(w[i] & 0xFFFFu));
+        r.v[2 * i + 1] = half_bits_to_float((uint16_t)(w[i] >> 16));
+    }
+    return r;
+}
+
+__device__ __forceinline__ uint4 pack8(const Halves8 &r)
+{
+    uint32_t w[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+        w[i] = (uint32_t)float_to_half_bits(r.v[2 * i]) | ((uint32_t)float_to_half_bits(r.v[2 * i + 1]) << 16);
+    return make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+__device__ __forceinline__ float round_half(float v) { return half_bits_to_float(float_to_half_bits(v)); }
+
+__device__ __forceinline__ uint4 silu_mul8(const uint4 gate, const uint4 up)
+{
+    const Halves8 g = unpack8(gate), u = unpack8(up);
+    Halves8 r;
+#pragma unroll
+    for (int i = 0; i < 8; i++) r.v[i] = round_half(g.v[i] / (1.f + __expf(-g.v[i]))) * u.v[i];
+    return pack8(r);
+}
+
+template <int S, int MODE, int BITS, int XMODE>
+__device__ __forceinline__ void matvec_body(
+    const uint32_t *__restrict__ comp, const uint32_t *__restrict__ codebook,
+    const uint4 *__restrict__ x, uint16_t *__restrict__ out, const MatvecArgs a, const XFuse fuse)
+{
     constexpr int WORDS = 2 * BITS;                        // words per stream element
     constexpr int kBatch = BITS == 2 ? 4 : 2;              // stream elements in flight per lane
     extern __shared__ uint32_t lds[];
@@ -187,11 +234,17 @@ __global__ __launch_bounds__(kMatvecThreads) void matvec_kernel(
         cbv[i] = table_value<S>(codebook, row);
     }
     constexpr int kXRegs = 2;
-    uint4 xv[kXRegs];
+    uint4 xv[kXRegs], xv2[kXRegs], xvw[kXRegs];
+    const uint4 zero4 = make_uint4(0, 0, 0, 0);
 #pragma unroll
     for (int u = 0; u < kXRegs; u++) {
         const int idx = tid + u * kMatvecThreads;
-        xv[u] = idx < n8 ? x[idx] : make_uint4(0, 0, 0, 0);
+        xv[u] = idx < n8 ? x[idx] : zero4;
+        if constexpr (XMODE == kXSiluMul) xv2[u] = idx < n8 ? x[n8 + idx] : zero4;
+        if constexpr (XMODE == kXAddRmsNorm) {
+            xv2[u] = (idx < n8 && fuse.x2) ? fuse.x2[idx] : zero4;
+            xvw[u] = idx < n8 ? fuse.norm_w[idx] : zero4;
+        }
     }
 
     // This wave's items: a contiguous piece of [slab 0 items][slab 1 items]...[ragged slab items].
@@ -253,6 +306,45 @@ __global__ __launch_bounds__(kMatvecThreads) void matvec_kernel(
     load_batch(it_begin);
     RPTC_STAMP(1);
 
+    // the element-wise step in front of the product, on the registers the small loads filled
+    if constexpr (XMODE == kXSiluMul) {
+#pragma unroll
+        for (int u = 0; u < kXRegs; u++) xv[u] = silu_mul8(xv[u], xv2[u]);
+    }
+    if constexpr (XMODE == kXAddRmsNorm) {
+        // host side guarantees n8 <= kXRegs * kMatvecThreads: the whole vector is in registers
+        Halves8 r[kXRegs];
+        float ss = 0.f;
+#pragma unroll
+        for (int u = 0; u < kXRegs; u++) {
+            r[u] = unpack8(xv[u]);
+            if (fuse.x2) {
+                const Halves8 d = unpack8(xv2[u]);
+#pragma unroll
+                for (int i = 0; i < 8; i++) r[u].v[i] = round_half(r[u].v[i] + d.v[i]);   // the fp16 residual stream
+            }
+#pragma unroll
+            for (int i = 0; i < 8; i++) ss += r[u].v[i] * r[u].v[i];
+            const int idx = tid + u * kMatvecThreads;
+            if (blockIdx.x == 0 && idx < n8) fuse.x_out[idx] = pack8(r[u]);
+        }
+        // sum over the workgroup in a fixed order; `part` is not in use before the barrier below
+        ss = wave_sum(ss);
+        if (lane == 63) part[wave] = ss;
+        __syncthreads();
+        float total_ss = 0.f;
+#pragma unroll
+        for (int w = 0; w < kMatvecWaves; w++) total_ss += part[w];
+        const float inv = rsqrtf(total_ss / (float)n + fuse.eps);
+#pragma unroll
+        for (int u = 0; u < kXRegs; u++) {
+            const Halves8 w8 = unpack8(xvw[u]);
+#pragma unroll
+            for (int i = 0; i < 8; i++) r[u].v[i] = round_half(r[u].v[i] * inv) * w8.v[i];
+            xv[u] = pack8(r[u]);
+        }
+    }
+
     // table (256 rows x 64 lane copies) and activation image into LDS
     uint4 *lds4 = reinterpret_cast<uint4 *>(lds);
 #pragma unroll
@@ -269,7 +361,8 @@ __global__ __launch_bounds__(kMatvecThreads) void matvec_kernel(
         const int idx = tid + u * kMatvecThreads;
         if (idx < n8) stage_x(idx, xv[u]);
     }
-    for (int idx = tid + kXRegs * kMatvecThreads; idx < n8; idx += kMatvecThreads) stage_x(idx, x[idx]);
+    for (int idx = tid + kXRegs * kMatvecThreads; idx < n8; idx += kMatvecThreads)
+        stage_x(idx, XMODE == kXSiluMul ? silu_mul8(x[idx], x[n8 + idx]) : x[idx]);
     __syncthreads();
     RPTC_STAMP(2);
 
@@ -354,6 +447,29 @@ __global__ __launch_bounds__(kMatvecThreads) void matvec_kernel(
     RPTC_STAMP(5);
 }
 
+template <int S, int MODE, int BITS>
+__global__ __launch_bounds__(kMatvecThreads) void matvec_kernel(
+    const uint32_t *__restrict__ comp, const uint32_t *__restrict__ codebook,
+    const uint4 *__restrict__ x, uint16_t *__restrict__ out, int arg_m, int arg_n, int arg_rows_per_block,
+    int arg_rw_tail, int arg_items_full, int arg_items_tail)
+{
+    // separate scalar arguments (not a struct) so that all of them are preloaded into SGPRs
+    const MatvecArgs a = {arg_m, arg_n, arg_rows_per_block, arg_rw_tail, arg_items_full, arg_items_tail};
+    matvec_body<S, MODE, BITS, kXPlain>(comp, codebook, x, out, a, XFuse{nullptr, nullptr, nullptr, 0.f});
+}
+
+// 2 bits per weight with an element-wise step fused in front (XMODE above)
+template <int S, int MODE, int XMODE>
+__global__ __launch_bounds__(kMatvecThreads) void matvec_fused_kernel(
+    const uint32_t *__restrict__ comp, const uint32_t *__restrict__ codebook,
+    const uint4 *__restrict__ x, uint16_t *__restrict__ out, int arg_m, int arg_n, int arg_rows_per_block,
+    int arg_rw_tail, int arg_items_full, int arg_items_tail, const uint4 *x2, const uint4 *norm_w, uint4 *x_out,
+    float eps)
+{
+    const MatvecArgs a = {arg_m, arg_n, arg_rows_per_block, arg_rw_tail, arg_items_full, arg_items_tail};
+    matvec_body<S, MODE, 2, XMODE>(comp, codebook, x, out, a, XFuse{x2, norm_w, x_out, eps});
+}
+
 // Dense export: one thread per stream element, 32 pairs scattered to their columns.
 template <int S, int MODE>
 __global__ __launch_bounds__(256) void matvec_dense_kernel(
@@ -395,37 +511,45 @@ static int matvec_lds_bytes(int n, int rows_per_block)
     return kTableBytes + 2 * n + 4 * (n / 64) * rows_per_block;
 }
 
-template <int S, int BITS = 2>
-static int launch_matvec(const int32_t *compressed, const uint16_t *codebook, const uint16_t *x,
-                         uint16_t *out, int64_t m, int64_t n, int carry_mode, void *stream, float *ms)
+// Argument checks and launch geometry shared by every mat-vec entry point.
+static int plan_matvec(const void *compressed, const void *codebook, const void *x, const void *out, int64_t m,
+                       int64_t n, int carry_mode, DeviceInfo **dev, MatvecArgs *a, int *lds_bytes, int *grid)
 {
     if (!compressed || !codebook || !x || !out) return RPTC_ENULL;
     if (m < 1 || n < 64 || n % 64 != 0) return RPTC_ESHAPE;
     if (carry_mode != RPTC_AS_WRITTEN && carry_mode != RPTC_CONTINUOUS) return RPTC_EMODE;
     if (!aligned16(compressed) || !aligned16(codebook) || !aligned16(x)) return RPTC_EALIGN;
     if (m >= (1 << 24) || n >= (1 << 20) || m * n >= ((int64_t)1 << 36)) return RPTC_ELIMIT;
-
-    DeviceInfo *dev;
-    int rc = device_info(&dev);
+    int rc = device_info(dev);
     if (rc) return rc;
     // one workgroup per CU when the per-row partial sums fit in LDS beside the table and the
     // activations, else as many rows per workgroup as do fit
-    MatvecArgs a;
-    a.m = (int)m;
-    a.n = (int)n;
-    a.rows_per_block = 2 * (int)((m + 2 * dev->cus - 1) / (2 * dev->cus));
-    const int fixed_bytes = matvec_lds_bytes(a.n, 0);
-    const int row_bytes = 4 * (a.n / 64);
+    a->m = (int)m;
+    a->n = (int)n;
+    a->rows_per_block = 2 * (int)((m + 2 * (*dev)->cus - 1) / (2 * (*dev)->cus));
+    const int fixed_bytes = matvec_lds_bytes(a->n, 0);
+    const int row_bytes = 4 * (a->n / 64);
     if (fixed_bytes + 2 * row_bytes > kMaxLds) return RPTC_ELIMIT;
     const int fit_rows = ((kMaxLds - fixed_bytes) / row_bytes) & ~1;
-    if (a.rows_per_block > fit_rows) a.rows_per_block = fit_rows;
-    const int lt = (a.n & 2047) >> 6;
-    a.rw_tail = lt ? 64 / lt : 1;
-    a.items_full = a.rows_per_block / 2;
-    a.items_tail = lt ? (a.rows_per_block + a.rw_tail - 1) / a.rw_tail : 0;
-    const int lds_bytes = matvec_lds_bytes(a.n, a.rows_per_block);
-    const int grid = (int)((m + a.rows_per_block - 1) / a.rows_per_block);
+    if (a->rows_per_block > fit_rows) a->rows_per_block = fit_rows;
+    const int lt = (a->n & 2047) >> 6;
+    a->rw_tail = lt ? 64 / lt : 1;
+    a->items_full = a->rows_per_block / 2;
+    a->items_tail = lt ? (a->rows_per_block + a->rw_tail - 1) / a->rw_tail : 0;
+    *lds_bytes = matvec_lds_bytes(a->n, a->rows_per_block);
+    *grid = (int)((m + a->rows_per_block - 1) / a->rows_per_block);
+    return 0;
+}
 
+template <int S, int BITS = 2>
+static int launch_matvec(const int32_t *compressed, const uint16_t *codebook, const uint16_t *x,
+                         uint16_t *out, int64_t m, int64_t n, int carry_mode, void *stream, float *ms)
+{
+    DeviceInfo *dev;
+    MatvecArgs a;
+    int lds_bytes, grid;
+    int rc = plan_matvec(compressed, codebook, x, out, m, n, carry_mode, &dev, &a, &lds_bytes, &grid);
+    if (rc) return rc;
     hipStream_t s = static_cast<hipStream_t>(stream);
     Timer t;
     rc = t.begin(dev, s, ms);
@@ -439,6 +563,37 @@ static int launch_matvec(const int32_t *compressed, const uint16_t *codebook, co
     else
         hipLaunchKernelGGL((matvec_kernel<S, RPTC_CONTINUOUS, BITS>), dim3(grid), dim3(kMatvecThreads), lds_bytes, s,
                            a_comp, a_cb, a_x, out, a.m, a.n, a.rows_per_block, a.rw_tail, a.items_full, a.items_tail);
+    return t.end();
+}
+
+template <int S, int XMODE>
+static int launch_matvec_fused(const int32_t *compressed, const uint16_t *codebook, const uint16_t *x,
+                               const uint16_t *x2, const uint16_t *norm_w, uint16_t *x_out, float eps, uint16_t *out,
+                               int64_t m, int64_t n, int carry_mode, void *stream, float *ms)
+{
+    DeviceInfo *dev;
+    MatvecArgs a;
+    int lds_bytes, grid;
+    int rc = plan_matvec(compressed, codebook, x, out, m, n, carry_mode, &dev, &a, &lds_bytes, &grid);
+    if (rc) return rc;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    Timer t;
+    rc = t.begin(dev, s, ms);
+    if (rc) return rc;
+    auto a_comp = reinterpret_cast<const uint32_t *>(compressed);
+    auto a_cb = reinterpret_cast<const uint32_t *>(codebook);
+    auto a_x = reinterpret_cast<const uint4 *>(x);
+    auto a_x2 = reinterpret_cast<const uint4 *>(x2);
+    auto a_w = reinterpret_cast<const uint4 *>(norm_w);
+    auto a_xo = reinterpret_cast<uint4 *>(x_out);
+    if (carry_mode == RPTC_AS_WRITTEN)
+        hipLaunchKernelGGL((matvec_fused_kernel<S, RPTC_AS_WRITTEN, XMODE>), dim3(grid), dim3(kMatvecThreads), lds_bytes,
+                           s, a_comp, a_cb, a_x, out, a.m, a.n, a.rows_per_block, a.rw_tail, a.items_full, a.items_tail,
+                           a_x2, a_w, a_xo, eps);
+    else
+        hipLaunchKernelGGL((matvec_fused_kernel<S, RPTC_CONTINUOUS, XMODE>), dim3(grid), dim3(kMatvecThreads), lds_bytes,
+                           s, a_comp, a_cb, a_x, out, a.m, a.n, a.rows_per_block, a.rw_tail, a.items_full, a.items_tail,
+                           a_x2, a_w, a_xo, eps);
     return t.end();
 }
 
@@ -525,6 +680,14 @@ int prepare_matvec()
     RPTC_SET_LIMITS(3)
     RPTC_SET_LIMITS(4)
 #undef RPTC_SET_LIMITS
+#define RPTC_SET_LIMITS(XMODE)                                                                    \
+    if ((rc = set_lds_limit(matvec_fused_kernel<6, RPTC_AS_WRITTEN, XMODE>))) return rc;             \
+    if ((rc = set_lds_limit(matvec_fused_kernel<6, RPTC_CONTINUOUS, XMODE>))) return rc;             \
+    if ((rc = set_lds_limit(matvec_fused_kernel<8, RPTC_AS_WRITTEN, XMODE>))) return rc;             \
+    if ((rc = set_lds_limit(matvec_fused_kernel<8, RPTC_CONTINUOUS, XMODE>))) return rc;
+    RPTC_SET_LIMITS(kXSiluMul)
+    RPTC_SET_LIMITS(kXAddRmsNorm)
+#undef RPTC_SET_LIMITS
     return 0;
 }
 
@@ -554,6 +717,29 @@ extern "C" int rptc_decompress_matvec_20_8_1(const int32_t *c, const uint16_t *c
                                              int64_t m, int64_t n, int mode, void *stream, float *ms)
 {
     return launch_matvec<8>(c, cb, x, out, m, n, mode, stream, ms);
+}
+
+extern "C" int rptc_decompress_matvec_silu(const int32_t *c, const uint16_t *cb, const uint16_t *gate_up, uint16_t *out,
+                                           int64_t m, int64_t n, int S, int mode, void *stream, float *ms)
+{
+    if (S != 6 && S != 8) return RPTC_ESHAPE;
+    return S == 6 ? launch_matvec_fused<6, kXSiluMul>(c, cb, gate_up, nullptr, nullptr, nullptr, 0.f, out, m, n, mode, stream, ms)
+                  : launch_matvec_fused<8, kXSiluMul>(c, cb, gate_up, nullptr, nullptr, nullptr, 0.f, out, m, n, mode, stream, ms);
+}
+
+extern "C" int rptc_decompress_matvec_rmsnorm(const int32_t *c, const uint16_t *cb, const uint16_t *x_in,
+                                              const uint16_t *delta, const uint16_t *weight, uint16_t *x_out,
+                                              uint16_t *out, int64_t m, int64_t n, float eps, int S, int mode,
+                                              void *stream, float *ms)
+{
+    if (!weight || !x_out) return RPTC_ENULL;
+    if (S != 6 && S != 8) return RPTC_ESHAPE;
+    // every workgroup reads x_in and delta while workgroup 0 writes x_out
+    if (x_out == x_in || x_out == delta) return RPTC_EALIAS;
+    if (!aligned16(delta) || !aligned16(weight) || !aligned16(x_out)) return RPTC_EALIGN;
+    if (n > 8 * 2 * kMatvecThreads) return RPTC_ELIMIT;      // the whole vector sits in two registers per thread
+    return S == 6 ? launch_matvec_fused<6, kXAddRmsNorm>(c, cb, x_in, delta, weight, x_out, eps, out, m, n, mode, stream, ms)
+                  : launch_matvec_fused<8, kXAddRmsNorm>(c, cb, x_in, delta, weight, x_out, eps, out, m, n, mode, stream, ms);
 }
 
 extern "C" int rptc_matvec_dense(const int32_t *compressed, const uint16_t *codebook, uint16_t *W, int64_t m,

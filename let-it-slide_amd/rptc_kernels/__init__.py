@@ -59,6 +59,10 @@ _SIGNATURES = {
     "rptc_rope_cache": ([_VP, _VP, _VP, _VP, _VP, _VP, _VP, _I64, _I64, _I64, _VP], _INT),
     "rptc_attn_decode": ([_VP, _VP, _VP, _VP, _VP, _I64, _I64, _I64, _VP], _INT),
     "rptc_silu_mul": ([_VP, _VP, _I64, _VP], _INT),
+    "rptc_rope_attn_decode": ([_VP, _VP, _VP, _VP, _VP, _VP, _VP, _I64, _I64, _I64, _VP], _INT),
+    "rptc_decompress_matvec_silu": ([_VP, _VP, _VP, _VP, _I64, _I64, _INT, _INT, _VP, _FP], _INT),
+    "rptc_decompress_matvec_rmsnorm": ([_VP, _VP, _VP, _VP, _VP, _VP, _VP, _I64, _I64, ctypes.c_float, _INT, _INT,
+                                        _VP, _FP], _INT),
 }
 
 
@@ -368,6 +372,52 @@ def decompress_matvec_bits(compressed, codebook, x, out, bits):
     _check(n % 64 == 0 and n >= 64 and m >= 1, "x.size(0) % 64 == 0")
     _check(compressed.numel() * 32 == m * n * bits, "compressed.numel() * 32 == m * n * bits")
     return _call(library().rptc_decompress_matvec_bits, (compressed, codebook, x, out), m, n, S, bits)
+
+
+def _fused_common(compressed, codebook, out, n):
+    _check_input(compressed, "compressed")
+    _check(compressed.dtype == torch.int32, "compressed.scalar_type() == torch::kInt32")
+    _check_input(codebook, "codebook")
+    _check(codebook.dim() == 1 and codebook.size(0) in (128, 512), "codebook.size(0) == 1<<(S+V), S in {6, 8}")
+    _check(codebook.dtype == torch.float16, "codebook.scalar_type() == torch::kFloat16")
+    _check_input(out, "out")
+    _check(out.dim() == 1 and out.dtype == torch.float16, "out must be a 1-D fp16 tensor")
+    m = out.size(0)
+    _check(n % 64 == 0 and n >= 64 and m >= 1, "x.size(0) % 64 == 0")
+    _check(compressed.numel() * 16 == m * n, "compressed.numel() * 16 == m * n")
+    return m, (6 if codebook.size(0) == 128 else 8)
+
+
+def decompress_matvec_silu(compressed, codebook, gate_up, out):
+    """out = W (silu(gate) * up) with gate_up = [gate | up] (fp16 [2n]): ``decompress_matvec_16_{S}_1`` with the
+    gate of a Llama MLP computed inside the kernel.  Returns elapsed ms."""
+    _check_input(gate_up, "gate_up")
+    _check(gate_up.dim() == 1 and gate_up.dtype == torch.float16 and gate_up.size(0) % 2 == 0,
+           "gate_up must be a 1-D fp16 tensor of even length")
+    n = gate_up.size(0) // 2
+    m, S = _fused_common(compressed, codebook, out, n)
+    return _call(library().rptc_decompress_matvec_silu, (compressed, codebook, gate_up, out), m, n, S)
+
+
+def decompress_matvec_rmsnorm(compressed, codebook, x_in, delta, weight, x_out, out, eps=1e-5):
+    """x_out = x_in + delta (delta may be None); out = W (rmsnorm(x_out) * weight): ``decompress_matvec_16_{S}_1``
+    with the residual add and RMS norm of a decoder layer computed inside the kernel.  ``x_out`` must be a
+    buffer of its own (not ``x_in``, not ``delta``).  Returns elapsed ms."""
+    for t, name in ((x_in, "x_in"), (weight, "weight"), (x_out, "x_out")) + (((delta, "delta"),) if delta is not None else ()):
+        _check_input(t, name)
+        _check(t.dim() == 1 and t.dtype == torch.float16 and t.size(0) == x_in.size(0), f"{name} must be fp16 [n]")
+    n = x_in.size(0)
+    m, S = _fused_common(compressed, codebook, out, n)
+    device = compressed.device
+    ms = ctypes.c_float(0.0)
+    with torch.cuda.device(device):
+        stream = torch.cuda.current_stream().cuda_stream
+        rc = library().rptc_decompress_matvec_rmsnorm(
+            compressed.data_ptr(), codebook.data_ptr(), x_in.data_ptr(), None if delta is None else delta.data_ptr(),
+            weight.data_ptr(), x_out.data_ptr(), out.data_ptr(), m, n, float(eps), S, _carry_mode,
+            ctypes.c_void_p(stream), ctypes.byref(ms) if _timing else None)
+    _status(rc)
+    return float(ms.value)
 
 
 def matvec_bits_dense(compressed, codebook, out, bits):

@@ -57,7 +57,7 @@ class QuantizedLlama(torch.nn.Module):
         self.v_cache = torch.zeros_like(self.k_cache)
         # work buffers of the one-token path
         z = lambda k: torch.zeros(k, dtype=torch.float16, device=device)
-        self._x, self._h, self._qkv, self._q, self._att = z(d), z(d), z(3 * d), z(d), z(d)
+        self._x, self._x2, self._h, self._qkv, self._q, self._att = z(d), z(d), z(d), z(3 * d), z(d), z(d)
         self._o, self._gu, self._act, self._down = z(d), z(2 * f), z(f), z(d)
 
     # ---------------------------------------------------------------- torch path (any number of tokens)
@@ -101,9 +101,13 @@ class QuantizedLlama(torch.nn.Module):
 
     # ---------------------------------------------------------------- fused one-token path
 
-    def decode_step(self, token, pos):
+    def decode_step(self, token, pos, fuse=True):
         """token [1] long, pos [1] long, both on the device (read by the kernels, so a captured graph can be
-        replayed with new values).  Returns the logits [1, vocab] (float)."""
+        replayed with new values).  Returns the logits [1, vocab] (float).
+
+        ``fuse`` (default): five launches per layer - the qkv and gate/up projections do the residual add and
+        RMS norm in their prologue, the down projection the SiLU gate, and one kernel rotates q and k, appends
+        to the cache and attends.  ``fuse=False``: the same arithmetic as nine launches per layer."""
         sh = self.shape
         lib = rk.library()
         stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
@@ -118,8 +122,33 @@ class QuantizedLlama(torch.nn.Module):
             ok(fn(layer.compressed.data_ptr(), layer.codebook.data_ptr(), x.data_ptr(), out.data_ptr(),
                   layer.out_features, layer.in_features, layer.carry_mode, stream, None))
 
+        def gemv_norm(layer, x_in, delta, weight, x_out, out):
+            ok(lib.rptc_decompress_matvec_rmsnorm(layer.compressed.data_ptr(), layer.codebook.data_ptr(), x_in.data_ptr(),
+                                                  delta, weight.data_ptr(), x_out.data_ptr(), out.data_ptr(),
+                                                  layer.out_features, layer.in_features, self.EPS, layer.S,
+                                                  layer.carry_mode, stream, None))
+
+        def gemv_silu(layer, gate_up, out):
+            ok(lib.rptc_decompress_matvec_silu(layer.compressed.data_ptr(), layer.codebook.data_ptr(), gate_up.data_ptr(),
+                                               out.data_ptr(), layer.out_features, layer.in_features, layer.S,
+                                               layer.carry_mode, stream, None))
+
         self._x.copy_(self.embed[token].reshape(-1))
         delta = None
+        if fuse:
+            xa, xb = self._x, self._x2          # the residual stream alternates between two buffers
+            for i, blk in enumerate(self.blocks):
+                gemv_norm(blk.qkv_proj, xa, delta, blk.norm1, xb, self._qkv)
+                ok(lib.rptc_rope_attn_decode(self._qkv.data_ptr(), self.cos.data_ptr(), self.sin.data_ptr(), pos.data_ptr(),
+                                             self.k_cache[i].data_ptr(), self.v_cache[i].data_ptr(), self._att.data_ptr(),
+                                             sh.heads, sh.head_dim, sh.max_len, stream))
+                gemv(blk.o_proj, self._att, self._o)
+                gemv_norm(blk.gate_up_proj, xb, self._o.data_ptr(), blk.norm2, xa, self._gu)
+                gemv_silu(blk.down_proj, self._gu, self._down)
+                delta = self._down.data_ptr()
+            ok(lib.rptc_add_rmsnorm(xa.data_ptr(), delta, self.final_norm.data_ptr(), xb.data_ptr(), self._h.data_ptr(), d,
+                                    self.EPS, stream))
+            return (self._h.unsqueeze(0) @ self.lm_head.t()).float()
         for i, blk in enumerate(self.blocks):
             ok(lib.rptc_add_rmsnorm(self._x.data_ptr(), delta, blk.norm1.data_ptr(), self._x.data_ptr(),
                                     self._h.data_ptr(), d, self.EPS, stream))
@@ -143,13 +172,19 @@ class QuantizedLlama(torch.nn.Module):
 
 def greedy_decode(model, prompt, new_tokens, mode="fused_graph"):
     """Prefill the prompt (in chunks of 32 tokens: the batch the fused mat-mat kernel takes), then decode
-    ``new_tokens`` greedily one at a time.  mode: "fused_graph" (glue kernels, one HIP graph per token),
-    "fused" (glue kernels, direct launches), "torch_graph" / "torch" (framework ops between the projections).
+    ``new_tokens`` greedily one at a time.  mode: "fused_graph" (five launches per layer, one HIP graph per
+    token), "fused" (the same, direct launches), "glue_graph" / "glue" (nine launches per layer: the
+    element-wise steps as kernels of their own), "torch_graph" / "torch" (framework ops between the projections).
     Returns (token list, seconds spent in the decode loop)."""
     dev = model.embed.device
     prompt = torch.as_tensor(prompt, dtype=torch.long, device=dev)
     P = prompt.numel()
-    step = model.decode_step if mode.startswith("fused") else model.forward_tokens
+    if mode.startswith("fused"):
+        step = model.decode_step
+    elif mode.startswith("glue"):
+        step = lambda t, p: model.decode_step(t, p, fuse=False)
+    else:
+        step = model.forward_tokens
     with torch.no_grad():
         logits = None
         for p0 in range(0, P, 32):

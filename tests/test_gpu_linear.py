@@ -3,7 +3,7 @@ import numpy as np
 import pytest
 import torch
 
-from util import rel_l2
+from util import rand_codes, rand_half, rel_l2
 
 pytestmark = pytest.mark.gpu
 
@@ -147,10 +147,11 @@ def test_llama_decode_paths_agree(rk):
     model = QuantizedLlama(shape, S=8, seed=7)
     prompt = torch.randint(0, shape.vocab, (40,), generator=torch.Generator().manual_seed(1))
     runs = {}
-    for mode in ("fused_graph", "fused", "torch_graph", "torch"):
+    for mode in ("fused_graph", "fused", "glue_graph", "glue", "torch_graph", "torch"):
         model.k_cache.zero_(); model.v_cache.zero_()
         runs[mode], _ = greedy_decode(model, prompt, 12, mode=mode)
     assert runs["fused_graph"] == runs["fused"]
+    assert runs["glue_graph"] == runs["glue"]
     assert runs["torch_graph"] == runs["torch"]
 
     # one decode step after the same prefill: fused glue vs torch glue
@@ -168,6 +169,12 @@ def test_llama_decode_paths_agree(rk):
         lf = model.decode_step(tok, p40)
         assert rel_l2(lf.cpu().numpy(), lt.cpu().numpy()) < 1e-2
         assert rel_l2(model.k_cache.float().cpu().numpy(), kt.float().cpu().numpy()) < 1e-2
+        # nine launches per layer against five: the same roundings, so nearly the same logits
+        kf = model.k_cache.clone()
+        model.k_cache.copy_(kc); model.v_cache.copy_(vc)
+        lg = model.decode_step(tok, p40, fuse=False)
+        assert rel_l2(lf.cpu().numpy(), lg.cpu().numpy()) < 2e-3
+        assert rel_l2(model.k_cache.float().cpu().numpy(), kf.float().cpu().numpy()) < 2e-3
 
     # dense reference: swap every QuantizedLinear for a matmul with its decoded weight
     class Dense(torch.nn.Module):
@@ -188,3 +195,118 @@ def test_llama_decode_paths_agree(rk):
         model.k_cache.zero_(); model.v_cache.zero_()
         logits_d = model.forward_tokens(prompt[:32].cuda(), pos[:32])
     assert rel_l2(logits_q.cpu().numpy(), logits_d.cpu().numpy()) < 2e-2
+
+
+# ------------------------------------------------------------------ projections with a fused element-wise prologue
+
+def _stream(m, n, S=8, seed=0):
+    comp = rand_codes(m * n // 16, seed=seed + m + n).cuda()
+    cb = rand_half(2 << S, seed=seed + S).cuda()
+    return comp, cb
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+@pytest.mark.parametrize("S", [6, 8])
+@pytest.mark.parametrize("m,n", [(64, 2048), (33, 704), (96, 4096 + 768), (32, 28672)])
+def test_matvec_silu_equals_silu_then_matvec(rk, mode, S, m, n):
+    """The gate is computed with the roundings of the stand-alone kernel, so the fused call is bit-identical."""
+    import ctypes
+    comp, cb = _stream(m, n, S, seed=3)
+    gu = rand_half(2 * n, seed=21).cuda()
+    act = torch.empty(n, dtype=torch.float16, device="cuda")
+    rc = rk.library().rptc_silu_mul(gu.data_ptr(), act.data_ptr(), n, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert rc == 0
+    want = torch.full((m,), float("nan"), dtype=torch.float16, device="cuda")
+    got = torch.full((m,), float("nan"), dtype=torch.float16, device="cuda")
+    prev = rk.set_carry_mode(mode)
+    try:
+        getattr(rk, f"decompress_matvec_16_{S}_1")(comp.reshape(n // 2048, m, 128) if n % 2048 == 0 else comp, cb, act, want)
+        ms = rk.decompress_matvec_silu(comp, cb, gu, got)
+    finally:
+        rk.set_carry_mode(prev)
+    assert ms > 0
+    g, u = gu[:n].float(), gu[n:].float()
+    assert rel_l2(act.float().cpu().numpy(), (torch.nn.functional.silu(g) * u).cpu().numpy()) < 1e-3
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+@pytest.mark.parametrize("with_delta", [False, True])
+@pytest.mark.parametrize("m,n", [(64, 2048), (40, 256), (96, 4096), (32, 16384)])
+def test_matvec_rmsnorm_equals_norm_then_matvec(rk, mode, with_delta, m, n):
+    import ctypes
+    S = 8
+    comp, cb = _stream(m, n, S, seed=5)
+    x = rand_half(n, seed=31).cuda()
+    delta = rand_half(n, seed=32, scale=0.5).cuda() if with_delta else None
+    w = (1.0 + 0.1 * rand_half(n, seed=33).float()).half().cuda()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    x_ref, h_ref = torch.empty_like(x), torch.empty_like(x)
+    rc = rk.library().rptc_add_rmsnorm(x.data_ptr(), None if delta is None else delta.data_ptr(), w.data_ptr(),
+                                       x_ref.data_ptr(), h_ref.data_ptr(), n, 1e-5, stream)
+    assert rc == 0
+    want = torch.full((m,), float("nan"), dtype=torch.float16, device="cuda")
+    got = torch.full((m,), float("nan"), dtype=torch.float16, device="cuda")
+    x_out = torch.full((n,), float("nan"), dtype=torch.float16, device="cuda")
+    prev = rk.set_carry_mode(mode)
+    try:
+        getattr(rk, f"decompress_matvec_16_{S}_1")(comp.reshape(n // 2048, m, 128) if n % 2048 == 0 else comp, cb, h_ref, want)
+        rk.decompress_matvec_rmsnorm(comp, cb, x, delta, w, x_out, got, eps=1e-5)
+    finally:
+        rk.set_carry_mode(prev)
+    assert torch.equal(x_out.view(torch.int16), x_ref.view(torch.int16))       # the residual stream is exact
+    # the norm: against float64 from the definition
+    r = x_ref.double()
+    h64 = r * torch.rsqrt((r * r).mean() + 1e-5) * w.double()
+    assert rel_l2(h_ref.float().cpu().numpy(), h64.cpu().numpy()) < 1e-3
+    # the sum of squares is added in another order, so the activations may differ in the last fp16 bit
+    assert rel_l2(got.float().cpu().numpy(), want.float().cpu().numpy()) < 1e-3
+
+
+def test_matvec_rmsnorm_rejects_aliases_and_long_vectors(rk):
+    m, n = 32, 2048
+    comp, cb = _stream(m, n, 8, seed=9)
+    x, w = rand_half(n, seed=1).cuda(), rand_half(n, seed=2).cuda()
+    out = torch.empty(m, dtype=torch.float16, device="cuda")
+    with pytest.raises(RuntimeError, match="aliases"):
+        rk.decompress_matvec_rmsnorm(comp, cb, x, None, w, x, out)
+    with pytest.raises(RuntimeError, match="aliases"):
+        rk.decompress_matvec_rmsnorm(comp, cb, x, w, w, w, out)
+    n2 = 16384 + 2048
+    comp2, _ = _stream(m, n2, 8, seed=10)
+    x2 = rand_half(n2, seed=3).cuda()
+    with pytest.raises(RuntimeError):
+        rk.decompress_matvec_rmsnorm(comp2, cb, x2, None, x2.clone(), torch.empty_like(x2), out)
+
+
+@pytest.mark.parametrize("heads,hd,max_len,pos", [(4, 64, 128, 0), (4, 64, 128, 77), (32, 128, 1024, 640), (2, 16, 64, 63)])
+def test_rope_attn_decode_equals_rope_then_attention(rk, heads, hd, max_len, pos):
+    import ctypes
+    lib = rk.library()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    d = heads * hd
+    g = torch.Generator().manual_seed(pos + heads)
+    qkv = torch.randn(3 * d, generator=g).half().cuda()
+    kc = torch.randn((heads, max_len, hd), generator=g).half().cuda()
+    vc = torch.randn((heads, max_len, hd), generator=g).half().cuda()
+    ang = torch.arange(max_len).float()[:, None] / (10000.0 ** (torch.arange(0, hd, 2).float() / hd))[None, :]
+    cos, sin = ang.cos().half().cuda().contiguous(), ang.sin().half().cuda().contiguous()
+    p = torch.tensor([pos], dtype=torch.long, device="cuda")
+    k1, v1, k2, v2 = kc.clone(), vc.clone(), kc.clone(), vc.clone()
+    q = torch.empty(d, dtype=torch.float16, device="cuda")
+    o1 = torch.empty(d, dtype=torch.float16, device="cuda")
+    o2 = torch.full((d,), float("nan"), dtype=torch.float16, device="cuda")
+    assert lib.rptc_rope_cache(qkv.data_ptr(), cos.data_ptr(), sin.data_ptr(), p.data_ptr(), q.data_ptr(), k1.data_ptr(),
+                               v1.data_ptr(), heads, hd, max_len, stream) == 0
+    assert lib.rptc_attn_decode(q.data_ptr(), k1.data_ptr(), v1.data_ptr(), p.data_ptr(), o1.data_ptr(), heads, hd, max_len,
+                                stream) == 0
+    assert lib.rptc_rope_attn_decode(qkv.data_ptr(), cos.data_ptr(), sin.data_ptr(), p.data_ptr(), k2.data_ptr(),
+                                     v2.data_ptr(), o2.data_ptr(), heads, hd, max_len, stream) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(k1.view(torch.int16), k2.view(torch.int16)) and torch.equal(v1.view(torch.int16), v2.view(torch.int16))
+    assert torch.equal(o1.view(torch.int16), o2.view(torch.int16))
+    # and against the definition in float64
+    kk, vv = k1[:, :pos + 1].double(), v1[:, :pos + 1].double()
+    sc = torch.einsum("hd,hsd->hs", q.view(heads, hd).double(), kk) / hd ** 0.5
+    want = torch.einsum("hs,hsd->hd", torch.softmax(sc, dim=-1), vv).reshape(-1)
+    assert rel_l2(o2.float().cpu().numpy(), want.cpu().numpy()) < 2e-3
