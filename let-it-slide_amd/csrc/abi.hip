@@ -11,6 +11,7 @@ int prepare_matvec();
 int prepare_matvec_t();
 int prepare_matmul(int device);
 int prepare_hadamard();
+int prepare_decode_glue(int device);
 
 constexpr int kMaxDevices = 64;
 static DeviceInfo g_devices[kMaxDevices];
@@ -39,6 +40,7 @@ int device_info(DeviceInfo **out)
         if ((rc = prepare_matvec_t())) return rc;
         if ((rc = prepare_matmul(dev))) return rc;
         if ((rc = prepare_hadamard())) return rc;
+        if ((rc = prepare_decode_glue(dev))) return rc;
         g_ready[dev] = true;
     }
     *out = &g_devices[dev];

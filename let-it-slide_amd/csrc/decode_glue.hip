@@ -91,44 +91,58 @@ __global__ __launch_bounds__(256) void rope_cache_kernel(const uint16_t *__restr
     v_cache[ce + 1] = qkv[2 * d + e + 1];
 }
 
-// One workgroup of 1024 threads per head: softmax(q . K^T / sqrt(hd)) V over cache positions 0..pos.
-// Scores: 16 lanes share a key (16 bytes of it each, so a wave reads 1 KiB of four consecutive
-// keys per load) and add their partial dot products with DPP-free shuffles inside the 16.
-// Values: a thread owns one pair of output dimensions, the keys are cut into 1024 / (hd/2)
-// interleaved groups whose sums are added in a fixed order.
-constexpr int kAttnThreads = 1024;
+// Single-query attention: softmax(q . K^T / sqrt(hd)) V over cache positions 0..pos.
+// A head's keys are cut into `splits` contiguous pieces, one 256-thread workgroup each, so that a
+// decode step with few heads still fills the chip (heads * splits workgroups).  A workgroup
+// produces the piece's maximum score m, the sum l of exp(score - m) and the unnormalised
+// acc = sum exp(score - m) * V; they go to a static scratch buffer with device-scope stores, and
+// the workgroup that arrives last at the head's counter merges the pieces in piece order:
+// out = sum_i acc_i * exp(m_i - M) / sum_i l_i * exp(m_i - M).  Every sum has a fixed order.
+// Scores: hd/8 lanes share a key (16 bytes of it each) and add their partial dot products with
+// shuffles.  Values: a thread owns one pair of output dimensions, the keys are cut into
+// 256 / (hd/2) interleaved groups whose sums are added in a fixed order.
+// ROPE = true: q is the projection output [q | k | v]; every workgroup rotates its head's q into
+// LDS, and the one whose piece holds *pos also rotates k and appends k and v to the caches (as
+// rope_cache_kernel does) before it reads that row back.
+constexpr int kAttnThreads = 256;
+constexpr int kAttnMaxParts = 4096;            // heads * splits
+constexpr int kAttnMaxHeads = 1024;
+constexpr int kAttnPartStride = 256 + 2;       // acc[hd <= 256], m, l
 
-// ROPE = true: q is the projection output [q | k | v]; the workgroup first rotates its head's q
-// and k (as rope_cache_kernel does), appends k and v to the caches at *pos and keeps q in LDS,
-// then attends.  Its own writes to the caches are ordered before its reads by the barrier.
+static __device__ __align__(256) float g_attn_part[kAttnMaxParts * kAttnPartStride];
+static __device__ __align__(256) uint32_t g_attn_arrived[kAttnMaxHeads];
+
 template <bool ROPE>
 __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(
     const uint16_t *__restrict__ q, uint16_t *k_cache, uint16_t *v_cache, const uint16_t *__restrict__ cos_t,
-    const uint16_t *__restrict__ sin_t, const int64_t *__restrict__ pos_p, uint16_t *__restrict__ out, int heads, int hd,
-    int max_len)
+    const uint16_t *__restrict__ sin_t, const int64_t *__restrict__ pos_p, uint16_t *__restrict__ out,
+    float *__restrict__ parts, uint32_t *__restrict__ arrived, int heads, int hd, int max_len, int splits,
+    int chunk_cap)
 {
     extern __shared__ float lds_f[];
-    float *scores = lds_f;                       // [max_len]
-    float *scratch = lds_f + max_len;            // [16]
-    float *acc = scratch + 16;                   // [groups][hd]
-    const int h = blockIdx.x, tid = threadIdx.x;
+    float *scores = lds_f;                       // [chunk_cap]
+    float *scratch = lds_f + chunk_cap;          // [16] (chunk_cap is a multiple of 16)
+    float *acc = scratch + 16;                   // [groups][hd] = 512 floats
+    uint16_t *q_rot = reinterpret_cast<uint16_t *>(acc + 512);   // [hd] halves, ROPE only
+    const int h = blockIdx.x / splits, sp = blockIdx.x - h * splits, tid = threadIdx.x;
     const int len = (int)*pos_p + 1;
+    // this workgroup's keys: [s_begin, s_end)
+    const int chunk = ((len + splits - 1) / splits + 15) & ~15;
+    const int s_begin = sp * chunk, s_end = min(len, s_begin + chunk), cnt = max(0, s_end - s_begin);
     uint16_t *kh = k_cache + (size_t)h * max_len * hd, *vh = v_cache + (size_t)h * max_len * hd;
     const float scale = rsqrtf((float)hd);
-    // [hd] halves behind acc, on a 16-byte boundary; ROPE only
-    uint16_t *q_rot = reinterpret_cast<uint16_t *>(lds_f + ((max_len + 16 + (kAttnThreads / (hd >> 1)) * hd + 3) & ~3));
     if (ROPE) {
         const int pos = len - 1, half = hd >> 1, d = heads * hd;
         if (tid < half) {
             const int i = tid, e = h * hd + 2 * i;
             const float c = half_bits_to_float(cos_t[pos * half + i]), s = half_bits_to_float(sin_t[pos * half + i]);
-            const float qa = half_bits_to_float(q[e]), qb = half_bits_to_float(q[e + 1]);
-            const float ka = half_bits_to_float(q[d + e]), kb = half_bits_to_float(q[d + e + 1]);
-            uint16_t *kd = kh + (size_t)pos * hd + 2 * i, *vd = vh + (size_t)pos * hd + 2 * i;
-            rope_pair(qa, qb, c, s, q_rot[2 * i], q_rot[2 * i + 1]);
-            rope_pair(ka, kb, c, s, kd[0], kd[1]);
-            vd[0] = q[2 * d + e];
-            vd[1] = q[2 * d + e + 1];
+            rope_pair(half_bits_to_float(q[e]), half_bits_to_float(q[e + 1]), c, s, q_rot[2 * i], q_rot[2 * i + 1]);
+            if (pos >= s_begin && pos < s_end) {
+                uint16_t *kd = kh + (size_t)pos * hd + 2 * i, *vd = vh + (size_t)pos * hd + 2 * i;
+                rope_pair(half_bits_to_float(q[d + e]), half_bits_to_float(q[d + e + 1]), c, s, kd[0], kd[1]);
+                vd[0] = q[2 * d + e];
+                vd[1] = q[2 * d + e + 1];
+            }
         }
         // the new cache row must have reached memory before other waves read it back
         __builtin_amdgcn_s_waitcnt(0);
@@ -149,13 +163,13 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(
             qf[2 * u + 1] = half_bits_to_float((uint16_t)(w[u] >> 16));
         }
     }
-    // four keys per thread in flight: the cache is far larger than L2, every load is an HBM round trip
-    for (int s0 = 0; s0 < len; s0 += 4 * slots) {
+    // four keys per thread in flight: the cache is far larger than L2, every load is a memory round trip
+    for (int s0 = 0; s0 < cnt; s0 += 4 * slots) {
         uint4 kv[4];
 #pragma unroll
         for (int u = 0; u < 4; u++) {
             const int s = s0 + u * slots + slot;
-            kv[u] = s < len ? *reinterpret_cast<const uint4 *>(kh + (size_t)s * hd + 8 * sub) : make_uint4(0, 0, 0, 0);
+            kv[u] = s < cnt ? *reinterpret_cast<const uint4 *>(kh + (size_t)(s_begin + s) * hd + 8 * sub) : make_uint4(0, 0, 0, 0);
         }
 #pragma unroll
         for (int u = 0; u < 4; u++) {
@@ -168,35 +182,35 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(
                 dot += half_bits_to_float((uint16_t)(w[c] >> 16)) * qf[2 * c + 1];
             }
             for (int off = lanes_per_key >> 1; off > 0; off >>= 1) dot += __shfl_xor(dot, off, 64);
-            if (s < len && sub == 0) scores[s] = dot * scale;
+            if (s < cnt && sub == 0) scores[s] = dot * scale;
         }
     }
     __syncthreads();
     float mx = -INFINITY;
-    for (int s = tid; s < len; s += kAttnThreads) mx = fmaxf(mx, scores[s]);
+    for (int s = tid; s < cnt; s += kAttnThreads) mx = fmaxf(mx, scores[s]);
     mx = block_max(mx, scratch);
     float sum = 0.f;
-    for (int s = tid; s < len; s += kAttnThreads) {
+    for (int s = tid; s < cnt; s += kAttnThreads) {
         const float p = __expf(scores[s] - mx);
         scores[s] = p;
         sum += p;
     }
-    const float inv = 1.f / block_sum(sum, scratch);     // (its barriers also publish the new scores)
+    sum = block_sum(sum, scratch);               // (its barriers also publish the new scores)
 
     // values
     const int pairs = hd >> 1, groups = kAttnThreads / pairs, grp = tid / pairs, dp = tid - grp * pairs;
     float a0 = 0.f, a1 = 0.f;
-    for (int s0 = grp; s0 < len; s0 += 8 * groups) {
+    for (int s0 = grp; s0 < cnt; s0 += 8 * groups) {
         uint32_t vv[8];
 #pragma unroll
         for (int u = 0; u < 8; u++) {
             const int s = s0 + u * groups;
-            vv[u] = s < len ? *reinterpret_cast<const uint32_t *>(vh + (size_t)s * hd + 2 * dp) : 0u;
+            vv[u] = s < cnt ? *reinterpret_cast<const uint32_t *>(vh + (size_t)(s_begin + s) * hd + 2 * dp) : 0u;
         }
 #pragma unroll
         for (int u = 0; u < 8; u++) {
             const int s = s0 + u * groups;
-            const float p = s < len ? scores[s] : 0.f;
+            const float p = s < cnt ? scores[s] : 0.f;
             a0 += p * half_bits_to_float((uint16_t)(vv[u] & 0xFFFFu));
             a1 += p * half_bits_to_float((uint16_t)(vv[u] >> 16));
         }
@@ -204,11 +218,60 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(
     acc[grp * hd + 2 * dp] = a0;
     acc[grp * hd + 2 * dp + 1] = a1;
     __syncthreads();
-    for (int i = tid; i < hd; i += kAttnThreads) {
-        float y = 0.f;
-        for (int gidx = 0; gidx < groups; gidx++) y += acc[gidx * hd + i];
-        out[h * hd + i] = float_to_half_bits(y * inv);
+    float y = 0.f;                               // thread i < hd: output dimension i of this piece
+    if (tid < hd)
+        for (int gidx = 0; gidx < groups; gidx++) y += acc[gidx * hd + tid];
+    if (splits == 1) {
+        if (tid < hd) out[h * hd + tid] = float_to_half_bits(y / sum);
+        return;
     }
+
+    // publish the piece, count the arrival, and let the last workgroup of the head merge
+    float *mine = parts + (size_t)blockIdx.x * kAttnPartStride;
+    if (tid < hd) __hip_atomic_store(&mine[tid], y, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (tid == 0) {
+        __hip_atomic_store(&mine[256], mx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(&mine[257], sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    // device-scope stores and loads bypass the XCD-private cache levels, so the only ordering needed
+    // is that this workgroup's stores have completed before its arrival is counted
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    uint32_t *flag = reinterpret_cast<uint32_t *>(scratch);
+    if (tid == 0) {
+        const uint32_t prev = __hip_atomic_fetch_add(&arrived[h], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const bool last = prev == (uint32_t)(splits - 1);
+        if (last) __hip_atomic_store(&arrived[h], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // for the next launch
+        *flag = last;
+    }
+    __syncthreads();
+    if (!*flag || tid >= hd) return;
+    const float *head_parts = parts + (size_t)h * splits * kAttnPartStride;
+    constexpr int kMaxSplits = 16;
+    float pm[kMaxSplits], pl[kMaxSplits], pa[kMaxSplits];
+#pragma unroll
+    for (int i = 0; i < kMaxSplits; i++) {
+        pm[i] = -INFINITY;
+        pl[i] = pa[i] = 0.f;
+        if (i < splits) {
+            const float *pp = head_parts + (size_t)i * kAttnPartStride;
+            pm[i] = __hip_atomic_load(&pp[256], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            pl[i] = __hip_atomic_load(&pp[257], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            pa[i] = __hip_atomic_load(&pp[tid], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+    float M = pm[0];                             // piece 0 is never empty
+#pragma unroll
+    for (int i = 1; i < kMaxSplits; i++) M = fmaxf(M, pm[i]);
+    float num = 0.f, den = 0.f;
+#pragma unroll
+    for (int i = 0; i < kMaxSplits; i++) {
+        const float w = __expf(pm[i] - M);       // an empty piece has m = -inf, so w = 0
+        num += pa[i] * w;
+        den += pl[i] * w;
+    }
+    out[h * hd + tid] = float_to_half_bits(num / den);
 }
 
 // gu = [gate | up], each f:  out = silu(gate) * up
@@ -247,18 +310,55 @@ extern "C" int rptc_rope_cache(const uint16_t *qkv, const uint16_t *cos_t, const
     return (int)hipGetLastError();
 }
 
+namespace rptc {
+struct AttnScratch {
+    float *parts;
+    uint32_t *arrived;
+};
+static AttnScratch g_attn[64];   // per device: addresses of the static scratch arrays
+
+int prepare_decode_glue(int device)
+{
+    // the device addresses of the static scratch arrays (the symbols themselves are not device addresses)
+    int rc = (int)hipGetSymbolAddress(reinterpret_cast<void **>(&g_attn[device].parts), HIP_SYMBOL(g_attn_part));
+    if (rc) return rc;
+    return (int)hipGetSymbolAddress(reinterpret_cast<void **>(&g_attn[device].arrived), HIP_SYMBOL(g_attn_arrived));
+}
+
+template <bool ROPE>
+static int launch_attn(const uint16_t *q, const uint16_t *cos_t, const uint16_t *sin_t, const int64_t *pos, uint16_t *k_cache,
+                       uint16_t *v_cache, uint16_t *out, int64_t heads, int64_t hd, int64_t max_len, void *stream)
+{
+    // hd a power of two in [16, 256]: 16 bytes per lane, whole keys per wave, whole groups per workgroup
+    if (heads < 1 || hd < 16 || hd > 256 || (hd & (hd - 1)) != 0 || max_len < 1) return RPTC_ESHAPE;
+    if (heads > kAttnMaxHeads || max_len > (1 << 20)) return RPTC_ELIMIT;
+    DeviceInfo *dev;
+    int rc = device_info(&dev);
+    if (rc) return rc;
+    // pieces per head: enough workgroups for every CU, at most 16, none shorter than 16 keys of max_len
+    int splits = (int)(dev->cus / heads);
+    if (splits > 16) splits = 16;
+    if (splits > max_len / 16) splits = (int)(max_len / 16);
+    if (splits < 1) splits = 1;
+    if (heads * splits > kAttnMaxParts) splits = (int)(kAttnMaxParts / heads);
+    const int chunk_cap = (int)(((max_len + splits - 1) / splits + 15) & ~(int64_t)15);
+    const size_t lds = (size_t)(chunk_cap + 16 + 512) * 4 + (size_t)hd * 2;
+    if (lds > 64 * 1024) return RPTC_ELIMIT;
+    const AttnScratch &sc = g_attn[dev->device];
+    hipLaunchKernelGGL(attn_decode_kernel<ROPE>, dim3((unsigned)(heads * splits)), dim3(kAttnThreads), lds,
+                       static_cast<hipStream_t>(stream), q, k_cache, v_cache, cos_t, sin_t, pos, out, sc.parts, sc.arrived,
+                       (int)heads, (int)hd, (int)max_len, splits, chunk_cap);
+    return (int)hipGetLastError();
+}
+}  // namespace rptc
+
 extern "C" int rptc_attn_decode(const uint16_t *q, const uint16_t *k_cache, const uint16_t *v_cache, const int64_t *pos,
                                 uint16_t *out, int64_t heads, int64_t hd, int64_t max_len, void *stream)
 {
     if (!q || !k_cache || !v_cache || !pos || !out) return RPTC_ENULL;
-    // hd a power of two in [16, 256]: 16 bytes per lane, whole keys per wave, whole groups per workgroup
-    if (heads < 1 || hd < 16 || hd > 256 || (hd & (hd - 1)) != 0 || max_len < 1) return RPTC_ESHAPE;
-    const size_t lds = (size_t)(max_len + 16 + (kAttnThreads / (hd / 2)) * hd) * 4;
-    if (lds > 64 * 1024) return RPTC_ELIMIT;
-    hipLaunchKernelGGL(attn_decode_kernel<false>, dim3((unsigned)heads), dim3(kAttnThreads), lds,
-                       static_cast<hipStream_t>(stream), q, const_cast<uint16_t *>(k_cache), const_cast<uint16_t *>(v_cache),
-                       nullptr, nullptr, pos, out, (int)heads, (int)hd, (int)max_len);
-    return (int)hipGetLastError();
+    if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache)) return RPTC_EALIGN;
+    return launch_attn<false>(q, nullptr, nullptr, pos, const_cast<uint16_t *>(k_cache), const_cast<uint16_t *>(v_cache), out,
+                              heads, hd, max_len, stream);
 }
 
 extern "C" int rptc_rope_attn_decode(const uint16_t *qkv, const uint16_t *cos_t, const uint16_t *sin_t, const int64_t *pos,
@@ -266,14 +366,8 @@ extern "C" int rptc_rope_attn_decode(const uint16_t *qkv, const uint16_t *cos_t,
                                      int64_t max_len, void *stream)
 {
     if (!qkv || !cos_t || !sin_t || !pos || !k_cache || !v_cache || !out) return RPTC_ENULL;
-    if (heads < 1 || hd < 16 || hd > 256 || (hd & (hd - 1)) != 0 || max_len < 1) return RPTC_ESHAPE;
     if (!aligned16(qkv) || !aligned16(k_cache) || !aligned16(v_cache)) return RPTC_EALIGN;
-    const size_t lds = (size_t)(max_len + 16 + (kAttnThreads / (hd / 2)) * hd + 4) * 4 + (size_t)hd * 2;
-    if (lds > 64 * 1024) return RPTC_ELIMIT;
-    hipLaunchKernelGGL(attn_decode_kernel<true>, dim3((unsigned)heads), dim3(kAttnThreads), lds,
-                       static_cast<hipStream_t>(stream), qkv, k_cache, v_cache, cos_t, sin_t, pos, out, (int)heads, (int)hd,
-                       (int)max_len);
-    return (int)hipGetLastError();
+    return launch_attn<true>(qkv, cos_t, sin_t, pos, k_cache, v_cache, out, heads, hd, max_len, stream);
 }
 
 extern "C" int rptc_silu_mul(const uint16_t *gate_up, uint16_t *out, int64_t f, void *stream)
