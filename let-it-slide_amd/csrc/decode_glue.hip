@@ -7,6 +7,11 @@
 // HIP graph can be replayed for successive tokens.
 #include "rptc_common.hpp"
 
+// Development hook: a probe build defines RPTC_ATTN_STAMP to record a per-workgroup timestamp at each phase.
+#ifndef RPTC_ATTN_STAMP
+#define RPTC_ATTN_STAMP(slot) ((void)0)
+#endif
+
 namespace rptc {
 
 __device__ __forceinline__ float block_sum(float v, float *scratch)
@@ -99,11 +104,11 @@ __global__ __launch_bounds__(256) void rope_cache_kernel(const uint16_t *__restr
 // the workgroup that arrives last at the head's counter merges the pieces in piece order:
 // out = sum_i acc_i * exp(m_i - M) / sum_i l_i * exp(m_i - M).  Every sum has a fixed order.
 // Scores: hd/8 lanes share a key (16 bytes of it each) and add their partial dot products with
-// shuffles.  Values: a thread owns one pair of output dimensions, the keys are cut into
-// 256 / (hd/2) interleaved groups whose sums are added in a fixed order.
+// shuffles.  Values: the same lanes read 16 bytes of a value row each and keep 8 output
+// dimensions; the 256 / (hd/8) interleaved key groups are added in a fixed order.
 // ROPE = true: q is the projection output [q | k | v]; every workgroup rotates its head's q into
 // LDS, and the one whose piece holds *pos also rotates k and appends k and v to the caches (as
-// rope_cache_kernel does) before it reads that row back.
+// rope_cache_kernel does); it uses the new row from LDS.
 constexpr int kAttnThreads = 256;
 constexpr int kAttnMaxParts = 4096;            // heads * splits
 constexpr int kAttnMaxHeads = 1024;
@@ -120,10 +125,11 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(
     int chunk_cap)
 {
     extern __shared__ float lds_f[];
+    RPTC_ATTN_STAMP(0);
     float *scores = lds_f;                       // [chunk_cap]
     float *scratch = lds_f + chunk_cap;          // [16] (chunk_cap is a multiple of 16)
-    float *acc = scratch + 16;                   // [groups][hd] = 512 floats
-    uint16_t *q_rot = reinterpret_cast<uint16_t *>(acc + 512);   // [hd] halves, ROPE only
+    float *acc = scratch + 16;                   // [slots][hd] = 2048 floats
+    uint16_t *q_rot = reinterpret_cast<uint16_t *>(acc + 2048);   // [3][hd] halves (q, new k, new v), ROPE only
     const int h = blockIdx.x / splits, sp = blockIdx.x - h * splits, tid = threadIdx.x;
     const int len = (int)*pos_p + 1;
     // this workgroup's keys: [s_begin, s_end)
@@ -131,27 +137,71 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(
     const int s_begin = sp * chunk, s_end = min(len, s_begin + chunk), cnt = max(0, s_end - s_begin);
     uint16_t *kh = k_cache + (size_t)h * max_len * hd, *vh = v_cache + (size_t)h * max_len * hd;
     const float scale = rsqrtf((float)hd);
-    if (ROPE) {
-        const int pos = len - 1, half = hd >> 1, d = heads * hd;
-        if (tid < half) {
-            const int i = tid, e = h * hd + 2 * i;
-            const float c = half_bits_to_float(cos_t[pos * half + i]), s = half_bits_to_float(sin_t[pos * half + i]);
-            rope_pair(half_bits_to_float(q[e]), half_bits_to_float(q[e + 1]), c, s, q_rot[2 * i], q_rot[2 * i + 1]);
-            if (pos >= s_begin && pos < s_end) {
-                uint16_t *kd = kh + (size_t)pos * hd + 2 * i, *vd = vh + (size_t)pos * hd + 2 * i;
-                rope_pair(half_bits_to_float(q[d + e]), half_bits_to_float(q[d + e + 1]), c, s, kd[0], kd[1]);
-                vd[0] = q[2 * d + e];
-                vd[1] = q[2 * d + e + 1];
-            }
-        }
-        // the new cache row must have reached memory before other waves read it back
-        __builtin_amdgcn_s_waitcnt(0);
-        __syncthreads();
-    }
+    const int pos = len - 1;
+    const bool owns_pos = ROPE && pos >= s_begin && pos < s_end;     // this piece holds the new row
 
-    // scores
+    // Every load the piece needs is requested before anything is used: up to kKeysInFlight keys and
+    // kValuesInFlight values per thread (the cache is far larger than L2: each load is a memory round
+    // trip, and the values do not depend on the scores).  Longer pieces take further rounds.
     const int lanes_per_key = hd >> 3;           // 16 bytes = 8 values per lane
     const int sub = tid % lanes_per_key, slot = tid / lanes_per_key, slots = kAttnThreads / lanes_per_key;
+    constexpr int kKeysInFlight = 8;
+    uint4 kv[kKeysInFlight], vv[kKeysInFlight];
+    auto load_keys = [&](int s0) {
+#pragma unroll
+        for (int u = 0; u < kKeysInFlight; u++) {
+            const int s = s0 + u * slots + slot;
+            kv[u] = s < cnt ? *reinterpret_cast<const uint4 *>(kh + (size_t)(s_begin + s) * hd + 8 * sub) : make_uint4(0, 0, 0, 0);
+        }
+    };
+    auto load_values = [&](int s0) {                  // same shape as the keys: 16 bytes of a row per lane
+#pragma unroll
+        for (int u = 0; u < kKeysInFlight; u++) {
+            const int s = s0 + u * slots + slot;
+            vv[u] = s < cnt ? *reinterpret_cast<const uint4 *>(vh + (size_t)(s_begin + s) * hd + 8 * sub) : make_uint4(0, 0, 0, 0);
+        }
+    };
+    uint16_t *k_new = q_rot + hd, *v_new = k_new + hd;            // the new row, ROPE only
+    if (ROPE) {
+        const int half = hd >> 1, d = heads * hd;
+        float qa = 0.f, qb = 0.f, ka = 0.f, kb = 0.f, c = 0.f, sn = 0.f;
+        uint16_t va = 0, vb = 0;
+        const int e = h * hd + 2 * tid;
+        if (tid < half) {
+            c = half_bits_to_float(cos_t[pos * half + tid]);
+            sn = half_bits_to_float(sin_t[pos * half + tid]);
+            qa = half_bits_to_float(q[e]);
+            qb = half_bits_to_float(q[e + 1]);
+            ka = half_bits_to_float(q[d + e]);
+            kb = half_bits_to_float(q[d + e + 1]);
+            va = q[2 * d + e];
+            vb = q[2 * d + e + 1];
+        }
+        load_keys(0);
+        load_values(0);
+        if (tid < half) {
+            rope_pair(qa, qb, c, sn, q_rot[2 * tid], q_rot[2 * tid + 1]);
+            if (owns_pos) {
+                // the row goes to the caches for later tokens; this launch takes it from LDS, because
+                // the loads above may have fetched the row before it was written
+                rope_pair(ka, kb, c, sn, k_new[2 * tid], k_new[2 * tid + 1]);
+                v_new[2 * tid] = va;
+                v_new[2 * tid + 1] = vb;
+                uint16_t *kd = kh + (size_t)pos * hd + 2 * tid, *vd = vh + (size_t)pos * hd + 2 * tid;
+                kd[0] = k_new[2 * tid];
+                kd[1] = k_new[2 * tid + 1];
+                vd[0] = va;
+                vd[1] = vb;
+            }
+        }
+        __syncthreads();
+    } else {
+        load_keys(0);
+        load_values(0);
+    }
+
+    RPTC_ATTN_STAMP(1);
+    // scores
     float qf[8];
     {
         const uint4 v = ROPE ? *reinterpret_cast<const uint4 *>(q_rot + 8 * sub)
@@ -163,18 +213,14 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(
             qf[2 * u + 1] = half_bits_to_float((uint16_t)(w[u] >> 16));
         }
     }
-    // four keys per thread in flight: the cache is far larger than L2, every load is a memory round trip
-    for (int s0 = 0; s0 < cnt; s0 += 4 * slots) {
-        uint4 kv[4];
+    for (int s0 = 0; s0 < cnt; s0 += kKeysInFlight * slots) {
+        if (s0 > 0) load_keys(s0);
 #pragma unroll
-        for (int u = 0; u < 4; u++) {
+        for (int u = 0; u < kKeysInFlight; u++) {
             const int s = s0 + u * slots + slot;
-            kv[u] = s < cnt ? *reinterpret_cast<const uint4 *>(kh + (size_t)(s_begin + s) * hd + 8 * sub) : make_uint4(0, 0, 0, 0);
-        }
-#pragma unroll
-        for (int u = 0; u < 4; u++) {
-            const int s = s0 + u * slots + slot;
-            const uint32_t w[4] = {kv[u].x, kv[u].y, kv[u].z, kv[u].w};
+            uint4 kq = kv[u];
+            if (owns_pos && s_begin + s == pos) kq = *reinterpret_cast<const uint4 *>(k_new + 8 * sub);
+            const uint32_t w[4] = {kq.x, kq.y, kq.z, kq.w};
             float dot = 0.f;
 #pragma unroll
             for (int c = 0; c < 4; c++) {
@@ -186,6 +232,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(
         }
     }
     __syncthreads();
+    RPTC_ATTN_STAMP(2);
     float mx = -INFINITY;
     for (int s = tid; s < cnt; s += kAttnThreads) mx = fmaxf(mx, scores[s]);
     mx = block_max(mx, scratch);
@@ -197,30 +244,33 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(
     }
     sum = block_sum(sum, scratch);               // (its barriers also publish the new scores)
 
-    // values
-    const int pairs = hd >> 1, groups = kAttnThreads / pairs, grp = tid / pairs, dp = tid - grp * pairs;
-    float a0 = 0.f, a1 = 0.f;
-    for (int s0 = grp; s0 < cnt; s0 += 8 * groups) {
-        uint32_t vv[8];
+    // values: thread (slot, sub) adds its keys' rows, 8 output dimensions each
+    float a8[8];
 #pragma unroll
-        for (int u = 0; u < 8; u++) {
-            const int s = s0 + u * groups;
-            vv[u] = s < cnt ? *reinterpret_cast<const uint32_t *>(vh + (size_t)(s_begin + s) * hd + 2 * dp) : 0u;
-        }
+    for (int c = 0; c < 8; c++) a8[c] = 0.f;
+    for (int s0 = 0; s0 < cnt; s0 += kKeysInFlight * slots) {
+        if (s0 > 0) load_values(s0);
 #pragma unroll
-        for (int u = 0; u < 8; u++) {
-            const int s = s0 + u * groups;
+        for (int u = 0; u < kKeysInFlight; u++) {
+            const int s = s0 + u * slots + slot;
+            uint4 vq = vv[u];
+            if (owns_pos && s_begin + s == pos) vq = *reinterpret_cast<const uint4 *>(v_new + 8 * sub);
             const float p = s < cnt ? scores[s] : 0.f;
-            a0 += p * half_bits_to_float((uint16_t)(vv[u] & 0xFFFFu));
-            a1 += p * half_bits_to_float((uint16_t)(vv[u] >> 16));
+            const uint32_t w[4] = {vq.x, vq.y, vq.z, vq.w};
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                a8[2 * c] += p * half_bits_to_float((uint16_t)(w[c] & 0xFFFFu));
+                a8[2 * c + 1] += p * half_bits_to_float((uint16_t)(w[c] >> 16));
+            }
         }
     }
-    acc[grp * hd + 2 * dp] = a0;
-    acc[grp * hd + 2 * dp + 1] = a1;
+    RPTC_ATTN_STAMP(3);
+#pragma unroll
+    for (int c = 0; c < 8; c++) acc[slot * hd + 8 * sub + c] = a8[c];
     __syncthreads();
     float y = 0.f;                               // thread i < hd: output dimension i of this piece
     if (tid < hd)
-        for (int gidx = 0; gidx < groups; gidx++) y += acc[gidx * hd + tid];
+        for (int gidx = 0; gidx < slots; gidx++) y += acc[gidx * hd + tid];
     if (splits == 1) {
         if (tid < hd) out[h * hd + tid] = float_to_half_bits(y / sum);
         return;
@@ -237,6 +287,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(
     // is that this workgroup's stores have completed before its arrival is counted
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __builtin_amdgcn_s_waitcnt(0);
+    RPTC_ATTN_STAMP(4);
     __syncthreads();
     uint32_t *flag = reinterpret_cast<uint32_t *>(scratch);
     if (tid == 0) {
@@ -246,6 +297,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(
         *flag = last;
     }
     __syncthreads();
+    RPTC_ATTN_STAMP(5);
     if (!*flag || tid >= hd) return;
     const float *head_parts = parts + (size_t)h * splits * kAttnPartStride;
     constexpr int kMaxSplits = 16;
@@ -272,6 +324,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(
         den += pl[i] * w;
     }
     out[h * hd + tid] = float_to_half_bits(num / den);
+    RPTC_ATTN_STAMP(6);
 }
 
 // gu = [gate | up], each f:  out = silu(gate) * up
@@ -279,9 +332,7 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const uint16_t *__restric
 {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= f) return;
-    const float g = half_bits_to_float(gu[i]), u = half_bits_to_float(gu[f + i]);
-    const float sg = half_bits_to_float(float_to_half_bits(g / (1.f + __expf(-g))));
-    out[i] = float_to_half_bits(sg * u);
+    out[i] = silu_mul_bits(gu[i], gu[f + i]);
 }
 
 }  // namespace rptc
@@ -342,7 +393,7 @@ static int launch_attn(const uint16_t *q, const uint16_t *cos_t, const uint16_t 
     if (splits < 1) splits = 1;
     if (heads * splits > kAttnMaxParts) splits = (int)(kAttnMaxParts / heads);
     const int chunk_cap = (int)(((max_len + splits - 1) / splits + 15) & ~(int64_t)15);
-    const size_t lds = (size_t)(chunk_cap + 16 + 512) * 4 + (size_t)hd * 2;
+    const size_t lds = (size_t)(chunk_cap + 16 + 2048) * 4 + (size_t)hd * 6;
     if (lds > 64 * 1024) return RPTC_ELIMIT;
     const AttnScratch &sc = g_attn[dev->device];
     hipLaunchKernelGGL(attn_decode_kernel<ROPE>, dim3((unsigned)(heads * splits)), dim3(kAttnThreads), lds,

@@ -194,11 +194,13 @@ __device__ __forceinline__ float round_half(float v) { return half_bits_to_float
 
 __device__ __forceinline__ uint4 silu_mul8(const uint4 gate, const uint4 up)
 {
-    const Halves8 g = unpack8(gate), u = unpack8(up);
-    Halves8 r;
+    const uint32_t g[4] = {gate.x, gate.y, gate.z, gate.w}, u[4] = {up.x, up.y, up.z, up.w};
+    uint32_t r[4];
 #pragma unroll
-    for (int i = 0; i < 8; i++) r.v[i] = round_half(g.v[i] / (1.f + __expf(-g.v[i]))) * u.v[i];
-    return pack8(r);
+    for (int i = 0; i < 4; i++)
+        r[i] = (uint32_t)silu_mul_bits((uint16_t)(g[i] & 0xFFFFu), (uint16_t)(u[i] & 0xFFFFu)) |
+               ((uint32_t)silu_mul_bits((uint16_t)(g[i] >> 16), (uint16_t)(u[i] >> 16)) << 16);
+    return make_uint4(r[0], r[1], r[2], r[3]);
 }
 
 template <int S, int MODE, int BITS, int XMODE>

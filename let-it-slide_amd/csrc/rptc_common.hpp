@@ -126,6 +126,19 @@ __device__ __forceinline__ float half_bits_to_float(uint16_t b)
 {
     return (float)__builtin_bit_cast(_Float16, b);
 }
+
+// silu(gate) * up on fp16 values: silu in fp32 through the hardware exp2 and reciprocal, rounded to
+// fp16, then an fp16 product.  One definition (no contraction) so that every kernel that computes
+// the gate rounds the same way.
+__device__ __forceinline__ uint16_t silu_mul_bits(uint16_t gate, uint16_t up)
+{
+#pragma clang fp contract(off)
+    const float g = half_bits_to_float(gate);
+    const float e = __builtin_amdgcn_exp2f(g * -1.44269504088896f);
+    const _Float16 sg = (_Float16)(g * __builtin_amdgcn_rcpf(1.f + e));
+    const _Float16 r = sg * __builtin_bit_cast(_Float16, up);
+    return __builtin_bit_cast(uint16_t, r);
+}
 #endif
 
 }  // namespace rptc
