@@ -203,7 +203,8 @@ __device__ __forceinline__ uint4 silu_mul8(const uint4 gate, const uint4 up)
     return make_uint4(r[0], r[1], r[2], r[3]);
 }
 
-template <int S, int MODE, int BITS, int XMODE>
+// COMPACT: partial sums per (row, full slab) and (row, ragged lane) instead of per (row, stream element)
+template <int S, int MODE, int BITS, int XMODE, bool COMPACT>
 __device__ __forceinline__ void matvec_body(
     const uint32_t *__restrict__ comp, const uint32_t *__restrict__ codebook,
     const uint4 *__restrict__ x, uint16_t *__restrict__ out, const MatvecArgs a, const XFuse fuse)
@@ -215,7 +216,11 @@ __device__ __forceinline__ void matvec_body(
     const int m = a.m, n = a.n;
     const int T = n >> 11, Lt = (n & 2047) >> 6, npr = n >> 6, n8 = n >> 3;
     uint32_t *sx = lds + kTableBytes / 4;                  // activation pairs, slot order
-    float *part = reinterpret_cast<float *>(sx + (n >> 1));   // [row in block][n / 64]
+    // Partial sums: [row in block][n / 64], one per stream element of the row.  A long row (large n)
+    // would not leave room for a CU's share of rows, so in compact mode the 32 lanes of a full slab
+    // are added with DPP first: [row][T full slabs + Lt ragged lanes].
+    float *part = reinterpret_cast<float *>(sx + (n >> 1));
+    const int pstride = COMPACT ? T + Lt : npr;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: keeps control flow scalar
@@ -237,15 +242,24 @@ __device__ __forceinline__ void matvec_body(
     }
     constexpr int kXRegs = 2;
     uint4 xv[kXRegs], xv2[kXRegs], xvw[kXRegs];
-    const uint4 zero4 = make_uint4(0, 0, 0, 0);
 #pragma unroll
     for (int u = 0; u < kXRegs; u++) {
         const int idx = tid + u * kMatvecThreads;
-        xv[u] = idx < n8 ? x[idx] : zero4;
-        if constexpr (XMODE == kXSiluMul) xv2[u] = idx < n8 ? x[n8 + idx] : zero4;
-        if constexpr (XMODE == kXAddRmsNorm) {
-            xv2[u] = (idx < n8 && fuse.x2) ? fuse.x2[idx] : zero4;
-            xvw[u] = idx < n8 ? fuse.norm_w[idx] : zero4;
+        xv[u] = idx < n8 ? x[idx] : make_uint4(0, 0, 0, 0);
+    }
+    if constexpr (XMODE == kXSiluMul) {
+#pragma unroll
+        for (int u = 0; u < kXRegs; u++) {
+            const int idx = tid + u * kMatvecThreads;
+            xv2[u] = idx < n8 ? x[n8 + idx] : make_uint4(0, 0, 0, 0);
+        }
+    }
+    if constexpr (XMODE == kXAddRmsNorm) {
+#pragma unroll
+        for (int u = 0; u < kXRegs; u++) {
+            const int idx = tid + u * kMatvecThreads;
+            xv2[u] = (idx < n8 && fuse.x2) ? fuse.x2[idx] : make_uint4(0, 0, 0, 0);
+            xvw[u] = idx < n8 ? fuse.norm_w[idx] : make_uint4(0, 0, 0, 0);
         }
     }
 
@@ -406,8 +420,8 @@ __device__ __forceinline__ void matvec_body(
 #pragma unroll
                     for (int q = 0; q < 32; q++) xr[q] = xp[q * sv.lanes];
                 }
-                part_lane = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(part)) +
-                            4u * (uint32_t)(sub * npr + sv.part_off + l);
+                const int col = COMPACT ? (slab < T ? slab : T + l) : sv.part_off + l;
+                part_lane = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(part)) + 4u * (uint32_t)(sub * pstride + col);
             }
             const int row_first = idx * sv.rows_per_item;
             const bool active = sub < sv.rows_per_item && row_first + sub < rows;
@@ -425,9 +439,14 @@ __device__ __forceinline__ void matvec_body(
             } else {
                 sum = decode_element_bits<BITS>(cur[u], carry, lane4, xr);
             }
-            if (active) {
+            bool writer = active;
+            if (COMPACT && slab < T) {
+                sum = half_wave_sum(sum);        // lanes 31 and 63 hold their row's 32 elements
+                writer = active && l == 31;
+            }
+            if (writer) {
                 typedef __attribute__((address_space(3))) float lds_float;
-                *reinterpret_cast<lds_float *>(static_cast<uintptr_t>(part_lane + 4u * (uint32_t)(row_first * npr))) = sum;
+                *reinterpret_cast<lds_float *>(static_cast<uintptr_t>(part_lane + 4u * (uint32_t)(row_first * pstride))) = sum;
             }
             if (base + u == it_begin) RPTC_STAMP(3);
             if (++idx == sv.items) {
@@ -439,17 +458,17 @@ __device__ __forceinline__ void matvec_body(
     }
     RPTC_STAMP(4);
     __syncthreads();
-    // one wave per row: add the row's n / 64 partial sums in a fixed order
+    // one wave per row: add the row's partial sums in a fixed order
     for (int r = wave; r < rows; r += kMatvecWaves) {
         float y = 0.f;
-        for (int i = lane; i < npr; i += kWave) y += part[r * npr + i];
+        for (int i = lane; i < pstride; i += kWave) y += part[r * pstride + i];
         y = wave_sum(y);
         if (lane == 63) out[row0 + r] = float_to_half_bits(y);
     }
     RPTC_STAMP(5);
 }
 
-template <int S, int MODE, int BITS>
+template <int S, int MODE, int BITS, bool COMPACT>
 __global__ __launch_bounds__(kMatvecThreads) void matvec_kernel(
     const uint32_t *__restrict__ comp, const uint32_t *__restrict__ codebook,
     const uint4 *__restrict__ x, uint16_t *__restrict__ out, int arg_m, int arg_n, int arg_rows_per_block,
@@ -457,11 +476,11 @@ __global__ __launch_bounds__(kMatvecThreads) void matvec_kernel(
 {
     // separate scalar arguments (not a struct) so that all of them are preloaded into SGPRs
     const MatvecArgs a = {arg_m, arg_n, arg_rows_per_block, arg_rw_tail, arg_items_full, arg_items_tail};
-    matvec_body<S, MODE, BITS, kXPlain>(comp, codebook, x, out, a, XFuse{nullptr, nullptr, nullptr, 0.f});
+    matvec_body<S, MODE, BITS, kXPlain, COMPACT>(comp, codebook, x, out, a, XFuse{nullptr, nullptr, nullptr, 0.f});
 }
 
 // 2 bits per weight with an element-wise step fused in front (XMODE above)
-template <int S, int MODE, int XMODE>
+template <int S, int MODE, int XMODE, bool COMPACT>
 __global__ __launch_bounds__(kMatvecThreads) void matvec_fused_kernel(
     const uint32_t *__restrict__ comp, const uint32_t *__restrict__ codebook,
     const uint4 *__restrict__ x, uint16_t *__restrict__ out, int arg_m, int arg_n, int arg_rows_per_block,
@@ -469,7 +488,7 @@ __global__ __launch_bounds__(kMatvecThreads) void matvec_fused_kernel(
     float eps)
 {
     const MatvecArgs a = {arg_m, arg_n, arg_rows_per_block, arg_rw_tail, arg_items_full, arg_items_tail};
-    matvec_body<S, MODE, 2, XMODE>(comp, codebook, x, out, a, XFuse{x2, norm_w, x_out, eps});
+    matvec_body<S, MODE, 2, XMODE, COMPACT>(comp, codebook, x, out, a, XFuse{x2, norm_w, x_out, eps});
 }
 
 // Dense export: one thread per stream element, 32 pairs scattered to their columns.
@@ -508,14 +527,20 @@ __global__ __launch_bounds__(256) void matvec_dense_kernel(
     }
 }
 
-static int matvec_lds_bytes(int n, int rows_per_block)
+static int matvec_part_stride(int n, bool compact)
 {
-    return kTableBytes + 2 * n + 4 * (n / 64) * rows_per_block;
+    return compact ? (n >> 11) + ((n & 2047) >> 6) : n / 64;
+}
+
+static int matvec_lds_bytes(int n, int rows_per_block, bool compact)
+{
+    return kTableBytes + 2 * n + 4 * matvec_part_stride(n, compact) * rows_per_block;
 }
 
 // Argument checks and launch geometry shared by every mat-vec entry point.
 static int plan_matvec(const void *compressed, const void *codebook, const void *x, const void *out, int64_t m,
-                       int64_t n, int carry_mode, DeviceInfo **dev, MatvecArgs *a, int *lds_bytes, int *grid)
+                       int64_t n, int carry_mode, bool allow_compact, DeviceInfo **dev, MatvecArgs *a, bool *compact,
+                       int *lds_bytes, int *grid)
 {
     if (!compressed || !codebook || !x || !out) return RPTC_ENULL;
     if (m < 1 || n < 64 || n % 64 != 0) return RPTC_ESHAPE;
@@ -524,13 +549,15 @@ static int plan_matvec(const void *compressed, const void *codebook, const void 
     if (m >= (1 << 24) || n >= (1 << 20) || m * n >= ((int64_t)1 << 36)) return RPTC_ELIMIT;
     int rc = device_info(dev);
     if (rc) return rc;
-    // one workgroup per CU when the per-row partial sums fit in LDS beside the table and the
-    // activations, else as many rows per workgroup as do fit
+    // one workgroup per CU; when a CU's share of rows with one partial sum per stream element does
+    // not fit in LDS beside the table and the activations, the compact partial layout is used where
+    // the kernel has one, and if nothing fits, as many rows per workgroup as do
     a->m = (int)m;
     a->n = (int)n;
     a->rows_per_block = 2 * (int)((m + 2 * (*dev)->cus - 1) / (2 * (*dev)->cus));
-    const int fixed_bytes = matvec_lds_bytes(a->n, 0);
-    const int row_bytes = 4 * (a->n / 64);
+    *compact = allow_compact && matvec_lds_bytes(a->n, a->rows_per_block, false) > kMaxLds;
+    const int fixed_bytes = matvec_lds_bytes(a->n, 0, *compact);
+    const int row_bytes = 4 * matvec_part_stride(a->n, *compact);
     if (fixed_bytes + 2 * row_bytes > kMaxLds) return RPTC_ELIMIT;
     const int fit_rows = ((kMaxLds - fixed_bytes) / row_bytes) & ~1;
     if (a->rows_per_block > fit_rows) a->rows_per_block = fit_rows;
@@ -538,7 +565,7 @@ static int plan_matvec(const void *compressed, const void *codebook, const void 
     a->rw_tail = lt ? 64 / lt : 1;
     a->items_full = a->rows_per_block / 2;
     a->items_tail = lt ? (a->rows_per_block + a->rw_tail - 1) / a->rw_tail : 0;
-    *lds_bytes = matvec_lds_bytes(a->n, a->rows_per_block);
+    *lds_bytes = matvec_lds_bytes(a->n, a->rows_per_block, *compact);
     *grid = (int)((m + a->rows_per_block - 1) / a->rows_per_block);
     return 0;
 }
@@ -550,7 +577,8 @@ static int launch_matvec(const int32_t *compressed, const uint16_t *codebook, co
     DeviceInfo *dev;
     MatvecArgs a;
     int lds_bytes, grid;
-    int rc = plan_matvec(compressed, codebook, x, out, m, n, carry_mode, &dev, &a, &lds_bytes, &grid);
+    bool compact;
+    int rc = plan_matvec(compressed, codebook, x, out, m, n, carry_mode, BITS == 2, &dev, &a, &compact, &lds_bytes, &grid);
     if (rc) return rc;
     hipStream_t s = static_cast<hipStream_t>(stream);
     Timer t;
@@ -559,12 +587,19 @@ static int launch_matvec(const int32_t *compressed, const uint16_t *codebook, co
     auto a_comp = reinterpret_cast<const uint32_t *>(compressed);
     auto a_cb = reinterpret_cast<const uint32_t *>(codebook);
     auto a_x = reinterpret_cast<const uint4 *>(x);
-    if (carry_mode == RPTC_AS_WRITTEN)
-        hipLaunchKernelGGL((matvec_kernel<S, RPTC_AS_WRITTEN, BITS>), dim3(grid), dim3(kMatvecThreads), lds_bytes, s,
-                           a_comp, a_cb, a_x, out, a.m, a.n, a.rows_per_block, a.rw_tail, a.items_full, a.items_tail);
-    else
-        hipLaunchKernelGGL((matvec_kernel<S, RPTC_CONTINUOUS, BITS>), dim3(grid), dim3(kMatvecThreads), lds_bytes, s,
-                           a_comp, a_cb, a_x, out, a.m, a.n, a.rows_per_block, a.rw_tail, a.items_full, a.items_tail);
+#define RPTC_LAUNCH(MODE, COMPACT)                                                                              \
+    hipLaunchKernelGGL((matvec_kernel<S, MODE, BITS, COMPACT>), dim3(grid), dim3(kMatvecThreads), lds_bytes, s, \
+                       a_comp, a_cb, a_x, out, a.m, a.n, a.rows_per_block, a.rw_tail, a.items_full, a.items_tail)
+    if constexpr (BITS == 2) {
+        if (compact) {
+            if (carry_mode == RPTC_AS_WRITTEN) RPTC_LAUNCH(RPTC_AS_WRITTEN, true);
+            else RPTC_LAUNCH(RPTC_CONTINUOUS, true);
+            return t.end();
+        }
+    }
+    if (carry_mode == RPTC_AS_WRITTEN) RPTC_LAUNCH(RPTC_AS_WRITTEN, false);
+    else RPTC_LAUNCH(RPTC_CONTINUOUS, false);
+#undef RPTC_LAUNCH
     return t.end();
 }
 
@@ -576,7 +611,10 @@ static int launch_matvec_fused(const int32_t *compressed, const uint16_t *codebo
     DeviceInfo *dev;
     MatvecArgs a;
     int lds_bytes, grid;
-    int rc = plan_matvec(compressed, codebook, x, out, m, n, carry_mode, &dev, &a, &lds_bytes, &grid);
+    bool compact;
+    // the norm variant holds the whole vector in registers (n <= 16384): never long enough to need compact sums
+    int rc = plan_matvec(compressed, codebook, x, out, m, n, carry_mode, XMODE == kXSiluMul, &dev, &a, &compact, &lds_bytes,
+                         &grid);
     if (rc) return rc;
     hipStream_t s = static_cast<hipStream_t>(stream);
     Timer t;
@@ -588,14 +626,20 @@ static int launch_matvec_fused(const int32_t *compressed, const uint16_t *codebo
     auto a_x2 = reinterpret_cast<const uint4 *>(x2);
     auto a_w = reinterpret_cast<const uint4 *>(norm_w);
     auto a_xo = reinterpret_cast<uint4 *>(x_out);
-    if (carry_mode == RPTC_AS_WRITTEN)
-        hipLaunchKernelGGL((matvec_fused_kernel<S, RPTC_AS_WRITTEN, XMODE>), dim3(grid), dim3(kMatvecThreads), lds_bytes,
-                           s, a_comp, a_cb, a_x, out, a.m, a.n, a.rows_per_block, a.rw_tail, a.items_full, a.items_tail,
-                           a_x2, a_w, a_xo, eps);
-    else
-        hipLaunchKernelGGL((matvec_fused_kernel<S, RPTC_CONTINUOUS, XMODE>), dim3(grid), dim3(kMatvecThreads), lds_bytes,
-                           s, a_comp, a_cb, a_x, out, a.m, a.n, a.rows_per_block, a.rw_tail, a.items_full, a.items_tail,
-                           a_x2, a_w, a_xo, eps);
+#define RPTC_LAUNCH(MODE, COMPACT)                                                                                  \
+    hipLaunchKernelGGL((matvec_fused_kernel<S, MODE, XMODE, COMPACT>), dim3(grid), dim3(kMatvecThreads), lds_bytes, \
+                       s, a_comp, a_cb, a_x, out, a.m, a.n, a.rows_per_block, a.rw_tail, a.items_full, a.items_tail, \
+                       a_x2, a_w, a_xo, eps)
+    if constexpr (XMODE == kXSiluMul) {
+        if (compact) {
+            if (carry_mode == RPTC_AS_WRITTEN) RPTC_LAUNCH(RPTC_AS_WRITTEN, true);
+            else RPTC_LAUNCH(RPTC_CONTINUOUS, true);
+            return t.end();
+        }
+    }
+    if (carry_mode == RPTC_AS_WRITTEN) RPTC_LAUNCH(RPTC_AS_WRITTEN, false);
+    else RPTC_LAUNCH(RPTC_CONTINUOUS, false);
+#undef RPTC_LAUNCH
     return t.end();
 }
 
@@ -673,22 +717,24 @@ static int set_lds_limit(F *kernel)
 int prepare_matvec()
 {
     int rc;
-#define RPTC_SET_LIMITS(BITS)                                                               \
-    if ((rc = set_lds_limit(matvec_kernel<6, RPTC_AS_WRITTEN, BITS>))) return rc;              \
-    if ((rc = set_lds_limit(matvec_kernel<6, RPTC_CONTINUOUS, BITS>))) return rc;              \
-    if ((rc = set_lds_limit(matvec_kernel<8, RPTC_AS_WRITTEN, BITS>))) return rc;              \
-    if ((rc = set_lds_limit(matvec_kernel<8, RPTC_CONTINUOUS, BITS>))) return rc;
-    RPTC_SET_LIMITS(2)
-    RPTC_SET_LIMITS(3)
-    RPTC_SET_LIMITS(4)
+#define RPTC_SET_LIMITS(BITS, COMPACT)                                                               \
+    if ((rc = set_lds_limit(matvec_kernel<6, RPTC_AS_WRITTEN, BITS, COMPACT>))) return rc;              \
+    if ((rc = set_lds_limit(matvec_kernel<6, RPTC_CONTINUOUS, BITS, COMPACT>))) return rc;              \
+    if ((rc = set_lds_limit(matvec_kernel<8, RPTC_AS_WRITTEN, BITS, COMPACT>))) return rc;              \
+    if ((rc = set_lds_limit(matvec_kernel<8, RPTC_CONTINUOUS, BITS, COMPACT>))) return rc;
+    RPTC_SET_LIMITS(2, false)
+    RPTC_SET_LIMITS(2, true)
+    RPTC_SET_LIMITS(3, false)
+    RPTC_SET_LIMITS(4, false)
 #undef RPTC_SET_LIMITS
-#define RPTC_SET_LIMITS(XMODE)                                                                    \
-    if ((rc = set_lds_limit(matvec_fused_kernel<6, RPTC_AS_WRITTEN, XMODE>))) return rc;             \
-    if ((rc = set_lds_limit(matvec_fused_kernel<6, RPTC_CONTINUOUS, XMODE>))) return rc;             \
-    if ((rc = set_lds_limit(matvec_fused_kernel<8, RPTC_AS_WRITTEN, XMODE>))) return rc;             \
-    if ((rc = set_lds_limit(matvec_fused_kernel<8, RPTC_CONTINUOUS, XMODE>))) return rc;
-    RPTC_SET_LIMITS(kXSiluMul)
-    RPTC_SET_LIMITS(kXAddRmsNorm)
+#define RPTC_SET_LIMITS(XMODE, COMPACT)                                                                    \
+    if ((rc = set_lds_limit(matvec_fused_kernel<6, RPTC_AS_WRITTEN, XMODE, COMPACT>))) return rc;             \
+    if ((rc = set_lds_limit(matvec_fused_kernel<6, RPTC_CONTINUOUS, XMODE, COMPACT>))) return rc;             \
+    if ((rc = set_lds_limit(matvec_fused_kernel<8, RPTC_AS_WRITTEN, XMODE, COMPACT>))) return rc;             \
+    if ((rc = set_lds_limit(matvec_fused_kernel<8, RPTC_CONTINUOUS, XMODE, COMPACT>))) return rc;
+    RPTC_SET_LIMITS(kXSiluMul, false)
+    RPTC_SET_LIMITS(kXSiluMul, true)
+    RPTC_SET_LIMITS(kXAddRmsNorm, false)
 #undef RPTC_SET_LIMITS
     return 0;
 }

@@ -116,6 +116,21 @@ __device__ __forceinline__ float wave_sum(float v)
     return v;
 }
 
+// Sums over lanes 0-31 and over lanes 32-63 (in lanes 31 and 63): wave_sum without its last step.
+__device__ __forceinline__ float half_wave_sum(float v)
+{
+#define RPTC_DPP_ADD(ctrl, row_mask, bank_mask)                                                      \
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0u, __builtin_bit_cast(uint32_t, v), \
+                                                               ctrl, row_mask, bank_mask, false))
+    RPTC_DPP_ADD(0x111, 0xF, 0xF);   // row_shr:1
+    RPTC_DPP_ADD(0x112, 0xF, 0xF);   // row_shr:2
+    RPTC_DPP_ADD(0x114, 0xF, 0xF);   // row_shr:4
+    RPTC_DPP_ADD(0x118, 0xF, 0xF);   // row_shr:8
+    RPTC_DPP_ADD(0x142, 0xA, 0xF);   // row_bcast:15 into rows 1 and 3
+#undef RPTC_DPP_ADD
+    return v;
+}
+
 __device__ __forceinline__ uint16_t float_to_half_bits(float f)
 {
     _Float16 h = (_Float16)f;   // v_cvt_f16_f32, round to nearest even

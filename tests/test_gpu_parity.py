@@ -205,6 +205,34 @@ def test_matvec_full_size(rk, oracle, m, n):
     assert rel_l2(np_f16(out12).astype(np.float64), np_f16(out).astype(np.float64) + np_f16(out2).astype(np.float64)) < 5e-3
 
 
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("m,n", [(8192, 28672), (8192, 28672 + 192)])
+def test_matvec_long_rows(rk, oracle, mode, m, n):
+    """Rows so long that a CU's share of them needs the compact partial-sum layout (one sum per row and
+    slab); the product must still match the double-precision product of the bit-exact dense matrix."""
+    S = 8
+    comp = rand_codes(m * n // 16, seed=52)
+    cb = rand_half(2 << S, seed=53)
+    x = rand_half(n, seed=54)
+    out = torch.full((m,), float("nan"), dtype=torch.float16, device="cuda")
+    c = comp.cuda().reshape(n // 2048, m, 128) if n % 2048 == 0 else comp.cuda()
+    with with_mode(rk, mode):
+        matvec_fn(rk, 16, S)(c, cb.cuda(), x.cuda(), out)
+        W = torch.zeros((m, n), dtype=torch.float16, device="cuda")
+        rk.matvec_dense(comp.cuda(), cb.cuda(), W, S)
+    y_dense = (W.double() @ x.cuda().double()).cpu().numpy()
+    assert rel_l2(np_f16(out), y_dense) < REL_L2_TOL
+    # the dense export is held to the oracle on the first rows (the whole matrix at this size takes the CPU a while)
+    rows = 64
+    idx = np_u32(comp).reshape(-1)
+    T, Lt = n // 2048, (n % 2048) // 64
+    parts = [idx[t * m * 128:(t * m + rows) * 128] for t in range(T)]
+    if Lt:
+        parts.append(idx[T * m * 128:T * m * 128 + rows * Lt * 4])
+    wantW = oracle.matvec_dense(np.concatenate(parts), np_f16(cb), rows, n, S, mode=mode)
+    assert np.array_equal(np_f16(W[:rows]).view(np.uint16), wantW.view(np.uint16))
+
+
 def test_matvec_zero_stream_closed_form(rk):
     m, n, S = 64, 4096, 6
     cb = rand_half(2 << S, seed=3)
