@@ -8,7 +8,7 @@ namespace rptc {
 
 int prepare_decompress();
 int prepare_matvec();
-int prepare_matvec_t();
+int prepare_matvec_t(int device);
 int prepare_matmul(int device);
 int prepare_hadamard();
 int prepare_decode_glue(int device);
@@ -37,7 +37,7 @@ int device_info(DeviceInfo **out)
         if ((rc = (int)hipEventCreate(&d.ev_stop))) return rc;
         if ((rc = prepare_decompress())) return rc;
         if ((rc = prepare_matvec())) return rc;
-        if ((rc = prepare_matvec_t())) return rc;
+        if ((rc = prepare_matvec_t(dev))) return rc;
         if ((rc = prepare_matmul(dev))) return rc;
         if ((rc = prepare_hadamard())) return rc;
         if ((rc = prepare_decode_glue(dev))) return rc;

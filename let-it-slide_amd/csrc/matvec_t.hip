@@ -6,16 +6,25 @@
 // same for the whole wave and come through the scalar cache, and nothing crosses lanes.
 //
 // gfx950 design: the whole codebook (128 KiB at L = 16) sits in LDS; the reference's
-// one-thread-per-row loop is split over the 8 waves of a workgroup along the columns, which the
-// stream allows because the decoder state after an element depends only on that element
-// (as written: the top nibbles of its four words, inference_t.cu:131-142; continuous: its last
-// L bits), so a wave warms its state up from the element before its range.
+// one-thread-per-row loop is split along the columns, over the 8 waves of a workgroup and, when
+// there are fewer 64-row blocks than CUs, over several workgroups per row block.  The stream
+// allows it because the decoder state after an element depends only on that element (as written:
+// the top nibbles of its four words, inference_t.cu:131-142; continuous: its last L bits), so a
+// wave warms its state up from the element before its range.  Waves are added in LDS in wave
+// order; workgroups of a row block publish fp32 partial sums in a static scratch buffer with
+// device-scope stores, and the one that arrives last at the row block's counter adds them in
+// workgroup order and accumulates into `out`: every sum has a fixed order.
 #include "rptc_common.hpp"
 
 namespace rptc {
 
 constexpr int kTThreads = 512;
 constexpr int kTWaves = kTThreads / kWave;
+constexpr int kTMaxParts = 4096;        // workgroups of a launch that splits the columns
+constexpr int kTMaxSplit = 16;
+
+static __device__ __align__(256) float g_t_part[kTMaxParts * kWave];
+static __device__ __align__(256) uint32_t g_t_arrived[kTMaxParts];
 
 template <int L>
 __device__ __forceinline__ uint32_t warm_state(const uint4 e, int mode)
@@ -33,7 +42,7 @@ __device__ __forceinline__ uint32_t warm_state(const uint4 e, int mode)
 template <int L, int MODE>
 __global__ __launch_bounds__(kTThreads) void matvec_t_kernel(
     const uint4 *__restrict__ comp, const uint4 *__restrict__ codebook, const uint32_t *__restrict__ x,
-    uint16_t *__restrict__ out, int m, int cols)
+    uint16_t *__restrict__ out, float *__restrict__ parts, uint32_t *__restrict__ arrived, int m, int cols, int ksplit)
 {
     extern __shared__ uint4 lds_u4[];
     constexpr int lut_u4 = (2 << L) / 16;
@@ -52,10 +61,14 @@ __global__ __launch_bounds__(kTThreads) void matvec_t_kernel(
     const uint16_t *lut = reinterpret_cast<const uint16_t *>(lds_u4);
     float *part = reinterpret_cast<float *>(lds_u4 + lut_u4);      // [wave][lane]
 
-    const int row = blockIdx.x * kWave + lane;
+    const int rb = blockIdx.x / ksplit, sp = blockIdx.x - rb * ksplit;
+    const int row = rb * kWave + lane;
     const bool valid = row < m;
-    const int per = (cols + kTWaves - 1) / kTWaves;
-    const int c0 = wave * per, c1 = min(cols, c0 + per);
+    // this workgroup's columns, then this wave's share of them
+    const int per_group = (cols + ksplit - 1) / ksplit;
+    const int g0 = min(cols, sp * per_group), g1 = min(cols, g0 + per_group);
+    const int per = (g1 - g0 + kTWaves - 1) / kTWaves;
+    const int c0 = min(g1, g0 + wave * per), c1 = min(g1, c0 + per);
     const uint4 zero = make_uint4(0, 0, 0, 0);
 
     uint32_t carry = 0;
@@ -93,13 +106,41 @@ __global__ __launch_bounds__(kTThreads) void matvec_t_kernel(
     }
     part[wave * kWave + lane] = acc;
     __syncthreads();
-    if (tid < kWave && valid) {
-        float y = 0.f;
+    float y = 0.f;
+    if (tid < kWave) {
 #pragma unroll
         for (int w = 0; w < kTWaves; w++) y += part[w * kWave + tid];
-        // the product is added to what out holds (inference_t.cu:170-171)
-        out[row] = float_to_half_bits(half_bits_to_float(out[row]) + y);
     }
+    if (ksplit == 1) {
+        // the product is added to what out holds (inference_t.cu:170-171)
+        if (tid < kWave && valid) out[row] = float_to_half_bits(half_bits_to_float(out[row]) + y);
+        return;
+    }
+    // Device-scope stores and loads bypass the XCD-private cache levels, so the only ordering needed
+    // is that this workgroup's stores have completed before its arrival is counted.
+    if (tid < kWave) __hip_atomic_store(&parts[(size_t)blockIdx.x * kWave + tid], y, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    uint32_t *flag = reinterpret_cast<uint32_t *>(part);
+    if (tid == 0) {
+        const uint32_t prev = __hip_atomic_fetch_add(&arrived[rb], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const bool last = prev == (uint32_t)(ksplit - 1);
+        if (last) __hip_atomic_store(&arrived[rb], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // for the next launch
+        *flag = last;
+    }
+    __syncthreads();
+    if (!*flag || tid >= kWave || !valid) return;
+    float p[kTMaxSplit];
+#pragma unroll
+    for (int i = 0; i < kTMaxSplit; i++)
+        p[i] = i < ksplit ? __hip_atomic_load(&parts[((size_t)rb * ksplit + i) * kWave + tid], __ATOMIC_RELAXED,
+                                              __HIP_MEMORY_SCOPE_AGENT)
+                          : 0.f;
+    float total = 0.f;
+#pragma unroll
+    for (int i = 0; i < kTMaxSplit; i++) total += p[i];
+    out[row] = float_to_half_bits(half_bits_to_float(out[row]) + total);
 }
 
 // Dense export: one thread per stream element.
@@ -141,6 +182,12 @@ __global__ __launch_bounds__(256) void matvec_t_dense_kernel(
 template <int L>
 static int lds_bytes_t() { return (2 << L) + kTThreads * 4; }
 
+struct TScratch {
+    float *parts;
+    uint32_t *arrived;
+};
+static TScratch g_t[64];   // per device: addresses of the static scratch arrays
+
 template <int L>
 static int launch_matvec_t(const int32_t *compressed, const uint16_t *codebook, const uint16_t *x,
                            uint16_t *out, int64_t m, int64_t n, int carry_mode, void *stream, float *ms)
@@ -158,16 +205,23 @@ static int launch_matvec_t(const int32_t *compressed, const uint16_t *codebook, 
     Timer t;
     rc = t.begin(dev, s, ms);
     if (rc) return rc;
-    const int grid = (int)((m + kWave - 1) / kWave);
+    const int row_blocks = (int)((m + kWave - 1) / kWave);
+    const int cols = (int)(n / 64);
+    // workgroups per row block: enough for every CU, each wave keeps at least one column
+    int ksplit = dev->cus / row_blocks;
+    if (ksplit > kTMaxSplit) ksplit = kTMaxSplit;
+    if (ksplit > cols / kTWaves) ksplit = cols / kTWaves;
+    if (ksplit < 1 || row_blocks * ksplit > kTMaxParts) ksplit = 1;
+    const TScratch &sc = g_t[dev->device];
     auto a_comp = reinterpret_cast<const uint4 *>(compressed);
     auto a_cb = reinterpret_cast<const uint4 *>(codebook);
     auto a_x = reinterpret_cast<const uint32_t *>(x);
     if (carry_mode == RPTC_AS_WRITTEN)
-        hipLaunchKernelGGL((matvec_t_kernel<L, RPTC_AS_WRITTEN>), dim3(grid), dim3(kTThreads), lds_bytes_t<L>(), s,
-                           a_comp, a_cb, a_x, out, (int)m, (int)(n / 64));
+        hipLaunchKernelGGL((matvec_t_kernel<L, RPTC_AS_WRITTEN>), dim3(row_blocks * ksplit), dim3(kTThreads),
+                           lds_bytes_t<L>(), s, a_comp, a_cb, a_x, out, sc.parts, sc.arrived, (int)m, cols, ksplit);
     else
-        hipLaunchKernelGGL((matvec_t_kernel<L, RPTC_CONTINUOUS>), dim3(grid), dim3(kTThreads), lds_bytes_t<L>(), s,
-                           a_comp, a_cb, a_x, out, (int)m, (int)(n / 64));
+        hipLaunchKernelGGL((matvec_t_kernel<L, RPTC_CONTINUOUS>), dim3(row_blocks * ksplit), dim3(kTThreads),
+                           lds_bytes_t<L>(), s, a_comp, a_cb, a_x, out, sc.parts, sc.arrived, (int)m, cols, ksplit);
     return t.end();
 }
 
@@ -187,8 +241,13 @@ static int launch_t_dense(const int32_t *compressed, const uint16_t *codebook, u
     return 0;
 }
 
-int prepare_matvec_t()
+int prepare_matvec_t(int device)
 {
+    // the device addresses of the static scratch arrays (the symbols themselves are not device addresses)
+    int rc0 = (int)hipGetSymbolAddress(reinterpret_cast<void **>(&g_t[device].parts), HIP_SYMBOL(g_t_part));
+    if (rc0) return rc0;
+    rc0 = (int)hipGetSymbolAddress(reinterpret_cast<void **>(&g_t[device].arrived), HIP_SYMBOL(g_t_arrived));
+    if (rc0) return rc0;
     const void *k[] = {
         reinterpret_cast<const void *>(matvec_t_kernel<16, RPTC_AS_WRITTEN>),
         reinterpret_cast<const void *>(matvec_t_kernel<16, RPTC_CONTINUOUS>),
