@@ -233,13 +233,13 @@ __device__ __forceinline__ void matvec_body(
 
     // Loads are returned in issue order, so the small loads the table and the activation image
     // wait for go first and the stream loads, which take longest, are issued right behind them.
-    constexpr int kTableWrites = kTableBytes / 16 / kMatvecThreads;     // 16-byte writes per thread
-    uint32_t cbv[kTableWrites];
+    // Table rows 16 * wave .. 16 * wave + 15 are this wave's to write.  A row is 64 copies of one
+    // value, so the value is wave-uniform and comes through the scalar cache: these loads neither
+    // queue with the vector loads nor return in order with them.
+    constexpr int kRowsPerWave = 256 / kMatvecWaves;
+    uint32_t cbv[kRowsPerWave];
 #pragma unroll
-    for (int i = 0; i < kTableWrites; i++) {
-        const int row = (i * kMatvecThreads + tid) >> 4;                // a table row is 16 uint4
-        cbv[i] = table_value<S>(codebook, row);
-    }
+    for (int i = 0; i < kRowsPerWave; i++) cbv[i] = table_value<S>(codebook, kRowsPerWave * wave + i);
     constexpr int kXRegs = 2;
     uint4 xv[kXRegs], xv2[kXRegs], xvw[kXRegs];
 #pragma unroll
@@ -362,10 +362,8 @@ __device__ __forceinline__ void matvec_body(
     }
 
     // table (256 rows x 64 lane copies) and activation image into LDS
-    uint4 *lds4 = reinterpret_cast<uint4 *>(lds);
 #pragma unroll
-    for (int i = 0; i < kTableWrites; i++)
-        lds4[i * kMatvecThreads + tid] = make_uint4(cbv[i], cbv[i], cbv[i], cbv[i]);
+    for (int i = 0; i < kRowsPerWave; i++) lds[(kRowsPerWave * wave + i) * 64 + lane] = cbv[i];
     auto stage_x = [&](int idx, const uint4 v) {          // halves 8idx .. 8idx+7 (inference.cu:215-221)
         sx[idx] = v.x;
         sx[idx + n8] = v.y;
