@@ -54,17 +54,48 @@ __device__ __forceinline__ void hadamard_pass(float *buf, int P, int s, int tid)
 
 __global__ __launch_bounds__(kHadThreads) void sign_hadamard_kernel(
     const uint16_t *__restrict__ x, const uint16_t *__restrict__ signs, uint16_t *__restrict__ out,
-    int n, int P, int log_p, int blocks_per_row, int signs_after)
+    int n, int P, int log_p, int blocks_per_row, int signs_after, int wide)
 {
     extern __shared__ float buf[];
     const int tid = threadIdx.x;
     const int row = blockIdx.x / blocks_per_row, blk = blockIdx.x - row * blocks_per_row;
     const size_t base = (size_t)row * n + (size_t)blk * P;
     const uint16_t *s = signs + (size_t)blk * P;
-    for (int i = tid; i < P; i += kHadThreads) {
-        float v = half_bits_to_float(x[base + i]);
-        if (!signs_after) v *= half_bits_to_float(s[i]);
-        buf[pad(i)] = v;
+    // wide != 0: P % 8 == 0 and 16-byte aligned pointers: 8 halves per load, up to four loads of a
+    // thread requested before the first is used (one at a time they would be a round trip each)
+    constexpr int kInFlight = 4;
+    if (wide) {
+        const uint4 *x4 = reinterpret_cast<const uint4 *>(x + base), *s4 = reinterpret_cast<const uint4 *>(s);
+        for (int c0 = tid; c0 < (P >> 3); c0 += kHadThreads * kInFlight) {
+            uint4 xv[kInFlight], sv[kInFlight];
+#pragma unroll
+            for (int u = 0; u < kInFlight; u++) {
+                const int c = c0 + u * kHadThreads;
+                xv[u] = sv[u] = make_uint4(0, 0, 0, 0);
+                if (c < (P >> 3)) {
+                    xv[u] = x4[c];
+                    if (!signs_after) sv[u] = s4[c];
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < kInFlight; u++) {
+                const int c = c0 + u * kHadThreads;
+                if (c >= (P >> 3)) break;
+                const uint32_t xw[4] = {xv[u].x, xv[u].y, xv[u].z, xv[u].w}, sw[4] = {sv[u].x, sv[u].y, sv[u].z, sv[u].w};
+#pragma unroll
+                for (int k = 0; k < 8; k++) {
+                    float v = half_bits_to_float((uint16_t)(xw[k >> 1] >> (16 * (k & 1))));
+                    if (!signs_after) v *= half_bits_to_float((uint16_t)(sw[k >> 1] >> (16 * (k & 1))));
+                    buf[pad(8 * c + k)] = v;
+                }
+            }
+        }
+    } else {
+        for (int i = tid; i < P; i += kHadThreads) {
+            float v = half_bits_to_float(x[base + i]);
+            if (!signs_after) v *= half_bits_to_float(s[i]);
+            buf[pad(i)] = v;
+        }
     }
     __syncthreads();
     int stage = 0;
@@ -78,10 +109,38 @@ __global__ __launch_bounds__(kHadThreads) void sign_hadamard_kernel(
     else if (rest == 1) hadamard_pass<1>(buf, P, stage, tid);
     if (rest) __syncthreads();
     const float scale = rsqrtf((float)P);
-    for (int i = tid; i < P; i += kHadThreads) {
-        float v = buf[pad(i)] * scale;
-        if (signs_after) v *= half_bits_to_float(s[i]);
-        out[base + i] = float_to_half_bits(v);
+    if (wide) {
+        const uint4 *s4 = reinterpret_cast<const uint4 *>(s);
+        uint4 *o4 = reinterpret_cast<uint4 *>(out + base);
+        for (int c0 = tid; c0 < (P >> 3); c0 += kHadThreads * kInFlight) {
+            uint4 sv[kInFlight];
+#pragma unroll
+            for (int u = 0; u < kInFlight; u++) {
+                const int c = c0 + u * kHadThreads;
+                sv[u] = make_uint4(0, 0, 0, 0);
+                if (signs_after && c < (P >> 3)) sv[u] = s4[c];
+            }
+#pragma unroll
+            for (int u = 0; u < kInFlight; u++) {
+                const int c = c0 + u * kHadThreads;
+                if (c >= (P >> 3)) break;
+                const uint32_t sw[4] = {sv[u].x, sv[u].y, sv[u].z, sv[u].w};
+                uint32_t ow[4] = {0, 0, 0, 0};
+#pragma unroll
+                for (int k = 0; k < 8; k++) {
+                    float v = buf[pad(8 * c + k)] * scale;
+                    if (signs_after) v *= half_bits_to_float((uint16_t)(sw[k >> 1] >> (16 * (k & 1))));
+                    ow[k >> 1] |= (uint32_t)float_to_half_bits(v) << (16 * (k & 1));
+                }
+                o4[c] = make_uint4(ow[0], ow[1], ow[2], ow[3]);
+            }
+        }
+    } else {
+        for (int i = tid; i < P; i += kHadThreads) {
+            float v = buf[pad(i)] * scale;
+            if (signs_after) v *= half_bits_to_float(s[i]);
+            out[base + i] = float_to_half_bits(v);
+        }
     }
 }
 
@@ -118,6 +177,7 @@ extern "C" int rptc_sign_hadamard(const uint16_t *x, const uint16_t *signs, uint
     int log_p = 0;
     while (((int64_t)1 << log_p) < P) log_p++;
     hipLaunchKernelGGL(sign_hadamard_kernel, dim3((unsigned)(batch * blocks_per_row)), dim3(kHadThreads),
-                       (size_t)(P + P / 32) * 4, s, x, signs, out, (int)n, (int)P, log_p, blocks_per_row, inverse ? 1 : 0);
+                       (size_t)(P + P / 32) * 4, s, x, signs, out, (int)n, (int)P, log_p, blocks_per_row, inverse ? 1 : 0,
+                       (P % 8 == 0 && aligned16(x) && aligned16(signs) && aligned16(out)) ? 1 : 0);
     return t.end();
 }
