@@ -232,10 +232,31 @@ def bench_matmul(a):
             "speedup_vs_decode_then_gemm": round(times["decode_then_gemm"] / us, 2),
             "rel_l2_vs_dense": float(f"{err:.3e}"),
         }
-    print(json.dumps({"metric": "fused decode+GEMM (MFMA) per call", "unit": "us", "n_gpus": 1,
-                      "config": {"workload": f"decompress_matmul_16_{S}_1 m={m} n={n} 2 bits/weight, {copies} rotating "
-                                             f"weight copies", "launch": "graph"},
-                      "results": results}))
+    other = {}
+    if a.extra_shapes:
+        # the other layer shapes at batch 16, fused kernel only
+        del weights, W
+        fn = getattr(rptc_kernels, f"decompress_matmul_16_{S}_1")
+        for mm, nn in ((11008, 4096), (8192, 8192), (28672, 8192), (8192, 28672)):
+            words = mm * nn // 16
+            cps = max(2, min(a.copies, (512 << 20) // (words * 4) + 1))
+            ws = [torch.randint(-(1 << 31), 1 << 31, (words,), generator=g, dtype=torch.int64, device="cuda").to(torch.int32)
+                  for _ in range(cps)]
+            x = torch.randn((16, nn), generator=g, device="cuda").to(torch.float16)
+            out = torch.zeros((16, mm), dtype=torch.float16, device="cuda")
+            us = _graph_time_us(lambda k: fn(ws[k % cps], cb, x, out), min(a.steps, 200))
+            flops = 2.0 * mm * nn * 16
+            other[f"{mm}x{nn} batch16"] = {"us": round(us, 2), "TFLOPs": round(flops / us / 1e6, 2),
+                                          "mfma_util": round(flops / us / 1e6 / MFMA_F16_PEAK_TFLOPS, 5),
+                                          "hbm_GBps": round(mm * nn / 4 / us / 1e3, 1)}
+            del ws
+    line = {"metric": "fused decode+GEMM (MFMA) per call", "unit": "us", "n_gpus": 1,
+            "config": {"workload": f"decompress_matmul_16_{S}_1 m={m} n={n} 2 bits/weight, {copies} rotating "
+                                   f"weight copies", "launch": "graph"},
+            "results": results}
+    if other:
+        line["other_shapes"] = other
+    print(json.dumps(line))
 
 
 def _graph_time_us(step, steps):
@@ -395,6 +416,46 @@ def main():
             "launch_us": round(launch_ms * 1e3, 3),
         },
     }
+    # the floor of this workload on this machine, in the same launch pattern (graph replay over the
+    # same rotating buffers): an empty launch, and a kernel that only reads the stream
+    lib = runner.lib
+
+    def floor_us(call):
+        steps = min(a.steps, 400)
+        for k in range(10):
+            call(k, torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            cs = torch.cuda.current_stream().cuda_stream
+            for k in range(steps):
+                call(k, cs)
+        graph.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        graph.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / steps * 1e3
+
+    def call_empty(k, cs):
+        if lib.rptc_probe_empty(ctypes.c_void_p(cs)):
+            raise RuntimeError("rptc_probe_empty failed")
+
+    def call_read(k, cs):
+        w = runner.weights[k % len(runner.weights)]
+        if lib.rptc_probe_read(w.data_ptr(), runner.bytes, None, ctypes.c_void_p(cs)):
+            raise RuntimeError("rptc_probe_read failed")
+
+    if a.launch == "graph":
+        empty_us, read_us = floor_us(call_empty), floor_us(call_read)
+        line["roofline"]["floor"] = {
+            "empty_launch_us": round(empty_us, 3),
+            "read_only_us": round(read_us, 3),
+            "read_only_GBps": round(runner.bytes / read_us / 1e3, 1),
+            "note": "same bytes, same graph-replayed launch pattern: an empty kernel, and a kernel that only reads the stream",
+        }
     if a.extra_shapes:
         extra = {}
         for (m, n) in ((4096, 4096), (11008, 4096), (8192, 8192), (28672, 8192), (8192, 28672)):

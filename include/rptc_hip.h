@@ -206,6 +206,17 @@ int rptc_decompress_matvec_rmsnorm(const int32_t *compressed, const uint16_t *co
                                    int64_t m, int64_t n, float eps, int S, int carry_mode, void *stream,
                                    float *ms);
 
+/*
+ * Measurement aids (no counterpart in the reference; not part of the product path).  bench.py times
+ * them in the same launch pattern as the mat-vec it grades, so that the achieved figure can be read
+ * against the floor for the workload's size on the machine at hand.
+ *   rptc_probe_empty  one empty 1024-thread workgroup per CU
+ *   rptc_probe_read   reads `bytes` (a multiple of 16, 16-byte aligned) with non-temporal 16-byte loads
+ *                     and writes nothing; `sink` may be NULL
+ */
+int rptc_probe_empty(void *stream);
+int rptc_probe_read(const void *data, int64_t bytes, void *sink, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -59,6 +59,8 @@ _SIGNATURES = {
     "rptc_rope_cache": ([_VP, _VP, _VP, _VP, _VP, _VP, _VP, _I64, _I64, _I64, _VP], _INT),
     "rptc_attn_decode": ([_VP, _VP, _VP, _VP, _VP, _I64, _I64, _I64, _VP], _INT),
     "rptc_silu_mul": ([_VP, _VP, _I64, _VP], _INT),
+    "rptc_probe_empty": ([_VP], _INT),
+    "rptc_probe_read": ([_VP, _I64, _VP, _VP], _INT),
     "rptc_rope_attn_decode": ([_VP, _VP, _VP, _VP, _VP, _VP, _VP, _I64, _I64, _I64, _VP], _INT),
     "rptc_decompress_matvec_silu": ([_VP, _VP, _VP, _VP, _I64, _I64, _INT, _INT, _VP, _FP], _INT),
     "rptc_decompress_matvec_rmsnorm": ([_VP, _VP, _VP, _VP, _VP, _VP, _VP, _I64, _I64, ctypes.c_float, _INT, _INT,
