@@ -250,6 +250,22 @@ def bench_matmul(a):
                                           "mfma_util": round(flops / us / 1e6 / MFMA_F16_PEAK_TFLOPS, 5),
                                           "hbm_GBps": round(mm * nn / 4 / us / 1e3, 1)}
             del ws
+    if a.extra_shapes:
+        # 3 and 4 bits per weight on the headline shape, batch 16
+        for bits in (3, 4):
+            mm, nn = 4096, 11008
+            words = mm * nn * bits // 32
+            cps = max(2, min(a.copies, (512 << 20) // (words * 4) + 1))
+            ws = [torch.randint(-(1 << 31), 1 << 31, (words,), generator=g, dtype=torch.int64, device="cuda").to(torch.int32)
+                  for _ in range(cps)]
+            x = torch.randn((16, nn), generator=g, device="cuda").to(torch.float16)
+            out = torch.zeros((16, mm), dtype=torch.float16, device="cuda")
+            us = _graph_time_us(lambda k: rptc_kernels.decompress_matmul_bits(ws[k % cps], cb, x, out, bits), min(a.steps, 200))
+            flops = 2.0 * mm * nn * 16
+            other[f"{mm}x{nn} {bits}b batch16"] = {"us": round(us, 2), "TFLOPs": round(flops / us / 1e6, 2),
+                                                  "mfma_util": round(flops / us / 1e6 / MFMA_F16_PEAK_TFLOPS, 5),
+                                                  "hbm_GBps": round(mm * nn * bits / 8 / us / 1e3, 1)}
+            del ws
     line = {"metric": "fused decode+GEMM (MFMA) per call", "unit": "us", "n_gpus": 1,
             "config": {"workload": f"decompress_matmul_16_{S}_1 m={m} n={n} 2 bits/weight, {copies} rotating "
                                    f"weight copies", "launch": "graph"},

@@ -134,6 +134,10 @@ int rptc_matvec_t_dense(const int32_t *compressed, const uint16_t *codebook, uin
 int rptc_decompress_matmul(const int32_t *compressed, const uint16_t *codebook, const uint16_t *x,
                            uint16_t *out, int64_t m, int64_t n, int64_t batch, int S, int carry_mode,
                            void *stream, float *ms);
+/* The same at `bits` (2, 3, 4) bits per weight: the stream of rptc_decompress_matvec_bits. */
+int rptc_decompress_matmul_bits(const int32_t *compressed, const uint16_t *codebook, const uint16_t *x,
+                                uint16_t *out, int64_t m, int64_t n, int64_t batch, int S, int bits,
+                                int carry_mode, void *stream, float *ms);
 
 /*
  * The hashed pair stream at `bits` = 2, 3 or 4 bits per weight, S in {6, 8}.  No counterpart in

@@ -101,17 +101,35 @@ __device__ __forceinline__ void gather2(uint32_t g, uint32_t lane4, uint32_t &w_
     w_lo = lds_read_abs(and_or(h, 0xFF00u, lane4));
 }
 
+// Row blocks a workgroup can hold in registers beside the activation pairs.
+__host__ __device__ constexpr int mm_max_row_blocks(int planes, int bits)
+{
+    return bits == 2 ? (planes == 1 ? kMmMaxRowBlocks : 6) : (planes == 1 ? 6 : 3);   // even for one plane
+}
+
+// Step s of an element multiplies activation slot 4k + j with k = 7, 0, 4, 1, 5, 2, 6, 3 for
+// s / 4 = 0..7 and j = s % 4 (inference.cu:237-250).
+__device__ constexpr int mm_k_of_step_block(int sb)
+{
+    constexpr int k_of[8] = {7, 0, 4, 1, 5, 2, 6, 3};
+    return k_of[sb];
+}
+
+// BITS: bits per weight.  2 is the reference stream (an element is 4 words, two windows per
+// v_alignbit_b32); at 3 and 4 an element is 2 * BITS words, a step advances 2 * BITS stream bits, and
+// the four windows of an MFMA's A operand are cut out one by one.
 // four waves per SIMD = two workgroups per CU: at most 128 vector registers
-template <int S, int MODE, int PLANES>
+template <int S, int MODE, int PLANES, int BITS>
 __global__ __launch_bounds__(kMmThreads) __attribute__((amdgpu_waves_per_eu(4, 4))) void matmul_kernel(
-    const uint4 *__restrict__ comp, const uint32_t *__restrict__ codebook, const uint32_t *__restrict__ xp32,
+    const uint32_t *__restrict__ comp32, const uint32_t *__restrict__ codebook, const uint32_t *__restrict__ xp32,
     float *__restrict__ partial, uint32_t *__restrict__ arrived, uint16_t *__restrict__ out, int m, int n, int batch,
     int max_rb, int groups_total, int group_base)
 {
     extern __shared__ uint32_t lds[];
     // 64 KiB of table + 16 KiB of tiles: two workgroups share a CU's 160 KiB whatever the batch
     constexpr int kPartBuffers = PLANES == 1 ? 2 : 1;
-    constexpr int kMaxRb = PLANES == 1 ? kMmMaxRowBlocks : 6;
+    constexpr int WORDS = 2 * BITS;                               // words per stream element
+    constexpr int kMaxRb = mm_max_row_blocks(PLANES, BITS);
     RPTC_MM_STAMP(0);
     float *part = reinterpret_cast<float *>(lds + kMmTableBytes / 4);   // [buffer][wave][plane][v][lane]
     // the "came last" flag reuses the first word of the tiles once they are no longer read (all LDS
@@ -130,7 +148,6 @@ __global__ __launch_bounds__(kMmThreads) __attribute__((amdgpu_waves_per_eu(4, 4
     const int rb_begin = (int)(((int64_t)(group_base + grp) * total_rb) / groups_total);
     const int row_blocks = (int)(((int64_t)(group_base + grp + 1) * total_rb) / groups_total) - rb_begin;
     const int row0 = rb_begin * 16;
-    const uint32_t *comp32 = reinterpret_cast<const uint32_t *>(comp);
 
     const int lanes = slab < T ? 32 : Lt;                        // elements per row in this slab
     const size_t elem0 = (size_t)(slab < T ? slab : T) * m * 32;
@@ -160,17 +177,29 @@ __global__ __launch_bounds__(kMmThreads) __attribute__((amdgpu_waves_per_eu(4, 4
     // element 0 instead, which is harmless: its products are multiplied by zero activations or land
     // in tile rows that are never stored.  Lane-of-row 0 reads its own last word as the carry
     // (inference.cu:232, as written) or lane 31 of the previous slab (continuous).
-    uint4 e_all[kMaxRb];
+    uint32_t e_all[kMaxRb][WORDS];
     uint32_t carry_all[kMaxRb];
 #pragma unroll
     for (int rb = 0; rb < kMaxRb; rb++) {
         const int row = row0 + 16 * rb + i;
         const bool valid = rb < row_blocks && has_l && row < m;
         const size_t ei = valid ? elem0 + (size_t)row * lanes + l : 0;
-        size_t ci = ei * 4 + 3;
-        if (l > 0 && valid) ci = ei * 4 - 1;                             // last word of the previous lane-of-row
-        else if (MODE == RPTC_CONTINUOUS && slab > 0 && valid) ci = (((size_t)(slab - 1) * m + row) * 32 + 31) * 4 + 3;
-        e_all[rb] = comp[ei];
+        size_t ci = ei * WORDS + WORDS - 1;
+        if (l > 0 && valid) ci = ei * WORDS - 1;                         // last word of the previous lane-of-row
+        else if (MODE == RPTC_CONTINUOUS && slab > 0 && valid) ci = (((size_t)(slab - 1) * m + row) * 32 + 31) * WORDS + WORDS - 1;
+        if constexpr (WORDS % 4 == 0) {
+#pragma unroll
+            for (int q = 0; q < WORDS / 4; q++) {
+                const uint4 v = reinterpret_cast<const uint4 *>(comp32 + ei * WORDS)[q];
+                e_all[rb][4 * q] = v.x, e_all[rb][4 * q + 1] = v.y, e_all[rb][4 * q + 2] = v.z, e_all[rb][4 * q + 3] = v.w;
+            }
+        } else {
+#pragma unroll
+            for (int q = 0; q < WORDS / 2; q++) {
+                const uint2 v = reinterpret_cast<const uint2 *>(comp32 + ei * WORDS)[q];
+                e_all[rb][2 * q] = v.x, e_all[rb][2 * q + 1] = v.y;
+            }
+        }
         carry_all[rb] = comp32[ci];
     }
     const bool no_carry = MODE == RPTC_CONTINUOUS && slab == 0 && l == 0;     // the stream starts here
@@ -193,27 +222,58 @@ __global__ __launch_bounds__(kMmThreads) __attribute__((amdgpu_waves_per_eu(4, 4
         if (rb >= row_blocks) break;
         float *buf = part + (kPartBuffers == 2 ? (rb & 1) : 0) * (kMmWaves * PLANES * 256);
         if (c < waves_used) {
-            const uint4 e = e_all[rb];
             const uint32_t carry = no_carry ? 0u : carry_all[rb];
             v4f32 d0[PLANES], d1[PLANES];
 #pragma unroll
             for (int p = 0; p < PLANES; p++) d0[p] = d1[p] = v4f32{0.f, 0.f, 0.f, 0.f};
+            if constexpr (BITS == 2) {
+                const uint4 e = make_uint4(e_all[rb][0], e_all[rb][1], e_all[rb][2], e_all[rb][3]);
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                const uint32_t sh = 12 - 4 * j;
-                const uint32_t gc = j == 3 ? e.x : alignbit(carry, e.x, sh);   // steps (7,j) and (0,j)
-                const uint32_t gx = j == 3 ? e.y : alignbit(e.x, e.y, sh);     // (4,j), (1,j)
-                const uint32_t gy = j == 3 ? e.z : alignbit(e.y, e.z, sh);     // (5,j), (2,j)
-                const uint32_t gz = j == 3 ? e.w : alignbit(e.z, e.w, sh);     // (6,j), (3,j)
-                uint32_t w0, w1, w2, w3, w4, w5, w6, w7;
-                gather2(gc, lane4, w0, w1);
-                gather2(gx, lane4, w2, w3);
-                gather2(gy, lane4, w4, w5);
-                gather2(gz, lane4, w6, w7);
+                for (int j = 0; j < 4; j++) {
+                    const uint32_t sh = 12 - 4 * j;
+                    const uint32_t gc = j == 3 ? e.x : alignbit(carry, e.x, sh);   // steps (7,j) and (0,j)
+                    const uint32_t gx = j == 3 ? e.y : alignbit(e.x, e.y, sh);     // (4,j), (1,j)
+                    const uint32_t gy = j == 3 ? e.z : alignbit(e.y, e.z, sh);     // (5,j), (2,j)
+                    const uint32_t gz = j == 3 ? e.w : alignbit(e.z, e.w, sh);     // (6,j), (3,j)
+                    uint32_t w0, w1, w2, w3, w4, w5, w6, w7;
+                    gather2(gc, lane4, w0, w1);
+                    gather2(gx, lane4, w2, w3);
+                    gather2(gy, lane4, w4, w5);
+                    gather2(gz, lane4, w6, w7);
 #pragma unroll
-                for (int p = 0; p < PLANES; p++) {
-                    d0[p] = mma4(w0, w1, w2, w3, xb[p][28 + j], xb[p][j], xb[p][16 + j], xb[p][4 + j], d0[p]);
-                    d1[p] = mma4(w4, w5, w6, w7, xb[p][20 + j], xb[p][8 + j], xb[p][24 + j], xb[p][12 + j], d1[p]);
+                    for (int p = 0; p < PLANES; p++) {
+                        d0[p] = mma4(w0, w1, w2, w3, xb[p][28 + j], xb[p][j], xb[p][16 + j], xb[p][4 + j], d0[p]);
+                        d1[p] = mma4(w4, w5, w6, w7, xb[p][20 + j], xb[p][8 + j], xb[p][24 + j], xb[p][12 + j], d1[p]);
+                    }
+                }
+            } else {
+                // four consecutive steps per MFMA: their slots are 4k .. 4k+3 of one k
+                constexpr int SB = 2 * BITS;
+#pragma unroll
+                for (int sb = 0; sb < 8; sb++) {
+                    uint32_t w[4];
+#pragma unroll
+                    for (int u = 0; u < 4; u++) {
+                        const int st = 4 * sb + u;
+                        const int end = SB * (st + 1), start = end - 16;
+                        uint32_t h;
+                        if (start < 0) {
+                            h = (carry << end) | (e_all[rb][0] >> (32 - end));
+                        } else {
+                            const int wi = start >> 5, o = start & 31;
+                            h = o <= 16 ? e_all[rb][wi] >> (16 - o)
+                                        : alignbit(e_all[rb][wi], e_all[rb][wi + 1 < WORDS ? wi + 1 : wi], 48 - o);
+                        }
+                        h &= 0xFFFFu;
+                        const uint32_t prod = __umul24(h, h) + h;             // low 16 bits of h * (h + 1)
+                        w[u] = lds_read_abs(and_or(prod, 0xFF00u, lane4));
+                    }
+                    const int k = mm_k_of_step_block(sb);
+#pragma unroll
+                    for (int p = 0; p < PLANES; p++) {
+                        v4f32 &d = (sb & 1) ? d1[p] : d0[p];
+                        d = mma4(w[0], w[1], w[2], w[3], xb[p][4 * k], xb[p][4 * k + 1], xb[p][4 * k + 2], xb[p][4 * k + 3], d);
+                    }
                 }
             }
             // tile element (row 4*(lane/16) + v, batch column lane%16) sits in register v of lane `lane`
@@ -311,14 +371,18 @@ static int mm_allow_lds(K kernel)
 int prepare_matmul(int device)
 {
     int rc;
-    if ((rc = mm_allow_lds(matmul_kernel<6, RPTC_AS_WRITTEN, 1>))) return rc;
-    if ((rc = mm_allow_lds(matmul_kernel<6, RPTC_CONTINUOUS, 1>))) return rc;
-    if ((rc = mm_allow_lds(matmul_kernel<8, RPTC_AS_WRITTEN, 1>))) return rc;
-    if ((rc = mm_allow_lds(matmul_kernel<8, RPTC_CONTINUOUS, 1>))) return rc;
-    if ((rc = mm_allow_lds(matmul_kernel<6, RPTC_AS_WRITTEN, 2>))) return rc;
-    if ((rc = mm_allow_lds(matmul_kernel<6, RPTC_CONTINUOUS, 2>))) return rc;
-    if ((rc = mm_allow_lds(matmul_kernel<8, RPTC_AS_WRITTEN, 2>))) return rc;
-    if ((rc = mm_allow_lds(matmul_kernel<8, RPTC_CONTINUOUS, 2>))) return rc;
+#define RPTC_MM_ALLOW(PLANES, BITS)                                                          \
+    if ((rc = mm_allow_lds(matmul_kernel<6, RPTC_AS_WRITTEN, PLANES, BITS>))) return rc;    \
+    if ((rc = mm_allow_lds(matmul_kernel<6, RPTC_CONTINUOUS, PLANES, BITS>))) return rc;    \
+    if ((rc = mm_allow_lds(matmul_kernel<8, RPTC_AS_WRITTEN, PLANES, BITS>))) return rc;    \
+    if ((rc = mm_allow_lds(matmul_kernel<8, RPTC_CONTINUOUS, PLANES, BITS>))) return rc;
+    RPTC_MM_ALLOW(1, 2)
+    RPTC_MM_ALLOW(2, 2)
+    RPTC_MM_ALLOW(1, 3)
+    RPTC_MM_ALLOW(2, 3)
+    RPTC_MM_ALLOW(1, 4)
+    RPTC_MM_ALLOW(2, 4)
+#undef RPTC_MM_ALLOW
     // the device addresses of the static scratch arrays (the symbols themselves are not device addresses)
     MmScratch &sc = g_mm[device];
     if ((rc = (int)hipGetSymbolAddress(reinterpret_cast<void **>(&sc.xpack), HIP_SYMBOL(g_xpack)))) return rc;
@@ -327,10 +391,10 @@ int prepare_matmul(int device)
 }
 
 // Number of row groups: as many as keep every workgroup of the launch resident at once (two per
-// CU), but no group larger than kMmMaxRowBlocks row blocks.
-static int mm_groups(int m, int slabs, int cus, int planes)
+// CU), but no group larger than the kernel's register budget allows.
+static int mm_groups(int m, int slabs, int cus, int planes, int bits)
 {
-    const int max_rb = planes == 1 ? kMmMaxRowBlocks : 6;
+    const int max_rb = mm_max_row_blocks(planes, bits);
     const int total = (m + 15) / 16;
     int groups = 2 * cus / slabs;
     if (groups < 1) groups = 1;
@@ -339,8 +403,8 @@ static int mm_groups(int m, int slabs, int cus, int planes)
     return groups < least ? least : groups;
 }
 
-template <int S, int PLANES>
-static void launch_matmul(const uint4 *comp, const uint32_t *cb, const MmScratch &sc, uint16_t *out, int m, int n,
+template <int S, int PLANES, int BITS>
+static void launch_matmul(const uint32_t *comp, const uint32_t *cb, const MmScratch &sc, uint16_t *out, int m, int n,
                           int batch, int carry_mode, int groups, int slabs, hipStream_t s)
 {
     const int lds_bytes = kMmTableBytes + kMmWaves * 2 * 256 * 4;
@@ -352,26 +416,34 @@ static void launch_matmul(const uint4 *comp, const uint32_t *cb, const MmScratch
     for (int g0 = 0; g0 < groups; g0 += (int)per_launch) {
         const int g_n = groups - g0 < per_launch ? groups - g0 : (int)per_launch;
         if (carry_mode == RPTC_AS_WRITTEN)
-            hipLaunchKernelGGL((matmul_kernel<S, RPTC_AS_WRITTEN, PLANES>), dim3(g_n * slabs), dim3(kMmThreads),
+            hipLaunchKernelGGL((matmul_kernel<S, RPTC_AS_WRITTEN, PLANES, BITS>), dim3(g_n * slabs), dim3(kMmThreads),
                                lds_bytes, s, comp, cb, sc.xpack, sc.partial, sc.arrived, out, m, n, batch, max_rb,
                                groups, g0);
         else
-            hipLaunchKernelGGL((matmul_kernel<S, RPTC_CONTINUOUS, PLANES>), dim3(g_n * slabs), dim3(kMmThreads),
+            hipLaunchKernelGGL((matmul_kernel<S, RPTC_CONTINUOUS, PLANES, BITS>), dim3(g_n * slabs), dim3(kMmThreads),
                                lds_bytes, s, comp, cb, sc.xpack, sc.partial, sc.arrived, out, m, n, batch, max_rb,
                                groups, g0);
     }
+}
+
+template <int S, int BITS>
+static void launch_matmul_planes(const uint32_t *comp, const uint32_t *cb, const MmScratch &sc, uint16_t *out, int m,
+                                 int n, int batch, int carry_mode, int cus, int slabs, hipStream_t s)
+{
+    if (batch <= 16) launch_matmul<S, 1, BITS>(comp, cb, sc, out, m, n, batch, carry_mode, mm_groups(m, slabs, cus, 1, BITS), slabs, s);
+    else launch_matmul<S, 2, BITS>(comp, cb, sc, out, m, n, batch, carry_mode, mm_groups(m, slabs, cus, 2, BITS), slabs, s);
 }
 
 }  // namespace rptc
 
 using namespace rptc;
 
-extern "C" int rptc_decompress_matmul(const int32_t *compressed, const uint16_t *codebook, const uint16_t *x,
-                                      uint16_t *out, int64_t m, int64_t n, int64_t batch, int S, int carry_mode,
-                                      void *stream, float *ms)
+extern "C" int rptc_decompress_matmul_bits(const int32_t *compressed, const uint16_t *codebook, const uint16_t *x,
+                                           uint16_t *out, int64_t m, int64_t n, int64_t batch, int S, int bits,
+                                           int carry_mode, void *stream, float *ms)
 {
     if (!compressed || !codebook || !x || !out) return RPTC_ENULL;
-    if (m < 1 || n < 64 || n % 64 != 0 || batch < 1 || (S != 6 && S != 8)) return RPTC_ESHAPE;
+    if (m < 1 || n < 64 || n % 64 != 0 || batch < 1 || (S != 6 && S != 8) || bits < 2 || bits > 4) return RPTC_ESHAPE;
     if (n > kMmMaxN || batch > kMmMaxBatch || m >= (1 << 24)) return RPTC_ELIMIT;
     if (carry_mode != RPTC_AS_WRITTEN && carry_mode != RPTC_CONTINUOUS) return RPTC_EMODE;
     if (!aligned16(compressed) || !aligned16(codebook) || !aligned16(x)) return RPTC_EALIGN;
@@ -379,23 +451,31 @@ extern "C" int rptc_decompress_matmul(const int32_t *compressed, const uint16_t 
     int rc = device_info(&dev);
     if (rc) return rc;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    auto a_comp = reinterpret_cast<const uint4 *>(compressed);
+    Timer t;
+    rc = t.begin(dev, s, ms);
+    if (rc) return rc;
+    auto a_comp = reinterpret_cast<const uint32_t *>(compressed);
     auto a_cb = reinterpret_cast<const uint32_t *>(codebook);
     const MmScratch &sc = g_mm[dev->device];
     const int planes = batch > 16 ? 2 : 1;
     const int slabs = (int)(n / 2048) + (n % 2048 ? 1 : 0);
-    const int groups = mm_groups((int)m, slabs, dev->cus, planes);
-    Timer t;
-    rc = t.begin(dev, s, ms);
-    if (rc) return rc;
+    const int groups = mm_groups((int)m, slabs, dev->cus, planes, bits);
     const int counters = groups < kMmMaxGroups ? groups : kMmMaxGroups;
     const int total = planes * (int)(n / 8) * 16;
     const int pack_threads = total > counters ? total : counters;
     hipLaunchKernelGGL(pack_x_kernel, dim3((pack_threads + 255) / 256), dim3(256), 0, s, reinterpret_cast<const uint4 *>(x), sc.xpack, sc.arrived,
                        counters, (int)n, (int)batch, planes);
-    if (S == 6 && planes == 1) launch_matmul<6, 1>(a_comp, a_cb, sc, out, (int)m, (int)n, (int)batch, carry_mode, groups, slabs, s);
-    else if (S == 6) launch_matmul<6, 2>(a_comp, a_cb, sc, out, (int)m, (int)n, (int)batch, carry_mode, groups, slabs, s);
-    else if (planes == 1) launch_matmul<8, 1>(a_comp, a_cb, sc, out, (int)m, (int)n, (int)batch, carry_mode, groups, slabs, s);
-    else launch_matmul<8, 2>(a_comp, a_cb, sc, out, (int)m, (int)n, (int)batch, carry_mode, groups, slabs, s);
+#define RPTC_MM_GO(SS, BB)                                                                                          \
+    if (S == SS && bits == BB)                                                                                       \
+        launch_matmul_planes<SS, BB>(a_comp, a_cb, sc, out, (int)m, (int)n, (int)batch, carry_mode, dev->cus, slabs, s);
+    RPTC_MM_GO(6, 2) RPTC_MM_GO(6, 3) RPTC_MM_GO(6, 4) RPTC_MM_GO(8, 2) RPTC_MM_GO(8, 3) RPTC_MM_GO(8, 4)
+#undef RPTC_MM_GO
     return t.end();
+}
+
+extern "C" int rptc_decompress_matmul(const int32_t *compressed, const uint16_t *codebook, const uint16_t *x,
+                                      uint16_t *out, int64_t m, int64_t n, int64_t batch, int S, int carry_mode,
+                                      void *stream, float *ms)
+{
+    return rptc_decompress_matmul_bits(compressed, codebook, x, out, m, n, batch, S, 2, carry_mode, stream, ms);
 }

@@ -52,6 +52,7 @@ _SIGNATURES = {
     "rptc_matvec_dense": ([_VP, _VP, _VP, _I64, _I64, _INT, _INT, _VP, _FP], _INT),
     "rptc_matvec_t_dense": ([_VP, _VP, _VP, _I64, _I64, _INT, _INT, _VP, _FP], _INT),
     "rptc_decompress_matmul": ([_VP, _VP, _VP, _VP, _I64, _I64, _I64, _INT, _INT, _VP, _FP], _INT),
+    "rptc_decompress_matmul_bits": ([_VP, _VP, _VP, _VP, _I64, _I64, _I64, _INT, _INT, _INT, _VP, _FP], _INT),
     "rptc_sign_hadamard": ([_VP, _VP, _VP, _I64, _I64, _I64, _INT, _VP, _FP], _INT),
     "rptc_decompress_matvec_bits": ([_VP, _VP, _VP, _VP, _I64, _I64, _INT, _INT, _INT, _VP, _FP], _INT),
     "rptc_matvec_bits_dense": ([_VP, _VP, _VP, _I64, _I64, _INT, _INT, _INT, _VP, _FP], _INT),
@@ -286,7 +287,7 @@ def matvec_t_dense(compressed, codebook, out, L):
     return _call(library().rptc_matvec_t_dense, (compressed, codebook, out), m, n, L)
 
 
-def _matmul(S, compressed, codebook, x, out):
+def _matmul(S, compressed, codebook, x, out, bits=2):
     _check_input(compressed, "compressed")
     _check(compressed.dtype == torch.int32, "compressed.scalar_type() == torch::kInt32")
     _check_input(x, "x")
@@ -301,11 +302,12 @@ def _matmul(S, compressed, codebook, x, out):
     _check(1 <= batch <= 32, "1 <= batch <= 32")
     _check(n % 64 == 0 and n >= 64 and m >= 1, "x.size(1) % 64 == 0")
     _check(n <= 32768, "x.size(1) <= 32768")
-    _check(compressed.numel() * 16 == m * n, "compressed.numel() * 16 == m * n")
+    _check(bits in (2, 3, 4), "bits must be 2, 3 or 4")
+    _check(compressed.numel() * 32 == m * n * bits, "compressed.numel() * 32 == m * n * bits")
     _check_input(codebook, "codebook")
     _check(codebook.dim() == 1 and codebook.size(0) == 1 << (S + 1), "codebook.size(0) == 1<<(S+V)")
     _check(codebook.dtype == torch.float16, "codebook.scalar_type() == torch::kFloat16")
-    return _call(library().rptc_decompress_matmul, (compressed, codebook, x, out), m, n, batch, S)
+    return _call(library().rptc_decompress_matmul_bits, (compressed, codebook, x, out), m, n, batch, S, bits)
 
 
 def decompress_matmul_16_6_1(compressed, codebook, x, out):
@@ -316,6 +318,14 @@ def decompress_matmul_16_6_1(compressed, codebook, x, out):
 def decompress_matmul_16_8_1(compressed, codebook, x, out):
     """out[b] = W x[b] for batch 1..32 on the hashed-codebook stream with 256 pairs; x [batch, n], out [batch, m]."""
     return _matmul(8, compressed, codebook, x, out)
+
+
+def decompress_matmul_bits(compressed, codebook, x, out, bits):
+    """out[b] = W x[b] for batch 1..32 on the hashed pair stream at ``bits`` (2, 3, 4) bits per weight; S from the
+    codebook length; x [batch, n], out [batch, m]."""
+    _check_input(codebook, "codebook")
+    _check(codebook.dim() == 1 and codebook.size(0) in (128, 512), "codebook.size(0) == 1<<(S+V), S in {6, 8}")
+    return _matmul(6 if codebook.size(0) == 128 else 8, compressed, codebook, x, out, bits=bits)
 
 
 def hadamard_block(n):

@@ -408,6 +408,67 @@ def test_matmul_identity_batch_recovers_weights_bit_exactly(rk, oracle, mode):
     assert np.all((g[~nz] & 0x7FFF) == 0)
 
 
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("bits", [3, 4])
+@pytest.mark.parametrize("S", [6, 8])
+@pytest.mark.parametrize("batch", [1, 16, 19, 32])
+@pytest.mark.parametrize("m,n", [(16, 2048), (33, 2048 + 704), (5, 704), (300, 6144)])
+def test_matmul_bits_output_within_tolerance(rk, oracle, mode, bits, S, batch, m, n):
+    """3 and 4 bits per weight on the matrix cores against the double-precision product of the oracle's dense matrix."""
+    comp = rand_codes(m * n * bits // 32, seed=m + n + batch + bits)
+    cb = rand_half(2 << S, seed=S + 60)
+    x = rand_half(batch * n, seed=19).reshape(batch, n)
+    out = torch.full((batch, m), float("nan"), dtype=torch.float16, device="cuda")
+    with with_mode(rk, mode):
+        ms = rk.decompress_matmul_bits(comp.cuda(), cb.cuda(), x.cuda(), out, bits)
+    assert ms > 0
+    W = oracle.bits_dense(np_u32(comp), np_f16(cb), m, n, S, bits, mode=mode)
+    want = np_f16(x).astype(np.float64) @ W.astype(np.float64).T
+    got = np_f16(out).astype(np.float64)
+    assert np.all(np.isfinite(got))
+    assert rel_l2(got, want) < REL_L2_TOL
+
+
+@pytest.mark.parametrize("bits", [3, 4])
+def test_matmul_bits_identity_batch_recovers_weights_bit_exactly(rk, oracle, bits):
+    S, m, n, mode = 8, 40, 2048 + 128, 1
+    comp = rand_codes(m * n * bits // 32, seed=654 + bits)
+    cb = rand_half(2 << S, seed=61)
+    want = oracle.bits_dense(np_u32(comp), np_f16(cb), m, n, S, bits, mode=mode)
+    c, cbd = comp.cuda(), cb.cuda()
+    got = np.zeros((m, n), dtype=np.float16)
+    out = torch.zeros((32, m), dtype=torch.float16, device="cuda")
+    prev_timing = rk.set_timing(False)
+    try:
+        with with_mode(rk, mode):
+            for p0 in range(0, n, 32):
+                x = torch.zeros((32, n), dtype=torch.float16, device="cuda")
+                x[torch.arange(32), torch.arange(p0, p0 + 32)] = 1.0
+                rk.decompress_matmul_bits(c, cbd, x, out, bits)
+                got[:, p0:p0 + 32] = np_f16(out).T
+    finally:
+        rk.set_timing(prev_timing)
+    g, w = got.view(np.uint16), want.view(np.uint16)
+    nz = (w & 0x7FFF) != 0
+    assert np.array_equal(g[nz], w[nz])
+    assert np.all((g[~nz] & 0x7FFF) == 0)
+
+
+@pytest.mark.parametrize("bits", [3, 4])
+def test_matmul_bits_full_size_equals_the_mat_vec(rk, bits):
+    """At the full layer size the batched product must agree, row by row, with the mat-vec kernel of the same stream."""
+    S, m, n, batch = 8, 4096, 11008, 16
+    comp = rand_codes(m * n * bits // 32, seed=42).cuda()
+    cb = rand_half(2 << S, seed=43).cuda()
+    x = rand_half(batch * n, seed=44).reshape(batch, n).cuda()
+    out = torch.zeros((batch, m), dtype=torch.float16, device="cuda")
+    rk.decompress_matmul_bits(comp, cb, x, out, bits)
+    for b in (0, 7, 15):
+        y = torch.zeros(m, dtype=torch.float16, device="cuda")
+        rk.decompress_matvec_bits(comp, cb, x[b].contiguous(), y, bits)
+        assert rel_l2(np_f16(out[b]), np_f16(y).astype(np.float64)) < REL_L2_TOL
+
+
 @pytest.mark.parametrize("batch", [8, 16, 32])
 def test_matmul_full_size_equals_decode_then_dense_gemm(rk, oracle, batch):
     S, m, n = 8, 4096, 11008
