@@ -21,18 +21,21 @@ REFERENCE_PATTERN = r"model\.layers\.(\d+)\.(self_attn\.(\w+)_proj|mlp\.(\w+)_pr
 
 
 class QuantizedLinear(torch.nn.Module):
-    """y = W x with W held as a hashed-pair trellis stream (2 bits/weight) plus the optional
-    row/column scales and biases of the reference's factorisation and an optional sign-Hadamard
-    transform of the input."""
+    """y = W x with W held as a hashed-pair trellis stream (2 bits/weight, the reference's format, or 3 or
+    4) plus the optional row/column scales and biases of the reference's factorisation and an optional
+    sign-Hadamard transform of the input."""
 
-    def __init__(self, in_features, out_features, S=8, carry_mode=rk.CONTINUOUS, device="cuda"):
+    def __init__(self, in_features, out_features, S=8, carry_mode=rk.CONTINUOUS, device="cuda", bits=2):
         super().__init__()
         if in_features % 64 != 0:
             raise ValueError("in_features must be a multiple of 64 (whole stream elements per row)")
         if S not in (6, 8):
             raise ValueError("S must be 6 or 8")
+        if bits not in (2, 3, 4):
+            raise ValueError("bits must be 2, 3 or 4")
         self.in_features, self.out_features, self.S, self.carry_mode = in_features, out_features, S, carry_mode
-        words = out_features * in_features // 16
+        self.bits = bits
+        words = out_features * in_features * bits // 32
         self.register_buffer("compressed", torch.zeros(words, dtype=torch.int32, device=device))
         self.register_buffer("codebook", torch.zeros(2 << S, dtype=torch.float16, device=device))
         for name in ("scales_out", "scales_in", "biases_out", "biases_in", "signs"):
@@ -56,17 +59,17 @@ class QuantizedLinear(torch.nn.Module):
 
     @classmethod
     def from_symbols(cls, symbols, codebook, out_features, S=8, device="cuda", **kw):
-        """symbols: 4-bit trellis symbols [out_features, in_features/2] in stream order (numpy or tensor)."""
+        """symbols: trellis symbols of 2*bits bits [out_features, in_features/2] in stream order (numpy or tensor)."""
         from rptc_kernels import packing
         import numpy as np
         sym = symbols.cpu().numpy() if isinstance(symbols, torch.Tensor) else np.asarray(symbols)
         layer = cls(2 * sym.shape[1], out_features, S=S, device=device, **kw)
-        layer.compressed.copy_(torch.from_numpy(packing.pack_matvec(sym)).to(device))
+        layer.compressed.copy_(torch.from_numpy(packing.pack_matvec(sym, bits=layer.bits)).to(device))
         layer.codebook.copy_(torch.as_tensor(codebook, dtype=torch.float16).to(device))
         return layer
 
     @classmethod
-    def from_weight(cls, weight, codebook=None, S=8, importance=None, seed=42, device="cuda"):
+    def from_weight(cls, weight, codebook=None, S=8, importance=None, seed=42, device="cuda", bits=2):
         """Quantize a dense weight [out, in] with the Viterbi search of ``rptc_kernels.quantize`` (run on
         ``device``) and pack the result.  codebook: fp16 [2^(S+1)] or None for a seeded Gaussian one
         scaled to the weight's standard deviation."""
@@ -76,8 +79,8 @@ class QuantizedLinear(torch.nn.Module):
             g = torch.Generator().manual_seed(seed)
             codebook = (torch.randn(2 << S, generator=g) * W.std().item()).to(torch.float16)
         codebook = torch.as_tensor(codebook, dtype=torch.float16)
-        symbols, mse = quantize.quantize_matrix(W, codebook.to(device), S, importance=importance)
-        layer = cls.from_symbols(symbols, codebook, W.size(0), S=S, device=device)
+        symbols, mse = quantize.quantize_matrix(W, codebook.to(device), S, importance=importance, bits=bits)
+        layer = cls.from_symbols(symbols, codebook, W.size(0), S=S, device=device, bits=bits)
         layer.quantization_mse = mse
         return layer
 
@@ -111,15 +114,14 @@ class QuantizedLinear(torch.nn.Module):
         out = torch.empty((batch, self.out_features), dtype=torch.float16, device=x2.device)
         lib = rk.library()
         if batch == 1:
-            fn = getattr(lib, f"rptc_decompress_matvec_16_{self.S}_1")
-            rk._call(fn, (self.compressed, self.codebook, x2, out), self.out_features, self.in_features,
-                     carry_mode=self.carry_mode)
+            rk._call(lib.rptc_decompress_matvec_bits, (self.compressed, self.codebook, x2, out), self.out_features,
+                     self.in_features, self.S, self.bits, carry_mode=self.carry_mode)
             return out
         for b0 in range(0, batch, 32):
             xb = x2[b0:b0 + 32]
             ob = out[b0:b0 + 32]
-            rk._call(lib.rptc_decompress_matmul, (self.compressed, self.codebook, xb, ob), self.out_features,
-                     self.in_features, xb.size(0), self.S, carry_mode=self.carry_mode)
+            rk._call(lib.rptc_decompress_matmul_bits, (self.compressed, self.codebook, xb, ob), self.out_features,
+                     self.in_features, xb.size(0), self.S, self.bits, carry_mode=self.carry_mode)
         return out
 
     def forward(self, x):
@@ -156,8 +158,8 @@ class QuantizedLinear(torch.nn.Module):
         W = torch.empty((self.out_features, self.in_features), dtype=torch.float16, device=self.compressed.device)
         prev = rk.set_timing(False)
         try:
-            rk._call(rk.library().rptc_matvec_dense, (self.compressed, self.codebook, W), self.out_features,
-                     self.in_features, self.S, carry_mode=self.carry_mode)
+            rk._call(rk.library().rptc_matvec_bits_dense, (self.compressed, self.codebook, W), self.out_features,
+                     self.in_features, self.S, self.bits, carry_mode=self.carry_mode)
         finally:
             rk.set_timing(prev)
         return W
@@ -166,7 +168,7 @@ class QuantizedLinear(torch.nn.Module):
         return self.compressed.numel() * 4
 
     def extra_repr(self):
-        return f"in_features={self.in_features}, out_features={self.out_features}, S={self.S}, bits_per_weight=2"
+        return f"in_features={self.in_features}, out_features={self.out_features}, S={self.S}, bits_per_weight={self.bits}"
 
 
 def patch_model(model, pattern=REFERENCE_PATTERN, S=8, seed=42, make_layer=None):

@@ -67,10 +67,11 @@ def viterbi_pairs(targets, table, weights=None, state_bits=STATE_BITS, step_bits
     return symbols, cost
 
 
-def quantize_matrix(W, codebook, S=8, importance=None, rows_per_batch=64):
-    """Quantize W [m, n] (n % 64 == 0) to 4-bit symbols [m, n/2] in stream order, for the decoder of
-    ``decompress_matvec_*`` in CONTINUOUS mode.  importance: optional [n] per-column weight (e.g. the
-    Hessian diagonal, quantize_hf.py:164).  Returns (symbols int64 [m, n/2] on the CPU, mse float)."""
+def quantize_matrix(W, codebook, S=8, importance=None, rows_per_batch=64, bits=2):
+    """Quantize W [m, n] (n % 64 == 0) to symbols of 2*bits bits [m, n/2] in stream order, for the decoder
+    of ``decompress_matvec_*`` (bits == 2) or ``decompress_matvec_bits`` in CONTINUOUS mode.  importance:
+    optional [n] per-column weight (e.g. the Hessian diagonal, quantize_hf.py:164).  Returns (symbols int64
+    [m, n/2] on the CPU, mse float)."""
     W = torch.as_tensor(W)
     m, n = W.shape
     dev = W.device
@@ -87,13 +88,13 @@ def quantize_matrix(W, codebook, S=8, importance=None, rows_per_batch=64):
     for r0 in range(0, m, rows_per_batch):
         tg = targets[r0:r0 + rows_per_batch]
         w = None if wts is None else wts.expand(tg.size(0), -1, -1)
-        sym, cost = viterbi_pairs(tg, table, w)
+        sym, cost = viterbi_pairs(tg, table, w, step_bits=2 * bits)
         out[r0:r0 + rows_per_batch] = sym.cpu()
         total += cost.sum().item()
     return out, total / (m * n)
 
 
-def dequantize_symbols(symbols, codebook, S=8):
+def dequantize_symbols(symbols, codebook, S=8, bits=2):
     """The dense matrix [m, n] a symbol array (stream order) decodes to, by walking the shift register
     (rptc.py:74-85 with 4-bit steps and the hashed pair lookup): the definition the kernels are held to."""
     symbols = torch.as_tensor(symbols, dtype=torch.int64)
@@ -104,7 +105,7 @@ def dequantize_symbols(symbols, codebook, S=8):
     state = torch.zeros(m, dtype=torch.int64)
     W = torch.empty((m, n), dtype=torch.float32)
     for p in range(half):
-        state = ((state << STEP_BITS) | symbols[:, p]) & ((1 << STATE_BITS) - 1)
+        state = ((state << (2 * bits)) | symbols[:, p]) & ((1 << STATE_BITS) - 1)
         W[:, cols[p]] = table[state, 0]
         W[:, cols[p] + 1] = table[state, 1]
     return W

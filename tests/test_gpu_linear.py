@@ -137,6 +137,32 @@ def test_from_weight_quantizes_and_runs(rk):
     assert rel_l2(y.cpu().numpy(), want.numpy()) < 1e-3
 
 
+@pytest.mark.parametrize("bits", [3, 4])
+@pytest.mark.parametrize("batch", [1, 20])
+def test_quantized_linear_at_3_and_4_bits(rk, bits, batch):
+    from rptc_kernels.linear import QuantizedLinear
+    n, m = 2048 + 192, 96
+    layer = QuantizedLinear.from_random(n, m, S=8, seed=3, bits=bits)
+    assert layer.compressed.numel() * 32 == m * n * bits
+    x = torch.randn((batch, n), generator=torch.Generator().manual_seed(4)).half().cuda()
+    y = layer(x)
+    W = layer.decoded_weight()
+    want = x.double() @ W.double().t()
+    assert rel_l2(y.cpu().numpy(), want.cpu().numpy()) < 1e-3
+
+
+def test_from_weight_at_3_bits_beats_2_bits(rk):
+    from rptc_kernels.linear import QuantizedLinear
+    g = torch.Generator().manual_seed(6)
+    W = torch.randn((8, 256), generator=g) * 0.05
+    l2 = QuantizedLinear.from_weight(W, S=8, bits=2)
+    l3 = QuantizedLinear.from_weight(W, S=8, bits=3)
+    assert l3.quantization_mse <= l2.quantization_mse
+    x = torch.randn((1, 256), generator=g).half().cuda()
+    want = x.double().cpu() @ l3.decoded_weight().double().cpu().t()
+    assert rel_l2(l3(x).cpu().numpy(), want.numpy()) < 1e-3
+
+
 def test_llama_decode_paths_agree(rk):
     """A 2-layer Llama-shaped model on streams: the fused one-token step matches the torch path's logits,
     graph replay reproduces direct launches token for token, and the logits match the same network run on

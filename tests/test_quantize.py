@@ -58,3 +58,23 @@ def test_quantize_matrix_round_trip_through_the_packed_stream(oracle):
     rand = quantize.dequantize_symbols(torch.from_numpy(g.integers(0, 16, (m, n // 2))), torch.from_numpy(cb), S).numpy()
     assert mse < 0.25 * ((W - rand) ** 2).mean()
     assert mse < 0.2          # unit-variance Gaussian at 2 bits/weight: rate-distortion bound 0.0625
+
+
+def test_quantize_matrix_at_3_and_4_bits_round_trips_and_gets_better_with_the_rate(oracle):
+    """More bits per step means more successors per state: the decoder walk, the packed stream decoded by the
+    oracle and the reported error agree, and the error falls with the rate."""
+    g = np.random.default_rng(5)
+    m, n, S = 2, 128, 8
+    W = g.standard_normal((m, n)).astype(np.float32)
+    cb = g.standard_normal(2 << S).astype(np.float16)
+    errors = {}
+    for bits in (2, 3, 4):
+        symbols, mse = quantize.quantize_matrix(torch.from_numpy(W), torch.from_numpy(cb), S, bits=bits)
+        assert symbols.shape == (m, n // 2) and int(symbols.max()) < (1 << (2 * bits))
+        What = quantize.dequantize_symbols(symbols, torch.from_numpy(cb), S, bits=bits).numpy()
+        stream = packing.pack_matvec(symbols.numpy(), bits=bits)
+        Wor = oracle.bits_dense(stream, cb, m, n, S, bits, mode=oracle.CONTINUOUS).astype(np.float32)
+        assert np.array_equal(What, Wor)
+        assert abs(((W - What) ** 2).mean() - mse) < 1e-5
+        errors[bits] = mse
+    assert errors[4] <= errors[3] <= errors[2]
