@@ -340,6 +340,37 @@ def test_matvec_t_full_size_4096(rk, oracle):
         assert rel_l2(np_f16(out), want) < REL_L2_TOL
 
 
+def test_matvec_t_at_the_reference_activation_limit(rk, oracle):
+    """n = 32768 is what the reference's 64 KiB of constant memory holds (inference_t.cu:49): accepted and right."""
+    L, m, n = 16, 64, 32768
+    comp = rand_codes(m * n // 16, seed=71)
+    cb = rand_half(1 << L, seed=72)
+    x = rand_half(n, seed=73)
+    out = torch.zeros((m,), dtype=torch.float16, device="cuda")
+    rk.decompress_matvec_t_16(comp.cuda(), cb.cuda(), x.cuda(), out)
+    want = oracle.matvec_t(np_u32(comp), np_f16(cb), np_f16(x), m, L, mode=0)
+    assert rel_l2(np_f16(out), want) < REL_L2_TOL
+
+
+def test_matvec_longest_row_and_beyond(rk, oracle):
+    """The activation image, the table and two rows of partial sums must fit in 160 KiB of LDS: n = 32768 does,
+    n = 65536 is refused with a status, not a fault."""
+    S, m = 8, 32
+    for n, ok in ((32768, True), (65536, False)):
+        comp = rand_codes(m * n // 16, seed=81)
+        cb = rand_half(2 << S, seed=82)
+        x = rand_half(n, seed=83)
+        out = torch.zeros((m,), dtype=torch.float16, device="cuda")
+        c = comp.cuda().reshape(n // 2048, m, 128)
+        if ok:
+            rk.decompress_matvec_16_8_1(c, cb.cuda(), x.cuda(), out)
+            want = oracle.matvec(np_u32(comp), np_f16(cb), np_f16(x), m, S, mode=0)
+            assert rel_l2(np_f16(out), want) < REL_L2_TOL
+        else:
+            with pytest.raises(RuntimeError, match="exceeds"):
+                rk.decompress_matvec_16_8_1(c, cb.cuda(), x.cuda(), out)
+
+
 def test_matvec_t_rejects_bad_arguments(rk):
     cb = torch.zeros(65536, dtype=torch.float16, device="cuda")
     comp = torch.zeros(256 * 64 // 16, dtype=torch.int32, device="cuda")
