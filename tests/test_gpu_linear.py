@@ -305,7 +305,8 @@ def test_matvec_rmsnorm_rejects_aliases_and_long_vectors(rk):
         rk.decompress_matvec_rmsnorm(comp2, cb, x2, None, x2.clone(), torch.empty_like(x2), out)
 
 
-@pytest.mark.parametrize("heads,hd,max_len,pos", [(4, 64, 128, 0), (4, 64, 128, 77), (32, 128, 1024, 640), (2, 16, 64, 63)])
+@pytest.mark.parametrize("heads,hd,max_len,pos", [(4, 64, 128, 0), (4, 64, 128, 77), (32, 128, 1024, 640), (2, 16, 64, 63),
+                                                 (256, 16, 32, 20), (64, 128, 2048, 2047), (3, 256, 48, 5)])
 def test_rope_attn_decode_equals_rope_then_attention(rk, heads, hd, max_len, pos):
     import ctypes
     lib = rk.library()
