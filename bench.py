@@ -316,8 +316,11 @@ def bench_other_ops(a):
     outs = [torch.empty((m, n), dtype=torch.float16, device="cuda") for _ in range(8)]
     us = _graph_time_us(lambda k: rk.decompress(comps[k % 8], cb16, outs[k % 8]), steps)
     byts = m * n // 4 + 2 * m * n
+    # the floor of a write-bound op of this size: the framework's fill of the same output buffers
+    fill_us = _graph_time_us(lambda k: outs[k % 8].fill_(1.0), steps)
     res["decompress 4096x4096"] = {"us": round(us, 2), "bytes": byts, "GBps": round(byts / us / 1e3, 1),
-                                   "frac_hbm": round(byts / us / 1e3 / HBM_PEAK_GBS, 4)}
+                                   "frac_hbm": round(byts / us / 1e3 / HBM_PEAK_GBS, 4),
+                                   "fill_of_the_output_us": round(fill_us, 2)}
     # transposed mat-vec, both carry modes
     for (m, n) in ((4096, 4096), (11008, 4096)):
         streams = [rand_words(m * n // 16) for _ in range(16)]
