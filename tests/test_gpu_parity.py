@@ -206,10 +206,11 @@ def test_matvec_full_size(rk, oracle, m, n):
 
 
 @pytest.mark.parametrize("mode", MODES)
-@pytest.mark.parametrize("m,n", [(8192, 28672), (8192, 28672 + 192)])
+@pytest.mark.parametrize("m,n", [(8192, 28672), (8192, 28672 + 192), (28672, 8192), (8192, 8192)])
 def test_matvec_long_rows(rk, oracle, mode, m, n):
-    """Rows so long that a CU's share of them needs the compact partial-sum layout (one sum per row and
-    slab); the product must still match the double-precision product of the bit-exact dense matrix."""
+    """The Llama-3-70B layer shapes.  At n = 28672 the rows are so long that a CU's share of them needs the
+    compact partial-sum layout (one sum per row and slab); the product must still match the double-precision
+    product of the bit-exact dense matrix."""
     S = 8
     comp = rand_codes(m * n // 16, seed=52)
     cb = rand_half(2 << S, seed=53)
@@ -220,7 +221,7 @@ def test_matvec_long_rows(rk, oracle, mode, m, n):
         matvec_fn(rk, 16, S)(c, cb.cuda(), x.cuda(), out)
         W = torch.zeros((m, n), dtype=torch.float16, device="cuda")
         rk.matvec_dense(comp.cuda(), cb.cuda(), W, S)
-    y_dense = (W.double() @ x.cuda().double()).cpu().numpy()
+    y_dense = torch.cat([W[r0:r0 + 4096].double() @ x.cuda().double() for r0 in range(0, m, 4096)]).cpu().numpy()
     assert rel_l2(np_f16(out), y_dense) < REL_L2_TOL
     # the dense export is held to the oracle on the first rows (the whole matrix at this size takes the CPU a while)
     rows = 64
@@ -498,6 +499,26 @@ def test_matmul_bits_full_size_equals_the_mat_vec(rk, bits):
         y = torch.zeros(m, dtype=torch.float16, device="cuda")
         rk.decompress_matvec_bits(comp, cb, x[b].contiguous(), y, bits)
         assert rel_l2(np_f16(out[b]), np_f16(y).astype(np.float64)) < REL_L2_TOL
+
+
+@pytest.mark.parametrize("m,n", [(8192, 8192), (28672, 8192), (8192, 28672)])
+def test_matmul_70b_shapes_batch_16(rk, m, n):
+    """Batch 16 on the Llama-3-70B layer shapes (several row groups per slab, up to 14 slabs to merge) against
+    the double-precision product of the exported dense matrix."""
+    S, batch = 8, 16
+    comp = rand_codes(m * n // 16, seed=91).cuda()
+    cb = rand_half(2 << S, seed=92).cuda()
+    x = rand_half(batch * n, seed=93).reshape(batch, n).cuda()
+    out = torch.full((batch, m), float("nan"), dtype=torch.float16, device="cuda")
+    rk.decompress_matmul_16_8_1(comp, cb, x, out)
+    W = torch.zeros((m, n), dtype=torch.float16, device="cuda")
+    rk.matvec_dense(comp, cb, W, S)
+    want = torch.cat([x.double() @ W[r0:r0 + 4096].double().t() for r0 in range(0, m, 4096)], dim=1)
+    assert rel_l2(np_f16(out), want.cpu().numpy()) < REL_L2_TOL
+    # twice in a row: the arrival counters must be back at zero after a call
+    out2 = torch.full_like(out, float("nan"))
+    rk.decompress_matmul_16_8_1(comp, cb, x, out2)
+    assert torch.equal(out.view(torch.int16), out2.view(torch.int16))
 
 
 @pytest.mark.parametrize("batch", [8, 16, 32])
