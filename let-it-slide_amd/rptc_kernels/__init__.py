@@ -18,6 +18,14 @@ Differences from the reference, all deliberate:
   ``set_timing(False)`` makes every op asynchronous and return 0.0.
 * ``decompress_matvec_*`` accumulates in fp32 and accepts any row count and any ``n % 64 == 0``
   (a ragged last slab); ``decompress_matvec_t_*`` accepts any row count.
+
+Beside the seven: ``matvec_dense`` / ``matvec_t_dense`` / ``matvec_bits_dense`` (the dense fp16 matrix
+a stream stands for), ``decompress_matmul_16_{6,8}_1`` and ``decompress_matmul_bits`` (batch 1..32 on
+the matrix cores), ``decompress_matvec_bits`` (2, 3, 4 bits per weight), ``decompress_matvec_silu`` and
+``decompress_matvec_rmsnorm`` (the mat-vec with a decoder layer's element-wise step in its prologue),
+``sign_hadamard``.  Sub-modules: ``packing`` (symbols -> streams), ``quantize`` (Viterbi search),
+``linear`` (``QuantizedLinear``, ``patch_model``), ``llama_decode`` (a Llama-shaped decode loop),
+``eval_ppl`` (perplexity on a token file).
 """
 import ctypes
 import os
