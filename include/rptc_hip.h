@@ -201,10 +201,16 @@ int rptc_rope_attn_decode(const uint16_t *qkv, const uint16_t *cos_t, const uint
  *   rptc_decompress_matvec_rmsnorm  r = x_in + delta (delta may be NULL); x_out = r;
  *                                   activations = r * rsqrt(mean(r^2) + eps) * weight; n <= 16384;
  *                                   x_out must not be x_in or delta (RPTC_EALIAS)
+ *   rptc_decompress_matvec_hadamard activations = H_P (signs .* x) / sqrt(P) per block of P elements: the
+ *                                   forward transform of rptc_sign_hadamard (block = 0: the largest power
+ *                                   of two dividing n); n <= 15360
  */
 int rptc_decompress_matvec_silu(const int32_t *compressed, const uint16_t *codebook, const uint16_t *gate_up,
                                 uint16_t *out, int64_t m, int64_t n, int S, int carry_mode, void *stream,
                                 float *ms);
+int rptc_decompress_matvec_hadamard(const int32_t *compressed, const uint16_t *codebook, const uint16_t *x,
+                                    const uint16_t *signs, uint16_t *out, int64_t m, int64_t n, int64_t block,
+                                    int S, int carry_mode, void *stream, float *ms);
 int rptc_decompress_matvec_rmsnorm(const int32_t *compressed, const uint16_t *codebook, const uint16_t *x_in,
                                    const uint16_t *delta, const uint16_t *weight, uint16_t *x_out, uint16_t *out,
                                    int64_t m, int64_t n, float eps, int S, int carry_mode, void *stream,

@@ -14,43 +14,14 @@
 // a 16-point transform in registers and scatters them back, so a 4096-point block needs three
 // passes and two barriers instead of twelve.  The op moves 4 bytes per element (fp16 in, fp16
 // out): HBM-bound, LDS traffic is local.
-#include "rptc_common.hpp"
+#include "hadamard_pass.hpp"
 
 namespace rptc {
 
 constexpr int kHadThreads = 256;
 constexpr int kHadMaxBlock = 32768;       // 132 KiB of fp32 in LDS (with padding)
 
-// Element i of the block lives at buf[pad(i)]: one unused float after every 32 keeps the 16-point
-// gathers (lane stride 16 floats in the first pass) off the same LDS bank.
-__device__ __forceinline__ int pad(int i) { return i + (i >> 5); }
-
-// stages s .. s+R_LOG-1 of the transform on the block in buf
-template <int R_LOG>
-__device__ __forceinline__ void hadamard_pass(float *buf, int P, int s, int tid)
-{
-    constexpr int R = 1 << R_LOG;
-    const int low_mask = (1 << s) - 1;
-    for (int grp = tid; grp < (P >> R_LOG); grp += kHadThreads) {
-        const int base = ((grp >> s) << (s + R_LOG)) | (grp & low_mask);
-        float v[R];
-#pragma unroll
-        for (int k = 0; k < R; k++) v[k] = buf[pad(base + (k << s))];
-#pragma unroll
-        for (int h = 1; h < R; h <<= 1) {
-#pragma unroll
-            for (int k = 0; k < R; k++) {
-                if ((k & h) == 0) {
-                    const float a = v[k], b = v[k | h];
-                    v[k] = a + b;
-                    v[k | h] = a - b;
-                }
-            }
-        }
-#pragma unroll
-        for (int k = 0; k < R; k++) buf[pad(base + (k << s))] = v[k];
-    }
-}
+__device__ __forceinline__ int pad(int i) { return had_pad(i); }
 
 __global__ __launch_bounds__(kHadThreads) void sign_hadamard_kernel(
     const uint16_t *__restrict__ x, const uint16_t *__restrict__ signs, uint16_t *__restrict__ out,
@@ -98,16 +69,7 @@ __global__ __launch_bounds__(kHadThreads) void sign_hadamard_kernel(
         }
     }
     __syncthreads();
-    int stage = 0;
-    for (; stage + 4 <= log_p; stage += 4) {
-        hadamard_pass<4>(buf, P, stage, tid);
-        __syncthreads();
-    }
-    const int rest = log_p - stage;
-    if (rest == 3) hadamard_pass<3>(buf, P, stage, tid);
-    else if (rest == 2) hadamard_pass<2>(buf, P, stage, tid);
-    else if (rest == 1) hadamard_pass<1>(buf, P, stage, tid);
-    if (rest) __syncthreads();
+    hadamard_stages<kHadThreads>(buf, P, log_p, tid);
     const float scale = rsqrtf((float)P);
     if (wide) {
         const uint4 *s4 = reinterpret_cast<const uint4 *>(s);

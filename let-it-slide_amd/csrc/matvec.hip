@@ -23,6 +23,7 @@
 //     wait for are issued first and every wave's stream loads right behind them, before the
 //     table is built; kernel arguments are preloaded into SGPRs.
 #include "decode_asm.hpp"
+#include "hadamard_pass.hpp"
 #include "rptc_common.hpp"
 
 // Development hook: a probe build defines RPTC_STAMP to record a per-wave timestamp at each phase.
@@ -155,14 +156,17 @@ struct MatvecArgs {
 // activations are silu(gate) * up.  AddRmsNorm: r = x (+ x2), activations = r * rsqrt(mean(r^2) +
 // eps) * norm_w, and workgroup 0 writes r to x_out: the element-wise step that precedes a
 // projection in a decoder layer, done while the stream loads are in flight instead of in a
-// kernel of its own.  The fp16 roundings are those of the stand-alone kernels (decode_glue.hip).
-constexpr int kXPlain = 0, kXSiluMul = 1, kXAddRmsNorm = 2;
+// kernel of its own.  SignHadamard: activations = H_P (x2 .* x) / sqrt(P) per block of P = 2^log_p
+// elements, x2 the +-1 signs: the incoherence transform of hadamard.hip, same passes, same order.
+// The fp16 roundings are those of the stand-alone kernels (decode_glue.hip, hadamard.hip).
+constexpr int kXPlain = 0, kXSiluMul = 1, kXAddRmsNorm = 2, kXSignHadamard = 3;
 
 struct XFuse {
     const uint4 *x2;       // AddRmsNorm: the residual delta, or null
     const uint4 *norm_w;   // AddRmsNorm: the norm's weight
     uint4 *x_out;          // AddRmsNorm: the updated residual stream (must not alias x or x2)
     float eps;
+    int log_p;             // SignHadamard: log2 of the block length
 };
 
 struct Halves8 {
@@ -252,6 +256,13 @@ __device__ __forceinline__ void matvec_body(
         for (int u = 0; u < kXRegs; u++) {
             const int idx = tid + u * kMatvecThreads;
             xv2[u] = idx < n8 ? x[n8 + idx] : make_uint4(0, 0, 0, 0);
+        }
+    }
+    if constexpr (XMODE == kXSignHadamard) {
+#pragma unroll
+        for (int u = 0; u < kXRegs; u++) {
+            const int idx = tid + u * kMatvecThreads;
+            xv2[u] = idx < n8 ? fuse.x2[idx] : make_uint4(0, 0, 0, 0);
         }
     }
     if constexpr (XMODE == kXAddRmsNorm) {
@@ -358,6 +369,34 @@ __device__ __forceinline__ void matvec_body(
 #pragma unroll
             for (int i = 0; i < 8; i++) r[u].v[i] = round_half(r[u].v[i] * inv) * w8.v[i];
             xv[u] = pack8(r[u]);
+        }
+    }
+
+    if constexpr (XMODE == kXSignHadamard) {
+        // the signed vector as fp32 behind the partial sums (the host sized LDS for it), the passes of
+        // the stand-alone transform over all blocks at once, then back to fp16 in the registers the
+        // staging below expects (n8 <= kXRegs * kMatvecThreads is guaranteed by the host)
+        float *hb = part + a.rows_per_block * pstride;
+        auto signed8 = [&](int idx, const uint4 xq, const uint4 sq) {
+            const Halves8 xs = unpack8(xq), ss = unpack8(sq);
+#pragma unroll
+            for (int k = 0; k < 8; k++) hb[had_pad(8 * idx + k)] = xs.v[k] * ss.v[k];
+        };
+#pragma unroll
+        for (int u = 0; u < kXRegs; u++) {
+            const int idx = tid + u * kMatvecThreads;
+            if (idx < n8) signed8(idx, xv[u], xv2[u]);
+        }
+        __syncthreads();
+        hadamard_stages<kMatvecThreads>(hb, n, fuse.log_p, tid);
+        const float scale = rsqrtf((float)(1 << fuse.log_p));
+#pragma unroll
+        for (int u = 0; u < kXRegs; u++) {
+            const int idx = tid + u * kMatvecThreads;
+            Halves8 r;
+#pragma unroll
+            for (int k = 0; k < 8; k++) r.v[k] = idx < n8 ? hb[had_pad(8 * idx + k)] * scale : 0.f;
+            xv[u] = pack8(r);
         }
     }
 
@@ -474,7 +513,7 @@ __global__ __launch_bounds__(kMatvecThreads) void matvec_kernel(
 {
     // separate scalar arguments (not a struct) so that all of them are preloaded into SGPRs
     const MatvecArgs a = {arg_m, arg_n, arg_rows_per_block, arg_rw_tail, arg_items_full, arg_items_tail};
-    matvec_body<S, MODE, BITS, kXPlain, COMPACT>(comp, codebook, x, out, a, XFuse{nullptr, nullptr, nullptr, 0.f});
+    matvec_body<S, MODE, BITS, kXPlain, COMPACT>(comp, codebook, x, out, a, XFuse{nullptr, nullptr, nullptr, 0.f, 0});
 }
 
 // 2 bits per weight with an element-wise step fused in front (XMODE above)
@@ -483,10 +522,10 @@ __global__ __launch_bounds__(kMatvecThreads) void matvec_fused_kernel(
     const uint32_t *__restrict__ comp, const uint32_t *__restrict__ codebook,
     const uint4 *__restrict__ x, uint16_t *__restrict__ out, int arg_m, int arg_n, int arg_rows_per_block,
     int arg_rw_tail, int arg_items_full, int arg_items_tail, const uint4 *x2, const uint4 *norm_w, uint4 *x_out,
-    float eps)
+    float eps, int log_p)
 {
     const MatvecArgs a = {arg_m, arg_n, arg_rows_per_block, arg_rw_tail, arg_items_full, arg_items_tail};
-    matvec_body<S, MODE, 2, XMODE, COMPACT>(comp, codebook, x, out, a, XFuse{x2, norm_w, x_out, eps});
+    matvec_body<S, MODE, 2, XMODE, COMPACT>(comp, codebook, x, out, a, XFuse{x2, norm_w, x_out, eps, log_p});
 }
 
 // Dense export: one thread per stream element, 32 pairs scattered to their columns.
@@ -537,8 +576,8 @@ static int matvec_lds_bytes(int n, int rows_per_block, bool compact)
 
 // Argument checks and launch geometry shared by every mat-vec entry point.
 static int plan_matvec(const void *compressed, const void *codebook, const void *x, const void *out, int64_t m,
-                       int64_t n, int carry_mode, bool allow_compact, DeviceInfo **dev, MatvecArgs *a, bool *compact,
-                       int *lds_bytes, int *grid)
+                       int64_t n, int carry_mode, bool allow_compact, int extra_lds_bytes, DeviceInfo **dev,
+                       MatvecArgs *a, bool *compact, int *lds_bytes, int *grid)
 {
     if (!compressed || !codebook || !x || !out) return RPTC_ENULL;
     if (m < 1 || n < 64 || n % 64 != 0) return RPTC_ESHAPE;
@@ -553,8 +592,8 @@ static int plan_matvec(const void *compressed, const void *codebook, const void 
     a->m = (int)m;
     a->n = (int)n;
     a->rows_per_block = 2 * (int)((m + 2 * (*dev)->cus - 1) / (2 * (*dev)->cus));
-    *compact = allow_compact && matvec_lds_bytes(a->n, a->rows_per_block, false) > kMaxLds;
-    const int fixed_bytes = matvec_lds_bytes(a->n, 0, *compact);
+    *compact = allow_compact && matvec_lds_bytes(a->n, a->rows_per_block, false) + extra_lds_bytes > kMaxLds;
+    const int fixed_bytes = matvec_lds_bytes(a->n, 0, *compact) + extra_lds_bytes;
     const int row_bytes = 4 * matvec_part_stride(a->n, *compact);
     if (fixed_bytes + 2 * row_bytes > kMaxLds) return RPTC_ELIMIT;
     const int fit_rows = ((kMaxLds - fixed_bytes) / row_bytes) & ~1;
@@ -563,7 +602,7 @@ static int plan_matvec(const void *compressed, const void *codebook, const void 
     a->rw_tail = lt ? 64 / lt : 1;
     a->items_full = a->rows_per_block / 2;
     a->items_tail = lt ? (a->rows_per_block + a->rw_tail - 1) / a->rw_tail : 0;
-    *lds_bytes = matvec_lds_bytes(a->n, a->rows_per_block, *compact);
+    *lds_bytes = matvec_lds_bytes(a->n, a->rows_per_block, *compact) + extra_lds_bytes;
     *grid = (int)((m + a->rows_per_block - 1) / a->rows_per_block);
     return 0;
 }
@@ -576,7 +615,7 @@ static int launch_matvec(const int32_t *compressed, const uint16_t *codebook, co
     MatvecArgs a;
     int lds_bytes, grid;
     bool compact;
-    int rc = plan_matvec(compressed, codebook, x, out, m, n, carry_mode, BITS == 2, &dev, &a, &compact, &lds_bytes, &grid);
+    int rc = plan_matvec(compressed, codebook, x, out, m, n, carry_mode, BITS == 2, 0, &dev, &a, &compact, &lds_bytes, &grid);
     if (rc) return rc;
     hipStream_t s = static_cast<hipStream_t>(stream);
     Timer t;
@@ -603,16 +642,18 @@ static int launch_matvec(const int32_t *compressed, const uint16_t *codebook, co
 
 template <int S, int XMODE>
 static int launch_matvec_fused(const int32_t *compressed, const uint16_t *codebook, const uint16_t *x,
-                               const uint16_t *x2, const uint16_t *norm_w, uint16_t *x_out, float eps, uint16_t *out,
-                               int64_t m, int64_t n, int carry_mode, void *stream, float *ms)
+                               const uint16_t *x2, const uint16_t *norm_w, uint16_t *x_out, float eps, int log_p,
+                               uint16_t *out, int64_t m, int64_t n, int carry_mode, void *stream, float *ms)
 {
     DeviceInfo *dev;
     MatvecArgs a;
     int lds_bytes, grid;
     bool compact;
-    // the norm variant holds the whole vector in registers (n <= 16384): never long enough to need compact sums
-    int rc = plan_matvec(compressed, codebook, x, out, m, n, carry_mode, XMODE == kXSiluMul, &dev, &a, &compact, &lds_bytes,
-                         &grid);
+    // The norm and Hadamard variants hold the whole vector in registers (n <= 16384): never long enough
+    // to need compact sums.  The Hadamard variant keeps the vector as padded fp32 behind the partial sums.
+    const int extra = XMODE == kXSignHadamard ? (int)(n + n / 32 + 1) * 4 : 0;
+    int rc = plan_matvec(compressed, codebook, x, out, m, n, carry_mode, XMODE == kXSiluMul, extra, &dev, &a, &compact,
+                         &lds_bytes, &grid);
     if (rc) return rc;
     hipStream_t s = static_cast<hipStream_t>(stream);
     Timer t;
@@ -627,7 +668,7 @@ static int launch_matvec_fused(const int32_t *compressed, const uint16_t *codebo
 #define RPTC_LAUNCH(MODE, COMPACT)                                                                                  \
     hipLaunchKernelGGL((matvec_fused_kernel<S, MODE, XMODE, COMPACT>), dim3(grid), dim3(kMatvecThreads), lds_bytes, \
                        s, a_comp, a_cb, a_x, out, a.m, a.n, a.rows_per_block, a.rw_tail, a.items_full, a.items_tail, \
-                       a_x2, a_w, a_xo, eps)
+                       a_x2, a_w, a_xo, eps, log_p)
     if constexpr (XMODE == kXSiluMul) {
         if (compact) {
             if (carry_mode == RPTC_AS_WRITTEN) RPTC_LAUNCH(RPTC_AS_WRITTEN, true);
@@ -733,6 +774,7 @@ int prepare_matvec()
     RPTC_SET_LIMITS(kXSiluMul, false)
     RPTC_SET_LIMITS(kXSiluMul, true)
     RPTC_SET_LIMITS(kXAddRmsNorm, false)
+    RPTC_SET_LIMITS(kXSignHadamard, false)
 #undef RPTC_SET_LIMITS
     return 0;
 }
@@ -769,8 +811,8 @@ extern "C" int rptc_decompress_matvec_silu(const int32_t *c, const uint16_t *cb,
                                            int64_t m, int64_t n, int S, int mode, void *stream, float *ms)
 {
     if (S != 6 && S != 8) return RPTC_ESHAPE;
-    return S == 6 ? launch_matvec_fused<6, kXSiluMul>(c, cb, gate_up, nullptr, nullptr, nullptr, 0.f, out, m, n, mode, stream, ms)
-                  : launch_matvec_fused<8, kXSiluMul>(c, cb, gate_up, nullptr, nullptr, nullptr, 0.f, out, m, n, mode, stream, ms);
+    return S == 6 ? launch_matvec_fused<6, kXSiluMul>(c, cb, gate_up, nullptr, nullptr, nullptr, 0.f, 0, out, m, n, mode, stream, ms)
+                  : launch_matvec_fused<8, kXSiluMul>(c, cb, gate_up, nullptr, nullptr, nullptr, 0.f, 0, out, m, n, mode, stream, ms);
 }
 
 extern "C" int rptc_decompress_matvec_rmsnorm(const int32_t *c, const uint16_t *cb, const uint16_t *x_in,
@@ -784,8 +826,29 @@ extern "C" int rptc_decompress_matvec_rmsnorm(const int32_t *c, const uint16_t *
     if (x_out == x_in || x_out == delta) return RPTC_EALIAS;
     if (!aligned16(delta) || !aligned16(weight) || !aligned16(x_out)) return RPTC_EALIGN;
     if (n > 8 * 2 * kMatvecThreads) return RPTC_ELIMIT;      // the whole vector sits in two registers per thread
-    return S == 6 ? launch_matvec_fused<6, kXAddRmsNorm>(c, cb, x_in, delta, weight, x_out, eps, out, m, n, mode, stream, ms)
-                  : launch_matvec_fused<8, kXAddRmsNorm>(c, cb, x_in, delta, weight, x_out, eps, out, m, n, mode, stream, ms);
+    return S == 6 ? launch_matvec_fused<6, kXAddRmsNorm>(c, cb, x_in, delta, weight, x_out, eps, 0, out, m, n, mode, stream, ms)
+                  : launch_matvec_fused<8, kXAddRmsNorm>(c, cb, x_in, delta, weight, x_out, eps, 0, out, m, n, mode, stream, ms);
+}
+
+extern "C" int rptc_decompress_matvec_hadamard(const int32_t *c, const uint16_t *cb, const uint16_t *x,
+                                               const uint16_t *signs, uint16_t *out, int64_t m, int64_t n,
+                                               int64_t block, int S, int mode, void *stream, float *ms)
+{
+    if (!signs) return RPTC_ENULL;
+    if (S != 6 && S != 8) return RPTC_ESHAPE;
+    if (n < 64 || n % 64 != 0) return RPTC_ESHAPE;
+    if (n > 15360) return RPTC_ELIMIT;                       // table + fp16 image + padded fp32 copy must fit in LDS
+    int64_t P = block;
+    if (P == 0) {                                            // the largest power of two that divides n
+        P = 1;
+        while (n % (2 * P) == 0) P *= 2;
+    }
+    if (P < 2 || (P & (P - 1)) != 0 || n % P != 0) return RPTC_ESHAPE;
+    if (!aligned16(signs)) return RPTC_EALIGN;
+    int log_p = 0;
+    while (((int64_t)1 << log_p) < P) log_p++;
+    return S == 6 ? launch_matvec_fused<6, kXSignHadamard>(c, cb, x, signs, nullptr, nullptr, 0.f, log_p, out, m, n, mode, stream, ms)
+                  : launch_matvec_fused<8, kXSignHadamard>(c, cb, x, signs, nullptr, nullptr, 0.f, log_p, out, m, n, mode, stream, ms);
 }
 
 extern "C" int rptc_matvec_dense(const int32_t *compressed, const uint16_t *codebook, uint16_t *W, int64_t m,

@@ -23,6 +23,7 @@ Beside the seven: ``matvec_dense`` / ``matvec_t_dense`` / ``matvec_bits_dense`` 
 a stream stands for), ``decompress_matmul_16_{6,8}_1`` and ``decompress_matmul_bits`` (batch 1..32 on
 the matrix cores), ``decompress_matvec_bits`` (2, 3, 4 bits per weight), ``decompress_matvec_silu`` and
 ``decompress_matvec_rmsnorm`` (the mat-vec with a decoder layer's element-wise step in its prologue),
+``decompress_matvec_hadamard`` (with the sign-Hadamard transform of its activations in its prologue),
 ``sign_hadamard``.  Sub-modules: ``packing`` (symbols -> streams), ``quantize`` (Viterbi search),
 ``linear`` (``QuantizedLinear``, ``patch_model``), ``llama_decode`` (a Llama-shaped decode loop),
 ``eval_ppl`` (perplexity on a token file).
@@ -72,6 +73,7 @@ _SIGNATURES = {
     "rptc_probe_read": ([_VP, _I64, _VP, _VP], _INT),
     "rptc_rope_attn_decode": ([_VP, _VP, _VP, _VP, _VP, _VP, _VP, _I64, _I64, _I64, _VP], _INT),
     "rptc_decompress_matvec_silu": ([_VP, _VP, _VP, _VP, _I64, _I64, _INT, _INT, _VP, _FP], _INT),
+    "rptc_decompress_matvec_hadamard": ([_VP, _VP, _VP, _VP, _VP, _I64, _I64, _I64, _INT, _INT, _VP, _FP], _INT),
     "rptc_decompress_matvec_rmsnorm": ([_VP, _VP, _VP, _VP, _VP, _VP, _VP, _I64, _I64, ctypes.c_float, _INT, _INT,
                                         _VP, _FP], _INT),
 }
@@ -417,6 +419,18 @@ def decompress_matvec_silu(compressed, codebook, gate_up, out):
     n = gate_up.size(0) // 2
     m, S = _fused_common(compressed, codebook, out, n)
     return _call(library().rptc_decompress_matvec_silu, (compressed, codebook, gate_up, out), m, n, S)
+
+
+def decompress_matvec_hadamard(compressed, codebook, x, signs, out, block=0):
+    """out = W (H (signs * x) / sqrt(block)): ``decompress_matvec_16_{S}_1`` with the forward ``sign_hadamard``
+    of its activations computed inside the kernel (x and signs fp16 [n], n <= 15360; block = 0: the largest
+    power of two dividing n).  Returns elapsed ms."""
+    for t, name in ((x, "x"), (signs, "signs")):
+        _check_input(t, name)
+        _check(t.dim() == 1 and t.dtype == torch.float16 and t.size(0) == x.size(0), f"{name} must be fp16 [n]")
+    n = x.size(0)
+    m, S = _fused_common(compressed, codebook, out, n)
+    return _call(library().rptc_decompress_matvec_hadamard, (compressed, codebook, x, signs, out), m, n, block, S)
 
 
 def decompress_matvec_rmsnorm(compressed, codebook, x_in, delta, weight, x_out, out, eps=1e-5):

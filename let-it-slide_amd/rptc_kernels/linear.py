@@ -130,6 +130,16 @@ class QuantizedLinear(torch.nn.Module):
         shape = x.shape
         x2 = x.reshape(-1, self.in_features).contiguous()
         xs = x2 * self.scales_in if self.scales_in is not None else x2
+        if self.signs is not None and xs.size(0) == 1 and self.bits == 2 and self.in_features <= 15360:
+            # one token: the transform runs in the prologue of the mat-vec
+            y = torch.empty((1, self.out_features), dtype=torch.float16, device=xs.device)
+            prev = rk.set_timing(False)
+            try:
+                rk._call(rk.library().rptc_decompress_matvec_hadamard, (self.compressed, self.codebook, xs, self.signs, y),
+                         self.out_features, self.in_features, 0, self.S, carry_mode=self.carry_mode)
+            finally:
+                rk.set_timing(prev)
+            return self._epilogue(y, x2, shape)
         if self.signs is not None:
             t = torch.empty_like(xs)
             prev = rk.set_timing(False)
@@ -143,6 +153,9 @@ class QuantizedLinear(torch.nn.Module):
             y = self._product(xs)
         finally:
             rk.set_timing(prev)
+        return self._epilogue(y, x2, shape)
+
+    def _epilogue(self, y, x2, shape):
         if self.scales_out is not None:
             y = y * self.scales_out
         if self.biases_out is not None:

@@ -80,6 +80,8 @@ def test_c_abi_rejects_bad_arguments_before_touching_a_device():
     assert lib.rptc_decompress_matvec_rmsnorm(16, 16, 32, None, 48, 32, 64, 32, 2048, 1e-5, 8, 0, None, None) == -7   # x_out is x_in
     assert lib.rptc_decompress_matvec_rmsnorm(16, 16, 32, None, 48, 64, 80, 32, 32768, 1e-5, 8, 0, None, None) == -5  # n > 16384
     assert lib.rptc_sign_hadamard(16, 16, 16, 1, 4096, 48, 0, None, None) == -2                  # block not a power of two
+    assert lib.rptc_decompress_matvec_hadamard(16, 16, 16, 16, 16, 32, 4096, 48, 8, 0, None, None) == -2   # block
+    assert lib.rptc_decompress_matvec_hadamard(16, 16, 16, 16, 16, 32, 16384, 0, 8, 0, None, None) == -5   # n > 15360
     assert lib.rptc_rope_attn_decode(16, 16, 16, 16, 16, 16, 16, 4, 48, 128, None) == -2         # head_dim not a power of two
     assert lib.rptc_attn_decode(16, 16, 16, None, 16, 4, 64, 128, None) == -1
     assert lib.rptc_probe_read(16, 100, None, None) == -2

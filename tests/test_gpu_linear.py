@@ -289,6 +289,40 @@ def test_matvec_rmsnorm_equals_norm_then_matvec(rk, mode, with_delta, m, n):
     assert rel_l2(got.float().cpu().numpy(), want.float().cpu().numpy()) < 1e-3
 
 
+@pytest.mark.parametrize("mode", [0, 1])
+@pytest.mark.parametrize("m,n,block", [(64, 4096, 0), (33, 11008, 0), (40, 2048 + 192, 0), (32, 8192, 0), (24, 14336, 0), (64, 4096, 256),
+                                       (16, 64, 0)])
+def test_matvec_hadamard_equals_transform_then_matvec(rk, mode, m, n, block):
+    """The butterflies are the stand-alone kernel's, in the same order, so the fused call is bit-identical."""
+    S = 8
+    comp, cb = _stream(m, n, S, seed=7)
+    x = rand_half(n, seed=51).cuda()
+    signs = torch.where(torch.rand(n, generator=torch.Generator().manual_seed(52)) < 0.5, -1.0, 1.0).half().cuda()
+    t = torch.empty_like(x)
+    rk.sign_hadamard(x, signs, t, block=block)
+    want = torch.full((m,), float("nan"), dtype=torch.float16, device="cuda")
+    got = torch.full((m,), float("nan"), dtype=torch.float16, device="cuda")
+    prev = rk.set_carry_mode(mode)
+    try:
+        getattr(rk, f"decompress_matvec_16_{S}_1")(comp.reshape(n // 2048, m, 128) if n % 2048 == 0 else comp, cb, t, want)
+        ms = rk.decompress_matvec_hadamard(comp, cb, x, signs, got, block=block)
+    finally:
+        rk.set_carry_mode(prev)
+    assert ms > 0
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+    with pytest.raises(RuntimeError):
+        rk.decompress_matvec_hadamard(comp, cb, x, signs, got, block=48)
+
+
+def test_matvec_hadamard_refuses_vectors_that_do_not_fit_in_lds(rk):
+    m, n = 32, 16384
+    comp, cb = _stream(m, n, 8, seed=11)
+    x = rand_half(n, seed=3).cuda()
+    out = torch.empty(m, dtype=torch.float16, device="cuda")
+    with pytest.raises(RuntimeError, match="exceeds"):
+        rk.decompress_matvec_hadamard(comp, cb, x, torch.ones_like(x), out)
+
+
 def test_matvec_rmsnorm_rejects_aliases_and_long_vectors(rk):
     m, n = 32, 2048
     comp, cb = _stream(m, n, 8, seed=9)
