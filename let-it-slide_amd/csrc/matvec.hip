@@ -300,14 +300,21 @@ __device__ __forceinline__ void matvec_body(
     // cursor of the loads and cursor of the decode (slab, item index inside the slab)
     int ld_slab = first_slab, ld_idx = first_idx;
     SlabView ld = view(ld_slab);
-    Elem<WORDS> buf[kBatch];
-    uint32_t cw[kBatch];
-    auto load_batch = [&](int base) {
+    // Two register sets of kBatch elements each: one is decoded while the loads of the other are in
+    // flight.  A lane with nothing to load keeps what it has: such a lane belongs to a row past
+    // the block's last one, and nothing it computes is written.
+    Elem<WORDS> buf_a[kBatch], buf_b[kBatch];
+    uint32_t cw_a[kBatch], cw_b[kBatch];
+#pragma unroll
+    for (int u = 0; u < kBatch; u++) {
+#pragma unroll
+        for (int i = 0; i < WORDS; i++) buf_a[u].w[i] = buf_b[u].w[i] = 0;
+        cw_a[u] = cw_b[u] = 0;
+    }
+    // requests items base .. base + kBatch - 1 (those the wave has) and moves the load cursor on
+    auto load_batch = [&](Elem<WORDS> (&buf)[kBatch], uint32_t (&cw)[kBatch], int base) {
 #pragma unroll
         for (int u = 0; u < kBatch; u++) {
-#pragma unroll
-            for (int i = 0; i < WORDS; i++) buf[u].w[i] = 0;
-            cw[u] = 0;
             if (base + u < it_end) {
                 const int row_first = ld_idx * ld.rows_per_item;           // row inside the block
                 const int rows_here = min(ld.rows_per_item, rows - row_first);
@@ -330,7 +337,7 @@ __device__ __forceinline__ void matvec_body(
             }
         }
     };
-    load_batch(it_begin);
+    load_batch(buf_a, cw_a, it_begin);
     RPTC_STAMP(1);
 
     // the element-wise step in front of the product, on the registers the small loads filled
@@ -424,15 +431,8 @@ __device__ __forceinline__ void matvec_body(
     SlabView sv = view(slab);
     int l = 0, sub = 0;                     // this lane's element inside a row, row inside the item
     uint32_t part_lane = 0;                 // LDS byte address of this lane's partial for row 0
-    for (int base = it_begin; base < it_end; base += kBatch) {
-        Elem<WORDS> cur[kBatch];
-        uint32_t ccw[kBatch];
-#pragma unroll
-        for (int u = 0; u < kBatch; u++) {
-            cur[u] = buf[u];
-            ccw[u] = cw[u];
-        }
-        if (base + kBatch < it_end) load_batch(base + kBatch);
+    uint64_t first_lanes = 0;               // the lanes with l == 0
+    auto decode_batch = [&](const Elem<WORDS> (&buf)[kBatch], const uint32_t (&cw)[kBatch], int base) {
 #pragma unroll
         for (int u = 0; u < kBatch; u++) {
             if (base + u >= it_end) break;
@@ -457,34 +457,43 @@ __device__ __forceinline__ void matvec_body(
 #pragma unroll
                     for (int q = 0; q < 32; q++) xr[q] = xp[q * sv.lanes];
                 }
+                first_lanes = __builtin_amdgcn_ballot_w64(l == 0);
                 const int col = COMPACT ? (slab < T ? slab : T + l) : sv.part_off + l;
                 part_lane = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(part)) + 4u * (uint32_t)(sub * pstride + col);
             }
             const int row_first = idx * sv.rows_per_item;
-            const bool active = sub < sv.rows_per_item && row_first + sub < rows;
+            // The lanes whose sum is kept, as a wave-uniform mask: the lanes of the item's rows that
+            // exist (the first `nact` lanes), and of those only the ones holding a row's sum.
+            const int nact = min(sv.rows_per_item, rows - row_first) * sv.lanes;
+            uint64_t keep = nact >= 64 ? ~0ull : (1ull << nact) - 1ull;
             // Previous lane's last word.  Lane 0 of a row keeps its own as written
             // (inference.cu:232: the shuffle hands lane 0 its own value back).
-            const uint32_t last = cur[u].w[WORDS - 1];
-            uint32_t carry = __builtin_amdgcn_update_dpp(0u, last, 0x138 /* wave_shr:1 */, 0xF, 0xF, false);
-            if (l == 0) carry = MODE == RPTC_CONTINUOUS ? ccw[u] : last;
+            const uint32_t last = buf[u].w[WORDS - 1];
+            const uint32_t own = MODE == RPTC_CONTINUOUS ? cw[u] : last;
             float sum;
             if constexpr (BITS == 2) {
-                float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
-                decode_element_asm(make_uint4(cur[u].w[0], cur[u].w[1], cur[u].w[2], cur[u].w[3]), carry, lane4, xr,
-                                   a0, a1, a2, a3);
+                float a0, a1, a2, a3;
+                decode_element_asm(make_uint4(buf[u].w[0], buf[u].w[1], buf[u].w[2], buf[u].w[3]), own, first_lanes,
+                                   lane4, xr, a0, a1, a2, a3);
                 sum = (a0 + a1) + (a2 + a3);
             } else {
-                sum = decode_element_bits<BITS>(cur[u], carry, lane4, xr);
+                uint32_t carry = __builtin_amdgcn_update_dpp(last, last, 0x138 /* wave_shr:1 */, 0xF, 0xF, false);
+                if (l == 0) carry = own;
+                sum = decode_element_bits<BITS>(buf[u], carry, lane4, xr);
             }
-            bool writer = active;
             if (COMPACT && slab < T) {
                 sum = half_wave_sum(sum);        // lanes 31 and 63 hold their row's 32 elements
-                writer = active && l == 31;
+                keep &= 0x8000000080000000ull;
             }
-            if (writer) {
-                typedef __attribute__((address_space(3))) float lds_float;
-                *reinterpret_cast<lds_float *>(static_cast<uintptr_t>(part_lane + 4u * (uint32_t)(row_first * pstride))) = sum;
-            }
+            // the store under the mask: set as the execution mask by hand, which costs no vector op
+            uint64_t saved_exec;
+            asm volatile("s_mov_b64 %[sv], exec\n"
+                         "s_and_b64 exec, exec, %[keep]\n"
+                         "ds_write_b32 %[addr], %[val]\n"
+                         "s_mov_b64 exec, %[sv]"
+                         : [sv] "=&s"(saved_exec)
+                         : [keep] "s"(keep), [addr] "v"(part_lane + 4u * (uint32_t)(row_first * pstride)), [val] "v"(sum)
+                         : "memory");
             if (base + u == it_begin) RPTC_STAMP(3);
             if (++idx == sv.items) {
                 idx = 0;
@@ -492,8 +501,22 @@ __device__ __forceinline__ void matvec_body(
                 sv = view(slab);
             }
         }
+    };
+    // wait for every load in flight, but for no other counter
+    auto loads_done = [] { __builtin_amdgcn_s_waitcnt(0x0F70); };
+    for (int base = it_begin; base < it_end; base += 2 * kBatch) {
+        // The wait stands in front of the next requests: behind them the compiler could only wait
+        // for those as well (it cannot count loads that are issued under a condition).
+        loads_done();
+        load_batch(buf_b, cw_b, base + kBatch);
+        decode_batch(buf_a, cw_a, base);
+        if (base + kBatch >= it_end) break;
+        loads_done();
+        load_batch(buf_a, cw_a, base + 2 * kBatch);
+        decode_batch(buf_b, cw_b, base + kBatch);
     }
     RPTC_STAMP(4);
+    __builtin_amdgcn_s_waitcnt(0);          // the stores above are not the compiler's to wait for
     __syncthreads();
     // one wave per row: add the row's partial sums in a fixed order
     for (int r = wave; r < rows; r += kMatvecWaves) {

@@ -126,8 +126,11 @@ __device__ __forceinline__ float half_wave_sum(float v)
     RPTC_DPP_ADD(0x112, 0xF, 0xF);   // row_shr:2
     RPTC_DPP_ADD(0x114, 0xF, 0xF);   // row_shr:4
     RPTC_DPP_ADD(0x118, 0xF, 0xF);   // row_shr:8
-    RPTC_DPP_ADD(0x142, 0xA, 0xF);   // row_bcast:15 into rows 1 and 3
 #undef RPTC_DPP_ADD
+    // row_bcast:15 into rows 1 and 3 as one instruction (the compiler makes three of it); the nop
+    // is the distance a DPP operand needs from the vector op that wrote it
+    asm("s_nop 1\n"
+        "v_add_f32_dpp %0, %0, %0 row_bcast:15 row_mask:0xa bank_mask:0xf" : "+v"(v));
     return v;
 }
 
