@@ -49,6 +49,7 @@ def parse():
     ap.add_argument("--extra-shapes", action="store_true", help="also time the other layer shapes")
     ap.add_argument("--other-ops", action="store_true",
                     help="time decompress, decompress_matvec_t_16 and sign_hadamard instead (prints its own JSON line)")
+    ap.add_argument("--quantize", action="store_true", help="time the Viterbi search kernel of the quantizer")
     ap.add_argument("--decode", action="store_true",
                     help="greedy decode with a Llama-2-7B-shaped random-init model whose projections are 2-bit streams "
                          "(prompt 512, 128 new tokens, batch 1); prints its own JSON line")
@@ -347,6 +348,68 @@ def bench_other_ops(a):
                       "config": {"launch": "graph", "steps": steps}, "results": res}))
 
 
+def bench_quantize(a):
+    """The Viterbi search kernel (the quantizer's inner loop) on the rows of one 4096 x 4096 layer:
+    trellis state updates per second against the vector-ALU rate that bounds it, with the same search in
+    framework ops on the GPU and the C restatement on the host's cores beside it."""
+    import time
+    import numpy as np
+    import torch
+    import rptc_kernels as rk
+    from rptc_kernels import quantize
+    g = torch.Generator(device="cuda")
+    g.manual_seed(42)
+    cb = torch.randn(512, generator=g, device="cuda").half()
+    rows, steps = 512, 2048                                         # two rows per CU, n = 4096
+    tg = torch.randn((rows, steps, 2), generator=g, device="cuda") * 0.7
+    best = None
+    for _ in range(max(2, min(a.steps, 5))):
+        sym, cost, end, ms = rk.viterbi_pairs(tg, cb)
+        best = ms if best is None else min(best, ms)
+    updates = rows * steps * 65536
+    # vector-ALU ceiling: 256 CUs x 64 lanes x 2.4 GHz lane-ops/s; a state update costs 5 vector ops
+    # (byte permute, add, and compare + two selects in the minimum over predecessors)
+    valu_peak = 256 * 64 * 2.4e9
+    res = {"viterbi_pairs rows 512 steps 2048": {
+        "ms": round(best, 3), "state_updates_per_s": float(f"{updates / best * 1e3:.4e}"),
+        "us_per_step_per_row_round": round(best * 1e3 / steps / (rows / 256), 3),
+        "vector_ops_per_update": 5, "frac_of_valu_peak": round(updates * 5 / (best * 1e-3) / valu_peak, 4)}}
+    # the same search in framework ops on the GPU (64 rows, 256 steps)
+    table = quantize.decode_table(cb, 8)
+    small = tg[:64, :256].contiguous()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    sym_t, cost_t = quantize.viterbi_pairs(small, table)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    sym_h, cost_h, _, _ = rk.viterbi_pairs(small, cb)
+    res["framework ops rows 64 steps 256"] = {"ms": round(dt * 1e3, 2),
+                                              "state_updates_per_s": float(f"{64 * 256 * 65536 / dt:.4e}"),
+                                              "same_path_as_kernel": bool(torch.equal(sym_t, sym_h.long()))}
+    if not a.no_cpu:
+        from oracle import rptc_oracle
+        t_np, c_np = table.cpu().numpy(), small[0, :64].cpu().numpy()
+        t0 = time.perf_counter()
+        osym, ocost, _ = rptc_oracle.viterbi(t_np, 4, c_np)
+        dt = time.perf_counter() - t0
+        res["cpu oracle 1 row 64 steps (1 core)"] = {"ms": round(dt * 1e3, 2),
+                                                     "state_updates_per_s": float(f"{64 * 65536 / dt:.4e}"),
+                                                     }
+        sym_1, _, _, _ = rk.viterbi_pairs(small[:1, :64].contiguous(), cb)
+        res["cpu oracle 1 row 64 steps (1 core)"]["same_path_as_kernel"] = bool(np.array_equal(osym, sym_1[0].cpu().numpy()))
+    # a whole layer through quantize_matrix (search + copies to the host)
+    W = torch.randn((4096, 4096), generator=g, device="cuda") * 0.7
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    _, mse = quantize.quantize_matrix(W, cb, 8)
+    torch.cuda.synchronize()
+    res["quantize_matrix 4096x4096"] = {"s": round(time.perf_counter() - t0, 3), "mse_over_variance": round(mse / float(W.var()), 4)}
+    print(json.dumps({"metric": "Viterbi search, trellis state updates per second", "unit": "updates/s", "n_gpus": 1,
+                      "value": res["viterbi_pairs rows 512 steps 2048"]["state_updates_per_s"], "data": "synthetic",
+                      "config": {"workload": "65536-state trellis, 4 bits and two weights per step, Gaussian targets, S=8"},
+                      "results": res}))
+
+
 def main():
     a = parse()
     if a.gpus != 1:
@@ -362,6 +425,9 @@ def main():
         return
     if a.other_ops:
         bench_other_ops(a)
+        return
+    if a.quantize:
+        bench_quantize(a)
         return
     if a.decode:
         from rptc_kernels.llama_decode import LlamaShape, QuantizedLlama, greedy_decode

@@ -217,6 +217,23 @@ int rptc_decompress_matvec_rmsnorm(const int32_t *compressed, const uint16_t *co
                                    float *ms);
 
 /*
+ * Viterbi search for the hashed pair stream: the symbols whose decode by rptc_decompress_matvec_16_{S}_1
+ * (carry mode continuous) is closest to the targets.  Replaces the search of the reference's quantizer
+ * (rptc.py:13-71, diag_only path: rho[0] = 0 at the start, first index on ties, best end state traced
+ * back), on the trellis its inference kernels decode (inference.cu:250-262): 65536 states, 4 stream bits
+ * and two weights per step.
+ *   targets   float [rows][steps][2], the weight pairs in stream order
+ *   weights   NULL, or float per-weight importance [.][steps][2]: row r reads weights + r * weights_row_stride
+ *             (0 = one set for all rows); a step costs c0*(x0-w0)^2 + c1*(x1-w1)^2, all sums in fp32
+ *   scratch   rptc_viterbi_scratch_bytes(rows, steps) bytes of device memory (the back pointers)
+ *   symbols   uint8 [rows][steps], values 0..15;  end_state int32 [rows];  cost float [rows]
+ */
+int64_t rptc_viterbi_scratch_bytes(int64_t rows, int64_t steps);
+int rptc_viterbi_pairs(const float *targets, const float *weights, int64_t weights_row_stride,
+                       const uint16_t *codebook, void *scratch, uint8_t *symbols, int32_t *end_state, float *cost,
+                       int64_t rows, int64_t steps, int S, void *stream, float *ms);
+
+/*
  * Measurement aids (no counterpart in the reference; not part of the product path).  bench.py times
  * them in the same launch pattern as the mat-vec it grades, so that the achieved figure can be read
  * against the floor for the workload's size on the machine at hand.

@@ -12,6 +12,7 @@ int prepare_matvec_t(int device);
 int prepare_matmul(int device);
 int prepare_hadamard();
 int prepare_decode_glue(int device);
+int prepare_viterbi();
 
 constexpr int kMaxDevices = 64;
 static DeviceInfo g_devices[kMaxDevices];
@@ -41,6 +42,7 @@ int device_info(DeviceInfo **out)
         if ((rc = prepare_matmul(dev))) return rc;
         if ((rc = prepare_hadamard())) return rc;
         if ((rc = prepare_decode_glue(dev))) return rc;
+        if ((rc = prepare_viterbi())) return rc;
         g_ready[dev] = true;
     }
     *out = &g_devices[dev];

@@ -1,0 +1,264 @@
+// Viterbi search for the hashed pair stream: the quantizer's inner loop.
+//
+// The search is the reference's (rptc.py:13-71, diag_only path): path costs rho over all trellis
+// states, rho[0] = 0 and infinity elsewhere at the start (rptc.py:55-56), per step the cheapest
+// of the predecessors of every state (rptc.py:27-28, first index on ties as argmin does) plus the
+// step's squared error (rptc.py:32), the cheapest end state traced back (rptc.py:60-65).  The
+// trellis is the one the inference kernels decode (inference.cu:250-262): 65536 states, a step
+// shifts 4 new bits in and emits the two weights the state's hash selects, so a state s' has the
+// 16 predecessors (d << 12) | (s' >> 4).
+//
+// One workgroup of 1024 threads searches one row.  Thread j keeps the costs of 64 states in
+// registers: the four predecessor groups g = 4j .. 4j+3 with all 16 values of d, so the minimum
+// over a group's predecessors never leaves the thread.  A step is
+//   1. every thread: the minimum and its d for its four groups -> LDS (16 KiB) and the back
+//      pointers (4 bits a group) -> memory; and the step's error for each distinct (entry, sign)
+//      pair (256 of them at S = 8, where the sign is the entry's top bit; 128 at S = 6) -> an LDS
+//      table with 32 copies of every value, so that the gathers below are free of bank conflicts;
+//   2. barrier; every thread: new cost of its 64 states = minimum of the state's group (16 LDS
+//      reads, each shared by four states) + the error of the state's pair (64 gathers).
+// Both LDS tables are double-buffered, which makes the one barrier enough.
+// All sums are fp32 in the order of the host-side restatement (rptc_kernels/quantize.py), with
+// contraction off, so the chosen path is the same bit for bit.  The trace back is a second kernel
+// with one thread per row: a chain of dependent loads, run for all rows side by side.
+#include "rptc_common.hpp"
+
+#include <math.h>
+
+namespace rptc {
+
+constexpr int kVitThreads = 1024;
+constexpr int kVitGroups = 4096;           // states >> 4
+constexpr int kVitCopies = 32;             // copies of a loss value, one per LDS bank
+constexpr int kVitLossRow = 64;            // floats in a table row (256 bytes): 32 copies for even steps, 32 for odd
+constexpr int kVitLossFloats = 256 * kVitLossRow;
+constexpr int kVitLdsBytes = (kVitLossFloats + 2 * kVitGroups) * 4 + 2 * kVitThreads * 4;
+
+#pragma clang fp contract(off)
+__device__ __forceinline__ float pair_loss(float x0, float x1, float w0, float w1)
+{
+    const float d0 = x0 - w0, d1 = x1 - w1;
+    return d0 * d0 + d1 * d1;
+}
+
+__device__ __forceinline__ float pair_loss_weighted(float x0, float x1, float w0, float w1, float c0, float c1)
+{
+    const float d0 = x0 - w0, d1 = x1 - w1;
+    return c0 * (d0 * d0) + c1 * (d1 * d1);
+}
+
+template <int S, bool WEIGHTED>
+__global__ __launch_bounds__(kVitThreads) void viterbi_pairs_kernel(
+    const float *__restrict__ targets, const float *__restrict__ weights, int64_t weights_row_stride,
+    const uint16_t *__restrict__ codebook, uint16_t *__restrict__ back, int32_t *__restrict__ end_state,
+    float *__restrict__ cost, int steps)
+{
+    extern __shared__ float lds[];
+    // The loss table is the first thing in LDS and the kernel has no static LDS, so it starts at
+    // LDS address 0 and a 16-bit byte offset reaches all of it.
+    float *loss = lds;                                  // [256][2][32]: a row holds 32 copies for even steps, 32 for odd
+    float *best = lds + kVitLossFloats;                 // [2][4096]
+    float *red_v = best + 2 * kVitGroups;               // [1024]
+    int *red_i = reinterpret_cast<int *>(red_v + kVitThreads);
+
+    const int j = threadIdx.x, copy = j & (kVitCopies - 1);
+    const int64_t row = blockIdx.x;
+    const uint32_t loss_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(loss));
+
+    // Register r = 16 * gi + d holds state (d << 12) | (4j + gi).  code[r / 4] byte r % 4 is the row of
+    // the loss table the state reads: its codebook entry, with the hash's sign bit on top at S = 6
+    // (at S = 8 the sign bit is the entry's own top bit, inference.cu:253-262).  A row starts every
+    // 256 bytes, so one byte permute makes the address out of the code and the thread's copy.
+    float rho[64];
+    uint32_t code[16];
+#pragma unroll
+    for (int r = 0; r < 64; r++) {
+        const uint32_t s = ((uint32_t)(r & 15) << 12) | (uint32_t)(4 * j + (r >> 4));
+        const uint32_t prod = s * (s + 1u);
+        const uint32_t c = S == 8 ? (prod >> 8) & 0xFFu : ((prod >> 8) & 63u) | (((prod >> 15) & 1u) << 6);
+        if (r & 3) code[r >> 2] |= c << (8 * (r & 3));
+        else code[r >> 2] = c;
+        rho[r] = (s == 0) ? 0.f : INFINITY;
+    }
+    const uint32_t copy4 = loss_base + 4u * (uint32_t)copy;
+
+    // the table row this thread fills: four threads a row, 8 copies each
+    const int c_mine = (j >> 2) & (S == 8 ? 255 : 127);
+    const int e_mine = S == 8 ? c_mine : c_mine & 63;
+    const bool neg_mine = S == 8 ? (c_mine >> 7) != 0 : (c_mine >> 6) != 0;
+    const float w0 = fabsf(half_bits_to_float(codebook[2 * e_mine])) * (neg_mine ? -1.f : 1.f);
+    const float w1 = half_bits_to_float(codebook[2 * e_mine + 1]);
+    float4 *loss_mine = reinterpret_cast<float4 *>(loss + c_mine * kVitLossRow + (j & 3) * 8);
+
+    const float *tg = targets + row * steps * 2;
+    const float *wt = WEIGHTED ? weights + row * weights_row_stride : nullptr;
+    uint16_t *back_row = back + row * steps * (int64_t)kVitThreads;
+    float x0 = tg[0], x1 = tg[1], c0 = WEIGHTED ? wt[0] : 1.f, c1 = WEIGHTED ? wt[1] : 1.f;
+    for (int t = 0; t < steps; t++) {
+        // the next step's targets are on their way while this step is computed
+        const int tn = t + 1 < steps ? t + 1 : t;
+        const float nx0 = tg[2 * tn], nx1 = tg[2 * tn + 1];
+        const float nc0 = WEIGHTED ? wt[2 * tn] : 1.f, nc1 = WEIGHTED ? wt[2 * tn + 1] : 1.f;
+
+        const float l = WEIGHTED ? pair_loss_weighted(x0, x1, w0, w1, c0, c1) : pair_loss(x0, x1, w0, w1);
+        const float4 l4 = make_float4(l, l, l, l);
+        // Both LDS tables have two halves that take turns, so a step needs one barrier: what this
+        // step overwrites was last read two steps ago, before the previous step's barrier.
+        float4 *lm = loss_mine + (t & 1) * (kVitCopies / 4);
+        lm[0] = l4;
+        lm[1] = l4;
+
+        float *bw = best + (t & 1) * kVitGroups;
+        uint32_t nib = 0;
+#pragma unroll
+        for (int gi = 0; gi < 4; gi++) {
+            float m = rho[16 * gi];
+            uint32_t arg = 0;
+#pragma unroll
+            for (int d = 1; d < 16; d++) {
+                const bool lt = rho[16 * gi + d] < m;      // the first minimum wins
+                m = lt ? rho[16 * gi + d] : m;
+                arg = lt ? (uint32_t)d : arg;
+            }
+            bw[4 * j + gi] = m;
+            nib |= arg << (4 * gi);
+        }
+        back_row[(int64_t)t * kVitThreads + j] = (uint16_t)nib;
+        __syncthreads();
+
+        const uint32_t copy4_t = copy4 + (uint32_t)(t & 1) * (kVitCopies * 4u);
+        // state (d << 12) | g comes from group ((d << 12) | g) >> 4 = (d << 8) | (j >> 2) for all four g
+#pragma unroll
+        for (int d = 0; d < 16; d++) {
+            const float b = bw[(d << 8) | (j >> 2)];
+#pragma unroll
+            for (int gi = 0; gi < 4; gi++) {
+                const int r = 16 * gi + d;
+                // byte 0: the copy's offset; byte 1: the state's code; the rest zero
+                const uint32_t off = perm(code[r >> 2], copy4_t, 0x0C0C0400u + ((uint32_t)(r & 3) << 8));
+                rho[r] = b + __builtin_bit_cast(float, lds_read_abs(off));
+            }
+            // a few gathers in flight at a time: all 64 at once would push registers out to memory
+            if ((d & 1) == 1) __builtin_amdgcn_sched_barrier(0);
+        }
+        x0 = nx0, x1 = nx1, c0 = nc0, c1 = nc1;
+    }
+
+    // cheapest end state, the lowest index among equals: in a thread the states are visited in
+    // rising order (d outer, gi inner)
+    float mv = rho[0];
+    int mi = 4 * j;
+#pragma unroll
+    for (int d = 0; d < 16; d++) {
+#pragma unroll
+        for (int gi = 0; gi < 4; gi++) {
+            const float v = rho[16 * gi + d];
+            const int s = (d << 12) | (4 * j + gi);
+            if (v < mv) {
+                mv = v;
+                mi = s;
+            }
+        }
+    }
+    red_v[j] = mv;
+    red_i[j] = mi;
+    __syncthreads();
+    for (int width = kVitThreads / 2; width > 0; width >>= 1) {
+        if (j < width) {
+            const float ov = red_v[j + width];
+            const int oi = red_i[j + width];
+            if (ov < red_v[j] || (ov == red_v[j] && oi < red_i[j])) {
+                red_v[j] = ov;
+                red_i[j] = oi;
+            }
+        }
+        __syncthreads();
+    }
+    if (j == 0) {
+        end_state[row] = red_i[0];
+        cost[row] = red_v[0];
+    }
+}
+
+// one thread per row walks the back pointers from the end state (rptc.py:60-65)
+__global__ __launch_bounds__(64) void viterbi_trace_kernel(const uint16_t *__restrict__ back,
+                                                           const int32_t *__restrict__ end_state,
+                                                           uint8_t *__restrict__ symbols, int rows, int steps)
+{
+    const int row = blockIdx.x * 64 + threadIdx.x;
+    if (row >= rows) return;
+    const uint16_t *back_row = back + (int64_t)row * steps * kVitThreads;
+    uint8_t *sym = symbols + (int64_t)row * steps;
+    uint32_t state = (uint32_t)end_state[row];
+    for (int t = steps - 1; t >= 0; t--) {
+        sym[t] = (uint8_t)(state & 15u);
+        const uint32_t low = state >> 4;                // the predecessor's low 12 bits = the group
+        const uint32_t nib = back_row[(int64_t)t * kVitThreads + (low >> 2)];
+        state = (((nib >> (4 * (low & 3u))) & 15u) << 12) | low;
+    }
+}
+
+template <typename K>
+static int vit_allow_lds(K kernel)
+{
+    return (int)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    kVitLdsBytes);
+}
+
+int prepare_viterbi()
+{
+    int rc;
+    if ((rc = vit_allow_lds(viterbi_pairs_kernel<6, false>))) return rc;
+    if ((rc = vit_allow_lds(viterbi_pairs_kernel<6, true>))) return rc;
+    if ((rc = vit_allow_lds(viterbi_pairs_kernel<8, false>))) return rc;
+    return vit_allow_lds(viterbi_pairs_kernel<8, true>);
+}
+
+template <int S, bool WEIGHTED>
+static void launch_viterbi(const float *targets, const float *weights, int64_t weights_row_stride, const uint16_t *codebook,
+                           uint16_t *back, int32_t *end_state, float *cost, int64_t rows, int64_t steps, hipStream_t s)
+{
+    hipLaunchKernelGGL((viterbi_pairs_kernel<S, WEIGHTED>), dim3((unsigned)rows), dim3(kVitThreads), kVitLdsBytes, s, targets,
+                       weights, weights_row_stride, codebook, back, end_state, cost, (int)steps);
+}
+
+}  // namespace rptc
+
+using namespace rptc;
+
+extern "C" int64_t rptc_viterbi_scratch_bytes(int64_t rows, int64_t steps)
+{
+    if (rows < 1 || steps < 1) return 0;
+    return rows * steps * (int64_t)kVitThreads * 2;
+}
+
+extern "C" int rptc_viterbi_pairs(const float *targets, const float *weights, int64_t weights_row_stride,
+                                  const uint16_t *codebook, void *scratch, uint8_t *symbols, int32_t *end_state,
+                                  float *cost, int64_t rows, int64_t steps, int S, void *stream, float *ms)
+{
+    if (!targets || !codebook || !scratch || !symbols || !end_state || !cost) return RPTC_ENULL;
+    if (S != 6 && S != 8) return RPTC_ESHAPE;
+    if (rows < 1 || steps < 1 || weights_row_stride < 0) return RPTC_ESHAPE;
+    if (weights && weights_row_stride != 0 && weights_row_stride < 2 * steps) return RPTC_ESHAPE;
+    if (rows >= ((int64_t)1 << 24) || steps >= ((int64_t)1 << 24)) return RPTC_ELIMIT;
+    DeviceInfo *dev;
+    int rc = device_info(&dev);
+    if (rc) return rc;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    Timer t;
+    rc = t.begin(dev, s, ms);
+    if (rc) return rc;
+    uint16_t *back = static_cast<uint16_t *>(scratch);
+    if (S == 6) {
+        if (weights) launch_viterbi<6, true>(targets, weights, weights_row_stride, codebook, back, end_state, cost, rows, steps, s);
+        else launch_viterbi<6, false>(targets, weights, weights_row_stride, codebook, back, end_state, cost, rows, steps, s);
+    } else {
+        if (weights) launch_viterbi<8, true>(targets, weights, weights_row_stride, codebook, back, end_state, cost, rows, steps, s);
+        else launch_viterbi<8, false>(targets, weights, weights_row_stride, codebook, back, end_state, cost, rows, steps, s);
+    }
+    rc = (int)hipGetLastError();
+    if (rc) return rc;
+    hipLaunchKernelGGL(viterbi_trace_kernel, dim3((unsigned)((rows + 63) / 64)), dim3(64), 0, s, back, end_state, symbols,
+                       (int)rows, (int)steps);
+    return t.end();
+}

@@ -24,7 +24,8 @@ a stream stands for), ``decompress_matmul_16_{6,8}_1`` and ``decompress_matmul_b
 the matrix cores), ``decompress_matvec_bits`` (2, 3, 4 bits per weight), ``decompress_matvec_silu`` and
 ``decompress_matvec_rmsnorm`` (the mat-vec with a decoder layer's element-wise step in its prologue),
 ``decompress_matvec_hadamard`` (with the sign-Hadamard transform of its activations in its prologue),
-``sign_hadamard``.  Sub-modules: ``packing`` (symbols -> streams), ``quantize`` (Viterbi search),
+``sign_hadamard``, ``viterbi_pairs`` (the quantizer's trellis search, rptc.py:13-71, as a kernel).
+Sub-modules: ``packing`` (symbols -> streams), ``quantize`` (the quantizer around that search),
 ``linear`` (``QuantizedLinear``, ``patch_model``), ``llama_decode`` (a Llama-shaped decode loop),
 ``eval_ppl`` (perplexity on a token file).
 """
@@ -62,6 +63,8 @@ _SIGNATURES = {
     "rptc_matvec_t_dense": ([_VP, _VP, _VP, _I64, _I64, _INT, _INT, _VP, _FP], _INT),
     "rptc_decompress_matmul": ([_VP, _VP, _VP, _VP, _I64, _I64, _I64, _INT, _INT, _VP, _FP], _INT),
     "rptc_decompress_matmul_bits": ([_VP, _VP, _VP, _VP, _I64, _I64, _I64, _INT, _INT, _INT, _VP, _FP], _INT),
+    "rptc_viterbi_scratch_bytes": ([_I64, _I64], _I64),
+    "rptc_viterbi_pairs": ([_VP, _VP, _I64, _VP, _VP, _VP, _VP, _VP, _I64, _I64, _INT, _VP, _FP], _INT),
     "rptc_sign_hadamard": ([_VP, _VP, _VP, _I64, _I64, _I64, _INT, _VP, _FP], _INT),
     "rptc_decompress_matvec_bits": ([_VP, _VP, _VP, _VP, _I64, _I64, _INT, _INT, _INT, _VP, _FP], _INT),
     "rptc_matvec_bits_dense": ([_VP, _VP, _VP, _I64, _I64, _INT, _INT, _INT, _VP, _FP], _INT),
@@ -372,6 +375,46 @@ def sign_hadamard(x, signs, out, block=0, inverse=False):
                                           ctypes.byref(ms) if _timing else None)
     _status(rc)
     return float(ms.value)
+
+
+def viterbi_pairs(targets, codebook, weights=None):
+    """Exact Viterbi search on the trellis of ``decompress_matvec_16_{S}_1`` (65536 states, 4 stream bits
+    and two weights per step; S from the codebook length), the search of rptc.py:13-71.
+
+    targets: float32 [rows, steps, 2] (weight pairs in stream order); weights: None, float32 [steps, 2]
+    (one importance set for all rows) or [rows, steps, 2].  Returns (symbols uint8 [rows, steps],
+    cost float32 [rows], end_state int32 [rows], elapsed ms).  Needs rows * steps * 2048 bytes of scratch."""
+    _check_input(targets, "targets")
+    _check_input(codebook, "codebook")
+    _check(targets.dtype == torch.float32 and targets.dim() == 3 and targets.size(2) == 2,
+           "targets must be float32 [rows, steps, 2]")
+    _check(codebook.dtype == torch.float16 and codebook.numel() in (128, 512), "codebook must be fp16 of length 128 or 512")
+    rows, steps = targets.size(0), targets.size(1)
+    _check(rows >= 1 and steps >= 1, "rows >= 1 and steps >= 1")
+    S = 6 if codebook.numel() == 128 else 8
+    stride = 0
+    if weights is not None:
+        _check_input(weights, "weights")
+        _check(weights.dtype == torch.float32, "weights must be float32")
+        _check(tuple(weights.shape) in ((steps, 2), (rows, steps, 2)), "weights must be [steps, 2] or [rows, steps, 2]")
+        stride = 0 if weights.dim() == 2 else 2 * steps
+    device = targets.device
+    lib = library()
+    with torch.cuda.device(device):
+        scratch = torch.empty(lib.rptc_viterbi_scratch_bytes(rows, steps), dtype=torch.uint8, device=device)
+        symbols = torch.empty((rows, steps), dtype=torch.uint8, device=device)
+        end_state = torch.empty(rows, dtype=torch.int32, device=device)
+        cost = torch.empty(rows, dtype=torch.float32, device=device)
+        ms = ctypes.c_float(0.0)
+        stream = torch.cuda.current_stream().cuda_stream
+        rc = lib.rptc_viterbi_pairs(targets.data_ptr(), weights.data_ptr() if weights is not None else None, stride,
+                                    codebook.data_ptr(), scratch.data_ptr(), symbols.data_ptr(), end_state.data_ptr(),
+                                    cost.data_ptr(), rows, steps, S, ctypes.c_void_p(stream),
+                                    ctypes.byref(ms) if _timing else None)
+        _status(rc)
+        if not _timing:
+            torch.cuda.current_stream().synchronize()     # scratch is freed on return
+    return symbols, cost, end_state, float(ms.value)
 
 
 def decompress_matvec_bits(compressed, codebook, x, out, bits):

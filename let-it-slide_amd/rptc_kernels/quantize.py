@@ -54,7 +54,7 @@ def viterbi_pairs(targets, table, weights=None, state_bits=STATE_BITS, step_bits
         if weights is None:
             loss = d0 * d0 + d1 * d1
         else:
-            loss = weights[:, t, 0:1] * d0 * d0 + weights[:, t, 1:2] * d1 * d1
+            loss = weights[:, t, 0:1] * (d0 * d0) + weights[:, t, 1:2] * (d1 * d1)     # rptc.py:32: c * (x - a)**2
         rho = best.repeat_interleave(R, dim=1) + loss
     cost, state = rho.min(dim=1)
     symbols = torch.empty((rows, steps), dtype=torch.int64, device=dev)
@@ -71,7 +71,8 @@ def quantize_matrix(W, codebook, S=8, importance=None, rows_per_batch=64, bits=2
     """Quantize W [m, n] (n % 64 == 0) to symbols of 2*bits bits [m, n/2] in stream order, for the decoder
     of ``decompress_matvec_*`` (bits == 2) or ``decompress_matvec_bits`` in CONTINUOUS mode.  importance:
     optional [n] per-column weight (e.g. the Hessian diagonal, quantize_hf.py:164).  Returns (symbols int64
-    [m, n/2] on the CPU, mse float)."""
+    [m, n/2] on the CPU, mse float).  A matrix on the GPU at 2 bits per weight is searched by the HIP kernel
+    (``rptc_kernels.viterbi_pairs``), which chooses the same path as ``viterbi_pairs`` here bit for bit."""
     W = torch.as_tensor(W)
     m, n = W.shape
     dev = W.device
@@ -85,10 +86,20 @@ def quantize_matrix(W, codebook, S=8, importance=None, rows_per_batch=64, bits=2
         wts = torch.stack([imp[cols], imp[cols + 1]], dim=1).unsqueeze(0)
     out = torch.empty((m, n // 2), dtype=torch.int64)
     total = 0.0
+    on_gpu = W.is_cuda and bits == 2
+    if on_gpu:
+        # the search kernel: one workgroup per row, 2048 bytes of back pointers per row and step
+        import rptc_kernels as rk
+        cb16 = torch.as_tensor(codebook).to(dev).to(torch.float16).contiguous()
+        shared = None if wts is None else wts[0].contiguous()
+        rows_per_batch = max(1, min(m, (1 << 30) // (1024 * n)))
     for r0 in range(0, m, rows_per_batch):
         tg = targets[r0:r0 + rows_per_batch]
-        w = None if wts is None else wts.expand(tg.size(0), -1, -1)
-        sym, cost = viterbi_pairs(tg, table, w, step_bits=2 * bits)
+        if on_gpu:
+            sym, cost, _, _ = rk.viterbi_pairs(tg.contiguous(), cb16, shared)
+        else:
+            w = None if wts is None else wts.expand(tg.size(0), -1, -1)
+            sym, cost = viterbi_pairs(tg, table, w, step_bits=2 * bits)
         out[r0:r0 + rows_per_batch] = sym.cpu()
         total += cost.sum().item()
     return out, total / (m * n)

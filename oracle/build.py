@@ -16,7 +16,7 @@ LIB = os.path.join(OUT_DIR, "librptc_oracle.so")
 
 def build(verbose=False):
     os.makedirs(OUT_DIR, exist_ok=True)
-    cmd = ["gcc", "-O3", "-march=x86-64-v2", "-fopenmp", "-shared", "-fPIC", "-Wall", "-Wextra",
+    cmd = ["gcc", "-O3", "-march=x86-64-v2", "-ffp-contract=off", "-fopenmp", "-shared", "-fPIC", "-Wall", "-Wextra",
            "-o", LIB, os.path.join(HERE, "rptc_oracle.c"), "-lm"]
     if verbose:
         print(" ".join(cmd))

@@ -27,6 +27,12 @@
  *   orc_lite_index_fn /   hand-computed known answers; PARITY UNPINNED beyond
  *   orc_lite_dequantize   those (the reference holds no vectors and its
  *                         Python needs jax, which is not installed)
+ *   orc_viterbi           exhaustive enumeration of every symbol sequence on
+ *                         trellises small enough for it (optimal cost, and the
+ *                         returned path has that cost); the tie rules are
+ *                         restated from rptc.py's argmin and checked on inputs
+ *                         built to tie.  PARITY UNPINNED against jnp.argmin
+ *                         itself (jax is not installed)
  *   orc_matvec (ragged n), orc_bits_dense, orc_sign_hadamard: formats and
  *                         ops of this build with no counterpart in the
  *                         reference; pinned by closed forms only.
@@ -667,6 +673,85 @@ int orc_matvec_f32(const uint32_t *compressed, const uint16_t *codebook,
         y[r] = acc0 + acc1;
     }
     free(sx);
+    return 0;
+}
+
+/* ------------------------------------------------------------- quantizer */
+
+/*
+ * The reference's trellis search (rptc.py:13-71, diag_only path), for a trellis
+ * of 2^L states that takes b bits per step and emits V values per state:
+ *   rho[0] = 0, rho[s] = inf otherwise                       (rptc.py:55-56)
+ *   per step, for every prefix p = s' >> b: the cheapest of the predecessors
+ *   (d << (L-b)) | p, lowest d on ties as argmin picks        (rptc.py:23-28)
+ *   rho'[s'] = rho[best predecessor] + loss(s')              (rptc.py:51)
+ *   loss(s') = sum_v c[t][v] * (x[t][v] - table[s'][v])^2     (rptc.py:32; c = 1
+ *   without weights), every product and sum rounded to fp32
+ *   the cheapest end state (lowest index on ties) is traced back (rptc.py:60-65)
+ * The reference has V = 1, b = 2 and a scalar weight per step; the hashed pair
+ * stream of inference.cu:250-262 is V = 2, b = 4 with table[s] the pair that
+ * state s decodes to.  symbols[t] = the b bits shifted in at step t.
+ */
+int orc_viterbi(const float *table, int L, int b, int V, const float *targets,
+                const float *weights, int64_t steps, int32_t *symbols,
+                float *cost, int32_t *end_state)
+{
+    if (L < 1 || L > 20 || b < 1 || b > L || V < 1 || V > 4 || steps < 1)
+        return -2;
+    const int64_t M = (int64_t)1 << L, P = M >> b, R = (int64_t)1 << b;
+    float *rho = (float *)malloc(sizeof(float) * (size_t)M);
+    float *best = (float *)malloc(sizeof(float) * (size_t)P);
+    uint16_t *back = (uint16_t *)malloc(sizeof(uint16_t) * (size_t)(P * steps));
+    if (!rho || !best || !back) {
+        free(rho);
+        free(best);
+        free(back);
+        return -1;
+    }
+    for (int64_t s = 0; s < M; s++)
+        rho[s] = INFINITY;
+    rho[0] = 0.0f;
+    for (int64_t t = 0; t < steps; t++) {
+        for (int64_t p = 0; p < P; p++) {
+            float m = rho[p];
+            int64_t arg = 0;
+            for (int64_t d = 1; d < R; d++) {
+                float v = rho[(d << (L - b)) | p];
+                if (v < m) {
+                    m = v;
+                    arg = d;
+                }
+            }
+            best[p] = m;
+            back[t * P + p] = (uint16_t)arg;
+        }
+        for (int64_t s = 0; s < M; s++) {
+            volatile float loss = 0.0f;
+            for (int v = 0; v < V; v++) {
+                volatile float d = targets[t * V + v] - table[s * V + v];
+                volatile float sq = d * d;
+                if (weights)
+                    sq = weights[t * V + v] * sq;
+                loss = (v == 0) ? sq : loss + sq;
+            }
+            volatile float r = best[s >> b] + loss;
+            rho[s] = r;
+        }
+    }
+    int64_t state = 0;
+    for (int64_t s = 1; s < M; s++)
+        if (rho[s] < rho[state])
+            state = s;
+    *cost = rho[state];
+    *end_state = (int32_t)state;
+    for (int64_t t = steps - 1; t >= 0; t--) {
+        symbols[t] = (int32_t)(state & (R - 1));
+        int64_t p = state >> b;
+        state = ((int64_t)back[t * P + p] << (L - b)) | p;
+    }
+    free(rho);
+    free(best);
+    free(back);
     return 0;
 }
 

@@ -48,6 +48,8 @@ def lib():
         _lib.orc_bits_dense.restype = i32
         _lib.orc_sign_hadamard.argtypes = [vp, vp, vp, i64, i64, i64, i32]
         _lib.orc_sign_hadamard.restype = i32
+        _lib.orc_viterbi.argtypes = [vp, i32, i32, i32, vp, vp, i64, vp, vp, vp]
+        _lib.orc_viterbi.restype = i32
         _lib.orc_num_threads.restype = i32
         _lib.orc_set_num_threads.argtypes = [i32]
     return _lib
@@ -82,6 +84,30 @@ def dequantize(alphabet, symbols):
     out = np.empty(symbols.shape[0], dtype=np.float32)
     lib().orc_dequantize(_p(alphabet), L, _p(symbols), symbols.shape[0], _p(out))
     return out
+
+
+def viterbi(table, step_bits, targets, weights=None):
+    """rptc.py:13-71 (diag_only) on a trellis of table.shape[0] = 2^L states that takes step_bits per step and
+    emits table.shape[1] values per state.  table float32 [2^L, V]; targets float32 [steps, V]; weights None
+    or [steps, V].  Returns (symbols int32 [steps], cost float32, end_state int)."""
+    table = np.ascontiguousarray(table, dtype=np.float32)
+    targets = np.ascontiguousarray(targets, dtype=np.float32)
+    if table.ndim == 1:
+        table, targets = table[:, None], targets.reshape(-1, 1)
+    M, V = table.shape
+    L = int(M).bit_length() - 1
+    assert M == 1 << L and targets.ndim == 2 and targets.shape[1] == V
+    steps = targets.shape[0]
+    w = None
+    if weights is not None:
+        w = np.ascontiguousarray(weights, dtype=np.float32).reshape(steps, V)
+    symbols = np.empty(steps, dtype=np.int32)
+    cost = np.zeros(1, dtype=np.float32)
+    end = np.zeros(1, dtype=np.int32)
+    rc = lib().orc_viterbi(_p(table), L, int(step_bits), V, _p(targets), _p(w) if w is not None else None, steps,
+                           _p(symbols), _p(cost), _p(end))
+    assert rc == 0, rc
+    return symbols, cost[0], int(end[0])
 
 
 def dequantize_h(alphabet, symbols):

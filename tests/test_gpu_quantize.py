@@ -1,0 +1,93 @@
+"""The Viterbi search kernel against the CPU restatement of rptc.py:13-71 and against the host-side
+search, bit for bit: the same path, the same fp32 cost, the same end state."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def rk():
+    import rptc_kernels
+    assert torch.cuda.is_available()
+    return rptc_kernels
+
+
+def _case(seed, rows, steps, S, weighted):
+    g = np.random.default_rng(seed)
+    cb = g.standard_normal(2 << S).astype(np.float16)
+    targets = (0.7 * g.standard_normal((rows, steps, 2))).astype(np.float32)
+    weights = None
+    if weighted == "shared":
+        weights = g.uniform(0.25, 4.0, (steps, 2)).astype(np.float32)
+    elif weighted == "rows":
+        weights = g.uniform(0.25, 4.0, (rows, steps, 2)).astype(np.float32)
+    return cb, targets, weights
+
+
+@pytest.mark.parametrize("S", [6, 8])
+@pytest.mark.parametrize("rows,steps,weighted", [(3, 1, None), (2, 33, None), (2, 64, "shared"), (3, 96, "rows"),
+                                                 (1, 300, None)])
+def test_viterbi_kernel_equals_the_oracle(rk, oracle, rows, steps, S, weighted):
+    from rptc_kernels import quantize
+    cb, targets, weights = _case(10 * steps + S, rows, steps, S, weighted)
+    table = quantize.decode_table(torch.from_numpy(cb), S).numpy()
+    sym, cost, end, ms = rk.viterbi_pairs(torch.from_numpy(targets).cuda(), torch.from_numpy(cb).cuda(),
+                                          None if weights is None else torch.from_numpy(weights).cuda())
+    assert ms > 0 and sym.dtype == torch.uint8 and sym.shape == (rows, steps)
+    sym, cost, end = sym.cpu().numpy(), cost.cpu().numpy(), end.cpu().numpy()
+    for r in range(rows):
+        w = None if weights is None else (weights if weights.ndim == 2 else weights[r])
+        osym, ocost, oend = oracle.viterbi(table, 4, targets[r], w)
+        assert np.array_equal(sym[r].astype(np.int32), osym), f"row {r}"
+        assert cost[r] == ocost and end[r] == oend
+
+
+def test_viterbi_kernel_ties_take_the_first_index(rk, oracle):
+    """Equal codebook pairs make many paths tie; the kernel resolves every tie as argmin does."""
+    from rptc_kernels import quantize
+    cb = np.zeros(512, dtype=np.float16)
+    cb[::2], cb[1::2] = 0.5, -0.25          # every entry the same pair up to the hash's sign bit
+    targets = np.zeros((2, 40, 2), dtype=np.float32)
+    targets[1, :, 0] = -0.5                 # row 1 prefers the states whose hash sets the sign
+    table = quantize.decode_table(torch.from_numpy(cb), 8).numpy()
+    sym, cost, end, _ = rk.viterbi_pairs(torch.from_numpy(targets).cuda(), torch.from_numpy(cb).cuda())
+    for r in range(2):
+        osym, ocost, oend = oracle.viterbi(table, 4, targets[r])
+        assert np.array_equal(sym[r].cpu().numpy().astype(np.int32), osym)
+        assert float(cost[r]) == float(ocost) and int(end[r]) == oend
+
+
+def test_quantize_matrix_on_the_gpu_uses_the_kernel_and_matches_the_host_search(rk, oracle):
+    from rptc_kernels import packing, quantize
+    g = np.random.default_rng(5)
+    m, n, S = 8, 512, 8
+    W = g.standard_normal((m, n)).astype(np.float32)
+    cb = g.standard_normal(2 << S).astype(np.float16)
+    imp = g.uniform(0.5, 2.0, n).astype(np.float32)
+    for importance in (None, imp):
+        sym_gpu, mse_gpu = quantize.quantize_matrix(torch.from_numpy(W).cuda(), torch.from_numpy(cb).cuda(), S,
+                                                    importance=importance)
+        sym_cpu, mse_cpu = quantize.quantize_matrix(torch.from_numpy(W), torch.from_numpy(cb), S, importance=importance)
+        assert torch.equal(sym_gpu, sym_cpu) and abs(mse_gpu - mse_cpu) < 1e-6
+    # and the symbols decode, through the packed stream and the mat-vec kernel's dense export, to the walk
+    stream = torch.from_numpy(packing.pack_matvec(sym_gpu.numpy())).cuda()
+    Wd = torch.empty((m, n), dtype=torch.float16, device="cuda")
+    prev = rk.set_carry_mode(rk.CONTINUOUS)
+    try:
+        rk.matvec_dense(stream, torch.from_numpy(cb).cuda(), Wd, S)
+    finally:
+        rk.set_carry_mode(prev)
+    walk = quantize.dequantize_symbols(sym_gpu, torch.from_numpy(cb), S)
+    assert torch.equal(Wd.cpu().float(), walk)
+
+
+def test_viterbi_rejects_bad_arguments(rk):
+    cb = torch.zeros(512, dtype=torch.float16, device="cuda")
+    with pytest.raises(RuntimeError):
+        rk.viterbi_pairs(torch.zeros((2, 8, 3), device="cuda"), cb)
+    with pytest.raises(RuntimeError):
+        rk.viterbi_pairs(torch.zeros((2, 8, 2), device="cuda"), cb[:100])
+    with pytest.raises(RuntimeError):
+        rk.viterbi_pairs(torch.zeros((2, 8, 2), device="cuda"), cb, torch.zeros((3, 8, 2), device="cuda"))

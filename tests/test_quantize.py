@@ -3,6 +3,7 @@ the kernels implement, and better than chance on a real-size state space."""
 import itertools
 
 import numpy as np
+import pytest
 import torch
 
 from rptc_kernels import packing, quantize
@@ -78,3 +79,60 @@ def test_quantize_matrix_at_3_and_4_bits_round_trips_and_gets_better_with_the_ra
         assert abs(((W - What) ** 2).mean() - mse) < 1e-5
         errors[bits] = mse
     assert errors[4] <= errors[3] <= errors[2]
+
+
+def _walk_cost(table, step_bits, targets, weights, seq):
+    """Cost of one symbol sequence by the decoder walk (rptc.py:74-85), in float64."""
+    M = table.shape[0]
+    state, c = 0, 0.0
+    for t, s in enumerate(seq):
+        state = ((state << step_bits) | int(s)) & (M - 1)
+        d = targets[t].astype(np.float64) - table[state].astype(np.float64)
+        w = np.ones_like(d) if weights is None else weights[t].astype(np.float64)
+        c += float((w * d * d).sum())
+    return c, state
+
+
+@pytest.mark.parametrize("L,b,V,steps,weighted", [(4, 2, 1, 6, False), (6, 2, 1, 5, True), (6, 2, 2, 6, False),
+                                                  (8, 4, 2, 3, True), (5, 1, 1, 9, False), (4, 4, 2, 3, False)])
+def test_oracle_viterbi_is_optimal_by_enumeration(oracle, L, b, V, steps, weighted):
+    """Every symbol sequence is tried: the oracle's cost is the smallest, and its path has that cost."""
+    g = np.random.default_rng(100 * L + b)
+    table = g.standard_normal((1 << L, V)).astype(np.float32)
+    targets = g.standard_normal((steps, V)).astype(np.float32)
+    weights = g.uniform(0.5, 2.0, (steps, V)).astype(np.float32) if weighted else None
+    sym, cost, end = oracle.viterbi(table, b, targets, weights)
+    best = min(_walk_cost(table, b, targets, weights, seq)[0] for seq in itertools.product(range(1 << b), repeat=steps))
+    assert abs(best - float(cost)) < 1e-5 * max(1.0, best)
+    c, state = _walk_cost(table, b, targets, weights, sym)
+    assert abs(c - best) < 1e-5 * max(1.0, best) and state == end
+    assert sym.min() >= 0 and sym.max() < (1 << b)
+
+
+def test_oracle_viterbi_tie_rules(oracle):
+    """A constant table makes every path cost the same: argmin's first index (rptc.py:27, 62) then picks
+    end state 0 and, walking back, the predecessor with d = 0 at every step, i.e. all-zero symbols."""
+    table = np.full((1 << 6, 1), 0.25, dtype=np.float32)
+    targets = np.zeros((7, 1), dtype=np.float32)
+    sym, cost, end = oracle.viterbi(table, 2, targets)
+    assert end == 0 and not sym.any() and cost == np.float32(7 * 0.0625)
+    # the trellis starts in state 0 (rptc.py:55-56): a table that makes state 0 expensive and state 1
+    # free still pays for leaving through the shift register, never starting elsewhere
+    table = np.ones((1 << 4, 1), dtype=np.float32)
+    table[1] = 0.0
+    sym, cost, end = oracle.viterbi(table, 2, np.zeros((1, 1), dtype=np.float32))
+    assert list(sym) == [1] and end == 1 and cost == 0.0
+
+
+def test_torch_viterbi_equals_the_oracle_bit_for_bit(oracle):
+    """The host-side search and the C restatement choose the same path and report the same fp32 cost."""
+    g = np.random.default_rng(7)
+    for (L, b, steps, weighted) in ((8, 4, 12, False), (10, 2, 20, True), (16, 4, 10, True)):
+        table = g.standard_normal((1 << L, 2)).astype(np.float32)
+        targets = g.standard_normal((2, steps, 2)).astype(np.float32)
+        weights = g.uniform(0.5, 2.0, (2, steps, 2)).astype(np.float32) if weighted else None
+        sym, cost = quantize.viterbi_pairs(torch.from_numpy(targets), torch.from_numpy(table),
+                                           None if weights is None else torch.from_numpy(weights), state_bits=L, step_bits=b)
+        for r in range(2):
+            osym, ocost, _ = oracle.viterbi(table, b, targets[r], None if weights is None else weights[r])
+            assert np.array_equal(sym[r].numpy(), osym) and float(cost[r]) == float(ocost)
