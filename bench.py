@@ -374,6 +374,17 @@ def bench_quantize(a):
         "ms": round(best, 3), "state_updates_per_s": float(f"{updates / best * 1e3:.4e}"),
         "us_per_step_per_row_round": round(best * 1e3 / steps / (rows / 256), 3),
         "vector_ops_per_update": 5, "frac_of_valu_peak": round(updates * 5 / (best * 1e-3) / valu_peak, 4)}}
+    # the reference's own trellis (2 bits and one alphabet value per step): 6 vector ops per update
+    # (mixed-precision subtract, square, add, and the minimum over four predecessors)
+    ab = torch.randn(1 << 16, generator=g, device="cuda").half()
+    tgs = torch.randn((256, 4096), generator=g, device="cuda")
+    best_s = None
+    for _ in range(3):
+        _, cost_s, _, ms = rk.viterbi_scalar(tgs, ab)
+        best_s = ms if best_s is None else min(best_s, ms)
+    res["viterbi_scalar L=16 rows 256 steps 4096"] = {
+        "ms": round(best_s, 3), "state_updates_per_s": float(f"{256 * 4096 * 65536 / best_s * 1e3:.4e}"),
+        "us_per_step": round(best_s * 1e3 / 4096, 3), "mse_unit_gaussian_2_bits": round(float(cost_s.sum()) / (256 * 4096), 4)}
     # the same search in framework ops on the GPU (64 rows, 256 steps)
     table = quantize.decode_table(cb, 8)
     small = tg[:64, :256].contiguous()

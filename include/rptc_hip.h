@@ -229,9 +229,23 @@ int rptc_decompress_matvec_rmsnorm(const int32_t *compressed, const uint16_t *co
  *   symbols   uint8 [rows][steps], values 0..15;  end_state int32 [rows];  cost float [rows]
  */
 int64_t rptc_viterbi_scratch_bytes(int64_t rows, int64_t steps);
+int64_t rptc_viterbi_scalar_scratch_bytes(int64_t rows, int64_t steps);
 int rptc_viterbi_pairs(const float *targets, const float *weights, int64_t weights_row_stride,
                        const uint16_t *codebook, void *scratch, uint8_t *symbols, int32_t *end_state, float *cost,
                        int64_t rows, int64_t steps, int S, void *stream, float *ms);
+
+/*
+ * The same search on the reference's own trellis (rptc.py:13-71 as it stands): 2^L states (L = 16 or 14),
+ * 2 stream bits and one value per step, the value of state s being alphabet[s]: the stream that
+ * rptc_decompress (L = 16) and rptc_decompress_matvec_t_{16,14} decode in carry mode continuous.
+ *   targets   float [rows][steps];  weights NULL or float [.][steps] (the reference's
+ *             sum(corrections[index]**2), rptc.py:32): a step costs c * (x - alphabet[s])^2 in fp32
+ *   alphabet  fp16 [2^L];  scratch rptc_viterbi_scalar_scratch_bytes(rows, steps) bytes
+ *   symbols   uint8 [rows][steps], values 0..3;  end_state int32 [rows];  cost float [rows]
+ */
+int rptc_viterbi_scalar(const float *targets, const float *weights, int64_t weights_row_stride,
+                        const uint16_t *alphabet, int L, void *scratch, uint8_t *symbols, int32_t *end_state,
+                        float *cost, int64_t rows, int64_t steps, void *stream, float *ms);
 
 /*
  * Measurement aids (no counterpart in the reference; not part of the product path).  bench.py times

@@ -21,6 +21,12 @@
 // All sums are fp32 in the order of the host-side restatement (rptc_kernels/quantize.py), with
 // contraction off, so the chosen path is the same bit for bit.  The trace back is a second kernel
 // with one thread per row: a chain of dependent loads, run for all rows side by side.
+//
+// viterbi_scalar_kernel is the same search on the reference's own trellis (rptc.py:13-71 as it
+// stands: 2^L states, 2 bits a step, one value a state from an arbitrary alphabet — the stream
+// decompress and decompress_matvec_t_* decode).  A state has four predecessors, thread j owns
+// 2^L / 4096 predecessor groups with all four d, and with no structure in the alphabet a thread
+// keeps its states' values in registers (two fp16 a register) and computes the error itself.
 #include "rptc_common.hpp"
 
 #include <math.h>
@@ -180,6 +186,154 @@ __global__ __launch_bounds__(kVitThreads) void viterbi_pairs_kernel(
     }
 }
 
+// x - (fp16 in the low / high half of v) in one op: x * 1.0 + (-half), the product exact, so the
+// result is the correctly rounded difference.  Written as asm also because the conversion alone
+// does not change from step to step: the compiler would convert all values once and keep them as
+// fp32, twice the registers.
+__device__ __forceinline__ float sub_half_lo(float x, uint32_t v)
+{
+    float d;
+    asm("v_fma_mix_f32 %0, %1, 1.0, -%2 op_sel_hi:[0,0,1]" : "=v"(d) : "v"(x), "v"(v));
+    return d;
+}
+
+__device__ __forceinline__ float sub_half_hi(float x, uint32_t v)
+{
+    float d;
+    asm("v_fma_mix_f32 %0, %1, 1.0, -%2 op_sel:[0,0,1] op_sel_hi:[0,0,1]" : "=v"(d) : "v"(x), "v"(v));
+    return d;
+}
+
+constexpr int scalar_lds_bytes(int L) { return 2 * ((1 << L) / 4) * 4 + 2 * kVitThreads * 4; }
+
+// L = 16 or 14.  NG = predecessor groups per thread; register r = 4 * gi + d holds state
+// (d << (L-2)) | (NG * j + gi).  Back pointers: 2 bits a group, one 32-bit word per thread and step.
+template <int L, bool WEIGHTED>
+__global__ __launch_bounds__(kVitThreads) void viterbi_scalar_kernel(
+    const float *__restrict__ targets, const float *__restrict__ weights, int64_t weights_row_stride,
+    const uint16_t *__restrict__ alphabet, uint32_t *__restrict__ back, int32_t *__restrict__ end_state,
+    float *__restrict__ cost, int steps)
+{
+    constexpr int M = 1 << L, G = M / 4, NG = G / kVitThreads, NS = 4 * NG;
+    static_assert(NG % 4 == 0, "four consecutive groups of a thread share a minimum");
+    extern __shared__ float lds[];
+    float *best = lds;                                  // [2][G]
+    float *red_v = best + 2 * G;                        // [1024]
+    int *red_i = reinterpret_cast<int *>(red_v + kVitThreads);
+    const int j = threadIdx.x;
+    const int64_t row = blockIdx.x;
+
+    float rho[NS];
+    uint32_t val[NS / 2];                               // the states' alphabet values, two fp16 a register
+#pragma unroll
+    for (int r = 0; r < NS; r++) {
+        const uint32_t s = ((uint32_t)(r & 3) << (L - 2)) | (uint32_t)(NG * j + (r >> 2));
+        const uint32_t a = alphabet[s];
+        if (r & 1) val[r >> 1] |= a << 16;
+        else val[r >> 1] = a;
+        rho[r] = (s == 0) ? 0.f : INFINITY;
+    }
+    const float *tg = targets + row * steps;
+    const float *wt = WEIGHTED ? weights + row * weights_row_stride : nullptr;
+    uint32_t *back_row = back + row * steps * (int64_t)kVitThreads;
+    float x = tg[0], c = WEIGHTED ? wt[0] : 1.f;
+    for (int t = 0; t < steps; t++) {
+        const int tn = t + 1 < steps ? t + 1 : t;
+        const float nx = tg[tn], nc = WEIGHTED ? wt[tn] : 1.f;
+        float *bw = best + (t & 1) * G;
+        uint32_t bp = 0;
+#pragma unroll
+        for (int gi = 0; gi < NG; gi++) {
+            float m = rho[4 * gi];
+            uint32_t arg = 0;
+#pragma unroll
+            for (int d = 1; d < 4; d++) {
+                const bool lt = rho[4 * gi + d] < m;       // the first minimum wins
+                m = lt ? rho[4 * gi + d] : m;
+                arg = lt ? (uint32_t)d : arg;
+            }
+            bw[NG * j + gi] = m;
+            bp |= arg << (2 * gi);
+        }
+        back_row[(int64_t)t * kVitThreads + j] = bp;
+        __syncthreads();       // one barrier a step: the halves of `best` take turns (see above)
+        // state (d << (L-2)) | g comes from group (d << (L-4)) | (g >> 2); g >> 2 = (NG/4) * j + gi / 4
+#pragma unroll
+        for (int d = 0; d < 4; d++) {
+            const float *brun = bw + (d << (L - 4)) + (NG / 4) * j;
+            float bq[NG / 4];
+            if constexpr (NG / 4 == 4) {
+                const float4 b = *reinterpret_cast<const float4 *>(brun);
+                bq[0] = b.x, bq[1] = b.y, bq[2] = b.z, bq[3] = b.w;
+            } else {
+#pragma unroll
+                for (int q = 0; q < NG / 4; q++) bq[q] = brun[q];
+            }
+#pragma unroll
+            for (int gi = 0; gi < NG; gi++) {
+                const int r = 4 * gi + d;
+                const float dd = (r & 1) ? sub_half_hi(x, val[r >> 1]) : sub_half_lo(x, val[r >> 1]);
+                float sq = dd * dd;
+                if (WEIGHTED) sq = c * sq;                 // rptc.py:32: c * (x - a)**2
+                rho[r] = bq[gi >> 2] + sq;
+            }
+        }
+        x = nx, c = nc;
+    }
+
+    float mv = rho[0];
+    int mi = NG * j;
+#pragma unroll
+    for (int d = 0; d < 4; d++) {
+#pragma unroll
+        for (int gi = 0; gi < NG; gi++) {
+            const float v = rho[4 * gi + d];
+            const int s = (d << (L - 2)) | (NG * j + gi);
+            if (v < mv) {
+                mv = v;
+                mi = s;
+            }
+        }
+    }
+    red_v[j] = mv;
+    red_i[j] = mi;
+    __syncthreads();
+    for (int width = kVitThreads / 2; width > 0; width >>= 1) {
+        if (j < width) {
+            const float ov = red_v[j + width];
+            const int oi = red_i[j + width];
+            if (ov < red_v[j] || (ov == red_v[j] && oi < red_i[j])) {
+                red_v[j] = ov;
+                red_i[j] = oi;
+            }
+        }
+        __syncthreads();
+    }
+    if (j == 0) {
+        end_state[row] = red_i[0];
+        cost[row] = red_v[0];
+    }
+}
+
+template <int L>
+__global__ __launch_bounds__(64) void viterbi_scalar_trace_kernel(const uint32_t *__restrict__ back,
+                                                                  const int32_t *__restrict__ end_state,
+                                                                  uint8_t *__restrict__ symbols, int rows, int steps)
+{
+    constexpr int NG = (1 << L) / 4 / kVitThreads;
+    const int row = blockIdx.x * 64 + threadIdx.x;
+    if (row >= rows) return;
+    const uint32_t *back_row = back + (int64_t)row * steps * kVitThreads;
+    uint8_t *sym = symbols + (int64_t)row * steps;
+    uint32_t state = (uint32_t)end_state[row];
+    for (int t = steps - 1; t >= 0; t--) {
+        sym[t] = (uint8_t)(state & 3u);
+        const uint32_t low = state >> 2;                // the predecessor's low L-2 bits = the group
+        const uint32_t bp = back_row[(int64_t)t * kVitThreads + low / NG];
+        state = (((bp >> (2 * (low % NG))) & 3u) << (L - 2)) | low;
+    }
+}
+
 // one thread per row walks the back pointers from the end state (rptc.py:60-65)
 __global__ __launch_bounds__(64) void viterbi_trace_kernel(const uint16_t *__restrict__ back,
                                                            const int32_t *__restrict__ end_state,
@@ -205,9 +359,19 @@ static int vit_allow_lds(K kernel)
                                     kVitLdsBytes);
 }
 
+template <typename K>
+static int vit_allow_scalar_lds(K kernel, int bytes)
+{
+    return (int)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+}
+
 int prepare_viterbi()
 {
     int rc;
+    if ((rc = vit_allow_scalar_lds(viterbi_scalar_kernel<16, false>, scalar_lds_bytes(16)))) return rc;
+    if ((rc = vit_allow_scalar_lds(viterbi_scalar_kernel<16, true>, scalar_lds_bytes(16)))) return rc;
+    if ((rc = vit_allow_scalar_lds(viterbi_scalar_kernel<14, false>, scalar_lds_bytes(14)))) return rc;
+    if ((rc = vit_allow_scalar_lds(viterbi_scalar_kernel<14, true>, scalar_lds_bytes(14)))) return rc;
     if ((rc = vit_allow_lds(viterbi_pairs_kernel<6, false>))) return rc;
     if ((rc = vit_allow_lds(viterbi_pairs_kernel<6, true>))) return rc;
     if ((rc = vit_allow_lds(viterbi_pairs_kernel<8, false>))) return rc;
@@ -222,14 +386,58 @@ static void launch_viterbi(const float *targets, const float *weights, int64_t w
                        weights, weights_row_stride, codebook, back, end_state, cost, (int)steps);
 }
 
+template <int L, bool WEIGHTED>
+static void launch_viterbi_scalar(const float *targets, const float *weights, int64_t weights_row_stride,
+                                  const uint16_t *alphabet, uint32_t *back, uint8_t *symbols, int32_t *end_state,
+                                  float *cost, int64_t rows, int64_t steps, hipStream_t s)
+{
+    hipLaunchKernelGGL((viterbi_scalar_kernel<L, WEIGHTED>), dim3((unsigned)rows), dim3(kVitThreads), scalar_lds_bytes(L), s,
+                       targets, weights, weights_row_stride, alphabet, back, end_state, cost, (int)steps);
+    hipLaunchKernelGGL(viterbi_scalar_trace_kernel<L>, dim3((unsigned)((rows + 63) / 64)), dim3(64), 0, s, back, end_state,
+                       symbols, (int)rows, (int)steps);
+}
+
 }  // namespace rptc
 
 using namespace rptc;
+
+extern "C" int rptc_viterbi_scalar(const float *targets, const float *weights, int64_t weights_row_stride,
+                                   const uint16_t *alphabet, int L, void *scratch, uint8_t *symbols, int32_t *end_state,
+                                   float *cost, int64_t rows, int64_t steps, void *stream, float *ms)
+{
+    if (!targets || !alphabet || !scratch || !symbols || !end_state || !cost) return RPTC_ENULL;
+    if (L != 16 && L != 14) return RPTC_ESHAPE;
+    if (rows < 1 || steps < 1 || weights_row_stride < 0) return RPTC_ESHAPE;
+    if (weights && weights_row_stride != 0 && weights_row_stride < steps) return RPTC_ESHAPE;
+    if (rows >= ((int64_t)1 << 24) || steps >= ((int64_t)1 << 24)) return RPTC_ELIMIT;
+    DeviceInfo *dev;
+    int rc = device_info(&dev);
+    if (rc) return rc;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    Timer t;
+    rc = t.begin(dev, s, ms);
+    if (rc) return rc;
+    uint32_t *back = static_cast<uint32_t *>(scratch);
+    if (L == 16) {
+        if (weights) launch_viterbi_scalar<16, true>(targets, weights, weights_row_stride, alphabet, back, symbols, end_state, cost, rows, steps, s);
+        else launch_viterbi_scalar<16, false>(targets, weights, weights_row_stride, alphabet, back, symbols, end_state, cost, rows, steps, s);
+    } else {
+        if (weights) launch_viterbi_scalar<14, true>(targets, weights, weights_row_stride, alphabet, back, symbols, end_state, cost, rows, steps, s);
+        else launch_viterbi_scalar<14, false>(targets, weights, weights_row_stride, alphabet, back, symbols, end_state, cost, rows, steps, s);
+    }
+    return t.end();
+}
 
 extern "C" int64_t rptc_viterbi_scratch_bytes(int64_t rows, int64_t steps)
 {
     if (rows < 1 || steps < 1) return 0;
     return rows * steps * (int64_t)kVitThreads * 2;
+}
+
+extern "C" int64_t rptc_viterbi_scalar_scratch_bytes(int64_t rows, int64_t steps)
+{
+    if (rows < 1 || steps < 1) return 0;
+    return rows * steps * (int64_t)kVitThreads * 4;
 }
 
 extern "C" int rptc_viterbi_pairs(const float *targets, const float *weights, int64_t weights_row_stride,

@@ -24,7 +24,8 @@ a stream stands for), ``decompress_matmul_16_{6,8}_1`` and ``decompress_matmul_b
 the matrix cores), ``decompress_matvec_bits`` (2, 3, 4 bits per weight), ``decompress_matvec_silu`` and
 ``decompress_matvec_rmsnorm`` (the mat-vec with a decoder layer's element-wise step in its prologue),
 ``decompress_matvec_hadamard`` (with the sign-Hadamard transform of its activations in its prologue),
-``sign_hadamard``, ``viterbi_pairs`` (the quantizer's trellis search, rptc.py:13-71, as a kernel).
+``sign_hadamard``, ``viterbi_pairs`` and ``viterbi_scalar`` (the quantizer's trellis search, rptc.py:13-71,
+as kernels: for the hashed pair stream and for the reference's own scalar trellis).
 Sub-modules: ``packing`` (symbols -> streams), ``quantize`` (the quantizer around that search),
 ``linear`` (``QuantizedLinear``, ``patch_model``), ``llama_decode`` (a Llama-shaped decode loop),
 ``eval_ppl`` (perplexity on a token file).
@@ -64,6 +65,8 @@ _SIGNATURES = {
     "rptc_decompress_matmul": ([_VP, _VP, _VP, _VP, _I64, _I64, _I64, _INT, _INT, _VP, _FP], _INT),
     "rptc_decompress_matmul_bits": ([_VP, _VP, _VP, _VP, _I64, _I64, _I64, _INT, _INT, _INT, _VP, _FP], _INT),
     "rptc_viterbi_scratch_bytes": ([_I64, _I64], _I64),
+    "rptc_viterbi_scalar_scratch_bytes": ([_I64, _I64], _I64),
+    "rptc_viterbi_scalar": ([_VP, _VP, _I64, _VP, _INT, _VP, _VP, _VP, _VP, _I64, _I64, _VP, _FP], _INT),
     "rptc_viterbi_pairs": ([_VP, _VP, _I64, _VP, _VP, _VP, _VP, _VP, _I64, _I64, _INT, _VP, _FP], _INT),
     "rptc_sign_hadamard": ([_VP, _VP, _VP, _I64, _I64, _I64, _INT, _VP, _FP], _INT),
     "rptc_decompress_matvec_bits": ([_VP, _VP, _VP, _VP, _I64, _I64, _INT, _INT, _INT, _VP, _FP], _INT),
@@ -411,6 +414,47 @@ def viterbi_pairs(targets, codebook, weights=None):
                                     codebook.data_ptr(), scratch.data_ptr(), symbols.data_ptr(), end_state.data_ptr(),
                                     cost.data_ptr(), rows, steps, S, ctypes.c_void_p(stream),
                                     ctypes.byref(ms) if _timing else None)
+        _status(rc)
+        if not _timing:
+            torch.cuda.current_stream().synchronize()     # scratch is freed on return
+    return symbols, cost, end_state, float(ms.value)
+
+
+def viterbi_scalar(targets, alphabet, weights=None):
+    """The reference's trellis search as it stands (rptc.py:13-71, diag_only): 2^L states (L = 16 or 14 from the
+    alphabet's length), 2 stream bits and one value per step, state s emitting alphabet[s]; the symbols are what
+    ``decompress`` (L = 16) and ``decompress_matvec_t_{16,14}`` decode in CONTINUOUS mode.
+
+    targets: float32 [rows, steps]; alphabet: fp16 [2^L]; weights: None, float32 [steps] or [rows, steps] (the
+    reference's ``sum(corrections[index]**2)``).  Returns (symbols uint8 [rows, steps], cost float32 [rows],
+    end_state int32 [rows], elapsed ms).  Needs rows * steps * 4096 bytes of scratch."""
+    _check_input(targets, "targets")
+    _check_input(alphabet, "alphabet")
+    _check(targets.dtype == torch.float32 and targets.dim() == 2, "targets must be float32 [rows, steps]")
+    _check(alphabet.dtype == torch.float16 and alphabet.numel() in (1 << 14, 1 << 16),
+           "alphabet must be fp16 of length 2^14 or 2^16")
+    rows, steps = targets.shape
+    _check(rows >= 1 and steps >= 1, "rows >= 1 and steps >= 1")
+    L = 14 if alphabet.numel() == 1 << 14 else 16
+    stride = 0
+    if weights is not None:
+        _check_input(weights, "weights")
+        _check(weights.dtype == torch.float32, "weights must be float32")
+        _check(tuple(weights.shape) in ((steps,), (rows, steps)), "weights must be [steps] or [rows, steps]")
+        stride = 0 if weights.dim() == 1 else steps
+    device = targets.device
+    lib = library()
+    with torch.cuda.device(device):
+        scratch = torch.empty(lib.rptc_viterbi_scalar_scratch_bytes(rows, steps), dtype=torch.uint8, device=device)
+        symbols = torch.empty((rows, steps), dtype=torch.uint8, device=device)
+        end_state = torch.empty(rows, dtype=torch.int32, device=device)
+        cost = torch.empty(rows, dtype=torch.float32, device=device)
+        ms = ctypes.c_float(0.0)
+        stream = torch.cuda.current_stream().cuda_stream
+        rc = lib.rptc_viterbi_scalar(targets.data_ptr(), weights.data_ptr() if weights is not None else None, stride,
+                                     alphabet.data_ptr(), L, scratch.data_ptr(), symbols.data_ptr(), end_state.data_ptr(),
+                                     cost.data_ptr(), rows, steps, ctypes.c_void_p(stream),
+                                     ctypes.byref(ms) if _timing else None)
         _status(rc)
         if not _timing:
             torch.cuda.current_stream().synchronize()     # scratch is freed on return

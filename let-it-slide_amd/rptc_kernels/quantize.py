@@ -67,6 +67,48 @@ def viterbi_pairs(targets, table, weights=None, state_bits=STATE_BITS, step_bits
     return symbols, cost
 
 
+def viterbi_scalar(targets, alphabet, weights=None):
+    """The reference's search as it stands (rptc.py:13-71, diag_only): 2 bits a step, state s emits alphabet[s].
+    targets [rows, steps] float; alphabet [2^L]; weights None or [rows, steps].  Returns (symbols int64
+    [rows, steps], cost float [rows])."""
+    alphabet = alphabet.to(torch.float32).reshape(-1)
+    L = alphabet.numel().bit_length() - 1
+    w = None if weights is None else torch.stack([weights, torch.zeros_like(weights)], dim=2)
+    table = torch.stack([alphabet, torch.zeros_like(alphabet)], dim=1)       # second value: always 0 error
+    tg = torch.stack([targets, torch.zeros_like(targets)], dim=2)
+    return viterbi_pairs(tg, table, w, state_bits=L, step_bits=2)
+
+
+def quantize_matrix_scalar(W, alphabet, importance=None, rows_per_batch=None):
+    """Quantize W [m, n] to 2-bit symbols [m, n] for the scalar-LUT streams (``packing.pack_rowmajor`` ->
+    ``decompress``, ``packing.pack_transposed`` -> ``decompress_matvec_t_*``, CONTINUOUS mode): the reference's
+    quantizer (rptc.py:13-71) row by row.  alphabet: [2^16] or [2^14]; importance: optional [n] per-column weight.
+    Returns (symbols int64 [m, n] on the CPU, mse float).  A matrix on the GPU is searched by the HIP kernel
+    (``rptc_kernels.viterbi_scalar``)."""
+    W = torch.as_tensor(W)
+    m, n = W.shape
+    dev = W.device
+    Wf = W.to(torch.float32).contiguous()
+    imp = None if importance is None else torch.as_tensor(importance, dtype=torch.float32, device=dev).contiguous()
+    out = torch.empty((m, n), dtype=torch.int64)
+    total = 0.0
+    if W.is_cuda:
+        import rptc_kernels as rk
+        ab16 = torch.as_tensor(alphabet).to(dev).to(torch.float16).contiguous()
+        rows_per_batch = rows_per_batch or max(1, min(m, (1 << 30) // (4096 * n)))
+    else:
+        rows_per_batch = rows_per_batch or 16
+    for r0 in range(0, m, rows_per_batch):
+        tg = Wf[r0:r0 + rows_per_batch]
+        if W.is_cuda:
+            sym, cost, _, _ = rk.viterbi_scalar(tg, ab16, imp)
+        else:
+            sym, cost = viterbi_scalar(tg, torch.as_tensor(alphabet), None if imp is None else imp.expand(tg.size(0), -1))
+        out[r0:r0 + rows_per_batch] = sym.cpu()
+        total += cost.sum().item()
+    return out, total / (m * n)
+
+
 def quantize_matrix(W, codebook, S=8, importance=None, rows_per_batch=64, bits=2):
     """Quantize W [m, n] (n % 64 == 0) to symbols of 2*bits bits [m, n/2] in stream order, for the decoder
     of ``decompress_matvec_*`` (bits == 2) or ``decompress_matvec_bits`` in CONTINUOUS mode.  importance:

