@@ -337,7 +337,45 @@ __device__ __forceinline__ void matvec_body(
             }
         }
     };
-    load_batch(it_begin);
+    // The first batch is requested by every lane of every wave, whatever the wave holds: a request
+    // under a condition cannot be counted by the compiler, which then waits for all loads in
+    // flight where it needs only the activations, and the staging below (and the element-wise
+    // prologues) would start when the stream data has arrived instead of while it is on its way.
+    // A lane past the item's rows repeats the last lane's address; a slot past the wave's items
+    // repeats the wave's first item (the first word of the stream for a wave with none).
+    auto load_first = [&]() {
+        const uint32_t *first_base = comp;
+        int first_nact = 1;
+#pragma unroll
+        for (int u = 0; u < kBatch; u++) {
+            const bool have = it_begin + u < it_end;
+            const int row_first = ld_idx * ld.rows_per_item;           // row inside the block
+            const int rows_here = min(ld.rows_per_item, rows - row_first);
+            const uint32_t *item_base = comp + (size_t)(ld.elem0 + (uint32_t)(row0 + row_first) * (uint32_t)ld.lanes) * WORDS;
+            if (u == 0 && have) {
+                first_base = item_base;
+                first_nact = rows_here * ld.lanes;
+            }
+            const uint32_t *wave_base = have ? item_base : first_base;
+            const int nact = have ? rows_here * ld.lanes : first_nact;
+            buf[u] = load_stream<WORDS>(wave_base, min(lane, nact - 1));
+            if (MODE == RPTC_CONTINUOUS) {
+                // the word in front of a row: last word of the row's lane 31 in the slab before
+                // (read by all lanes of the row; used by its first lane, and only past slab 0)
+                const bool prev = have && ld_slab > 0;
+                const int sub = min(ld_slab < T ? lane >> 5 : lane / ld.lanes, rows_here - 1);
+                const uint32_t *row_base =
+                    prev ? comp + (((size_t)(ld_slab - 1) * m + row0 + row_first) * 32 + 31) * WORDS + WORDS - 1 : comp;
+                cw[u] = row_base[sub * (prev ? 32 * WORDS : 0)];
+            }
+            if (have && ++ld_idx == ld.items) {
+                ld_idx = 0;
+                ld_slab++;
+                ld = view(ld_slab);
+            }
+        }
+    };
+    load_first();
     RPTC_STAMP(1);
 
     // the element-wise step in front of the product, on the registers the small loads filled
@@ -469,7 +507,7 @@ __device__ __forceinline__ void matvec_body(
             // Previous lane's last word.  Lane 0 of a row keeps its own as written
             // (inference.cu:232: the shuffle hands lane 0 its own value back).
             const uint32_t last = cur[u].w[WORDS - 1];
-            const uint32_t own = MODE == RPTC_CONTINUOUS ? ccw[u] : last;
+            const uint32_t own = MODE == RPTC_CONTINUOUS ? (slab > 0 ? ccw[u] : 0u) : last;
             float sum;
             if constexpr (BITS == 2) {
                 float a0, a1, a2, a3;
