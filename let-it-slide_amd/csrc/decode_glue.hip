@@ -103,9 +103,10 @@ __global__ __launch_bounds__(256) void rope_cache_kernel(const uint16_t *__restr
 // acc = sum exp(score - m) * V; they go to a static scratch buffer with device-scope stores, and
 // the workgroup that arrives last at the head's counter merges the pieces in piece order:
 // out = sum_i acc_i * exp(m_i - M) / sum_i l_i * exp(m_i - M).  Every sum has a fixed order.
-// Scores: hd/8 lanes share a key (16 bytes of it each) and add their partial dot products with
-// shuffles.  Values: the same lanes read 16 bytes of a value row each and keep 8 output
-// dimensions; the 256 / (hd/8) interleaved key groups are added in a fixed order.
+// hd/8 lanes share a key (16 bytes of it each), add their partial dot products with shuffles, and
+// read 16 bytes of the key's value row each (8 output dimensions).  Such a group keeps a running
+// softmax over its own keys (maximum, sum of exponentials, unnormalised value sum), the groups of
+// a wave are merged with shuffles and the waves through LDS, always in the same order.
 // ROPE = true: q is the projection output [q | k | v]; every workgroup rotates its head's q into
 // LDS, and the one whose piece holds *pos also rotates k and appends k and v to the caches (as
 // rope_cache_kernel does); it uses the new row from LDS.
@@ -121,14 +122,12 @@ template <bool ROPE>
 __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(
     const uint16_t *__restrict__ q, uint16_t *k_cache, uint16_t *v_cache, const uint16_t *__restrict__ cos_t,
     const uint16_t *__restrict__ sin_t, const int64_t *__restrict__ pos_p, uint16_t *__restrict__ out,
-    float *__restrict__ parts, uint32_t *__restrict__ arrived, int heads, int hd, int max_len, int splits,
-    int chunk_cap)
+    float *__restrict__ parts, uint32_t *__restrict__ arrived, int heads, int hd, int max_len, int splits)
 {
     extern __shared__ float lds_f[];
     RPTC_ATTN_STAMP(0);
-    float *scores = lds_f;                       // [chunk_cap]
-    float *scratch = lds_f + chunk_cap;          // [16] (chunk_cap is a multiple of 16)
-    float *acc = scratch + 16;                   // [slots][hd] = 2048 floats
+    float *scratch = lds_f;                      // [16]: the "came last" flag
+    float *acc = scratch + 16;                   // the waves' sums [waves][hd], then their m and l: < 2048 floats
     uint16_t *q_rot = reinterpret_cast<uint16_t *>(acc + 2048);   // [3][hd] halves (q, new k, new v), ROPE only
     const int h = blockIdx.x / splits, sp = blockIdx.x - h * splits, tid = threadIdx.x;
     const int len = (int)*pos_p + 1;
@@ -201,7 +200,10 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(
     }
 
     RPTC_ATTN_STAMP(1);
-    // scores
+    // The lanes that share a key (a group) keep a running softmax of their own keys: maximum m,
+    // sum l of exp(score - m) and the unnormalised value sum a8 (8 output dimensions a lane), so
+    // nothing leaves the group before the piece's last key.  Then the groups of a wave are merged
+    // with shuffles, the waves through LDS: one barrier for the whole piece.
     float qf[8];
     {
         const uint4 v = ROPE ? *reinterpret_cast<const uint4 *>(q_rot + 8 * sub)
@@ -213,8 +215,16 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(
             qf[2 * u + 1] = half_bits_to_float((uint16_t)(w[u] >> 16));
         }
     }
+    float m_g = -INFINITY, l_g = 0.f, a8[8];
+#pragma unroll
+    for (int c = 0; c < 8; c++) a8[c] = 0.f;
     for (int s0 = 0; s0 < cnt; s0 += kKeysInFlight * slots) {
-        if (s0 > 0) load_keys(s0);
+        if (s0 > 0) {
+            load_keys(s0);
+            load_values(s0);
+        }
+        float sc[kKeysInFlight];
+        float m_new = m_g;
 #pragma unroll
         for (int u = 0; u < kKeysInFlight; u++) {
             const int s = s0 + u * slots + slot;
@@ -228,34 +238,23 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(
                 dot += half_bits_to_float((uint16_t)(w[c] >> 16)) * qf[2 * c + 1];
             }
             for (int off = lanes_per_key >> 1; off > 0; off >>= 1) dot += __shfl_xor(dot, off, 64);
-            if (s < cnt && sub == 0) scores[s] = dot * scale;
+            sc[u] = s < cnt ? dot * scale : -INFINITY;
+            m_new = fmaxf(m_new, sc[u]);
         }
-    }
-    __syncthreads();
-    RPTC_ATTN_STAMP(2);
-    float mx = -INFINITY;
-    for (int s = tid; s < cnt; s += kAttnThreads) mx = fmaxf(mx, scores[s]);
-    mx = block_max(mx, scratch);
-    float sum = 0.f;
-    for (int s = tid; s < cnt; s += kAttnThreads) {
-        const float p = __expf(scores[s] - mx);
-        scores[s] = p;
-        sum += p;
-    }
-    sum = block_sum(sum, scratch);               // (its barriers also publish the new scores)
-
-    // values: thread (slot, sub) adds its keys' rows, 8 output dimensions each
-    float a8[8];
+        if (s0 == 0) RPTC_ATTN_STAMP(2);
+        // a group with no key yet keeps m = -inf: its factors must be 0, not exp(-inf - -inf)
+        const float keep = m_g == -INFINITY ? 0.f : __expf(m_g - m_new);
+        l_g *= keep;
 #pragma unroll
-    for (int c = 0; c < 8; c++) a8[c] = 0.f;
-    for (int s0 = 0; s0 < cnt; s0 += kKeysInFlight * slots) {
-        if (s0 > 0) load_values(s0);
+        for (int c = 0; c < 8; c++) a8[c] *= keep;
+        m_g = m_new;
 #pragma unroll
         for (int u = 0; u < kKeysInFlight; u++) {
             const int s = s0 + u * slots + slot;
             uint4 vq = vv[u];
             if (owns_pos && s_begin + s == pos) vq = *reinterpret_cast<const uint4 *>(v_new + 8 * sub);
-            const float p = s < cnt ? scores[s] : 0.f;
+            const float p = sc[u] == -INFINITY ? 0.f : __expf(sc[u] - m_g);
+            l_g += p;
             const uint32_t w[4] = {vq.x, vq.y, vq.z, vq.w};
 #pragma unroll
             for (int c = 0; c < 4; c++) {
@@ -265,12 +264,40 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(
         }
     }
     RPTC_ATTN_STAMP(3);
+    // the groups of a wave (lanes sub, sub + lanes_per_key, ...): butterfly over the lane bits above
+    // the group's, in a fixed order
+    for (int off = lanes_per_key; off < 64; off <<= 1) {
+        const float m_o = __shfl_xor(m_g, off, 64), l_o = __shfl_xor(l_g, off, 64);
+        const float m_n = fmaxf(m_g, m_o);
+        const float f_s = m_g == -INFINITY ? 0.f : __expf(m_g - m_n), f_o = m_o == -INFINITY ? 0.f : __expf(m_o - m_n);
+        l_g = l_g * f_s + l_o * f_o;
 #pragma unroll
-    for (int c = 0; c < 8; c++) acc[slot * hd + 8 * sub + c] = a8[c];
+        for (int c = 0; c < 8; c++) a8[c] = a8[c] * f_s + __shfl_xor(a8[c], off, 64) * f_o;
+        m_g = m_n;
+    }
+    // the waves: [wave][hd] sums, then m and l of each wave behind them
+    constexpr int kWaves = kAttnThreads / 64;
+    float *w_acc = acc, *w_m = acc + kWaves * 256, *w_l = w_m + kWaves;
+    const int wave = tid >> 6, lane = tid & 63;
+    if (lane < lanes_per_key) {
+#pragma unroll
+        for (int c = 0; c < 8; c++) w_acc[wave * hd + 8 * sub + c] = a8[c];
+        if (lane == 0) {
+            w_m[wave] = m_g;
+            w_l[wave] = l_g;
+        }
+    }
     __syncthreads();
-    float y = 0.f;                               // thread i < hd: output dimension i of this piece
-    if (tid < hd)
-        for (int gidx = 0; gidx < slots; gidx++) y += acc[gidx * hd + tid];
+    float mx = w_m[0];
+#pragma unroll
+    for (int w = 1; w < kWaves; w++) mx = fmaxf(mx, w_m[w]);
+    float y = 0.f, sum = 0.f;                    // thread i < hd: output dimension i of this piece
+#pragma unroll
+    for (int w = 0; w < kWaves; w++) {
+        const float f = w_m[w] == -INFINITY ? 0.f : __expf(w_m[w] - mx);
+        sum += w_l[w] * f;
+        if (tid < hd) y += w_acc[w * hd + tid] * f;
+    }
     if (splits == 1) {
         if (tid < hd) out[h * hd + tid] = float_to_half_bits(y / sum);
         return;
@@ -392,13 +419,11 @@ static int launch_attn(const uint16_t *q, const uint16_t *cos_t, const uint16_t 
     if (splits > max_len / 16) splits = (int)(max_len / 16);
     if (splits < 1) splits = 1;
     if (heads * splits > kAttnMaxParts) splits = (int)(kAttnMaxParts / heads);
-    const int chunk_cap = (int)(((max_len + splits - 1) / splits + 15) & ~(int64_t)15);
-    const size_t lds = (size_t)(chunk_cap + 16 + 2048) * 4 + (size_t)hd * 6;
-    if (lds > 64 * 1024) return RPTC_ELIMIT;
+    const size_t lds = (size_t)(16 + 2048) * 4 + (size_t)hd * 6;
     const AttnScratch &sc = g_attn[dev->device];
     hipLaunchKernelGGL(attn_decode_kernel<ROPE>, dim3((unsigned)(heads * splits)), dim3(kAttnThreads), lds,
                        static_cast<hipStream_t>(stream), q, k_cache, v_cache, cos_t, sin_t, pos, out, sc.parts, sc.arrived,
-                       (int)heads, (int)hd, (int)max_len, splits, chunk_cap);
+                       (int)heads, (int)hd, (int)max_len, splits);
     return (int)hipGetLastError();
 }
 }  // namespace rptc
