@@ -374,6 +374,14 @@ def bench_quantize(a):
         "ms": round(best, 3), "state_updates_per_s": float(f"{updates / best * 1e3:.4e}"),
         "us_per_step_per_row_round": round(best * 1e3 / steps / (rows / 256), 3),
         "vector_ops_per_update": 5, "frac_of_valu_peak": round(updates * 5 / (best * 1e-3) / valu_peak, 4)}}
+    # 3 and 4 bits per weight: 6 and 8 stream bits per step, 64 and 256 predecessors per state
+    for bits in (3, 4):
+        b_ms = None
+        for _ in range(3):
+            _, _, _, ms = rk.viterbi_pairs(tg[:256], cb, bits=bits)
+            b_ms = ms if b_ms is None else min(b_ms, ms)
+        res[f"viterbi_pairs {bits} bits rows 256 steps 2048"] = {
+            "ms": round(b_ms, 3), "state_updates_per_s": float(f"{256 * steps * 65536 / b_ms * 1e3:.4e}")}
     # the reference's own trellis (2 bits and one alphabet value per step): 6 vector ops per update
     # (mixed-precision subtract, square, add, and the minimum over four predecessors)
     ab = torch.randn(1 << 16, generator=g, device="cuda").half()

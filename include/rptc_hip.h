@@ -233,6 +233,11 @@ int64_t rptc_viterbi_scalar_scratch_bytes(int64_t rows, int64_t steps);
 int rptc_viterbi_pairs(const float *targets, const float *weights, int64_t weights_row_stride,
                        const uint16_t *codebook, void *scratch, uint8_t *symbols, int32_t *end_state, float *cost,
                        int64_t rows, int64_t steps, int S, void *stream, float *ms);
+/* the same for the streams of rptc_decompress_matvec_bits: bits = 2, 3, 4 per weight, i.e. 4, 6, 8 stream
+ * bits per step and symbols 0..15, 0..63, 0..255 */
+int rptc_viterbi_pairs_bits(const float *targets, const float *weights, int64_t weights_row_stride,
+                            const uint16_t *codebook, void *scratch, uint8_t *symbols, int32_t *end_state, float *cost,
+                            int64_t rows, int64_t steps, int S, int bits, void *stream, float *ms);
 
 /*
  * The same search on the reference's own trellis (rptc.py:13-71 as it stands): 2^L states (L = 16 or 14),

@@ -8,6 +8,7 @@
 // shifts 4 new bits in and emits the two weights the state's hash selects, so a state s' has the
 // 16 predecessors (d << 12) | (s' >> 4).
 //
+// (The 3- and 4-bit streams take 6 and 8 bits a step: 64 and 256 predecessors, see vit_state.)
 // One workgroup of 1024 threads searches one row.  Thread j keeps the costs of 64 states in
 // registers: the four predecessor groups g = 4j .. 4j+3 with all 16 values of d, so the minimum
 // over a group's predecessors never leaves the thread.  A step is
@@ -53,7 +54,21 @@ __device__ __forceinline__ float pair_loss_weighted(float x0, float x1, float w0
     return c0 * (d0 * d0) + c1 * (d1 * d1);
 }
 
-template <int S, bool WEIGHTED>
+// Which state register r of thread j holds, for a trellis that takes STEP bits per step (a state has
+// 2^STEP predecessors (d << (16 - STEP)) | group, group = state >> STEP):
+//   STEP 4: r = 16 * gi + d, state (d << 12) | (4j + gi): four groups with their 16 predecessors;
+//   STEP 6: r = d,           state (d << 10) | j:          one group with its 64 predecessors;
+//   STEP 8: r = d % 64,      state (d << 8) | (j / 4), d = 64 * (j % 4) + r: a quarter of a group's 256
+//           predecessors; the four lanes of a group finish the minimum with two shuffles.
+template <int STEP>
+__device__ __forceinline__ uint32_t vit_state(int r, int j)
+{
+    if (STEP == 4) return ((uint32_t)(r & 15) << 12) | (uint32_t)(4 * j + (r >> 4));
+    if (STEP == 6) return ((uint32_t)r << 10) | (uint32_t)j;
+    return ((uint32_t)(64 * (j & 3) + r) << 8) | (uint32_t)(j >> 2);
+}
+
+template <int S, int STEP, bool WEIGHTED>
 __global__ __launch_bounds__(kVitThreads) void viterbi_pairs_kernel(
     const float *__restrict__ targets, const float *__restrict__ weights, int64_t weights_row_stride,
     const uint16_t *__restrict__ codebook, uint16_t *__restrict__ back, int32_t *__restrict__ end_state,
@@ -71,15 +86,14 @@ __global__ __launch_bounds__(kVitThreads) void viterbi_pairs_kernel(
     const int64_t row = blockIdx.x;
     const uint32_t loss_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(loss));
 
-    // Register r = 16 * gi + d holds state (d << 12) | (4j + gi).  code[r / 4] byte r % 4 is the row of
-    // the loss table the state reads: its codebook entry, with the hash's sign bit on top at S = 6
+    // code[r / 4] byte r % 4 is the row of the loss table the state of register r reads: its codebook entry, with the hash's sign bit on top at S = 6
     // (at S = 8 the sign bit is the entry's own top bit, inference.cu:253-262).  A row starts every
     // 256 bytes, so one byte permute makes the address out of the code and the thread's copy.
     float rho[64];
     uint32_t code[16];
 #pragma unroll
     for (int r = 0; r < 64; r++) {
-        const uint32_t s = ((uint32_t)(r & 15) << 12) | (uint32_t)(4 * j + (r >> 4));
+        const uint32_t s = vit_state<STEP>(r, j);
         const uint32_t prod = s * (s + 1u);
         const uint32_t c = S == 8 ? (prod >> 8) & 0xFFu : ((prod >> 8) & 63u) | (((prod >> 15) & 1u) << 6);
         if (r & 3) code[r >> 2] |= c << (8 * (r & 3));
@@ -115,55 +129,90 @@ __global__ __launch_bounds__(kVitThreads) void viterbi_pairs_kernel(
         lm[1] = l4;
 
         float *bw = best + (t & 1) * kVitGroups;
-        uint32_t nib = 0;
-#pragma unroll
-        for (int gi = 0; gi < 4; gi++) {
-            float m = rho[16 * gi];
-            uint32_t arg = 0;
-#pragma unroll
-            for (int d = 1; d < 16; d++) {
-                const bool lt = rho[16 * gi + d] < m;      // the first minimum wins
-                m = lt ? rho[16 * gi + d] : m;
-                arg = lt ? (uint32_t)d : arg;
-            }
-            bw[4 * j + gi] = m;
-            nib |= arg << (4 * gi);
-        }
-        back_row[(int64_t)t * kVitThreads + j] = (uint16_t)nib;
-        __syncthreads();
-
         const uint32_t copy4_t = copy4 + (uint32_t)(t & 1) * (kVitCopies * 4u);
-        // state (d << 12) | g comes from group ((d << 12) | g) >> 4 = (d << 8) | (j >> 2) for all four g
-#pragma unroll
-        for (int d = 0; d < 16; d++) {
-            const float b = bw[(d << 8) | (j >> 2)];
+        // byte 0 of a gather's address: the copy's offset; byte 1: the state's code; the rest zero
+        auto loss_of = [&](int r) {
+            const uint32_t off = perm(code[r >> 2], copy4_t, 0x0C0C0400u + ((uint32_t)(r & 3) << 8));
+            return __builtin_bit_cast(float, lds_read_abs(off));
+        };
+        if constexpr (STEP == 4) {
+            uint32_t nib = 0;
 #pragma unroll
             for (int gi = 0; gi < 4; gi++) {
-                const int r = 16 * gi + d;
-                // byte 0: the copy's offset; byte 1: the state's code; the rest zero
-                const uint32_t off = perm(code[r >> 2], copy4_t, 0x0C0C0400u + ((uint32_t)(r & 3) << 8));
-                rho[r] = b + __builtin_bit_cast(float, lds_read_abs(off));
+                float m = rho[16 * gi];
+                uint32_t arg = 0;
+#pragma unroll
+                for (int d = 1; d < 16; d++) {
+                    const bool lt = rho[16 * gi + d] < m;      // the first minimum wins
+                    m = lt ? rho[16 * gi + d] : m;
+                    arg = lt ? (uint32_t)d : arg;
+                }
+                bw[4 * j + gi] = m;
+                nib |= arg << (4 * gi);
             }
-            // a few gathers in flight at a time: all 64 at once would push registers out to memory
-            if ((d & 1) == 1) __builtin_amdgcn_sched_barrier(0);
+            back_row[(int64_t)t * kVitThreads + j] = (uint16_t)nib;
+            __syncthreads();
+            // state (d << 12) | g comes from group ((d << 12) | g) >> 4 = (d << 8) | (j >> 2) for all four g
+#pragma unroll
+            for (int d = 0; d < 16; d++) {
+                const float b = bw[(d << 8) | (j >> 2)];
+#pragma unroll
+                for (int gi = 0; gi < 4; gi++) rho[16 * gi + d] = b + loss_of(16 * gi + d);
+                // a few gathers in flight at a time: all 64 at once would push registers out to memory
+                if ((d & 1) == 1) __builtin_amdgcn_sched_barrier(0);
+            }
+        } else {
+            float m = rho[0];
+            uint32_t arg = STEP == 8 ? 64u * (uint32_t)(j & 3) : 0u;
+#pragma unroll
+            for (int r = 1; r < 64; r++) {
+                const bool lt = rho[r] < m;                    // the first minimum wins
+                m = lt ? rho[r] : m;
+                arg = lt ? (STEP == 8 ? 64u * (uint32_t)(j & 3) : 0u) + (uint32_t)r : arg;
+            }
+            if constexpr (STEP == 8) {
+                // the other three quarters of the group sit in the neighbouring lanes; equal minima
+                // go to the lower d, i.e. the lower lane
+#pragma unroll
+                for (int off = 1; off <= 2; off <<= 1) {
+                    const float om = __shfl_xor(m, off, 64);
+                    const uint32_t oarg = __shfl_xor(arg, off, 64);
+                    const bool take = om < m || (om == m && oarg < arg);
+                    m = take ? om : m;
+                    arg = take ? oarg : arg;
+                }
+                if ((j & 3) == 0) {
+                    bw[j >> 2] = m;
+                    back_row[(int64_t)t * kVitThreads + j] = (uint16_t)arg;
+                }
+            } else {
+                bw[j] = m;
+                back_row[(int64_t)t * kVitThreads + j] = (uint16_t)arg;
+            }
+            __syncthreads();
+            // STEP 6: state (d << 10) | j comes from group (d << 4) | (j >> 6);
+            // STEP 8: state (d << 8) | g comes from group d
+#pragma unroll
+            for (int r = 0; r < 64; r++) {
+                const float b = STEP == 6 ? bw[(r << 4) | (j >> 6)] : bw[64 * (j & 3) + r];
+                rho[r] = b + loss_of(r);
+                if ((r & 7) == 7) __builtin_amdgcn_sched_barrier(0);
+            }
         }
         x0 = nx0, x1 = nx1, c0 = nc0, c1 = nc1;
     }
 
     // cheapest end state, the lowest index among equals: in a thread the states are visited in
-    // rising order (d outer, gi inner)
+    // rising order (STEP 4: d outer, gi inner; otherwise r)
     float mv = rho[0];
-    int mi = 4 * j;
+    int mi = (int)vit_state<STEP>(0, j);
 #pragma unroll
-    for (int d = 0; d < 16; d++) {
-#pragma unroll
-        for (int gi = 0; gi < 4; gi++) {
-            const float v = rho[16 * gi + d];
-            const int s = (d << 12) | (4 * j + gi);
-            if (v < mv) {
-                mv = v;
-                mi = s;
-            }
+    for (int a = 0; a < 64; a++) {
+        const int r = STEP == 4 ? 16 * (a & 3) + (a >> 2) : a;
+        const float v = rho[r];
+        if (v < mv) {
+            mv = v;
+            mi = (int)vit_state<STEP>(r, j);
         }
     }
     red_v[j] = mv;
@@ -335,6 +384,7 @@ __global__ __launch_bounds__(64) void viterbi_scalar_trace_kernel(const uint32_t
 }
 
 // one thread per row walks the back pointers from the end state (rptc.py:60-65)
+template <int STEP>
 __global__ __launch_bounds__(64) void viterbi_trace_kernel(const uint16_t *__restrict__ back,
                                                            const int32_t *__restrict__ end_state,
                                                            uint8_t *__restrict__ symbols, int rows, int steps)
@@ -345,10 +395,13 @@ __global__ __launch_bounds__(64) void viterbi_trace_kernel(const uint16_t *__res
     uint8_t *sym = symbols + (int64_t)row * steps;
     uint32_t state = (uint32_t)end_state[row];
     for (int t = steps - 1; t >= 0; t--) {
-        sym[t] = (uint8_t)(state & 15u);
-        const uint32_t low = state >> 4;                // the predecessor's low 12 bits = the group
-        const uint32_t nib = back_row[(int64_t)t * kVitThreads + (low >> 2)];
-        state = (((nib >> (4 * (low & 3u))) & 15u) << 12) | low;
+        sym[t] = (uint8_t)(state & ((1u << STEP) - 1u));
+        const uint32_t low = state >> STEP;             // the predecessor's low bits = the group
+        uint32_t d;
+        if (STEP == 4) d = (back_row[(int64_t)t * kVitThreads + (low >> 2)] >> (4 * (low & 3u))) & 15u;
+        else if (STEP == 6) d = back_row[(int64_t)t * kVitThreads + low];
+        else d = back_row[(int64_t)t * kVitThreads + 4 * low];
+        state = (d << (16 - STEP)) | low;
     }
 }
 
@@ -372,18 +425,31 @@ int prepare_viterbi()
     if ((rc = vit_allow_scalar_lds(viterbi_scalar_kernel<16, true>, scalar_lds_bytes(16)))) return rc;
     if ((rc = vit_allow_scalar_lds(viterbi_scalar_kernel<14, false>, scalar_lds_bytes(14)))) return rc;
     if ((rc = vit_allow_scalar_lds(viterbi_scalar_kernel<14, true>, scalar_lds_bytes(14)))) return rc;
-    if ((rc = vit_allow_lds(viterbi_pairs_kernel<6, false>))) return rc;
-    if ((rc = vit_allow_lds(viterbi_pairs_kernel<6, true>))) return rc;
-    if ((rc = vit_allow_lds(viterbi_pairs_kernel<8, false>))) return rc;
-    return vit_allow_lds(viterbi_pairs_kernel<8, true>);
+#define RPTC_VIT_ALLOW(STEP)                                                       \
+    if ((rc = vit_allow_lds(viterbi_pairs_kernel<6, STEP, false>))) return rc;     \
+    if ((rc = vit_allow_lds(viterbi_pairs_kernel<6, STEP, true>))) return rc;      \
+    if ((rc = vit_allow_lds(viterbi_pairs_kernel<8, STEP, false>))) return rc;     \
+    if ((rc = vit_allow_lds(viterbi_pairs_kernel<8, STEP, true>))) return rc;
+    RPTC_VIT_ALLOW(4)
+    RPTC_VIT_ALLOW(6)
+    RPTC_VIT_ALLOW(8)
+#undef RPTC_VIT_ALLOW
+    return 0;
 }
 
-template <int S, bool WEIGHTED>
+template <int S, int STEP>
 static void launch_viterbi(const float *targets, const float *weights, int64_t weights_row_stride, const uint16_t *codebook,
-                           uint16_t *back, int32_t *end_state, float *cost, int64_t rows, int64_t steps, hipStream_t s)
+                           uint16_t *back, uint8_t *symbols, int32_t *end_state, float *cost, int64_t rows, int64_t steps,
+                           hipStream_t s)
 {
-    hipLaunchKernelGGL((viterbi_pairs_kernel<S, WEIGHTED>), dim3((unsigned)rows), dim3(kVitThreads), kVitLdsBytes, s, targets,
-                       weights, weights_row_stride, codebook, back, end_state, cost, (int)steps);
+    if (weights)
+        hipLaunchKernelGGL((viterbi_pairs_kernel<S, STEP, true>), dim3((unsigned)rows), dim3(kVitThreads), kVitLdsBytes, s,
+                           targets, weights, weights_row_stride, codebook, back, end_state, cost, (int)steps);
+    else
+        hipLaunchKernelGGL((viterbi_pairs_kernel<S, STEP, false>), dim3((unsigned)rows), dim3(kVitThreads), kVitLdsBytes, s,
+                           targets, weights, weights_row_stride, codebook, back, end_state, cost, (int)steps);
+    hipLaunchKernelGGL(viterbi_trace_kernel<STEP>, dim3((unsigned)((rows + 63) / 64)), dim3(64), 0, s, back, end_state, symbols,
+                       (int)rows, (int)steps);
 }
 
 template <int L, bool WEIGHTED>
@@ -440,12 +506,12 @@ extern "C" int64_t rptc_viterbi_scalar_scratch_bytes(int64_t rows, int64_t steps
     return rows * steps * (int64_t)kVitThreads * 4;
 }
 
-extern "C" int rptc_viterbi_pairs(const float *targets, const float *weights, int64_t weights_row_stride,
-                                  const uint16_t *codebook, void *scratch, uint8_t *symbols, int32_t *end_state,
-                                  float *cost, int64_t rows, int64_t steps, int S, void *stream, float *ms)
+extern "C" int rptc_viterbi_pairs_bits(const float *targets, const float *weights, int64_t weights_row_stride,
+                                       const uint16_t *codebook, void *scratch, uint8_t *symbols, int32_t *end_state,
+                                       float *cost, int64_t rows, int64_t steps, int S, int bits, void *stream, float *ms)
 {
     if (!targets || !codebook || !scratch || !symbols || !end_state || !cost) return RPTC_ENULL;
-    if (S != 6 && S != 8) return RPTC_ESHAPE;
+    if ((S != 6 && S != 8) || bits < 2 || bits > 4) return RPTC_ESHAPE;
     if (rows < 1 || steps < 1 || weights_row_stride < 0) return RPTC_ESHAPE;
     if (weights && weights_row_stride != 0 && weights_row_stride < 2 * steps) return RPTC_ESHAPE;
     if (rows >= ((int64_t)1 << 24) || steps >= ((int64_t)1 << 24)) return RPTC_ELIMIT;
@@ -457,16 +523,18 @@ extern "C" int rptc_viterbi_pairs(const float *targets, const float *weights, in
     rc = t.begin(dev, s, ms);
     if (rc) return rc;
     uint16_t *back = static_cast<uint16_t *>(scratch);
-    if (S == 6) {
-        if (weights) launch_viterbi<6, true>(targets, weights, weights_row_stride, codebook, back, end_state, cost, rows, steps, s);
-        else launch_viterbi<6, false>(targets, weights, weights_row_stride, codebook, back, end_state, cost, rows, steps, s);
-    } else {
-        if (weights) launch_viterbi<8, true>(targets, weights, weights_row_stride, codebook, back, end_state, cost, rows, steps, s);
-        else launch_viterbi<8, false>(targets, weights, weights_row_stride, codebook, back, end_state, cost, rows, steps, s);
-    }
-    rc = (int)hipGetLastError();
-    if (rc) return rc;
-    hipLaunchKernelGGL(viterbi_trace_kernel, dim3((unsigned)((rows + 63) / 64)), dim3(64), 0, s, back, end_state, symbols,
-                       (int)rows, (int)steps);
+#define RPTC_VIT_GO(SS, BB)                                                                                        \
+    if (S == SS && bits == BB)                                                                                      \
+        launch_viterbi<SS, 2 * BB>(targets, weights, weights_row_stride, codebook, back, symbols, end_state, cost, rows, steps, s);
+    RPTC_VIT_GO(6, 2) RPTC_VIT_GO(6, 3) RPTC_VIT_GO(6, 4) RPTC_VIT_GO(8, 2) RPTC_VIT_GO(8, 3) RPTC_VIT_GO(8, 4)
+#undef RPTC_VIT_GO
     return t.end();
+}
+
+extern "C" int rptc_viterbi_pairs(const float *targets, const float *weights, int64_t weights_row_stride,
+                                  const uint16_t *codebook, void *scratch, uint8_t *symbols, int32_t *end_state,
+                                  float *cost, int64_t rows, int64_t steps, int S, void *stream, float *ms)
+{
+    return rptc_viterbi_pairs_bits(targets, weights, weights_row_stride, codebook, scratch, symbols, end_state, cost, rows,
+                                   steps, S, 2, stream, ms);
 }

@@ -68,6 +68,7 @@ _SIGNATURES = {
     "rptc_viterbi_scalar_scratch_bytes": ([_I64, _I64], _I64),
     "rptc_viterbi_scalar": ([_VP, _VP, _I64, _VP, _INT, _VP, _VP, _VP, _VP, _I64, _I64, _VP, _FP], _INT),
     "rptc_viterbi_pairs": ([_VP, _VP, _I64, _VP, _VP, _VP, _VP, _VP, _I64, _I64, _INT, _VP, _FP], _INT),
+    "rptc_viterbi_pairs_bits": ([_VP, _VP, _I64, _VP, _VP, _VP, _VP, _VP, _I64, _I64, _INT, _INT, _VP, _FP], _INT),
     "rptc_sign_hadamard": ([_VP, _VP, _VP, _I64, _I64, _I64, _INT, _VP, _FP], _INT),
     "rptc_decompress_matvec_bits": ([_VP, _VP, _VP, _VP, _I64, _I64, _INT, _INT, _INT, _VP, _FP], _INT),
     "rptc_matvec_bits_dense": ([_VP, _VP, _VP, _I64, _I64, _INT, _INT, _INT, _VP, _FP], _INT),
@@ -380,9 +381,10 @@ def sign_hadamard(x, signs, out, block=0, inverse=False):
     return float(ms.value)
 
 
-def viterbi_pairs(targets, codebook, weights=None):
+def viterbi_pairs(targets, codebook, weights=None, bits=2):
     """Exact Viterbi search on the trellis of ``decompress_matvec_16_{S}_1`` (65536 states, 4 stream bits
-    and two weights per step; S from the codebook length), the search of rptc.py:13-71.
+    and two weights per step; S from the codebook length), the search of rptc.py:13-71; ``bits`` = 3 or 4: the
+    trellis of ``decompress_matvec_bits`` (6 or 8 stream bits per step, symbols up to 63 or 255).
 
     targets: float32 [rows, steps, 2] (weight pairs in stream order); weights: None, float32 [steps, 2]
     (one importance set for all rows) or [rows, steps, 2].  Returns (symbols uint8 [rows, steps],
@@ -394,6 +396,7 @@ def viterbi_pairs(targets, codebook, weights=None):
     _check(codebook.dtype == torch.float16 and codebook.numel() in (128, 512), "codebook must be fp16 of length 128 or 512")
     rows, steps = targets.size(0), targets.size(1)
     _check(rows >= 1 and steps >= 1, "rows >= 1 and steps >= 1")
+    _check(bits in (2, 3, 4), "bits must be 2, 3 or 4")
     S = 6 if codebook.numel() == 128 else 8
     stride = 0
     if weights is not None:
@@ -410,10 +413,10 @@ def viterbi_pairs(targets, codebook, weights=None):
         cost = torch.empty(rows, dtype=torch.float32, device=device)
         ms = ctypes.c_float(0.0)
         stream = torch.cuda.current_stream().cuda_stream
-        rc = lib.rptc_viterbi_pairs(targets.data_ptr(), weights.data_ptr() if weights is not None else None, stride,
-                                    codebook.data_ptr(), scratch.data_ptr(), symbols.data_ptr(), end_state.data_ptr(),
-                                    cost.data_ptr(), rows, steps, S, ctypes.c_void_p(stream),
-                                    ctypes.byref(ms) if _timing else None)
+        rc = lib.rptc_viterbi_pairs_bits(targets.data_ptr(), weights.data_ptr() if weights is not None else None, stride,
+                                         codebook.data_ptr(), scratch.data_ptr(), symbols.data_ptr(), end_state.data_ptr(),
+                                         cost.data_ptr(), rows, steps, S, bits, ctypes.c_void_p(stream),
+                                         ctypes.byref(ms) if _timing else None)
         _status(rc)
         if not _timing:
             torch.cuda.current_stream().synchronize()     # scratch is freed on return

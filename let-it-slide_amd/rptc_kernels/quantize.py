@@ -113,7 +113,7 @@ def quantize_matrix(W, codebook, S=8, importance=None, rows_per_batch=64, bits=2
     """Quantize W [m, n] (n % 64 == 0) to symbols of 2*bits bits [m, n/2] in stream order, for the decoder
     of ``decompress_matvec_*`` (bits == 2) or ``decompress_matvec_bits`` in CONTINUOUS mode.  importance:
     optional [n] per-column weight (e.g. the Hessian diagonal, quantize_hf.py:164).  Returns (symbols int64
-    [m, n/2] on the CPU, mse float).  A matrix on the GPU at 2 bits per weight is searched by the HIP kernel
+    [m, n/2] on the CPU, mse float).  A matrix on the GPU is searched by the HIP kernel
     (``rptc_kernels.viterbi_pairs``), which chooses the same path as ``viterbi_pairs`` here bit for bit."""
     W = torch.as_tensor(W)
     m, n = W.shape
@@ -128,7 +128,7 @@ def quantize_matrix(W, codebook, S=8, importance=None, rows_per_batch=64, bits=2
         wts = torch.stack([imp[cols], imp[cols + 1]], dim=1).unsqueeze(0)
     out = torch.empty((m, n // 2), dtype=torch.int64)
     total = 0.0
-    on_gpu = W.is_cuda and bits == 2
+    on_gpu = W.is_cuda
     if on_gpu:
         # the search kernel: one workgroup per row, 2048 bytes of back pointers per row and step
         import rptc_kernels as rk
@@ -138,7 +138,7 @@ def quantize_matrix(W, codebook, S=8, importance=None, rows_per_batch=64, bits=2
     for r0 in range(0, m, rows_per_batch):
         tg = targets[r0:r0 + rows_per_batch]
         if on_gpu:
-            sym, cost, _, _ = rk.viterbi_pairs(tg.contiguous(), cb16, shared)
+            sym, cost, _, _ = rk.viterbi_pairs(tg.contiguous(), cb16, shared, bits=bits)
         else:
             w = None if wts is None else wts.expand(tg.size(0), -1, -1)
             sym, cost = viterbi_pairs(tg, table, w, step_bits=2 * bits)

@@ -89,6 +89,7 @@ def test_c_abi_rejects_bad_arguments_before_touching_a_device():
     assert lib.rptc_viterbi_pairs(16, None, 0, 16, None, 16, 16, 16, 4, 64, 8, None, None) == -1  # no scratch
     assert lib.rptc_viterbi_pairs(16, 16, 100, 16, 16, 16, 16, 16, 4, 64, 8, None, None) == -2    # weight stride < 2 * steps
     assert lib.rptc_viterbi_scratch_bytes(4, 64) == 4 * 64 * 2048
+    assert lib.rptc_viterbi_pairs_bits(16, None, 0, 16, 16, 16, 16, 16, 4, 64, 8, 5, None, None) == -2   # bits
     assert lib.rptc_viterbi_scalar(16, None, 0, 16, 15, 16, 16, 16, 16, 4, 64, None, None) == -2     # L
     assert lib.rptc_viterbi_scalar(16, None, 0, None, 16, 16, 16, 16, 16, 4, 64, None, None) == -1   # no alphabet
     assert lib.rptc_viterbi_scalar_scratch_bytes(4, 64) == 4 * 64 * 4096

@@ -156,3 +156,49 @@ def test_quantize_matrix_scalar_on_the_gpu_matches_the_host_search(rk):
         sym_cpu, mse_cpu = quantize.quantize_matrix_scalar(torch.from_numpy(W), torch.from_numpy(alphabet),
                                                            importance=importance)
         assert torch.equal(sym_gpu, sym_cpu) and abs(mse_gpu - mse_cpu) < 1e-6
+
+
+def test_viterbi_kernels_on_a_full_length_row(rk, oracle):
+    """One row of a 4096-column layer (2048 steps of the pair trellis, 4096 of the scalar one): path, cost and
+    end state equal the oracle's after thousands of steps of accumulated fp32 sums."""
+    from rptc_kernels import quantize
+    g = np.random.default_rng(77)
+    cb = g.standard_normal(512).astype(np.float16)
+    targets = (0.7 * g.standard_normal((1, 2048, 2))).astype(np.float32)
+    sym, cost, end, _ = rk.viterbi_pairs(torch.from_numpy(targets).cuda(), torch.from_numpy(cb).cuda())
+    osym, ocost, oend = oracle.viterbi(quantize.decode_table(torch.from_numpy(cb), 8).numpy(), 4, targets[0])
+    assert np.array_equal(sym[0].cpu().numpy().astype(np.int32), osym) and float(cost[0]) == float(ocost) and int(end[0]) == oend
+    alphabet = g.standard_normal(1 << 16).astype(np.float16)
+    row = g.standard_normal((1, 4096)).astype(np.float32)
+    sym, cost, end, _ = rk.viterbi_scalar(torch.from_numpy(row).cuda(), torch.from_numpy(alphabet).cuda())
+    osym, ocost, oend = oracle.viterbi(alphabet.astype(np.float32), 2, row[0])
+    assert np.array_equal(sym[0].cpu().numpy().astype(np.int32), osym) and float(cost[0]) == float(ocost) and int(end[0]) == oend
+
+
+@pytest.mark.parametrize("bits", [3, 4])
+@pytest.mark.parametrize("S,rows,steps,weighted", [(8, 2, 1, None), (8, 2, 40, None), (6, 2, 33, "shared"), (8, 2, 25, "rows")])
+def test_viterbi_kernel_at_3_and_4_bits_equals_the_oracle(rk, oracle, bits, S, rows, steps, weighted):
+    """6 and 8 stream bits per step: 64 and 256 predecessors per state (a group's minimum spans four lanes at 8)."""
+    from rptc_kernels import quantize
+    cb, targets, weights = _case(100 * bits + steps + S, rows, steps, S, weighted)
+    table = quantize.decode_table(torch.from_numpy(cb), S).numpy()
+    sym, cost, end, _ = rk.viterbi_pairs(torch.from_numpy(targets).cuda(), torch.from_numpy(cb).cuda(),
+                                         None if weights is None else torch.from_numpy(weights).cuda(), bits=bits)
+    sym, cost, end = sym.cpu().numpy(), cost.cpu().numpy(), end.cpu().numpy()
+    for r in range(rows):
+        w = None if weights is None else (weights if weights.ndim == 2 else weights[r])
+        osym, ocost, oend = oracle.viterbi(table, 2 * bits, targets[r], w)
+        assert np.array_equal(sym[r].astype(np.int32), osym), f"row {r}"
+        assert cost[r] == ocost and end[r] == oend
+
+
+@pytest.mark.parametrize("bits", [3, 4])
+def test_quantize_matrix_at_3_and_4_bits_on_the_gpu_matches_the_host_search(rk, bits):
+    from rptc_kernels import quantize
+    g = np.random.default_rng(40 + bits)
+    m, n, S = 4, 256, 8
+    W = g.standard_normal((m, n)).astype(np.float32)
+    cb = g.standard_normal(2 << S).astype(np.float16)
+    sym_gpu, mse_gpu = quantize.quantize_matrix(torch.from_numpy(W).cuda(), torch.from_numpy(cb).cuda(), S, bits=bits)
+    sym_cpu, mse_cpu = quantize.quantize_matrix(torch.from_numpy(W), torch.from_numpy(cb), S, bits=bits)
+    assert torch.equal(sym_gpu, sym_cpu) and abs(mse_gpu - mse_cpu) < 1e-6
