@@ -162,3 +162,97 @@ def dequantize_symbols(symbols, codebook, S=8, bits=2):
         W[:, cols[p]] = table[state, 0]
         W[:, cols[p] + 1] = table[state, 1]
     return W
+
+
+def factorize(W, iterations=64):
+    """The reference's row/column factorisation W = b_out + b_in + s_out * s_in * N (quantize_hf.py:77-117):
+    64 rounds of alternately re-estimating the biases (means of the scaled residual) and the scales (RMS of
+    the residual), each followed by the balancing step that keeps the two biases' means and the two scales'
+    geometric means equal.  W float [out, in] on any device.  Returns (b_out [out, 1], b_in [1, in],
+    s_out [out, 1], s_in [1, in], N [out, in]); N has row and column RMS close to 1."""
+    W = torch.as_tensor(W).to(torch.float32)
+    out_features, in_features = W.shape
+    b_out = torch.zeros((out_features, 1), dtype=torch.float32, device=W.device)
+    b_in = torch.zeros((1, in_features), dtype=torch.float32, device=W.device)
+    s_out = torch.ones_like(b_out)
+    s_in = torch.ones_like(b_in)
+    for _ in range(iterations):
+        nb_out = ((W - b_in) / s_in).mean(dim=1, keepdim=True) / (1 / s_in).mean()
+        nb_in = ((W - nb_out) / s_out).mean(dim=0, keepdim=True) / (1 / s_out).mean()
+        balancer = (nb_in.mean() - nb_out.mean()) / 2
+        nb_out = nb_out + balancer
+        nb_in = nb_in - balancer
+        ns_out = (((W - nb_out - nb_in) / s_in) ** 2).mean(dim=1, keepdim=True).sqrt()
+        ns_in = (((W - nb_out - nb_in) / ns_out) ** 2).mean(dim=0, keepdim=True).sqrt()
+        balancer = torch.exp((ns_in.log().mean() - ns_out.log().mean()) / 2)
+        ns_out = ns_out * balancer
+        ns_in = ns_in / balancer
+        b_out, b_in, s_out, s_in = nb_out, nb_in, ns_out, ns_in
+    N = (W - b_out - b_in) / s_out / s_in
+    return b_out, b_in, s_out, s_in, N
+
+
+def quantile_alphabet(values, L=16, seed=0):
+    """The reference's per-bank alphabet (quantize_hf.py:137-141): 2^L values read off the sorted sample at the
+    mid-point quantiles (linear interpolation), then shuffled.  The shuffle is seeded with torch, not with
+    jax.random.permutation."""
+    fp = torch.sort(values.reshape(-1).to(torch.float32)).values
+    M, K = 1 << L, fp.numel()
+    x = (2 * torch.arange(M, dtype=torch.float64, device=fp.device) + 1) / 2 / M
+    pos = (x * K - 0.5).clamp(0, K - 1)                 # xp[k] = (2k + 1) / 2K  ->  k = x K - 1/2
+    lo = pos.floor().long()
+    hi = (lo + 1).clamp(max=K - 1)
+    frac = (pos - lo.to(torch.float64)).to(torch.float32)
+    alphabet = fp[lo] * (1 - frac) + fp[hi] * frac
+    g = torch.Generator().manual_seed(seed)
+    return alphabet[torch.randperm(M, generator=g).to(fp.device)]
+
+
+def quantize_layer(W, hessian_diag=None, L=16, banks=32, seed=0):
+    """quantize_hf.py:120-170 for one layer: factorise, weigh column i by (H_ii * s_in_i)^2 (the reference
+    passes diag(H) * s_in as ``corrections`` and the search squares it, rptc.py:32), cut the rows into
+    ``banks`` groups with one shuffled quantile alphabet each, search every row on the scalar trellis
+    (``viterbi_scalar``: the HIP kernel for a matrix on the GPU), and put the layer back together.
+    Returns a dict with the reconstruction ``recon`` [out, in], the 2-bit ``symbols`` [out, in], the
+    ``alphabets`` [banks, 2^L] (fp16 values as float32) and the factors; out % banks == 0."""
+    W = torch.as_tensor(W).to(torch.float32)
+    out_features, in_features = W.shape
+    if out_features % banks != 0:
+        raise ValueError("the row count must be a multiple of the number of banks")
+    b_out, b_in, s_out, s_in, N = factorize(W)
+    imp = None
+    if hessian_diag is not None:
+        h = torch.as_tensor(hessian_diag, dtype=torch.float32, device=W.device).reshape(-1)
+        imp = (h * s_in.reshape(-1)) ** 2
+    rows_per_bank = out_features // banks
+    symbols = torch.empty((out_features, in_features), dtype=torch.int64)
+    rounded = torch.empty_like(N)
+    alphabets = []
+    for b in range(banks):
+        rows = slice(b * rows_per_bank, (b + 1) * rows_per_bank)
+        alphabet = quantile_alphabet(N[rows], L, seed + b).to(torch.float16)      # the kernels' table is fp16
+        sym, _ = quantize_matrix_scalar(N[rows], alphabet, importance=imp)
+        symbols[rows] = sym
+        state = torch.zeros(rows_per_bank, dtype=torch.int64)
+        af = alphabet.to(torch.float32).cpu()
+        vals = torch.empty((rows_per_bank, in_features), dtype=torch.float32)
+        for t in range(in_features):                                              # rptc.py:74-85
+            state = ((state << 2) | sym[:, t]) & ((1 << L) - 1)
+            vals[:, t] = af[state]
+        rounded[rows] = vals.to(W.device)
+        alphabets.append(af)
+    recon = b_out + b_in + s_out * s_in * rounded
+    return {"recon": recon, "symbols": symbols, "alphabets": torch.stack(alphabets), "biases_out": b_out, "biases_in": b_in,
+            "scales_out": s_out, "scales_in": s_in, "normalized": N}
+
+
+def evaluate_layer(W, recon, hessian_diag=None):
+    """Relative errors of a reconstruction (quantize_hf.py:173-187): Frobenius, and weighted by the Hessian
+    diagonal when one is given."""
+    W = torch.as_tensor(W).to(torch.float32)
+    E = W - recon.to(W.device)
+    res = {"frob": float((E ** 2).sum() / (W ** 2).sum())}
+    if hessian_diag is not None:
+        h = torch.as_tensor(hessian_diag, dtype=torch.float32, device=W.device).reshape(1, -1)
+        res["proxy_diag"] = float(((E * h) * E).sum() / ((W * h) * W).sum())
+    return res

@@ -202,3 +202,37 @@ def test_quantize_matrix_at_3_and_4_bits_on_the_gpu_matches_the_host_search(rk, 
     sym_gpu, mse_gpu = quantize.quantize_matrix(torch.from_numpy(W).cuda(), torch.from_numpy(cb).cuda(), S, bits=bits)
     sym_cpu, mse_cpu = quantize.quantize_matrix(torch.from_numpy(W), torch.from_numpy(cb), S, bits=bits)
     assert torch.equal(sym_gpu, sym_cpu) and abs(mse_gpu - mse_cpu) < 1e-6
+
+
+def test_quantize_layer_feeds_the_scalar_lut_kernels(rk):
+    """The reference's layer quantizer (quantize_hf.py:120-170) with the search kernel, then its symbols through
+    the packers into the reference's two scalar-LUT kernels: decompress reproduces the rounded normalised
+    weights bit for bit, decompress_matvec_t_16 their product with a vector."""
+    from rptc_kernels import packing, quantize
+    from util import rel_l2
+    g = torch.Generator().manual_seed(9)
+    out_f, in_f, banks = 64, 2048, 2
+    W = torch.randn((out_f, in_f), generator=g) * (0.5 + torch.rand((out_f, 1), generator=g)) * 0.02
+    h = 0.5 + torch.rand(in_f, generator=g)
+    res = quantize.quantize_layer(W.cuda(), h.cuda(), L=16, banks=banks, seed=3)
+    err = quantize.evaluate_layer(W.cuda(), res["recon"], h.cuda())
+    assert err["frob"] < 0.09 and err["proxy_diag"] < 0.09      # 2 bits/weight; rate-distortion bound 0.0625
+    rows = out_f // banks
+    x = torch.randn(in_f, generator=g).half().cuda()
+    prev = rk.set_carry_mode(rk.CONTINUOUS)
+    try:
+        for b in range(banks):
+            sym = res["symbols"][b * rows:(b + 1) * rows].numpy()
+            alphabet = res["alphabets"][b].half().cuda()
+            stream = torch.from_numpy(packing.pack_rowmajor(sym)).cuda()
+            dec = torch.empty((rows, in_f), dtype=torch.float16, device="cuda")
+            rk.decompress(stream, alphabet, dec)
+            rounded = (res["recon"][b * rows:(b + 1) * rows] - res["biases_out"][b * rows:(b + 1) * rows] - res["biases_in"]) \
+                / res["scales_out"][b * rows:(b + 1) * rows] / res["scales_in"]
+            assert torch.allclose(dec.float(), rounded, atol=2e-3, rtol=1e-3)      # recon was put together in fp32
+            y = torch.zeros(rows, dtype=torch.float16, device="cuda")
+            rk.decompress_matvec_t_16(torch.from_numpy(packing.pack_transposed(sym)).cuda(), alphabet, x, y)
+            want = dec.double() @ x.double()
+            assert rel_l2(y.float().cpu().numpy(), want.cpu().numpy()) < 2e-3
+    finally:
+        rk.set_carry_mode(prev)

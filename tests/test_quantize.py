@@ -153,3 +153,44 @@ def test_scalar_quantizer_equals_the_oracle_and_decodes_through_the_packed_strea
             assert np.array_equal(sym[r].numpy(), osym)
     got = oracle.dequantize_h(alphabet, sym[0].numpy().astype(np.int32))
     assert got.shape == (n,)
+
+
+def test_factorize_is_exact_and_balanced():
+    """quantize_hf.py:77-117: the factors reproduce W exactly (that is how N is defined), N has unit row and
+    column RMS and zero row and column means at the fixed point, and the balancing steps hold."""
+    g = torch.Generator().manual_seed(3)
+    out_f, in_f = 48, 80
+    W = (torch.randn((out_f, in_f), generator=g) * (0.5 + torch.rand((out_f, 1), generator=g))
+         * (0.5 + torch.rand((1, in_f), generator=g)) + 0.3 * torch.randn((out_f, 1), generator=g)
+         + 0.2 * torch.randn((1, in_f), generator=g))
+    b_out, b_in, s_out, s_in, N = quantize.factorize(W)
+    assert torch.allclose(b_out + b_in + s_out * s_in * N, W, atol=1e-5)
+    assert torch.allclose((N ** 2).mean(dim=0).sqrt(), torch.ones(in_f), atol=1e-3)
+    assert torch.allclose((N ** 2).mean(dim=1).sqrt(), torch.ones(out_f), atol=2e-2)
+    assert abs(float(b_out.mean() - b_in.mean())) < 1e-5
+    assert abs(float(s_out.log().mean() - s_in.log().mean())) < 1e-4
+    # and rows and columns of N are centred (the biases are the means of the scaled residual)
+    assert float(N.mean(dim=1).abs().max()) < 2e-2 and float(N.mean(dim=0).abs().max()) < 2e-2
+
+
+def test_quantile_alphabet_matches_numpy_interp():
+    g = np.random.default_rng(4)
+    vals = g.standard_normal(1000).astype(np.float32)
+    L = 8
+    got = np.sort(quantize.quantile_alphabet(torch.from_numpy(vals), L, seed=1).numpy())
+    M = 1 << L
+    want = np.interp((2 * np.arange(M) + 1) / 2 / M, (2 * np.arange(vals.size) + 1) / 2 / vals.size, np.sort(vals))
+    assert np.allclose(got, want, atol=1e-6)
+
+
+def test_quantize_layer_reconstructs_better_than_a_scalar_quantizer():
+    """quantize_hf.py:160-170 end to end on a small layer (CPU search): the reconstruction's relative error at
+    2 bits per weight is far below that of rounding to four levels."""
+    g = torch.Generator().manual_seed(5)
+    out_f, in_f = 16, 128
+    W = torch.randn((out_f, in_f), generator=g) * (0.5 + torch.rand((out_f, 1), generator=g))
+    h = 0.5 + torch.rand(in_f, generator=g)
+    res = quantize.quantize_layer(W, h, L=10, banks=2, seed=1)
+    err = quantize.evaluate_layer(W, res["recon"], h)
+    assert res["symbols"].shape == (out_f, in_f) and int(res["symbols"].max()) <= 3
+    assert err["frob"] < 0.12 and err["proxy_diag"] < 0.12       # 2-bit Lloyd-Max scalar quantizer: 0.1175
