@@ -69,12 +69,15 @@ class QuantizedLinear(torch.nn.Module):
         return layer
 
     @classmethod
-    def from_weight(cls, weight, codebook=None, S=8, importance=None, seed=42, device="cuda", bits=2):
+    def from_weight(cls, weight, codebook=None, S=8, importance=None, seed=42, device="cuda", bits=2, signs=None):
         """Quantize a dense weight [out, in] with the Viterbi search of ``rptc_kernels.quantize`` (run on
         ``device``) and pack the result.  codebook: fp16 [2^(S+1)] or None for a seeded Gaussian one
-        scaled to the weight's standard deviation."""
+        scaled to the weight's standard deviation.  signs: +-1 per input feature; the layer then stores
+        the weight in the sign-Hadamard basis (outliers spread over a block) and transforms its input."""
         from rptc_kernels import quantize
         W = torch.as_tensor(weight).to(device=device, dtype=torch.float32)
+        if signs is not None:
+            W = quantize.sign_hadamard_rows(W, signs)
         if codebook is None:
             g = torch.Generator().manual_seed(seed)
             codebook = (torch.randn(2 << S, generator=g) * W.std().item()).to(torch.float16)
@@ -82,6 +85,8 @@ class QuantizedLinear(torch.nn.Module):
         symbols, mse = quantize.quantize_matrix(W, codebook.to(device), S, importance=importance, bits=bits)
         layer = cls.from_symbols(symbols, codebook, W.size(0), S=S, device=device, bits=bits)
         layer.quantization_mse = mse
+        if signs is not None:
+            layer.set_signs(signs)
         return layer
 
     def set_affine(self, scales_out=None, scales_in=None, biases_out=None, biases_in=None):

@@ -256,3 +256,27 @@ def evaluate_layer(W, recon, hessian_diag=None):
         h = torch.as_tensor(hessian_diag, dtype=torch.float32, device=W.device).reshape(1, -1)
         res["proxy_diag"] = float(((E * h) * E).sum() / ((W * h) * W).sum())
     return res
+
+
+def sign_hadamard_rows(W, signs, block=0):
+    """Every row of W [m, n] through the forward sign-Hadamard transform of ``rptc_kernels.sign_hadamard``
+    (y = H_P (signs * x) / sqrt(P) per block of P columns; block 0: the largest power of two dividing n), in
+    float32.  With T that (orthogonal) map, W x = (W T^t)(T x) and row r of W T^t is T applied to row r of W:
+    the weights a layer stores when its input goes through the transform first."""
+    W = torch.as_tensor(W).to(torch.float32)
+    m, n = W.shape
+    P = block
+    if P == 0:
+        P = 1
+        while n % (2 * P) == 0 and 2 * P <= 32768:
+            P *= 2
+    if P < 2 or P & (P - 1) or n % P:
+        raise ValueError("block must be a power of two dividing n")
+    y = (W * torch.as_tensor(signs).to(W.device, torch.float32).reshape(1, n)).reshape(m, n // P, P)
+    h = 1
+    while h < P:                                         # Sylvester order: butterflies over strides 1, 2, 4, ...
+        y = y.reshape(m, n // P, P // (2 * h), 2, h)
+        a, b = y[:, :, :, 0, :], y[:, :, :, 1, :]
+        y = torch.stack([a + b, a - b], dim=3)
+        h *= 2
+    return (y.reshape(m, n) / P ** 0.5)

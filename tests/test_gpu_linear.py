@@ -50,6 +50,25 @@ def test_quantized_linear_with_sign_hadamard(rk):
     assert rel_l2(y.reshape(6, m).cpu().numpy(), want.cpu().numpy()) < 1e-3
 
 
+def test_from_weight_in_the_sign_hadamard_basis_spreads_outliers(rk):
+    """A weight with a few large columns: quantized as it is, the outliers cost most of the error; in the
+    sign-Hadamard basis they are spread over their block, and the layer (which transforms its input) is closer
+    to the dense product."""
+    from rptc_kernels.linear import QuantizedLinear
+    g = torch.Generator().manual_seed(12)
+    m, n = 64, 1024
+    W = torch.randn((m, n), generator=g) * 0.02
+    W[:, ::97] *= 12.0
+    signs = torch.where(torch.rand(n, generator=g) < 0.5, -1.0, 1.0)
+    x = torch.randn((4, n), generator=g).half().cuda()
+    want = x.double() @ W.double().cuda().t()
+    errs = []
+    for sg in (None, signs):
+        layer = QuantizedLinear.from_weight(W, S=8, seed=5, signs=sg)
+        errs.append(rel_l2(layer(x).float().cpu().numpy(), want.cpu().numpy()))
+    assert errs[1] < 0.6 * errs[0] and errs[1] < 0.4
+
+
 def test_from_symbols_decodes_the_trellis_path(rk):
     from rptc_kernels.linear import QuantizedLinear
     from rptc_kernels import packing

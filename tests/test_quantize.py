@@ -194,3 +194,14 @@ def test_quantize_layer_reconstructs_better_than_a_scalar_quantizer():
     err = quantize.evaluate_layer(W, res["recon"], h)
     assert res["symbols"].shape == (out_f, in_f) and int(res["symbols"].max()) <= 3
     assert err["frob"] < 0.12 and err["proxy_diag"] < 0.12       # 2-bit Lloyd-Max scalar quantizer: 0.1175
+
+
+def test_sign_hadamard_rows_is_the_oracle_transform_and_orthogonal(oracle):
+    g = np.random.default_rng(6)
+    m, n = 3, 768                        # blocks of 256
+    W = g.standard_normal((m, n)).astype(np.float16)
+    signs = np.where(g.random(n) < 0.5, -1.0, 1.0).astype(np.float16)
+    got = quantize.sign_hadamard_rows(torch.from_numpy(W.astype(np.float32)), torch.from_numpy(signs)).numpy()
+    want = oracle.sign_hadamard(W, signs, 256)
+    assert np.allclose(got, want, atol=1e-5)
+    assert np.allclose((got ** 2).sum(axis=1), (W.astype(np.float64) ** 2).sum(axis=1), rtol=1e-5)
