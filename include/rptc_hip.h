@@ -217,6 +217,31 @@ int rptc_decompress_matvec_rmsnorm(const int32_t *compressed, const uint16_t *co
                                    float *ms);
 
 /*
+ * The same mat-vecs with the row/column factorisation the reference's quantizer puts around a
+ * quantized matrix, W = b_out + b_in + s_out * s_in * W_hat (quantize_hf.py:77-117 finds the four
+ * vectors, quantize_hf.py:167 is this formula; the reference applies it to a dense copy of W_hat):
+ *     out[r] = s_out[r] * (W_hat (s_in .* a))[r] + b_out[r] * sum(a) + (b_in . a)
+ * with a the activations (x; silu(gate) * up; the normed residual), s_in .* a rounded to fp16 and
+ * everything behind it in fp32 with one rounding at the end.  scales_in, biases_in: fp16 [n];
+ * scales_out, biases_out: fp16 [m]; each may be NULL (scale 1, bias 0).  n <= 16384 (RPTC_ELIMIT
+ * above: apply the vectors around the plain call instead).
+ */
+int rptc_decompress_matvec_affine(const int32_t *compressed, const uint16_t *codebook, const uint16_t *x,
+                                  const uint16_t *scales_in, const uint16_t *biases_in,
+                                  const uint16_t *scales_out, const uint16_t *biases_out, uint16_t *out,
+                                  int64_t m, int64_t n, int S, int carry_mode, void *stream, float *ms);
+int rptc_decompress_matvec_silu_affine(const int32_t *compressed, const uint16_t *codebook, const uint16_t *gate_up,
+                                       const uint16_t *scales_in, const uint16_t *biases_in,
+                                       const uint16_t *scales_out, const uint16_t *biases_out, uint16_t *out,
+                                       int64_t m, int64_t n, int S, int carry_mode, void *stream, float *ms);
+int rptc_decompress_matvec_rmsnorm_affine(const int32_t *compressed, const uint16_t *codebook, const uint16_t *x_in,
+                                          const uint16_t *delta, const uint16_t *weight, uint16_t *x_out,
+                                          const uint16_t *scales_in, const uint16_t *biases_in,
+                                          const uint16_t *scales_out, const uint16_t *biases_out, uint16_t *out,
+                                          int64_t m, int64_t n, float eps, int S, int carry_mode, void *stream,
+                                          float *ms);
+
+/*
  * Viterbi search for the hashed pair stream: the symbols whose decode by rptc_decompress_matvec_16_{S}_1
  * (carry mode continuous) is closest to the targets.  Replaces the search of the reference's quantizer
  * (rptc.py:13-71, diag_only path: rho[0] = 0 at the start, first index on ties, best end state traced

@@ -168,7 +168,14 @@ struct XFuse {
     uint4 *x_out;          // AddRmsNorm: the updated residual stream (must not alias x or x2)
     float eps;
     int log_p;             // SignHadamard: log2 of the block length
+    // AFFINE (the reference's reconstruction W = b_out + b_in + s_out * s_in * W_hat, quantize_hf.py:167):
+    // out[r] = s_out[r] * (W_hat (s_in .* a))[r] + b_out[r] * sum(a) + (b_in . a), a = the activations above;
+    // any of the four may be null (scale 1, bias 0)
+    const uint4 *s_in, *b_in;
+    const uint16_t *s_out, *b_out;
 };
+
+constexpr int kRedFloats = 48;   // workgroup reductions of the prologues: 16 waves x up to 3 values
 
 struct Halves8 {
     float v[8];
@@ -209,7 +216,7 @@ __device__ __forceinline__ uint4 silu_mul8(const uint4 gate, const uint4 up)
 }
 
 // COMPACT: partial sums per (row, full slab) and (row, ragged lane) instead of per (row, stream element)
-template <int S, int MODE, int BITS, int XMODE, bool COMPACT>
+template <int S, int MODE, int BITS, int XMODE, bool COMPACT, bool AFFINE = false>
 __device__ __forceinline__ void matvec_body(
     const uint32_t *__restrict__ comp, const uint32_t *__restrict__ codebook,
     const uint4 *__restrict__ x, uint16_t *__restrict__ out, const MatvecArgs a, const XFuse fuse)
@@ -226,6 +233,7 @@ __device__ __forceinline__ void matvec_body(
     // are added with DPP first: [row][T full slabs + Lt ragged lanes].
     float *part = reinterpret_cast<float *>(sx + (n >> 1));
     const int pstride = COMPACT ? T + Lt : npr;
+    float *red = part + a.rows_per_block * pstride;        // kRedFloats, present when a prologue reduces
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: keeps control flow scalar
@@ -273,6 +281,20 @@ __device__ __forceinline__ void matvec_body(
             xv2[u] = (idx < n8 && fuse.x2) ? fuse.x2[idx] : make_uint4(0, 0, 0, 0);
             xvw[u] = idx < n8 ? fuse.norm_w[idx] : make_uint4(0, 0, 0, 0);
         }
+    }
+
+    uint4 xsi[kXRegs], xbi[kXRegs];
+    uint16_t so_bits = 0x3C00u, bo_bits = 0;                // 1.0, 0.0: lane j holds the values of row wave + 16 j
+    if constexpr (AFFINE) {
+#pragma unroll
+        for (int u = 0; u < kXRegs; u++) {
+            const int idx = tid + u * kMatvecThreads;
+            xsi[u] = (idx < n8 && fuse.s_in) ? fuse.s_in[idx] : make_uint4(0, 0, 0, 0);
+            xbi[u] = (idx < n8 && fuse.b_in) ? fuse.b_in[idx] : make_uint4(0, 0, 0, 0);
+        }
+        const int my_row = wave + kMatvecWaves * lane;
+        if (fuse.s_out && my_row < rows) so_bits = fuse.s_out[row0 + my_row];
+        if (fuse.b_out && my_row < rows) bo_bits = fuse.b_out[row0 + my_row];
     }
 
     // This wave's items: a contiguous piece of [slab 0 items][slab 1 items]...[ragged slab items].
@@ -400,13 +422,13 @@ __device__ __forceinline__ void matvec_body(
             const int idx = tid + u * kMatvecThreads;
             if (blockIdx.x == 0 && idx < n8) fuse.x_out[idx] = pack8(r[u]);
         }
-        // sum over the workgroup in a fixed order; `part` is not in use before the barrier below
+        // sum over the workgroup in a fixed order
         ss = wave_sum(ss);
-        if (lane == 63) part[wave] = ss;
+        if (lane == 63) red[wave] = ss;
         __syncthreads();
         float total_ss = 0.f;
 #pragma unroll
-        for (int w = 0; w < kMatvecWaves; w++) total_ss += part[w];
+        for (int w = 0; w < kMatvecWaves; w++) total_ss += red[w];
         const float inv = rsqrtf(total_ss / (float)n + fuse.eps);
 #pragma unroll
         for (int u = 0; u < kXRegs; u++) {
@@ -445,6 +467,29 @@ __device__ __forceinline__ void matvec_body(
         }
     }
 
+    float act_sum = 0.f, act_bias = 0.f;                   // sum(a), b_in . a
+    if constexpr (AFFINE) {
+        // host side guarantees n8 <= kXRegs * kMatvecThreads: the whole vector is in registers
+#pragma unroll
+        for (int u = 0; u < kXRegs; u++) {
+            Halves8 v = unpack8(xv[u]);                     // zero past the end of the vector
+            const Halves8 bi = unpack8(xbi[u]), si = unpack8(xsi[u]);
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                act_sum += v.v[i];
+                act_bias += v.v[i] * bi.v[i];
+                if (fuse.s_in) v.v[i] *= si.v[i];
+            }
+            if (fuse.s_in) xv[u] = pack8(v);
+        }
+        act_sum = wave_sum(act_sum);
+        act_bias = wave_sum(act_bias);
+        if (lane == 63) {
+            red[kMatvecWaves + 2 * wave] = act_sum;
+            red[kMatvecWaves + 2 * wave + 1] = act_bias;
+        }
+    }
+
     // table (256 rows x 64 lane copies) and activation image into LDS
 #pragma unroll
     for (int i = 0; i < kRowsPerWave; i++) lds[(kRowsPerWave * wave + i) * 64 + lane] = cbv[i];
@@ -463,6 +508,17 @@ __device__ __forceinline__ void matvec_body(
         stage_x(idx, XMODE == kXSiluMul ? silu_mul8(x[idx], x[n8 + idx]) : x[idx]);
     __syncthreads();
     RPTC_STAMP(2);
+    if constexpr (AFFINE) {
+        act_sum = act_bias = 0.f;
+#pragma unroll
+        for (int w = 0; w < kMatvecWaves; w++) {
+            act_sum += red[kMatvecWaves + 2 * w];
+            act_bias += red[kMatvecWaves + 2 * w + 1];
+        }
+        // the same in every lane: kept in scalar registers until the row sums are written
+        act_sum = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, act_sum)));
+        act_bias = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, act_bias)));
+    }
 
     uint32_t xr[32];
     int slab = first_slab, idx = first_idx, cur_slab = -1;
@@ -554,10 +610,15 @@ __device__ __forceinline__ void matvec_body(
     RPTC_STAMP(4);
     __syncthreads();
     // one wave per row: add the row's partial sums in a fixed order
-    for (int r = wave; r < rows; r += kMatvecWaves) {
+    for (int r = wave, k = 0; r < rows; r += kMatvecWaves, k++) {
         float y = 0.f;
         for (int i = lane; i < pstride; i += kWave) y += part[r * pstride + i];
         y = wave_sum(y);
+        if constexpr (AFFINE) {
+            const float so = half_bits_to_float((uint16_t)__builtin_amdgcn_readlane((int)so_bits, k & 63));
+            const float bo = half_bits_to_float((uint16_t)__builtin_amdgcn_readlane((int)bo_bits, k & 63));
+            y = so * y + (bo * act_sum + act_bias);
+        }
         if (lane == 63) out[row0 + r] = float_to_half_bits(y);
     }
     RPTC_STAMP(5);
@@ -571,7 +632,7 @@ __global__ __launch_bounds__(kMatvecThreads) void matvec_kernel(
 {
     // separate scalar arguments (not a struct) so that all of them are preloaded into SGPRs
     const MatvecArgs a = {arg_m, arg_n, arg_rows_per_block, arg_rw_tail, arg_items_full, arg_items_tail, arg_full_magic};
-    matvec_body<S, MODE, BITS, kXPlain, COMPACT>(comp, codebook, x, out, a, XFuse{nullptr, nullptr, nullptr, 0.f, 0});
+    matvec_body<S, MODE, BITS, kXPlain, COMPACT>(comp, codebook, x, out, a, XFuse{nullptr, nullptr, nullptr, 0.f, 0, nullptr, nullptr, nullptr, nullptr});
 }
 
 // 2 bits per weight with an element-wise step fused in front (XMODE above)
@@ -583,7 +644,20 @@ __global__ __launch_bounds__(kMatvecThreads) void matvec_fused_kernel(
     float eps, int log_p)
 {
     const MatvecArgs a = {arg_m, arg_n, arg_rows_per_block, arg_rw_tail, arg_items_full, arg_items_tail, arg_full_magic};
-    matvec_body<S, MODE, 2, XMODE, COMPACT>(comp, codebook, x, out, a, XFuse{x2, norm_w, x_out, eps, log_p});
+    matvec_body<S, MODE, 2, XMODE, COMPACT>(comp, codebook, x, out, a, XFuse{x2, norm_w, x_out, eps, log_p, nullptr, nullptr, nullptr, nullptr});
+}
+
+// 2 bits per weight with the row/column scales and biases of the reference's factorisation applied in
+// the prologue (input side) and where the row sums are written (output side), after any XMODE step
+template <int S, int MODE, int XMODE>
+__global__ __launch_bounds__(kMatvecThreads) void matvec_affine_kernel(
+    const uint32_t *__restrict__ comp, const uint32_t *__restrict__ codebook,
+    const uint4 *__restrict__ x, uint16_t *__restrict__ out, int arg_m, int arg_n, int arg_rows_per_block,
+    int arg_rw_tail, int arg_items_full, int arg_items_tail, uint32_t arg_full_magic, const uint4 *x2, const uint4 *norm_w, uint4 *x_out,
+    float eps, const uint4 *s_in, const uint4 *b_in, const uint16_t *s_out, const uint16_t *b_out)
+{
+    const MatvecArgs a = {arg_m, arg_n, arg_rows_per_block, arg_rw_tail, arg_items_full, arg_items_tail, arg_full_magic};
+    matvec_body<S, MODE, 2, XMODE, false, true>(comp, codebook, x, out, a, XFuse{x2, norm_w, x_out, eps, 0, s_in, b_in, s_out, b_out});
 }
 
 // Dense export: one thread per stream element, 32 pairs scattered to their columns.
@@ -710,7 +784,7 @@ static int launch_matvec_fused(const int32_t *compressed, const uint16_t *codebo
     bool compact;
     // The norm and Hadamard variants hold the whole vector in registers (n <= 16384): never long enough
     // to need compact sums.  The Hadamard variant keeps the vector as padded fp32 behind the partial sums.
-    const int extra = XMODE == kXSignHadamard ? (int)(n + n / 32 + 1) * 4 : 0;
+    const int extra = XMODE == kXSignHadamard ? (int)(n + n / 32 + 1) * 4 : XMODE == kXAddRmsNorm ? kRedFloats * 4 : 0;
     int rc = plan_matvec(compressed, codebook, x, out, m, n, carry_mode, XMODE == kXSiluMul, extra, &dev, &a, &compact,
                          &lds_bytes, &grid);
     if (rc) return rc;
@@ -737,6 +811,44 @@ static int launch_matvec_fused(const int32_t *compressed, const uint16_t *codebo
     }
     if (carry_mode == RPTC_AS_WRITTEN) RPTC_LAUNCH(RPTC_AS_WRITTEN, false);
     else RPTC_LAUNCH(RPTC_CONTINUOUS, false);
+#undef RPTC_LAUNCH
+    return t.end();
+}
+
+template <int S, int XMODE>
+static int launch_matvec_affine(const int32_t *compressed, const uint16_t *codebook, const uint16_t *x,
+                                const uint16_t *x2, const uint16_t *norm_w, uint16_t *x_out, float eps,
+                                const uint16_t *s_in, const uint16_t *b_in, const uint16_t *s_out, const uint16_t *b_out,
+                                uint16_t *out, int64_t m, int64_t n, int carry_mode, void *stream, float *ms)
+{
+    // the whole activation vector sits in two registers per thread
+    if (n > 8 * 2 * kMatvecThreads) return RPTC_ELIMIT;
+    if (!aligned16(s_in) || !aligned16(b_in)) return RPTC_EALIGN;
+    DeviceInfo *dev;
+    MatvecArgs a;
+    int lds_bytes, grid;
+    bool compact;
+    int rc = plan_matvec(compressed, codebook, x, out, m, n, carry_mode, false, kRedFloats * 4, &dev, &a, &compact,
+                         &lds_bytes, &grid);
+    if (rc) return rc;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    Timer t;
+    rc = t.begin(dev, s, ms);
+    if (rc) return rc;
+    auto a_comp = reinterpret_cast<const uint32_t *>(compressed);
+    auto a_cb = reinterpret_cast<const uint32_t *>(codebook);
+    auto a_x = reinterpret_cast<const uint4 *>(x);
+    auto a_x2 = reinterpret_cast<const uint4 *>(x2);
+    auto a_w = reinterpret_cast<const uint4 *>(norm_w);
+    auto a_xo = reinterpret_cast<uint4 *>(x_out);
+    auto a_si = reinterpret_cast<const uint4 *>(s_in);
+    auto a_bi = reinterpret_cast<const uint4 *>(b_in);
+#define RPTC_LAUNCH(MODE)                                                                                      \
+    hipLaunchKernelGGL((matvec_affine_kernel<S, MODE, XMODE>), dim3(grid), dim3(kMatvecThreads), lds_bytes, s, \
+                       a_comp, a_cb, a_x, out, a.m, a.n, a.rows_per_block, a.rw_tail, a.items_full, a.items_tail, \
+                       a.full_magic, a_x2, a_w, a_xo, eps, a_si, a_bi, s_out, b_out)
+    if (carry_mode == RPTC_AS_WRITTEN) RPTC_LAUNCH(RPTC_AS_WRITTEN);
+    else RPTC_LAUNCH(RPTC_CONTINUOUS);
 #undef RPTC_LAUNCH
     return t.end();
 }
@@ -835,6 +947,15 @@ int prepare_matvec()
     RPTC_SET_LIMITS(kXAddRmsNorm, false)
     RPTC_SET_LIMITS(kXSignHadamard, false)
 #undef RPTC_SET_LIMITS
+#define RPTC_SET_LIMITS(XMODE)                                                                     \
+    if ((rc = set_lds_limit(matvec_affine_kernel<6, RPTC_AS_WRITTEN, XMODE>))) return rc;             \
+    if ((rc = set_lds_limit(matvec_affine_kernel<6, RPTC_CONTINUOUS, XMODE>))) return rc;             \
+    if ((rc = set_lds_limit(matvec_affine_kernel<8, RPTC_AS_WRITTEN, XMODE>))) return rc;             \
+    if ((rc = set_lds_limit(matvec_affine_kernel<8, RPTC_CONTINUOUS, XMODE>))) return rc;
+    RPTC_SET_LIMITS(kXPlain)
+    RPTC_SET_LIMITS(kXSiluMul)
+    RPTC_SET_LIMITS(kXAddRmsNorm)
+#undef RPTC_SET_LIMITS
     return 0;
 }
 
@@ -887,6 +1008,41 @@ extern "C" int rptc_decompress_matvec_rmsnorm(const int32_t *c, const uint16_t *
     if (n > 8 * 2 * kMatvecThreads) return RPTC_ELIMIT;      // the whole vector sits in two registers per thread
     return S == 6 ? launch_matvec_fused<6, kXAddRmsNorm>(c, cb, x_in, delta, weight, x_out, eps, 0, out, m, n, mode, stream, ms)
                   : launch_matvec_fused<8, kXAddRmsNorm>(c, cb, x_in, delta, weight, x_out, eps, 0, out, m, n, mode, stream, ms);
+}
+
+extern "C" int rptc_decompress_matvec_affine(const int32_t *c, const uint16_t *cb, const uint16_t *x,
+                                             const uint16_t *scales_in, const uint16_t *biases_in,
+                                             const uint16_t *scales_out, const uint16_t *biases_out, uint16_t *out,
+                                             int64_t m, int64_t n, int S, int mode, void *stream, float *ms)
+{
+    if (S != 6 && S != 8) return RPTC_ESHAPE;
+    return S == 6 ? launch_matvec_affine<6, kXPlain>(c, cb, x, nullptr, nullptr, nullptr, 0.f, scales_in, biases_in, scales_out, biases_out, out, m, n, mode, stream, ms)
+                  : launch_matvec_affine<8, kXPlain>(c, cb, x, nullptr, nullptr, nullptr, 0.f, scales_in, biases_in, scales_out, biases_out, out, m, n, mode, stream, ms);
+}
+
+extern "C" int rptc_decompress_matvec_silu_affine(const int32_t *c, const uint16_t *cb, const uint16_t *gate_up,
+                                                  const uint16_t *scales_in, const uint16_t *biases_in,
+                                                  const uint16_t *scales_out, const uint16_t *biases_out, uint16_t *out,
+                                                  int64_t m, int64_t n, int S, int mode, void *stream, float *ms)
+{
+    if (S != 6 && S != 8) return RPTC_ESHAPE;
+    return S == 6 ? launch_matvec_affine<6, kXSiluMul>(c, cb, gate_up, nullptr, nullptr, nullptr, 0.f, scales_in, biases_in, scales_out, biases_out, out, m, n, mode, stream, ms)
+                  : launch_matvec_affine<8, kXSiluMul>(c, cb, gate_up, nullptr, nullptr, nullptr, 0.f, scales_in, biases_in, scales_out, biases_out, out, m, n, mode, stream, ms);
+}
+
+extern "C" int rptc_decompress_matvec_rmsnorm_affine(const int32_t *c, const uint16_t *cb, const uint16_t *x_in,
+                                                     const uint16_t *delta, const uint16_t *weight, uint16_t *x_out,
+                                                     const uint16_t *scales_in, const uint16_t *biases_in,
+                                                     const uint16_t *scales_out, const uint16_t *biases_out,
+                                                     uint16_t *out, int64_t m, int64_t n, float eps, int S, int mode,
+                                                     void *stream, float *ms)
+{
+    if (!weight || !x_out) return RPTC_ENULL;
+    if (S != 6 && S != 8) return RPTC_ESHAPE;
+    if (x_out == x_in || x_out == delta) return RPTC_EALIAS;
+    if (!aligned16(delta) || !aligned16(weight) || !aligned16(x_out)) return RPTC_EALIGN;
+    return S == 6 ? launch_matvec_affine<6, kXAddRmsNorm>(c, cb, x_in, delta, weight, x_out, eps, scales_in, biases_in, scales_out, biases_out, out, m, n, mode, stream, ms)
+                  : launch_matvec_affine<8, kXAddRmsNorm>(c, cb, x_in, delta, weight, x_out, eps, scales_in, biases_in, scales_out, biases_out, out, m, n, mode, stream, ms);
 }
 
 extern "C" int rptc_decompress_matvec_hadamard(const int32_t *c, const uint16_t *cb, const uint16_t *x,

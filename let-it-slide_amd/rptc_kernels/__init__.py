@@ -24,6 +24,8 @@ a stream stands for), ``decompress_matmul_16_{6,8}_1`` and ``decompress_matmul_b
 the matrix cores), ``decompress_matvec_bits`` (2, 3, 4 bits per weight), ``decompress_matvec_silu`` and
 ``decompress_matvec_rmsnorm`` (the mat-vec with a decoder layer's element-wise step in its prologue),
 ``decompress_matvec_hadamard`` (with the sign-Hadamard transform of its activations in its prologue),
+``decompress_matvec_affine`` / ``_silu_affine`` / ``_rmsnorm_affine`` (with the row/column scales and biases of
+the reference's factorisation, quantize_hf.py:167, applied inside the kernel),
 ``sign_hadamard``, ``viterbi_pairs`` and ``viterbi_scalar`` (the quantizer's trellis search, rptc.py:13-71,
 as kernels: for the hashed pair stream and for the reference's own scalar trellis).
 Sub-modules: ``packing`` (symbols -> streams), ``quantize`` (the quantizer around that search),
@@ -83,6 +85,9 @@ _SIGNATURES = {
     "rptc_decompress_matvec_hadamard": ([_VP, _VP, _VP, _VP, _VP, _I64, _I64, _I64, _INT, _INT, _VP, _FP], _INT),
     "rptc_decompress_matvec_rmsnorm": ([_VP, _VP, _VP, _VP, _VP, _VP, _VP, _I64, _I64, ctypes.c_float, _INT, _INT,
                                         _VP, _FP], _INT),
+    "rptc_decompress_matvec_affine": ([_VP] * 8 + [_I64, _I64, _INT, _INT, _VP, _FP], _INT),
+    "rptc_decompress_matvec_silu_affine": ([_VP] * 8 + [_I64, _I64, _INT, _INT, _VP, _FP], _INT),
+    "rptc_decompress_matvec_rmsnorm_affine": ([_VP] * 11 + [_I64, _I64, ctypes.c_float, _INT, _INT, _VP, _FP], _INT),
 }
 
 
@@ -542,6 +547,75 @@ def decompress_matvec_rmsnorm(compressed, codebook, x_in, delta, weight, x_out, 
             ctypes.c_void_p(stream), ctypes.byref(ms) if _timing else None)
     _status(rc)
     return float(ms.value)
+
+
+def _affine_ptrs(n, m, scales_in, biases_in, scales_out, biases_out):
+    ptrs = []
+    for t, name, length in ((scales_in, "scales_in", n), (biases_in, "biases_in", n),
+                            (scales_out, "scales_out", m), (biases_out, "biases_out", m)):
+        if t is None:
+            ptrs.append(None)
+            continue
+        _check_input(t, name)
+        _check(t.dim() == 1 and t.dtype == torch.float16 and t.size(0) == length, f"{name} must be fp16 [{length}]")
+        ptrs.append(t.data_ptr())
+    return ptrs
+
+
+def _call_affine(fn, head, tail, device, carry_mode):
+    ms = ctypes.c_float(0.0)
+    mode = _carry_mode if carry_mode is None else carry_mode
+    with torch.cuda.device(device):
+        stream = torch.cuda.current_stream().cuda_stream
+        rc = fn(*head, *tail, mode, ctypes.c_void_p(stream), ctypes.byref(ms) if _timing else None)
+    _status(rc)
+    return float(ms.value)
+
+
+def decompress_matvec_affine(compressed, codebook, x, out, scales_in=None, biases_in=None, scales_out=None,
+                             biases_out=None, carry_mode=None):
+    """out = scales_out * (W_hat (scales_in * x)) + biases_out * sum(x) + biases_in . x: the product with the
+    matrix the reference's quantizer reconstructs, W = b_out + b_in + s_out * s_in * W_hat
+    (quantize_hf.py:167), in one launch.  The four vectors are fp16 ([n], [n], [m], [m]) or None; n <= 16384.
+    Returns elapsed ms."""
+    _check_input(x, "x")
+    _check(x.dim() == 1 and x.dtype == torch.float16, "x must be a 1-D fp16 tensor")
+    n = x.size(0)
+    m, S = _fused_common(compressed, codebook, out, n)
+    aff = _affine_ptrs(n, m, scales_in, biases_in, scales_out, biases_out)
+    return _call_affine(library().rptc_decompress_matvec_affine,
+                        (compressed.data_ptr(), codebook.data_ptr(), x.data_ptr(), *aff, out.data_ptr()), (m, n, S),
+                        compressed.device, carry_mode)
+
+
+def decompress_matvec_silu_affine(compressed, codebook, gate_up, out, scales_in=None, biases_in=None, scales_out=None,
+                                  biases_out=None, carry_mode=None):
+    """``decompress_matvec_affine`` on silu(gate) * up, gate_up = [gate | up] (fp16 [2n])."""
+    _check_input(gate_up, "gate_up")
+    _check(gate_up.dim() == 1 and gate_up.dtype == torch.float16 and gate_up.size(0) % 2 == 0,
+           "gate_up must be a 1-D fp16 tensor of even length")
+    n = gate_up.size(0) // 2
+    m, S = _fused_common(compressed, codebook, out, n)
+    aff = _affine_ptrs(n, m, scales_in, biases_in, scales_out, biases_out)
+    return _call_affine(library().rptc_decompress_matvec_silu_affine,
+                        (compressed.data_ptr(), codebook.data_ptr(), gate_up.data_ptr(), *aff, out.data_ptr()), (m, n, S),
+                        compressed.device, carry_mode)
+
+
+def decompress_matvec_rmsnorm_affine(compressed, codebook, x_in, delta, weight, x_out, out, eps=1e-5, scales_in=None,
+                                     biases_in=None, scales_out=None, biases_out=None, carry_mode=None):
+    """``decompress_matvec_affine`` on rmsnorm(x_in + delta) * weight; x_out = x_in + delta (see
+    ``decompress_matvec_rmsnorm``)."""
+    for t, name in ((x_in, "x_in"), (weight, "weight"), (x_out, "x_out")) + (((delta, "delta"),) if delta is not None else ()):
+        _check_input(t, name)
+        _check(t.dim() == 1 and t.dtype == torch.float16 and t.size(0) == x_in.size(0), f"{name} must be fp16 [n]")
+    n = x_in.size(0)
+    m, S = _fused_common(compressed, codebook, out, n)
+    aff = _affine_ptrs(n, m, scales_in, biases_in, scales_out, biases_out)
+    return _call_affine(library().rptc_decompress_matvec_rmsnorm_affine,
+                        (compressed.data_ptr(), codebook.data_ptr(), x_in.data_ptr(),
+                         None if delta is None else delta.data_ptr(), weight.data_ptr(), x_out.data_ptr(), *aff,
+                         out.data_ptr()), (m, n, float(eps), S), compressed.device, carry_mode)
 
 
 def matvec_bits_dense(compressed, codebook, out, bits):

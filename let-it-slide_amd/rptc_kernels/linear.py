@@ -134,6 +134,17 @@ class QuantizedLinear(torch.nn.Module):
             raise RuntimeError("QuantizedLinear runs on fp16 CUDA tensors only (there is no CPU path)")
         shape = x.shape
         x2 = x.reshape(-1, self.in_features).contiguous()
+        affine = (self.scales_in, self.biases_in, self.scales_out, self.biases_out)
+        if (x2.size(0) == 1 and self.bits == 2 and self.signs is None and self.in_features <= 16384
+                and any(v is not None for v in affine)):
+            # one token: scales and biases are applied inside the mat-vec
+            y = torch.empty((1, self.out_features), dtype=torch.float16, device=x2.device)
+            prev = rk.set_timing(False)
+            try:
+                rk.decompress_matvec_affine(self.compressed, self.codebook, x2[0], y[0], *affine, carry_mode=self.carry_mode)
+            finally:
+                rk.set_timing(prev)
+            return y.reshape(shape[:-1] + (self.out_features,))
         xs = x2 * self.scales_in if self.scales_in is not None else x2
         if self.signs is not None and xs.size(0) == 1 and self.bits == 2 and self.in_features <= 15360:
             # one token: the transform runs in the prologue of the mat-vec

@@ -358,6 +358,118 @@ def test_matvec_rmsnorm_rejects_aliases_and_long_vectors(rk):
         rk.decompress_matvec_rmsnorm(comp2, cb, x2, None, x2.clone(), torch.empty_like(x2), out)
 
 
+def _affine_vectors(m, n, which, seed):
+    g = torch.Generator().manual_seed(seed)
+    si = (torch.rand(n, generator=g) + 0.5).half().cuda() if "si" in which else None
+    bi = (torch.randn(n, generator=g) * 0.02).half().cuda() if "bi" in which else None
+    so = (torch.rand(m, generator=g) + 0.5).half().cuda() if "so" in which else None
+    bo = (torch.randn(m, generator=g) * 0.02).half().cuda() if "bo" in which else None
+    return si, bi, so, bo
+
+
+def _affine_truth(W, a, si, bi, so, bo):
+    """quantize_hf.py:167 in float64 on the decoded matrix W and the fp16 activations a (s_in * a rounded to
+    fp16, as every path of this library stages it)."""
+    a64 = a.double()
+    xs = (a * si).double() if si is not None else a64            # fp16 product, rounded
+    y = W.double() @ xs
+    if so is not None:
+        y = y * so.double()
+    if bo is not None:
+        y = y + bo.double() * a64.sum()
+    if bi is not None:
+        y = y + (bi.double() * a64).sum()
+    return y
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+@pytest.mark.parametrize("which", [(), ("si",), ("bi",), ("so",), ("bo",), ("si", "bi", "so", "bo")])
+@pytest.mark.parametrize("S,m,n", [(8, 64, 2048), (6, 33, 704), (8, 96, 4096 + 768), (8, 600, 4096), (8, 32, 16384), (8, 2, 64)])
+def test_matvec_affine_applies_the_factorisation(rk, mode, which, S, m, n):
+    comp, cb = _stream(m, n, S, seed=13)
+    x = rand_half(n, seed=61).cuda()
+    si, bi, so, bo = _affine_vectors(m, n, which, seed=62)
+    W = torch.empty((m, n), dtype=torch.float16, device="cuda")
+    got = torch.full((m,), float("nan"), dtype=torch.float16, device="cuda")
+    prev = rk.set_carry_mode(mode)
+    try:
+        rk.matvec_dense(comp, cb, W, S)
+        ms = rk.decompress_matvec_affine(comp, cb, x, got, si, bi, so, bo)
+        if not which:
+            plain = torch.empty_like(got)
+            getattr(rk, f"decompress_matvec_16_{S}_1")(comp.reshape(n // 2048, m, 128) if n % 2048 == 0 else comp, cb, x, plain)
+            assert torch.equal(got.view(torch.int16), plain.view(torch.int16))
+    finally:
+        rk.set_carry_mode(prev)
+    assert ms > 0
+    want = _affine_truth(W, x, si, bi, so, bo)
+    assert rel_l2(got.float().cpu().numpy(), want.cpu().numpy()) < 1e-3
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+@pytest.mark.parametrize("m,n", [(64, 2048), (96, 4096 + 768), (40, 11008)])
+def test_matvec_silu_affine(rk, mode, m, n):
+    import ctypes
+    S = 8
+    comp, cb = _stream(m, n, S, seed=15)
+    gu = rand_half(2 * n, seed=71).cuda()
+    act = torch.empty(n, dtype=torch.float16, device="cuda")
+    assert rk.library().rptc_silu_mul(gu.data_ptr(), act.data_ptr(), n, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)) == 0
+    si, bi, so, bo = _affine_vectors(m, n, ("si", "bi", "so", "bo"), seed=72)
+    W = torch.empty((m, n), dtype=torch.float16, device="cuda")
+    got = torch.full((m,), float("nan"), dtype=torch.float16, device="cuda")
+    prev = rk.set_carry_mode(mode)
+    try:
+        rk.matvec_dense(comp, cb, W, S)
+        rk.decompress_matvec_silu_affine(comp, cb, gu, got, si, bi, so, bo)
+    finally:
+        rk.set_carry_mode(prev)
+    assert rel_l2(got.float().cpu().numpy(), _affine_truth(W, act, si, bi, so, bo).cpu().numpy()) < 1e-3
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+@pytest.mark.parametrize("with_delta", [False, True])
+@pytest.mark.parametrize("m,n", [(64, 2048), (40, 256), (96, 4096), (32, 16384)])
+def test_matvec_rmsnorm_affine(rk, mode, with_delta, m, n):
+    import ctypes
+    S = 8
+    comp, cb = _stream(m, n, S, seed=17)
+    x = rand_half(n, seed=81).cuda()
+    delta = rand_half(n, seed=82, scale=0.5).cuda() if with_delta else None
+    w = (1.0 + 0.1 * rand_half(n, seed=83).float()).half().cuda()
+    x_ref, h_ref = torch.empty_like(x), torch.empty_like(x)
+    assert rk.library().rptc_add_rmsnorm(x.data_ptr(), None if delta is None else delta.data_ptr(), w.data_ptr(),
+                                         x_ref.data_ptr(), h_ref.data_ptr(), n, 1e-5,
+                                         ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)) == 0
+    si, bi, so, bo = _affine_vectors(m, n, ("si", "bi", "so", "bo"), seed=84)
+    W = torch.empty((m, n), dtype=torch.float16, device="cuda")
+    got = torch.full((m,), float("nan"), dtype=torch.float16, device="cuda")
+    x_out = torch.full((n,), float("nan"), dtype=torch.float16, device="cuda")
+    prev = rk.set_carry_mode(mode)
+    try:
+        rk.matvec_dense(comp, cb, W, S)
+        rk.decompress_matvec_rmsnorm_affine(comp, cb, x, delta, w, x_out, got, 1e-5, si, bi, so, bo)
+    finally:
+        rk.set_carry_mode(prev)
+    assert torch.equal(x_out.view(torch.int16), x_ref.view(torch.int16))
+    # the normed activations may differ from the stand-alone kernel's in the last fp16 bit (order of the sum of squares)
+    assert rel_l2(got.float().cpu().numpy(), _affine_truth(W, h_ref, si, bi, so, bo).cpu().numpy()) < 1e-3
+
+
+def test_matvec_affine_refuses_long_vectors_and_checks_lengths(rk):
+    m, n = 32, 16384 + 2048
+    comp, cb = _stream(m, n, 8, seed=19)
+    x = rand_half(n, seed=3).cuda()
+    out = torch.empty(m, dtype=torch.float16, device="cuda")
+    with pytest.raises(RuntimeError, match="exceeds"):
+        rk.decompress_matvec_affine(comp, cb, x, out, scales_in=torch.ones_like(x))
+    m, n = 32, 2048
+    comp, cb = _stream(m, n, 8, seed=20)
+    x = rand_half(n, seed=4).cuda()
+    with pytest.raises(RuntimeError):
+        rk.decompress_matvec_affine(comp, cb, x, out, scales_out=torch.ones(n, dtype=torch.float16, device="cuda"))
+
+
 @pytest.mark.parametrize("heads,hd,max_len,pos", [(4, 64, 128, 0), (4, 64, 128, 77), (32, 128, 1024, 640), (2, 16, 64, 63),
                                                  (256, 16, 32, 20), (64, 128, 2048, 2047), (3, 256, 48, 5)])
 def test_rope_attn_decode_equals_rope_then_attention(rk, heads, hd, max_len, pos):
