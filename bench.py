@@ -54,6 +54,10 @@ def parse():
                     help="greedy decode with a Llama-2-7B-shaped random-init model whose projections are 2-bit streams "
                          "(prompt 512, 128 new tokens, batch 1); prints its own JSON line")
     ap.add_argument("--decode-layers", type=int, default=32)
+    ap.add_argument("--decode-quantized", action="store_true",
+                    help="with --decode: the projections are random-init dense weights put through the quantizer "
+                         "(row/column factorisation + trellis search) instead of random streams; their scales and "
+                         "biases are applied inside the mat-vec kernels")
     ap.add_argument("--matmul", action="store_true",
                     help="time the batch 8/16/32 fused decode + MFMA mat-mat instead (prints its own JSON line)")
     return ap.parse_args()
@@ -451,11 +455,21 @@ def main():
     if a.decode:
         from rptc_kernels.llama_decode import LlamaShape, QuantizedLlama, greedy_decode
         shape = LlamaShape(layers=a.decode_layers)
-        model = QuantizedLlama(shape, S=a.S)
+        t0 = time.perf_counter()
+        model = QuantizedLlama(shape, S=a.S, quantize_init=a.decode_quantized)
+        torch.cuda.synchronize()
+        build_s = time.perf_counter() - t0
         g = torch.Generator().manual_seed(42)
         prompt = torch.randint(0, shape.vocab, (512,), generator=g)
         res = {}
-        for mode in ("fused_graph", "fused", "glue_graph", "torch_graph", "torch"):
+        if a.decode_quantized:
+            blk = model.blocks[0]
+            res["quantizer"] = {"seconds_for_the_model": round(build_s, 1),
+                                "mse_of_the_normalised_weights_layer_0": {
+                                    name: round(getattr(blk, name).quantization_mse, 4)
+                                    for name in ("qkv_proj", "o_proj", "gate_up_proj", "down_proj")}}
+        for mode in (("fused_graph", "glue_graph") if a.decode_quantized else
+                     ("fused_graph", "fused", "glue_graph", "torch_graph", "torch")):
             model.k_cache.zero_()
             model.v_cache.zero_()
             toks, dt = greedy_decode(model, prompt, 128, mode=mode)
@@ -464,7 +478,10 @@ def main():
         print(json.dumps({"metric": "decode tok/s Llama-2-7B-shape bs=1", "value": res["fused_graph"]["tok_per_s"], "unit": "tok/s",
                           "n_gpus": 1, "data": "synthetic",
                           "config": {"workload": f"{shape.layers} layers d=4096 heads=32 mlp=11008 vocab=32000, random-init, "
-                                                 f"projections as seeded random 2-bit streams ({stream_bytes} bytes), prompt 512 "
+                                                 + ("projections random-init dense weights quantized to 2 bits (factorisation + trellis search), "
+                                                    "their scales and biases applied in the kernels " if a.decode_quantized else
+                                                    "projections as seeded random 2-bit streams ") +
+                                                 f"({stream_bytes} bytes), prompt 512 "
                                                  f"random ids, 128 greedy tokens; fused_graph = five launches per layer (element-wise steps inside the projections) in one HIP graph per token; glue_graph = nine launches per layer"},
                           "results": res}))
         return

@@ -470,17 +470,20 @@ __device__ __forceinline__ void matvec_body(
     float act_sum = 0.f, act_bias = 0.f;                   // sum(a), b_in . a
     if constexpr (AFFINE) {
         // host side guarantees n8 <= kXRegs * kMatvecThreads: the whole vector is in registers
+        // two-term dot products for the sums (fp32 inside) and packed fp16 products for the scaling: a
+        // product of two fp16 values rounded once to fp16 either way
 #pragma unroll
         for (int u = 0; u < kXRegs; u++) {
-            Halves8 v = unpack8(xv[u]);                     // zero past the end of the vector
-            const Halves8 bi = unpack8(xbi[u]), si = unpack8(xsi[u]);
+            uint32_t v[4] = {xv[u].x, xv[u].y, xv[u].z, xv[u].w};      // zero past the end of the vector
+            const uint32_t bi[4] = {xbi[u].x, xbi[u].y, xbi[u].z, xbi[u].w}, si[4] = {xsi[u].x, xsi[u].y, xsi[u].z, xsi[u].w};
 #pragma unroll
-            for (int i = 0; i < 8; i++) {
-                act_sum += v.v[i];
-                act_bias += v.v[i] * bi.v[i];
-                if (fuse.s_in) v.v[i] *= si.v[i];
+            for (int i = 0; i < 4; i++) {
+                act_sum = dot2(v[i], 0x3C003C00u, act_sum);            // (1.0, 1.0)
+                act_bias = dot2(v[i], bi[i], act_bias);
+                if (fuse.s_in)
+                    v[i] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, v[i]) * __builtin_bit_cast(half2_t, si[i]));
             }
-            if (fuse.s_in) xv[u] = pack8(v);
+            if (fuse.s_in) xv[u] = make_uint4(v[0], v[1], v[2], v[3]);
         }
         act_sum = wave_sum(act_sum);
         act_bias = wave_sum(act_bias);

@@ -69,13 +69,27 @@ class QuantizedLinear(torch.nn.Module):
         return layer
 
     @classmethod
-    def from_weight(cls, weight, codebook=None, S=8, importance=None, seed=42, device="cuda", bits=2, signs=None):
+    def from_weight(cls, weight, codebook=None, S=8, importance=None, seed=42, device="cuda", bits=2, signs=None,
+                    factorize=False):
         """Quantize a dense weight [out, in] with the Viterbi search of ``rptc_kernels.quantize`` (run on
         ``device``) and pack the result.  codebook: fp16 [2^(S+1)] or None for a seeded Gaussian one
         scaled to the weight's standard deviation.  signs: +-1 per input feature; the layer then stores
-        the weight in the sign-Hadamard basis (outliers spread over a block) and transforms its input."""
+        the weight in the sign-Hadamard basis (outliers spread over a block) and transforms its input.
+        factorize: take the reference's row/column scales and biases out first (quantize_hf.py:77-117), search
+        on the normalised matrix with column i weighted by importance_i * s_in_i^2 (the reference hands
+        diag(H) * s_in to a search that squares it, quantize_hf.py:139 and rptc.py:32; here ``importance`` is
+        the loss weight itself) and keep the four vectors on the layer (``set_affine``)."""
         from rptc_kernels import quantize
         W = torch.as_tensor(weight).to(device=device, dtype=torch.float32)
+        if factorize:
+            if signs is not None:
+                raise ValueError("factorize and signs are two ways to condition a weight: use one")
+            b_out, b_in, s_out, s_in, N = quantize.factorize(W)
+            imp = None
+            if importance is not None:
+                imp = torch.as_tensor(importance, dtype=torch.float32, device=device).reshape(-1) * s_in.reshape(-1) ** 2
+            layer = cls.from_weight(N, codebook=codebook, S=S, importance=imp, seed=seed, device=device, bits=bits)
+            return layer.set_affine(s_out.reshape(-1), s_in.reshape(-1), b_out.reshape(-1), b_in.reshape(-1))
         if signs is not None:
             W = quantize.sign_hadamard_rows(W, signs)
         if codebook is None:
@@ -191,6 +205,22 @@ class QuantizedLinear(torch.nn.Module):
                      self.in_features, self.S, self.bits, carry_mode=self.carry_mode)
         finally:
             rk.set_timing(prev)
+        return W
+
+    def reconstructed_weight(self):
+        """The dense matrix this layer multiplies by, float32 [m, n]: b_out + b_in + s_out * s_in * W_hat
+        (quantize_hf.py:167) with the vectors that are set; without signs."""
+        if self.signs is not None:
+            raise RuntimeError("a layer with a sign-Hadamard transform has no dense matrix in the input's own basis here")
+        W = self.decoded_weight().float()
+        if self.scales_in is not None:
+            W = W * self.scales_in.float()[None, :]
+        if self.scales_out is not None:
+            W = W * self.scales_out.float()[:, None]
+        if self.biases_out is not None:
+            W = W + self.biases_out.float()[:, None]
+        if self.biases_in is not None:
+            W = W + self.biases_in.float()[None, :]
         return W
 
     def compressed_bytes(self):

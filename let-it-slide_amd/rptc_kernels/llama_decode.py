@@ -5,8 +5,8 @@ HuggingFace Llama-2-7B (quantize_hf.py:189) but writes dense weights back and ge
 ``transformers`` (quantize_hf.py:229-236).  Here the same projections run on the packed streams,
 grouped the way the reference groups them for its Hessians (quantize_hf.py:14-22: q, k, v -> one
 "qkv" matrix, gate and up -> one "up" matrix), which is one kernel launch per group.  The model is
-built from its shape only (random-init norms, embeddings and lm_head; seeded random streams for the
-projections): nothing is downloaded.
+built from its shape only (random-init norms, embeddings and lm_head; for the projections seeded random
+streams, or random-init dense weights quantized with the reference's procedure): nothing is downloaded.
 
 Two ways through a token: ``forward_tokens`` (torch ops between the projections; used for the
 prompt, any number of tokens) and ``decode_step`` (this library's fused glue kernels, one token).
@@ -31,7 +31,12 @@ class LlamaShape:
 class QuantizedLlama(torch.nn.Module):
     EPS = 1e-5
 
-    def __init__(self, shape, S=8, seed=42, device="cuda"):
+    def __init__(self, shape, S=8, seed=42, device="cuda", quantize_init=False, init_std=0.02):
+        """quantize_init=False: seeded random streams (decode cost does not depend on the data).
+        quantize_init=True: every projection is a random-init dense weight (normal, ``init_std``: the
+        initialisation of the reference's model class) put through the reference's procedure - row/column
+        factorisation (quantize_hf.py:77-117), then the trellis search on the normalised matrix - and run
+        with its four vectors applied inside the mat-vec kernels."""
         super().__init__()
         self.shape = shape
         g = torch.Generator(device=device)
@@ -41,11 +46,21 @@ class QuantizedLlama(torch.nn.Module):
         self.lm_head = (torch.randn((shape.vocab, d), generator=g, device=device) * d ** -0.5).half()
         self.final_norm = torch.ones(d, dtype=torch.float16, device=device)
         self.blocks = torch.nn.ModuleList()
+        codebook = None
+        if quantize_init:
+            # the normalised matrices have unit RMS: one unit-variance codebook serves every projection
+            codebook = torch.randn(2 << S, generator=torch.Generator().manual_seed(seed)).to(torch.float16)
         for i in range(shape.layers):
             blk = torch.nn.Module()
             for j, (name, n_in, n_out) in enumerate((("qkv_proj", d, 3 * d), ("o_proj", d, d),
                                                      ("gate_up_proj", d, 2 * f), ("down_proj", f, d))):
-                setattr(blk, name, QuantizedLinear.from_random(n_in, n_out, S=S, seed=seed + 16 * i + j, device=device))
+                if quantize_init:
+                    W = torch.randn((n_out, n_in), generator=g, device=device) * init_std
+                    layer = QuantizedLinear.from_weight(W, codebook=codebook, S=S, device=device, factorize=True)
+                    del W
+                else:
+                    layer = QuantizedLinear.from_random(n_in, n_out, S=S, seed=seed + 16 * i + j, device=device)
+                setattr(blk, name, layer)
             blk.norm1 = torch.ones(d, dtype=torch.float16, device=device)
             blk.norm2 = torch.ones(d, dtype=torch.float16, device=device)
             self.blocks.append(blk)
@@ -117,18 +132,51 @@ class QuantizedLlama(torch.nn.Module):
             if rc:
                 raise RuntimeError(lib.rptc_status_string(rc).decode())
 
+        def affine(layer):
+            # the four vectors of the reference's factorisation as pointers, or None when the layer has none
+            vs = (layer.scales_in, layer.biases_in, layer.scales_out, layer.biases_out)
+            if all(v is None for v in vs):
+                return None
+            return [None if v is None else v.data_ptr() for v in vs]
+
         def gemv(layer, x, out):
+            aff = affine(layer)
+            if aff is not None and layer.in_features > 16384:
+                out.copy_(layer(x.unsqueeze(0))[0])        # too long for the fused form: framework ops around the plain call
+                return
+            if aff is not None:
+                ok(lib.rptc_decompress_matvec_affine(layer.compressed.data_ptr(), layer.codebook.data_ptr(), x.data_ptr(), *aff,
+                                                     out.data_ptr(), layer.out_features, layer.in_features, layer.S,
+                                                     layer.carry_mode, stream, None))
+                return
             fn = getattr(lib, f"rptc_decompress_matvec_16_{layer.S}_1")
             ok(fn(layer.compressed.data_ptr(), layer.codebook.data_ptr(), x.data_ptr(), out.data_ptr(),
                   layer.out_features, layer.in_features, layer.carry_mode, stream, None))
 
         def gemv_norm(layer, x_in, delta, weight, x_out, out):
+            aff = affine(layer)
+            if aff is not None:
+                ok(lib.rptc_decompress_matvec_rmsnorm_affine(layer.compressed.data_ptr(), layer.codebook.data_ptr(),
+                                                             x_in.data_ptr(), delta, weight.data_ptr(), x_out.data_ptr(), *aff,
+                                                             out.data_ptr(), layer.out_features, layer.in_features, self.EPS,
+                                                             layer.S, layer.carry_mode, stream, None))
+                return
             ok(lib.rptc_decompress_matvec_rmsnorm(layer.compressed.data_ptr(), layer.codebook.data_ptr(), x_in.data_ptr(),
                                                   delta, weight.data_ptr(), x_out.data_ptr(), out.data_ptr(),
                                                   layer.out_features, layer.in_features, self.EPS, layer.S,
                                                   layer.carry_mode, stream, None))
 
         def gemv_silu(layer, gate_up, out):
+            aff = affine(layer)
+            if aff is not None and layer.in_features > 16384:
+                ok(lib.rptc_silu_mul(gate_up.data_ptr(), self._act.data_ptr(), layer.in_features, stream))
+                gemv(layer, self._act, out)
+                return
+            if aff is not None:
+                ok(lib.rptc_decompress_matvec_silu_affine(layer.compressed.data_ptr(), layer.codebook.data_ptr(),
+                                                          gate_up.data_ptr(), *aff, out.data_ptr(), layer.out_features,
+                                                          layer.in_features, layer.S, layer.carry_mode, stream, None))
+                return
             ok(lib.rptc_decompress_matvec_silu(layer.compressed.data_ptr(), layer.codebook.data_ptr(), gate_up.data_ptr(),
                                                out.data_ptr(), layer.out_features, layer.in_features, layer.S,
                                                layer.carry_mode, stream, None))

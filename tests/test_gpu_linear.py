@@ -242,6 +242,58 @@ def test_llama_decode_paths_agree(rk):
     assert rel_l2(logits_q.cpu().numpy(), logits_d.cpu().numpy()) < 2e-2
 
 
+def test_llama_built_from_dense_weights_through_the_reference_procedure(rk):
+    """Random-init dense projections, factorised and searched (quantize_hf.py:77-170's flow on the hashed pair
+    stream): every decode path agrees, and the logits are those of the same network on the matrices the layers
+    reconstruct (quantize_hf.py:167)."""
+    from rptc_kernels.llama_decode import LlamaShape, QuantizedLlama, greedy_decode
+    from rptc_kernels.linear import QuantizedLinear
+    shape = LlamaShape(layers=2, d_model=256, heads=4, d_ff=704, vocab=1000, max_len=128)
+    model = QuantizedLlama(shape, S=8, seed=11, quantize_init=True)
+    blk = model.blocks[0]
+    for name in ("qkv_proj", "o_proj", "gate_up_proj", "down_proj"):
+        layer = getattr(blk, name)
+        assert all(v is not None for v in (layer.scales_in, layer.scales_out, layer.biases_in, layer.biases_out))
+        # the search did its work: 2 bits per weight on a Gaussian matrix lands well under the variance
+        assert layer.quantization_mse < 0.12
+    prompt = torch.randint(0, shape.vocab, (40,), generator=torch.Generator().manual_seed(2))
+    runs = {}
+    for mode in ("fused_graph", "fused", "glue", "torch"):
+        model.k_cache.zero_(); model.v_cache.zero_()
+        runs[mode], _ = greedy_decode(model, prompt, 10, mode=mode)
+    assert runs["fused_graph"] == runs["fused"]
+
+    pos = torch.arange(40, device="cuda")
+    with torch.no_grad():
+        model.k_cache.zero_(); model.v_cache.zero_()
+        for p0 in (0, 32):
+            model.forward_tokens(prompt[p0:p0 + 32].cuda(), pos[p0:p0 + 32])
+        tok = torch.tensor([5], device="cuda")
+        p40 = torch.tensor([40], device="cuda")
+        kc, vc = model.k_cache.clone(), model.v_cache.clone()
+        lf = model.decode_step(tok, p40)
+        model.k_cache.copy_(kc); model.v_cache.copy_(vc)
+        lg = model.decode_step(tok, p40, fuse=False)
+        assert rel_l2(lf.cpu().numpy(), lg.cpu().numpy()) < 5e-3
+
+        # dense reference on the reconstructed matrices, float32 products
+        class Dense(torch.nn.Module):
+            def __init__(self, w):
+                super().__init__()
+                self.w = w
+
+            def forward(self, x):
+                return (x.float() @ self.w.t()).half()
+
+        for b in model.blocks:
+            for name, child in list(b.named_children()):
+                if isinstance(child, QuantizedLinear):
+                    setattr(b, name, Dense(child.reconstructed_weight()))
+        model.k_cache.copy_(kc); model.v_cache.copy_(vc)
+        ld = model.forward_tokens(tok, p40)
+    assert rel_l2(lf.cpu().numpy(), ld.cpu().numpy()) < 2e-2
+
+
 # ------------------------------------------------------------------ projections with a fused element-wise prologue
 
 def _stream(m, n, S=8, seed=0):
