@@ -426,9 +426,9 @@ __device__ __forceinline__ void matvec_body(
         ss = wave_sum(ss);
         if (lane == 63) red[wave] = ss;
         __syncthreads();
-        float total_ss = 0.f;
-#pragma unroll
-        for (int w = 0; w < kMatvecWaves; w++) total_ss += red[w];
+        // one value per lane and a sum across the lanes: one LDS round trip instead of sixteen in a row
+        float total_ss = wave_sum(lane < kMatvecWaves ? red[lane] : 0.f);
+        total_ss = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, total_ss), 63));
         const float inv = rsqrtf(total_ss / (float)n + fuse.eps);
 #pragma unroll
         for (int u = 0; u < kXRegs; u++) {
@@ -485,12 +485,6 @@ __device__ __forceinline__ void matvec_body(
             }
             if (fuse.s_in) xv[u] = make_uint4(v[0], v[1], v[2], v[3]);
         }
-        act_sum = wave_sum(act_sum);
-        act_bias = wave_sum(act_bias);
-        if (lane == 63) {
-            red[kMatvecWaves + 2 * wave] = act_sum;
-            red[kMatvecWaves + 2 * wave + 1] = act_bias;
-        }
     }
 
     // table (256 rows x 64 lane copies) and activation image into LDS
@@ -512,15 +506,14 @@ __device__ __forceinline__ void matvec_body(
     __syncthreads();
     RPTC_STAMP(2);
     if constexpr (AFFINE) {
-        act_sum = act_bias = 0.f;
-#pragma unroll
-        for (int w = 0; w < kMatvecWaves; w++) {
-            act_sum += red[kMatvecWaves + 2 * w];
-            act_bias += red[kMatvecWaves + 2 * w + 1];
+        // the two sums are needed when the row sums are written: their reduction runs beside the decode,
+        // not in front of the barrier every wave waits at
+        act_sum = wave_sum(act_sum);
+        act_bias = wave_sum(act_bias);
+        if (lane == 63) {
+            red[kMatvecWaves + 2 * wave] = act_sum;
+            red[kMatvecWaves + 2 * wave + 1] = act_bias;
         }
-        // the same in every lane: kept in scalar registers until the row sums are written
-        act_sum = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, act_sum)));
-        act_bias = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, act_bias)));
     }
 
     uint32_t xr[32];
@@ -612,6 +605,13 @@ __device__ __forceinline__ void matvec_body(
     }
     RPTC_STAMP(4);
     __syncthreads();
+    if constexpr (AFFINE) {
+        // one pair per lane and sums across the lanes; the totals are the same for every lane
+        act_sum = wave_sum(lane < kMatvecWaves ? red[kMatvecWaves + 2 * lane] : 0.f);
+        act_bias = wave_sum(lane < kMatvecWaves ? red[kMatvecWaves + 2 * lane + 1] : 0.f);
+        act_sum = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, act_sum), 63));
+        act_bias = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, act_bias), 63));
+    }
     // one wave per row: add the row's partial sums in a fixed order
     for (int r = wave, k = 0; r < rows; r += kMatvecWaves, k++) {
         float y = 0.f;
