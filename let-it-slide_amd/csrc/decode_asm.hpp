@@ -137,4 +137,63 @@ __device__ __forceinline__ void decode_element_asm(const uint4 e, const uint32_t
         : "vcc");
 }
 
+// The same block for 4 bits per weight: a step consumes 8 stream bits, an element is 8 words, and the
+// window of step s is the 16 bits that end 8 (s + 1) bits into the element.  Word i as it is holds the
+// windows of steps 4i + 1 (high half) and 4i + 3 (low half); the 32 bits that start 8 bits before word
+// i - one v_alignbit_b32 with the word in front (the previous lane's last word for i = 0) - hold those
+// of steps 4i and 4i + 2.  Per two words: 2 v_alignbit_b32, 4 v_pk_mad_u16, 8 address ops, 8 gathers,
+// 8 products.
+#define RPTC_WINDOWS4(WP, WA, WB)                             \
+    "v_alignbit_b32 %[g0], " WP ", " WA ", 8\n"               \
+    "v_alignbit_b32 %[g2], " WA ", " WB ", 8\n"               \
+    "v_pk_mad_u16 %[g0], %[g0], %[g0], %[g0]\n"               \
+    "v_pk_mad_u16 %[g1], " WA ", " WA ", " WA "\n"            \
+    "v_pk_mad_u16 %[g2], %[g2], %[g2], %[g2]\n"               \
+    "v_pk_mad_u16 %[g3], " WB ", " WB ", " WB "\n"
+
+// xs[q]: activation pair of the q-th step in stream order.  The gathers of a block of eight steps land
+// in the order of steps 0, 2, 1, 3, 4, 6, 5, 7 of the block.
+__device__ __forceinline__ void decode_element_asm4(const uint32_t (&w)[8], const uint32_t own, const uint64_t first_lanes,
+                                                    const uint32_t lane4, const uint32_t (&xs)[32], float &a0,
+                                                    float &a1, float &a2, float &a3)
+{
+    uint32_t carry;
+    uint32_t g0, g1, g2, g3, t0, t1, t2, t3, t4, t5, t6, t7, u0, u1, u2, u3, u4, u5, u6, u7;
+    asm volatile(
+        "s_nop 1\n"
+        "s_mov_b64 vcc, %[first]\n"
+        "v_cndmask_b32_dpp %[cy], %[w7], %[own], vcc wave_shr:1 row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        RPTC_WINDOWS4("%[cy]", "%[w0]", "%[w1]") RPTC_READS_X(RPTC_TA)
+        RPTC_WINDOWS4("%[w1]", "%[w2]", "%[w3]") RPTC_READS_X(RPTC_TB)
+        "s_waitcnt lgkmcnt(8)\n"
+        RPTC_DOTS_FIRST_X(RPTC_TA, "x0", "x2", "x1", "x3", "x4", "x6", "x5", "x7")
+        RPTC_WINDOWS4("%[w3]", "%[w4]", "%[w5]") RPTC_READS_X(RPTC_TA)
+        "s_waitcnt lgkmcnt(8)\n"
+        RPTC_DOTS_X(RPTC_TB, "x8", "x10", "x9", "x11", "x12", "x14", "x13", "x15")
+        RPTC_WINDOWS4("%[w5]", "%[w6]", "%[w7]") RPTC_READS_X(RPTC_TB)
+        "s_waitcnt lgkmcnt(8)\n"
+        RPTC_DOTS_X(RPTC_TA, "x16", "x18", "x17", "x19", "x20", "x22", "x21", "x23")
+        "s_waitcnt lgkmcnt(0)\n"
+        RPTC_DOTS_X(RPTC_TB, "x24", "x26", "x25", "x27", "x28", "x30", "x29", "x31")
+        "s_nop 3\n"
+        : [a0] "=&v"(a0), [a1] "=&v"(a1), [a2] "=&v"(a2), [a3] "=&v"(a3),
+          [cy] "=&v"(carry), [g0] "=&v"(g0), [g1] "=&v"(g1), [g2] "=&v"(g2), [g3] "=&v"(g3),
+          [t0] "=&v"(t0), [t1] "=&v"(t1), [t2] "=&v"(t2), [t3] "=&v"(t3),
+          [t4] "=&v"(t4), [t5] "=&v"(t5), [t6] "=&v"(t6), [t7] "=&v"(t7),
+          [u0] "=&v"(u0), [u1] "=&v"(u1), [u2] "=&v"(u2), [u3] "=&v"(u3),
+          [u4] "=&v"(u4), [u5] "=&v"(u5), [u6] "=&v"(u6), [u7] "=&v"(u7)
+        : [w0] "v"(w[0]), [w1] "v"(w[1]), [w2] "v"(w[2]), [w3] "v"(w[3]), [w4] "v"(w[4]), [w5] "v"(w[5]),
+          [w6] "v"(w[6]), [w7] "v"(w[7]), [own] "v"(own), [first] "s"(first_lanes),
+          [lane4] "v"(lane4), [mask] "s"(0xFF00u), [sel] "s"(0x0C0C0700u),
+          [x0] "v"(xs[0]), [x1] "v"(xs[1]), [x2] "v"(xs[2]), [x3] "v"(xs[3]),
+          [x4] "v"(xs[4]), [x5] "v"(xs[5]), [x6] "v"(xs[6]), [x7] "v"(xs[7]),
+          [x8] "v"(xs[8]), [x9] "v"(xs[9]), [x10] "v"(xs[10]), [x11] "v"(xs[11]),
+          [x12] "v"(xs[12]), [x13] "v"(xs[13]), [x14] "v"(xs[14]), [x15] "v"(xs[15]),
+          [x16] "v"(xs[16]), [x17] "v"(xs[17]), [x18] "v"(xs[18]), [x19] "v"(xs[19]),
+          [x20] "v"(xs[20]), [x21] "v"(xs[21]), [x22] "v"(xs[22]), [x23] "v"(xs[23]),
+          [x24] "v"(xs[24]), [x25] "v"(xs[25]), [x26] "v"(xs[26]), [x27] "v"(xs[27]),
+          [x28] "v"(xs[28]), [x29] "v"(xs[29]), [x30] "v"(xs[30]), [x31] "v"(xs[31])
+        : "vcc");
+}
+
 }  // namespace rptc

@@ -264,8 +264,9 @@ __global__ __launch_bounds__(kMmThreads) __attribute__((amdgpu_waves_per_eu(4, 4
                             h = o <= 16 ? e_all[rb][wi] >> (16 - o)
                                         : alignbit(e_all[rb][wi], e_all[rb][wi + 1 < WORDS ? wi + 1 : wi], 48 - o);
                         }
-                        h &= 0xFFFFu;
-                        const uint32_t prod = __umul24(h, h) + h;             // low 16 bits of h * (h + 1)
+                        // hash of the low half (what sits in the high half is cut off by the address mask)
+                        uint32_t prod;                                        // low 16 bits of h * (h + 1)
+                        asm("v_pk_mad_u16 %0, %1, %1, %1" : "=v"(prod) : "v"(h));
                         w[u] = lds_read_abs(and_or(prod, 0xFF00u, lane4));
                     }
                     const int k = mm_k_of_step_block(sb);

@@ -124,8 +124,10 @@ __device__ __forceinline__ float decode_element_bits(const Elem<2 * BITS> &e, ui
                 const int wi = start >> 5, o = start & 31;
                 h = o <= 16 ? e.w[wi] >> (16 - o) : alignbit(e.w[wi], e.w[wi + 1 < 2 * BITS ? wi + 1 : wi], 48 - o);
             }
-            h &= 0xFFFFu;
-            const uint32_t prod = __umul24(h, h) + h;                 // low 16 bits of h * (h + 1)
+            // the hash of the low half by a packed 16-bit multiply-add: whatever sits in the high half of h
+            // stays there and is cut off by the address mask
+            uint32_t prod;                                            // low 16 bits: h * (h + 1)
+            asm("v_pk_mad_u16 %0, %1, %1, %1" : "=v"(prod) : "v"(h));
             wv[u] = lds_read_abs(and_or(prod, 0xFF00u, lane4));
         }
 #pragma unroll
@@ -565,6 +567,13 @@ __device__ __forceinline__ void matvec_body(
                 float a0, a1, a2, a3;
                 decode_element_asm(make_uint4(cur[u].w[0], cur[u].w[1], cur[u].w[2], cur[u].w[3]), own, first_lanes,
                                    lane4, xr, a0, a1, a2, a3);
+                sum = (a0 + a1) + (a2 + a3);
+            } else if constexpr (BITS == 4) {
+                uint32_t xs[32];                        // the activation pairs in stream order of the steps
+#pragma unroll
+                for (int q = 0; q < 32; q++) xs[q] = xr[slot_of_step(q)];
+                float a0, a1, a2, a3;
+                decode_element_asm4(cur[u].w, own, first_lanes, lane4, xs, a0, a1, a2, a3);
                 sum = (a0 + a1) + (a2 + a3);
             } else {
                 uint32_t carry = __builtin_amdgcn_update_dpp(last, last, 0x138 /* wave_shr:1 */, 0xF, 0xF, false);
