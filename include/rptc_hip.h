@@ -223,8 +223,8 @@ int rptc_decompress_matvec_rmsnorm(const int32_t *compressed, const uint16_t *co
  *     out[r] = s_out[r] * (W_hat (s_in .* a))[r] + b_out[r] * sum(a) + (b_in . a)
  * with a the activations (x; silu(gate) * up; the normed residual), s_in .* a rounded to fp16 and
  * everything behind it in fp32 with one rounding at the end.  scales_in, biases_in: fp16 [n];
- * scales_out, biases_out: fp16 [m]; each may be NULL (scale 1, bias 0).  n <= 16384 (RPTC_ELIMIT
- * above: apply the vectors around the plain call instead).
+ * scales_out, biases_out: fp16 [m]; each may be NULL (scale 1, bias 0).  n <= 16384 and at most 1024 rows
+ * per compute unit (RPTC_ELIMIT above: apply the vectors around the plain call instead).
  */
 int rptc_decompress_matvec_affine(const int32_t *compressed, const uint16_t *codebook, const uint16_t *x,
                                   const uint16_t *scales_in, const uint16_t *biases_in,

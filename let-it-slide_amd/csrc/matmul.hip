@@ -252,6 +252,13 @@ __global__ __launch_bounds__(kMmThreads) __attribute__((amdgpu_waves_per_eu(4, 4
 #pragma unroll
                 for (int sb = 0; sb < 8; sb++) {
                     uint32_t w[4];
+                    if constexpr (BITS == 4) {
+                        // a step is 8 bits: word sb as it is holds the windows of steps 4sb+1 and 4sb+3, and the
+                        // 32 bits that start 8 bits before it those of steps 4sb and 4sb+2
+                        const uint32_t front = sb == 0 ? carry : e_all[rb][sb > 0 ? sb - 1 : 0];
+                        gather2(alignbit(front, e_all[rb][sb], 8), lane4, w[0], w[2]);
+                        gather2(e_all[rb][sb], lane4, w[1], w[3]);
+                    } else
 #pragma unroll
                     for (int u = 0; u < 4; u++) {
                         const int st = 4 * sb + u;

@@ -843,6 +843,8 @@ static int launch_matvec_affine(const int32_t *compressed, const uint16_t *codeb
     int rc = plan_matvec(compressed, codebook, x, out, m, n, carry_mode, false, kRedFloats * 4, &dev, &a, &compact,
                          &lds_bytes, &grid);
     if (rc) return rc;
+    // lane j of a wave holds the output-side factors of row wave + 16 j of the workgroup's block
+    if (a.rows_per_block > kMatvecWaves * kWave) return RPTC_ELIMIT;
     hipStream_t s = static_cast<hipStream_t>(stream);
     Timer t;
     rc = t.begin(dev, s, ms);

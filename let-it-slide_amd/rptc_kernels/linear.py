@@ -150,6 +150,7 @@ class QuantizedLinear(torch.nn.Module):
         x2 = x.reshape(-1, self.in_features).contiguous()
         affine = (self.scales_in, self.biases_in, self.scales_out, self.biases_out)
         if (x2.size(0) == 1 and self.bits == 2 and self.signs is None and self.in_features <= 16384
+                and self.out_features <= 1024 * torch.cuda.get_device_properties(x2.device).multi_processor_count
                 and any(v is not None for v in affine)):
             # one token: scales and biases are applied inside the mat-vec
             y = torch.empty((1, self.out_features), dtype=torch.float16, device=x2.device)
