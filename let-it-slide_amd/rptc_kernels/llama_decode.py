@@ -250,17 +250,27 @@ def greedy_decode(model, prompt, new_tokens, mode="fused_graph"):
             with torch.cuda.stream(side):
                 step(s_tok, s_pos)
             torch.cuda.current_stream().wait_stream(side)
+            # the token hand-over is part of the graph: the new token becomes the next input, is appended
+            # to the output buffer, and position and output index move on, so a token is one replay
+            s_idx = torch.zeros(1, dtype=torch.long, device=dev)
+            s_out = torch.zeros(max(new_tokens - 1, 1), dtype=torch.long, device=dev)
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
                 s_next = step(s_tok, s_pos).argmax(-1)
+                s_out.index_copy_(0, s_idx, s_next)
+                s_tok.copy_(s_next)
+                s_pos.add_(1)
+                s_idx.add_(1)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for _ in range(new_tokens - 1):
-            if graph is not None:
+        if graph is not None:
+            for _ in range(new_tokens - 1):
                 graph.replay()
-                nxt = s_next
-            else:
-                nxt = step(s_tok, s_pos).argmax(-1)
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
+            return [int(out[0])] + [int(t) for t in s_out[:new_tokens - 1]], dt
+        for _ in range(new_tokens - 1):
+            nxt = step(s_tok, s_pos).argmax(-1)
             s_tok.copy_(nxt)
             s_pos.add_(1)
             out.append(nxt.clone())
