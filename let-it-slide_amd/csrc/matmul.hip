@@ -156,8 +156,13 @@ __global__ __launch_bounds__(kMmThreads) __attribute__((amdgpu_waves_per_eu(4, 4
     const bool has_l = l < lanes;
     const int waves_used = (lanes + 3) >> 2;
 
-    // first request: this thread's row of the table (vector loads return in order)
-    const uint32_t table_value = mm_table_value<S>(codebook, tid >> 1);
+    // Table rows 32 * c .. 32 * c + 31 are this wave's to write.  A row is 64 copies of one value, so the
+    // value is wave-uniform and comes through the scalar cache: these loads neither queue with the vector
+    // loads below nor return in order with them.
+    constexpr int kTableRowsPerWave = 256 / kMmWaves;
+    uint32_t table_values[kTableRowsPerWave];
+#pragma unroll
+    for (int r = 0; r < kTableRowsPerWave; r++) table_values[r] = mm_table_value<S>(codebook, kTableRowsPerWave * c + r);
 
     // Everything comes straight into registers, all requests before the first use: the activation
     // pairs of this lane's 32 steps for its batch column(s) (lanes of one group read 64 consecutive
@@ -205,12 +210,9 @@ __global__ __launch_bounds__(kMmThreads) __attribute__((amdgpu_waves_per_eu(4, 4
     const bool no_carry = MODE == RPTC_CONTINUOUS && slab == 0 && l == 0;     // the stream starts here
 
     {
-        // table row r = tid / 2 (64 lane copies of one pair): each thread writes 32 copies of the value
-        // it asked for before anything else
-        uint4 *dst = reinterpret_cast<uint4 *>(lds) + (tid >> 1) * 16 + (tid & 1) * 8;
-        const uint4 v4 = make_uint4(table_value, table_value, table_value, table_value);
+        // 64 lane copies of each of the wave's rows
 #pragma unroll
-        for (int k = 0; k < 8; k++) dst[k] = v4;
+        for (int r = 0; r < kTableRowsPerWave; r++) lds[(kTableRowsPerWave * c + r) * 64 + lane] = table_values[r];
     }
     RPTC_MM_STAMP(1);
     __syncthreads();                                              // the table is complete
