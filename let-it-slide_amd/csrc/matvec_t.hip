@@ -48,19 +48,6 @@ __global__ __launch_bounds__(kTThreads) void matvec_t_kernel(
     constexpr int lut_u4 = (2 << L) / 16;
     constexpr uint32_t mask = (1u << L) - 1u;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    {
-        // all of a thread's share of the table is requested before any of it is stored
-        constexpr int kPerThread = lut_u4 / kTThreads;
-        uint4 t[kPerThread];
-#pragma unroll
-        for (int i = 0; i < kPerThread; i++) t[i] = codebook[i * kTThreads + tid];
-#pragma unroll
-        for (int i = 0; i < kPerThread; i++) lds_u4[i * kTThreads + tid] = t[i];
-    }
-    __syncthreads();
-    const uint16_t *lut = reinterpret_cast<const uint16_t *>(lds_u4);
-    float *part = reinterpret_cast<float *>(lds_u4 + lut_u4);      // [wave][lane]
-
     const int rb = blockIdx.x / ksplit, sp = blockIdx.x - rb * ksplit;
     const int row = rb * kWave + lane;
     const bool valid = row < m;
@@ -69,15 +56,32 @@ __global__ __launch_bounds__(kTThreads) void matvec_t_kernel(
     const int g0 = min(cols, sp * per_group), g1 = min(cols, g0 + per_group);
     const int per = (g1 - g0 + kTWaves - 1) / kTWaves;
     const int c0 = min(g1, g0 + wave * per), c1 = min(g1, c0 + per);
-    const uint4 zero = make_uint4(0, 0, 0, 0);
+
+    // Requests in the order their data is needed: the thread's share of the table, then the element in
+    // front of the wave's range (its state warms up the decoder) and the first two elements of the range.
+    // The stream requests are unconditional (clamped to an element that exists) so that the table can be
+    // stored while they are still on their way; what a clamped request returns is never used.
+    constexpr int kPerThread = lut_u4 / kTThreads;
+    uint4 t[kPerThread];
+#pragma unroll
+    for (int i = 0; i < kPerThread; i++) t[i] = codebook[i * kTThreads + tid];
+    const int row_c = min(row, m - 1), last_col = cols - 1;
+    const uint4 before = comp[(size_t)min(max(c0 - 1, 0), last_col) * m + row_c];
+    uint4 next = comp[(size_t)min(c0, last_col) * m + row_c];
+    uint4 next2 = comp[(size_t)min(c0 + 1, last_col) * m + row_c];
+#pragma unroll
+    for (int i = 0; i < kPerThread; i++) lds_u4[i * kTThreads + tid] = t[i];
+    __syncthreads();
+    const uint16_t *lut = reinterpret_cast<const uint16_t *>(lds_u4);
+    float *part = reinterpret_cast<float *>(lds_u4 + lut_u4);      // [wave][lane]
 
     uint32_t carry = 0;
-    if (c0 > 0 && c0 < c1 && valid) carry = warm_state<L>(comp[(size_t)(c0 - 1) * m + row], MODE);
+    if (c0 > 0 && c0 < c1 && valid) carry = warm_state<L>(before, MODE);
     float acc = 0.f;
-    uint4 next = (c0 < c1 && valid) ? comp[(size_t)c0 * m + row] : zero;
     for (int col = c0; col < c1; col++) {
         const uint4 e = next;
-        if (col + 1 < c1 && valid) next = comp[(size_t)(col + 1) * m + row];
+        next = next2;
+        if (col + 2 < c1) next2 = comp[(size_t)(col + 2) * m + row_c];
         const uint32_t words[4] = {e.x, e.y, e.z, e.w};
 #pragma unroll
         for (int k = 0; k < 4; k++) {
