@@ -123,7 +123,7 @@ template <int S, int MODE, int PLANES, int BITS>
 __global__ __launch_bounds__(kMmThreads) __attribute__((amdgpu_waves_per_eu(4, 4))) void matmul_kernel(
     const uint32_t *__restrict__ comp32, const uint32_t *__restrict__ codebook, const uint32_t *__restrict__ xp32,
     float *__restrict__ partial, uint32_t *__restrict__ arrived, uint16_t *__restrict__ out, int m, int n, int batch,
-    int max_rb, int groups_total, int group_base)
+    int max_rb, int rb_quot, int rb_rem, int group_base)
 {
     extern __shared__ uint32_t lds[];
     // 64 KiB of table + 16 KiB of tiles: two workgroups share a CU's 160 KiB whatever the batch
@@ -143,10 +143,12 @@ __global__ __launch_bounds__(kMmThreads) __attribute__((amdgpu_waves_per_eu(4, 4
     const int T = n >> 11, Lt = (n & 2047) >> 6, slabs = T + (Lt ? 1 : 0);
     // grp counts the row groups of this launch (a very tall matrix takes several launches)
     const int grp = blockIdx.x / slabs, slab = blockIdx.x - grp * slabs;
-    // the row blocks (16 rows each) are dealt to the groups as evenly as integers allow
-    const int total_rb = (m + 15) >> 4;
-    const int rb_begin = (int)(((int64_t)(group_base + grp) * total_rb) / groups_total);
-    const int row_blocks = (int)(((int64_t)(group_base + grp + 1) * total_rb) / groups_total) - rb_begin;
+    // the row blocks (16 rows each) are dealt to the groups as evenly as integers allow: rb_quot each,
+    // one more for the first rb_rem groups (quotient and remainder of row blocks / groups, from the host:
+    // a division here would be a loop of a few hundred instructions in front of the first request)
+    const int g_all = group_base + grp;
+    const int rb_begin = g_all * rb_quot + min(g_all, rb_rem);
+    const int row_blocks = rb_quot + (g_all < rb_rem ? 1 : 0);
     const int row0 = rb_begin * 16;
 
     const int lanes = slab < T ? 32 : Lt;                        // elements per row in this slab
@@ -428,11 +430,11 @@ static void launch_matmul(const uint32_t *comp, const uint32_t *cb, const MmScra
         if (carry_mode == RPTC_AS_WRITTEN)
             hipLaunchKernelGGL((matmul_kernel<S, RPTC_AS_WRITTEN, PLANES, BITS>), dim3(g_n * slabs), dim3(kMmThreads),
                                lds_bytes, s, comp, cb, sc.xpack, sc.partial, sc.arrived, out, m, n, batch, max_rb,
-                               groups, g0);
+                               total / groups, total % groups, g0);
         else
             hipLaunchKernelGGL((matmul_kernel<S, RPTC_CONTINUOUS, PLANES, BITS>), dim3(g_n * slabs), dim3(kMmThreads),
                                lds_bytes, s, comp, cb, sc.xpack, sc.partial, sc.arrived, out, m, n, batch, max_rb,
-                               groups, g0);
+                               total / groups, total % groups, g0);
     }
 }
 
