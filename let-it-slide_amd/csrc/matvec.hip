@@ -639,11 +639,12 @@ __device__ __forceinline__ void matvec_body(
 template <int S, int MODE, int BITS, bool COMPACT>
 __global__ __launch_bounds__(kMatvecThreads) void matvec_kernel(
     const uint32_t *__restrict__ comp, const uint32_t *__restrict__ codebook,
-    const uint4 *__restrict__ x, uint16_t *__restrict__ out, int arg_m, int arg_n, int arg_rows_per_block,
-    int arg_rw_tail, int arg_items_full, int arg_items_tail, uint32_t arg_full_magic)
+    const uint4 *__restrict__ x, int arg_m, int arg_n, int arg_rows_per_block,
+    int arg_rw_tail, int arg_items_tail, uint32_t arg_full_magic, uint16_t *__restrict__ out)
 {
-    // separate scalar arguments (not a struct) so that all of them are preloaded into SGPRs
-    const MatvecArgs a = {arg_m, arg_n, arg_rows_per_block, arg_rw_tail, arg_items_full, arg_items_tail, arg_full_magic};
+    // Separate scalar arguments (not a struct), and what the first requests need in the first 14 dwords:
+    // those arrive in SGPRs with the wave, the rest (the output pointer is needed last) through a scalar load.
+    const MatvecArgs a = {arg_m, arg_n, arg_rows_per_block, arg_rw_tail, arg_rows_per_block >> 1, arg_items_tail, arg_full_magic};
     matvec_body<S, MODE, BITS, kXPlain, COMPACT>(comp, codebook, x, out, a, XFuse{nullptr, nullptr, nullptr, 0.f, 0, nullptr, nullptr, nullptr, nullptr});
 }
 
@@ -651,11 +652,11 @@ __global__ __launch_bounds__(kMatvecThreads) void matvec_kernel(
 template <int S, int MODE, int XMODE, bool COMPACT>
 __global__ __launch_bounds__(kMatvecThreads) void matvec_fused_kernel(
     const uint32_t *__restrict__ comp, const uint32_t *__restrict__ codebook,
-    const uint4 *__restrict__ x, uint16_t *__restrict__ out, int arg_m, int arg_n, int arg_rows_per_block,
-    int arg_rw_tail, int arg_items_full, int arg_items_tail, uint32_t arg_full_magic, const uint4 *x2, const uint4 *norm_w, uint4 *x_out,
-    float eps, int log_p)
+    const uint4 *__restrict__ x, int arg_m, int arg_n, int arg_rows_per_block,
+    int arg_rw_tail, int arg_items_tail, uint32_t arg_full_magic, const uint4 *x2, uint16_t *__restrict__ out, const uint4 *norm_w,
+    uint4 *x_out, float eps, int log_p)
 {
-    const MatvecArgs a = {arg_m, arg_n, arg_rows_per_block, arg_rw_tail, arg_items_full, arg_items_tail, arg_full_magic};
+    const MatvecArgs a = {arg_m, arg_n, arg_rows_per_block, arg_rw_tail, arg_rows_per_block >> 1, arg_items_tail, arg_full_magic};
     matvec_body<S, MODE, 2, XMODE, COMPACT>(comp, codebook, x, out, a, XFuse{x2, norm_w, x_out, eps, log_p, nullptr, nullptr, nullptr, nullptr});
 }
 
@@ -664,11 +665,11 @@ __global__ __launch_bounds__(kMatvecThreads) void matvec_fused_kernel(
 template <int S, int MODE, int XMODE>
 __global__ __launch_bounds__(kMatvecThreads) void matvec_affine_kernel(
     const uint32_t *__restrict__ comp, const uint32_t *__restrict__ codebook,
-    const uint4 *__restrict__ x, uint16_t *__restrict__ out, int arg_m, int arg_n, int arg_rows_per_block,
-    int arg_rw_tail, int arg_items_full, int arg_items_tail, uint32_t arg_full_magic, const uint4 *x2, const uint4 *norm_w, uint4 *x_out,
-    float eps, const uint4 *s_in, const uint4 *b_in, const uint16_t *s_out, const uint16_t *b_out)
+    const uint4 *__restrict__ x, int arg_m, int arg_n, int arg_rows_per_block,
+    int arg_rw_tail, int arg_items_tail, uint32_t arg_full_magic, const uint4 *x2, uint16_t *__restrict__ out, const uint4 *norm_w,
+    uint4 *x_out, float eps, const uint4 *s_in, const uint4 *b_in, const uint16_t *s_out, const uint16_t *b_out)
 {
-    const MatvecArgs a = {arg_m, arg_n, arg_rows_per_block, arg_rw_tail, arg_items_full, arg_items_tail, arg_full_magic};
+    const MatvecArgs a = {arg_m, arg_n, arg_rows_per_block, arg_rw_tail, arg_rows_per_block >> 1, arg_items_tail, arg_full_magic};
     matvec_body<S, MODE, 2, XMODE, false, true>(comp, codebook, x, out, a, XFuse{x2, norm_w, x_out, eps, 0, s_in, b_in, s_out, b_out});
 }
 
@@ -771,7 +772,7 @@ static int launch_matvec(const int32_t *compressed, const uint16_t *codebook, co
     auto a_x = reinterpret_cast<const uint4 *>(x);
 #define RPTC_LAUNCH(MODE, COMPACT)                                                                              \
     hipLaunchKernelGGL((matvec_kernel<S, MODE, BITS, COMPACT>), dim3(grid), dim3(kMatvecThreads), lds_bytes, s, \
-                       a_comp, a_cb, a_x, out, a.m, a.n, a.rows_per_block, a.rw_tail, a.items_full, a.items_tail, a.full_magic)
+                       a_comp, a_cb, a_x, a.m, a.n, a.rows_per_block, a.rw_tail, a.items_tail, a.full_magic, out)
     if constexpr (BITS == 2) {
         if (compact) {
             if (carry_mode == RPTC_AS_WRITTEN) RPTC_LAUNCH(RPTC_AS_WRITTEN, true);
@@ -812,8 +813,8 @@ static int launch_matvec_fused(const int32_t *compressed, const uint16_t *codebo
     auto a_xo = reinterpret_cast<uint4 *>(x_out);
 #define RPTC_LAUNCH(MODE, COMPACT)                                                                                  \
     hipLaunchKernelGGL((matvec_fused_kernel<S, MODE, XMODE, COMPACT>), dim3(grid), dim3(kMatvecThreads), lds_bytes, \
-                       s, a_comp, a_cb, a_x, out, a.m, a.n, a.rows_per_block, a.rw_tail, a.items_full, a.items_tail, a.full_magic, \
-                       a_x2, a_w, a_xo, eps, log_p)
+                       s, a_comp, a_cb, a_x, a.m, a.n, a.rows_per_block, a.rw_tail, a.items_tail, a.full_magic, a_x2, out, \
+                       a_w, a_xo, eps, log_p)
     if constexpr (XMODE == kXSiluMul) {
         if (compact) {
             if (carry_mode == RPTC_AS_WRITTEN) RPTC_LAUNCH(RPTC_AS_WRITTEN, true);
@@ -859,8 +860,8 @@ static int launch_matvec_affine(const int32_t *compressed, const uint16_t *codeb
     auto a_bi = reinterpret_cast<const uint4 *>(b_in);
 #define RPTC_LAUNCH(MODE)                                                                                      \
     hipLaunchKernelGGL((matvec_affine_kernel<S, MODE, XMODE>), dim3(grid), dim3(kMatvecThreads), lds_bytes, s, \
-                       a_comp, a_cb, a_x, out, a.m, a.n, a.rows_per_block, a.rw_tail, a.items_full, a.items_tail, \
-                       a.full_magic, a_x2, a_w, a_xo, eps, a_si, a_bi, s_out, b_out)
+                       a_comp, a_cb, a_x, a.m, a.n, a.rows_per_block, a.rw_tail, a.items_tail, a.full_magic, a_x2, out, \
+                       a_w, a_xo, eps, a_si, a_bi, s_out, b_out)
     if (carry_mode == RPTC_AS_WRITTEN) RPTC_LAUNCH(RPTC_AS_WRITTEN);
     else RPTC_LAUNCH(RPTC_CONTINUOUS);
 #undef RPTC_LAUNCH
