@@ -118,11 +118,13 @@ constexpr int kAttnPartStride = 256 + 2;       // acc[hd <= 256], m, l
 static __device__ __align__(256) float g_attn_part[kAttnMaxParts * kAttnPartStride];
 static __device__ __align__(256) uint32_t g_attn_arrived[kAttnMaxHeads];
 
+// (arguments in the order of their first use: the first 14 dwords arrive preloaded in SGPRs)
 template <bool ROPE>
 __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(
-    const uint16_t *__restrict__ q, uint16_t *k_cache, uint16_t *v_cache, const uint16_t *__restrict__ cos_t,
-    const uint16_t *__restrict__ sin_t, const int64_t *__restrict__ pos_p, uint16_t *__restrict__ out,
-    float *__restrict__ parts, uint32_t *__restrict__ arrived, int heads, int hd, int max_len, int splits)
+    const int64_t *__restrict__ pos_p, const uint16_t *__restrict__ q, uint16_t *k_cache, uint16_t *v_cache,
+    int heads, int hd, int max_len, int splits, const uint16_t *__restrict__ cos_t,
+    const uint16_t *__restrict__ sin_t, uint16_t *__restrict__ out, float *__restrict__ parts,
+    uint32_t *__restrict__ arrived)
 {
     extern __shared__ float lds_f[];
     RPTC_ATTN_STAMP(0);
@@ -422,8 +424,8 @@ static int launch_attn(const uint16_t *q, const uint16_t *cos_t, const uint16_t 
     const size_t lds = (size_t)(16 + 2048) * 4 + (size_t)hd * 6;
     const AttnScratch &sc = g_attn[dev->device];
     hipLaunchKernelGGL(attn_decode_kernel<ROPE>, dim3((unsigned)(heads * splits)), dim3(kAttnThreads), lds,
-                       static_cast<hipStream_t>(stream), q, k_cache, v_cache, cos_t, sin_t, pos, out, sc.parts, sc.arrived,
-                       (int)heads, (int)hd, (int)max_len, splits);
+                       static_cast<hipStream_t>(stream), pos, q, k_cache, v_cache, (int)heads, (int)hd, (int)max_len, splits,
+                       cos_t, sin_t, out, sc.parts, sc.arrived);
     return (int)hipGetLastError();
 }
 }  // namespace rptc

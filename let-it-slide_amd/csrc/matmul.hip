@@ -119,11 +119,12 @@ __device__ constexpr int mm_k_of_step_block(int sb)
 // v_alignbit_b32); at 3 and 4 an element is 2 * BITS words, a step advances 2 * BITS stream bits, and
 // the four windows of an MFMA's A operand are cut out one by one.
 // four waves per SIMD = two workgroups per CU: at most 128 vector registers
+// (arguments in the order of their first use: the first 14 dwords arrive preloaded in SGPRs)
 template <int S, int MODE, int PLANES, int BITS>
 __global__ __launch_bounds__(kMmThreads) __attribute__((amdgpu_waves_per_eu(4, 4))) void matmul_kernel(
     const uint32_t *__restrict__ comp32, const uint32_t *__restrict__ codebook, const uint32_t *__restrict__ xp32,
-    float *__restrict__ partial, uint32_t *__restrict__ arrived, uint16_t *__restrict__ out, int m, int n, int batch,
-    int max_rb, int rb_quot, int rb_rem, int group_base)
+    int m, int n, int rb_quot, int rb_rem, int group_base, int max_rb, float *__restrict__ partial,
+    uint32_t *__restrict__ arrived, uint16_t *__restrict__ out, int batch)
 {
     extern __shared__ uint32_t lds[];
     // 64 KiB of table + 16 KiB of tiles: two workgroups share a CU's 160 KiB whatever the batch
@@ -429,12 +430,12 @@ static void launch_matmul(const uint32_t *comp, const uint32_t *cb, const MmScra
         const int g_n = groups - g0 < per_launch ? groups - g0 : (int)per_launch;
         if (carry_mode == RPTC_AS_WRITTEN)
             hipLaunchKernelGGL((matmul_kernel<S, RPTC_AS_WRITTEN, PLANES, BITS>), dim3(g_n * slabs), dim3(kMmThreads),
-                               lds_bytes, s, comp, cb, sc.xpack, sc.partial, sc.arrived, out, m, n, batch, max_rb,
-                               total / groups, total % groups, g0);
+                               lds_bytes, s, comp, cb, sc.xpack, m, n, total / groups, total % groups, g0, max_rb,
+                               sc.partial, sc.arrived, out, batch);
         else
             hipLaunchKernelGGL((matmul_kernel<S, RPTC_CONTINUOUS, PLANES, BITS>), dim3(g_n * slabs), dim3(kMmThreads),
-                               lds_bytes, s, comp, cb, sc.xpack, sc.partial, sc.arrived, out, m, n, batch, max_rb,
-                               total / groups, total % groups, g0);
+                               lds_bytes, s, comp, cb, sc.xpack, m, n, total / groups, total % groups, g0, max_rb,
+                               sc.partial, sc.arrived, out, batch);
     }
 }
 

@@ -39,10 +39,11 @@ __device__ __forceinline__ uint32_t warm_state(const uint4 e, int mode)
     return c;
 }
 
+// Arguments in the order of their first use: the first 14 dwords arrive preloaded in SGPRs.
 template <int L, int MODE>
 __global__ __launch_bounds__(kTThreads) void matvec_t_kernel(
     const uint4 *__restrict__ comp, const uint4 *__restrict__ codebook, const uint32_t *__restrict__ x,
-    uint16_t *__restrict__ out, float *__restrict__ parts, uint32_t *__restrict__ arrived, int m, int cols, int ksplit)
+    int m, int cols, int ksplit, uint16_t *__restrict__ out, float *__restrict__ parts, uint32_t *__restrict__ arrived)
 {
     extern __shared__ uint4 lds_u4[];
     constexpr int lut_u4 = (2 << L) / 16;
@@ -222,10 +223,10 @@ static int launch_matvec_t(const int32_t *compressed, const uint16_t *codebook, 
     auto a_x = reinterpret_cast<const uint32_t *>(x);
     if (carry_mode == RPTC_AS_WRITTEN)
         hipLaunchKernelGGL((matvec_t_kernel<L, RPTC_AS_WRITTEN>), dim3(row_blocks * ksplit), dim3(kTThreads),
-                           lds_bytes_t<L>(), s, a_comp, a_cb, a_x, out, sc.parts, sc.arrived, (int)m, cols, ksplit);
+                           lds_bytes_t<L>(), s, a_comp, a_cb, a_x, (int)m, cols, ksplit, out, sc.parts, sc.arrived);
     else
         hipLaunchKernelGGL((matvec_t_kernel<L, RPTC_CONTINUOUS>), dim3(row_blocks * ksplit), dim3(kTThreads),
-                           lds_bytes_t<L>(), s, a_comp, a_cb, a_x, out, sc.parts, sc.arrived, (int)m, cols, ksplit);
+                           lds_bytes_t<L>(), s, a_comp, a_cb, a_x, (int)m, cols, ksplit, out, sc.parts, sc.arrived);
     return t.end();
 }
 
