@@ -148,18 +148,21 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(
     const int sub = tid % lanes_per_key, slot = tid / lanes_per_key, slots = kAttnThreads / lanes_per_key;
     constexpr int kKeysInFlight = 8;
     uint4 kv[kKeysInFlight], vv[kKeysInFlight];
+    // Requests without a condition (a slot past the piece repeats the last position of the context: a row
+    // that exists, and what it returns is masked out below): requests under a condition cannot be counted,
+    // and the rotation of q would then wait for every key and value instead of for its own five loads.
     auto load_keys = [&](int s0) {
 #pragma unroll
         for (int u = 0; u < kKeysInFlight; u++) {
-            const int s = s0 + u * slots + slot;
-            kv[u] = s < cnt ? *reinterpret_cast<const uint4 *>(kh + (size_t)(s_begin + s) * hd + 8 * sub) : make_uint4(0, 0, 0, 0);
+            const int row = min(s_begin + s0 + u * slots + slot, len - 1);
+            kv[u] = *reinterpret_cast<const uint4 *>(kh + (size_t)row * hd + 8 * sub);
         }
     };
     auto load_values = [&](int s0) {                  // same shape as the keys: 16 bytes of a row per lane
 #pragma unroll
         for (int u = 0; u < kKeysInFlight; u++) {
-            const int s = s0 + u * slots + slot;
-            vv[u] = s < cnt ? *reinterpret_cast<const uint4 *>(vh + (size_t)(s_begin + s) * hd + 8 * sub) : make_uint4(0, 0, 0, 0);
+            const int row = min(s_begin + s0 + u * slots + slot, len - 1);
+            vv[u] = *reinterpret_cast<const uint4 *>(vh + (size_t)row * hd + 8 * sub);
         }
     };
     uint16_t *k_new = q_rot + hd, *v_new = k_new + hd;            // the new row, ROPE only
@@ -167,10 +170,12 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(
         const int half = hd >> 1, d = heads * hd;
         float qa = 0.f, qb = 0.f, ka = 0.f, kb = 0.f, c = 0.f, sn = 0.f;
         uint16_t va = 0, vb = 0;
-        const int e = h * hd + 2 * tid;
         if (tid < half) {
-            c = half_bits_to_float(cos_t[pos * half + tid]);
-            sn = half_bits_to_float(sin_t[pos * half + tid]);
+            // (under a condition, and in front of the keys and values: a block the compiler does not move
+            // loads out of, so these come back first)
+            const int tp = tid, e = h * hd + 2 * tp;
+            c = half_bits_to_float(cos_t[pos * half + tp]);
+            sn = half_bits_to_float(sin_t[pos * half + tp]);
             qa = half_bits_to_float(q[e]);
             qb = half_bits_to_float(q[e + 1]);
             ka = half_bits_to_float(q[d + e]);
@@ -178,19 +183,26 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(
             va = q[2 * d + e];
             vb = q[2 * d + e + 1];
         }
+        // those few loads come back first, and the rotation runs while the keys and values are on their way
         load_keys(0);
         load_values(0);
+        // both rotations in every thread (so that none of the loads above moves under the condition below)
+        uint16_t qra, qrb, kra, krb;
+        rope_pair(qa, qb, c, sn, qra, qrb);
+        rope_pair(ka, kb, c, sn, kra, krb);
         if (tid < half) {
-            rope_pair(qa, qb, c, sn, q_rot[2 * tid], q_rot[2 * tid + 1]);
+            q_rot[2 * tid] = qra;
+            q_rot[2 * tid + 1] = qrb;
             if (owns_pos) {
                 // the row goes to the caches for later tokens; this launch takes it from LDS, because
                 // the loads above may have fetched the row before it was written
-                rope_pair(ka, kb, c, sn, k_new[2 * tid], k_new[2 * tid + 1]);
+                k_new[2 * tid] = kra;
+                k_new[2 * tid + 1] = krb;
                 v_new[2 * tid] = va;
                 v_new[2 * tid + 1] = vb;
                 uint16_t *kd = kh + (size_t)pos * hd + 2 * tid, *vd = vh + (size_t)pos * hd + 2 * tid;
-                kd[0] = k_new[2 * tid];
-                kd[1] = k_new[2 * tid + 1];
+                kd[0] = kra;
+                kd[1] = krb;
                 vd[0] = va;
                 vd[1] = vb;
             }
