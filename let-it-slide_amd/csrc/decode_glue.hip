@@ -269,7 +269,10 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(
             if (owns_pos && s_begin + s == pos) vq = *reinterpret_cast<const uint4 *>(v_new + 8 * sub);
             const float p = sc[u] == -INFINITY ? 0.f : __expf(sc[u] - m_g);
             l_g += p;
-            const uint32_t w[4] = {vq.x, vq.y, vq.z, vq.w};
+            // a slot past the piece holds whatever the repeated row held (possibly not a number): cleared,
+            // since 0 * NaN is not 0
+            const uint32_t live = s < cnt ? 0xFFFFFFFFu : 0u;
+            const uint32_t w[4] = {vq.x & live, vq.y & live, vq.z & live, vq.w & live};
 #pragma unroll
             for (int c = 0; c < 4; c++) {
                 a8[2 * c] += p * half_bits_to_float((uint16_t)(w[c] & 0xFFFFu));

@@ -533,6 +533,10 @@ def test_rope_attn_decode_equals_rope_then_attention(rk, heads, hd, max_len, pos
     qkv = torch.randn(3 * d, generator=g).half().cuda()
     kc = torch.randn((heads, max_len, hd), generator=g).half().cuda()
     vc = torch.randn((heads, max_len, hd), generator=g).half().cuda()
+    # positions the context has not reached hold whatever an allocator left there: not-a-numbers here,
+    # which must not leak into the result (the kernels may read such rows, and mask them)
+    kc[:, pos:] = float("nan")
+    vc[:, pos:] = float("nan")
     ang = torch.arange(max_len).float()[:, None] / (10000.0 ** (torch.arange(0, hd, 2).float() / hd))[None, :]
     cos, sin = ang.cos().half().cuda().contiguous(), ang.sin().half().cuda().contiguous()
     p = torch.tensor([pos], dtype=torch.long, device="cuda")
@@ -549,6 +553,7 @@ def test_rope_attn_decode_equals_rope_then_attention(rk, heads, hd, max_len, pos
     torch.cuda.synchronize()
     assert torch.equal(k1.view(torch.int16), k2.view(torch.int16)) and torch.equal(v1.view(torch.int16), v2.view(torch.int16))
     assert torch.equal(o1.view(torch.int16), o2.view(torch.int16))
+    assert torch.isfinite(o2.float()).all()
     # and against the definition in float64
     kk, vv = k1[:, :pos + 1].double(), v1[:, :pos + 1].double()
     sc = torch.einsum("hd,hsd->hs", q.view(heads, hd).double(), kk) / hd ** 0.5
