@@ -179,6 +179,10 @@ int rptc_sign_hadamard(const uint16_t *x, const uint16_t *signs, uint16_t *out, 
  *   rptc_attn_decode  out[h] = softmax(q[h] . K[h]^T / sqrt(hd)) V[h] over cache positions 0..*pos
  *   rptc_silu_mul     gate_up = [gate|up], each f: out = silu(gate) * up
  *   rptc_rope_attn_decode  rptc_rope_cache followed by rptc_attn_decode in one launch (q stays on chip)
+ *   rptc_greedy_next  greedy hand-over to the next token: *token = argmax(logits[0..vocab)) (first of equal
+ *                     maxima), out_list[*out_index] = *token, x[0..d) = embed[*token][0..d), then
+ *                     *out_index += 1 and *pos += 1; all pointers are device memory (the caller makes
+ *                     out_list long enough), so a captured graph needs nothing from the host per token
  */
 int rptc_add_rmsnorm(const uint16_t *x_in, const uint16_t *delta, const uint16_t *weight, uint16_t *x_out,
                      uint16_t *h_out, int64_t d, float eps, void *stream);
@@ -188,6 +192,8 @@ int rptc_rope_cache(const uint16_t *qkv, const uint16_t *cos_t, const uint16_t *
 int rptc_attn_decode(const uint16_t *q, const uint16_t *k_cache, const uint16_t *v_cache, const int64_t *pos,
                      uint16_t *out, int64_t heads, int64_t hd, int64_t max_len, void *stream);
 int rptc_silu_mul(const uint16_t *gate_up, uint16_t *out, int64_t f, void *stream);
+int rptc_greedy_next(const uint16_t *logits, int64_t vocab, const uint16_t *embed, int64_t d, int64_t *token,
+                     int64_t *out_list, int64_t *out_index, int64_t *pos, uint16_t *x, void *stream);
 int rptc_rope_attn_decode(const uint16_t *qkv, const uint16_t *cos_t, const uint16_t *sin_t, const int64_t *pos,
                           uint16_t *k_cache, uint16_t *v_cache, uint16_t *out, int64_t heads, int64_t hd,
                           int64_t max_len, void *stream);

@@ -379,9 +379,74 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const uint16_t *__restric
     out[i] = silu_mul_bits(gu[i], gu[f + i]);
 }
 
+// Greedy hand-over from one token to the next in one launch: the arg-max of the logits (the first of
+// equal maxima, as the framework's argmax), appended to the output list, becomes the next input token,
+// whose embedding row is copied to the decoder's input; the position and the output index move on.
+// One workgroup: the vocabulary is scanned once, 16 bytes a thread and step.
+constexpr int kGreedyThreads = 1024;
+
+__global__ __launch_bounds__(kGreedyThreads) void greedy_next_kernel(
+    const uint16_t *__restrict__ logits, int vocab, const uint16_t *__restrict__ embed, int d, int64_t *token,
+    int64_t *out_list, int64_t *out_index, int64_t *pos, uint16_t *__restrict__ x)
+{
+    __shared__ float s_val[kGreedyThreads / 64];
+    __shared__ int s_idx[kGreedyThreads / 64];
+    __shared__ int s_best;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    float best = -INFINITY;
+    int best_i = 0x7FFFFFFF;
+    for (int i = tid; i < vocab; i += kGreedyThreads) {
+        const float v = half_bits_to_float(logits[i]);
+        if (v > best) {                        // indices rise along a thread's scan: the first maximum stays
+            best = v;
+            best_i = i;
+        }
+    }
+    // the larger value wins, the smaller index among equal values
+    for (int off = 1; off < 64; off <<= 1) {
+        const float ov = __shfl_xor(best, off, 64);
+        const int oi = __shfl_xor(best_i, off, 64);
+        if (ov > best || (ov == best && oi < best_i)) {
+            best = ov;
+            best_i = oi;
+        }
+    }
+    if (lane == 0) {
+        s_val[wave] = best;
+        s_idx[wave] = best_i;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        for (int w = 1; w < kGreedyThreads / 64; w++)
+            if (s_val[w] > best || (s_val[w] == best && s_idx[w] < best_i)) {
+                best = s_val[w];
+                best_i = s_idx[w];
+            }
+        if (best_i >= vocab) best_i = 0;       // no logit compared greater than -inf (all not-a-numbers)
+        s_best = best_i;
+        *token = best_i;
+        out_list[*out_index] = best_i;
+        *out_index += 1;
+        *pos += 1;
+    }
+    __syncthreads();
+    const uint16_t *row = embed + (size_t)s_best * d;
+    for (int i = tid; i < d; i += kGreedyThreads) x[i] = row[i];
+}
+
 }  // namespace rptc
 
 using namespace rptc;
+
+extern "C" int rptc_greedy_next(const uint16_t *logits, int64_t vocab, const uint16_t *embed, int64_t d, int64_t *token,
+                                int64_t *out_list, int64_t *out_index, int64_t *pos, uint16_t *x, void *stream)
+{
+    if (!logits || !embed || !token || !out_list || !out_index || !pos || !x) return RPTC_ENULL;
+    if (vocab < 1 || vocab >= ((int64_t)1 << 31) || d < 1 || d > (1 << 20)) return RPTC_ESHAPE;
+    hipLaunchKernelGGL(greedy_next_kernel, dim3(1), dim3(kGreedyThreads), 0, static_cast<hipStream_t>(stream), logits,
+                       (int)vocab, embed, (int)d, token, out_list, out_index, pos, x);
+    return (int)hipGetLastError();
+}
 
 extern "C" int rptc_add_rmsnorm(const uint16_t *x_in, const uint16_t *delta, const uint16_t *weight, uint16_t *x_out,
                                 uint16_t *h_out, int64_t d, float eps, void *stream)

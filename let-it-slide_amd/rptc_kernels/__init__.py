@@ -78,6 +78,7 @@ _SIGNATURES = {
     "rptc_rope_cache": ([_VP, _VP, _VP, _VP, _VP, _VP, _VP, _I64, _I64, _I64, _VP], _INT),
     "rptc_attn_decode": ([_VP, _VP, _VP, _VP, _VP, _I64, _I64, _I64, _VP], _INT),
     "rptc_silu_mul": ([_VP, _VP, _I64, _VP], _INT),
+    "rptc_greedy_next": ([_VP, _I64, _VP, _I64, _VP, _VP, _VP, _VP, _VP, _VP], _INT),
     "rptc_probe_empty": ([_VP], _INT),
     "rptc_probe_read": ([_VP, _I64, _VP, _VP], _INT),
     "rptc_rope_attn_decode": ([_VP, _VP, _VP, _VP, _VP, _VP, _VP, _I64, _I64, _I64, _VP], _INT),

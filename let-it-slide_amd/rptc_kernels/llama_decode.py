@@ -116,9 +116,11 @@ class QuantizedLlama(torch.nn.Module):
 
     # ---------------------------------------------------------------- fused one-token path
 
-    def decode_step(self, token, pos, fuse=True):
+    def decode_step(self, token, pos, fuse=True, half_logits=False, input_ready=False):
         """token [1] long, pos [1] long, both on the device (read by the kernels, so a captured graph can be
-        replayed with new values).  Returns the logits [1, vocab] (float).
+        replayed with new values).  Returns the logits [1, vocab] (float; fp16 as the lm_head product leaves
+        them with ``half_logits``).  ``input_ready``: the token's embedding row is already in the decoder's
+        input buffer (``rptc_greedy_next`` put it there), so it is not gathered again.
 
         ``fuse`` (default): five launches per layer - the qkv and gate/up projections do the residual add and
         RMS norm in their prologue, the down projection the SiLU gate, and one kernel rotates q and k, appends
@@ -181,7 +183,8 @@ class QuantizedLlama(torch.nn.Module):
                                                out.data_ptr(), layer.out_features, layer.in_features, layer.S,
                                                layer.carry_mode, stream, None))
 
-        self._x.copy_(self.embed[token].reshape(-1))
+        if not input_ready:
+            self._x.copy_(self.embed[token].reshape(-1))
         delta = None
         if fuse:
             xa, xb = self._x, self._x2          # the residual stream alternates between two buffers
@@ -196,7 +199,8 @@ class QuantizedLlama(torch.nn.Module):
                 delta = self._down.data_ptr()
             ok(lib.rptc_add_rmsnorm(xa.data_ptr(), delta, self.final_norm.data_ptr(), xb.data_ptr(), self._h.data_ptr(), d,
                                     self.EPS, stream))
-            return (self._h.unsqueeze(0) @ self.lm_head.t()).float()
+            logits = self._h.unsqueeze(0) @ self.lm_head.t()
+            return logits if half_logits else logits.float()
         for i, blk in enumerate(self.blocks):
             ok(lib.rptc_add_rmsnorm(self._x.data_ptr(), delta, blk.norm1.data_ptr(), self._x.data_ptr(),
                                     self._h.data_ptr(), d, self.EPS, stream))
@@ -215,7 +219,8 @@ class QuantizedLlama(torch.nn.Module):
             delta = self._down.data_ptr()
         ok(lib.rptc_add_rmsnorm(self._x.data_ptr(), delta, self.final_norm.data_ptr(), self._x.data_ptr(),
                                 self._h.data_ptr(), d, self.EPS, stream))
-        return (self._h.unsqueeze(0) @ self.lm_head.t()).float()
+        logits = self._h.unsqueeze(0) @ self.lm_head.t()
+        return logits if half_logits else logits.float()
 
 
 def greedy_decode(model, prompt, new_tokens, mode="fused_graph"):
@@ -255,12 +260,24 @@ def greedy_decode(model, prompt, new_tokens, mode="fused_graph"):
             s_idx = torch.zeros(1, dtype=torch.long, device=dev)
             s_out = torch.zeros(max(new_tokens - 1, 1), dtype=torch.long, device=dev)
             graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
-                s_next = step(s_tok, s_pos).argmax(-1)
-                s_out.index_copy_(0, s_idx, s_next)
-                s_tok.copy_(s_next)
-                s_pos.add_(1)
-                s_idx.add_(1)
+            if mode.startswith("fused"):
+                # the hand-over is one kernel of the library: arg-max, output list, next embedding row, counters
+                lib = rk.library()
+                model._x.copy_(model.embed[s_tok].reshape(-1))
+                with torch.cuda.graph(graph):
+                    logits16 = model.decode_step(s_tok, s_pos, half_logits=True, input_ready=True)
+                    rc = lib.rptc_greedy_next(logits16.data_ptr(), model.shape.vocab, model.embed.data_ptr(), model.shape.d_model,
+                                              s_tok.data_ptr(), s_out.data_ptr(), s_idx.data_ptr(), s_pos.data_ptr(),
+                                              model._x.data_ptr(), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+                    if rc:
+                        raise RuntimeError(lib.rptc_status_string(rc).decode())
+            else:
+                with torch.cuda.graph(graph):
+                    s_next = step(s_tok, s_pos).argmax(-1)
+                    s_out.index_copy_(0, s_idx, s_next)
+                    s_tok.copy_(s_next)
+                    s_pos.add_(1)
+                    s_idx.add_(1)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         if graph is not None:

@@ -84,6 +84,8 @@ def test_c_abi_rejects_bad_arguments_before_touching_a_device():
     assert lib.rptc_decompress_matvec_affine(16, 16, 32, None, None, None, None, 64, 32, 2048, 7, 0, None, None) == -2   # S
     assert lib.rptc_decompress_matvec_silu_affine(16, 16, None, None, None, None, None, 64, 32, 2048, 8, 0, None, None) == -1
     assert lib.rptc_decompress_matvec_rmsnorm_affine(16, 16, 32, None, 48, 32, None, None, None, None, 64, 32, 2048, 1e-5, 8, 0, None, None) == -7
+    assert lib.rptc_greedy_next(16, 0, 16, 64, 16, 16, 16, 16, 16, None) == -2                   # empty vocabulary
+    assert lib.rptc_greedy_next(16, 1000, None, 64, 16, 16, 16, 16, 16, None) == -1
     assert lib.rptc_sign_hadamard(16, 16, 16, 1, 4096, 48, 0, None, None) == -2                  # block not a power of two
     assert lib.rptc_decompress_matvec_hadamard(16, 16, 16, 16, 16, 32, 4096, 48, 8, 0, None, None) == -2   # block
     assert lib.rptc_decompress_matvec_hadamard(16, 16, 16, 16, 16, 32, 16384, 0, 8, 0, None, None) == -5   # n > 15360

@@ -294,6 +294,35 @@ def test_llama_built_from_dense_weights_through_the_reference_procedure(rk):
     assert rel_l2(lf.cpu().numpy(), ld.cpu().numpy()) < 2e-2
 
 
+@pytest.mark.parametrize("vocab,d", [(32000, 4096), (1000, 256), (5, 64), (70001, 128)])
+def test_greedy_next_is_argmax_plus_bookkeeping(rk, vocab, d):
+    import ctypes
+    lib = rk.library()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    g = torch.Generator().manual_seed(vocab)
+    embed = torch.randn((vocab, d), generator=g).half().cuda()
+    out_list = torch.full((8,), -1, dtype=torch.long, device="cuda")
+    idx = torch.tensor([2], dtype=torch.long, device="cuda")
+    pos = torch.tensor([40], dtype=torch.long, device="cuda")
+    tok = torch.tensor([7], dtype=torch.long, device="cuda")
+    x = torch.zeros(d, dtype=torch.float16, device="cuda")
+    for case in range(3):
+        logits = torch.randn(vocab, generator=g).half().cuda()
+        if case == 1:                               # equal maxima: the first one wins, as torch.argmax
+            top = logits.max()
+            logits[vocab // 2] = top
+            logits[vocab - 1] = top
+        if case == 2:
+            logits[:] = 0.0                         # all equal: index 0
+        want = int(logits.argmax())
+        assert lib.rptc_greedy_next(logits.data_ptr(), vocab, embed.data_ptr(), d, tok.data_ptr(), out_list.data_ptr(),
+                                    idx.data_ptr(), pos.data_ptr(), x.data_ptr(), stream) == 0
+        torch.cuda.synchronize()
+        assert int(tok) == want and int(out_list[2 + case]) == want
+        assert int(idx) == 3 + case and int(pos) == 41 + case
+        assert torch.equal(x.view(torch.int16), embed[want].view(torch.int16))
+
+
 # ------------------------------------------------------------------ projections with a fused element-wise prologue
 
 def _stream(m, n, S=8, seed=0):
