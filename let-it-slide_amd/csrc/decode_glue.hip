@@ -395,13 +395,33 @@ __global__ __launch_bounds__(kGreedyThreads) void greedy_next_kernel(
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     float best = -INFINITY;
     int best_i = 0x7FFFFFFF;
-    for (int i = tid; i < vocab; i += kGreedyThreads) {
-        const float v = half_bits_to_float(logits[i]);
-        if (v > best) {                        // indices rise along a thread's scan: the first maximum stays
+    auto take = [&](float v, int i) {          // indices rise along a thread's scan: the first maximum stays
+        if (v > best) {
             best = v;
             best_i = i;
         }
+    };
+    // 16 bytes a load, four loads of a thread asked for before the first is looked at
+    const int n8 = vocab >> 3;
+    const uint4 *l4 = reinterpret_cast<const uint4 *>(logits);
+    constexpr int kInFlight = 4;
+    for (int c0 = tid; c0 < n8; c0 += kGreedyThreads * kInFlight) {
+        uint4 v[kInFlight];
+#pragma unroll
+        for (int u = 0; u < kInFlight; u++) v[u] = l4[min(c0 + u * kGreedyThreads, n8 - 1)];
+#pragma unroll
+        for (int u = 0; u < kInFlight; u++) {
+            const int c = c0 + u * kGreedyThreads;
+            if (c >= n8) break;
+            const uint32_t w[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                take(half_bits_to_float((uint16_t)(w[k] & 0xFFFFu)), 8 * c + 2 * k);
+                take(half_bits_to_float((uint16_t)(w[k] >> 16)), 8 * c + 2 * k + 1);
+            }
+        }
     }
+    for (int i = 8 * n8 + tid; i < vocab; i += kGreedyThreads) take(half_bits_to_float(logits[i]), i);
     // the larger value wins, the smaller index among equal values
     for (int off = 1; off < 64; off <<= 1) {
         const float ov = __shfl_xor(best, off, 64);
@@ -431,7 +451,13 @@ __global__ __launch_bounds__(kGreedyThreads) void greedy_next_kernel(
     }
     __syncthreads();
     const uint16_t *row = embed + (size_t)s_best * d;
-    for (int i = tid; i < d; i += kGreedyThreads) x[i] = row[i];
+    if ((d & 7) == 0) {                        // rows are 16-byte aligned when the table is
+        const uint4 *r4 = reinterpret_cast<const uint4 *>(row);
+        uint4 *x4 = reinterpret_cast<uint4 *>(x);
+        for (int i = tid; i < (d >> 3); i += kGreedyThreads) x4[i] = r4[i];
+    } else {
+        for (int i = tid; i < d; i += kGreedyThreads) x[i] = row[i];
+    }
 }
 
 }  // namespace rptc
@@ -443,6 +469,7 @@ extern "C" int rptc_greedy_next(const uint16_t *logits, int64_t vocab, const uin
 {
     if (!logits || !embed || !token || !out_list || !out_index || !pos || !x) return RPTC_ENULL;
     if (vocab < 1 || vocab >= ((int64_t)1 << 31) || d < 1 || d > (1 << 20)) return RPTC_ESHAPE;
+    if (!aligned16(logits) || !aligned16(embed) || !aligned16(x)) return RPTC_EALIGN;
     hipLaunchKernelGGL(greedy_next_kernel, dim3(1), dim3(kGreedyThreads), 0, static_cast<hipStream_t>(stream), logits,
                        (int)vocab, embed, (int)d, token, out_list, out_index, pos, x);
     return (int)hipGetLastError();
