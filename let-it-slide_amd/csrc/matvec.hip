@@ -366,22 +366,19 @@ __device__ __forceinline__ void matvec_body(
     // flight where it needs only the activations, and the staging below (and the element-wise
     // prologues) would start when the stream data has arrived instead of while it is on its way.
     // A lane past the item's rows repeats the last lane's address; a slot past the wave's items
-    // repeats the wave's first item (the first word of the stream for a wave with none).
+    // repeats the first element of the wave's first item (of the stream for a wave with none).
     auto load_first = [&]() {
         const uint32_t *first_base = comp;
-        int first_nact = 1;
 #pragma unroll
         for (int u = 0; u < kBatch; u++) {
             const bool have = it_begin + u < it_end;
             const int row_first = ld_idx * ld.rows_per_item;           // row inside the block
             const int rows_here = min(ld.rows_per_item, rows - row_first);
             const uint32_t *item_base = comp + (size_t)(ld.elem0 + (uint32_t)(row0 + row_first) * (uint32_t)ld.lanes) * WORDS;
-            if (u == 0 && have) {
-                first_base = item_base;
-                first_nact = rows_here * ld.lanes;
-            }
+            if (u == 0 && have) first_base = item_base;
             const uint32_t *wave_base = have ? item_base : first_base;
-            const int nact = have ? rows_here * ld.lanes : first_nact;
+            // a slot the wave has no item for asks for one element in every lane: one cache line, not eight
+            const int nact = have ? rows_here * ld.lanes : 1;
             buf[u] = load_stream<WORDS>(wave_base, min(lane, nact - 1));
             if (MODE == RPTC_CONTINUOUS) {
                 // the word in front of a row: last word of the row's lane 31 in the slab before
