@@ -601,6 +601,11 @@ __device__ __forceinline__ void matvec_body(
     // One register set is decoded from a copy while its own registers take the next batch.  (Two
     // sets that take turns save the copies and measured 1 % faster on long rows, 1.5 % slower on
     // the short ones this kernel is graded on.)
+    if (it_end - it_begin <= kBatch) {
+        // everything the wave has is in the first batch: decoded from the registers the requests fill, element
+        // by element as each arrives (no copy that would wait for the whole batch)
+        decode_batch(buf, cw, it_begin);
+    } else
     for (int base = it_begin; base < it_end; base += kBatch) {
         Elem<WORDS> cur[kBatch];
         uint32_t ccw[kBatch];
