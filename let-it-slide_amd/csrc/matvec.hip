@@ -218,16 +218,18 @@ __device__ __forceinline__ uint4 silu_mul8(const uint4 gate, const uint4 up)
 }
 
 // COMPACT: partial sums per (row, full slab) and (row, ragged lane) instead of per (row, stream element)
-// KB: stream elements a lane has in flight.  Three when no wave of the launch has more than three items (one
-// batch, decoded as it arrives), two otherwise: a batch is decoded when all of it has arrived, and two
-// elements per lane (32 KB per CU) are what the memory latency asks for.
-template <int S, int MODE, int BITS, int XMODE, bool COMPACT, int KB, bool AFFINE = false>
+template <int S, int MODE, int BITS, int XMODE, bool COMPACT, bool AFFINE = false>
 __device__ __forceinline__ void matvec_body(
     const uint32_t *__restrict__ comp, const uint32_t *__restrict__ codebook,
     const uint4 *__restrict__ x, uint16_t *__restrict__ out, const MatvecArgs a, const XFuse fuse)
 {
     constexpr int WORDS = 2 * BITS;                        // words per stream element
-    constexpr int kBatch = KB;                             // stream elements in flight per lane
+    // Stream elements a lane asks for at a time: one, and the next one when that one is about to be decoded.
+    // The sixteen waves of a CU then have 16 KB on their way at the start and 32 KB in steady state, which is
+    // what the memory latency asks for; with two, three or four elements per lane the first data arrives later
+    // (the CU's address unit takes the requests one line at a time) and a batch is decoded only when all of
+    // it has arrived: measured slower on every shape.
+    constexpr int kBatch = 1;
     extern __shared__ uint32_t lds[];
     RPTC_STAMP(0);
     const int m = a.m, n = a.n;
@@ -641,7 +643,7 @@ __device__ __forceinline__ void matvec_body(
     RPTC_STAMP(5);
 }
 
-template <int S, int MODE, int BITS, bool COMPACT, int KB>
+template <int S, int MODE, int BITS, bool COMPACT>
 __global__ __launch_bounds__(kMatvecThreads) void matvec_kernel(
     const uint32_t *__restrict__ comp, const uint32_t *__restrict__ codebook,
     const uint4 *__restrict__ x, int arg_m, int arg_n, int arg_rows_per_block,
@@ -650,11 +652,11 @@ __global__ __launch_bounds__(kMatvecThreads) void matvec_kernel(
     // Separate scalar arguments (not a struct), and what the first requests need in the first 14 dwords:
     // those arrive in SGPRs with the wave, the rest (the output pointer is needed last) through a scalar load.
     const MatvecArgs a = {arg_m, arg_n, arg_rows_per_block, arg_rw_tail, arg_rows_per_block >> 1, arg_items_tail, arg_full_magic};
-    matvec_body<S, MODE, BITS, kXPlain, COMPACT, KB>(comp, codebook, x, out, a, XFuse{nullptr, nullptr, nullptr, 0.f, 0, nullptr, nullptr, nullptr, nullptr});
+    matvec_body<S, MODE, BITS, kXPlain, COMPACT>(comp, codebook, x, out, a, XFuse{nullptr, nullptr, nullptr, 0.f, 0, nullptr, nullptr, nullptr, nullptr});
 }
 
 // 2 bits per weight with an element-wise step fused in front (XMODE above)
-template <int S, int MODE, int XMODE, bool COMPACT, int KB>
+template <int S, int MODE, int XMODE, bool COMPACT>
 __global__ __launch_bounds__(kMatvecThreads) void matvec_fused_kernel(
     const uint32_t *__restrict__ comp, const uint32_t *__restrict__ codebook,
     const uint4 *__restrict__ x, int arg_m, int arg_n, int arg_rows_per_block,
@@ -662,12 +664,12 @@ __global__ __launch_bounds__(kMatvecThreads) void matvec_fused_kernel(
     uint4 *x_out, float eps, int log_p)
 {
     const MatvecArgs a = {arg_m, arg_n, arg_rows_per_block, arg_rw_tail, arg_rows_per_block >> 1, arg_items_tail, arg_full_magic};
-    matvec_body<S, MODE, 2, XMODE, COMPACT, KB>(comp, codebook, x, out, a, XFuse{x2, norm_w, x_out, eps, log_p, nullptr, nullptr, nullptr, nullptr});
+    matvec_body<S, MODE, 2, XMODE, COMPACT>(comp, codebook, x, out, a, XFuse{x2, norm_w, x_out, eps, log_p, nullptr, nullptr, nullptr, nullptr});
 }
 
 // 2 bits per weight with the row/column scales and biases of the reference's factorisation applied in
 // the prologue (input side) and where the row sums are written (output side), after any XMODE step
-template <int S, int MODE, int XMODE, int KB>
+template <int S, int MODE, int XMODE>
 __global__ __launch_bounds__(kMatvecThreads) void matvec_affine_kernel(
     const uint32_t *__restrict__ comp, const uint32_t *__restrict__ codebook,
     const uint4 *__restrict__ x, int arg_m, int arg_n, int arg_rows_per_block,
@@ -675,7 +677,7 @@ __global__ __launch_bounds__(kMatvecThreads) void matvec_affine_kernel(
     uint4 *x_out, float eps, const uint4 *s_in, const uint4 *b_in, const uint16_t *s_out, const uint16_t *b_out)
 {
     const MatvecArgs a = {arg_m, arg_n, arg_rows_per_block, arg_rw_tail, arg_rows_per_block >> 1, arg_items_tail, arg_full_magic};
-    matvec_body<S, MODE, 2, XMODE, false, KB, true>(comp, codebook, x, out, a, XFuse{x2, norm_w, x_out, eps, 0, s_in, b_in, s_out, b_out});
+    matvec_body<S, MODE, 2, XMODE, false, true>(comp, codebook, x, out, a, XFuse{x2, norm_w, x_out, eps, 0, s_in, b_in, s_out, b_out});
 }
 
 // Dense export: one thread per stream element, 32 pairs scattered to their columns.
@@ -758,13 +760,6 @@ static int plan_matvec(const void *compressed, const void *codebook, const void 
     return 0;
 }
 
-// Three elements in flight per lane when the busiest wave of a workgroup has exactly three items, two otherwise.
-static bool matvec_three_in_flight(const MatvecArgs &a)
-{
-    const int total = (a.n >> 11) * a.items_full + a.items_tail;
-    return (total + kMatvecWaves - 1) / kMatvecWaves == 3;
-}
-
 template <int S, int BITS = 2>
 static int launch_matvec(const int32_t *compressed, const uint16_t *codebook, const uint16_t *x,
                          uint16_t *out, int64_t m, int64_t n, int carry_mode, void *stream, float *ms)
@@ -782,19 +777,9 @@ static int launch_matvec(const int32_t *compressed, const uint16_t *codebook, co
     auto a_comp = reinterpret_cast<const uint32_t *>(compressed);
     auto a_cb = reinterpret_cast<const uint32_t *>(codebook);
     auto a_x = reinterpret_cast<const uint4 *>(x);
-    const bool three = BITS == 2 && matvec_three_in_flight(a);
-#define RPTC_LAUNCH_KB(MODE, COMPACT, KB)                                                                           \
-    hipLaunchKernelGGL((matvec_kernel<S, MODE, BITS, COMPACT, KB>), dim3(grid), dim3(kMatvecThreads), lds_bytes, s, \
+#define RPTC_LAUNCH(MODE, COMPACT)                                                                              \
+    hipLaunchKernelGGL((matvec_kernel<S, MODE, BITS, COMPACT>), dim3(grid), dim3(kMatvecThreads), lds_bytes, s, \
                        a_comp, a_cb, a_x, a.m, a.n, a.rows_per_block, a.rw_tail, a.items_tail, a.full_magic, out)
-#define RPTC_LAUNCH(MODE, COMPACT)                                        \
-    do {                                                                  \
-        if constexpr (BITS == 2) {                                        \
-            if (three) RPTC_LAUNCH_KB(MODE, COMPACT, 3);                  \
-            else RPTC_LAUNCH_KB(MODE, COMPACT, 2);                        \
-        } else {                                                          \
-            RPTC_LAUNCH_KB(MODE, COMPACT, 2);                             \
-        }                                                                 \
-    } while (0)
     if constexpr (BITS == 2) {
         if (compact) {
             if (carry_mode == RPTC_AS_WRITTEN) RPTC_LAUNCH(RPTC_AS_WRITTEN, true);
@@ -805,7 +790,6 @@ static int launch_matvec(const int32_t *compressed, const uint16_t *codebook, co
     if (carry_mode == RPTC_AS_WRITTEN) RPTC_LAUNCH(RPTC_AS_WRITTEN, false);
     else RPTC_LAUNCH(RPTC_CONTINUOUS, false);
 #undef RPTC_LAUNCH
-#undef RPTC_LAUNCH_KB
     return t.end();
 }
 
@@ -834,16 +818,10 @@ static int launch_matvec_fused(const int32_t *compressed, const uint16_t *codebo
     auto a_x2 = reinterpret_cast<const uint4 *>(x2);
     auto a_w = reinterpret_cast<const uint4 *>(norm_w);
     auto a_xo = reinterpret_cast<uint4 *>(x_out);
-    const bool three = matvec_three_in_flight(a);
-#define RPTC_LAUNCH_KB(MODE, COMPACT, KB)                                                                               \
-    hipLaunchKernelGGL((matvec_fused_kernel<S, MODE, XMODE, COMPACT, KB>), dim3(grid), dim3(kMatvecThreads), lds_bytes, \
+#define RPTC_LAUNCH(MODE, COMPACT)                                                                                  \
+    hipLaunchKernelGGL((matvec_fused_kernel<S, MODE, XMODE, COMPACT>), dim3(grid), dim3(kMatvecThreads), lds_bytes, \
                        s, a_comp, a_cb, a_x, a.m, a.n, a.rows_per_block, a.rw_tail, a.items_tail, a.full_magic, a_x2, out, \
                        a_w, a_xo, eps, log_p)
-#define RPTC_LAUNCH(MODE, COMPACT)                        \
-    do {                                                  \
-        if (three) RPTC_LAUNCH_KB(MODE, COMPACT, 3);      \
-        else RPTC_LAUNCH_KB(MODE, COMPACT, 2);            \
-    } while (0)
     if constexpr (XMODE == kXSiluMul) {
         if (compact) {
             if (carry_mode == RPTC_AS_WRITTEN) RPTC_LAUNCH(RPTC_AS_WRITTEN, true);
@@ -854,7 +832,6 @@ static int launch_matvec_fused(const int32_t *compressed, const uint16_t *codebo
     if (carry_mode == RPTC_AS_WRITTEN) RPTC_LAUNCH(RPTC_AS_WRITTEN, false);
     else RPTC_LAUNCH(RPTC_CONTINUOUS, false);
 #undef RPTC_LAUNCH
-#undef RPTC_LAUNCH_KB
     return t.end();
 }
 
@@ -888,20 +865,13 @@ static int launch_matvec_affine(const int32_t *compressed, const uint16_t *codeb
     auto a_xo = reinterpret_cast<uint4 *>(x_out);
     auto a_si = reinterpret_cast<const uint4 *>(s_in);
     auto a_bi = reinterpret_cast<const uint4 *>(b_in);
-    const bool three = matvec_three_in_flight(a);
-#define RPTC_LAUNCH_KB(MODE, KB)                                                                                   \
-    hipLaunchKernelGGL((matvec_affine_kernel<S, MODE, XMODE, KB>), dim3(grid), dim3(kMatvecThreads), lds_bytes, s, \
+#define RPTC_LAUNCH(MODE)                                                                                      \
+    hipLaunchKernelGGL((matvec_affine_kernel<S, MODE, XMODE>), dim3(grid), dim3(kMatvecThreads), lds_bytes, s, \
                        a_comp, a_cb, a_x, a.m, a.n, a.rows_per_block, a.rw_tail, a.items_tail, a.full_magic, a_x2, out, \
                        a_w, a_xo, eps, a_si, a_bi, s_out, b_out)
-#define RPTC_LAUNCH(MODE)                        \
-    do {                                         \
-        if (three) RPTC_LAUNCH_KB(MODE, 3);      \
-        else RPTC_LAUNCH_KB(MODE, 2);            \
-    } while (0)
     if (carry_mode == RPTC_AS_WRITTEN) RPTC_LAUNCH(RPTC_AS_WRITTEN);
     else RPTC_LAUNCH(RPTC_CONTINUOUS);
 #undef RPTC_LAUNCH
-#undef RPTC_LAUNCH_KB
     return t.end();
 }
 
@@ -979,43 +949,34 @@ static int set_lds_limit(F *kernel)
 int prepare_matvec()
 {
     int rc;
-#define RPTC_SET_LIMITS(BITS, COMPACT, KB)                                                               \
-    if ((rc = set_lds_limit(matvec_kernel<6, RPTC_AS_WRITTEN, BITS, COMPACT, KB>))) return rc;              \
-    if ((rc = set_lds_limit(matvec_kernel<6, RPTC_CONTINUOUS, BITS, COMPACT, KB>))) return rc;              \
-    if ((rc = set_lds_limit(matvec_kernel<8, RPTC_AS_WRITTEN, BITS, COMPACT, KB>))) return rc;              \
-    if ((rc = set_lds_limit(matvec_kernel<8, RPTC_CONTINUOUS, BITS, COMPACT, KB>))) return rc;
-    RPTC_SET_LIMITS(2, false, 2)
-    RPTC_SET_LIMITS(2, false, 3)
-    RPTC_SET_LIMITS(2, true, 2)
-    RPTC_SET_LIMITS(2, true, 3)
-    RPTC_SET_LIMITS(3, false, 2)
-    RPTC_SET_LIMITS(4, false, 2)
+#define RPTC_SET_LIMITS(BITS, COMPACT)                                                               \
+    if ((rc = set_lds_limit(matvec_kernel<6, RPTC_AS_WRITTEN, BITS, COMPACT>))) return rc;              \
+    if ((rc = set_lds_limit(matvec_kernel<6, RPTC_CONTINUOUS, BITS, COMPACT>))) return rc;              \
+    if ((rc = set_lds_limit(matvec_kernel<8, RPTC_AS_WRITTEN, BITS, COMPACT>))) return rc;              \
+    if ((rc = set_lds_limit(matvec_kernel<8, RPTC_CONTINUOUS, BITS, COMPACT>))) return rc;
+    RPTC_SET_LIMITS(2, false)
+    RPTC_SET_LIMITS(2, true)
+    RPTC_SET_LIMITS(3, false)
+    RPTC_SET_LIMITS(4, false)
 #undef RPTC_SET_LIMITS
-#define RPTC_SET_LIMITS(XMODE, COMPACT, KB)                                                                    \
-    if ((rc = set_lds_limit(matvec_fused_kernel<6, RPTC_AS_WRITTEN, XMODE, COMPACT, KB>))) return rc;             \
-    if ((rc = set_lds_limit(matvec_fused_kernel<6, RPTC_CONTINUOUS, XMODE, COMPACT, KB>))) return rc;             \
-    if ((rc = set_lds_limit(matvec_fused_kernel<8, RPTC_AS_WRITTEN, XMODE, COMPACT, KB>))) return rc;             \
-    if ((rc = set_lds_limit(matvec_fused_kernel<8, RPTC_CONTINUOUS, XMODE, COMPACT, KB>))) return rc;
-    RPTC_SET_LIMITS(kXSiluMul, false, 2)
-    RPTC_SET_LIMITS(kXSiluMul, false, 3)
-    RPTC_SET_LIMITS(kXSiluMul, true, 2)
-    RPTC_SET_LIMITS(kXSiluMul, true, 3)
-    RPTC_SET_LIMITS(kXAddRmsNorm, false, 2)
-    RPTC_SET_LIMITS(kXAddRmsNorm, false, 3)
-    RPTC_SET_LIMITS(kXSignHadamard, false, 2)
-    RPTC_SET_LIMITS(kXSignHadamard, false, 3)
+#define RPTC_SET_LIMITS(XMODE, COMPACT)                                                                    \
+    if ((rc = set_lds_limit(matvec_fused_kernel<6, RPTC_AS_WRITTEN, XMODE, COMPACT>))) return rc;             \
+    if ((rc = set_lds_limit(matvec_fused_kernel<6, RPTC_CONTINUOUS, XMODE, COMPACT>))) return rc;             \
+    if ((rc = set_lds_limit(matvec_fused_kernel<8, RPTC_AS_WRITTEN, XMODE, COMPACT>))) return rc;             \
+    if ((rc = set_lds_limit(matvec_fused_kernel<8, RPTC_CONTINUOUS, XMODE, COMPACT>))) return rc;
+    RPTC_SET_LIMITS(kXSiluMul, false)
+    RPTC_SET_LIMITS(kXSiluMul, true)
+    RPTC_SET_LIMITS(kXAddRmsNorm, false)
+    RPTC_SET_LIMITS(kXSignHadamard, false)
 #undef RPTC_SET_LIMITS
-#define RPTC_SET_LIMITS(XMODE, KB)                                                                     \
-    if ((rc = set_lds_limit(matvec_affine_kernel<6, RPTC_AS_WRITTEN, XMODE, KB>))) return rc;             \
-    if ((rc = set_lds_limit(matvec_affine_kernel<6, RPTC_CONTINUOUS, XMODE, KB>))) return rc;             \
-    if ((rc = set_lds_limit(matvec_affine_kernel<8, RPTC_AS_WRITTEN, XMODE, KB>))) return rc;             \
-    if ((rc = set_lds_limit(matvec_affine_kernel<8, RPTC_CONTINUOUS, XMODE, KB>))) return rc;
-    RPTC_SET_LIMITS(kXPlain, 2)
-    RPTC_SET_LIMITS(kXPlain, 3)
-    RPTC_SET_LIMITS(kXSiluMul, 2)
-    RPTC_SET_LIMITS(kXSiluMul, 3)
-    RPTC_SET_LIMITS(kXAddRmsNorm, 2)
-    RPTC_SET_LIMITS(kXAddRmsNorm, 3)
+#define RPTC_SET_LIMITS(XMODE)                                                                     \
+    if ((rc = set_lds_limit(matvec_affine_kernel<6, RPTC_AS_WRITTEN, XMODE>))) return rc;             \
+    if ((rc = set_lds_limit(matvec_affine_kernel<6, RPTC_CONTINUOUS, XMODE>))) return rc;             \
+    if ((rc = set_lds_limit(matvec_affine_kernel<8, RPTC_AS_WRITTEN, XMODE>))) return rc;             \
+    if ((rc = set_lds_limit(matvec_affine_kernel<8, RPTC_CONTINUOUS, XMODE>))) return rc;
+    RPTC_SET_LIMITS(kXPlain)
+    RPTC_SET_LIMITS(kXSiluMul)
+    RPTC_SET_LIMITS(kXAddRmsNorm)
 #undef RPTC_SET_LIMITS
     return 0;
 }
