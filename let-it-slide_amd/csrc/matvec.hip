@@ -256,16 +256,24 @@ __device__ __forceinline__ void matvec_body(
     // Table rows 16 * wave .. 16 * wave + 15 are this wave's to write.  A row is 64 copies of one
     // value, so the value is wave-uniform and comes through the scalar cache: these loads neither
     // queue with the vector loads nor return in order with them.
+    // The sign bit of a row is bit 7 of the row number, the same for a wave's sixteen rows: it is merged in
+    // by the vector op that moves the value to the register the LDS write takes (v_and_or_b32), so a row
+    // costs one vector op and no scalar one in front of the barrier.
     constexpr int kRowsPerWave = 256 / kMatvecWaves;
     uint32_t cbv[kRowsPerWave];
 #pragma unroll
-    for (int i = 0; i < kRowsPerWave; i++) cbv[i] = table_value<S>(codebook, kRowsPerWave * wave + i);
+    for (int i = 0; i < kRowsPerWave; i++) cbv[i] = codebook[(kRowsPerWave * wave + i) & ((1 << S) - 1)];
+    const uint32_t table_sign = (uint32_t)(wave >> 3) << 15;
     constexpr int kXRegs = 2;
     uint4 xv[kXRegs], xv2[kXRegs], xvw[kXRegs];
 #pragma unroll
     for (int u = 0; u < kXRegs; u++) {
         const int idx = tid + u * kMatvecThreads;
-        xv[u] = idx < n8 ? x[idx] : make_uint4(0, 0, 0, 0);
+        if constexpr (XMODE == kXPlain && !AFFINE) {
+            if (idx < n8) xv[u] = x[idx];               // staged under the same condition: nothing reads the rest
+        } else {
+            xv[u] = idx < n8 ? x[idx] : make_uint4(0, 0, 0, 0);
+        }
     }
     if constexpr (XMODE == kXSiluMul) {
 #pragma unroll
@@ -308,7 +316,7 @@ __device__ __forceinline__ void matvec_body(
     const int total = T * a.items_full + a.items_tail;
     // The first total % 16 waves take one item more.  Waves w, w+4, w+8, w+12 share a SIMD, so
     // this also spreads the remainder evenly over the four SIMDs.
-    const int per_wave = total / kMatvecWaves, extra = total % kMatvecWaves;
+    const int per_wave = (int)((uint32_t)total / kMatvecWaves), extra = (int)((uint32_t)total % kMatvecWaves);
     const int it_begin = wave * per_wave + min(wave, extra);
     const int it_end = it_begin + per_wave + (wave < extra ? 1 : 0);
     auto view = [&](int slab) {
@@ -345,6 +353,13 @@ __device__ __forceinline__ void matvec_body(
 #pragma unroll
         for (int u = 0; u < kBatch; u++) {
             if (base + u < it_end) {
+                // the cursor stands at the item requested last: moving it on here, not behind the request,
+                // keeps that arithmetic out of the instructions in front of the barrier
+                if (++ld_idx == ld.items) {
+                    ld_idx = 0;
+                    ld_slab++;
+                    ld = view(ld_slab);
+                }
                 const int row_first = ld_idx * ld.rows_per_item;           // row inside the block
                 const int rows_here = min(ld.rows_per_item, rows - row_first);
                 if (lane < rows_here * ld.lanes) {
@@ -357,11 +372,6 @@ __device__ __forceinline__ void matvec_body(
                         if (l == 0)
                             cw[u] = comp[(((size_t)(ld_slab - 1) * m + row0 + row_first + sub) * 32 + 31) * WORDS + WORDS - 1];
                     }
-                }
-                if (++ld_idx == ld.items) {
-                    ld_idx = 0;
-                    ld_slab++;
-                    ld = view(ld_slab);
                 }
             }
         }
@@ -380,27 +390,25 @@ __device__ __forceinline__ void matvec_body(
             const int row_first = ld_idx * ld.rows_per_item;           // row inside the block
             const int rows_here = min(ld.rows_per_item, rows - row_first);
             const uint32_t *item_base = comp + (size_t)(ld.elem0 + (uint32_t)(row0 + row_first) * (uint32_t)ld.lanes) * WORDS;
-            if (u == 0 && have) first_base = item_base;
-            const uint32_t *wave_base = have ? item_base : first_base;
-            // a slot the wave has no item for asks for one element in every lane: one cache line, not eight
-            const int nact = have ? rows_here * ld.lanes : 1;
+            if (u == 0 && have && rows_here > 0) first_base = item_base;
+            // a slot the wave has no item for, or whose item lies past the block's last row, asks for one
+            // element in every lane: one cache line, not eight
+            const bool real = have && rows_here > 0;
+            const uint32_t *wave_base = real ? item_base : first_base;
+            const int nact = real ? rows_here * ld.lanes : 1;
             buf[u] = load_stream<WORDS>(wave_base, min(lane, nact - 1));
             if (MODE == RPTC_CONTINUOUS) {
                 // the word in front of a row: last word of the row's lane 31 in the slab before
                 // (read by all lanes of the row; used by its first lane, and only past slab 0)
-                const bool prev = have && ld_slab > 0;
-                const int sub = min(ld_slab < T ? lane >> 5 : lane / ld.lanes, rows_here - 1);
+                const bool prev = real && ld_slab > 0;
+                const int sub = min(ld_slab < T ? lane >> 5 : lane / ld.lanes, max(rows_here, 1) - 1);
                 const uint32_t *row_base =
                     prev ? comp + (((size_t)(ld_slab - 1) * m + row0 + row_first) * 32 + 31) * WORDS + WORDS - 1 : comp;
                 cw[u] = row_base[sub * (prev ? 32 * WORDS : 0)];
             }
-            if (have && ++ld_idx == ld.items) {
-                ld_idx = 0;
-                ld_slab++;
-                ld = view(ld_slab);
-            }
         }
     };
+    static_assert(kBatch == 1, "the load cursor stands at the one item the first request asked for");
     load_first();
     RPTC_STAMP(1);
 
@@ -493,7 +501,11 @@ __device__ __forceinline__ void matvec_body(
 
     // table (256 rows x 64 lane copies) and activation image into LDS
 #pragma unroll
-    for (int i = 0; i < kRowsPerWave; i++) lds[(kRowsPerWave * wave + i) * 64 + lane] = cbv[i];
+    for (int i = 0; i < kRowsPerWave; i++) {
+        uint32_t tv;
+        asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(tv) : "s"(cbv[i]), "v"(0xFFFF7FFFu), "v"(table_sign));
+        lds[(kRowsPerWave * wave + i) * 64 + lane] = tv;
+    }
     auto stage_x = [&](int idx, const uint4 v) {          // halves 8idx .. 8idx+7 (inference.cu:215-221)
         sx[idx] = v.x;
         sx[idx + n8] = v.y;
@@ -545,8 +557,13 @@ __device__ __forceinline__ void matvec_body(
                 // step q of element l multiplies pair slot(slab, q, l) (inference.cu:249)
                 const uint32_t *xp = sx + (slab < T ? 1024 * slab : 1024 * T) + l;
                 if (slab < T) {
+                    // one address and 32 immediate offsets (as inline assembly, or the compiler merges these
+                    // reads with those of the ragged slab and forms 31 addresses with vector adds)
+                    const uint32_t xa = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(xp));
 #pragma unroll
-                    for (int q = 0; q < 32; q++) xr[q] = xp[32 * q];
+                    for (int q = 0; q < 32; q++)
+                        asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(xr[q]) : "v"(xa), "n"(128 * q));
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
                 } else {
 #pragma unroll
                     for (int q = 0; q < 32; q++) xr[q] = xp[q * sv.lanes];
@@ -558,7 +575,7 @@ __device__ __forceinline__ void matvec_body(
             const int row_first = idx * sv.rows_per_item;
             // The lanes whose sum is kept, as a wave-uniform mask: the lanes of the item's rows that
             // exist (the first `nact` lanes), and of those only the ones holding a row's sum.
-            const int nact = min(sv.rows_per_item, rows - row_first) * sv.lanes;
+            const int nact = max(min(sv.rows_per_item, rows - row_first), 0) * sv.lanes;   // 0 for an item past the last row
             uint64_t keep = nact >= 64 ? ~0ull : (1ull << nact) - 1ull;
             // Previous lane's last word.  Lane 0 of a row keeps its own as written
             // (inference.cu:232: the shuffle hands lane 0 its own value back).
