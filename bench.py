@@ -28,7 +28,7 @@ HBM_PEAK_GBS = 8000.0
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a copy kernel
 # of known size; the runs are summarised under profiles/).  Keyed by (m, n, S); other workloads report null.
-MEASURED_TRAFFIC_BYTES = {(4096, 11008, 8): 11598600}
+MEASURED_TRAFFIC_BYTES = {(4096, 11008, 8): 11528200}
 
 
 def parse():
