@@ -33,7 +33,11 @@
 
 namespace rptc {
 
-constexpr int kMatvecThreads = 1024;
+#ifndef RPTC_MATVEC_THREADS
+#define RPTC_MATVEC_THREADS 1024
+#endif
+constexpr int kMatvecThreads = RPTC_MATVEC_THREADS;
+constexpr int kXRegs = 2048 / kMatvecThreads;   // activation registers per thread: vectors of up to 16384 halves
 constexpr int kMatvecWaves = kMatvecThreads / kWave;
 constexpr int kTableBytes = 256 * 256;     // 256 rows of 64 lane copies of one half2
 
@@ -71,7 +75,7 @@ struct Elem {
 };
 
 template <int WORDS>
-__device__ __forceinline__ Elem<WORDS> load_stream(const uint32_t *wave_base, int lane)
+__device__ __forceinline__ Elem<WORDS> load_stream(const uint32_t *wave_base, uint32_t lane)
 {
     typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
     typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
@@ -263,14 +267,13 @@ __device__ __forceinline__ void matvec_body(
     uint32_t cbv[kRowsPerWave];
 #pragma unroll
     for (int i = 0; i < kRowsPerWave; i++) cbv[i] = codebook[(kRowsPerWave * wave + i) & ((1 << S) - 1)];
-    const uint32_t table_sign = (uint32_t)(wave >> 3) << 15;
-    constexpr int kXRegs = 2;
+    const uint32_t table_sign = (uint32_t)((kRowsPerWave * wave) >> 7) << 15;
     uint4 xv[kXRegs], xv2[kXRegs], xvw[kXRegs];
 #pragma unroll
     for (int u = 0; u < kXRegs; u++) {
         const int idx = tid + u * kMatvecThreads;
         if constexpr (XMODE == kXPlain && !AFFINE) {
-            if (idx < n8) xv[u] = x[idx];               // staged under the same condition: nothing reads the rest
+            xv[u] = x[min(idx, n8 - 1)];                // every lane asks (no masked region); staged only where idx < n8
         } else {
             xv[u] = idx < n8 ? x[idx] : make_uint4(0, 0, 0, 0);
         }
@@ -383,29 +386,22 @@ __device__ __forceinline__ void matvec_body(
     // A lane past the item's rows repeats the last lane's address; a slot past the wave's items
     // repeats the first element of the wave's first item (of the stream for a wave with none).
     auto load_first = [&]() {
-        const uint32_t *first_base = comp;
-#pragma unroll
-        for (int u = 0; u < kBatch; u++) {
-            const bool have = it_begin + u < it_end;
-            const int row_first = ld_idx * ld.rows_per_item;           // row inside the block
-            const int rows_here = min(ld.rows_per_item, rows - row_first);
-            const uint32_t *item_base = comp + (size_t)(ld.elem0 + (uint32_t)(row0 + row_first) * (uint32_t)ld.lanes) * WORDS;
-            if (u == 0 && have && rows_here > 0) first_base = item_base;
-            // a slot the wave has no item for, or whose item lies past the block's last row, asks for one
-            // element in every lane: one cache line, not eight
-            const bool real = have && rows_here > 0;
-            const uint32_t *wave_base = real ? item_base : first_base;
-            const int nact = real ? rows_here * ld.lanes : 1;
-            buf[u] = load_stream<WORDS>(wave_base, min(lane, nact - 1));
-            if (MODE == RPTC_CONTINUOUS) {
-                // the word in front of a row: last word of the row's lane 31 in the slab before
-                // (read by all lanes of the row; used by its first lane, and only past slab 0)
-                const bool prev = real && ld_slab > 0;
-                const int sub = min(ld_slab < T ? lane >> 5 : lane / ld.lanes, max(rows_here, 1) - 1);
-                const uint32_t *row_base =
-                    prev ? comp + (((size_t)(ld_slab - 1) * m + row0 + row_first) * 32 + 31) * WORDS + WORDS - 1 : comp;
-                cw[u] = row_base[sub * (prev ? 32 * WORDS : 0)];
-            }
+        const int row_first = ld_idx * ld.rows_per_item;           // row inside the block
+        const int rows_here = min(ld.rows_per_item, rows - row_first);
+        // a wave without an item, or whose item lies past the block's last row, asks for the first element of
+        // the stream in every lane: one cache line, not eight
+        const bool real = it_begin < it_end && rows_here > 0;
+        const uint32_t elem = real ? ld.elem0 + (uint32_t)(row0 + row_first) * (uint32_t)ld.lanes : 0u;
+        const uint32_t last = real ? (uint32_t)(rows_here * ld.lanes - 1) : 0u;
+        buf[0] = load_stream<WORDS>(comp + (size_t)elem * WORDS, min((uint32_t)lane, last));
+        if (MODE == RPTC_CONTINUOUS) {
+            // the word in front of a row: last word of the row's lane 31 in the slab before
+            // (read by all lanes of the row; used by its first lane, and only past slab 0)
+            const bool prev = real && ld_slab > 0;
+            const int sub = min(ld_slab < T ? lane >> 5 : lane / ld.lanes, max(rows_here, 1) - 1);
+            const uint32_t *row_base =
+                prev ? comp + (((size_t)(ld_slab - 1) * m + row0 + row_first) * 32 + 31) * WORDS + WORDS - 1 : comp;
+            cw[0] = row_base[sub * (prev ? 32 * WORDS : 0)];
         }
     };
     static_assert(kBatch == 1, "the load cursor stands at the one item the first request asked for");
@@ -512,13 +508,23 @@ __device__ __forceinline__ void matvec_body(
         sx[idx + 2 * n8] = v.z;
         sx[idx + 3 * n8] = v.w;
     };
+    {
+        // a thread's second register lands 4096 bytes behind its first: four addresses and immediate offsets
+        uint32_t *const s0 = sx + tid, *const s1 = s0 + n8, *const s2 = s1 + n8, *const s3 = s2 + n8;
 #pragma unroll
-    for (int u = 0; u < kXRegs; u++) {
-        const int idx = tid + u * kMatvecThreads;
-        if (idx < n8) stage_x(idx, xv[u]);
+        for (int u = 0; u < kXRegs; u++) {
+            if (tid + u * kMatvecThreads < n8) {
+                s0[u * kMatvecThreads] = xv[u].x;
+                s1[u * kMatvecThreads] = xv[u].y;
+                s2[u * kMatvecThreads] = xv[u].z;
+                s3[u * kMatvecThreads] = xv[u].w;
+            }
+        }
     }
-    for (int idx = tid + kXRegs * kMatvecThreads; idx < n8; idx += kMatvecThreads)
-        stage_x(idx, XMODE == kXSiluMul ? silu_mul8(x[idx], x[n8 + idx]) : x[idx]);
+    if (n8 > kXRegs * kMatvecThreads) {                   // wave-uniform: short vectors skip the loop's set-up
+        for (int idx = tid + kXRegs * kMatvecThreads; idx < n8; idx += kMatvecThreads)
+            stage_x(idx, XMODE == kXSiluMul ? silu_mul8(x[idx], x[n8 + idx]) : x[idx]);
+    }
     __syncthreads();
     RPTC_STAMP(2);
     if constexpr (AFFINE) {
@@ -859,7 +865,7 @@ static int launch_matvec_affine(const int32_t *compressed, const uint16_t *codeb
                                 uint16_t *out, int64_t m, int64_t n, int carry_mode, void *stream, float *ms)
 {
     // the whole activation vector sits in two registers per thread
-    if (n > 8 * 2 * kMatvecThreads) return RPTC_ELIMIT;
+    if (n > 8 * kXRegs * kMatvecThreads) return RPTC_ELIMIT;
     if (!aligned16(s_in) || !aligned16(b_in)) return RPTC_EALIGN;
     DeviceInfo *dev;
     MatvecArgs a;
@@ -1044,7 +1050,7 @@ extern "C" int rptc_decompress_matvec_rmsnorm(const int32_t *c, const uint16_t *
     // every workgroup reads x_in and delta while workgroup 0 writes x_out
     if (x_out == x_in || x_out == delta) return RPTC_EALIAS;
     if (!aligned16(delta) || !aligned16(weight) || !aligned16(x_out)) return RPTC_EALIGN;
-    if (n > 8 * 2 * kMatvecThreads) return RPTC_ELIMIT;      // the whole vector sits in two registers per thread
+    if (n > 8 * kXRegs * kMatvecThreads) return RPTC_ELIMIT;      // the whole vector sits in two registers per thread
     return S == 6 ? launch_matvec_fused<6, kXAddRmsNorm>(c, cb, x_in, delta, weight, x_out, eps, 0, out, m, n, mode, stream, ms)
                   : launch_matvec_fused<8, kXAddRmsNorm>(c, cb, x_in, delta, weight, x_out, eps, 0, out, m, n, mode, stream, ms);
 }
