@@ -317,11 +317,28 @@ __device__ __forceinline__ void matvec_body(
 
     // This wave's items: a contiguous piece of [slab 0 items][slab 1 items]...[ragged slab items].
     const int total = T * a.items_full + a.items_tail;
-    // The first total % 16 waves take one item more.  Waves w, w+4, w+8, w+12 share a SIMD, so
-    // this also spreads the remainder evenly over the four SIMDs.
-    const int per_wave = (int)((uint32_t)total / kMatvecWaves), extra = (int)((uint32_t)total % kMatvecWaves);
-    const int it_begin = wave * per_wave + min(wave, extra);
-    const int it_end = it_begin + per_wave + (wave < extra ? 1 : 0);
+    // Waves w, w+4, w+8, w+12 share a SIMD, and the SIMD issues from the oldest wave that is ready: with equal
+    // shares wave w finishes long before wave w+12, and the SIMD ends its work with one wave that cannot
+    // keep it busy.  From three items a wave on, the four waves of a SIMD get shares near the proportion
+    // they are served in (kCum64 / 64 of the items for waves 0-3, 0-7, 0-11), split evenly inside each group
+    // of four, the remainders dealt to the SIMDs in turn so that no SIMD has more than one item above
+    // another.  With fewer items the first total % 16 waves take one more than the rest (older waves, again).
+    static_assert(kMatvecWaves == 16, "four waves per SIMD");
+    constexpr uint32_t kCum64 = 0x382A18u;                    // 24, 42, 56: shares of 24, 18, 14 and 8 of 64
+    int it_begin, it_end;
+    if (total >= 3 * kMatvecWaves) {
+        const uint32_t group = (uint32_t)wave >> 2;
+        const uint32_t cum_lo = group == 0 ? 0u : ((uint32_t)total * ((kCum64 >> (8 * group - 8)) & 0xFFu)) >> 6;
+        const uint32_t cum_hi = group == 3 ? (uint32_t)total : ((uint32_t)total * ((kCum64 >> (8 * group)) & 0xFFu)) >> 6;
+        const uint32_t cnt = cum_hi - cum_lo, per_wave = cnt >> 2, extra = cnt & 3u;
+        const uint32_t turn = ((uint32_t)wave - cum_lo) & 3u;
+        it_begin = (int)(cum_lo + turn * per_wave + min(turn, extra));
+        it_end = it_begin + (int)per_wave + (turn < extra ? 1 : 0);
+    } else {
+        const int per_wave = (int)((uint32_t)total / kMatvecWaves), extra = (int)((uint32_t)total % kMatvecWaves);
+        it_begin = wave * per_wave + min(wave, extra);
+        it_end = it_begin + per_wave + (wave < extra ? 1 : 0);
+    }
     auto view = [&](int slab) {
         SlabView v;
         const bool full = slab < T;
