@@ -215,9 +215,7 @@ __device__ __forceinline__ uint4 silu_mul8(const uint4 gate, const uint4 up)
     const uint32_t g[4] = {gate.x, gate.y, gate.z, gate.w}, u[4] = {up.x, up.y, up.z, up.w};
     uint32_t r[4];
 #pragma unroll
-    for (int i = 0; i < 4; i++)
-        r[i] = (uint32_t)silu_mul_bits((uint16_t)(g[i] & 0xFFFFu), (uint16_t)(u[i] & 0xFFFFu)) |
-               ((uint32_t)silu_mul_bits((uint16_t)(g[i] >> 16), (uint16_t)(u[i] >> 16)) << 16);
+    for (int i = 0; i < 4; i++) r[i] = silu_mul_pair(g[i], u[i]);
     return make_uint4(r[0], r[1], r[2], r[3]);
 }
 
@@ -431,21 +429,25 @@ __device__ __forceinline__ void matvec_body(
         for (int u = 0; u < kXRegs; u++) xv[u] = silu_mul8(xv[u], xv2[u]);
     }
     if constexpr (XMODE == kXAddRmsNorm) {
-        // host side guarantees n8 <= kXRegs * kMatvecThreads: the whole vector is in registers
-        Halves8 r[kXRegs];
+        // host side guarantees n8 <= kXRegs * kMatvecThreads: the whole vector is in registers.
+        // Every workgroup does this for the whole vector in front of its barrier, where the instruction count
+        // is what costs, so the halves stay packed: the residual add is a packed fp16 add (the sum of two fp16
+        // values rounded once: what an fp32 add rounded to fp16 gives as well), the squares are two-term dot
+        // products with an fp32 sum, the scaling converts, multiplies and rounds each half once, and the
+        // weight is a packed fp16 multiply (an exact product rounded once, as the fp32 product was).
+        uint32_t r[kXRegs][4];
         float ss = 0.f;
 #pragma unroll
         for (int u = 0; u < kXRegs; u++) {
-            r[u] = unpack8(xv[u]);
-            if (fuse.x2) {
-                const Halves8 d = unpack8(xv2[u]);
+            const uint32_t xw[4] = {xv[u].x, xv[u].y, xv[u].z, xv[u].w}, dw[4] = {xv2[u].x, xv2[u].y, xv2[u].z, xv2[u].w};
 #pragma unroll
-                for (int i = 0; i < 8; i++) r[u].v[i] = round_half(r[u].v[i] + d.v[i]);   // the fp16 residual stream
+            for (int i = 0; i < 4; i++) {
+                r[u][i] = fuse.x2 ? __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, xw[i]) + __builtin_bit_cast(half2_t, dw[i]))
+                                  : xw[i];                                    // the fp16 residual stream
+                ss = dot2(r[u][i], r[u][i], ss);
             }
-#pragma unroll
-            for (int i = 0; i < 8; i++) ss += r[u].v[i] * r[u].v[i];
             const int idx = tid + u * kMatvecThreads;
-            if (blockIdx.x == 0 && idx < n8) fuse.x_out[idx] = pack8(r[u]);
+            if (blockIdx.x == 0 && idx < n8) fuse.x_out[idx] = make_uint4(r[u][0], r[u][1], r[u][2], r[u][3]);
         }
         // sum over the workgroup in a fixed order
         ss = wave_sum(ss);
@@ -457,10 +459,17 @@ __device__ __forceinline__ void matvec_body(
         const float inv = rsqrtf(total_ss / (float)n + fuse.eps);
 #pragma unroll
         for (int u = 0; u < kXRegs; u++) {
-            const Halves8 w8 = unpack8(xvw[u]);
+            const uint32_t ww[4] = {xvw[u].x, xvw[u].y, xvw[u].z, xvw[u].w};
+            uint32_t h[4];
 #pragma unroll
-            for (int i = 0; i < 8; i++) r[u].v[i] = round_half(r[u].v[i] * inv) * w8.v[i];
-            xv[u] = pack8(r[u]);
+            for (int i = 0; i < 4; i++) {
+                const half2_t rv = __builtin_bit_cast(half2_t, r[u][i]);
+                half2_t sv;
+                sv.x = (_Float16)((float)rv.x * inv);
+                sv.y = (_Float16)((float)rv.y * inv);
+                h[i] = __builtin_bit_cast(uint32_t, sv * __builtin_bit_cast(half2_t, ww[i]));
+            }
+            xv[u] = make_uint4(h[0], h[1], h[2], h[3]);
         }
     }
 

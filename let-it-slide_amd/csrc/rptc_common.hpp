@@ -157,6 +157,20 @@ __device__ __forceinline__ uint16_t silu_mul_bits(uint16_t gate, uint16_t up)
     const _Float16 r = sg * __builtin_bit_cast(_Float16, up);
     return __builtin_bit_cast(uint16_t, r);
 }
+
+// The same for a register of two halves: the same operations on each half (so the same roundings), with the
+// halves left packed for the conversions' sake and one packed fp16 multiply at the end.
+__device__ __forceinline__ uint32_t silu_mul_pair(uint32_t gate, uint32_t up)
+{
+#pragma clang fp contract(off)
+    const half2_t g2 = __builtin_bit_cast(half2_t, gate);
+    const float g0 = (float)g2.x, g1 = (float)g2.y;
+    const float e0 = __builtin_amdgcn_exp2f(g0 * -1.44269504088896f), e1 = __builtin_amdgcn_exp2f(g1 * -1.44269504088896f);
+    half2_t sg;
+    sg.x = (_Float16)(g0 * __builtin_amdgcn_rcpf(1.f + e0));
+    sg.y = (_Float16)(g1 * __builtin_amdgcn_rcpf(1.f + e1));
+    return __builtin_bit_cast(uint32_t, sg * __builtin_bit_cast(half2_t, up));
+}
 #endif
 
 }  // namespace rptc
