@@ -111,6 +111,27 @@ __global__ __launch_bounds__(256) void rope_cache_kernel(const uint16_t *__restr
 // LDS, and the one whose piece holds *pos also rotates k and appends k and v to the caches (as
 // rope_cache_kernel does); it uses the new row from LDS.
 constexpr int kAttnThreads = 256;
+
+// v + (v of the lane the DPP pattern names): one vector op, no trip through LDS
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float v)
+{
+    return v + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0u, __builtin_bit_cast(uint32_t, v), CTRL, 0xF, 0xF, true));
+}
+
+// Sum over the lanes_per_key (2, 4, 8, 16 or 32) consecutive lanes that share a key, the same value in each of
+// them: neighbours, pairs of neighbours, the mirrored half row and the mirrored row (after the first two steps
+// the four lanes of a quad hold one value, so a mirror pairs the right quads), all as DPP adds.  (A loop of
+// cross-lane shuffles with a run-time distance is a trip through the LDS hardware per step and key.)
+__device__ __forceinline__ float group_sum(float v, int lanes_per_key)
+{
+    v = dpp_add<0xB1>(v);                                   // quad_perm [1, 0, 3, 2]
+    if (lanes_per_key > 2) v = dpp_add<0x4E>(v);            // quad_perm [2, 3, 0, 1]
+    if (lanes_per_key > 4) v = dpp_add<0x141>(v);           // row_half_mirror
+    if (lanes_per_key > 8) v = dpp_add<0x140>(v);           // row_mirror
+    if (lanes_per_key > 16) v += __shfl_xor(v, 16, 64);
+    return v;
+}
 constexpr int kAttnMaxParts = 4096;            // heads * splits
 constexpr int kAttnMaxHeads = 1024;
 constexpr int kAttnPartStride = 256 + 2;       // acc[hd <= 256], m, l
@@ -251,7 +272,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(
                 dot += half_bits_to_float((uint16_t)(w[c] & 0xFFFFu)) * qf[2 * c];
                 dot += half_bits_to_float((uint16_t)(w[c] >> 16)) * qf[2 * c + 1];
             }
-            for (int off = lanes_per_key >> 1; off > 0; off >>= 1) dot += __shfl_xor(dot, off, 64);
+            dot = group_sum(dot, lanes_per_key);
             sc[u] = s < cnt ? dot * scale : -INFINITY;
             m_new = fmaxf(m_new, sc[u]);
         }
