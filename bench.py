@@ -3,8 +3,10 @@
 
 One step = one call of decompress_matvec_16_8_1 (hashed-codebook stream, 2 bits/weight, 16-bit
 window) on the Llama-2-7B down-projection shape m=4096, n=11008, batch 1, through the C ABI.
-Steps rotate over distinct weight copies (default 32 x 11.27 MB > the 256 MB Infinity Cache) so
-every launch streams its weights from HBM.  The metric is GB/s of compressed weight bytes.
+Steps rotate over distinct weight copies whose total is at least 600 MB (more than twice the 256 MB
+Infinity Cache) whatever --steps is, and the caches are flushed with a 1 GiB read-modify-write pass between
+the untimed and the timed replay, so every timed launch streams its weights from HBM.  The metric is GB/s
+of compressed weight bytes.
 
 The line printed at the end also carries
   roofline      compressed bytes per launch / average launch duration (HIP events on the launch
@@ -36,7 +38,8 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=100)
-    ap.add_argument("--copies", type=int, default=32, help="distinct weight copies to rotate over")
+    ap.add_argument("--copies", type=int, default=0,
+                    help="distinct weight copies to rotate over (0: as many as make 600 MB, at least 32)")
     ap.add_argument("--m", type=int, default=4096)
     ap.add_argument("--n", type=int, default=11008)
     ap.add_argument("--S", type=int, default=8, choices=(6, 8))
@@ -61,6 +64,38 @@ def parse():
     ap.add_argument("--matmul", action="store_true",
                     help="time the batch 8/16/32 fused decode + MFMA mat-mat instead (prints its own JSON line)")
     return ap.parse_args()
+
+
+COLD_SET_BYTES = 600 << 20      # the rotating copies add up to at least this: > 2 x the 256 MB Infinity Cache
+
+
+def cold_copies(asked, layer_bytes):
+    """Copies to rotate over: what was asked for, but never fewer than make COLD_SET_BYTES (so that a copy is
+    revisited only after more than two cache sizes of other data), and at least 32."""
+    need = max(32, -(-COLD_SET_BYTES // layer_bytes))
+    return max(asked, need)
+
+
+_evict_buffer = None
+
+
+def evict_caches():
+    """A read-modify-write pass over 1 GiB: whatever the L2s and the Infinity Cache held is gone afterwards."""
+    import torch
+    global _evict_buffer
+    if _evict_buffer is None:
+        _evict_buffer = torch.zeros(1 << 28, dtype=torch.int32, device="cuda")
+    _evict_buffer.add_(1)
+    torch.cuda.synchronize()
+
+
+def aids_library():
+    """librptc_bench_aids.so: an empty launch and a read-only kernel (measurement aids, not the product)."""
+    path = os.path.join(ROOT, "let-it-slide_amd", "librptc_bench_aids.so")
+    lib = ctypes.CDLL(path)
+    lib.rptc_probe_empty.argtypes = [ctypes.c_int, ctypes.c_void_p]
+    lib.rptc_probe_read.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p]
+    return lib
 
 
 class Runner:
@@ -117,6 +152,7 @@ class Runner:
                     self.launch(k, cs)
             graph.replay()                      # untimed: first replay uploads the graph
             torch.cuda.synchronize()
+            evict_caches()                      # the timed replay starts with cold caches
             t0 = time.perf_counter()
             ev0.record()
             graph.replay()
@@ -124,6 +160,7 @@ class Runner:
             torch.cuda.synchronize()
             t1 = time.perf_counter()
         else:
+            evict_caches()
             t0 = time.perf_counter()
             ev0.record()
             for k in range(steps):
@@ -186,7 +223,7 @@ def bench_matmul(a):
     g = torch.Generator(device="cuda")
     g.manual_seed(42)
     words = m * n // 16
-    copies = max(2, min(a.copies, (512 << 20) // (words * 4) + 1))
+    copies = cold_copies(a.copies, words * 4)
     weights = [torch.randint(-(1 << 31), 1 << 31, (words,), generator=g, dtype=torch.int64, device="cuda").to(torch.int32)
                for _ in range(copies)]
     cb = torch.randn(2 << S, generator=g, device="cuda").to(torch.float16)
@@ -216,6 +253,7 @@ def bench_matmul(a):
                     step(k)
             graph.replay()
             torch.cuda.synchronize()
+            evict_caches()
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record()
             graph.replay()
@@ -244,7 +282,7 @@ def bench_matmul(a):
         fn = getattr(rptc_kernels, f"decompress_matmul_16_{S}_1")
         for mm, nn in ((11008, 4096), (8192, 8192), (28672, 8192), (8192, 28672)):
             words = mm * nn // 16
-            cps = max(2, min(a.copies, (512 << 20) // (words * 4) + 1))
+            cps = cold_copies(0, words * 4)
             ws = [torch.randint(-(1 << 31), 1 << 31, (words,), generator=g, dtype=torch.int64, device="cuda").to(torch.int32)
                   for _ in range(cps)]
             x = torch.randn((16, nn), generator=g, device="cuda").to(torch.float16)
@@ -260,7 +298,7 @@ def bench_matmul(a):
         for bits in (3, 4):
             mm, nn = 4096, 11008
             words = mm * nn * bits // 32
-            cps = max(2, min(a.copies, (512 << 20) // (words * 4) + 1))
+            cps = cold_copies(0, words * 4)
             ws = [torch.randint(-(1 << 31), 1 << 31, (words,), generator=g, dtype=torch.int64, device="cuda").to(torch.int32)
                   for _ in range(cps)]
             x = torch.randn((16, nn), generator=g, device="cuda").to(torch.float16)
@@ -292,6 +330,7 @@ def _graph_time_us(step, steps):
             step(k)
     graph.replay()
     torch.cuda.synchronize()
+    evict_caches()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record()
     graph.replay()
@@ -328,12 +367,13 @@ def bench_other_ops(a):
                                    "fill_of_the_output_us": round(fill_us, 2)}
     # transposed mat-vec, both carry modes
     for (m, n) in ((4096, 4096), (11008, 4096)):
-        streams = [rand_words(m * n // 16) for _ in range(16)]
+        ncp = cold_copies(0, m * n // 4)
+        streams = [rand_words(m * n // 16) for _ in range(ncp)]
         x = torch.randn(n, generator=g, device="cuda").half()
         out = torch.zeros(m, dtype=torch.float16, device="cuda")
         for mode, name in ((rk.AS_WRITTEN, "as_written"), (rk.CONTINUOUS, "continuous")):
             rk.set_carry_mode(mode)
-            us = _graph_time_us(lambda k: rk.decompress_matvec_t_16(streams[k % 16], cb16, x, out), steps)
+            us = _graph_time_us(lambda k: rk.decompress_matvec_t_16(streams[k % ncp], cb16, x, out), steps)
             byts = m * n // 4
             res[f"decompress_matvec_t_16 {m}x{n} {name}"] = {
                 "us": round(us, 2), "bytes": byts, "GBps": round(byts / us / 1e3, 1),
@@ -485,6 +525,7 @@ def main():
                                                  f"random ids, 128 greedy tokens; fused_graph = five launches per layer (element-wise steps inside the projections) in one HIP graph per token; glue_graph = nine launches per layer"},
                           "results": res}))
         return
+    a.copies = cold_copies(a.copies, a.m * a.n // 4)
     runner = Runner(a.m, a.n, a.S, a.copies)
     if a.pmc_probe:
         # calibration: an int32 -> float32 conversion copy is a plain streaming kernel that reads
@@ -520,7 +561,9 @@ def main():
         "data": "synthetic",
         "config": {
             "workload": f"decompress_matvec_16_{a.S}_1 m={a.m} n={a.n} 2 bits/weight batch 1 "
-                        f"(Llama-2-7B down_proj shape), {a.copies} rotating weight copies (cold cache)",
+                        f"(Llama-2-7B down_proj shape), {a.copies} rotating weight copies of {runner.bytes} bytes "
+                        f"({a.copies * runner.bytes >> 20} MiB), caches flushed before the timed region",
+            "distinct_copies_touched": min(a.steps, a.copies),
             "launch": a.launch,
             "accumulate": "f32",
             "carry_mode": "as_written",
@@ -539,7 +582,8 @@ def main():
     }
     # the floor of this workload on this machine, in the same launch pattern (graph replay over the
     # same rotating buffers): an empty launch, and a kernel that only reads the stream
-    lib = runner.lib
+    aids = aids_library()
+    grid = -(-a.m // (2 * -(-a.m // (2 * torch.cuda.get_device_properties(0).multi_processor_count))))
 
     def floor_us(call):
         steps = min(a.steps, 400)
@@ -553,6 +597,7 @@ def main():
                 call(k, cs)
         graph.replay()
         torch.cuda.synchronize()
+        evict_caches()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
         graph.replay()
@@ -561,12 +606,12 @@ def main():
         return e0.elapsed_time(e1) / steps * 1e3
 
     def call_empty(k, cs):
-        if lib.rptc_probe_empty(ctypes.c_void_p(cs)):
+        if aids.rptc_probe_empty(grid, ctypes.c_void_p(cs)):
             raise RuntimeError("rptc_probe_empty failed")
 
     def call_read(k, cs):
         w = runner.weights[k % len(runner.weights)]
-        if lib.rptc_probe_read(w.data_ptr(), runner.bytes, None, ctypes.c_void_p(cs)):
+        if aids.rptc_probe_read(w.data_ptr(), runner.bytes, None, ctypes.c_void_p(cs)):
             raise RuntimeError("rptc_probe_read failed")
 
     if a.launch == "graph":
@@ -580,7 +625,7 @@ def main():
     if a.extra_shapes:
         extra = {}
         for (m, n) in ((4096, 4096), (11008, 4096), (8192, 8192), (28672, 8192), (8192, 28672)):
-            r = Runner(m, n, a.S, max(2, min(a.copies, (512 << 20) // (m * n // 4) + 1)))
+            r = Runner(m, n, a.S, cold_copies(0, m * n // 4))
             r.check()
             _, ms = r.run(a.steps, a.warmup, a.launch)
             us = ms / a.steps * 1e3
@@ -590,7 +635,7 @@ def main():
             torch.cuda.empty_cache()
         for bits in (3, 4):
             for (m, n) in ((4096, 11008), (11008, 4096)):
-                r = Runner(m, n, a.S, max(2, min(a.copies, (512 << 20) // (m * n * bits // 8) + 1)), bits=bits)
+                r = Runner(m, n, a.S, cold_copies(0, m * n * bits // 8), bits=bits)
                 r.check()
                 _, ms = r.run(a.steps, a.warmup, a.launch)
                 us = ms / a.steps * 1e3

@@ -55,6 +55,17 @@ const char *rptc_status_string(int status);
 int rptc_init(void);
 
 /*
+ * The ops that split one output over several workgroups (rptc_decompress_matmul*, rptc_decompress_matvec_t_*
+ * on short matrices, rptc_attn_decode / rptc_rope_attn_decode) count arrivals in counters that live in static
+ * device memory and return to zero at the end of every launch.  A launch that never finished (a fault in another
+ * kernel, a reset) can leave one non-zero, and later launches would then merge too early.  This call counts the
+ * counters of the current device that are not zero into *nonzero and, with reset != 0, clears them.  It waits for
+ * `stream` (host-synchronous; not for use inside a stream capture) and must not overlap with the ops above.
+ * No counterpart in the reference.
+ */
+int rptc_scratch_check(int reset, int *nonzero, void *stream);
+
+/*
  * Decode only.  Replaces `float decompress(Tensor& compressed, Tensor& codebook, Tensor& out)`
  * (inference.cu:99-160, kernel inference.cu:42-96; bound at wrapper.cpp:60).
  *   compressed  int32 [m][words_per_row], words_per_row % 128 == 0 (inference.cu:106)
@@ -138,6 +149,17 @@ int rptc_decompress_matmul(const int32_t *compressed, const uint16_t *codebook, 
 int rptc_decompress_matmul_bits(const int32_t *compressed, const uint16_t *codebook, const uint16_t *x,
                                 uint16_t *out, int64_t m, int64_t n, int64_t batch, int S, int bits,
                                 int carry_mode, void *stream, float *ms);
+/*
+ * The same with the scratch memory (packed activations, partial tiles, arrival counters) in a buffer the caller
+ * brings: `workspace` is device memory, 256-byte aligned, of at least
+ * rptc_decompress_matmul_workspace_bytes(m, n, batch, bits) bytes (< 0: an RPTC_E* status for those sizes); its
+ * contents need no initialisation and mean nothing afterwards.  Calls with different workspaces may overlap on
+ * different streams of one device; the output is bit-identical to rptc_decompress_matmul_bits.
+ */
+int64_t rptc_decompress_matmul_workspace_bytes(int64_t m, int64_t n, int64_t batch, int bits);
+int rptc_decompress_matmul_ws(const int32_t *compressed, const uint16_t *codebook, const uint16_t *x,
+                              uint16_t *out, int64_t m, int64_t n, int64_t batch, int S, int bits,
+                              int carry_mode, void *workspace, int64_t workspace_bytes, void *stream, float *ms);
 
 /*
  * The hashed pair stream at `bits` = 2, 3 or 4 bits per weight, S in {6, 8}.  No counterpart in
@@ -172,7 +194,9 @@ int rptc_sign_hadamard(const uint16_t *x, const uint16_t *signs, uint16_t *out, 
  * The small kernels between the quantized projections of a Llama decoder layer, batch 1, one token
  * per call (no counterpart in the reference, which generates with transformers on dense weights,
  * quantize_hf.py:229-236).  fp16 in and out, fp32 arithmetic, asynchronous on `stream`; `pos` is a
- * device pointer to the token's position so that a captured HIP graph can be replayed.
+ * device pointer to the token's position so that a captured HIP graph can be replayed.  A position outside
+ * [0, max_len) makes rptc_rope_cache, rptc_attn_decode and rptc_rope_attn_decode write nothing (no cache row,
+ * no output) instead of indexing the tables and caches out of bounds.
  *   rptc_add_rmsnorm  x_out = x_in + delta (delta may be NULL); h_out = rmsnorm(x_out) * weight; all [d]
  *   rptc_rope_cache   qkv = [q|k|v], each heads*hd: rotate the (2i, 2i+1) pairs of q and k by
  *                     cos/sin [max_len][hd/2] at *pos, write q_out and k, v into caches [heads][max_len][hd]
@@ -282,17 +306,6 @@ int rptc_viterbi_pairs_bits(const float *targets, const float *weights, int64_t 
 int rptc_viterbi_scalar(const float *targets, const float *weights, int64_t weights_row_stride,
                         const uint16_t *alphabet, int L, void *scratch, uint8_t *symbols, int32_t *end_state,
                         float *cost, int64_t rows, int64_t steps, void *stream, float *ms);
-
-/*
- * Measurement aids (no counterpart in the reference; not part of the product path).  bench.py times
- * them in the same launch pattern as the mat-vec it grades, so that the achieved figure can be read
- * against the floor for the workload's size on the machine at hand.
- *   rptc_probe_empty  one empty 1024-thread workgroup per CU
- *   rptc_probe_read   reads `bytes` (a multiple of 16, 16-byte aligned) with non-temporal 16-byte loads
- *                     and writes nothing; `sink` may be NULL
- */
-int rptc_probe_empty(void *stream);
-int rptc_probe_read(const void *data, int64_t bytes, void *sink, void *stream);
 
 #ifdef __cplusplus
 }

@@ -1,10 +1,12 @@
-// Measurement aids: what the machine does with no decode at all, for the same bytes and the same
-// launch pattern as the mat-vec.  bench.py times them beside the kernel it grades, so that the
-// roofline figure can be read against the floor of this workload size: the time of an empty
-// launch, and the time of a kernel that only reads the stream.  Not part of the product path.
-#include "rptc_common.hpp"
+// Measurement aids (librptc_bench_aids.so): what the machine does with no decode at all, for the
+// same bytes and the same launch pattern as the mat-vec.  bench.py times them beside the kernel it
+// grades, so that the roofline figure can be read against the floor of this workload size: the time
+// of an empty launch, and the time of a kernel that only reads the stream.  A library of its own:
+// nothing here is part of the product path or of its header.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
 
-namespace rptc {
+namespace {
 
 __global__ __launch_bounds__(1024) void probe_empty_kernel() {}
 
@@ -30,31 +32,26 @@ __global__ __launch_bounds__(1024) void probe_read_kernel(const uint32_t *__rest
     if (s == 0x9E3779B9u && sink) sink[0] = s;
 }
 
-}  // namespace rptc
+}  // namespace
 
-using namespace rptc;
-
-extern "C" int rptc_probe_empty(void *stream)
+// one empty 1024-thread workgroup per workgroup of the mat-vec's grid
+extern "C" int rptc_probe_empty(int workgroups, void *stream)
 {
-    DeviceInfo *dev;
-    int rc = device_info(&dev);
-    if (rc) return rc;
-    hipLaunchKernelGGL(probe_empty_kernel, dim3(dev->cus), dim3(1024), 0, static_cast<hipStream_t>(stream));
+    if (workgroups < 1) return -2;
+    hipLaunchKernelGGL(probe_empty_kernel, dim3(workgroups), dim3(1024), 0, static_cast<hipStream_t>(stream));
     return (int)hipGetLastError();
 }
 
+// reads `bytes` (a multiple of 16, 16-byte aligned) with non-temporal 16-byte loads and writes nothing
 extern "C" int rptc_probe_read(const void *data, int64_t bytes, void *sink, void *stream)
 {
-    if (!data) return RPTC_ENULL;
-    if (bytes < 16 || bytes % 16 != 0) return RPTC_ESHAPE;
-    if (!aligned16(data)) return RPTC_EALIGN;
-    DeviceInfo *dev;
-    int rc = device_info(&dev);
-    if (rc) return rc;
+    if (!data) return -1;
+    if (bytes < 16 || bytes % 16 != 0) return -2;
+    if (reinterpret_cast<uintptr_t>(data) & 15u) return -3;
     const size_t total16 = (size_t)bytes / 16;
     const size_t per_block = (size_t)1024 * kPerThread;
     const size_t grid = (total16 + per_block - 1) / per_block;
-    if (grid >= ((size_t)1 << 31)) return RPTC_ELIMIT;
+    if (grid >= ((size_t)1 << 31)) return -5;
     hipLaunchKernelGGL(probe_read_kernel, dim3((unsigned)grid), dim3(1024), 0, static_cast<hipStream_t>(stream),
                        static_cast<const uint32_t *>(data), static_cast<uint32_t *>(sink), total16);
     return (int)hipGetLastError();

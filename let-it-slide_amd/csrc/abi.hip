@@ -13,6 +13,9 @@ int prepare_matmul(int device);
 int prepare_hadamard();
 int prepare_decode_glue(int device);
 int prepare_viterbi();
+void matmul_counters(int device, uint32_t **counters, int *count);
+void matvec_t_counters(int device, uint32_t **counters, int *count);
+void attn_counters(int device, uint32_t **counters, int *count);
 
 constexpr int kMaxDevices = 64;
 static DeviceInfo g_devices[kMaxDevices];
@@ -49,9 +52,50 @@ int device_info(DeviceInfo **out)
     return 0;
 }
 
+// Counts the arrival counters that are not zero, and clears them when asked to.
+static __device__ __align__(256) uint32_t g_check_result[64];
+
+__global__ void scratch_check_clear_kernel(uint32_t *result) { *result = 0u; }
+
+__global__ __launch_bounds__(256) void scratch_check_kernel(uint32_t *counters, int count, int reset, uint32_t *result)
+{
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= count) return;
+    if (__hip_atomic_load(&counters[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) {
+        atomicAdd(result, 1u);
+        if (reset) __hip_atomic_store(&counters[i], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+
 }  // namespace rptc
 
-extern "C" int rptc_version(void) { return 100; }
+extern "C" int rptc_scratch_check(int reset, int *nonzero, void *stream)
+{
+    using namespace rptc;
+    if (!nonzero) return RPTC_ENULL;
+    DeviceInfo *d;
+    int rc = device_info(&d);
+    if (rc) return rc;
+    uint32_t *result;
+    if ((rc = (int)hipGetSymbolAddress(reinterpret_cast<void **>(&result), HIP_SYMBOL(g_check_result)))) return rc;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    hipLaunchKernelGGL(scratch_check_clear_kernel, dim3(1), dim3(1), 0, s, result);
+    void (*const sets[3])(int, uint32_t **, int *) = {matmul_counters, matvec_t_counters, attn_counters};
+    for (auto get : sets) {
+        uint32_t *counters;
+        int count;
+        get(d->device, &counters, &count);
+        hipLaunchKernelGGL(scratch_check_kernel, dim3((count + 255) / 256), dim3(256), 0, s, counters, count, reset, result);
+    }
+    if ((rc = (int)hipGetLastError())) return rc;
+    uint32_t host = 0;
+    if ((rc = (int)hipMemcpyAsync(&host, result, sizeof(uint32_t), hipMemcpyDeviceToHost, s))) return rc;
+    if ((rc = (int)hipStreamSynchronize(s))) return rc;
+    *nonzero = (int)host;
+    return 0;
+}
+
+extern "C" int rptc_version(void) { return 200; }
 
 extern "C" int rptc_init(void)
 {

@@ -12,17 +12,11 @@
 namespace rptc {
 
 // hash, two addresses, two gathers for window register G (high window -> TH, low window -> TL)
-#ifndef RPTC_ABLATE_LDS
 #define RPTC_RD2(G, TH, TL)                                   \
     "v_perm_b32 " TH ", " G ", %[lane4], %[sel]\n"            \
     "v_and_or_b32 " TL ", " G ", %[mask], %[lane4]\n"         \
     "ds_read_b32 " TH ", " TH "\n"                            \
     "ds_read_b32 " TL ", " TL "\n"
-#else   // development probe: the same vector ops without the gathers
-#define RPTC_RD2(G, TH, TL)                                   \
-    "v_perm_b32 " TH ", " G ", %[lane4], %[sel]\n"            \
-    "v_and_or_b32 " TL ", " G ", %[mask], %[lane4]\n"
-#endif
 
 #define RPTC_WINDOWS(SH)                                      \
     "v_alignbit_b32 %[g0], %[cy], %[ex], " #SH "\n"           \
@@ -48,10 +42,6 @@ namespace rptc {
 
 // products of block j: {carry,x}: steps 28+j (high), j (low); {x,y}: 16+j, 4+j; {y,z}: 20+j, 8+j;
 // {z,w}: 24+j, 12+j
-#ifdef RPTC_ABLATE_DOT   // development probe: the gathers without the products
-#define RPTC_DOTS(T0, T1, T2, T3, T4, T5, T6, T7, XA, XB, XC, XD, XE, XF, XG, XH) \
-    "v_dot2c_f32_f16 %[a0], " T0 ", %[" XA "]\n"
-#else
 #define RPTC_DOTS(T0, T1, T2, T3, T4, T5, T6, T7, XA, XB, XC, XD, XE, XF, XG, XH) \
     "v_dot2c_f32_f16 %[a0], " T0 ", %[" XA "]\n"              \
     "v_dot2c_f32_f16 %[a1], " T1 ", %[" XB "]\n"              \
@@ -61,14 +51,8 @@ namespace rptc {
     "v_dot2c_f32_f16 %[a1], " T5 ", %[" XF "]\n"              \
     "v_dot2c_f32_f16 %[a2], " T6 ", %[" XG "]\n"              \
     "v_dot2c_f32_f16 %[a3], " T7 ", %[" XH "]\n"
-#endif
 
 // the first products of an element start the four sums (no accumulator to clear beforehand)
-#ifdef RPTC_ABLATE_DOT
-#define RPTC_DOTS_FIRST(T0, T1, T2, T3, T4, T5, T6, T7, XA, XB, XC, XD, XE, XF, XG, XH) \
-    "v_dot2_f32_f16 %[a0], " T0 ", %[" XA "], 0\n"           \
-    "v_mov_b32 %[a1], 0\n v_mov_b32 %[a2], 0\n v_mov_b32 %[a3], 0\n"
-#else
 #define RPTC_DOTS_FIRST(T0, T1, T2, T3, T4, T5, T6, T7, XA, XB, XC, XD, XE, XF, XG, XH) \
     "v_dot2_f32_f16 %[a0], " T0 ", %[" XA "], 0\n"           \
     "v_dot2_f32_f16 %[a1], " T1 ", %[" XB "], 0\n"           \
@@ -78,7 +62,6 @@ namespace rptc {
     "v_dot2c_f32_f16 %[a1], " T5 ", %[" XF "]\n"             \
     "v_dot2c_f32_f16 %[a2], " T6 ", %[" XG "]\n"             \
     "v_dot2c_f32_f16 %[a3], " T7 ", %[" XH "]\n"
-#endif
 
 // one more expansion pass so that a register-list macro can stand for eight arguments
 #define RPTC_READS_X(...) RPTC_READS(__VA_ARGS__)

@@ -7,11 +7,6 @@
 // HIP graph can be replayed for successive tokens.
 #include "rptc_common.hpp"
 
-// Development hook: a probe build defines RPTC_ATTN_STAMP to record a per-workgroup timestamp at each phase.
-#ifndef RPTC_ATTN_STAMP
-#define RPTC_ATTN_STAMP(slot) ((void)0)
-#endif
-
 namespace rptc {
 
 __device__ __forceinline__ float block_sum(float v, float *scratch)
@@ -80,7 +75,10 @@ __global__ __launch_bounds__(256) void rope_cache_kernel(const uint16_t *__restr
                                                          uint16_t *__restrict__ q_out, uint16_t *__restrict__ k_cache,
                                                          uint16_t *__restrict__ v_cache, int heads, int hd, int max_len)
 {
-    const int pos = (int)*pos_p;
+    const int64_t pos64 = *pos_p;
+    // a position outside the caches (a graph replayed past max_len) writes nothing
+    if (pos64 < 0 || pos64 >= (int64_t)max_len) return;
+    const int pos = (int)pos64;
     const int half = hd >> 1, d = heads * hd;
     const int t = blockIdx.x * blockDim.x + threadIdx.x;        // one (head, pair) per thread
     if (t >= heads * half) return;
@@ -148,12 +146,15 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(
     uint32_t *__restrict__ arrived)
 {
     extern __shared__ float lds_f[];
-    RPTC_ATTN_STAMP(0);
     float *scratch = lds_f;                      // [16]: the "came last" flag
     float *acc = scratch + 16;                   // the waves' sums [waves][hd], then their m and l: < 2048 floats
     uint16_t *q_rot = reinterpret_cast<uint16_t *>(acc + 2048);   // [3][hd] halves (q, new k, new v), ROPE only
     const int h = blockIdx.x / splits, sp = blockIdx.x - h * splits, tid = threadIdx.x;
-    const int len = (int)*pos_p + 1;
+    // A position outside the caches (a graph replayed past max_len) would index the tables and the caches out
+    // of bounds: every workgroup of the launch leaves at once (the same value for all), `out` keeps what it held.
+    const int64_t pos64 = *pos_p;
+    if (pos64 < 0 || pos64 >= (int64_t)max_len) return;
+    const int len = (int)pos64 + 1;
     // this workgroup's keys: [s_begin, s_end)
     const int chunk = ((len + splits - 1) / splits + 15) & ~15;
     const int s_begin = sp * chunk, s_end = min(len, s_begin + chunk), cnt = max(0, s_end - s_begin);
@@ -234,7 +235,6 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(
         load_values(0);
     }
 
-    RPTC_ATTN_STAMP(1);
     // The lanes that share a key (a group) keep a running softmax of their own keys: maximum m,
     // sum l of exp(score - m) and the unnormalised value sum a8 (8 output dimensions a lane), so
     // nothing leaves the group before the piece's last key.  Then the groups of a wave are merged
@@ -276,7 +276,6 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(
             sc[u] = s < cnt ? dot * scale : -INFINITY;
             m_new = fmaxf(m_new, sc[u]);
         }
-        if (s0 == 0) RPTC_ATTN_STAMP(2);
         // a group with no key yet keeps m = -inf: its factors must be 0, not exp(-inf - -inf)
         const float keep = m_g == -INFINITY ? 0.f : __expf(m_g - m_new);
         l_g *= keep;
@@ -301,7 +300,6 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(
             }
         }
     }
-    RPTC_ATTN_STAMP(3);
     // the groups of a wave (lanes sub, sub + lanes_per_key, ...): butterfly over the lane bits above
     // the group's, in a fixed order
     for (int off = lanes_per_key; off < 64; off <<= 1) {
@@ -348,22 +346,21 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(
         __hip_atomic_store(&mine[256], mx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __hip_atomic_store(&mine[257], sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-    // device-scope stores and loads bypass the XCD-private cache levels, so the only ordering needed
-    // is that this workgroup's stores have completed before its arrival is counted
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    __builtin_amdgcn_s_waitcnt(0);
-    RPTC_ATTN_STAMP(4);
+    // Release / acquire at agent scope: the storing threads release the piece before the barrier lets thread 0
+    // count the arrival (an acquire-release read-modify-write), and the workgroup that sees the last arrival
+    // acquires before it reads the other pieces, whichever XCD they were computed on.
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
     __syncthreads();
     uint32_t *flag = reinterpret_cast<uint32_t *>(scratch);
     if (tid == 0) {
-        const uint32_t prev = __hip_atomic_fetch_add(&arrived[h], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const uint32_t prev = __hip_atomic_fetch_add(&arrived[h], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
         const bool last = prev == (uint32_t)(splits - 1);
         if (last) __hip_atomic_store(&arrived[h], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // for the next launch
         *flag = last;
     }
     __syncthreads();
-    RPTC_ATTN_STAMP(5);
     if (!*flag || tid >= hd) return;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
     const float *head_parts = parts + (size_t)h * splits * kAttnPartStride;
     constexpr int kMaxSplits = 16;
     float pm[kMaxSplits], pl[kMaxSplits], pa[kMaxSplits];
@@ -389,7 +386,6 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(
         den += pl[i] * w;
     }
     out[h * hd + tid] = float_to_half_bits(num / den);
-    RPTC_ATTN_STAMP(6);
 }
 
 // gu = [gate | up], each f:  out = silu(gate) * up
@@ -531,6 +527,12 @@ int prepare_decode_glue(int device)
     int rc = (int)hipGetSymbolAddress(reinterpret_cast<void **>(&g_attn[device].parts), HIP_SYMBOL(g_attn_part));
     if (rc) return rc;
     return (int)hipGetSymbolAddress(reinterpret_cast<void **>(&g_attn[device].arrived), HIP_SYMBOL(g_attn_arrived));
+}
+
+void attn_counters(int device, uint32_t **counters, int *count)
+{
+    *counters = g_attn[device].arrived;
+    *count = kAttnMaxHeads;
 }
 
 template <bool ROPE>

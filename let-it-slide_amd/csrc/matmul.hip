@@ -28,11 +28,6 @@
 //   * batch 17..32 decodes once and feeds two sets of MFMAs (two planes of 16 batch columns).
 #include "rptc_common.hpp"
 
-// Development hook: a probe build defines RPTC_MM_STAMP to record a per-wave timestamp at each phase.
-#ifndef RPTC_MM_STAMP
-#define RPTC_MM_STAMP(slot) ((void)0)
-#endif
-
 namespace rptc {
 
 constexpr int kMmThreads = 512;
@@ -131,7 +126,6 @@ __global__ __launch_bounds__(kMmThreads) __attribute__((amdgpu_waves_per_eu(4, 4
     constexpr int kPartBuffers = PLANES == 1 ? 2 : 1;
     constexpr int WORDS = 2 * BITS;                               // words per stream element
     constexpr int kMaxRb = mm_max_row_blocks(PLANES, BITS);
-    RPTC_MM_STAMP(0);
     float *part = reinterpret_cast<float *>(lds + kMmTableBytes / 4);   // [buffer][wave][plane][v][lane]
     // the "came last" flag reuses the first word of the tiles once they are no longer read (all LDS
     // is dynamic, and 64 + 16 KiB lets two workgroups share a CU)
@@ -217,9 +211,7 @@ __global__ __launch_bounds__(kMmThreads) __attribute__((amdgpu_waves_per_eu(4, 4
 #pragma unroll
         for (int r = 0; r < kTableRowsPerWave; r++) lds[(kTableRowsPerWave * c + r) * 64 + lane] = table_values[r];
     }
-    RPTC_MM_STAMP(1);
     __syncthreads();                                              // the table is complete
-    RPTC_MM_STAMP(2);
 
     float *my_partial = partial + ((size_t)blockIdx.x * max_rb) * (PLANES * 256);
 #pragma unroll
@@ -297,7 +289,6 @@ __global__ __launch_bounds__(kMmThreads) __attribute__((amdgpu_waves_per_eu(4, 4
                 for (int v = 0; v < 4; v++) buf[((c * PLANES + p) * 4 + v) * 64 + lane] = d[v];
             }
         }
-        if (rb == 0) RPTC_MM_STAMP(3);
         // With two buffers one barrier per row block is enough: the halves of `part` alternate, and a
         // wave can only reach the write of row block rb+2 after it passed the barrier of rb+1, which
         // every wave reaches after its sum of rb.
@@ -314,23 +305,21 @@ __global__ __launch_bounds__(kMmThreads) __attribute__((amdgpu_waves_per_eu(4, 4
     }
 
     // The workgroup that arrives last at its row group's counter adds the slabs' tiles, in slab order.
-    // Every partial tile is stored and loaded with device-scope atomic accesses, which bypass the
-    // XCD-private cache levels, so the only ordering needed is that this workgroup's stores have
-    // completed before its arrival is counted (the wait below, then the barrier).
-    RPTC_MM_STAMP(4);
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    __builtin_amdgcn_s_waitcnt(0);
-    RPTC_MM_STAMP(5);
+    // Release / acquire at agent scope: every thread that stored part of a tile releases its stores (they have
+    // reached device-coherent memory before the barrier lets thread 0 count the arrival), thread 0's counter
+    // update is an acquire-release read-modify-write, and the workgroup that sees the last arrival acquires
+    // before it reads the other workgroups' tiles, whichever XCD they ran on.
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
     __syncthreads();
     if (tid == 0) {
-        const uint32_t prev = __hip_atomic_fetch_add(&arrived[grp], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const uint32_t prev = __hip_atomic_fetch_add(&arrived[grp], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
         const bool last = prev == (uint32_t)(slabs - 1);
         if (last) __hip_atomic_store(&arrived[grp], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // for the next launch
         *s_last = last;
     }
     __syncthreads();
-    RPTC_MM_STAMP(6);
     if (!*s_last) return;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
     const int tile_floats = row_blocks * PLANES * 256, tile_stride = max_rb * PLANES * 256;
     const float *grp_partial = partial + (size_t)grp * slabs * tile_stride;
     // every thread requests its share of four slabs' tiles before it adds any of them: the loads go
@@ -364,13 +353,13 @@ __global__ __launch_bounds__(kMmThreads) __attribute__((amdgpu_waves_per_eu(4, 4
         const int b = 16 * p + (ln & 15), row = row0 + 16 * rb + 4 * (ln >> 4) + v;
         if (b < batch && row < m) out[(size_t)b * m + row] = float_to_half_bits(y[k]);
     }
-    RPTC_MM_STAMP(7);
 }
 
 struct MmScratch {
     uint32_t *xpack;
     float *partial;
     uint32_t *arrived;
+    int64_t partial_floats;     // capacity of `partial`
 };
 static MmScratch g_mm[64];   // per device: addresses of the static scratch arrays
 
@@ -400,7 +389,14 @@ int prepare_matmul(int device)
     MmScratch &sc = g_mm[device];
     if ((rc = (int)hipGetSymbolAddress(reinterpret_cast<void **>(&sc.xpack), HIP_SYMBOL(g_xpack)))) return rc;
     if ((rc = (int)hipGetSymbolAddress(reinterpret_cast<void **>(&sc.partial), HIP_SYMBOL(g_partial)))) return rc;
+    sc.partial_floats = kMmScratchFloats;
     return (int)hipGetSymbolAddress(reinterpret_cast<void **>(&sc.arrived), HIP_SYMBOL(g_arrived));
+}
+
+void matmul_counters(int device, uint32_t **counters, int *count)
+{
+    *counters = g_mm[device].arrived;
+    *count = kMmMaxGroups;
 }
 
 // Number of row groups: as many as keep every workgroup of the launch resident at once (two per
@@ -420,11 +416,12 @@ template <int S, int PLANES, int BITS>
 static void launch_matmul(const uint32_t *comp, const uint32_t *cb, const MmScratch &sc, uint16_t *out, int m, int n,
                           int batch, int carry_mode, int groups, int slabs, hipStream_t s)
 {
+    // sc.partial_floats: how many partial-tile floats the scratch holds (the static buffer, or the caller's)
     const int lds_bytes = kMmTableBytes + kMmWaves * 2 * 256 * 4;
     const int total = (m + 15) / 16;
     const int max_rb = (total + groups - 1) / groups;
     // as many row groups per launch as the scratch buffer holds partial tiles for
-    int64_t per_launch = kMmScratchFloats / ((int64_t)slabs * max_rb * PLANES * 256);
+    int64_t per_launch = sc.partial_floats / ((int64_t)slabs * max_rb * PLANES * 256);
     if (per_launch > kMmMaxGroups) per_launch = kMmMaxGroups;
     for (int g0 = 0; g0 < groups; g0 += (int)per_launch) {
         const int g_n = groups - g0 < per_launch ? groups - g0 : (int)per_launch;
@@ -451,39 +448,70 @@ static void launch_matmul_planes(const uint32_t *comp, const uint32_t *cb, const
 
 using namespace rptc;
 
-extern "C" int rptc_decompress_matmul_bits(const int32_t *compressed, const uint16_t *codebook, const uint16_t *x,
-                                           uint16_t *out, int64_t m, int64_t n, int64_t batch, int S, int bits,
-                                           int carry_mode, void *stream, float *ms)
+namespace rptc {
+
+struct MmPlan {
+    int planes, slabs, groups, counters;
+    int64_t xpack_words, partial_floats;      // what one launch over all row groups needs
+};
+
+static int plan_matmul(const void *compressed, const void *codebook, const void *x, const void *out, int64_t m, int64_t n,
+                       int64_t batch, int S, int bits, int carry_mode, DeviceInfo **dev, MmPlan *p)
 {
     if (!compressed || !codebook || !x || !out) return RPTC_ENULL;
     if (m < 1 || n < 64 || n % 64 != 0 || batch < 1 || (S != 6 && S != 8) || bits < 2 || bits > 4) return RPTC_ESHAPE;
     if (n > kMmMaxN || batch > kMmMaxBatch || m >= (1 << 24)) return RPTC_ELIMIT;
     if (carry_mode != RPTC_AS_WRITTEN && carry_mode != RPTC_CONTINUOUS) return RPTC_EMODE;
     if (!aligned16(compressed) || !aligned16(codebook) || !aligned16(x)) return RPTC_EALIGN;
-    DeviceInfo *dev;
-    int rc = device_info(&dev);
+    int rc = device_info(dev);
     if (rc) return rc;
+    p->planes = batch > 16 ? 2 : 1;
+    p->slabs = (int)(n / 2048) + (n % 2048 ? 1 : 0);
+    p->groups = mm_groups((int)m, p->slabs, (*dev)->cus, p->planes, bits);
+    p->counters = p->groups < kMmMaxGroups ? p->groups : kMmMaxGroups;
+    const int total = ((int)m + 15) / 16;
+    const int max_rb = (total + p->groups - 1) / p->groups;
+    p->xpack_words = (int64_t)p->planes * (n / 2) * 16;
+    p->partial_floats = (int64_t)p->groups * p->slabs * max_rb * p->planes * 256;
+    return 0;
+}
+
+static int run_matmul(const int32_t *compressed, const uint16_t *codebook, const uint16_t *x, uint16_t *out, int64_t m,
+                      int64_t n, int64_t batch, int S, int bits, int carry_mode, const MmScratch &sc, const MmPlan &p,
+                      DeviceInfo *dev, void *stream, float *ms)
+{
     hipStream_t s = static_cast<hipStream_t>(stream);
     Timer t;
-    rc = t.begin(dev, s, ms);
+    int rc = t.begin(dev, s, ms);
     if (rc) return rc;
     auto a_comp = reinterpret_cast<const uint32_t *>(compressed);
     auto a_cb = reinterpret_cast<const uint32_t *>(codebook);
-    const MmScratch &sc = g_mm[dev->device];
-    const int planes = batch > 16 ? 2 : 1;
-    const int slabs = (int)(n / 2048) + (n % 2048 ? 1 : 0);
-    const int groups = mm_groups((int)m, slabs, dev->cus, planes, bits);
-    const int counters = groups < kMmMaxGroups ? groups : kMmMaxGroups;
-    const int total = planes * (int)(n / 8) * 16;
-    const int pack_threads = total > counters ? total : counters;
+    const int total = p.planes * (int)(n / 8) * 16;
+    const int pack_threads = total > p.counters ? total : p.counters;
     hipLaunchKernelGGL(pack_x_kernel, dim3((pack_threads + 255) / 256), dim3(256), 0, s, reinterpret_cast<const uint4 *>(x), sc.xpack, sc.arrived,
-                       counters, (int)n, (int)batch, planes);
+                       p.counters, (int)n, (int)batch, p.planes);
 #define RPTC_MM_GO(SS, BB)                                                                                          \
     if (S == SS && bits == BB)                                                                                       \
-        launch_matmul_planes<SS, BB>(a_comp, a_cb, sc, out, (int)m, (int)n, (int)batch, carry_mode, dev->cus, slabs, s);
+        launch_matmul_planes<SS, BB>(a_comp, a_cb, sc, out, (int)m, (int)n, (int)batch, carry_mode, dev->cus, p.slabs, s);
     RPTC_MM_GO(6, 2) RPTC_MM_GO(6, 3) RPTC_MM_GO(6, 4) RPTC_MM_GO(8, 2) RPTC_MM_GO(8, 3) RPTC_MM_GO(8, 4)
 #undef RPTC_MM_GO
     return t.end();
+}
+
+// layout of a caller's workspace: [packed activations | partial tiles | arrival counters], each 256-byte aligned
+static int64_t ws_round(int64_t bytes) { return (bytes + 255) & ~(int64_t)255; }
+
+}  // namespace rptc
+
+extern "C" int rptc_decompress_matmul_bits(const int32_t *compressed, const uint16_t *codebook, const uint16_t *x,
+                                           uint16_t *out, int64_t m, int64_t n, int64_t batch, int S, int bits,
+                                           int carry_mode, void *stream, float *ms)
+{
+    DeviceInfo *dev;
+    MmPlan p;
+    int rc = plan_matmul(compressed, codebook, x, out, m, n, batch, S, bits, carry_mode, &dev, &p);
+    if (rc) return rc;
+    return run_matmul(compressed, codebook, x, out, m, n, batch, S, bits, carry_mode, g_mm[dev->device], p, dev, stream, ms);
 }
 
 extern "C" int rptc_decompress_matmul(const int32_t *compressed, const uint16_t *codebook, const uint16_t *x,
@@ -491,4 +519,38 @@ extern "C" int rptc_decompress_matmul(const int32_t *compressed, const uint16_t 
                                       void *stream, float *ms)
 {
     return rptc_decompress_matmul_bits(compressed, codebook, x, out, m, n, batch, S, 2, carry_mode, stream, ms);
+}
+
+extern "C" int64_t rptc_decompress_matmul_workspace_bytes(int64_t m, int64_t n, int64_t batch, int bits)
+{
+    if (m < 1 || n < 64 || n % 64 != 0 || batch < 1 || bits < 2 || bits > 4) return RPTC_ESHAPE;
+    if (n > kMmMaxN || batch > kMmMaxBatch || m >= (1 << 24)) return RPTC_ELIMIT;
+    DeviceInfo *dev;
+    MmPlan p;
+    const void *any = reinterpret_cast<const void *>(16);      // the plan only tests pointers for NULL and alignment
+    int rc = plan_matmul(any, any, any, any, m, n, batch, 8, bits, RPTC_AS_WRITTEN, &dev, &p);
+    if (rc) return rc < 0 ? rc : RPTC_EDEVICE;
+    return ws_round(p.xpack_words * 4) + ws_round(p.partial_floats * 4) + ws_round((int64_t)p.counters * 4);
+}
+
+extern "C" int rptc_decompress_matmul_ws(const int32_t *compressed, const uint16_t *codebook, const uint16_t *x,
+                                         uint16_t *out, int64_t m, int64_t n, int64_t batch, int S, int bits,
+                                         int carry_mode, void *workspace, int64_t workspace_bytes, void *stream,
+                                         float *ms)
+{
+    DeviceInfo *dev;
+    MmPlan p;
+    int rc = plan_matmul(compressed, codebook, x, out, m, n, batch, S, bits, carry_mode, &dev, &p);
+    if (rc) return rc;
+    if (!workspace) return RPTC_ENULL;
+    if (reinterpret_cast<uintptr_t>(workspace) & 255u) return RPTC_EALIGN;
+    const int64_t xb = ws_round(p.xpack_words * 4), pb = ws_round(p.partial_floats * 4), cb = ws_round((int64_t)p.counters * 4);
+    if (workspace_bytes < xb + pb + cb) return RPTC_ELIMIT;
+    char *base = static_cast<char *>(workspace);
+    MmScratch sc;
+    sc.xpack = reinterpret_cast<uint32_t *>(base);
+    sc.partial = reinterpret_cast<float *>(base + xb);
+    sc.arrived = reinterpret_cast<uint32_t *>(base + xb + pb);
+    sc.partial_floats = p.partial_floats;
+    return run_matmul(compressed, codebook, x, out, m, n, batch, S, bits, carry_mode, sc, p, dev, stream, ms);
 }

@@ -26,17 +26,9 @@
 #include "hadamard_pass.hpp"
 #include "rptc_common.hpp"
 
-// Development hook: a probe build defines RPTC_STAMP to record a per-wave timestamp at each phase.
-#ifndef RPTC_STAMP
-#define RPTC_STAMP(slot) ((void)0)
-#endif
-
 namespace rptc {
 
-#ifndef RPTC_MATVEC_THREADS
-#define RPTC_MATVEC_THREADS 1024
-#endif
-constexpr int kMatvecThreads = RPTC_MATVEC_THREADS;
+constexpr int kMatvecThreads = 1024;
 constexpr int kXRegs = 2048 / kMatvecThreads;   // activation registers per thread: vectors of up to 16384 halves
 constexpr int kMatvecWaves = kMatvecThreads / kWave;
 constexpr int kTableBytes = 256 * 256;     // 256 rows of 64 lane copies of one half2
@@ -233,7 +225,6 @@ __device__ __forceinline__ void matvec_body(
     // it has arrived: measured slower on every shape.
     constexpr int kBatch = 1;
     extern __shared__ uint32_t lds[];
-    RPTC_STAMP(0);
     const int m = a.m, n = a.n;
     const int T = n >> 11, Lt = (n & 2047) >> 6, npr = n >> 6, n8 = n >> 3;
     uint32_t *sx = lds + kTableBytes / 4;                  // activation pairs, slot order
@@ -421,7 +412,6 @@ __device__ __forceinline__ void matvec_body(
     };
     static_assert(kBatch == 1, "the load cursor stands at the one item the first request asked for");
     load_first();
-    RPTC_STAMP(1);
 
     // the element-wise step in front of the product, on the registers the small loads filled
     if constexpr (XMODE == kXSiluMul) {
@@ -552,7 +542,6 @@ __device__ __forceinline__ void matvec_body(
             stage_x(idx, XMODE == kXSiluMul ? silu_mul8(x[idx], x[n8 + idx]) : x[idx]);
     }
     __syncthreads();
-    RPTC_STAMP(2);
     if constexpr (AFFINE) {
         // the two sums are needed when the row sums are written: their reduction runs beside the decode,
         // not in front of the barrier every wave waits at
@@ -641,7 +630,6 @@ __device__ __forceinline__ void matvec_body(
                 typedef __attribute__((address_space(3))) float lds_float;
                 *reinterpret_cast<lds_float *>(static_cast<uintptr_t>(part_lane + 4u * (uint32_t)(row_first * pstride))) = sum;
             }
-            if (base + u == it_begin) RPTC_STAMP(3);
             if (++idx == sv.items) {
                 idx = 0;
                 slab++;
@@ -668,7 +656,6 @@ __device__ __forceinline__ void matvec_body(
         if (base + kBatch < it_end) load_batch(base + kBatch);
         decode_batch(cur, ccw, base);
     }
-    RPTC_STAMP(4);
     __syncthreads();
     if constexpr (AFFINE) {
         // one pair per lane and sums across the lanes; the totals are the same for every lane
@@ -689,7 +676,6 @@ __device__ __forceinline__ void matvec_body(
         }
         if (lane == 63) out[row0 + r] = float_to_half_bits(y);
     }
-    RPTC_STAMP(5);
 }
 
 template <int S, int MODE, int BITS, bool COMPACT>

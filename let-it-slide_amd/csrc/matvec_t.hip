@@ -121,21 +121,22 @@ __global__ __launch_bounds__(kTThreads) void matvec_t_kernel(
         if (tid < kWave && valid) out[row] = float_to_half_bits(half_bits_to_float(out[row]) + y);
         return;
     }
-    // Device-scope stores and loads bypass the XCD-private cache levels, so the only ordering needed
-    // is that this workgroup's stores have completed before its arrival is counted.
+    // Release / acquire at agent scope: the storing threads release their partial sums before the barrier lets
+    // thread 0 count the arrival (an acquire-release read-modify-write), and the workgroup that sees the last
+    // arrival acquires before it reads the other workgroups' sums, whichever XCD they ran on.
     if (tid < kWave) __hip_atomic_store(&parts[(size_t)blockIdx.x * kWave + tid], y, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    __builtin_amdgcn_s_waitcnt(0);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
     __syncthreads();
     uint32_t *flag = reinterpret_cast<uint32_t *>(part);
     if (tid == 0) {
-        const uint32_t prev = __hip_atomic_fetch_add(&arrived[rb], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const uint32_t prev = __hip_atomic_fetch_add(&arrived[rb], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
         const bool last = prev == (uint32_t)(ksplit - 1);
         if (last) __hip_atomic_store(&arrived[rb], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // for the next launch
         *flag = last;
     }
     __syncthreads();
     if (!*flag || tid >= kWave || !valid) return;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
     float p[kTMaxSplit];
 #pragma unroll
     for (int i = 0; i < kTMaxSplit; i++)
@@ -244,6 +245,12 @@ static int launch_t_dense(const int32_t *compressed, const uint16_t *codebook, u
         hipLaunchKernelGGL((matvec_t_dense_kernel<L, RPTC_CONTINUOUS>), grid, dim3(256), 0, s, a_comp, codebook, a_w,
                            (int)m, (int)(n / 64));
     return 0;
+}
+
+void matvec_t_counters(int device, uint32_t **counters, int *count)
+{
+    *counters = g_t[device].arrived;
+    *count = kTMaxParts;
 }
 
 int prepare_matvec_t(int device)

@@ -66,6 +66,9 @@ _SIGNATURES = {
     "rptc_matvec_t_dense": ([_VP, _VP, _VP, _I64, _I64, _INT, _INT, _VP, _FP], _INT),
     "rptc_decompress_matmul": ([_VP, _VP, _VP, _VP, _I64, _I64, _I64, _INT, _INT, _VP, _FP], _INT),
     "rptc_decompress_matmul_bits": ([_VP, _VP, _VP, _VP, _I64, _I64, _I64, _INT, _INT, _INT, _VP, _FP], _INT),
+    "rptc_decompress_matmul_workspace_bytes": ([_I64, _I64, _I64, _INT], _I64),
+    "rptc_decompress_matmul_ws": ([_VP, _VP, _VP, _VP, _I64, _I64, _I64, _INT, _INT, _INT, _VP, _I64, _VP, _FP], _INT),
+    "rptc_scratch_check": ([_INT, ctypes.POINTER(ctypes.c_int), _VP], _INT),
     "rptc_viterbi_scratch_bytes": ([_I64, _I64], _I64),
     "rptc_viterbi_scalar_scratch_bytes": ([_I64, _I64], _I64),
     "rptc_viterbi_scalar": ([_VP, _VP, _I64, _VP, _INT, _VP, _VP, _VP, _VP, _I64, _I64, _VP, _FP], _INT),
@@ -79,8 +82,6 @@ _SIGNATURES = {
     "rptc_attn_decode": ([_VP, _VP, _VP, _VP, _VP, _I64, _I64, _I64, _VP], _INT),
     "rptc_silu_mul": ([_VP, _VP, _I64, _VP], _INT),
     "rptc_greedy_next": ([_VP, _I64, _VP, _I64, _VP, _VP, _VP, _VP, _VP, _VP], _INT),
-    "rptc_probe_empty": ([_VP], _INT),
-    "rptc_probe_read": ([_VP, _I64, _VP, _VP], _INT),
     "rptc_rope_attn_decode": ([_VP, _VP, _VP, _VP, _VP, _VP, _VP, _I64, _I64, _I64, _VP], _INT),
     "rptc_decompress_matvec_silu": ([_VP, _VP, _VP, _VP, _I64, _I64, _INT, _INT, _VP, _FP], _INT),
     "rptc_decompress_matvec_hadamard": ([_VP, _VP, _VP, _VP, _VP, _I64, _I64, _I64, _INT, _INT, _VP, _FP], _INT),
@@ -156,7 +157,9 @@ def _status(rc):
         raise RuntimeError(f"rptc_kernels: {text} (status {rc})")
 
 
-def _call(fn, tensors, *args, carry_mode=None):
+def _call(fn, tensors, *args, carry_mode=None, timed=None):
+    """timed: None = the module-wide setting (``set_timing``); False = this call passes a NULL ``ms`` pointer and
+    is asynchronous whatever the setting (what a layer inside a model wants: no global is touched)."""
     device = tensors[0].device
     for t in tensors[1:]:
         _check(t.device == device, "all tensors must be on the same device")
@@ -165,7 +168,7 @@ def _call(fn, tensors, *args, carry_mode=None):
     with torch.cuda.device(device):
         stream = torch.cuda.current_stream().cuda_stream
         rc = fn(*[t.data_ptr() for t in tensors], *args, mode, ctypes.c_void_p(stream),
-                ctypes.byref(ms) if _timing else None)
+                ctypes.byref(ms) if (_timing if timed is None else timed) else None)
     _status(rc)
     return float(ms.value)
 
@@ -359,7 +362,7 @@ def hadamard_block(n):
     return p
 
 
-def sign_hadamard(x, signs, out, block=0, inverse=False):
+def sign_hadamard(x, signs, out, block=0, inverse=False, timed=None):
     """Blockwise random-sign Hadamard transform of the rows of x ([n] or [batch, n], fp16).
 
     forward: out = H (signs * x) / sqrt(block); inverse: out = signs * (H x) / sqrt(block), per block of
@@ -382,7 +385,7 @@ def sign_hadamard(x, signs, out, block=0, inverse=False):
         stream = torch.cuda.current_stream().cuda_stream
         rc = library().rptc_sign_hadamard(x.data_ptr(), signs.data_ptr(), out.data_ptr(), batch, n, p,
                                           1 if inverse else 0, ctypes.c_void_p(stream),
-                                          ctypes.byref(ms) if _timing else None)
+                                          ctypes.byref(ms) if (_timing if timed is None else timed) else None)
     _status(rc)
     return float(ms.value)
 
@@ -563,18 +566,19 @@ def _affine_ptrs(n, m, scales_in, biases_in, scales_out, biases_out):
     return ptrs
 
 
-def _call_affine(fn, head, tail, device, carry_mode):
+def _call_affine(fn, head, tail, device, carry_mode, timed=None):
     ms = ctypes.c_float(0.0)
     mode = _carry_mode if carry_mode is None else carry_mode
     with torch.cuda.device(device):
         stream = torch.cuda.current_stream().cuda_stream
-        rc = fn(*head, *tail, mode, ctypes.c_void_p(stream), ctypes.byref(ms) if _timing else None)
+        rc = fn(*head, *tail, mode, ctypes.c_void_p(stream),
+                ctypes.byref(ms) if (_timing if timed is None else timed) else None)
     _status(rc)
     return float(ms.value)
 
 
 def decompress_matvec_affine(compressed, codebook, x, out, scales_in=None, biases_in=None, scales_out=None,
-                             biases_out=None, carry_mode=None):
+                             biases_out=None, carry_mode=None, timed=None):
     """out = scales_out * (W_hat (scales_in * x)) + biases_out * sum(x) + biases_in . x: the product with the
     matrix the reference's quantizer reconstructs, W = b_out + b_in + s_out * s_in * W_hat
     (quantize_hf.py:167), in one launch.  The four vectors are fp16 ([n], [n], [m], [m]) or None; n <= 16384.
@@ -586,7 +590,7 @@ def decompress_matvec_affine(compressed, codebook, x, out, scales_in=None, biase
     aff = _affine_ptrs(n, m, scales_in, biases_in, scales_out, biases_out)
     return _call_affine(library().rptc_decompress_matvec_affine,
                         (compressed.data_ptr(), codebook.data_ptr(), x.data_ptr(), *aff, out.data_ptr()), (m, n, S),
-                        compressed.device, carry_mode)
+                        compressed.device, carry_mode, timed)
 
 
 def decompress_matvec_silu_affine(compressed, codebook, gate_up, out, scales_in=None, biases_in=None, scales_out=None,

@@ -38,6 +38,9 @@ class QuantizedLinear(torch.nn.Module):
         words = out_features * in_features * bits // 32
         self.register_buffer("compressed", torch.zeros(words, dtype=torch.int32, device=device))
         self.register_buffer("codebook", torch.zeros(2 << S, dtype=torch.float16, device=device))
+        # Optional vectors: registered as None, so ``state_dict`` only holds the ones that are set, and
+        # ``load_state_dict`` into a fresh layer restores them only if the layer first gets buffers of the right
+        # shape (``set_affine`` / ``set_signs`` with placeholders); ``from_*`` constructors are the usual way.
         for name in ("scales_out", "scales_in", "biases_out", "biases_in", "signs"):
             self.register_buffer(name, None)
 
@@ -134,13 +137,13 @@ class QuantizedLinear(torch.nn.Module):
         lib = rk.library()
         if batch == 1:
             rk._call(lib.rptc_decompress_matvec_bits, (self.compressed, self.codebook, x2, out), self.out_features,
-                     self.in_features, self.S, self.bits, carry_mode=self.carry_mode)
+                     self.in_features, self.S, self.bits, carry_mode=self.carry_mode, timed=False)
             return out
         for b0 in range(0, batch, 32):
             xb = x2[b0:b0 + 32]
             ob = out[b0:b0 + 32]
             rk._call(lib.rptc_decompress_matmul_bits, (self.compressed, self.codebook, xb, ob), self.out_features,
-                     self.in_features, xb.size(0), self.S, self.bits, carry_mode=self.carry_mode)
+                     self.in_features, xb.size(0), self.S, self.bits, carry_mode=self.carry_mode, timed=False)
         return out
 
     def forward(self, x):
@@ -154,36 +157,21 @@ class QuantizedLinear(torch.nn.Module):
                 and any(v is not None for v in affine)):
             # one token: scales and biases are applied inside the mat-vec
             y = torch.empty((1, self.out_features), dtype=torch.float16, device=x2.device)
-            prev = rk.set_timing(False)
-            try:
-                rk.decompress_matvec_affine(self.compressed, self.codebook, x2[0], y[0], *affine, carry_mode=self.carry_mode)
-            finally:
-                rk.set_timing(prev)
+            rk.decompress_matvec_affine(self.compressed, self.codebook, x2[0], y[0], *affine, carry_mode=self.carry_mode,
+                                        timed=False)
             return y.reshape(shape[:-1] + (self.out_features,))
         xs = x2 * self.scales_in if self.scales_in is not None else x2
         if self.signs is not None and xs.size(0) == 1 and self.bits == 2 and self.in_features <= 15360:
             # one token: the transform runs in the prologue of the mat-vec
             y = torch.empty((1, self.out_features), dtype=torch.float16, device=xs.device)
-            prev = rk.set_timing(False)
-            try:
-                rk._call(rk.library().rptc_decompress_matvec_hadamard, (self.compressed, self.codebook, xs, self.signs, y),
-                         self.out_features, self.in_features, 0, self.S, carry_mode=self.carry_mode)
-            finally:
-                rk.set_timing(prev)
+            rk._call(rk.library().rptc_decompress_matvec_hadamard, (self.compressed, self.codebook, xs, self.signs, y),
+                     self.out_features, self.in_features, 0, self.S, carry_mode=self.carry_mode, timed=False)
             return self._epilogue(y, x2, shape)
         if self.signs is not None:
             t = torch.empty_like(xs)
-            prev = rk.set_timing(False)
-            try:
-                rk.sign_hadamard(xs, self.signs, t)
-            finally:
-                rk.set_timing(prev)
+            rk.sign_hadamard(xs, self.signs, t, timed=False)
             xs = t
-        prev = rk.set_timing(False)
-        try:
-            y = self._product(xs)
-        finally:
-            rk.set_timing(prev)
+        y = self._product(xs)
         return self._epilogue(y, x2, shape)
 
     def _epilogue(self, y, x2, shape):
@@ -200,12 +188,8 @@ class QuantizedLinear(torch.nn.Module):
     def decoded_weight(self):
         """W_hat, fp16 [m, n], bit-exact decode of the stream."""
         W = torch.empty((self.out_features, self.in_features), dtype=torch.float16, device=self.compressed.device)
-        prev = rk.set_timing(False)
-        try:
-            rk._call(rk.library().rptc_matvec_bits_dense, (self.compressed, self.codebook, W), self.out_features,
-                     self.in_features, self.S, self.bits, carry_mode=self.carry_mode)
-        finally:
-            rk.set_timing(prev)
+        rk._call(rk.library().rptc_matvec_bits_dense, (self.compressed, self.codebook, W), self.out_features,
+                 self.in_features, self.S, self.bits, carry_mode=self.carry_mode, timed=False)
         return W
 
     def reconstructed_weight(self):

@@ -122,6 +122,9 @@ class QuantizedLlama(torch.nn.Module):
         them with ``half_logits``).  ``input_ready``: the token's embedding row is already in the decoder's
         input buffer (``rptc_greedy_next`` put it there), so it is not gathered again.
 
+        The position must be below ``shape.max_len``: it lives on the device, so it is not checked here
+        (``greedy_decode`` checks its whole range up front; the kernels skip a position outside the caches).
+
         ``fuse`` (default): five launches per layer - the qkv and gate/up projections do the residual add and
         RMS norm in their prologue, the down projection the SiLU gate, and one kernel rotates q and k, appends
         to the cache and attends.  ``fuse=False``: the same arithmetic as nine launches per layer."""
@@ -223,6 +226,17 @@ class QuantizedLlama(torch.nn.Module):
         return logits if half_logits else logits.float()
 
 
+def check_context(shape, prompt_len, new_tokens):
+    """The caches and the rotary tables hold ``shape.max_len`` positions; the last token generated is never fed
+    back, so positions 0 .. prompt_len + new_tokens - 2 are written.  Raises ValueError when they do not fit
+    (the kernels themselves skip a position outside the caches rather than write out of bounds)."""
+    if prompt_len < 1 or new_tokens < 1:
+        raise ValueError("the prompt and the number of new tokens must be at least 1")
+    if prompt_len + new_tokens - 1 > shape.max_len:
+        raise ValueError(f"prompt of {prompt_len} tokens + {new_tokens} new tokens needs {prompt_len + new_tokens - 1} "
+                         f"cache positions, the model was built with max_len = {shape.max_len}")
+
+
 def greedy_decode(model, prompt, new_tokens, mode="fused_graph"):
     """Prefill the prompt (in chunks of 32 tokens: the batch the fused mat-mat kernel takes), then decode
     ``new_tokens`` greedily one at a time.  mode: "fused_graph" (five launches per layer, one HIP graph per
@@ -232,6 +246,7 @@ def greedy_decode(model, prompt, new_tokens, mode="fused_graph"):
     dev = model.embed.device
     prompt = torch.as_tensor(prompt, dtype=torch.long, device=dev)
     P = prompt.numel()
+    check_context(model.shape, P, new_tokens)
     if mode.startswith("fused"):
         step = model.decode_step
     elif mode.startswith("glue"):

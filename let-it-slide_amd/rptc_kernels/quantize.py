@@ -165,7 +165,8 @@ def dequantize_symbols(symbols, codebook, S=8, bits=2):
 
 
 def factorize(W, iterations=64):
-    """The reference's row/column factorisation W = b_out + b_in + s_out * s_in * N (quantize_hf.py:77-117):
+    """The reference's row/column factorisation W = b_out + b_in + s_out * s_in * N, transliterated from
+    quantize_hf.py:77-117 (jax.numpy -> torch, statement for statement, so that the iteration is the same):
     64 rounds of alternately re-estimating the biases (means of the scaled residual) and the scales (RMS of
     the residual), each followed by the balancing step that keeps the two biases' means and the two scales'
     geometric means equal.  W float [out, in] on any device.  Returns (b_out [out, 1], b_in [1, in],
@@ -247,11 +248,13 @@ def quantize_layer(W, hessian_diag=None, L=16, banks=32, seed=0):
 
 
 def evaluate_layer(W, recon, hessian_diag=None):
-    """Relative errors of a reconstruction (quantize_hf.py:173-187): Frobenius, and weighted by the Hessian
-    diagonal when one is given."""
+    """Errors of a reconstruction as the reference reports them (quantize_hf.py:172-185): ``frob`` =
+    sum(E^2) / sqrt(sum(W^2)) (the reference divides the squared error by the NORM of W, not by its square,
+    so the figure scales with ||W||), and ``proxy_diag`` = sum(E^2 h) / sum(W^2 h) with h the Hessian
+    diagonal when one is given.  ``frob_rel`` = sum(E^2) / sum(W^2) is this library's addition (scale-free)."""
     W = torch.as_tensor(W).to(torch.float32)
     E = W - recon.to(W.device)
-    res = {"frob": float((E ** 2).sum() / (W ** 2).sum())}
+    res = {"frob": float((E ** 2).sum() / (W ** 2).sum().sqrt()), "frob_rel": float((E ** 2).sum() / (W ** 2).sum())}
     if hessian_diag is not None:
         h = torch.as_tensor(hessian_diag, dtype=torch.float32, device=W.device).reshape(1, -1)
         res["proxy_diag"] = float(((E * h) * E).sum() / ((W * h) * W).sum())

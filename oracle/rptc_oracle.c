@@ -24,9 +24,16 @@
  *   orc_matvec_dense      same
  *   orc_matvec_t          brute-force numpy restatement; closed form of the
  *                         as-written nibble rule
- *   orc_lite_index_fn /   hand-computed known answers; PARITY UNPINNED beyond
- *   orc_lite_dequantize   those (the reference holds no vectors and its
- *                         Python needs jax, which is not installed)
+ *   orc_lite_index_fn     hand-computed known answers; every state of a 16-bit
+ *                         register, every 16-bit pattern at the top of the
+ *                         word and a sample of the int32 range against an
+ *                         element-wise int32-array evaluation (wrapping
+ *                         product, arithmetic shift: the semantics of the
+ *                         reference's jax int32)
+ *   orc_lite_dequantize   the unmasked int32 register is a window of L bits
+ *                         (bits above L never reach the index: tested), so the
+ *                         output equals alphabet[index of the last L stream
+ *                         bits] over sequences that wrap the register
  *   orc_viterbi           exhaustive enumeration of every symbol sequence on
  *                         trellises small enough for it (optimal cost, and the
  *                         returned path has that cost); the tie rules are

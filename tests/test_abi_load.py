@@ -91,7 +91,6 @@ def test_c_abi_rejects_bad_arguments_before_touching_a_device():
     assert lib.rptc_decompress_matvec_hadamard(16, 16, 16, 16, 16, 32, 16384, 0, 8, 0, None, None) == -5   # n > 15360
     assert lib.rptc_rope_attn_decode(16, 16, 16, 16, 16, 16, 16, 4, 48, 128, None) == -2         # head_dim not a power of two
     assert lib.rptc_attn_decode(16, 16, 16, None, 16, 4, 64, 128, None) == -1
-    assert lib.rptc_probe_read(16, 100, None, None) == -2
     assert lib.rptc_viterbi_pairs(16, None, 0, 16, 16, 16, 16, 16, 4, 64, 7, None, None) == -2    # S
     assert lib.rptc_viterbi_pairs(16, None, 0, 16, None, 16, 16, 16, 4, 64, 8, None, None) == -1  # no scratch
     assert lib.rptc_viterbi_pairs(16, 16, 100, 16, 16, 16, 16, 16, 4, 64, 8, None, None) == -2    # weight stride < 2 * steps

@@ -588,3 +588,74 @@ def test_rope_attn_decode_equals_rope_then_attention(rk, heads, hd, max_len, pos
     sc = torch.einsum("hd,hsd->hs", q.view(heads, hd).double(), kk) / hd ** 0.5
     want = torch.einsum("hs,hsd->hd", torch.softmax(sc, dim=-1), vv).reshape(-1)
     assert rel_l2(o2.float().cpu().numpy(), want.cpu().numpy()) < 2e-3
+
+
+@pytest.mark.parametrize("quantize_init", [False, True])
+def test_llama_2_7b_shaped_layer_at_position_600(rk, quantize_init):
+    """One decoder layer at the Llama-2-7B shape (d 4096, 32 heads x 128, MLP 11008, vocabulary 32000), one token at
+    position 600 over a cache of 600 seeded rows: the five-launch fused step (12288x4096 and 22016x4096 with the
+    add + RMS norm prologue, rotation + cache append + 32-head attention, 4096x4096, 4096x11008 with the SiLU
+    prologue) against the same arithmetic in framework ops on the decoded (or reconstructed) dense weights.
+    Each projection is held to rel-L2 1e-3 on the input the fused step itself fed it; the logits to 2e-2."""
+    from rptc_kernels.llama_decode import LlamaShape, QuantizedLlama
+    shape = LlamaShape(layers=1, d_model=4096, heads=32, d_ff=11008, vocab=32000, max_len=1024)
+    model = QuantizedLlama(shape, S=8, seed=5, quantize_init=quantize_init)
+    blk = model.blocks[0]
+    d, f, pos_i = shape.d_model, shape.d_ff, 600
+    g = torch.Generator(device="cuda").manual_seed(17)
+    blk.norm1.copy_((1 + 0.1 * torch.randn(d, generator=g, device="cuda")).half())
+    blk.norm2.copy_((1 + 0.1 * torch.randn(d, generator=g, device="cuda")).half())
+    model.k_cache[:, :, :pos_i].copy_((torch.randn((1, shape.heads, pos_i, shape.head_dim), generator=g, device="cuda") * 0.5).half())
+    model.v_cache[:, :, :pos_i].copy_((torch.randn((1, shape.heads, pos_i, shape.head_dim), generator=g, device="cuda") * 0.5).half())
+    kc, vc = model.k_cache.clone(), model.v_cache.clone()
+    tok = torch.tensor([1234], device="cuda")
+    pos = torch.tensor([pos_i], device="cuda")
+
+    def dense(layer):
+        return (layer.reconstructed_weight() if quantize_init else layer.decoded_weight()).double()
+
+    with torch.no_grad():
+        logits_f = model.decode_step(tok, pos)
+        torch.cuda.synchronize()
+        x0 = model.embed[tok].reshape(-1)
+        # q, k, v: the norm of the embedding row through the fused 12288 x 4096 projection
+        h1 = model._rms(x0[None], blk.norm1)[0]
+        want = dense(blk.qkv_proj) @ h1.double()
+        assert rel_l2(model._qkv.double().cpu().numpy(), want.cpu().numpy()) < 1e-3
+        # rotation + cache append + attention, from the projection's own output
+        q, k, v = model._qkv.split(d)
+        qr = model._rope(q.reshape(1, shape.heads, shape.head_dim), pos)
+        kr = model._rope(k.reshape(1, shape.heads, shape.head_dim), pos)
+        assert torch.equal(model.k_cache[0, :, pos_i], kr[0]) and torch.equal(model.v_cache[0, :, pos_i], v.reshape(shape.heads, -1))
+        assert torch.equal(model.k_cache[0, :, :pos_i], kc[0, :, :pos_i]) and torch.equal(model.k_cache[0, :, pos_i + 1:], kc[0, :, pos_i + 1:])
+        K, V = model.k_cache[0, :, :pos_i + 1].double(), model.v_cache[0, :, :pos_i + 1].double()
+        att = torch.softmax(torch.einsum("hd,hsd->hs", qr[0].double(), K) / shape.head_dim ** 0.5, dim=-1)
+        want = torch.einsum("hs,hsd->hd", att, V).reshape(-1)
+        assert rel_l2(model._att.double().cpu().numpy(), want.cpu().numpy()) < 2e-3
+        # o projection on the attention output the step produced
+        want = dense(blk.o_proj) @ model._att.double()
+        assert rel_l2(model._o.double().cpu().numpy(), want.cpu().numpy()) < 1e-3
+        # gate / up: residual add + norm prologue of the 22016 x 4096 projection
+        x1 = x0 + model._o
+        h2 = model._rms(x1[None], blk.norm2)[0]
+        want = dense(blk.gate_up_proj) @ h2.double()
+        assert rel_l2(model._gu.double().cpu().numpy(), want.cpu().numpy()) < 1e-3
+        # down: SiLU prologue of the 4096 x 11008 projection
+        act = torch.nn.functional.silu(model._gu[:f].float()).half() * model._gu[f:]
+        want = dense(blk.down_proj) @ act.double()
+        assert rel_l2(model._down.double().cpu().numpy(), want.cpu().numpy()) < 2e-3
+
+        # the whole step against framework ops on the dense matrices
+        class Dense(torch.nn.Module):
+            def __init__(self, w):
+                super().__init__()
+                self.w = w.float()
+
+            def forward(self, x):
+                return (x.float() @ self.w.t()).half()
+
+        for name in ("qkv_proj", "o_proj", "gate_up_proj", "down_proj"):
+            setattr(blk, name, Dense(dense(getattr(blk, name))))
+        model.k_cache.copy_(kc); model.v_cache.copy_(vc)
+        logits_d = model.forward_tokens(tok, pos)
+    assert rel_l2(logits_f.cpu().numpy(), logits_d.cpu().numpy()) < 2e-2

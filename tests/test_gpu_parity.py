@@ -522,9 +522,10 @@ def test_matmul_70b_shapes_batch_16(rk, m, n):
     assert torch.equal(out.view(torch.int16), out2.view(torch.int16))
 
 
+@pytest.mark.parametrize("m,n", [(4096, 11008), (11008, 4096)])
 @pytest.mark.parametrize("batch", [8, 16, 32])
-def test_matmul_full_size_equals_decode_then_dense_gemm(rk, oracle, batch):
-    S, m, n = 8, 4096, 11008
+def test_matmul_full_size_equals_decode_then_dense_gemm(rk, oracle, batch, m, n):
+    S = 8
     comp = rand_codes(m * n // 16, seed=42)
     cb = rand_half(2 << S, seed=43)
     x = rand_half(batch * n, seed=44).reshape(batch, n)
@@ -538,6 +539,60 @@ def test_matmul_full_size_equals_decode_then_dense_gemm(rk, oracle, batch):
     y = torch.zeros((m,), dtype=torch.float16, device="cuda")
     rk.decompress_matvec_16_8_1(comp.cuda(), cb.cuda(), x[0].cuda().contiguous(), y)
     assert rel_l2(np_f16(y), want[0]) < REL_L2_TOL
+
+
+@pytest.mark.parametrize("bits", [2, 4])
+@pytest.mark.parametrize("batch", [8, 32])
+def test_matmul_with_a_caller_workspace_is_bit_identical_and_reentrant(rk, bits, batch):
+    """rptc_decompress_matmul_ws: the same kernels with the scratch in a buffer of the caller; two calls with two
+    workspaces on two streams may overlap, and each equals the static-scratch entry point bit for bit."""
+    import ctypes
+    lib = rk.library()
+    S, m, n = 8, 1024 + 48, 4096 + 768
+    comp = rand_codes(m * n * bits // 32, seed=11).cuda()
+    cb = rand_half(2 << S, seed=12).cuda()
+    xs = [rand_half(batch * n, seed=13 + i).reshape(batch, n).cuda() for i in range(2)]
+    want = [torch.zeros((batch, m), dtype=torch.float16, device="cuda") for _ in range(2)]
+    for i in range(2):
+        rk.decompress_matmul_bits(comp, cb, xs[i], want[i], bits)
+    need = lib.rptc_decompress_matmul_workspace_bytes(m, n, batch, bits)
+    assert need > 0
+    ws = [torch.full((need,), 0xA5, dtype=torch.uint8, device="cuda") for _ in range(2)]      # garbage on purpose
+    got = [torch.full((batch, m), float("nan"), dtype=torch.float16, device="cuda") for _ in range(2)]
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    torch.cuda.synchronize()
+    for rep in range(3):
+        for i in range(2):
+            rc = lib.rptc_decompress_matmul_ws(comp.data_ptr(), cb.data_ptr(), xs[i].data_ptr(), got[i].data_ptr(), m, n, batch,
+                                               S, bits, 0, ws[i].data_ptr(), need, ctypes.c_void_p(streams[i].cuda_stream), None)
+            assert rc == 0, lib.rptc_status_string(rc)
+    torch.cuda.synchronize()
+    for i in range(2):
+        assert torch.equal(got[i].view(torch.int16), want[i].view(torch.int16))
+    # too small a workspace, a misaligned one, none at all
+    assert lib.rptc_decompress_matmul_ws(comp.data_ptr(), cb.data_ptr(), xs[0].data_ptr(), got[0].data_ptr(), m, n, batch, S, bits,
+                                         0, ws[0].data_ptr(), need - 256, None, None) == -5
+    assert lib.rptc_decompress_matmul_ws(comp.data_ptr(), cb.data_ptr(), xs[0].data_ptr(), got[0].data_ptr(), m, n, batch, S, bits,
+                                         0, ws[0].data_ptr() + 16, need, None, None) == -3
+    assert lib.rptc_decompress_matmul_ws(comp.data_ptr(), cb.data_ptr(), xs[0].data_ptr(), got[0].data_ptr(), m, n, batch, S, bits,
+                                         0, None, need, None, None) == -1
+
+
+def test_arrival_counters_are_zero_after_the_split_ops(rk):
+    """rptc_scratch_check: after ops that merge across workgroups (batched product, transposed mat-vec on a short
+    matrix) every arrival counter is back at zero."""
+    import ctypes
+    lib = rk.library()
+    S, m, n, batch = 8, 512, 4096, 8
+    comp = rand_codes(m * n // 16, seed=21).cuda()
+    out = torch.zeros((batch, m), dtype=torch.float16, device="cuda")
+    rk.decompress_matmul_16_8_1(comp, rand_half(2 << S, seed=22).cuda(), rand_half(batch * n, seed=23).reshape(batch, n).cuda(), out)
+    y = torch.zeros(m, dtype=torch.float16, device="cuda")
+    rk.decompress_matvec_t_16(comp, rand_half(1 << 16, seed=24).cuda(), rand_half(n, seed=25).cuda(), y)
+    nz = ctypes.c_int(-1)
+    assert lib.rptc_scratch_check(0, ctypes.byref(nz), None) == 0
+    assert nz.value == 0
+    assert lib.rptc_scratch_check(1, None, None) == -1
 
 
 def test_matmul_rejects_bad_arguments(rk):
@@ -652,3 +707,14 @@ def test_matvec_bits_full_size(rk, bits, m, n):
     rk.matvec_bits_dense(comp, cb, W, bits)
     want = (W.double() @ x.double()).cpu().numpy()
     assert rel_l2(np_f16(out), want) < REL_L2_TOL
+    # the dense export is held to the oracle on a subset of rows taken from all over the matrix (the whole matrix
+    # at this size takes the CPU a while): a stream of just those rows has the same layout with m = rows
+    rows = np.array(sorted({0, 1, 31, 32, 33, m // 2 - 1, m // 2, m - 64, m - 2, m - 1} | set(range(1000, 1032))))
+    words = 2 * bits
+    idx = np_u32(comp).reshape(-1)
+    T, Lt = n // 2048, (n % 2048) // 64
+    parts = [idx[t * m * 32 * words:(t + 1) * m * 32 * words].reshape(m, 32 * words)[rows].reshape(-1) for t in range(T)]
+    if Lt:
+        parts.append(idx[T * m * 32 * words:].reshape(m, Lt * words)[rows].reshape(-1))
+    wantW = oracle.bits_dense(np.concatenate(parts), np_f16(cb), len(rows), n, S, bits, mode=0)
+    assert np.array_equal(np_f16(W[torch.from_numpy(rows).cuda()]).view(np.uint16), wantW.view(np.uint16))

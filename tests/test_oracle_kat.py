@@ -338,6 +338,67 @@ def test_lite_index_fn_known_answers(oracle):
         assert oracle.lite_index_fn(int(x), 16, 9) == _index_fn_python(int(x), 16, 9)
 
 
+def _index_fn_numpy_int32(x, L, S):
+    """rptc_lite.py:12-16 evaluated the way the reference evaluates it: element-wise on int32 arrays, where the
+    product wraps around and >> is an arithmetic shift (jax's default integer type is int32; numpy's int32 arrays
+    have the same two properties).  Independent of the C restatement's unsigned arithmetic and casts."""
+    x = np.asarray(x).astype(np.int32)
+    with np.errstate(over="ignore"):
+        x = x * (np.int32(2) * x + np.int32(1))
+    x = x ^ (x >> np.int32(L - S))
+    return x & np.int32((1 << S) - 1)
+
+
+@pytest.mark.parametrize("L,S", [(16, 9), (16, 8), (12, 6), (20, 10), (16, 16)])
+def test_lite_index_fn_exhaustive_against_int32_arrays(oracle, L, S):
+    """Every state of the shift register (all 2^L values, L <= 16: 65536 of them; a 2^16 sample otherwise), every
+    16-bit pattern shifted to the top of the word (negative int32 values: the arithmetic shift matters there),
+    and a random sample of the whole int32 range."""
+    states = np.arange(1 << min(L, 16), dtype=np.int64)
+    if L > 16:
+        states = rng(L).integers(0, 1 << L, 1 << 16)
+    high = (np.arange(1 << 16, dtype=np.int64) << 16) - (1 << 31)
+    anywhere = rng(S).integers(-(1 << 31), 1 << 31, 1 << 16)
+    for xs in (states, high, anywhere):
+        want = _index_fn_numpy_int32(xs, L, S)
+        got = np.array([oracle.lite_index_fn(int(x) & 0xFFFFFFFF, L, S) for x in xs], dtype=np.int32)
+        assert np.array_equal(got, want)
+        assert want.min() >= 0 and want.max() < (1 << S)
+
+
+def test_lite_index_fn_depends_on_the_low_L_bits_only(oracle):
+    """x (2x + 1) mod 2^L depends on x mod 2^L only, and the index reads bits [0, S) and [L-S, L) of the product:
+    bits of x above L never reach it.  This is why the reference's unmasked register (rptc_lite.py:65) is a
+    window of L bits."""
+    L, S = 16, 9
+    g = rng(7)
+    low = g.integers(0, 1 << L, 4096)
+    high = g.integers(0, 1 << (32 - L), 4096)
+    for lo, hi in zip(low, high):
+        assert oracle.lite_index_fn(int((hi << L) | lo), L, S) == oracle.lite_index_fn(int(lo), L, S)
+
+
+@pytest.mark.parametrize("L,S,R,V", [(16, 9, 4, 2), (16, 8, 2, 1), (12, 6, 3, 4), (16, 9, 8, 2)])
+def test_lite_dequantize_is_a_window_of_L_bits(oracle, L, S, R, V):
+    """rptc_lite.py:63-73 on sequences long enough for the int32 register to wrap many times: the output at step t
+    is alphabet[index_fn(last L stream bits)], the index taken with the int32-array evaluation above on a register
+    MASKED to L bits (which the reference never does; the property above says it changes nothing)."""
+    g = rng(L * 100 + R)
+    alphabet = g.standard_normal((1 << S, V)).astype(np.float32)
+    symbols = g.integers(0, 1 << R, 300)
+    got = oracle.lite_dequantize(alphabet, L, S, R, symbols)
+    state, want_idx = 0, []
+    for s in symbols:
+        state = ((state << R) | int(s)) & ((1 << L) - 1)
+        want_idx.append(state)
+    want = alphabet[_index_fn_numpy_int32(np.array(want_idx), L, S)]
+    assert np.array_equal(got, want)
+    # the first steps, by hand: state = s0, then (s0 << R) | s1
+    s0, s1 = int(symbols[0]), int(symbols[1])
+    assert np.array_equal(got[0], alphabet[int(_index_fn_numpy_int32([s0], L, S)[0])])
+    assert np.array_equal(got[1], alphabet[int(_index_fn_numpy_int32([(s0 << R) | s1], L, S)[0])])
+
+
 def test_lite_dequantize_window(oracle):
     L, S, R, V = 16, 9, 4, 2
     g = rng(2)

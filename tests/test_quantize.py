@@ -193,7 +193,19 @@ def test_quantize_layer_reconstructs_better_than_a_scalar_quantizer():
     res = quantize.quantize_layer(W, h, L=10, banks=2, seed=1)
     err = quantize.evaluate_layer(W, res["recon"], h)
     assert res["symbols"].shape == (out_f, in_f) and int(res["symbols"].max()) <= 3
-    assert err["frob"] < 0.12 and err["proxy_diag"] < 0.12       # 2-bit Lloyd-Max scalar quantizer: 0.1175
+    assert err["frob_rel"] < 0.12 and err["proxy_diag"] < 0.12       # 2-bit Lloyd-Max scalar quantizer: 0.1175
+
+
+def test_evaluate_layer_known_answer():
+    """quantize_hf.py:172-185 by hand: W = [[3, 4]], recon = [[2, 2]] -> E = [[1, 2]];
+    frob = (1 + 4) / sqrt(9 + 16) = 1 (the reference divides by the norm, not its square);
+    proxy_diag with h = [2, 1]: (1*2 + 4*1) / (9*2 + 16*1) = 6 / 34."""
+    W = torch.tensor([[3.0, 4.0]])
+    recon = torch.tensor([[2.0, 2.0]])
+    err = quantize.evaluate_layer(W, recon, torch.tensor([2.0, 1.0]))
+    assert err["frob"] == pytest.approx(1.0)
+    assert err["frob_rel"] == pytest.approx(5.0 / 25.0)
+    assert err["proxy_diag"] == pytest.approx(6.0 / 34.0)
 
 
 def test_sign_hadamard_rows_is_the_oracle_transform_and_orthogonal(oracle):
