@@ -696,7 +696,7 @@ def test_matvec_bits_fused_kernel_decodes_bit_exactly(rk, oracle, bits):
 
 @pytest.mark.parametrize("bits", [3, 4])
 @pytest.mark.parametrize("m,n", [(4096, 11008), (11008, 4096)])
-def test_matvec_bits_full_size(rk, bits, m, n):
+def test_matvec_bits_full_size(rk, oracle, bits, m, n):
     S = 8
     comp = rand_codes(m * n * bits // 32, seed=42).cuda()
     cb = rand_half(2 << S, seed=43).cuda()
