@@ -139,8 +139,15 @@ int rptc_matvec_t_dense(const int32_t *compressed, const uint16_t *codebook, uin
  * No counterpart in the reference, which only has the batch-1 kernels (inference.cu:189-277).
  *   x    fp16 [batch][n], batch in [1, 32], n % 64 == 0, n <= 32768
  *   out  fp16 [batch][m], overwritten
- * fp16 products accumulated in fp32 on the matrix cores, rounded once.  The call stages the
- * activations in a static device buffer: calls on different streams of one device must not overlap.
+ * fp16 products accumulated in fp32 on the matrix cores, rounded once.
+ * This is the entry point that allocates nothing: it has no counterpart in the reference and is for callers
+ * that cannot allocate device memory or bring a workspace (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  Its scratch - packed activations (2 MiB), partial tiles (32 MiB), arrival
+ * counters (128 KiB) - sits in static device arrays that each GPU the library runs on holds until the process
+ * ends; a matrix whose partial tiles exceed the 32 MiB is done in several launches, n > 32768 or batch > 32 is
+ * refused with RPTC_ELIMIT.  Every call on a device shares those arrays (the counters are cleared at the start
+ * of each call): calls that overlap on one device race, whatever their streams.  rptc_decompress_matmul_ws
+ * below is the same product with the scratch in a buffer of the caller, for calls that must overlap.
  */
 int rptc_decompress_matmul(const int32_t *compressed, const uint16_t *codebook, const uint16_t *x,
                            uint16_t *out, int64_t m, int64_t n, int64_t batch, int S, int carry_mode,
