@@ -104,6 +104,45 @@ int rptc_decompress_matvec_20_8_1(const int32_t *compressed, const uint16_t *cod
                                   int carry_mode, void *stream, float *ms);
 
 /*
+ * A chain of the mat-vecs above in ONE launch: layer k computes out_k = W_k x_k for its own stream, activations
+ * and output (the arithmetic of rptc_decompress_matvec_16_{S}_1, one codebook and one carry mode for the whole
+ * chain; 2 bits per weight; n <= 16384).  No counterpart in the reference, whose ops are one launch per layer
+ * (inference.cu:318-342).  The grid stays resident: the codebook table is built once, stream elements are
+ * requested across layer boundaries, and a wave that has finished its share of a layer starts the next one.
+ * Dependencies are found from the pointers: a layer whose activations overlap an earlier layer's output, or whose
+ * output overlaps an earlier layer's activations or output, starts when every workgroup has finished the layers in
+ * front of it (a grid-wide arrival counter); other layers overlap freely.  The result is the same, bit for bit,
+ * as `count` separate launches in order would give, except that a row's slabs are added per slab first.
+ *
+ *   rptc_chain_desc_bytes(count)   device bytes the caller provides for the chain's descriptors (< 0: status)
+ *   rptc_chain_plan(...)           checks the layers, writes the descriptors into device_desc (256-byte aligned
+ *                                  device memory; copied on `stream`, which is waited for: a set-up call, not
+ *                                  for stream capture) and fills *plan (host memory, opaque).  The plan and the
+ *                                  descriptors stay valid until the caller frees device_desc; pointers and
+ *                                  sizes of the layers are fixed in them, the contents of the buffers are not.
+ *   rptc_decompress_matvec_chain   one launch on `stream` (asynchronous unless ms != NULL); the same plan must
+ *                                  not run twice at once (the arrival counters live behind its descriptors)
+ *   rptc_chain_status              waits for `stream`, then *status = 0 when the last runs completed; bit 0: a
+ *                                  bounded wait inside the kernel ran out (the kernel exits, outputs are
+ *                                  incomplete); bit 1: an arrival counter is not zero (plan again to clear)
+ */
+typedef struct rptc_chain_layer {
+    const int32_t *compressed;     /* the stream of rptc_decompress_matvec_16_{S}_1 for m x n */
+    const uint16_t *x;             /* fp16 [n] */
+    uint16_t *out;                 /* fp16 [m], overwritten */
+    int64_t m, n;
+} rptc_chain_layer;
+typedef struct rptc_chain_t {
+    uint64_t opaque[10];
+} rptc_chain_t;
+int64_t rptc_chain_desc_bytes(int64_t count);
+int rptc_chain_plan(const rptc_chain_layer *layers, int64_t count, void *device_desc, int64_t device_desc_bytes,
+                    rptc_chain_t *plan, void *stream);
+int rptc_decompress_matvec_chain(const rptc_chain_t *plan, const uint16_t *codebook, int S, int carry_mode,
+                                 void *stream, float *ms);
+int rptc_chain_status(const rptc_chain_t *plan, int *status, void *stream);
+
+/*
  * Fused decode + mat-vec on the column-interleaved stream with a scalar 2^L codebook.
  * Replace `float decompress_matvec_t_{16,14}(Tensor& compressed, Tensor& codebook, Tensor& x,
  * Tensor& out)` (inference_t.cu:178-268, kernel inference_t.cu:68-175; bound at

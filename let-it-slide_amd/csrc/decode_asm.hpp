@@ -75,49 +75,63 @@ namespace rptc {
 // a0..a3 receive four partial sums of the element's 32 products (they are written, not added to).
 // The 16 bits in front of the element are the end of the previous lane's last word, except in the
 // lanes of `first_lanes` (the first element of a row), which take the end of `own`.
-__device__ __forceinline__ void decode_element_asm(const uint4 e, const uint32_t own, const uint64_t first_lanes,
+// WAIT_VMCNT >= 0: the block starts with s_waitcnt vmcnt(WAIT_VMCNT).  For a caller that issued the load of `e`
+// (and `own`) by hand and has not touched those registers since: nothing outside this block then reads them
+// before they have arrived.
+#define RPTC_DECODE_BODY                                                                              \
+        /* a DPP operand must not have been written by a vector op in the two instructions before */ \
+        "s_nop 1\n"                                                                                   \
+        "s_mov_b64 vcc, %[first]\n"                                                                   \
+        "v_cndmask_b32_dpp %[cy], %[ew], %[own], vcc wave_shr:1 row_mask:0xf bank_mask:0xf bound_ctrl:1\n" \
+        RPTC_WINDOWS(12) RPTC_READS_X(RPTC_TA)                                                        \
+        RPTC_WINDOWS(8) RPTC_READS_X(RPTC_TB)                                                         \
+        "s_waitcnt lgkmcnt(8)\n"                                                                      \
+        RPTC_DOTS_FIRST_X(RPTC_TA, "x28", "x0", "x16", "x4", "x20", "x8", "x24", "x12")               \
+        RPTC_WINDOWS(4) RPTC_READS_X(RPTC_TA)                                                         \
+        "s_waitcnt lgkmcnt(8)\n"                                                                      \
+        RPTC_DOTS_X(RPTC_TB, "x29", "x1", "x17", "x5", "x21", "x9", "x25", "x13")                     \
+        RPTC_WINDOWS_SH0 RPTC_READS_X(RPTC_TB)                                                        \
+        "s_waitcnt lgkmcnt(8)\n"                                                                      \
+        RPTC_DOTS_X(RPTC_TA, "x30", "x2", "x18", "x6", "x22", "x10", "x26", "x14")                    \
+        "s_waitcnt lgkmcnt(0)\n"                                                                      \
+        RPTC_DOTS_X(RPTC_TB, "x31", "x3", "x19", "x7", "x23", "x11", "x27", "x15")                    \
+        /* a dot product's result must not be read by another kind of VALU op for 3 wait states, */  \
+        /* and the compiler cannot see inside this block */                                          \
+        "s_nop 3\n"
+#define RPTC_DECODE_OUTPUTS                                                                           \
+          [a0] "=&v"(a0), [a1] "=&v"(a1), [a2] "=&v"(a2), [a3] "=&v"(a3),                             \
+          [cy] "=&v"(carry), [g0] "=&v"(g0), [g1] "=&v"(g1), [g2] "=&v"(g2), [g3] "=&v"(g3),          \
+          [t0] "=&v"(t0), [t1] "=&v"(t1), [t2] "=&v"(t2), [t3] "=&v"(t3),                             \
+          [t4] "=&v"(t4), [t5] "=&v"(t5), [t6] "=&v"(t6), [t7] "=&v"(t7),                             \
+          [u0] "=&v"(u0), [u1] "=&v"(u1), [u2] "=&v"(u2), [u3] "=&v"(u3),                             \
+          [u4] "=&v"(u4), [u5] "=&v"(u5), [u6] "=&v"(u6), [u7] "=&v"(u7)
+#define RPTC_DECODE_INPUTS                                                                            \
+          [ex] "v"(e.x), [ey] "v"(e.y), [ez] "v"(e.z), [ew] "v"(e.w), [own] "v"(own), [first] "s"(first_lanes), \
+          [lane4] "v"(lane4), [mask] "s"(0xFF00u), [sel] "s"(0x0C0C0700u),                            \
+          [x0] "v"(xr[0]), [x1] "v"(xr[1]), [x2] "v"(xr[2]), [x3] "v"(xr[3]),                         \
+          [x4] "v"(xr[4]), [x5] "v"(xr[5]), [x6] "v"(xr[6]), [x7] "v"(xr[7]),                         \
+          [x8] "v"(xr[8]), [x9] "v"(xr[9]), [x10] "v"(xr[10]), [x11] "v"(xr[11]),                     \
+          [x12] "v"(xr[12]), [x13] "v"(xr[13]), [x14] "v"(xr[14]), [x15] "v"(xr[15]),                 \
+          [x16] "v"(xr[16]), [x17] "v"(xr[17]), [x18] "v"(xr[18]), [x19] "v"(xr[19]),                 \
+          [x20] "v"(xr[20]), [x21] "v"(xr[21]), [x22] "v"(xr[22]), [x23] "v"(xr[23]),                 \
+          [x24] "v"(xr[24]), [x25] "v"(xr[25]), [x26] "v"(xr[26]), [x27] "v"(xr[27]),                 \
+          [x28] "v"(xr[28]), [x29] "v"(xr[29]), [x30] "v"(xr[30]), [x31] "v"(xr[31])
+
+template <int WAIT_VMCNT = -1, typename E>
+__device__ __forceinline__ void decode_element_asm(const E &e, const uint32_t own, const uint64_t first_lanes,
                                                    const uint32_t lane4, const uint32_t (&xr)[32], float &a0,
                                                    float &a1, float &a2, float &a3)
 {
     uint32_t carry;
     uint32_t g0, g1, g2, g3, t0, t1, t2, t3, t4, t5, t6, t7, u0, u1, u2, u3, u4, u5, u6, u7;
-    asm volatile(
-        // a DPP operand must not have been written by a vector op in the two instructions before
-        "s_nop 1\n"
-        "s_mov_b64 vcc, %[first]\n"
-        "v_cndmask_b32_dpp %[cy], %[ew], %[own], vcc wave_shr:1 row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
-        RPTC_WINDOWS(12) RPTC_READS_X(RPTC_TA)
-        RPTC_WINDOWS(8) RPTC_READS_X(RPTC_TB)
-        "s_waitcnt lgkmcnt(8)\n"
-        RPTC_DOTS_FIRST_X(RPTC_TA, "x28", "x0", "x16", "x4", "x20", "x8", "x24", "x12")
-        RPTC_WINDOWS(4) RPTC_READS_X(RPTC_TA)
-        "s_waitcnt lgkmcnt(8)\n"
-        RPTC_DOTS_X(RPTC_TB, "x29", "x1", "x17", "x5", "x21", "x9", "x25", "x13")
-        RPTC_WINDOWS_SH0 RPTC_READS_X(RPTC_TB)
-        "s_waitcnt lgkmcnt(8)\n"
-        RPTC_DOTS_X(RPTC_TA, "x30", "x2", "x18", "x6", "x22", "x10", "x26", "x14")
-        "s_waitcnt lgkmcnt(0)\n"
-        RPTC_DOTS_X(RPTC_TB, "x31", "x3", "x19", "x7", "x23", "x11", "x27", "x15")
-        // a dot product's result must not be read by another kind of VALU op for 3 wait states,
-        // and the compiler cannot see inside this block
-        "s_nop 3\n"
-        : [a0] "=&v"(a0), [a1] "=&v"(a1), [a2] "=&v"(a2), [a3] "=&v"(a3),
-          [cy] "=&v"(carry), [g0] "=&v"(g0), [g1] "=&v"(g1), [g2] "=&v"(g2), [g3] "=&v"(g3),
-          [t0] "=&v"(t0), [t1] "=&v"(t1), [t2] "=&v"(t2), [t3] "=&v"(t3),
-          [t4] "=&v"(t4), [t5] "=&v"(t5), [t6] "=&v"(t6), [t7] "=&v"(t7),
-          [u0] "=&v"(u0), [u1] "=&v"(u1), [u2] "=&v"(u2), [u3] "=&v"(u3),
-          [u4] "=&v"(u4), [u5] "=&v"(u5), [u6] "=&v"(u6), [u7] "=&v"(u7)
-        : [ex] "v"(e.x), [ey] "v"(e.y), [ez] "v"(e.z), [ew] "v"(e.w), [own] "v"(own), [first] "s"(first_lanes),
-          [lane4] "v"(lane4), [mask] "s"(0xFF00u), [sel] "s"(0x0C0C0700u),
-          [x0] "v"(xr[0]), [x1] "v"(xr[1]), [x2] "v"(xr[2]), [x3] "v"(xr[3]),
-          [x4] "v"(xr[4]), [x5] "v"(xr[5]), [x6] "v"(xr[6]), [x7] "v"(xr[7]),
-          [x8] "v"(xr[8]), [x9] "v"(xr[9]), [x10] "v"(xr[10]), [x11] "v"(xr[11]),
-          [x12] "v"(xr[12]), [x13] "v"(xr[13]), [x14] "v"(xr[14]), [x15] "v"(xr[15]),
-          [x16] "v"(xr[16]), [x17] "v"(xr[17]), [x18] "v"(xr[18]), [x19] "v"(xr[19]),
-          [x20] "v"(xr[20]), [x21] "v"(xr[21]), [x22] "v"(xr[22]), [x23] "v"(xr[23]),
-          [x24] "v"(xr[24]), [x25] "v"(xr[25]), [x26] "v"(xr[26]), [x27] "v"(xr[27]),
-          [x28] "v"(xr[28]), [x29] "v"(xr[29]), [x30] "v"(xr[30]), [x31] "v"(xr[31])
-        : "vcc");
+    if constexpr (WAIT_VMCNT >= 0) {
+        asm volatile("s_waitcnt vmcnt(%[vm])\n" RPTC_DECODE_BODY
+                     : RPTC_DECODE_OUTPUTS
+                     : RPTC_DECODE_INPUTS, [vm] "n"(WAIT_VMCNT)
+                     : "vcc", "memory");
+    } else {
+        asm volatile(RPTC_DECODE_BODY : RPTC_DECODE_OUTPUTS : RPTC_DECODE_INPUTS : "vcc");
+    }
 }
 
 // The same block for 4 bits per weight: a step consumes 8 stream bits, an element is 8 words, and the

@@ -50,6 +50,18 @@ _timing = True
 _VP, _I64, _INT = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
 _FP = ctypes.POINTER(ctypes.c_float)
 
+
+
+class ChainLayer(ctypes.Structure):
+    """rptc_chain_layer of include/rptc_hip.h."""
+    _fields_ = [("compressed", _VP), ("x", _VP), ("out", _VP), ("m", _I64), ("n", _I64)]
+
+
+class ChainPlan(ctypes.Structure):
+    """rptc_chain_t of include/rptc_hip.h (opaque)."""
+    _fields_ = [("opaque", ctypes.c_uint64 * 10)]
+
+
 _MATVEC_ARGS = [_VP, _VP, _VP, _VP, _I64, _I64, _INT, _VP, _FP]
 _SIGNATURES = {
     "rptc_version": ([], _INT),
@@ -62,6 +74,10 @@ _SIGNATURES = {
     "rptc_decompress_matvec_20_8_1": (_MATVEC_ARGS, _INT),
     "rptc_decompress_matvec_t_16": (_MATVEC_ARGS, _INT),
     "rptc_decompress_matvec_t_14": (_MATVEC_ARGS, _INT),
+    "rptc_chain_desc_bytes": ([_I64], _I64),
+    "rptc_chain_plan": ([ctypes.POINTER(ChainLayer), _I64, _VP, _I64, ctypes.POINTER(ChainPlan), _VP], _INT),
+    "rptc_decompress_matvec_chain": ([ctypes.POINTER(ChainPlan), _VP, _INT, _INT, _VP, _FP], _INT),
+    "rptc_chain_status": ([ctypes.POINTER(ChainPlan), ctypes.POINTER(ctypes.c_int), _VP], _INT),
     "rptc_matvec_dense": ([_VP, _VP, _VP, _I64, _I64, _INT, _INT, _VP, _FP], _INT),
     "rptc_matvec_t_dense": ([_VP, _VP, _VP, _I64, _I64, _INT, _INT, _VP, _FP], _INT),
     "rptc_decompress_matmul": ([_VP, _VP, _VP, _VP, _I64, _I64, _I64, _INT, _INT, _VP, _FP], _INT),
@@ -621,6 +637,67 @@ def decompress_matvec_rmsnorm_affine(compressed, codebook, x_in, delta, weight, 
                         (compressed.data_ptr(), codebook.data_ptr(), x_in.data_ptr(),
                          None if delta is None else delta.data_ptr(), weight.data_ptr(), x_out.data_ptr(), *aff,
                          out.data_ptr()), (m, n, float(eps), S), compressed.device, carry_mode)
+
+
+class MatvecChain:
+    """A chain of ``decompress_matvec_16_{S}_1`` products in one launch (``rptc_decompress_matvec_chain``).
+
+    ``layers`` is a sequence of ``(compressed, x, out)`` tensor triples (int32 stream, fp16 [n], fp16 [m]); the
+    tensors are kept alive by the object and their addresses are fixed in the plan, their contents are read at
+    run time.  Dependencies between layers are found from the addresses (a layer that reads what an earlier one
+    writes waits for it).  One codebook and one carry mode serve the whole chain."""
+
+    def __init__(self, layers, codebook):
+        layers = list(layers)
+        _check(len(layers) >= 1, "a chain needs at least one layer")
+        _check_input(codebook, "codebook")
+        _check(codebook.dim() == 1 and codebook.size(0) in (128, 512) and codebook.dtype == torch.float16,
+               "codebook must be fp16 of length 128 or 512")
+        self.S = 6 if codebook.size(0) == 128 else 8
+        self.codebook = codebook
+        self.layers = layers
+        arr = (ChainLayer * len(layers))()
+        for i, (c, x, out) in enumerate(layers):
+            for t, name in ((c, "compressed"), (x, "x"), (out, "out")):
+                _check_input(t, name)
+                _check(t.device == codebook.device, "all tensors must be on the same device")
+            _check(c.dtype == torch.int32, "compressed.scalar_type() == torch::kInt32")
+            _check(x.dim() == 1 and x.dtype == torch.float16, "x must be a 1-D fp16 tensor")
+            _check(out.dim() == 1 and out.dtype == torch.float16, "out must be a 1-D fp16 tensor")
+            n, m = x.size(0), out.size(0)
+            _check(n % 64 == 0 and n >= 64 and m >= 1, "x.size(0) % 64 == 0")
+            _check(c.numel() * 16 == m * n, "compressed.numel() * 16 == m * n")
+            arr[i] = ChainLayer(c.data_ptr(), x.data_ptr(), out.data_ptr(), m, n)
+        lib = library()
+        need = lib.rptc_chain_desc_bytes(len(layers))
+        _check(need > 0, "too many layers")
+        with torch.cuda.device(codebook.device):
+            self.desc = torch.zeros(need + 256, dtype=torch.uint8, device=codebook.device)
+            base = (self.desc.data_ptr() + 255) & ~255
+            self.plan = ChainPlan()
+            stream = torch.cuda.current_stream().cuda_stream
+            _status(lib.rptc_chain_plan(arr, len(layers), base, need, ctypes.byref(self.plan), ctypes.c_void_p(stream)))
+
+    def run(self, carry_mode=None, timed=None):
+        """One launch on the current stream; returns elapsed ms (0.0 when not timed)."""
+        ms = ctypes.c_float(0.0)
+        mode = _carry_mode if carry_mode is None else carry_mode
+        with torch.cuda.device(self.codebook.device):
+            stream = torch.cuda.current_stream().cuda_stream
+            rc = library().rptc_decompress_matvec_chain(ctypes.byref(self.plan), self.codebook.data_ptr(), self.S, mode,
+                                                        ctypes.c_void_p(stream),
+                                                        ctypes.byref(ms) if (_timing if timed is None else timed) else None)
+        _status(rc)
+        return float(ms.value)
+
+    def status(self):
+        """Waits for the current stream; 0 when every run so far completed (bit 0: a bounded wait inside the kernel
+        ran out; bit 1: an arrival counter is not zero)."""
+        st = ctypes.c_int(-1)
+        with torch.cuda.device(self.codebook.device):
+            stream = torch.cuda.current_stream().cuda_stream
+            _status(library().rptc_chain_status(ctypes.byref(self.plan), ctypes.byref(st), ctypes.c_void_p(stream)))
+        return st.value
 
 
 def matvec_bits_dense(compressed, codebook, out, bits):

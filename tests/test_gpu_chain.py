@@ -1,0 +1,218 @@
+"""rptc_decompress_matvec_chain on the GPU: a chain of fused decode + mat-vecs in one launch.  Every layer's output is
+held to the double-precision product of the bit-exact dense matrix (rel-L2 1e-3, the mat-vec's bar) on the input
+the chain itself fed it, to the per-launch kernel on the same input, and to itself from run to run (bit for bit)."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from util import np_f16, np_u32, rand_codes, rand_half, rel_l2
+
+pytestmark = pytest.mark.gpu
+
+REL_L2_TOL = 1e-3
+
+
+@pytest.fixture(scope="module")
+def rk():
+    import rptc_kernels
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    assert rptc_kernels.library().rptc_init() == 0
+    return rptc_kernels
+
+
+@pytest.fixture(autouse=True)
+def _announce(request):
+    print(f"\n[case] {request.node.nodeid}", flush=True)
+    yield
+
+
+def dense_of(rk, comp, cb, m, n, S, mode):
+    W = torch.zeros((m, n), dtype=torch.float16, device="cuda")
+    prev = rk.set_carry_mode(mode)
+    try:
+        rk.matvec_dense(comp, cb, W, S)
+    finally:
+        rk.set_carry_mode(prev)
+    return W
+
+
+def check_layer(rk, comp, cb, x, out, S, mode):
+    m, n = out.numel(), x.numel()
+    W = dense_of(rk, comp, cb, m, n, S, mode)
+    want = (W.double() @ x.double()).cpu().numpy()
+    assert rel_l2(np_f16(out), want) < REL_L2_TOL
+    # the per-launch kernel on the same input (another order of the same fp32 sums)
+    y = torch.zeros(m, dtype=torch.float16, device="cuda")
+    prev = rk.set_carry_mode(mode)
+    try:
+        getattr(rk, f"decompress_matvec_16_{S}_1")(comp.reshape(n // 2048, m, 128) if n % 2048 == 0 else comp, cb, x, y)
+    finally:
+        rk.set_carry_mode(prev)
+    assert rel_l2(np_f16(out), np_f16(y).astype(np.float64)) < REL_L2_TOL
+
+
+SHAPES = [(64, 2048), (33, 4096 + 768), (7, 704), (512, 6144), (300, 64), (1024, 2048 + 64), (5, 16384), (2000, 1984)]
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+@pytest.mark.parametrize("S", [6, 8])
+def test_chain_of_independent_layers(rk, oracle, S, mode):
+    """Layers of many shapes (ragged rows, odd row counts, fewer rows than workgroups, the longest row) with
+    inputs and outputs of their own: nothing orders them, so waves run from one into the next."""
+    cb = rand_half(2 << S, seed=5).cuda()
+    layers = []
+    for i, (m, n) in enumerate(SHAPES * 2):
+        comp = rand_codes(m * n // 16, seed=100 + i).cuda()
+        x = rand_half(n, seed=200 + i).cuda()
+        out = torch.full((m,), float("nan"), dtype=torch.float16, device="cuda")
+        layers.append((comp, x, out))
+    chain = rk.MatvecChain(layers, cb)
+    chain.run(carry_mode=mode)
+    assert chain.status() == 0
+    first = [out.clone() for _, _, out in layers]
+    for comp, x, out in layers:
+        assert not torch.isnan(out).any()
+        check_layer(rk, comp, cb, x, out, S, mode)
+    # decoded weights through the fused path, bit for bit: one-hot activations read single matrix entries
+    m, n = SHAPES[1]
+    comp = layers[1][0]
+    Wd = oracle.matvec_dense(np_u32(comp), np_f16(cb), m, n, S, mode=mode)
+    cols = [0, 1, 63, 64, 2047, 2048, 4095, 4096, n - 1]
+    hot = []
+    for c in cols:
+        x = torch.zeros(n, dtype=torch.float16, device="cuda")
+        x[c] = 1.0
+        hot.append((comp, x, torch.zeros(m, dtype=torch.float16, device="cuda")))
+    rk.MatvecChain(hot, cb).run(carry_mode=mode)
+    for c, (_, _, out) in zip(cols, hot):
+        assert np.array_equal(np_f16(out).astype(np.float32), Wd[:, c].astype(np.float32))
+    # again: every sum has a fixed order, so the bits repeat
+    for _, _, out in layers:
+        out.fill_(float("nan"))
+    chain.run(carry_mode=mode)
+    assert chain.status() == 0
+    for (_, _, out), ref in zip(layers, first):
+        assert torch.equal(out.view(torch.int16), ref.view(torch.int16))
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+def test_chain_of_dependent_layers_at_the_llama_shapes(rk, mode):
+    """out of one layer is the next one's input (4096 -> 4096 -> 11008 -> 4096 -> 4096): every layer starts behind the
+    grid-wide counter.  Each layer is checked on the input the chain gave it."""
+    S = 8
+    cb = (rand_half(2 << S, seed=6).float() * 0.02).half().cuda()       # keeps the activations in fp16 range
+    dims = [4096, 4096, 11008, 4096, 4096]
+    bufs = [rand_half(dims[0], seed=7).cuda()] + [torch.full((d,), float("nan"), dtype=torch.float16, device="cuda") for d in dims[1:]]
+    layers = []
+    for i in range(len(dims) - 1):
+        n, m = dims[i], dims[i + 1]
+        layers.append((rand_codes(m * n // 16, seed=300 + i).cuda(), bufs[i], bufs[i + 1]))
+    chain = rk.MatvecChain(layers, cb)
+    for rep in range(3):
+        for b in bufs[1:]:
+            b.fill_(float("nan"))
+        chain.run(carry_mode=mode)
+        assert chain.status() == 0
+        for comp, x, out in layers:
+            assert not torch.isnan(out).any()
+            check_layer(rk, comp, cb, x, out, S, mode)
+        if rep == 0:
+            first = [b.clone() for b in bufs[1:]]
+        else:
+            for b, ref in zip(bufs[1:], first):
+                assert torch.equal(b.view(torch.int16), ref.view(torch.int16))
+
+
+def test_chain_orders_layers_that_share_a_buffer(rk):
+    """Two layers write the same output (the later one wins), and a third reads an input that an earlier one
+    overwrites afterwards (it must read the old contents): the plan finds the hazards from the addresses."""
+    S, m, n = 8, 1024, 2048
+    cb = rand_half(2 << S, seed=8).cuda()
+    c = [rand_codes(m * n // 16, seed=400 + i).cuda() for i in range(4)]
+    x0, x1 = rand_half(n, seed=9).cuda(), rand_half(n, seed=10).cuda()
+    shared = torch.zeros(m, dtype=torch.float16, device="cuda")
+    a = torch.zeros(n, dtype=torch.float16, device="cuda")
+    layers = [(c[0], x0, shared), (c[1], x1, shared)]
+    rk.MatvecChain(layers, cb).run()
+    y = torch.zeros(m, dtype=torch.float16, device="cuda")
+    rk.decompress_matvec_16_8_1(c[1].reshape(1, m, 128), cb, x1, y)
+    assert rel_l2(np_f16(shared), np_f16(y).astype(np.float64)) < REL_L2_TOL
+    # write after read: layer 0 reads `a`, layer 1 overwrites `a` (square layers)
+    m2 = n2 = 2048
+    c2 = [rand_codes(m2 * n2 // 16, seed=500 + i).cuda() for i in range(2)]
+    a.copy_(rand_half(n2, seed=11).cuda())
+    a_before = a.clone()
+    out0 = torch.zeros(m2, dtype=torch.float16, device="cuda")
+    rk.MatvecChain([(c2[0], a, out0), (c2[1], x0, a)], cb).run()
+    y0 = torch.zeros(m2, dtype=torch.float16, device="cuda")
+    rk.decompress_matvec_16_8_1(c2[0].reshape(1, m2, 128), cb, a_before, y0)
+    assert rel_l2(np_f16(out0), np_f16(y0).astype(np.float64)) < REL_L2_TOL
+    y1 = torch.zeros(m2, dtype=torch.float16, device="cuda")
+    rk.decompress_matvec_16_8_1(c2[1].reshape(1, m2, 128), cb, x0, y1)
+    assert rel_l2(np_f16(a), np_f16(y1).astype(np.float64)) < REL_L2_TOL
+
+
+def test_long_chain_reuses_slots_and_counters(rk):
+    """200 layers over 8 streams (the three activation slots, two partial-sum buffers and their counters go round
+    many times), the headline shape included; outputs of layers with equal inputs are equal bit for bit."""
+    S = 8
+    cb = rand_half(2 << S, seed=12).cuda()
+    m, n = 4096, 11008
+    comps = [rand_codes(m * n // 16, seed=600 + i).cuda() for i in range(8)]
+    xs = [rand_half(n, seed=700 + i).cuda() for i in range(3)]
+    outs = [torch.full((m,), float("nan"), dtype=torch.float16, device="cuda") for _ in range(200)]
+    layers = [(comps[i % 8], xs[i % 3], outs[i]) for i in range(200)]
+    chain = rk.MatvecChain(layers, cb)
+    chain.run()
+    assert chain.status() == 0
+    for i in range(24):
+        check_layer(rk, comps[i % 8], cb, xs[i % 3], outs[i], S, 0)
+    for i in range(24, 200):
+        assert torch.equal(outs[i].view(torch.int16), outs[i % 24].view(torch.int16))
+
+
+def test_chain_gives_up_when_the_grid_cannot_arrive(rk):
+    """A plan that expects one more workgroup than the grid has can never pass its grid-wide counter: with a small
+    spin limit every wave gives up, the kernel ends by itself and the status says so.  (Forced from the host: the
+    expected arrivals and the spin limit are fields of the plan.)"""
+    S, m, n = 8, 2048, 2048
+    cb = rand_half(2 << S, seed=13).cuda()
+    a = rand_half(n, seed=14).cuda()
+    b = torch.zeros(m, dtype=torch.float16, device="cuda")
+    c = torch.zeros(m, dtype=torch.float16, device="cuda")
+    comps = [rand_codes(m * n // 16, seed=800 + i).cuda() for i in range(2)]
+    chain = rk.MatvecChain([(comps[0], a, b), (comps[1], b, c)], cb)
+    words = (ctypes.c_uint32 * 20).from_buffer(chain.plan)
+    grid = words[5]
+    assert words[11] == grid                       # arrivals
+    words[11] = grid + 1
+    words[12] = 2000                               # spin limit
+    chain.run()
+    st = chain.status()                            # waits for the kernel: it must have ended
+    assert st & 1
+    # planned again, the chain runs to the end
+    chain = rk.MatvecChain([(comps[0], a, b), (comps[1], b, c)], cb)
+    chain.run()
+    assert chain.status() == 0
+    check_layer(rk, comps[1], cb, b, c, S, 0)
+
+
+def test_chain_rejects_bad_arguments(rk):
+    lib = rk.library()
+    cb = torch.zeros(512, dtype=torch.float16, device="cuda")
+    ok = (torch.zeros(64 * 2048 // 16, dtype=torch.int32, device="cuda"), torch.zeros(2048, dtype=torch.float16, device="cuda"),
+          torch.zeros(64, dtype=torch.float16, device="cuda"))
+    with pytest.raises(RuntimeError):
+        rk.MatvecChain([], cb)
+    with pytest.raises(RuntimeError):                       # n too long for a thread's two registers
+        rk.MatvecChain([(torch.zeros(4 * 16448 // 16, dtype=torch.int32, device="cuda"),
+                         torch.zeros(16448, dtype=torch.float16, device="cuda"), torch.zeros(4, dtype=torch.float16, device="cuda"))], cb)
+    chain = rk.MatvecChain([ok], cb)
+    assert lib.rptc_decompress_matvec_chain(None, cb.data_ptr(), 8, 0, None, None) == -1
+    assert lib.rptc_decompress_matvec_chain(ctypes.byref(chain.plan), cb.data_ptr(), 7, 0, None, None) == -2
+    assert lib.rptc_decompress_matvec_chain(ctypes.byref(chain.plan), cb.data_ptr(), 8, 3, None, None) == -4
+    blank = rk.ChainPlan()
+    assert lib.rptc_decompress_matvec_chain(ctypes.byref(blank), cb.data_ptr(), 8, 0, None, None) == -2
+    assert lib.rptc_chain_desc_bytes(0) == -2
