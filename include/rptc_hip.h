@@ -114,7 +114,8 @@ int rptc_decompress_matvec_20_8_1(const int32_t *compressed, const uint16_t *cod
  * front of it (a grid-wide arrival counter); other layers overlap freely.  The result is the same, bit for bit,
  * as `count` separate launches in order would give, except that a row's slabs are added per slab first.
  *
- *   rptc_chain_desc_bytes(count)   device bytes the caller provides for the chain's descriptors (< 0: status)
+ *   rptc_chain_desc_bytes(...)     device bytes the caller provides for the chain's descriptors and item tables
+ *                                  (< 0: a status; at most 65535 layers, each stream below 4 GiB)
  *   rptc_chain_plan(...)           checks the layers, writes the descriptors into device_desc (256-byte aligned
  *                                  device memory; copied on `stream`, which is waited for: a set-up call, not
  *                                  for stream capture) and fills *plan (host memory, opaque).  The plan and the
@@ -135,7 +136,7 @@ typedef struct rptc_chain_layer {
 typedef struct rptc_chain_t {
     uint64_t opaque[10];
 } rptc_chain_t;
-int64_t rptc_chain_desc_bytes(int64_t count);
+int64_t rptc_chain_desc_bytes(const rptc_chain_layer *layers, int64_t count);
 int rptc_chain_plan(const rptc_chain_layer *layers, int64_t count, void *device_desc, int64_t device_desc_bytes,
                     rptc_chain_t *plan, void *stream);
 int rptc_decompress_matvec_chain(const rptc_chain_t *plan, const uint16_t *codebook, int S, int carry_mode,

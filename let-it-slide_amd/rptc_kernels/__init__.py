@@ -74,7 +74,7 @@ _SIGNATURES = {
     "rptc_decompress_matvec_20_8_1": (_MATVEC_ARGS, _INT),
     "rptc_decompress_matvec_t_16": (_MATVEC_ARGS, _INT),
     "rptc_decompress_matvec_t_14": (_MATVEC_ARGS, _INT),
-    "rptc_chain_desc_bytes": ([_I64], _I64),
+    "rptc_chain_desc_bytes": ([ctypes.POINTER(ChainLayer), _I64], _I64),
     "rptc_chain_plan": ([ctypes.POINTER(ChainLayer), _I64, _VP, _I64, ctypes.POINTER(ChainPlan), _VP], _INT),
     "rptc_decompress_matvec_chain": ([ctypes.POINTER(ChainPlan), _VP, _INT, _INT, _VP, _FP], _INT),
     "rptc_chain_status": ([ctypes.POINTER(ChainPlan), ctypes.POINTER(ctypes.c_int), _VP], _INT),
@@ -669,8 +669,9 @@ class MatvecChain:
             _check(c.numel() * 16 == m * n, "compressed.numel() * 16 == m * n")
             arr[i] = ChainLayer(c.data_ptr(), x.data_ptr(), out.data_ptr(), m, n)
         lib = library()
-        need = lib.rptc_chain_desc_bytes(len(layers))
-        _check(need > 0, "too many layers")
+        need = lib.rptc_chain_desc_bytes(arr, len(layers))
+        if need < 0:
+            _status(int(need))
         with torch.cuda.device(codebook.device):
             self.desc = torch.zeros(need + 256, dtype=torch.uint8, device=codebook.device)
             base = (self.desc.data_ptr() + 255) & ~255

@@ -215,4 +215,4 @@ def test_chain_rejects_bad_arguments(rk):
     assert lib.rptc_decompress_matvec_chain(ctypes.byref(chain.plan), cb.data_ptr(), 8, 3, None, None) == -4
     blank = rk.ChainPlan()
     assert lib.rptc_decompress_matvec_chain(ctypes.byref(blank), cb.data_ptr(), 8, 0, None, None) == -2
-    assert lib.rptc_chain_desc_bytes(0) == -2
+    assert lib.rptc_chain_desc_bytes(None, 1) == -1
