@@ -49,8 +49,9 @@ def parse():
                          "direct: one host call per step")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--pmc-probe", action="store_true",
-                    help="for `rocprofv3 --pmc`: a few direct launches of the kernel plus a plain device copy of "
-                         "known size (the calibration for FETCH_SIZE / WRITE_SIZE); prints no benchmark line")
+                    help="for `rocprofv3 --pmc`: a few direct launches of the kernel, of the chain, of the transposed "
+                         "mat-vec and of the batch-16 product, plus a plain device copy of known size (the calibration "
+                         "for FETCH_SIZE / WRITE_SIZE); prints no benchmark line")
     ap.add_argument("--extra-shapes", action="store_true", help="also time the other layer shapes")
     ap.add_argument("--other-ops", action="store_true",
                     help="time decompress, decompress_matvec_t_16 and sign_hadamard instead (prints its own JSON line)")
@@ -173,14 +174,15 @@ class Runner:
         return t1 - t0, ev0.elapsed_time(ev1)
 
     def chain_run(self, steps, warmup):
-        """`steps` layers (step k = weight copy k % copies, an output of its own per copy) as ONE chain launch.
+        """`steps` layers (step k = weight copy k % copies, an output of its own per step: two layers that write one
+        buffer would be ordered by the chain, behind a grid-wide counter) as ONE chain launch.
         Returns (wall seconds, event milliseconds, rel-L2 of the last layer's output against the dense product)."""
         torch = self.torch
         import rptc_kernels
         copies = len(self.weights)
-        outs = [torch.zeros(self.m, dtype=torch.float16, device="cuda") for _ in range(copies)]
-        chain = rptc_kernels.MatvecChain([(self.weights[k % copies], self.x, outs[k % copies]) for k in range(steps)], self.codebook)
-        warm = rptc_kernels.MatvecChain([(self.weights[k % copies], self.x, outs[k % copies]) for k in range(max(warmup, 1))],
+        outs = torch.zeros((max(steps, warmup, 1), self.m), dtype=torch.float16, device="cuda")
+        chain = rptc_kernels.MatvecChain([(self.weights[k % copies], self.x, outs[k]) for k in range(steps)], self.codebook)
+        warm = rptc_kernels.MatvecChain([(self.weights[k % copies], self.x, outs[k]) for k in range(max(warmup, 1))],
                                         self.codebook)
         warm.run(carry_mode=0, timed=False)
         torch.cuda.synchronize()
@@ -195,11 +197,10 @@ class Runner:
         t1 = time.perf_counter()
         if chain.status() != 0:
             raise RuntimeError("the chain did not complete")
-        last = (steps - 1) % copies
         W = torch.zeros((self.m, self.n), dtype=torch.float16, device="cuda")
-        rptc_kernels.matvec_bits_dense(self.weights[last], self.codebook, W, 2)
+        rptc_kernels.matvec_bits_dense(self.weights[(steps - 1) % copies], self.codebook, W, 2)
         want = W.double() @ self.x.double()
-        err = ((outs[last].double() - want).norm() / want.norm()).item()
+        err = ((outs[steps - 1].double() - want).norm() / want.norm()).item()
         if not err < 1e-3:
             raise RuntimeError(f"chain output is wrong: rel-L2 {err}")
         return t1 - t0, ev0.elapsed_time(ev1), err
@@ -564,6 +565,7 @@ def main():
     if a.pmc_probe:
         # calibration: an int32 -> float32 conversion copy is a plain streaming kernel that reads
         # 64 MiB and writes 64 MiB
+        import rptc_kernels as rk
         src = torch.randint(0, 1 << 20, (16 << 20,), dtype=torch.int32, device="cuda")
         dst = torch.empty(16 << 20, dtype=torch.float32, device="cuda")
         stream = torch.cuda.current_stream().cuda_stream
@@ -571,8 +573,35 @@ def main():
             dst.copy_(src)
             runner.launch(k, stream)
         torch.cuda.synchronize()
-        print(f"pmc-probe: 8 conversion copies of {src.numel() * 4} bytes in / {dst.numel() * 4} bytes out "
-              f"and 8 launches of {runner.bytes} compressed bytes")
+        # the chain: one launch of `copies` independent layers, twice (counters per dispatch = per `copies` layers)
+        outs = torch.zeros((a.copies, a.m), dtype=torch.float16, device="cuda")
+        chain = rk.MatvecChain([(runner.weights[k], runner.x, outs[k]) for k in range(a.copies)], runner.codebook)
+        for _ in range(2):
+            chain.run(carry_mode=0, timed=False)
+        torch.cuda.synchronize()
+        # the transposed mat-vec (4096 x 4096, scalar 2^16 codebook, both carry modes) and the batched product (batch 16)
+        g = torch.Generator(device="cuda")
+        g.manual_seed(7)
+        rk.set_timing(False)
+        cb16 = torch.randn(65536, generator=g, device="cuda").half()
+        xt = torch.randn(4096, generator=g, device="cuda").half()
+        yt = torch.zeros(4096, dtype=torch.float16, device="cuda")
+        streams = [torch.randint(-(1 << 31), 1 << 31, (4096 * 4096 // 16,), generator=g, dtype=torch.int64, device="cuda").to(torch.int32)
+                   for _ in range(8)]
+        for mode in (rk.AS_WRITTEN, rk.CONTINUOUS):
+            rk.set_carry_mode(mode)
+            for k in range(8):
+                rk.decompress_matvec_t_16(streams[k], cb16, xt, yt)
+        rk.set_carry_mode(rk.AS_WRITTEN)
+        xb = torch.randn((16, a.n), generator=g, device="cuda").half()
+        yb = torch.zeros((16, a.m), dtype=torch.float16, device="cuda")
+        for k in range(8):
+            getattr(rk, f"decompress_matmul_16_{a.S}_1")(runner.weights[k % a.copies], runner.codebook, xb, yb)
+        torch.cuda.synchronize()
+        print(f"pmc-probe: 8 conversion copies of {src.numel() * 4} bytes in / {dst.numel() * 4} bytes out, "
+              f"8 launches of {runner.bytes} compressed bytes, 2 chain launches of {a.copies} such layers, "
+              f"8 + 8 launches of decompress_matvec_t_16 on 4096 x 4096 (as written, continuous), "
+              f"8 launches of the batch-16 product on {a.m} x {a.n}")
         return
     err = runner.check()
     per_launch = None
@@ -608,7 +637,7 @@ def main():
                         f"({a.copies * runner.bytes >> 20} MiB), caches flushed before the timed region",
             "distinct_copies_touched": min(a.steps, a.copies),
             "launch": a.launch if a.launch != "chain" else "chain: the steps are the layers of one rptc_decompress_matvec_chain launch "
-                                                            "(independent layers, an output buffer per weight copy)",
+                                                            "(independent layers, an output buffer per layer)",
             "accumulate": "f32",
             "carry_mode": "as_written",
             "compressed_bytes": runner.bytes,

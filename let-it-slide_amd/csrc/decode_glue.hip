@@ -346,21 +346,18 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(
         __hip_atomic_store(&mine[256], mx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __hip_atomic_store(&mine[257], sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-    // Release / acquire at agent scope: the storing threads release the piece before the barrier lets thread 0
-    // count the arrival (an acquire-release read-modify-write), and the workgroup that sees the last arrival
-    // acquires before it reads the other pieces, whichever XCD they were computed on.
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+    // (the hand-off between workgroups: see published() / arrive() in rptc_common.hpp)
+    published();
     __syncthreads();
     uint32_t *flag = reinterpret_cast<uint32_t *>(scratch);
     if (tid == 0) {
-        const uint32_t prev = __hip_atomic_fetch_add(&arrived[h], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        const uint32_t prev = arrive(&arrived[h]);
         const bool last = prev == (uint32_t)(splits - 1);
         if (last) __hip_atomic_store(&arrived[h], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // for the next launch
         *flag = last;
     }
     __syncthreads();
     if (!*flag || tid >= hd) return;
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
     const float *head_parts = parts + (size_t)h * splits * kAttnPartStride;
     constexpr int kMaxSplits = 16;
     float pm[kMaxSplits], pl[kMaxSplits], pa[kMaxSplits];

@@ -305,21 +305,17 @@ __global__ __launch_bounds__(kMmThreads) __attribute__((amdgpu_waves_per_eu(4, 4
     }
 
     // The workgroup that arrives last at its row group's counter adds the slabs' tiles, in slab order.
-    // Release / acquire at agent scope: every thread that stored part of a tile releases its stores (they have
-    // reached device-coherent memory before the barrier lets thread 0 count the arrival), thread 0's counter
-    // update is an acquire-release read-modify-write, and the workgroup that sees the last arrival acquires
-    // before it reads the other workgroups' tiles, whichever XCD they ran on.
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+    // (the hand-off between workgroups: see published() / arrive() in rptc_common.hpp)
+    published();
     __syncthreads();
     if (tid == 0) {
-        const uint32_t prev = __hip_atomic_fetch_add(&arrived[grp], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        const uint32_t prev = arrive(&arrived[grp]);
         const bool last = prev == (uint32_t)(slabs - 1);
         if (last) __hip_atomic_store(&arrived[grp], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // for the next launch
         *s_last = last;
     }
     __syncthreads();
     if (!*s_last) return;
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
     const int tile_floats = row_blocks * PLANES * 256, tile_stride = max_rb * PLANES * 256;
     const float *grp_partial = partial + (size_t)grp * slabs * tile_stride;
     // every thread requests its share of four slabs' tiles before it adds any of them: the loads go

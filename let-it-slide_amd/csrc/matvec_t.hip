@@ -22,6 +22,7 @@ constexpr int kTThreads = 512;
 constexpr int kTWaves = kTThreads / kWave;
 constexpr int kTMaxParts = 4096;        // workgroups of a launch that splits the columns
 constexpr int kTMaxSplit = 16;
+constexpr int kTRing = 8;               // stream elements a wave has requested ahead of the decode
 
 static __device__ __align__(256) float g_t_part[kTMaxParts * kWave];
 static __device__ __align__(256) uint32_t g_t_arrived[kTMaxParts];
@@ -59,53 +60,92 @@ __global__ __launch_bounds__(kTThreads) void matvec_t_kernel(
     const int c0 = min(g1, g0 + wave * per), c1 = min(g1, c0 + per);
 
     // Requests in the order their data is needed: the thread's share of the table, then the element in
-    // front of the wave's range (its state warms up the decoder) and the first two elements of the range.
+    // front of the wave's range (its state warms up the decoder) and the first kTRing elements of the range.
+    // A wave's elements come from memory with a latency of a few thousand clocks and are decoded in a few
+    // hundred each, so the time of the loop is the latency times the elements divided by the requests in
+    // flight: the ring holds eight (all of a wave's elements when the columns are split eight ways or more).
     // The stream requests are unconditional (clamped to an element that exists) so that the table can be
     // stored while they are still on their way; what a clamped request returns is never used.
     constexpr int kPerThread = lut_u4 / kTThreads;
+    uint4 xa = make_uint4(0u, 0u, 0u, 0u), xb = xa;
+    if (MODE == RPTC_AS_WRITTEN && tid < 4 * (g1 - g0)) {
+        const uint4 *xv = reinterpret_cast<const uint4 *>(x + 32 * g0 + 8 * tid);
+        xa = xv[0];
+        xb = xv[1];
+    }
     uint4 t[kPerThread];
 #pragma unroll
     for (int i = 0; i < kPerThread; i++) t[i] = codebook[i * kTThreads + tid];
     const int row_c = min(row, m - 1), last_col = cols - 1;
     const uint4 before = comp[(size_t)min(max(c0 - 1, 0), last_col) * m + row_c];
-    uint4 next = comp[(size_t)min(c0, last_col) * m + row_c];
-    uint4 next2 = comp[(size_t)min(c0 + 1, last_col) * m + row_c];
+    uint4 ring[kTRing];
+#pragma unroll
+    for (int i = 0; i < kTRing; i++) ring[i] = comp[(size_t)min(c0 + i, last_col) * m + row_c];
+    // As written, the eight steps of a stream word multiply the same two table values (inference_t.cu:125-134), so
+    // what a word needs of its sixteen activations is the sum of the even and the sum of the odd ones: two fp32
+    // values per word, added up here once per workgroup and kept in LDS (every lane of a wave reads the same ones:
+    // a broadcast).  Their loads were the first requests of the kernel, so they are here before the table is.
+    // (Reading the sixteen through the scalar cache in the loop, one wait per word for data requested a few
+    // instructions earlier, made an element cost a thousand clocks.  The continuous mode, where every step has
+    // table values of its own, still does that.)
+    float *part = reinterpret_cast<float *>(lds_u4 + lut_u4);      // [wave][lane]
+    uint32_t *xs = reinterpret_cast<uint32_t *>(part + kTThreads);
+    if (MODE == RPTC_AS_WRITTEN) {
+        for (int wd = tid; wd < 4 * (g1 - g0); wd += kTThreads) {
+            const uint32_t d[8] = {xa.x, xa.y, xa.z, xa.w, xb.x, xb.y, xb.z, xb.w};
+            float lo = 0.f, hi = 0.f;
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                lo += half_bits_to_float((uint16_t)(d[j] & 0xFFFFu));
+                hi += half_bits_to_float((uint16_t)(d[j] >> 16));
+            }
+            reinterpret_cast<float2 *>(xs)[wd] = make_float2(lo, hi);
+            if (wd + kTThreads < 4 * (g1 - g0)) {
+                const uint4 *xv = reinterpret_cast<const uint4 *>(x + 32 * g0 + 8 * (wd + kTThreads));
+                xa = xv[0];
+                xb = xv[1];
+            }
+        }
+    }
 #pragma unroll
     for (int i = 0; i < kPerThread; i++) lds_u4[i * kTThreads + tid] = t[i];
     __syncthreads();
     const uint16_t *lut = reinterpret_cast<const uint16_t *>(lds_u4);
-    float *part = reinterpret_cast<float *>(lds_u4 + lut_u4);      // [wave][lane]
 
     uint32_t carry = 0;
     if (c0 > 0 && c0 < c1 && valid) carry = warm_state<L>(before, MODE);
     float acc = 0.f;
-    for (int col = c0; col < c1; col++) {
-        const uint4 e = next;
-        next = next2;
-        if (col + 2 < c1) next2 = comp[(size_t)(col + 2) * m + row_c];
-        const uint32_t words[4] = {e.x, e.y, e.z, e.w};
+    for (int col0 = c0; col0 < c1; col0 += kTRing) {
 #pragma unroll
-        for (int k = 0; k < 4; k++) {
-            const uint32_t word = words[k];
-            const uint32_t *xp = x + 32 * col + 8 * k;      // wave-uniform
-            if (MODE == RPTC_AS_WRITTEN) {
-                // all eight steps of a word see the carry the word started with
-                // (inference_t.cu:125-134), and the carry becomes the 4-bit-advanced state
-                const uint32_t s2 = mask & ((carry << 2) | (word >> 30));
-                const uint32_t s4 = mask & ((carry << 4) | (word >> 28));
-                carry = s4;
-                const uint32_t w = (uint32_t)lut[s2] | ((uint32_t)lut[s4] << 16);
+        for (int i = 0; i < kTRing; i++) {
+            const int col = col0 + i;
+            if (col >= c1) break;                                   // (wave-uniform)
+            const uint4 e = ring[i];
+            if (col + kTRing < c1) ring[i] = comp[(size_t)(col + kTRing) * m + row_c];
+            const uint32_t words[4] = {e.x, e.y, e.z, e.w};
 #pragma unroll
-                for (int j = 0; j < 8; j++) acc = dot2(w, xp[j], acc);
-            } else {
+            for (int k = 0; k < 4; k++) {
+                const uint32_t word = words[k];
+                if (MODE == RPTC_AS_WRITTEN) {
+                    // all eight steps of a word see the carry the word started with
+                    // (inference_t.cu:125-134), and the carry becomes the 4-bit-advanced state
+                    const uint32_t s2 = mask & ((carry << 2) | (word >> 30));
+                    const uint32_t s4 = mask & ((carry << 4) | (word >> 28));
+                    carry = s4;
+                    const float2 xw = reinterpret_cast<const float2 *>(xs)[4 * (col - g0) + k];     // wave-uniform
+                    acc = fmaf(half_bits_to_float(lut[s2]), xw.x, acc);
+                    acc = fmaf(half_bits_to_float(lut[s4]), xw.y, acc);
+                } else {
+                    const uint32_t *xp = x + 32 * col + 8 * k;                                         // wave-uniform, scalar loads
 #pragma unroll
-                for (int j = 0; j < 8; j++) {
-                    const uint32_t s2 = mask & alignbit(carry, word, 30 - 4 * j);
-                    const uint32_t s4 = mask & alignbit(carry, word, 28 - 4 * j);
-                    const uint32_t w = (uint32_t)lut[s2] | ((uint32_t)lut[s4] << 16);
-                    acc = dot2(w, xp[j], acc);
+                    for (int j = 0; j < 8; j++) {
+                        const uint32_t s2 = mask & alignbit(carry, word, 30 - 4 * j);
+                        const uint32_t s4 = mask & alignbit(carry, word, 28 - 4 * j);
+                        const uint32_t w = (uint32_t)lut[s2] | ((uint32_t)lut[s4] << 16);
+                        acc = dot2(w, xp[j], acc);
+                    }
+                    carry = word & mask;
                 }
-                carry = word & mask;
             }
         }
     }
@@ -121,22 +161,19 @@ __global__ __launch_bounds__(kTThreads) void matvec_t_kernel(
         if (tid < kWave && valid) out[row] = float_to_half_bits(half_bits_to_float(out[row]) + y);
         return;
     }
-    // Release / acquire at agent scope: the storing threads release their partial sums before the barrier lets
-    // thread 0 count the arrival (an acquire-release read-modify-write), and the workgroup that sees the last
-    // arrival acquires before it reads the other workgroups' sums, whichever XCD they ran on.
+    // (the hand-off between workgroups: see published() / arrive() in rptc_common.hpp)
     if (tid < kWave) __hip_atomic_store(&parts[(size_t)blockIdx.x * kWave + tid], y, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+    published();
     __syncthreads();
     uint32_t *flag = reinterpret_cast<uint32_t *>(part);
     if (tid == 0) {
-        const uint32_t prev = __hip_atomic_fetch_add(&arrived[rb], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        const uint32_t prev = arrive(&arrived[rb]);
         const bool last = prev == (uint32_t)(ksplit - 1);
         if (last) __hip_atomic_store(&arrived[rb], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // for the next launch
         *flag = last;
     }
     __syncthreads();
     if (!*flag || tid >= kWave || !valid) return;
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
     float p[kTMaxSplit];
 #pragma unroll
     for (int i = 0; i < kTMaxSplit; i++)
@@ -185,8 +222,13 @@ __global__ __launch_bounds__(256) void matvec_t_dense_kernel(
     }
 }
 
+// LDS: the table, one partial sum per thread and, as written, two fp32 sums of activations per stream word of the
+// workgroup's columns (32 bytes a column)
 template <int L>
-static int lds_bytes_t() { return (2 << L) + kTThreads * 4; }
+static int lds_bytes_t(int cols_per_group, int mode)
+{
+    return (2 << L) + kTThreads * 4 + (mode == RPTC_AS_WRITTEN ? cols_per_group * 32 : 0);
+}
 
 struct TScratch {
     float *parts;
@@ -213,21 +255,30 @@ static int launch_matvec_t(const int32_t *compressed, const uint16_t *codebook, 
     if (rc) return rc;
     const int row_blocks = (int)((m + kWave - 1) / kWave);
     const int cols = (int)(n / 64);
-    // workgroups per row block: enough for every CU, each wave keeps at least one column
+    // Workgroups per row block.  Splitting the columns spreads the table look-ups, which bound the decode (two-byte
+    // gathers from 128 KiB: about twelve clocks of a CU's LDS per wave and look-up), over more CUs, and costs three
+    // dependent trips to memory at the end (partial sums out, arrival counted, partial sums in: 3-4 us measured).
+    // As written a column costs a workgroup about 0.03 us, so the split pays from 128 columns on, and a workgroup
+    // keeps at least 32; in continuous mode (eight times the look-ups) it nearly always pays, and a wave keeps at
+    // least one column.  Never more workgroups than CUs: each one fills its own table first.
     int ksplit = dev->cus / row_blocks;
     if (ksplit > kTMaxSplit) ksplit = kTMaxSplit;
-    if (ksplit > cols / kTWaves) ksplit = cols / kTWaves;
+    const int keep = carry_mode == RPTC_AS_WRITTEN ? 32 : kTWaves;
+    if (ksplit > cols / keep) ksplit = cols / keep;
+    if (carry_mode == RPTC_AS_WRITTEN && cols < 128) ksplit = 1;
     if (ksplit < 1 || row_blocks * ksplit > kTMaxParts) ksplit = 1;
+    const int lds_bytes = lds_bytes_t<L>((cols + ksplit - 1) / ksplit, carry_mode);     // (at most 146 KiB: n <= 32768)
+    if (lds_bytes > kMaxLds) return RPTC_ELIMIT;
     const TScratch &sc = g_t[dev->device];
     auto a_comp = reinterpret_cast<const uint4 *>(compressed);
     auto a_cb = reinterpret_cast<const uint4 *>(codebook);
     auto a_x = reinterpret_cast<const uint32_t *>(x);
     if (carry_mode == RPTC_AS_WRITTEN)
         hipLaunchKernelGGL((matvec_t_kernel<L, RPTC_AS_WRITTEN>), dim3(row_blocks * ksplit), dim3(kTThreads),
-                           lds_bytes_t<L>(), s, a_comp, a_cb, a_x, (int)m, cols, ksplit, out, sc.parts, sc.arrived);
+                           lds_bytes, s, a_comp, a_cb, a_x, (int)m, cols, ksplit, out, sc.parts, sc.arrived);
     else
         hipLaunchKernelGGL((matvec_t_kernel<L, RPTC_CONTINUOUS>), dim3(row_blocks * ksplit), dim3(kTThreads),
-                           lds_bytes_t<L>(), s, a_comp, a_cb, a_x, (int)m, cols, ksplit, out, sc.parts, sc.arrived);
+                           lds_bytes, s, a_comp, a_cb, a_x, (int)m, cols, ksplit, out, sc.parts, sc.arrived);
     return t.end();
 }
 

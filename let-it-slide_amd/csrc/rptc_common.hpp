@@ -134,6 +134,28 @@ __device__ __forceinline__ float half_wave_sum(float v)
     return v;
 }
 
+// Hand-off of partial results between workgroups (which may run on different XCDs, each with an L2 of its own).
+// The producing threads write their results with agent-scope stores (`__hip_atomic_store(..., __ATOMIC_RELAXED,
+// __HIP_MEMORY_SCOPE_AGENT)`: global_store ... sc1, written through to the level all XCDs share), then call
+// published() and meet at a workgroup barrier; one thread then counts the arrival with arrive().  The workgroup
+// that sees the last arrival reads the others' results with agent-scope loads (global_load ... sc1, which do not
+// hit in a cache that another XCD's store did not update).
+// What makes this enough on gfx942 / gfx950: the vector memory counter of a wave is decremented for a store only
+// when the store has been acknowledged at the level its scope bits name, so after `s_waitcnt vmcnt(0)` the wave's
+// sc1 stores are visible to every sc1 load of the device; the barrier orders all producing waves of the workgroup
+// before the counter update; the counter update and the last arrival's loads are separated by the data dependence
+// on the returned count, a barrier and a branch.  A release fence at agent scope in front of the barrier and an
+// acquire fence behind the branch say the same in the language's memory model, and are what a first version used:
+// the compiler turns them into a write-back and an invalidate of the whole L2 of the XCD (buffer_wbl2 sc1,
+// buffer_inv sc1), which nothing here needs (no plain store is part of the hand-off) and which costs 15-25 us per
+// launch, measured on the transposed mat-vec (4096 x 4096: 27 us with the fences, 8 us without) and on the batched
+// product (batch 16 on 4096 x 11008: 67 us against 15 us).
+__device__ __forceinline__ void published() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+__device__ __forceinline__ uint32_t arrive(uint32_t *counter)
+{
+    return __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 __device__ __forceinline__ uint16_t float_to_half_bits(float f)
 {
     _Float16 h = (_Float16)f;   // v_cvt_f16_f32, round to nearest even
