@@ -28,9 +28,10 @@ for p in (ROOT, os.path.join(ROOT, "let-it-slide_amd")):
 
 HBM_PEAK_GBS = 8000.0
 
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a copy kernel
-# of known size; the runs are summarised under profiles/).  Keyed by (m, n, S); other workloads report null.
-MEASURED_TRAFFIC_BYTES = {(4096, 11008, 8): 11528200}
+# HBM bytes per launch (per layer for the chain) measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on
+# `bench.py --pmc-probe` (scaled by a copy kernel of known size; the runs are summarised under profiles/).
+# Keyed by (launch kind, m, n, S); other workloads report null.
+MEASURED_TRAFFIC_BYTES = {("launch", 4096, 11008, 8): 11528200, ("chain", 4096, 11008, 8): 11288800}
 
 
 def parse():
@@ -185,6 +186,10 @@ class Runner:
         warm = rptc_kernels.MatvecChain([(self.weights[k % copies], self.x, outs[k]) for k in range(max(warmup, 1))],
                                         self.codebook)
         warm.run(carry_mode=0, timed=False)
+        # one untimed launch of the chain itself, as the graph of the per-launch pattern is replayed once before it is
+        # timed: the first long launch after the set-up work runs at clocks that are still rising (5.9 us a layer
+        # against 5.0-5.4 for every later one)
+        chain.run(carry_mode=0, timed=False)
         torch.cuda.synchronize()
         evict_caches()
         ev0 = torch.cuda.Event(enable_timing=True)
@@ -247,9 +252,22 @@ def cpu_baseline(runner, min_seconds=8.0):
 MFMA_F16_PEAK_TFLOPS = 2516.6
 
 
+# HBM traffic of the batch-16 product on 4096 x 11008 (same --pmc-probe runs as above): 14 071 KiB read (stream,
+# partial tiles read back, packed activations) + 1 683 KiB written (partial tiles, packed activations, output)
+MEASURED_MATMUL_TRAFFIC_BYTES = {(4096, 11008, 8, 16, 2): 16132000}
+
+
+def _hbm_roofline(stream_bytes, us, traffic=None):
+    """The roofline object of a stream-bound call: its algorithmic bytes are the compressed stream (the layers are at
+    128-256 flop/byte at batch 16-32, below the 315 flop/byte ridge of fp16 MFMA over HBM)."""
+    gbs = stream_bytes / us / 1e3
+    return {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": traffic}
+
+
 def bench_matmul(a):
     """Batch 8/16/32 fused decode + mat-mat on the same layer, next to decode-then-dense-GEMM
-    (dense export kernel + torch.matmul on the decoded fp16 matrix)."""
+    (dense export kernel + torch.matmul on the decoded fp16 matrix) and to the batch-1 mat-vec on the same stream."""
     import torch
     import rptc_kernels
     lib = rptc_kernels.library()
@@ -263,6 +281,11 @@ def bench_matmul(a):
                for _ in range(copies)]
     cb = torch.randn(2 << S, generator=g, device="cuda").to(torch.float16)
     W = torch.zeros((m, n), dtype=torch.float16, device="cuda")
+    x1 = torch.randn(n, generator=g, device="cuda").to(torch.float16)
+    y1 = torch.zeros(m, dtype=torch.float16, device="cuda")
+    mv = getattr(rptc_kernels, f"decompress_matvec_16_{S}_1")
+    matvec_us = _graph_time_us(lambda k: mv(weights[k % copies].reshape(n // 2048, m, 128) if n % 2048 == 0 else weights[k % copies],
+                                            cb, x1, y1), min(a.steps, 200))
     results = {}
     for batch in (8, 16, 32):
         x = torch.randn((batch, n), generator=g, device="cuda").to(torch.float16)
@@ -308,7 +331,9 @@ def bench_matmul(a):
             "hbm_GBps": round(m * n / 4 / us / 1e3, 1), "hbm_frac": round(m * n / 4 / us / 1e3 / HBM_PEAK_GBS, 4),
             "decode_then_gemm_us": round(times["decode_then_gemm"], 2),
             "speedup_vs_decode_then_gemm": round(times["decode_then_gemm"] / us, 2),
+            "matvec_us": round(matvec_us, 2), "times_the_matvec": round(us / matvec_us, 2),
             "rel_l2_vs_dense": float(f"{err:.3e}"),
+            "roofline": _hbm_roofline(m * n // 4, us, MEASURED_MATMUL_TRAFFIC_BYTES.get((m, n, S, batch, 2))),
         }
     other = {}
     if a.extra_shapes:
@@ -326,7 +351,8 @@ def bench_matmul(a):
             flops = 2.0 * mm * nn * 16
             other[f"{mm}x{nn} batch16"] = {"us": round(us, 2), "TFLOPs": round(flops / us / 1e6, 2),
                                           "mfma_util": round(flops / us / 1e6 / MFMA_F16_PEAK_TFLOPS, 5),
-                                          "hbm_GBps": round(mm * nn / 4 / us / 1e3, 1)}
+                                          "hbm_GBps": round(mm * nn / 4 / us / 1e3, 1),
+                                          "roofline": _hbm_roofline(mm * nn // 4, us)}
             del ws
     if a.extra_shapes:
         # 3 and 4 bits per weight on the headline shape, batch 16
@@ -342,7 +368,8 @@ def bench_matmul(a):
             flops = 2.0 * mm * nn * 16
             other[f"{mm}x{nn} {bits}b batch16"] = {"us": round(us, 2), "TFLOPs": round(flops / us / 1e6, 2),
                                                   "mfma_util": round(flops / us / 1e6 / MFMA_F16_PEAK_TFLOPS, 5),
-                                                  "hbm_GBps": round(mm * nn * bits / 8 / us / 1e3, 1)}
+                                                  "hbm_GBps": round(mm * nn * bits / 8 / us / 1e3, 1),
+                                                  "roofline": _hbm_roofline(mm * nn * bits // 8, us)}
             del ws
     line = {"metric": "fused decode+GEMM (MFMA) per call", "unit": "us", "n_gpus": 1,
             "config": {"workload": f"decompress_matmul_16_{S}_1 m={m} n={n} 2 bits/weight, {copies} rotating "
@@ -649,12 +676,13 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4),
-            "traffic": MEASURED_TRAFFIC_BYTES.get((a.m, a.n, a.S)),
+            "traffic": MEASURED_TRAFFIC_BYTES.get(("chain" if a.launch == "chain" else "launch", a.m, a.n, a.S)),
             "launch_us": round(launch_ms * 1e3, 3),
         },
     }
     if per_launch is not None:
         line["roofline"]["kernel"] = "matvec_chain_kernel: achieved = steps x compressed bytes / the one launch's duration; launch_us is per layer"
+        per_launch["traffic"] = MEASURED_TRAFFIC_BYTES.get(("launch", a.m, a.n, a.S))
         line["per_launch"] = per_launch
     # the floor of this workload on this machine, in the same launch pattern (graph replay over the
     # same rotating buffers): an empty launch, and a kernel that only reads the stream
