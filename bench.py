@@ -450,6 +450,24 @@ def bench_other_ops(a):
         byts = 4 * batch * n
         res[f"sign_hadamard batch {batch} n {n}"] = {"us": round(us, 2), "bytes": byts,
                                                      "GBps": round(byts / us / 1e3, 1)}
+    # the general (L, S, R, V) trellis of rptc_lite.py at the reference's own setting (rptc_lite.py:141-146), 2^24
+    # steps in sequences of 1024: 4 bytes of symbols read and 8 bytes of outputs written per step
+    L, S, R, V, rows, T = 16, 9, 4, 2, 16384, 1024
+    alphabet = torch.randn((1 << S, V), generator=g, device="cuda")
+    syms = [torch.randint(0, 1 << R, (rows, T), generator=g, dtype=torch.int32, device="cuda") for _ in range(2)]
+    deq = [torch.empty((rows, T, V), dtype=torch.float32, device="cuda") for _ in range(2)]
+    lib = rk.library()
+
+    def lite(k):
+        rc = lib.rptc_lite_dequantize(alphabet.data_ptr(), L, S, R, V, syms[k % 2].data_ptr(), rows, T, deq[k % 2].data_ptr(),
+                                      ctypes.c_void_p(torch.cuda.current_stream().cuda_stream), None)
+        assert rc == 0, rc
+    us = _graph_time_us(lite, min(steps, 50))
+    byts = rows * T * (4 + 4 * V)
+    fill_us = _graph_time_us(lambda k: deq[k % 2].fill_(1.0), min(steps, 50))
+    res[f"lite_dequantize L{L} S{S} R{R} V{V} {rows}x{T}"] = {"us": round(us, 2), "bytes": byts, "GBps": round(byts / us / 1e3, 1),
+                                                            "frac_hbm": round(byts / us / 1e3 / HBM_PEAK_GBS, 4),
+                                                            "fill_of_the_output_us": round(fill_us, 2)}
     print(json.dumps({"metric": "other ops, microseconds per call", "unit": "us", "n_gpus": 1,
                       "config": {"launch": "graph", "steps": steps}, "results": res}))
 

@@ -319,6 +319,19 @@ int rptc_decompress_matvec_rmsnorm_affine(const int32_t *compressed, const uint1
                                           float *ms);
 
 /*
+ * The general (L, S, R, V) trellis of the reference's rptc_lite.py: replaces rptc_lite.dequantize
+ * (rptc_lite.py:63-73) with its index_fn (rptc_lite.py:12-16).  Per sequence: an int32 register, 0 at the start,
+ * register = (register << R) | symbol at every step (never masked, as there), and the step's V outputs are
+ * alphabet[index_fn(register)], index_fn(x) = x * (2x + 1) with int32 wraparound, x ^= x >> (L - S) with the
+ * arithmetic shift of a signed value, the low S bits.
+ *   alphabet  float [2^S][V];  symbols  int32 [rows][length], used with all their 32 bits as the reference uses
+ *   them;  out  float [rows][length][V], overwritten
+ *   1 <= R <= 16, 1 <= S <= 16, S <= L <= 31, 1 <= V <= 8; alphabet and out 8-byte aligned when V == 2
+ */
+int rptc_lite_dequantize(const float *alphabet, int L, int S, int R, int V, const int32_t *symbols, int64_t rows,
+                         int64_t length, float *out, void *stream, float *ms);
+
+/*
  * Viterbi search for the hashed pair stream: the symbols whose decode by rptc_decompress_matvec_16_{S}_1
  * (carry mode continuous) is closest to the targets.  Replaces the search of the reference's quantizer
  * (rptc.py:13-71, diag_only path: rho[0] = 0 at the start, first index on ties, best end state traced

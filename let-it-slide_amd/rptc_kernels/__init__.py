@@ -90,6 +90,7 @@ _SIGNATURES = {
     "rptc_viterbi_scalar": ([_VP, _VP, _I64, _VP, _INT, _VP, _VP, _VP, _VP, _I64, _I64, _VP, _FP], _INT),
     "rptc_viterbi_pairs": ([_VP, _VP, _I64, _VP, _VP, _VP, _VP, _VP, _I64, _I64, _INT, _VP, _FP], _INT),
     "rptc_viterbi_pairs_bits": ([_VP, _VP, _I64, _VP, _VP, _VP, _VP, _VP, _I64, _I64, _INT, _INT, _VP, _FP], _INT),
+    "rptc_lite_dequantize": ([_VP, _INT, _INT, _INT, _INT, _VP, _I64, _I64, _VP, _VP, _FP], _INT),
     "rptc_sign_hadamard": ([_VP, _VP, _VP, _I64, _I64, _I64, _INT, _VP, _FP], _INT),
     "rptc_decompress_matvec_bits": ([_VP, _VP, _VP, _VP, _I64, _I64, _INT, _INT, _INT, _VP, _FP], _INT),
     "rptc_matvec_bits_dense": ([_VP, _VP, _VP, _I64, _I64, _INT, _INT, _INT, _VP, _FP], _INT),
@@ -404,6 +405,35 @@ def sign_hadamard(x, signs, out, block=0, inverse=False, timed=None):
                                           ctypes.byref(ms) if (_timing if timed is None else timed) else None)
     _status(rc)
     return float(ms.value)
+
+
+def lite_dequantize(alphabet, L, S, R, quantized, timed=None):
+    """``rptc_lite.dequantize(alphabet, L, S, R, quantized)`` (rptc_lite.py:63-73): the outputs of the general
+    hashed-codebook trellis for a symbol sequence.
+
+    alphabet: float32 [2^S, V]; quantized: int32 [length] or [rows, length] (every row a sequence of its own that
+    starts from register 0).  Returns (dequantized float32 [length, V] or [rows, length, V], elapsed ms)."""
+    _check_input(alphabet, "alphabet")
+    _check_input(quantized, "quantized")
+    _check(alphabet.dtype == torch.float32 and alphabet.dim() == 2, "alphabet must be float32 [2^S, V]")
+    _check(quantized.dtype == torch.int32 and quantized.dim() in (1, 2), "quantized must be int32 [length] or [rows, length]")
+    _check(1 <= R <= 16 and 1 <= S <= 16 and S <= L <= 31, "1 <= R <= 16, 1 <= S <= 16, S <= L <= 31")
+    _check(alphabet.size(0) == 1 << S, "alphabet.size(0) == 1 << S")
+    V = alphabet.size(1)
+    _check(1 <= V <= 8, "1 <= V <= 8")
+    rows = quantized.size(0) if quantized.dim() == 2 else 1
+    length = quantized.size(-1)
+    _check(rows >= 1 and length >= 1, "rows >= 1 and length >= 1")
+    device = alphabet.device
+    _check(quantized.device == device, "all tensors must be on the same device")
+    ms = ctypes.c_float(0.0)
+    with torch.cuda.device(device):
+        out = torch.empty(tuple(quantized.shape) + (V,), dtype=torch.float32, device=device)
+        stream = torch.cuda.current_stream().cuda_stream
+        rc = library().rptc_lite_dequantize(alphabet.data_ptr(), L, S, R, V, quantized.data_ptr(), rows, length, out.data_ptr(),
+                                            ctypes.c_void_p(stream), ctypes.byref(ms) if (_timing if timed is None else timed) else None)
+    _status(rc)
+    return out, float(ms.value)
 
 
 def viterbi_pairs(targets, codebook, weights=None, bits=2):

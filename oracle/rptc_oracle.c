@@ -547,7 +547,7 @@ int orc_matvec_t_dense(const uint32_t *compressed, const uint16_t *codebook,
     return 0;
 }
 
-/* ------------------------------ rptc_lite.py:12-16, 63-73 (off the kernels) */
+/* ------------------------------ rptc_lite.py:12-16, 63-73 (the checker of rptc_lite_dequantize) */
 
 /* index_fn on int32 with wraparound; >> on a signed value is arithmetic */
 int32_t orc_lite_index_fn(int32_t x, int L, int S)
