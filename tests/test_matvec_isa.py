@@ -1,12 +1,12 @@
-"""A property of the chain kernel's compiled code that its source cannot express.
+"""A property of the mat-vec kernels' compiled code that their source cannot express.
 
-`csrc/matvec_chain.hip` reloads a slab's 32 activation registers with `ds_read_b32` instructions written as `asm`
-statements and waits for them in a further `asm` statement.  The data of such a read lands in its register some
+`csrc/matvec.hip` and `csrc/matvec_chain.hip` reload a slab's 32 activation registers with `ds_read_b32` instructions
+written as `asm` statements and wait for them in a further `asm` statement.  The data of such a read lands in its register some
 time after the instruction; until the wait, the register's contents are undefined, and the compiler does not know
 that.  It is free to place its own instructions between the statements, and a copy or a reuse of one of those
-registers there reads or overwrites a value that has not arrived.  This test compiles the kernel to assembly with the
+registers there reads or overwrites a value that has not arrived.  This test compiles the kernels to assembly with the
 library's flags and checks that no compiler-generated instruction names a register of those reads between the first
-read of a reload and its wait."""
+read of a reload and its wait (every template instantiation of both files)."""
 import importlib.util
 import os
 import re
@@ -64,9 +64,10 @@ def reload_sites(lines):
 
 
 @pytest.mark.skipif(shutil.which("hipcc") is None, reason="needs hipcc")
-def test_no_compiler_instruction_touches_a_register_with_an_lds_read_in_flight(tmp_path):
-    out = tmp_path / "matvec_chain.s"
-    cmd = ["hipcc", *_flags(), "--cuda-device-only", "-S", os.path.join(PKG, "csrc", "matvec_chain.hip"), "-o", str(out)]
+@pytest.mark.parametrize("source", ["matvec_chain.hip", "matvec.hip"])
+def test_no_compiler_instruction_touches_a_register_with_an_lds_read_in_flight(tmp_path, source):
+    out = tmp_path / (source + ".s")
+    cmd = ["hipcc", *_flags(), "--cuda-device-only", "-S", os.path.join(PKG, "csrc", source), "-o", str(out)]
     subprocess.run(cmd, check=True, capture_output=True)
     sites = list(reload_sites(out.read_text().split("\n")))
     assert len(sites) >= 4, "the reload of the activation registers was not found in the assembly"
