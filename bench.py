@@ -65,6 +65,8 @@ def parse():
                     help="with --decode: the projections are random-init dense weights put through the quantizer "
                          "(row/column factorisation + trellis search) instead of random streams; their scales and "
                          "biases are applied inside the mat-vec kernels")
+    ap.add_argument("--valu-probe", action="store_true",
+                    help="issue rate of the vector instructions the decode consists of (four waves a SIMD, registers only)")
     ap.add_argument("--matmul", action="store_true",
                     help="time the batch 8/16/32 fused decode + MFMA mat-mat instead (prints its own JSON line)")
     return ap.parse_args()
@@ -99,6 +101,7 @@ def aids_library():
     lib = ctypes.CDLL(path)
     lib.rptc_probe_empty.argtypes = [ctypes.c_int, ctypes.c_void_p]
     lib.rptc_probe_read.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p]
+    lib.rptc_probe_valu.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
     return lib
 
 
@@ -472,6 +475,38 @@ def bench_other_ops(a):
                       "config": {"launch": "graph", "steps": steps}, "results": res}))
 
 
+def bench_valu_probe(a):
+    """Time per instruction and SIMD of the decode's vector instructions, four waves a SIMD as in the mat-vec, against
+    v_fma_f32; and from it the vector-ALU time of one 4096 x 11008 layer (12 wave-items a SIMD; per stream element
+    12 v_alignbit_b32, 16 v_pk_mad_u16, 32 address ops (v_perm_b32 / v_and_or_b32), 32 v_dot2c_f32_f16)."""
+    import torch
+    aids = aids_library()
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    names = ["v_dot2c_f32_f16", "v_pk_mad_u16", "v_perm_b32", "v_alignbit_b32", "v_and_or_b32", "v_fma_f32"]
+    iters = 4000
+    res = {}
+    stream = torch.cuda.current_stream().cuda_stream
+    for kind, name in enumerate(names):
+        best = None
+        for rep in range(4):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            rc = aids.rptc_probe_valu(kind, iters, cus, None, ctypes.c_void_p(stream))
+            assert rc == 0, rc
+            e1.record()
+            torch.cuda.synchronize()
+            t = e0.elapsed_time(e1) * 1e6 / (iters * 32 * 4)          # ns per instruction and SIMD (4 waves a SIMD)
+            best = t if best is None or t < best else best
+        res[name] = round(best, 4)
+    fma = res["v_fma_f32"]
+    rel = {k: round(v / fma, 3) for k, v in res.items()}
+    per_element = 12 * res["v_alignbit_b32"] + 16 * res["v_pk_mad_u16"] + 16 * res["v_perm_b32"] + 16 * res["v_and_or_b32"] + 32 * res["v_dot2c_f32_f16"]
+    print(json.dumps({"metric": "vector instruction issue time, ns per instruction and SIMD", "unit": "ns", "n_gpus": 1,
+                      "config": {"waves_per_simd": 4, "instructions_per_wave": iters * 32}, "results": res,
+                      "relative_to_v_fma_f32": rel,
+                      "decode_valu_us_per_4096x11008_layer": round(12 * per_element / 1e3, 3)}))
+
+
 def bench_quantize(a):
     """The Viterbi search kernel (the quantizer's inner loop) on the rows of one 4096 x 4096 layer:
     trellis state updates per second against the vector-ALU rate that bounds it, with the same search in
@@ -563,6 +598,9 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
     torch.cuda.set_device(0)
+    if a.valu_probe:
+        bench_valu_probe(a)
+        return
     if a.matmul:
         bench_matmul(a)
         return

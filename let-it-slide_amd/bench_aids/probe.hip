@@ -32,7 +32,67 @@ __global__ __launch_bounds__(1024) void probe_read_kernel(const uint32_t *__rest
     if (s == 0x9E3779B9u && sink) sink[0] = s;
 }
 
+// Issue rate of the vector instructions the decode is made of: every wave runs `iters` rounds of 32 instructions of
+// one kind on eight independent registers (a chain of eight never waits for its own result), one 1024-thread
+// workgroup per compute unit, i.e. four waves a SIMD as in the mat-vec.  Nothing is read; the result is stored only
+// if it equals a value it cannot take.
+#define RPTC_PROBE_8(TEXT)                                                                                            \
+    asm volatile(TEXT(%0) TEXT(%1) TEXT(%2) TEXT(%3) TEXT(%4) TEXT(%5) TEXT(%6) TEXT(%7)                              \
+                 : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]), "+v"(r[4]), "+v"(r[5]), "+v"(r[6]), "+v"(r[7])   \
+                 : "v"(a), "v"(b), "s"(sel))
+#define RPTC_I_DOT2C(R) "v_dot2c_f32_f16 " #R ", %8, %9\n"
+#define RPTC_I_PKMAD(R) "v_pk_mad_u16 " #R ", %8, %8, " #R "\n"
+#define RPTC_I_PERM(R) "v_perm_b32 " #R ", " #R ", %9, %10\n"
+#define RPTC_I_ALIGN(R) "v_alignbit_b32 " #R ", " #R ", %8, 7\n"
+#define RPTC_I_ANDOR(R) "v_and_or_b32 " #R ", " #R ", %10, %9\n"
+#define RPTC_I_FMA(R) "v_fma_f32 " #R ", %8, %9, " #R "\n"
+
+template <int KIND>
+__global__ __launch_bounds__(1024) void probe_valu_kernel(int iters, uint32_t seed, uint32_t *sink)
+{
+    uint32_t r[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) r[i] = seed + threadIdx.x * 8u + i;
+    const uint32_t a = 0x3C003800u ^ (threadIdx.x << 3), b = 0x38003C00u + blockIdx.x;
+    const uint32_t sel = 0x0C0C0500u;
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            if (KIND == 0) RPTC_PROBE_8(RPTC_I_DOT2C);
+            else if (KIND == 1) RPTC_PROBE_8(RPTC_I_PKMAD);
+            else if (KIND == 2) RPTC_PROBE_8(RPTC_I_PERM);
+            else if (KIND == 3) RPTC_PROBE_8(RPTC_I_ALIGN);
+            else if (KIND == 4) RPTC_PROBE_8(RPTC_I_ANDOR);
+            else RPTC_PROBE_8(RPTC_I_FMA);
+        }
+    }
+    uint32_t x = 0;
+#pragma unroll
+    for (int i = 0; i < 8; i++) x ^= r[i];
+    if (x == 0x9E3779B9u && sink) sink[0] = x;
+}
+
 }  // namespace
+
+// `iters` rounds of 32 vector instructions of one kind in every wave of `workgroups` 1024-thread workgroups;
+// kind: 0 v_dot2c_f32_f16, 1 v_pk_mad_u16, 2 v_perm_b32, 3 v_alignbit_b32, 4 v_and_or_b32, 5 v_fma_f32
+extern "C" int rptc_probe_valu(int kind, int iters, int workgroups, void *sink, void *stream)
+{
+    if (kind < 0 || kind > 5 || iters < 1 || workgroups < 1) return -2;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    uint32_t *out = static_cast<uint32_t *>(sink);
+#define RPTC_PROBE_GO(K) hipLaunchKernelGGL(probe_valu_kernel<K>, dim3(workgroups), dim3(1024), 0, s, iters, 12345u, out)
+    switch (kind) {
+    case 0: RPTC_PROBE_GO(0); break;
+    case 1: RPTC_PROBE_GO(1); break;
+    case 2: RPTC_PROBE_GO(2); break;
+    case 3: RPTC_PROBE_GO(3); break;
+    case 4: RPTC_PROBE_GO(4); break;
+    default: RPTC_PROBE_GO(5); break;
+    }
+#undef RPTC_PROBE_GO
+    return (int)hipGetLastError();
+}
 
 // one empty 1024-thread workgroup per workgroup of the mat-vec's grid
 extern "C" int rptc_probe_empty(int workgroups, void *stream)

@@ -23,7 +23,6 @@
 //     wait for are issued first and every wave's stream loads right behind them, before the
 //     table is built; kernel arguments are preloaded into SGPRs.
 #include "decode_asm.hpp"
-#include "matvec_loop.hpp"
 #include "hadamard_pass.hpp"
 #include "rptc_common.hpp"
 
@@ -717,256 +716,6 @@ __global__ __launch_bounds__(kMatvecThreads) void matvec_affine_kernel(
 }
 
 // Dense export: one thread per stream element, 32 pairs scattered to their columns.
-// ------------------------------------------------------------------------------------------------------------
-// A chain of independent layers in one launch: the body above in a loop over layers (2 bits, plain activations, one
-// partial sum per stream element).  What a launch per layer pays every time is paid once or hidden:
-//   * the table is written once;
-//   * a layer costs ONE workgroup barrier: two activation images and two sets of partial sums take turns, so the
-//     barrier that publishes layer k's activations is also the one behind which layer k - 1's rows are added up;
-//   * the activations of layer k + 1 are requested when layer k's decode starts, and a wave requests the first
-//     stream element of layer k + 1 when it starts on its last element of layer k.
-// Layers must not depend on each other (the host checks the addresses): nothing orders a layer's reads behind another
-// layer's writes.
-template <int S, int MODE>
-__global__ __launch_bounds__(kMatvecThreads) void matvec_loop_kernel(
-    const LoopLayer *__restrict__ layers, const uint32_t *__restrict__ codebook, int count, int xslot_words, int part_floats)
-{
-    constexpr int WORDS = 4;
-    extern __shared__ uint32_t lds[];
-    uint32_t *const sx0 = lds + kTableBytes / 4;                                   // two activation images, slot order
-    float *const part0 = reinterpret_cast<float *>(sx0 + 2 * xslot_words);         // two sets of [row in block][n / 64]
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const uint32_t lane4 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds)) + lane * 4;   // the table is at LDS address 0
-
-    // The pointers come out of a descriptor in memory, so their address space is stated: global loads and stores,
-    // not flat ones.
-    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-    typedef const __attribute__((address_space(1))) uint32_t *global_words;
-    typedef const __attribute__((address_space(1))) u32x4 *global_vec4;
-    typedef __attribute__((address_space(1))) uint16_t *global_halves;
-    struct Work {                 // a layer as this wave sees it (all wave-uniform)
-        global_words comp;
-        global_vec4 x;
-        global_halves out;
-        int m, T, Lt, npr, n8, rw_tail, items_full, items_tail;
-        int row0, rows;           // rows <= 0: no row of this layer is this workgroup's
-        int it_begin, it_end, first_slab, first_idx;
-    };
-    auto setup = [&](int k) {
-        Work w;
-        const LoopLayer &d = layers[k];
-        const int n = d.n, rpb = d.rows_per_block;
-        w.comp = reinterpret_cast<global_words>(reinterpret_cast<uintptr_t>(d.comp));
-        w.x = reinterpret_cast<global_vec4>(reinterpret_cast<uintptr_t>(d.x));
-        w.out = reinterpret_cast<global_halves>(reinterpret_cast<uintptr_t>(d.out));
-        w.m = d.m;
-        w.T = n >> 11, w.Lt = (n & 2047) >> 6, w.npr = n >> 6, w.n8 = n >> 3;
-        w.rw_tail = d.rw_tail, w.items_full = rpb >> 1, w.items_tail = d.items_tail;
-        w.row0 = blockIdx.x * rpb;
-        w.rows = min(rpb, w.m - w.row0);
-        // the split of the per-launch kernel (see matvec_body): shares in the proportion a SIMD serves its waves in
-        // from three items a wave on, else the first total % 16 waves take one more
-        const int total = w.rows > 0 ? w.T * w.items_full + w.items_tail : 0;
-        constexpr uint32_t kCum64 = 0x382A18u;
-        if (total >= 3 * kMatvecWaves) {
-            const uint32_t group = (uint32_t)wave >> 2;
-            const uint32_t cum_lo = group == 0 ? 0u : ((uint32_t)total * ((kCum64 >> (8 * group - 8)) & 0xFFu)) >> 6;
-            const uint32_t cum_hi = group == 3 ? (uint32_t)total : ((uint32_t)total * ((kCum64 >> (8 * group)) & 0xFFu)) >> 6;
-            const uint32_t cnt = cum_hi - cum_lo, per_wave = cnt >> 2, extra = cnt & 3u;
-            const uint32_t turn = ((uint32_t)wave - cum_lo) & 3u;
-            w.it_begin = (int)(cum_lo + turn * per_wave + min(turn, extra));
-            w.it_end = w.it_begin + (int)per_wave + (turn < extra ? 1 : 0);
-        } else {
-            const int per_wave = (int)((uint32_t)total / kMatvecWaves), extra = (int)((uint32_t)total % kMatvecWaves);
-            w.it_begin = wave * per_wave + min(wave, extra);
-            w.it_end = w.it_begin + per_wave + (wave < extra ? 1 : 0);
-        }
-        int first_slab = w.items_full == 1 ? w.it_begin : (int)__umulhi((uint32_t)w.it_begin, d.full_magic);
-        w.first_slab = min(first_slab, w.T);
-        w.first_idx = w.it_begin - w.first_slab * w.items_full;
-        return w;
-    };
-    auto view = [&](const Work &w, int slab) {
-        SlabView v;
-        const bool full = slab < w.T;
-        v.lanes = full ? 32 : w.Lt;
-        v.rows_per_item = full ? 2 : w.rw_tail;
-        v.items = full ? w.items_full : w.items_tail;
-        v.part_off = slab * 32;
-        v.elem0 = (uint32_t)(full ? slab : w.T) * (uint32_t)w.m * 32u;
-        return v;
-    };
-    // a thread's share of a layer's activations (every lane asks, with a clamped index: the compiler can count them)
-    auto load_x = [&](const Work &w, uint4 (&xv)[kXRegs]) {
-#pragma unroll
-        for (int u = 0; u < kXRegs; u++) {
-            const u32x4 v = w.x[min(tid + u * kMatvecThreads, w.n8 - 1)];
-            xv[u] = make_uint4(v.x, v.y, v.z, v.w);
-        }
-    };
-    // the first element of a wave's first item of layer w, asked for by every lane whatever the wave holds (a lane
-    // past the item's rows repeats the last lane's address; a wave without an item asks for the first element of
-    // the stream in every lane)
-    // a stream element is read once: non-temporal, wave-uniform base plus 16 bytes per lane
-    auto load_element = [&](global_words wave_base, uint32_t at_lane) {
-        const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<global_vec4>(wave_base + at_lane * WORDS));
-        Elem<WORDS> e;
-        e.w[0] = v.x, e.w[1] = v.y, e.w[2] = v.z, e.w[3] = v.w;
-        return e;
-    };
-    auto load_first = [&](const Work &w, Elem<WORDS> &buf, uint32_t &cw) {
-        const SlabView ld = view(w, w.first_slab);
-        const int row_first = w.first_idx * ld.rows_per_item;
-        const int rows_here = min(ld.rows_per_item, w.rows - row_first);
-        const bool real = w.it_begin < w.it_end && rows_here > 0;
-        const uint32_t elem = real ? ld.elem0 + (uint32_t)(w.row0 + row_first) * (uint32_t)ld.lanes : 0u;
-        const uint32_t last = real ? (uint32_t)(rows_here * ld.lanes - 1) : 0u;
-        buf = load_element(w.comp + (size_t)elem * WORDS, min((uint32_t)lane, last));
-        if (MODE == RPTC_CONTINUOUS) {
-            const bool prev = real && w.first_slab > 0;
-            const int sub = min(w.first_slab < w.T ? lane >> 5 : lane / ld.lanes, max(rows_here, 1) - 1);
-            const global_words row_base =
-                prev ? w.comp + (((size_t)(w.first_slab - 1) * w.m + w.row0 + row_first) * 32 + 31) * WORDS + WORDS - 1 : w.comp;
-            cw = row_base[sub * (prev ? 32 * WORDS : 0)];
-        }
-    };
-
-    Work cur = setup(0), prev = cur;
-    uint4 xv[kXRegs];
-    Elem<WORDS> buf;
-    uint32_t cw = 0;
-    // requests first (the activations, then the stream), the table behind them
-    constexpr int kRowsPerWave = 256 / kMatvecWaves;
-    uint32_t cbv[kRowsPerWave];
-#pragma unroll
-    for (int i = 0; i < kRowsPerWave; i++) cbv[i] = codebook[(kRowsPerWave * wave + i) & ((1 << S) - 1)];
-    const uint32_t table_sign = (uint32_t)((kRowsPerWave * wave) >> 7) << 15;
-    load_x(cur, xv);
-    load_first(cur, buf, cw);
-#pragma unroll
-    for (int i = 0; i < kRowsPerWave; i++) {
-        uint32_t tv;
-        asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(tv) : "s"(cbv[i]), "v"(0xFFFF7FFFu), "v"(table_sign));
-        lds[(kRowsPerWave * wave + i) * 64 + lane] = tv;
-    }
-
-    uint32_t xr[32];
-#pragma unroll
-    for (int q = 0; q < 32; q++) xr[q] = 0;
-    for (int k = 0; k <= count; k++) {
-        if (k < count) {
-            // layer k's activations into image k & 1 (halves 8 idx .. 8 idx + 7 to the four planes, inference.cu:215-221)
-            uint32_t *const sx = sx0 + (k & 1) * xslot_words;
-            const int n8 = cur.n8;
-            uint32_t *const s0 = sx + tid, *const s1 = s0 + n8, *const s2 = s1 + n8, *const s3 = s2 + n8;
-#pragma unroll
-            for (int u = 0; u < kXRegs; u++) {
-                if (tid + u * kMatvecThreads < n8) {
-                    s0[u * kMatvecThreads] = xv[u].x;
-                    s1[u * kMatvecThreads] = xv[u].y;
-                    s2[u * kMatvecThreads] = xv[u].z;
-                    s3[u * kMatvecThreads] = xv[u].w;
-                }
-            }
-        }
-        // the one barrier of a layer: layer k's activations (and, at k = 0, the table) are in place, and every partial
-        // sum of layer k - 1 is written
-        __syncthreads();
-        if (k > 0) {
-            // layer k - 1: one wave per row adds the row's partial sums in a fixed order
-            const float *part = part0 + ((k - 1) & 1) * part_floats;
-            for (int r = wave; r < prev.rows; r += kMatvecWaves) {
-                float y = 0.f;
-                for (int i = lane; i < prev.npr; i += kWave) y += part[r * prev.npr + i];
-                y = wave_sum(y);
-                if (lane == 63) prev.out[prev.row0 + r] = float_to_half_bits(y);
-            }
-        }
-        if (k == count) break;
-        const bool has_next = k + 1 < count;
-        Work nxt = cur;
-        if (has_next) {
-            nxt = setup(k + 1);
-            load_x(nxt, xv);
-        }
-        const Work w = cur;
-        const uint32_t *const sx = sx0 + (k & 1) * xslot_words;
-        float *const part = part0 + (k & 1) * part_floats;
-        const int pstride = w.npr;
-        int ld_slab = w.first_slab, ld_idx = w.first_idx;       // the load cursor stands at the item requested last
-        SlabView ld = view(w, ld_slab);
-        int slab = w.first_slab, idx = w.first_idx, cur_slab = -1;
-        SlabView sv = view(w, slab);
-        int l = 0, sub = 0;
-        uint32_t part_lane = 0;
-        uint64_t first_lanes = 0;
-        if (w.it_begin == w.it_end && has_next) load_first(nxt, buf, cw);
-        for (int base = w.it_begin; base < w.it_end; base++) {
-            const Elem<WORDS> e = buf;
-            const uint32_t ccw = cw;
-            if (base + 1 < w.it_end) {
-                if (++ld_idx == ld.items) {
-                    ld_idx = 0;
-                    ld_slab++;
-                    ld = view(w, ld_slab);
-                }
-                const int row_first = ld_idx * ld.rows_per_item;
-                const int rows_here = min(ld.rows_per_item, w.rows - row_first);
-                if (lane < rows_here * ld.lanes) {
-                    const global_words wave_base = w.comp + (size_t)(ld.elem0 + (uint32_t)(w.row0 + row_first) * (uint32_t)ld.lanes) * WORDS;
-                    buf = load_element(wave_base, lane);
-                    if (MODE == RPTC_CONTINUOUS && ld_slab > 0) {
-                        const int lsub = ld_slab < w.T ? lane >> 5 : lane / ld.lanes;
-                        const int ll = lane - lsub * ld.lanes;
-                        if (ll == 0)
-                            cw = w.comp[(((size_t)(ld_slab - 1) * w.m + w.row0 + row_first + lsub) * 32 + 31) * WORDS + WORDS - 1];
-                    }
-                }
-            } else if (has_next) {
-                load_first(nxt, buf, cw);            // the next layer's first element travels while this one is decoded
-            }
-            if (slab != cur_slab) {
-                cur_slab = slab;
-                if (slab < w.T) {
-                    sub = lane >> 5;
-                    l = lane & 31;
-                } else {
-                    sub = lane / sv.lanes;
-                    l = lane - sub * sv.lanes;
-                    if (sub >= sv.rows_per_item) l = 0;
-                }
-                // step q of element l multiplies pair slot(slab, q, l) (inference.cu:249): 32 slots, sv.lanes apart
-                // (plain LDS reads: the compiler forms the 32 addresses and waits for the data itself)
-                const uint32_t *xp = sx + (slab < w.T ? 1024 * slab : 1024 * w.T) + l;
-#pragma unroll
-                for (int q = 0; q < 32; q++) xr[q] = xp[q * sv.lanes];
-                first_lanes = __builtin_amdgcn_ballot_w64(l == 0);
-                part_lane = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(part)) + 4u * (uint32_t)(sub * pstride + sv.part_off + l);
-            }
-            const int row_first = idx * sv.rows_per_item;
-            const int nact = max(min(sv.rows_per_item, w.rows - row_first), 0) * sv.lanes;
-            const uint64_t keep = nact >= 64 ? ~0ull : (1ull << nact) - 1ull;
-            const uint32_t last = e.w[WORDS - 1];
-            const uint32_t own = MODE == RPTC_CONTINUOUS ? (slab > 0 ? ccw : 0u) : last;
-            float a0, a1, a2, a3;
-            decode_element_asm(make_uint4(e.w[0], e.w[1], e.w[2], e.w[3]), own, first_lanes, lane4, xr, a0, a1, a2, a3);
-            const float sum = (a0 + a1) + (a2 + a3);
-            if ((keep >> lane) & 1ull) {
-                typedef __attribute__((address_space(3))) float lds_float;
-                *reinterpret_cast<lds_float *>(static_cast<uintptr_t>(part_lane + 4u * (uint32_t)(row_first * pstride))) = sum;
-            }
-            if (++idx == sv.items) {
-                idx = 0;
-                slab++;
-                sv = view(w, slab);
-            }
-        }
-        prev = cur;
-        cur = nxt;
-    }
-}
-
 template <int S, int MODE>
 __global__ __launch_bounds__(256) void matvec_dense_kernel(
     const uint4 *__restrict__ comp, const uint32_t *__restrict__ codebook, uint32_t *__restrict__ W,
@@ -1265,60 +1014,6 @@ int prepare_matvec()
     RPTC_SET_LIMITS(kXAddRmsNorm)
 #undef RPTC_SET_LIMITS
     return 0;
-}
-
-int prepare_matvec_loop()
-{
-    int rc;
-    if ((rc = set_lds_limit(matvec_loop_kernel<6, RPTC_AS_WRITTEN>))) return rc;
-    if ((rc = set_lds_limit(matvec_loop_kernel<6, RPTC_CONTINUOUS>))) return rc;
-    if ((rc = set_lds_limit(matvec_loop_kernel<8, RPTC_AS_WRITTEN>))) return rc;
-    return set_lds_limit(matvec_loop_kernel<8, RPTC_CONTINUOUS>);
-}
-
-int matvec_loop_plan(const rptc_chain_layer *layers, int64_t count, int cus, LoopLayer *out, int *xslot_words,
-                     int *part_floats, int *lds_bytes)
-{
-    int64_t n_max = 0, part_max = 0;
-    for (int64_t k = 0; k < count; k++) {
-        const rptc_chain_layer &u = layers[k];
-        if (u.n > (int64_t)8 * kXRegs * kMatvecThreads) return RPTC_ELIMIT;      // a thread's two registers hold its share
-        LoopLayer &d = out[k];
-        d = LoopLayer{};
-        d.comp = reinterpret_cast<const uint32_t *>(u.compressed);
-        d.x = reinterpret_cast<const uint4 *>(u.x);
-        d.out = u.out;
-        d.m = (int32_t)u.m;
-        d.n = (int32_t)u.n;
-        d.rows_per_block = 2 * (int32_t)((u.m + 2 * cus - 1) / (2 * cus));
-        const int lt = (int)((u.n & 2047) >> 6), items_full = d.rows_per_block / 2;
-        d.rw_tail = lt ? 64 / lt : 1;
-        d.items_tail = lt ? (d.rows_per_block + d.rw_tail - 1) / d.rw_tail : 0;
-        d.full_magic = items_full > 1 ? (uint32_t)(((uint64_t)1 << 32) / (uint64_t)items_full) + 1u : 0u;
-        if (u.n > n_max) n_max = u.n;
-        const int64_t part = (int64_t)d.rows_per_block * (u.n / 64);
-        if (part > part_max) part_max = part;
-    }
-    const int64_t bytes = kTableBytes + 2 * (2 * n_max) + 2 * 4 * part_max;
-    if (bytes > kMaxLds) return RPTC_ELIMIT;
-    *xslot_words = (int)(n_max / 2);
-    *part_floats = (int)part_max;
-    *lds_bytes = (int)bytes;
-    return 0;
-}
-
-int matvec_loop_launch(const LoopLayer *device_layers, const uint32_t *codebook, int count, int xslot_words,
-                       int part_floats, int lds_bytes, int grid, int S, int carry_mode, hipStream_t stream)
-{
-#define RPTC_LOOP_GO(SS, MM)                                                                                          \
-    hipLaunchKernelGGL((matvec_loop_kernel<SS, MM>), dim3(grid), dim3(kMatvecThreads), lds_bytes, stream, device_layers, \
-                       codebook, count, xslot_words, part_floats)
-    if (S == 6 && carry_mode == RPTC_AS_WRITTEN) RPTC_LOOP_GO(6, RPTC_AS_WRITTEN);
-    else if (S == 6) RPTC_LOOP_GO(6, RPTC_CONTINUOUS);
-    else if (carry_mode == RPTC_AS_WRITTEN) RPTC_LOOP_GO(8, RPTC_AS_WRITTEN);
-    else RPTC_LOOP_GO(8, RPTC_CONTINUOUS);
-#undef RPTC_LOOP_GO
-    return (int)hipGetLastError();
 }
 
 }  // namespace rptc
