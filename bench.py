@@ -102,6 +102,7 @@ def aids_library():
     lib.rptc_probe_empty.argtypes = [ctypes.c_int, ctypes.c_void_p]
     lib.rptc_probe_read.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p]
     lib.rptc_probe_valu.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
+    lib.rptc_probe_decode.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
     return lib
 
 
@@ -482,7 +483,8 @@ def bench_valu_probe(a):
     import torch
     aids = aids_library()
     cus = torch.cuda.get_device_properties(0).multi_processor_count
-    names = ["v_dot2c_f32_f16", "v_pk_mad_u16", "v_perm_b32", "v_alignbit_b32", "v_and_or_b32", "v_fma_f32"]
+    names = ["v_dot2c_f32_f16", "v_pk_mad_u16", "v_perm_b32", "v_alignbit_b32", "v_and_or_b32", "v_fma_f32",
+             "v_dot2c_f32_f16 on four sums in turn"]
     iters = 4000
     res = {}
     stream = torch.cuda.current_stream().cuda_stream
@@ -498,12 +500,28 @@ def bench_valu_probe(a):
             t = e0.elapsed_time(e1) * 1e6 / (iters * 32 * 4)          # ns per instruction and SIMD (4 waves a SIMD)
             best = t if best is None or t < best else best
         res[name] = round(best, 4)
+    # the decode block by itself (registers and the LDS table only) at 1, 2 and 4 waves a SIMD
+    decode = {}
+    for threads in (256, 512, 1024):
+        best = None
+        n_el = 3000
+        for rep in range(4):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            rc = aids.rptc_probe_decode(n_el, threads, cus, None, ctypes.c_void_p(stream))
+            assert rc == 0, rc
+            e1.record()
+            torch.cuda.synchronize()
+            t = e0.elapsed_time(e1) * 1e6 / (n_el * (threads // 256))      # ns per element and SIMD
+            best = t if best is None or t < best else best
+        decode[f"{threads // 256} waves a SIMD"] = round(best, 2)
     fma = res["v_fma_f32"]
     rel = {k: round(v / fma, 3) for k, v in res.items()}
     per_element = 12 * res["v_alignbit_b32"] + 16 * res["v_pk_mad_u16"] + 16 * res["v_perm_b32"] + 16 * res["v_and_or_b32"] + 32 * res["v_dot2c_f32_f16"]
     print(json.dumps({"metric": "vector instruction issue time, ns per instruction and SIMD", "unit": "ns", "n_gpus": 1,
                       "config": {"waves_per_simd": 4, "instructions_per_wave": iters * 32}, "results": res,
-                      "relative_to_v_fma_f32": rel,
+                      "relative_to_v_fma_f32": rel, "decode_block_ns_per_element_and_simd": decode,
+                      "decode_block_us_per_4096x11008_layer": round(12 * decode["4 waves a SIMD"] / 1e3, 3),
                       "decode_valu_us_per_4096x11008_layer": round(12 * per_element / 1e3, 3)}))
 
 

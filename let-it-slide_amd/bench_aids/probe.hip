@@ -6,6 +6,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "../csrc/decode_asm.hpp"
+
 namespace {
 
 __global__ __launch_bounds__(1024) void probe_empty_kernel() {}
@@ -46,6 +48,11 @@ __global__ __launch_bounds__(1024) void probe_read_kernel(const uint32_t *__rest
 #define RPTC_I_ALIGN(R) "v_alignbit_b32 " #R ", " #R ", %8, 7\n"
 #define RPTC_I_ANDOR(R) "v_and_or_b32 " #R ", " #R ", %10, %9\n"
 #define RPTC_I_FMA(R) "v_fma_f32 " #R ", %8, %9, " #R "\n"
+// v_dot2c_f32_f16 on four sums in turn, as the decode block has them (a sum is added to every fourth instruction)
+#define RPTC_PROBE_4X2(TEXT)                                                                                          \
+    asm volatile(TEXT(%0) TEXT(%1) TEXT(%2) TEXT(%3) TEXT(%0) TEXT(%1) TEXT(%2) TEXT(%3)                              \
+                 : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]), "+v"(r[4]), "+v"(r[5]), "+v"(r[6]), "+v"(r[7])   \
+                 : "v"(a), "v"(b), "s"(sel))
 
 template <int KIND>
 __global__ __launch_bounds__(1024) void probe_valu_kernel(int iters, uint32_t seed, uint32_t *sink)
@@ -63,7 +70,8 @@ __global__ __launch_bounds__(1024) void probe_valu_kernel(int iters, uint32_t se
             else if (KIND == 2) RPTC_PROBE_8(RPTC_I_PERM);
             else if (KIND == 3) RPTC_PROBE_8(RPTC_I_ALIGN);
             else if (KIND == 4) RPTC_PROBE_8(RPTC_I_ANDOR);
-            else RPTC_PROBE_8(RPTC_I_FMA);
+            else if (KIND == 5) RPTC_PROBE_8(RPTC_I_FMA);
+            else RPTC_PROBE_4X2(RPTC_I_DOT2C);
         }
     }
     uint32_t x = 0;
@@ -72,13 +80,56 @@ __global__ __launch_bounds__(1024) void probe_valu_kernel(int iters, uint32_t se
     if (x == 0x9E3779B9u && sink) sink[0] = x;
 }
 
+// The decode block of the mat-vec by itself: every wave decodes `iters` stream elements that it makes up from
+// registers (no global memory, the 64 KiB table in LDS as in the kernels), so the time per element and SIMD is what the
+// block costs at that number of waves a SIMD with nothing else in the way.
+__global__ void probe_decode_kernel(int iters, uint32_t seed, uint32_t *sink)
+{
+    extern __shared__ uint32_t probe_lds[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    for (int i = tid; i < 16384; i += blockDim.x) probe_lds[i] = 0x3C003800u + (uint32_t)(i >> 6);
+    __syncthreads();
+    const uint32_t lane4 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(probe_lds)) + lane * 4;
+    uint32_t xr[32];
+#pragma unroll
+    for (int q = 0; q < 32; q++) xr[q] = 0x38003C00u + (uint32_t)q;
+    uint4 e = make_uint4(seed + tid, seed * 3u + tid, seed * 5u + tid, seed * 7u + tid);
+    const uint64_t first_lanes = 0x0000000100000001ull;
+    float acc = 0.f;
+    for (int it = 0; it < iters; it++) {
+        float a0, a1, a2, a3;
+        rptc::decode_element_asm(e, e.w, first_lanes, lane4, xr, a0, a1, a2, a3);
+        acc += (a0 + a1) + (a2 + a3);
+        e.x += 0x9E3779B9u;          // the next element (a scalar-cheap change; the block does not depend on the last one)
+        e.z ^= e.x;
+    }
+    if (__builtin_bit_cast(uint32_t, acc) == 0x9E3779B9u && sink) sink[0] = 1u;
+}
+
 }  // namespace
 
+// `iters` elements decoded by every wave of `workgroups` workgroups of `threads` threads (64..1024: 1 to 4 waves a SIMD)
+extern "C" int rptc_probe_decode(int iters, int threads, int workgroups, void *sink, void *stream)
+{
+    if (iters < 1 || threads < 64 || threads > 1024 || threads % 64 || workgroups < 1) return -2;
+    static bool allowed = false;
+    if (!allowed) {
+        int rc = (int)hipFuncSetAttribute(reinterpret_cast<const void *>(probe_decode_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (rc) return rc;
+        allowed = true;
+    }
+    // 150 KiB of LDS: one workgroup per compute unit, as the mat-vec has it
+    hipLaunchKernelGGL(probe_decode_kernel, dim3(workgroups), dim3(threads), 150 * 1024, static_cast<hipStream_t>(stream), iters, 12345u,
+                       static_cast<uint32_t *>(sink));
+    return (int)hipGetLastError();
+}
+
 // `iters` rounds of 32 vector instructions of one kind in every wave of `workgroups` 1024-thread workgroups;
-// kind: 0 v_dot2c_f32_f16, 1 v_pk_mad_u16, 2 v_perm_b32, 3 v_alignbit_b32, 4 v_and_or_b32, 5 v_fma_f32
+// kind: 0 v_dot2c_f32_f16, 1 v_pk_mad_u16, 2 v_perm_b32, 3 v_alignbit_b32, 4 v_and_or_b32, 5 v_fma_f32,
+// 6 v_dot2c_f32_f16 on four sums in turn instead of eight
 extern "C" int rptc_probe_valu(int kind, int iters, int workgroups, void *sink, void *stream)
 {
-    if (kind < 0 || kind > 5 || iters < 1 || workgroups < 1) return -2;
+    if (kind < 0 || kind > 6 || iters < 1 || workgroups < 1) return -2;
     hipStream_t s = static_cast<hipStream_t>(stream);
     uint32_t *out = static_cast<uint32_t *>(sink);
 #define RPTC_PROBE_GO(K) hipLaunchKernelGGL(probe_valu_kernel<K>, dim3(workgroups), dim3(1024), 0, s, iters, 12345u, out)
@@ -88,7 +139,8 @@ extern "C" int rptc_probe_valu(int kind, int iters, int workgroups, void *sink, 
     case 2: RPTC_PROBE_GO(2); break;
     case 3: RPTC_PROBE_GO(3); break;
     case 4: RPTC_PROBE_GO(4); break;
-    default: RPTC_PROBE_GO(5); break;
+    case 5: RPTC_PROBE_GO(5); break;
+    default: RPTC_PROBE_GO(6); break;
     }
 #undef RPTC_PROBE_GO
     return (int)hipGetLastError();

@@ -23,6 +23,7 @@
 //     wait for are issued first and every wave's stream loads right behind them, before the
 //     table is built; kernel arguments are preloaded into SGPRs.
 #include "decode_asm.hpp"
+#include "matvec_loop.hpp"
 #include "hadamard_pass.hpp"
 #include "rptc_common.hpp"
 
@@ -716,6 +717,279 @@ __global__ __launch_bounds__(kMatvecThreads) void matvec_affine_kernel(
 }
 
 // Dense export: one thread per stream element, 32 pairs scattered to their columns.
+// ------------------------------------------------------------------------------------------------------------
+// A chain of independent layers in one launch: the body above in a loop over layers (2 bits, plain activations, one
+// partial sum per stream element).  What a launch per layer pays every time is paid once or hidden:
+//   * the table is written once;
+//   * a layer costs ONE workgroup barrier: two activation images and two sets of partial sums take turns, so the
+//     barrier that publishes layer k's activations is also the one behind which layer k - 1's rows are added up;
+//   * everything layer k + 1 reads from memory -- all of a wave's stream elements (at most MAXI) and a thread's share of
+//     the activations -- is requested when layer k's decode starts, into registers of their own: it has a whole layer
+//     to arrive, and nothing in the loop ever waits for a request it has just made.
+// Layers must not depend on each other (the host checks the addresses): nothing orders a layer's reads behind another
+// layer's writes.  Every load is unconditional (clamped addresses), so the compiler counts them exactly.
+template <int S, int MODE, int MAXI>
+__global__ __launch_bounds__(kMatvecThreads) void matvec_loop_kernel(
+    const LoopLayer *__restrict__ layers, const uint32_t *__restrict__ codebook, int count, int xslot_words, int part_floats)
+{
+    constexpr int WORDS = 4;
+    extern __shared__ uint32_t lds[];
+    uint32_t *const sx0 = lds + kTableBytes / 4;                                   // two activation images, slot order
+    float *const part0 = reinterpret_cast<float *>(sx0 + 2 * xslot_words);         // two sets of [row in block][n / 64]
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t lane4 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds)) + lane * 4;   // the table is at LDS address 0
+
+    // The pointers come out of a descriptor in memory, so their address space is stated: global loads and stores,
+    // not flat ones.
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    typedef const __attribute__((address_space(1))) uint32_t *global_words;
+    typedef const __attribute__((address_space(1))) u32x4 *global_vec4;
+    typedef __attribute__((address_space(1))) uint16_t *global_halves;
+    struct Work {                 // a layer as this wave sees it (all wave-uniform)
+        global_words comp;
+        global_vec4 x;
+        global_halves out;
+        int m, T, Lt, npr, n8, rw_tail, items_full, items_tail;
+        int row0, rows;           // rows <= 0: no row of this layer is this workgroup's
+        int it_begin, it_end, first_slab, first_idx;
+    };
+    // `like`: the layer in front; a layer of the same shape takes its geometry over and reads the three pointers only
+    // (chains of equal layers are the common case, and the set-up is ~200 scalar instructions of every wave)
+    auto setup = [&](int k, const Work &like, bool have_like) {
+        Work w;
+        const LoopLayer &d = layers[k];
+        if (have_like && d.same_shape_as_previous) {
+            w = like;
+            w.comp = reinterpret_cast<global_words>(reinterpret_cast<uintptr_t>(d.comp));
+            w.x = reinterpret_cast<global_vec4>(reinterpret_cast<uintptr_t>(d.x));
+            w.out = reinterpret_cast<global_halves>(reinterpret_cast<uintptr_t>(d.out));
+            return w;
+        }
+        const int n = d.n, rpb = d.rows_per_block;
+        w.comp = reinterpret_cast<global_words>(reinterpret_cast<uintptr_t>(d.comp));
+        w.x = reinterpret_cast<global_vec4>(reinterpret_cast<uintptr_t>(d.x));
+        w.out = reinterpret_cast<global_halves>(reinterpret_cast<uintptr_t>(d.out));
+        w.m = d.m;
+        w.T = n >> 11, w.Lt = (n & 2047) >> 6, w.npr = n >> 6, w.n8 = n >> 3;
+        w.rw_tail = d.rw_tail, w.items_full = rpb >> 1, w.items_tail = d.items_tail;
+        w.row0 = blockIdx.x * rpb;
+        w.rows = min(rpb, w.m - w.row0);
+        // equal shares: the first total % 16 waves take one element more (at most MAXI each: the host checks)
+        const int total = w.rows > 0 ? w.T * w.items_full + w.items_tail : 0;
+        const int per_wave = (int)((uint32_t)total / kMatvecWaves), extra = (int)((uint32_t)total % kMatvecWaves);
+        w.it_begin = wave * per_wave + min(wave, extra);
+        w.it_end = w.it_begin + per_wave + (wave < extra ? 1 : 0);
+        int first_slab = w.items_full == 1 ? w.it_begin : (int)__umulhi((uint32_t)w.it_begin, d.full_magic);
+        w.first_slab = min(first_slab, w.T);
+        w.first_idx = w.it_begin - w.first_slab * w.items_full;
+        return w;
+    };
+    auto view = [&](const Work &w, int slab) {
+        SlabView v;
+        const bool full = slab < w.T;
+        v.lanes = full ? 32 : w.Lt;
+        v.rows_per_item = full ? 2 : w.rw_tail;
+        v.items = full ? w.items_full : w.items_tail;
+        v.part_off = slab * 32;
+        v.elem0 = (uint32_t)(full ? slab : w.T) * (uint32_t)w.m * 32u;
+        return v;
+    };
+    // a thread's share of a layer's activations (every lane asks, with a clamped index)
+    auto load_x = [&](const Work &w, uint4 (&xv)[kXRegs]) {
+#pragma unroll
+        for (int u = 0; u < kXRegs; u++) {
+            const u32x4 v = w.x[min(tid + u * kMatvecThreads, w.n8 - 1)];
+            xv[u] = make_uint4(v.x, v.y, v.z, v.w);
+        }
+    };
+    // All of the wave's elements of layer w, requested by every lane whatever the wave holds: a lane past the item's
+    // rows repeats the last lane's address, and a slot the wave has no item for asks for the first element of the
+    // stream in every lane (one cache line).
+    auto load_items = [&](const Work &w, Elem<WORDS> (&buf)[MAXI], uint32_t (&cw)[MAXI]) {
+        int slab = w.first_slab, idx = w.first_idx;
+        SlabView ld = view(w, slab);
+#pragma unroll
+        for (int u = 0; u < MAXI; u++) {
+            const int row_first = idx * ld.rows_per_item;
+            const int rows_here = min(ld.rows_per_item, w.rows - row_first);
+            const bool real = w.it_begin + u < w.it_end && rows_here > 0;
+            const uint32_t elem = real ? ld.elem0 + (uint32_t)(w.row0 + row_first) * (uint32_t)ld.lanes : 0u;
+            const uint32_t last = real ? (uint32_t)(rows_here * ld.lanes - 1) : 0u;
+            const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<global_vec4>(w.comp + ((size_t)elem + min((uint32_t)lane, last)) * WORDS));
+            buf[u].w[0] = v.x, buf[u].w[1] = v.y, buf[u].w[2] = v.z, buf[u].w[3] = v.w;
+            if (MODE == RPTC_CONTINUOUS) {
+                // the word in front of a row: last word of the row's lane 31 in the slab before (read by all lanes of
+                // the row; used by its first lane, and only past slab 0)
+                const bool prev = real && slab > 0;
+                const int sub = min(slab < w.T ? lane >> 5 : lane / max(ld.lanes, 1), max(rows_here, 1) - 1);
+                const global_words row_base =
+                    prev ? w.comp + (((size_t)(slab - 1) * w.m + w.row0 + row_first) * 32 + 31) * WORDS + WORDS - 1 : w.comp;
+                cw[u] = row_base[sub * (prev ? 32 * WORDS : 0)];
+            }
+            if (real && ++idx == ld.items) {
+                idx = 0;
+                slab++;
+                ld = view(w, slab);
+            }
+        }
+    };
+
+    Work cur = setup(0, Work{}, false), prev = cur, nxt = count > 1 ? setup(1, cur, true) : cur;
+    uint4 xv[kXRegs];
+    Elem<WORDS> buf[MAXI], nbuf[MAXI];
+    uint32_t cw[MAXI], ncw[MAXI];
+#pragma unroll
+    for (int u = 0; u < MAXI; u++) cw[u] = ncw[u] = 0;
+    // requests first (the activations, then the stream), the table behind them
+    constexpr int kRowsPerWave = 256 / kMatvecWaves;
+    uint32_t cbv[kRowsPerWave];
+#pragma unroll
+    for (int i = 0; i < kRowsPerWave; i++) cbv[i] = codebook[(kRowsPerWave * wave + i) & ((1 << S) - 1)];
+    const uint32_t table_sign = (uint32_t)((kRowsPerWave * wave) >> 7) << 15;
+    load_x(cur, xv);
+    load_items(cur, nbuf, ncw);
+#pragma unroll
+    for (int i = 0; i < kRowsPerWave; i++) {
+        uint32_t tv;
+        asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(tv) : "s"(cbv[i]), "v"(0xFFFF7FFFu), "v"(table_sign));
+        lds[(kRowsPerWave * wave + i) * 64 + lane] = tv;
+    }
+    // a layer's activations into an image (halves 8 idx .. 8 idx + 7 to the four planes, inference.cu:215-221)
+    auto stage_x = [&](uint32_t *sx, int n8) {
+        uint32_t *const s0 = sx + tid, *const s1 = s0 + n8, *const s2 = s1 + n8, *const s3 = s2 + n8;
+#pragma unroll
+        for (int u = 0; u < kXRegs; u++) {
+            if (tid + u * kMatvecThreads < n8) {
+                s0[u * kMatvecThreads] = xv[u].x;
+                s1[u * kMatvecThreads] = xv[u].y;
+                s2[u * kMatvecThreads] = xv[u].z;
+                s3[u * kMatvecThreads] = xv[u].w;
+            }
+        }
+    };
+    // one wave per row adds the row's partial sums in a fixed order
+    auto write_rows = [&](const Work &w, const float *part) {
+        for (int r = wave; r < w.rows; r += kMatvecWaves) {
+            float y = 0.f;
+            for (int i = lane; i < w.npr; i += kWave) y += part[r * w.npr + i];
+            y = wave_sum(y);
+            if (lane == 63) w.out[w.row0 + r] = float_to_half_bits(y);
+        }
+    };
+    stage_x(sx0, cur.n8);
+    // Layer 0's elements change registers here, as every later layer's do at the end of the iteration before: the loop
+    // is entered with no request in flight, so the compiler puts no wait for memory in front of a decode.
+#pragma unroll
+    for (int u = 0; u < MAXI; u++) {
+        buf[u] = nbuf[u];
+        cw[u] = ncw[u];
+    }
+
+    uint32_t xr[32];
+#pragma unroll
+    for (int q = 0; q < 32; q++) xr[q] = 0;
+    // Iteration k, behind the layer's one barrier (layer k's activations are in image k & 1 and every partial sum of
+    // layer k - 1 is written): request what layer k + 1 reads, decode layer k from registers filled a layer ago, then
+    // the rows of layer k - 1, the activations of layer k + 1 into the other image, the geometry of layer k + 2.
+    for (int k = 0; k < count; k++) {
+        __syncthreads();
+        const bool has_next = k + 1 < count;
+        if (has_next) {
+            load_x(nxt, xv);
+            load_items(nxt, nbuf, ncw);
+        }
+        const Work w = cur;
+        const uint32_t *const sx = sx0 + (k & 1) * xslot_words;
+        float *const part = part0 + (k & 1) * part_floats;
+        const int pstride = w.npr;
+        int slab = w.first_slab, idx = w.first_idx, cur_slab = -1;
+        SlabView sv = view(w, slab);
+        int l = 0, sub = 0;
+        uint32_t part_lane = 0;
+        uint64_t first_lanes = 0;
+#pragma unroll
+        for (int u = 0; u < MAXI; u++) {
+            if (w.it_begin + u >= w.it_end) break;
+            if (slab != cur_slab) {
+                cur_slab = slab;
+                if (slab < w.T) {
+                    sub = lane >> 5;
+                    l = lane & 31;
+                } else {
+                    sub = lane / sv.lanes;
+                    l = lane - sub * sv.lanes;
+                    if (sub >= sv.rows_per_item) l = 0;
+                }
+                // step q of element l multiplies pair slot(slab, q, l) (inference.cu:249): 32 slots, sv.lanes apart
+                // (plain LDS reads: the compiler forms the 32 addresses and waits for the data itself)
+                const uint32_t *xp = sx + (slab < w.T ? 1024 * slab : 1024 * w.T) + l;
+                if (slab < w.T) {
+                    // One address and 32 immediate offsets.  The reads and their wait are ONE statement: a register
+                    // that such a read writes holds nothing until the wait, and between two statements the compiler
+                    // may copy or reuse it.  Early-clobber outputs: none may share the address register.
+                    const uint32_t xa = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(xp));
+                    asm volatile(
+                        "ds_read_b32 %0, %32 offset:0\n ds_read_b32 %1, %32 offset:128\n ds_read_b32 %2, %32 offset:256\n"
+                        "ds_read_b32 %3, %32 offset:384\n ds_read_b32 %4, %32 offset:512\n ds_read_b32 %5, %32 offset:640\n"
+                        "ds_read_b32 %6, %32 offset:768\n ds_read_b32 %7, %32 offset:896\n ds_read_b32 %8, %32 offset:1024\n"
+                        "ds_read_b32 %9, %32 offset:1152\n ds_read_b32 %10, %32 offset:1280\n ds_read_b32 %11, %32 offset:1408\n"
+                        "ds_read_b32 %12, %32 offset:1536\n ds_read_b32 %13, %32 offset:1664\n ds_read_b32 %14, %32 offset:1792\n"
+                        "ds_read_b32 %15, %32 offset:1920\n ds_read_b32 %16, %32 offset:2048\n ds_read_b32 %17, %32 offset:2176\n"
+                        "ds_read_b32 %18, %32 offset:2304\n ds_read_b32 %19, %32 offset:2432\n ds_read_b32 %20, %32 offset:2560\n"
+                        "ds_read_b32 %21, %32 offset:2688\n ds_read_b32 %22, %32 offset:2816\n ds_read_b32 %23, %32 offset:2944\n"
+                        "ds_read_b32 %24, %32 offset:3072\n ds_read_b32 %25, %32 offset:3200\n ds_read_b32 %26, %32 offset:3328\n"
+                        "ds_read_b32 %27, %32 offset:3456\n ds_read_b32 %28, %32 offset:3584\n ds_read_b32 %29, %32 offset:3712\n"
+                        "ds_read_b32 %30, %32 offset:3840\n ds_read_b32 %31, %32 offset:3968\n s_waitcnt lgkmcnt(0)\n"
+                        : "=&v"(xr[0]), "=&v"(xr[1]), "=&v"(xr[2]), "=&v"(xr[3]), "=&v"(xr[4]), "=&v"(xr[5]), "=&v"(xr[6]), "=&v"(xr[7]),
+                          "=&v"(xr[8]), "=&v"(xr[9]), "=&v"(xr[10]), "=&v"(xr[11]), "=&v"(xr[12]), "=&v"(xr[13]), "=&v"(xr[14]),
+                          "=&v"(xr[15]), "=&v"(xr[16]), "=&v"(xr[17]), "=&v"(xr[18]), "=&v"(xr[19]), "=&v"(xr[20]), "=&v"(xr[21]),
+                          "=&v"(xr[22]), "=&v"(xr[23]), "=&v"(xr[24]), "=&v"(xr[25]), "=&v"(xr[26]), "=&v"(xr[27]), "=&v"(xr[28]),
+                          "=&v"(xr[29]), "=&v"(xr[30]), "=&v"(xr[31])
+                        : "v"(xa)
+                        : "memory");
+                } else {
+#pragma unroll
+                    for (int q = 0; q < 32; q++) xr[q] = xp[q * sv.lanes];
+                }
+                first_lanes = __builtin_amdgcn_ballot_w64(l == 0);
+                part_lane = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(part)) + 4u * (uint32_t)(sub * pstride + sv.part_off + l);
+            }
+            const int row_first = idx * sv.rows_per_item;
+            const int nact = max(min(sv.rows_per_item, w.rows - row_first), 0) * sv.lanes;
+            const uint64_t keep = nact >= 64 ? ~0ull : (1ull << nact) - 1ull;
+            const uint32_t last = buf[u].w[WORDS - 1];
+            const uint32_t own = MODE == RPTC_CONTINUOUS ? (slab > 0 ? cw[u] : 0u) : last;
+            float a0, a1, a2, a3;
+            decode_element_asm(make_uint4(buf[u].w[0], buf[u].w[1], buf[u].w[2], buf[u].w[3]), own, first_lanes, lane4, xr, a0, a1, a2, a3);
+            const float sum = (a0 + a1) + (a2 + a3);
+            if ((keep >> lane) & 1ull) {
+                typedef __attribute__((address_space(3))) float lds_float;
+                *reinterpret_cast<lds_float *>(static_cast<uintptr_t>(part_lane + 4u * (uint32_t)(row_first * pstride))) = sum;
+            }
+            if (++idx == sv.items) {
+                idx = 0;
+                slab++;
+                sv = view(w, slab);
+            }
+        }
+        if (k > 0) write_rows(prev, part0 + ((k - 1) & 1) * part_floats);
+        if (has_next) {
+            stage_x(sx0 + ((k + 1) & 1) * xslot_words, nxt.n8);
+#pragma unroll
+            for (int u = 0; u < MAXI; u++) {
+                buf[u] = nbuf[u];
+                cw[u] = ncw[u];
+            }
+        }
+        prev = cur;
+        cur = nxt;
+        if (k + 2 < count) nxt = setup(k + 2, cur, true);
+    }
+    __syncthreads();
+    write_rows(prev, part0 + ((count - 1) & 1) * part_floats);
+}
+
 template <int S, int MODE>
 __global__ __launch_bounds__(256) void matvec_dense_kernel(
     const uint4 *__restrict__ comp, const uint32_t *__restrict__ codebook, uint32_t *__restrict__ W,
@@ -1014,6 +1288,66 @@ int prepare_matvec()
     RPTC_SET_LIMITS(kXAddRmsNorm)
 #undef RPTC_SET_LIMITS
     return 0;
+}
+
+constexpr int kLoopMaxItems = 3;      // stream elements of a layer a wave holds in registers
+
+int prepare_matvec_loop()
+{
+    int rc;
+    if ((rc = set_lds_limit(matvec_loop_kernel<6, RPTC_AS_WRITTEN, kLoopMaxItems>))) return rc;
+    if ((rc = set_lds_limit(matvec_loop_kernel<6, RPTC_CONTINUOUS, kLoopMaxItems>))) return rc;
+    if ((rc = set_lds_limit(matvec_loop_kernel<8, RPTC_AS_WRITTEN, kLoopMaxItems>))) return rc;
+    return set_lds_limit(matvec_loop_kernel<8, RPTC_CONTINUOUS, kLoopMaxItems>);
+}
+
+int matvec_loop_plan(const rptc_chain_layer *layers, int64_t count, int cus, LoopLayer *out, int *xslot_words,
+                     int *part_floats, int *lds_bytes)
+{
+    int64_t n_max = 0, part_max = 0;
+    for (int64_t k = 0; k < count; k++) {
+        const rptc_chain_layer &u = layers[k];
+        if (u.n > (int64_t)8 * kXRegs * kMatvecThreads) return RPTC_ELIMIT;      // a thread's two registers hold its share
+        LoopLayer &d = out[k];
+        d = LoopLayer{};
+        d.comp = reinterpret_cast<const uint32_t *>(u.compressed);
+        d.x = reinterpret_cast<const uint4 *>(u.x);
+        d.out = u.out;
+        d.m = (int32_t)u.m;
+        d.n = (int32_t)u.n;
+        d.rows_per_block = 2 * (int32_t)((u.m + 2 * cus - 1) / (2 * cus));
+        const int lt = (int)((u.n & 2047) >> 6), items_full = d.rows_per_block / 2;
+        d.rw_tail = lt ? 64 / lt : 1;
+        d.items_tail = lt ? (d.rows_per_block + d.rw_tail - 1) / d.rw_tail : 0;
+        d.full_magic = items_full > 1 ? (uint32_t)(((uint64_t)1 << 32) / (uint64_t)items_full) + 1u : 0u;
+        d.same_shape_as_previous = k > 0 && layers[k - 1].m == u.m && layers[k - 1].n == u.n;
+        // a wave keeps all its elements of a layer in registers: at most kLoopMaxItems of them
+        const int64_t total = (u.n >> 11) * (int64_t)items_full + d.items_tail;
+        if ((total + kMatvecWaves - 1) / kMatvecWaves > kLoopMaxItems) return RPTC_ELIMIT;
+        if (u.n > n_max) n_max = u.n;
+        const int64_t part = (int64_t)d.rows_per_block * (u.n / 64);
+        if (part > part_max) part_max = part;
+    }
+    const int64_t bytes = kTableBytes + 2 * (2 * n_max) + 2 * 4 * part_max;
+    if (bytes > kMaxLds) return RPTC_ELIMIT;
+    *xslot_words = (int)(n_max / 2);
+    *part_floats = (int)part_max;
+    *lds_bytes = (int)bytes;
+    return 0;
+}
+
+int matvec_loop_launch(const LoopLayer *device_layers, const uint32_t *codebook, int count, int xslot_words,
+                       int part_floats, int lds_bytes, int grid, int S, int carry_mode, hipStream_t stream)
+{
+#define RPTC_LOOP_GO(SS, MM)                                                                                          \
+    hipLaunchKernelGGL((matvec_loop_kernel<SS, MM, kLoopMaxItems>), dim3(grid), dim3(kMatvecThreads), lds_bytes, stream, device_layers, \
+                       codebook, count, xslot_words, part_floats)
+    if (S == 6 && carry_mode == RPTC_AS_WRITTEN) RPTC_LOOP_GO(6, RPTC_AS_WRITTEN);
+    else if (S == 6) RPTC_LOOP_GO(6, RPTC_CONTINUOUS);
+    else if (carry_mode == RPTC_AS_WRITTEN) RPTC_LOOP_GO(8, RPTC_AS_WRITTEN);
+    else RPTC_LOOP_GO(8, RPTC_CONTINUOUS);
+#undef RPTC_LOOP_GO
+    return (int)hipGetLastError();
 }
 
 }  // namespace rptc

@@ -29,6 +29,7 @@
 #include <vector>
 
 #include "decode_asm.hpp"
+#include "matvec_loop.hpp"
 #include "rptc_common.hpp"
 
 namespace rptc {
@@ -519,7 +520,9 @@ struct ChainPlanHost {            // what rptc_chain_t holds (see the header): w
     int32_t count, grid, lds_bytes, nb, xslot_words, part_floats, uses_grid;
     uint32_t arrivals, spin_limit;
     int32_t device;
-    int32_t reserved[3];
+    // a chain without dependencies runs in the per-launch kernel's loop form (matvec.hip) when that fits:
+    int32_t loop_at_256;          // its descriptors start 256 * this many bytes into the descriptor area (0: not used)
+    int32_t loop_lds_bytes, loop_part_floats;
 };
 static_assert(sizeof(ChainPlanHost) <= sizeof(rptc_chain_t), "the public struct holds the plan");
 
@@ -593,7 +596,7 @@ static void chain_build_table(const ChainShape &sh, uint32_t *words)
 // checks the layers and finds the distinct shapes; the layout of the descriptor area is
 // [descriptors][sync words][one item table per shape]
 static int chain_layout(const rptc_chain_layer *layers, int64_t count, int grid, std::vector<ChainShape> *shapes,
-                        std::vector<int> *shape_of, int64_t *total_bytes)
+                        std::vector<int> *shape_of, int64_t *total_bytes, int64_t *loop_at = nullptr)
 {
     if (!layers) return RPTC_ENULL;
     if (count < 1 || count > 65535) return RPTC_ESHAPE;
@@ -625,6 +628,9 @@ static int chain_layout(const rptc_chain_layer *layers, int64_t count, int grid,
         }
         (*shape_of)[(size_t)k] = found;
     }
+    // the descriptors of the loop form (one 64-byte line a layer), used when no layer depends on another
+    if (loop_at) *loop_at = at;
+    at += (count * (int64_t)sizeof(LoopLayer) + 255) & ~(int64_t)255;
     *total_bytes = at;
     return 0;
 }
@@ -656,8 +662,8 @@ extern "C" int rptc_chain_plan(const rptc_chain_layer *layers, int64_t count, vo
     const int grid = dev->cus;
     std::vector<ChainShape> shapes;
     std::vector<int> shape_of;
-    int64_t total_bytes = 0;
-    if ((rc = chain_layout(layers, count, grid, &shapes, &shape_of, &total_bytes))) return rc;
+    int64_t total_bytes = 0, loop_at = 0;
+    if ((rc = chain_layout(layers, count, grid, &shapes, &shape_of, &total_bytes, &loop_at))) return rc;
     if (device_desc_bytes < total_bytes) return RPTC_ELIMIT;
     std::vector<uint32_t> image((size_t)total_bytes / 4, 0u);
     ChainDesc *descs = reinterpret_cast<ChainDesc *>(image.data());
@@ -716,6 +722,12 @@ extern "C" int rptc_chain_plan(const rptc_chain_layer *layers, int64_t count, vo
     }
     if (any)
         for (int64_t k = 0; k < count; k++) descs[k].flags |= kChFence;
+    // No layer reads or writes what another writes (every pair was looked at: without a guarded layer "earlier"
+    // reaches back to the start): the loop form of the per-launch kernel runs the chain when it fits.
+    int loop_xslot_words = 0, loop_part_floats = 0, loop_lds_bytes = 0;
+    const bool loop = !any && (loop_at >> 8) < (int64_t)1 << 31 &&
+                      matvec_loop_plan(layers, count, grid, reinterpret_cast<LoopLayer *>(image.data() + loop_at / 4),
+                                       &loop_xslot_words, &loop_part_floats, &loop_lds_bytes) == 0;
     // the sync words behind the descriptors start at zero
     hipStream_t s = static_cast<hipStream_t>(stream);
     if ((rc = (int)hipMemcpyAsync(device_desc, image.data(), (size_t)total_bytes, hipMemcpyHostToDevice, s))) return rc;
@@ -734,6 +746,11 @@ extern "C" int rptc_chain_plan(const rptc_chain_layer *layers, int64_t count, vo
     p.arrivals = (uint32_t)grid;
     p.spin_limit = 1u << 22;
     p.device = dev->device;
+    if (loop) {
+        p.loop_at_256 = (int32_t)(loop_at >> 8);
+        p.loop_lds_bytes = loop_lds_bytes;
+        p.loop_part_floats = loop_part_floats;       // (the activation image is xslot_words long in both forms)
+    }
     memset(plan, 0, sizeof(*plan));
     memcpy(plan, &p, sizeof(p));
     return 0;
@@ -759,6 +776,13 @@ extern "C" int rptc_decompress_matvec_chain(const rptc_chain_t *plan, const uint
     if (rc) return rc;
     auto a_desc = reinterpret_cast<const ChainDesc *>(p.device_desc);
     auto a_cb = reinterpret_cast<const uint32_t *>(codebook);
+    if (p.loop_at_256 > 0) {
+        if (p.loop_lds_bytes > kMaxLds) return RPTC_EDEVICE;
+        auto a_loop = reinterpret_cast<const LoopLayer *>(static_cast<const char *>(p.device_desc) + ((int64_t)p.loop_at_256 << 8));
+        rc = matvec_loop_launch(a_loop, a_cb, p.count, p.xslot_words, p.loop_part_floats, p.loop_lds_bytes, p.grid, S, carry_mode, s);
+        if (rc) return rc;
+        return t.end();
+    }
     auto a_sync = reinterpret_cast<uint32_t *>(static_cast<char *>(p.device_desc) + (size_t)p.count * sizeof(ChainDesc));
 #define RPTC_CHAIN_GO(SS, MM)                                                                                              \
     hipLaunchKernelGGL((matvec_chain_kernel<SS, MM, kChainDepth>), dim3(p.grid), dim3(kChainThreads), p.lds_bytes, s, a_desc, \

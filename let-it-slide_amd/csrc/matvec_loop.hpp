@@ -1,0 +1,28 @@
+// A chain of independent mat-vecs in one launch of the per-launch kernel's body (matvec.hip): what the chain's host
+// code (matvec_chain.hip) needs to plan and launch it.
+#pragma once
+#include "rptc_common.hpp"
+
+namespace rptc {
+
+struct LoopLayer {               // one layer as the kernel reads it (through the scalar cache): 64 bytes
+    const uint32_t *comp;        // [T][m][32] uint4, then the ragged slab [m][Lt]
+    const uint4 *x;              // fp16 [n]
+    uint16_t *out;               // fp16 [m]
+    int32_t m, n, rows_per_block, rw_tail, items_tail;
+    uint32_t full_magic;         // floor(2^32 / items_full) + 1 (0 for items_full = 1)
+    int32_t same_shape_as_previous;   // m and n equal those of the layer in front: its geometry can be taken over
+    int32_t pad[3];
+};
+static_assert(sizeof(LoopLayer) == 64, "a descriptor is one 64-byte line");
+
+// Fills `out[count]` for a device of `cus` compute units.  Returns 0 when the kernel can run the chain (every layer's
+// activations fit a thread's two registers, two activation images and two sets of partial sums fit in LDS beside the
+// table), RPTC_ELIMIT when it cannot; the caller has checked pointers, shapes and that no layer depends on another.
+int matvec_loop_plan(const rptc_chain_layer *layers, int64_t count, int cus, LoopLayer *out, int *xslot_words,
+                     int *part_floats, int *lds_bytes);
+// One launch over `count` layers whose descriptors are in device memory; returns hipGetLastError()'s value.
+int matvec_loop_launch(const LoopLayer *device_layers, const uint32_t *codebook, int count, int xslot_words,
+                       int part_floats, int lds_bytes, int grid, int S, int carry_mode, hipStream_t stream);
+
+}  // namespace rptc
