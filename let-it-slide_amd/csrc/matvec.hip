@@ -1290,21 +1290,26 @@ int prepare_matvec()
     return 0;
 }
 
-constexpr int kLoopMaxItems = 3;      // stream elements of a layer a wave holds in registers
+constexpr int kLoopMaxItems = 4;      // stream elements of a layer a wave holds in registers (kernels for 3 and for 4)
 
 int prepare_matvec_loop()
 {
     int rc;
-    if ((rc = set_lds_limit(matvec_loop_kernel<6, RPTC_AS_WRITTEN, kLoopMaxItems>))) return rc;
-    if ((rc = set_lds_limit(matvec_loop_kernel<6, RPTC_CONTINUOUS, kLoopMaxItems>))) return rc;
-    if ((rc = set_lds_limit(matvec_loop_kernel<8, RPTC_AS_WRITTEN, kLoopMaxItems>))) return rc;
-    return set_lds_limit(matvec_loop_kernel<8, RPTC_CONTINUOUS, kLoopMaxItems>);
+#define RPTC_SET_LIMITS(MAXI)                                                                  \
+    if ((rc = set_lds_limit(matvec_loop_kernel<6, RPTC_AS_WRITTEN, MAXI>))) return rc;          \
+    if ((rc = set_lds_limit(matvec_loop_kernel<6, RPTC_CONTINUOUS, MAXI>))) return rc;          \
+    if ((rc = set_lds_limit(matvec_loop_kernel<8, RPTC_AS_WRITTEN, MAXI>))) return rc;          \
+    if ((rc = set_lds_limit(matvec_loop_kernel<8, RPTC_CONTINUOUS, MAXI>))) return rc;
+    RPTC_SET_LIMITS(3)
+    RPTC_SET_LIMITS(4)
+#undef RPTC_SET_LIMITS
+    return 0;
 }
 
 int matvec_loop_plan(const rptc_chain_layer *layers, int64_t count, int cus, LoopLayer *out, int *xslot_words,
-                     int *part_floats, int *lds_bytes)
+                     int *part_floats, int *lds_bytes, int *max_items)
 {
-    int64_t n_max = 0, part_max = 0;
+    int64_t n_max = 0, part_max = 0, items_max = 1;
     for (int64_t k = 0; k < count; k++) {
         const rptc_chain_layer &u = layers[k];
         if (u.n > (int64_t)8 * kXRegs * kMatvecThreads) return RPTC_ELIMIT;      // a thread's two registers hold its share
@@ -1323,7 +1328,9 @@ int matvec_loop_plan(const rptc_chain_layer *layers, int64_t count, int cus, Loo
         d.same_shape_as_previous = k > 0 && layers[k - 1].m == u.m && layers[k - 1].n == u.n;
         // a wave keeps all its elements of a layer in registers: at most kLoopMaxItems of them
         const int64_t total = (u.n >> 11) * (int64_t)items_full + d.items_tail;
-        if ((total + kMatvecWaves - 1) / kMatvecWaves > kLoopMaxItems) return RPTC_ELIMIT;
+        const int64_t per_wave = (total + kMatvecWaves - 1) / kMatvecWaves;
+        if (per_wave > kLoopMaxItems) return RPTC_ELIMIT;
+        if (per_wave > items_max) items_max = per_wave;
         if (u.n > n_max) n_max = u.n;
         const int64_t part = (int64_t)d.rows_per_block * (u.n / 64);
         if (part > part_max) part_max = part;
@@ -1333,15 +1340,23 @@ int matvec_loop_plan(const rptc_chain_layer *layers, int64_t count, int cus, Loo
     *xslot_words = (int)(n_max / 2);
     *part_floats = (int)part_max;
     *lds_bytes = (int)bytes;
+    *max_items = items_max <= 3 ? 3 : 4;
     return 0;
 }
 
 int matvec_loop_launch(const LoopLayer *device_layers, const uint32_t *codebook, int count, int xslot_words,
-                       int part_floats, int lds_bytes, int grid, int S, int carry_mode, hipStream_t stream)
+                       int part_floats, int lds_bytes, int max_items, int grid, int S, int carry_mode, hipStream_t stream)
 {
+    if (max_items != 3 && max_items != 4) return RPTC_ESHAPE;
 #define RPTC_LOOP_GO(SS, MM)                                                                                          \
-    hipLaunchKernelGGL((matvec_loop_kernel<SS, MM, kLoopMaxItems>), dim3(grid), dim3(kMatvecThreads), lds_bytes, stream, device_layers, \
-                       codebook, count, xslot_words, part_floats)
+    do {                                                                                                              \
+        if (max_items == 3)                                                                                           \
+            hipLaunchKernelGGL((matvec_loop_kernel<SS, MM, 3>), dim3(grid), dim3(kMatvecThreads), lds_bytes, stream,   \
+                               device_layers, codebook, count, xslot_words, part_floats);                            \
+        else                                                                                                          \
+            hipLaunchKernelGGL((matvec_loop_kernel<SS, MM, 4>), dim3(grid), dim3(kMatvecThreads), lds_bytes, stream,   \
+                               device_layers, codebook, count, xslot_words, part_floats);                            \
+    } while (0)
     if (S == 6 && carry_mode == RPTC_AS_WRITTEN) RPTC_LOOP_GO(6, RPTC_AS_WRITTEN);
     else if (S == 6) RPTC_LOOP_GO(6, RPTC_CONTINUOUS);
     else if (carry_mode == RPTC_AS_WRITTEN) RPTC_LOOP_GO(8, RPTC_AS_WRITTEN);

@@ -522,7 +522,7 @@ struct ChainPlanHost {            // what rptc_chain_t holds (see the header): w
     int32_t device;
     // a chain without dependencies runs in the per-launch kernel's loop form (matvec.hip) when that fits:
     int32_t loop_at_256;          // its descriptors start 256 * this many bytes into the descriptor area (0: not used)
-    int32_t loop_lds_bytes, loop_part_floats;
+    int32_t loop_lds_bytes, loop_part_floats, loop_max_items;
 };
 static_assert(sizeof(ChainPlanHost) <= sizeof(rptc_chain_t), "the public struct holds the plan");
 
@@ -724,10 +724,10 @@ extern "C" int rptc_chain_plan(const rptc_chain_layer *layers, int64_t count, vo
         for (int64_t k = 0; k < count; k++) descs[k].flags |= kChFence;
     // No layer reads or writes what another writes (every pair was looked at: without a guarded layer "earlier"
     // reaches back to the start): the loop form of the per-launch kernel runs the chain when it fits.
-    int loop_xslot_words = 0, loop_part_floats = 0, loop_lds_bytes = 0;
+    int loop_xslot_words = 0, loop_part_floats = 0, loop_lds_bytes = 0, loop_max_items = 0;
     const bool loop = !any && (loop_at >> 8) < (int64_t)1 << 31 &&
                       matvec_loop_plan(layers, count, grid, reinterpret_cast<LoopLayer *>(image.data() + loop_at / 4),
-                                       &loop_xslot_words, &loop_part_floats, &loop_lds_bytes) == 0;
+                                       &loop_xslot_words, &loop_part_floats, &loop_lds_bytes, &loop_max_items) == 0;
     // the sync words behind the descriptors start at zero
     hipStream_t s = static_cast<hipStream_t>(stream);
     if ((rc = (int)hipMemcpyAsync(device_desc, image.data(), (size_t)total_bytes, hipMemcpyHostToDevice, s))) return rc;
@@ -750,6 +750,7 @@ extern "C" int rptc_chain_plan(const rptc_chain_layer *layers, int64_t count, vo
         p.loop_at_256 = (int32_t)(loop_at >> 8);
         p.loop_lds_bytes = loop_lds_bytes;
         p.loop_part_floats = loop_part_floats;       // (the activation image is xslot_words long in both forms)
+        p.loop_max_items = loop_max_items;
     }
     memset(plan, 0, sizeof(*plan));
     memcpy(plan, &p, sizeof(p));
@@ -779,7 +780,7 @@ extern "C" int rptc_decompress_matvec_chain(const rptc_chain_t *plan, const uint
     if (p.loop_at_256 > 0) {
         if (p.loop_lds_bytes > kMaxLds) return RPTC_EDEVICE;
         auto a_loop = reinterpret_cast<const LoopLayer *>(static_cast<const char *>(p.device_desc) + ((int64_t)p.loop_at_256 << 8));
-        rc = matvec_loop_launch(a_loop, a_cb, p.count, p.xslot_words, p.loop_part_floats, p.loop_lds_bytes, p.grid, S, carry_mode, s);
+        rc = matvec_loop_launch(a_loop, a_cb, p.count, p.xslot_words, p.loop_part_floats, p.loop_lds_bytes, p.loop_max_items, p.grid, S, carry_mode, s);
         if (rc) return rc;
         return t.end();
     }
