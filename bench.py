@@ -31,7 +31,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch (per layer for the chain) measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on
 # `bench.py --pmc-probe` (scaled by a copy kernel of known size; the runs are summarised under profiles/).
 # Keyed by (launch kind, m, n, S); other workloads report null.
-MEASURED_TRAFFIC_BYTES = {("launch", 4096, 11008, 8): 11528200, ("chain", 4096, 11008, 8): 11288800}
+MEASURED_TRAFFIC_BYTES = {("launch", 4096, 11008, 8): 11528200, ("chain", 4096, 11008, 8): 11248300}
 
 
 def parse():
@@ -755,7 +755,7 @@ def main():
         },
     }
     if per_launch is not None:
-        line["roofline"]["kernel"] = "matvec_chain_kernel: achieved = steps x compressed bytes / the one launch's duration; launch_us is per layer"
+        line["roofline"]["kernel"] = "matvec_loop_kernel (the form rptc_decompress_matvec_chain takes for independent layers): achieved = steps x compressed bytes / the one launch's duration; launch_us is per layer"
         per_launch["traffic"] = MEASURED_TRAFFIC_BYTES.get(("launch", a.m, a.n, a.S))
         line["per_launch"] = per_launch
     # the floor of this workload on this machine, in the same launch pattern (graph replay over the
