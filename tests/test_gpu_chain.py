@@ -173,6 +173,46 @@ def test_long_chain_reuses_slots_and_counters(rk):
         assert torch.equal(outs[i].view(torch.int16), outs[i % 24].view(torch.int16))
 
 
+@pytest.mark.parametrize("count", [1, 2, 3])
+def test_short_chains(rk, count):
+    """One, two and three independent layers: the loop that serves such chains requests a layer ahead and sums the rows a
+    layer behind, so its first and last iterations are special cases."""
+    S = 8
+    cb = rand_half(2 << S, seed=21).cuda()
+    shapes = [(300, 4096 + 64), (64, 2048), (1024, 704)][:count]
+    layers = []
+    for i, (m, n) in enumerate(shapes):
+        layers.append((rand_codes(m * n // 16, seed=900 + i).cuda(), rand_half(n, seed=910 + i).cuda(),
+                       torch.full((m,), float("nan"), dtype=torch.float16, device="cuda")))
+    chain = rk.MatvecChain(layers, cb)
+    for mode in (0, 1):
+        chain.run(carry_mode=mode)
+        assert chain.status() == 0
+        for comp, x, out in layers:
+            assert not torch.isnan(out).any()
+            check_layer(rk, comp, cb, x, out, S, mode)
+
+
+def test_chain_with_four_elements_a_wave(rk):
+    """8192 x 8192 layers: a workgroup has 64 stream elements of a layer, four a wave (the variant of the loop that holds
+    four), and 12288 x 4096 beside it (three)."""
+    S = 8
+    cb = rand_half(2 << S, seed=22).cuda()
+    layers = []
+    for i, (m, n) in enumerate([(8192, 8192), (12288, 4096), (8192, 8192)]):
+        layers.append((rand_codes(m * n // 16, seed=920 + i).cuda(), rand_half(n, seed=930 + i).cuda(),
+                       torch.full((m,), float("nan"), dtype=torch.float16, device="cuda")))
+    chain = rk.MatvecChain(layers, cb)
+    chain.run(carry_mode=1)
+    assert chain.status() == 0
+    first = [out.clone() for _, _, out in layers]
+    for comp, x, out in layers:
+        check_layer(rk, comp, cb, x, out, S, 1)
+    chain.run(carry_mode=1)
+    for (_, _, out), ref in zip(layers, first):
+        assert torch.equal(out.view(torch.int16), ref.view(torch.int16))
+
+
 def test_chain_gives_up_when_the_grid_cannot_arrive(rk):
     """A plan that expects one more workgroup than the grid has can never pass its grid-wide counter: with a small
     spin limit every wave gives up, the kernel ends by itself and the status says so.  (Forced from the host: the
