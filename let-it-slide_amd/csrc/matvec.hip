@@ -746,6 +746,11 @@ __global__ __launch_bounds__(kMatvecThreads) void matvec_loop_kernel(
     typedef const __attribute__((address_space(1))) uint32_t *global_words;
     typedef const __attribute__((address_space(1))) u32x4 *global_vec4;
     typedef __attribute__((address_space(1))) uint16_t *global_halves;
+    typedef const __attribute__((address_space(1))) char *global_bytes;
+    // a wave-uniform address plus a 32-bit byte offset of the lane's: the form a global load takes a scalar base for
+    auto at = [](const __attribute__((address_space(1))) void *base, uint32_t bytes) {
+        return reinterpret_cast<global_bytes>(base) + bytes;
+    };
     struct Work {                 // a layer as this wave sees it (all wave-uniform)
         global_words comp;
         global_vec4 x;
@@ -758,7 +763,7 @@ __global__ __launch_bounds__(kMatvecThreads) void matvec_loop_kernel(
     // (chains of equal layers are the common case, and the set-up is ~200 scalar instructions of every wave)
     auto setup = [&](int k, const Work &like, bool have_like) {
         Work w;
-        const LoopLayer &d = layers[k];
+        const LoopLayer d = layers[k];          // the whole descriptor in one request: one wait, not one per branch
         if (have_like && d.same_shape_as_previous) {
             w = like;
             w.comp = reinterpret_cast<global_words>(reinterpret_cast<uintptr_t>(d.comp));
@@ -799,7 +804,7 @@ __global__ __launch_bounds__(kMatvecThreads) void matvec_loop_kernel(
     auto load_x = [&](const Work &w, uint4 (&xv)[kXRegs]) {
 #pragma unroll
         for (int u = 0; u < kXRegs; u++) {
-            const u32x4 v = w.x[min(tid + u * kMatvecThreads, w.n8 - 1)];
+            const u32x4 v = *reinterpret_cast<global_vec4>(at(w.x, 16u * (uint32_t)min(tid + u * kMatvecThreads, w.n8 - 1)));
             xv[u] = make_uint4(v.x, v.y, v.z, v.w);
         }
     };
@@ -816,7 +821,7 @@ __global__ __launch_bounds__(kMatvecThreads) void matvec_loop_kernel(
             const bool real = w.it_begin + u < w.it_end && rows_here > 0;
             const uint32_t elem = real ? ld.elem0 + (uint32_t)(w.row0 + row_first) * (uint32_t)ld.lanes : 0u;
             const uint32_t last = real ? (uint32_t)(rows_here * ld.lanes - 1) : 0u;
-            const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<global_vec4>(w.comp + ((size_t)elem + min((uint32_t)lane, last)) * WORDS));
+            const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<global_vec4>(at(w.comp + (size_t)elem * WORDS, 4u * WORDS * min((uint32_t)lane, last))));
             buf[u].w[0] = v.x, buf[u].w[1] = v.y, buf[u].w[2] = v.z, buf[u].w[3] = v.w;
             if (MODE == RPTC_CONTINUOUS) {
                 // the word in front of a row: last word of the row's lane 31 in the slab before (read by all lanes of
@@ -825,7 +830,7 @@ __global__ __launch_bounds__(kMatvecThreads) void matvec_loop_kernel(
                 const int sub = min(slab < w.T ? lane >> 5 : lane / max(ld.lanes, 1), max(rows_here, 1) - 1);
                 const global_words row_base =
                     prev ? w.comp + (((size_t)(slab - 1) * w.m + w.row0 + row_first) * 32 + 31) * WORDS + WORDS - 1 : w.comp;
-                cw[u] = row_base[sub * (prev ? 32 * WORDS : 0)];
+                cw[u] = *reinterpret_cast<global_words>(at(row_base, (uint32_t)sub * (prev ? 4u * 32 * WORDS : 0u)));
             }
             if (real && ++idx == ld.items) {
                 idx = 0;
@@ -868,9 +873,13 @@ __global__ __launch_bounds__(kMatvecThreads) void matvec_loop_kernel(
             }
         }
     };
-    // one wave per row adds the row's partial sums in a fixed order
+    // One wave per row adds the row's partial sums in a fixed order.  The rows are the older half's: a SIMD serves its
+    // oldest wave first, so the waves started first are through with a layer's decode while the younger ones have most
+    // of theirs in front of them, and would only wait at the barrier.
+    constexpr int kRowWaves = kMatvecWaves / 2;
     auto write_rows = [&](const Work &w, const float *part) {
-        for (int r = wave; r < w.rows; r += kMatvecWaves) {
+        if (wave >= kRowWaves) return;
+        for (int r = wave; r < w.rows; r += kRowWaves) {
             float y = 0.f;
             for (int i = lane; i < w.npr; i += kWave) y += part[r * w.npr + i];
             y = wave_sum(y);
@@ -957,13 +966,12 @@ __global__ __launch_bounds__(kMatvecThreads) void matvec_loop_kernel(
             }
             const int row_first = idx * sv.rows_per_item;
             const int nact = max(min(sv.rows_per_item, w.rows - row_first), 0) * sv.lanes;
-            const uint64_t keep = nact >= 64 ? ~0ull : (1ull << nact) - 1ull;
             const uint32_t last = buf[u].w[WORDS - 1];
             const uint32_t own = MODE == RPTC_CONTINUOUS ? (slab > 0 ? cw[u] : 0u) : last;
             float a0, a1, a2, a3;
             decode_element_asm(make_uint4(buf[u].w[0], buf[u].w[1], buf[u].w[2], buf[u].w[3]), own, first_lanes, lane4, xr, a0, a1, a2, a3);
             const float sum = (a0 + a1) + (a2 + a3);
-            if ((keep >> lane) & 1ull) {
+            if (lane < nact) {
                 typedef __attribute__((address_space(3))) float lds_float;
                 *reinterpret_cast<lds_float *>(static_cast<uintptr_t>(part_lane + 4u * (uint32_t)(row_first * pstride))) = sum;
             }
