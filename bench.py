@@ -31,7 +31,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch (per layer for the chain) measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on
 # `bench.py --pmc-probe` (scaled by a copy kernel of known size; the runs are summarised under profiles/).
 # Keyed by (launch kind, m, n, S); other workloads report null.
-MEASURED_TRAFFIC_BYTES = {("launch", 4096, 11008, 8): 11528200, ("chain", 4096, 11008, 8): 11248300}
+MEASURED_TRAFFIC_BYTES = {("launch", 4096, 11008, 8): 11529600, ("chain", 4096, 11008, 8): 11248000}
 
 
 def parse():
