@@ -1,0 +1,174 @@
+"""The chain's loop kernel and the general trellis' dequantize kernels, as compiled, run on the CPU in a functional wave
+model (`tests/wave_model.py`) against the oracle: every global access bounds-checked, loads completing late, registers and LDS full of garbage at the start, the
+sixteen waves of a workgroup interleaved at random.  What the GPU tests cannot show: an access outside the buffers, or
+a register used before its wait, is a test failure that names the instruction here and a dead process there.
+
+Needs hipcc (cross-compiles without a GPU).  The descriptors are packed here as `matvec_loop_plan` packs them
+(`csrc/matvec.hip`, `struct LoopLayer` in `csrc/matvec_loop.hpp`)."""
+import importlib.util
+import os
+import shutil
+import struct
+import subprocess
+
+import numpy as np
+import pytest
+
+import wave_model
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+PKG = os.path.join(ROOT, "let-it-slide_amd")
+CUS = 256                        # the grid the planner makes on the target: one workgroup per compute unit
+
+
+def compile_to_assembly(tmp_path_factory, name):
+    if shutil.which("hipcc") is None:
+        pytest.skip("hipcc not found")
+    spec = importlib.util.spec_from_file_location("rptc_build", os.path.join(PKG, "build.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    out = str(tmp_path_factory.mktemp("isa") / (name + ".s"))
+    subprocess.run(["hipcc", *mod.FLAGS, "--cuda-device-only", "-S", os.path.join(PKG, "csrc", name + ".hip"), "-o", out],
+                   check=True, capture_output=True)
+    return out
+
+
+@pytest.fixture(scope="module")
+def matvec_isa(tmp_path_factory):
+    return compile_to_assembly(tmp_path_factory, "matvec")
+
+
+@pytest.fixture(scope="module")
+def lite_isa(tmp_path_factory):
+    return compile_to_assembly(tmp_path_factory, "lite")
+
+
+def plan(shapes, addresses):
+    """LoopLayer records and the launch's LDS geometry for layers of `shapes`, as the host planner computes them."""
+    raw = bytearray()
+    n_max = part_max = items_max = 0
+    for i, ((m, n), (comp_at, x_at, out_at)) in enumerate(zip(shapes, addresses)):
+        rpb = 2 * ((m + 2 * CUS - 1) // (2 * CUS))
+        lt = (n & 2047) >> 6
+        items_full = rpb // 2
+        rw_tail = 64 // lt if lt else 1
+        items_tail = (rpb + rw_tail - 1) // rw_tail if lt else 0
+        magic = ((1 << 32) // items_full + 1) if items_full > 1 else 0
+        same = 1 if i > 0 and shapes[i - 1] == (m, n) else 0
+        raw += struct.pack("<QQQiiiiiIiiii", comp_at, x_at, out_at, m, n, rpb, rw_tail, items_tail, magic, same, 0, 0, 0)
+        n_max, part_max = max(n_max, n), max(part_max, rpb * (n // 64))
+        items_max = max(items_max, -(-((n >> 11) * items_full + items_tail) // 16))
+    assert items_max <= 4
+    lds_bytes = 65536 + 2 * (2 * n_max) + 2 * 4 * part_max
+    assert lds_bytes <= 160 * 1024
+    return np.frombuffer(bytes(raw), dtype=np.uint8).copy(), n_max // 2, part_max, lds_bytes, 3 if items_max <= 3 else 4
+
+
+def run_chain(isa, oracle, shapes, S, mode, blocks, seed=7, burst=8, latency=(400, 60), shorten=None):
+    rng = np.random.default_rng(seed)
+    mem = wave_model.Memory()
+    cb = (rng.standard_normal(2 << S) * 0.1).astype(np.float16)
+    cb_at = 0x7f5000003400
+    mem.add(cb_at, cb.view(np.uint8).copy(), "codebook")
+    layers, addresses = [], []
+    for i, (m, n) in enumerate(shapes):
+        # one stream straddles a 4 GiB boundary (the carry into the high half of an address), the others sit at odd distances from one
+        comp_at = 0x7f4100000000 + (i << 33) - (4096 if i % 3 == 1 else -0x23456700)
+        x_at, out_at = 0x7f3ffff0fe00 + (i << 16), 0x7f2ffffe0100 + (i << 15)
+        comp = rng.integers(0, 256, m * n // 4, dtype=np.uint8)
+        x = (rng.standard_normal(n) * 0.5).astype(np.float16).view(np.uint8).copy()
+        out = np.full(2 * m, 0xEE, dtype=np.uint8)
+        mem.add(comp_at, comp[:len(comp) - shorten] if shorten and i == len(shapes) - 1 else comp, f"stream {i}")
+        mem.add(x_at, x, f"activations {i}")
+        mem.add(out_at, out, f"output {i}")
+        layers.append((comp, x, out, m, n))
+        addresses.append((comp_at, x_at, out_at))
+    desc, xslot_words, part_floats, lds_bytes, maxi = plan(shapes, addresses)
+    desc_at = 0x7f6000001000
+    mem.add(desc_at, desc, "descriptors")
+    kernel = wave_model.Kernel(isa, "_ZN4rptc18matvec_loop_kernelILi%dELi%dELi%dE" % (S, mode, maxi))
+    wave_model.Wave.vm_latency, wave_model.Wave.lgkm_latency = latency
+    kernel.launch(mem, (CUS,), 1024, [("ptr", desc_at), ("ptr", cb_at), ("i32", len(shapes)), ("i32", xslot_words), ("i32", part_floats)],
+                  lds_bytes=lds_bytes, groups=[(b, 0, 0) for b in blocks], seed=seed, burst=burst)
+    for i, (comp, x, out, m, n) in enumerate(layers):
+        want = oracle.matvec(comp.view(np.uint32), cb, x.view(np.float16), m, S, mode=mode)
+        got = out.view(np.float16).astype(np.float64)
+        rpb = 2 * ((m + 2 * CUS - 1) // (2 * CUS))
+        touched = np.zeros(m, dtype=bool)
+        for b in blocks:
+            r0, r1 = b * rpb, min(m, (b + 1) * rpb)
+            if r0 >= r1:
+                continue
+            touched[r0:r1] = True
+            err = np.abs(got[r0:r1] - want[r0:r1]).max() / (np.abs(want).max() + 1e-9)
+            assert err < 2e-3, f"layer {i} ({m}x{n}), workgroup {b}: rows {r0}..{r1 - 1} differ by {err:.3g} of the layer's largest output"
+        # rows of workgroups that did not run still hold the fill pattern
+        assert (out.view(np.uint16)[~touched] == 0xEEEE).all(), f"layer {i}: a row outside the simulated workgroups was written"
+
+
+RAGGED = [(33, 4096 + 768), (300, 64), (7, 704)]
+MIXED = [(64, 2048), (33, 4096 + 768), (512, 6144), (1024, 2048 + 64), (2000, 1984), (2000, 1984)]
+
+
+@pytest.mark.parametrize("S,mode", [(8, 0), (8, 1), (6, 0), (6, 1)])
+def test_loop_kernel_matches_the_oracle(matvec_isa, oracle, S, mode):
+    run_chain(matvec_isa, oracle, RAGGED, S, mode, blocks=[0, 1, 255])
+
+
+def test_loop_kernel_on_mixed_shapes(matvec_isa, oracle):
+    run_chain(matvec_isa, oracle, MIXED, 8, 1, blocks=[0, 16, 255])
+
+
+def test_loop_kernel_with_one_layer(matvec_isa, oracle):
+    run_chain(matvec_isa, oracle, [(64, 2048)], 8, 0, blocks=[0, 31, 32])
+
+
+@pytest.mark.parametrize("burst,latency", [(10 ** 6, (400, 60)), (8, (3000, 300)), (8, (40, 10))])
+def test_loop_kernel_under_other_interleavings_and_latencies(matvec_isa, oracle, burst, latency):
+    """Every wave running until it blocks; memory that answers very late; memory that answers at once."""
+    run_chain(matvec_isa, oracle, RAGGED, 8, 1, blocks=[0, 255], seed=11, burst=burst, latency=latency)
+
+
+def test_the_model_reports_an_access_outside_the_buffers(matvec_isa, oracle):
+    """The last workgroup with rows reads the stream's last element: with the buffer 16 bytes short the model must say so."""
+    with pytest.raises(wave_model.Fault, match="outside every region"):
+        run_chain(matvec_isa, oracle, [(64, 2048)], 8, 0, blocks=[31], shorten=16)
+
+
+@pytest.mark.parametrize("L,S,R,V,rows,length", [(16, 9, 4, 2, 3, 1000), (16, 9, 4, 2, 3, 2048), (16, 9, 4, 2, 2, 1023),
+                                                  (20, 13, 3, 2, 2, 515), (16, 8, 2, 3, 2, 300), (12, 6, 5, 1, 3, 77)])
+def test_lite_dequantize_kernels_match_the_oracle(lite_isa, oracle, L, S, R, V, rows, length):
+    """Both kernels of `csrc/lite.hip` (pairs with the alphabet in LDS and without, and the general one), launched as
+    `rptc_lite_dequantize` launches them, with fewer workgroups than sequences so that the row loop strides, outputs
+    at 8- and 16-byte alignments, and one symbol outside its range."""
+    pairs = V == 2
+    name = "_ZN4rptc28lite_dequantize_pairs_kernelILb%dE" % (1 if S <= 12 else 0) if pairs else "_ZN4rptc22lite_dequantize_kernelE"
+    kernel = wave_model.Kernel(lite_isa, name)
+    rng = np.random.default_rng(L * 1000 + length)
+    alphabet = rng.standard_normal((1 << S, V)).astype(np.float32)
+    symbols = rng.integers(0, 1 << R, (rows, length), dtype=np.int32)
+    symbols[0, 17] = -5
+    out = np.full((rows, length, V), np.nan, dtype=np.float32)
+    out_bytes = out.view(np.uint8).reshape(-1)
+    a_at, s_at, o_at = 0x7f0000100000, 0x7f0000300004, 0x7f0000500000 + (8 if length % 3 == 0 else 0)
+    history = (32 + R - 1) // R - 1
+    grid_y = min(rows, 2)
+    for latency in ((400, 60), (30, 8)):
+        mem = wave_model.Memory()
+        mem.add(a_at, alphabet.view(np.uint8).reshape(-1), "alphabet")
+        mem.add(s_at, symbols.view(np.uint8).reshape(-1), "symbols")
+        mem.add(o_at, out_bytes, "output")
+        out_bytes[:] = 0xFF
+        wave_model.Wave.vm_latency, wave_model.Wave.lgkm_latency = latency
+        if pairs:
+            lds = (32 + 512) * 4 + ((8 << S) if S <= 12 else 0)
+            kernel.launch(mem, ((length + 511) // 512, grid_y), 256,
+                          [("ptr", a_at), ("ptr", s_at), ("ptr", o_at), ("i64", length), ("i32", rows), ("i32", R), ("i32", history),
+                           ("i32", L - S), ("u32", (1 << S) - 1)], lds_bytes=lds)
+        else:
+            chunks = (length + 7) // 8
+            kernel.launch(mem, ((chunks + 255) // 256, grid_y), 256,
+                          [("ptr", a_at), ("ptr", s_at), ("ptr", o_at), ("i64", length), ("i32", rows), ("u32", chunks), ("i32", R),
+                           ("i32", history), ("i32", L - S), ("u32", (1 << S) - 1), ("i32", V)])
+        want = np.stack([oracle.lite_dequantize(alphabet, L, S, R, symbols[r]) for r in range(rows)])
+        assert np.array_equal(out.view(np.uint32), want.reshape(out.shape).view(np.uint32))
