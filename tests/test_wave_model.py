@@ -1,4 +1,5 @@
-"""The chain's loop kernel and the general trellis' dequantize kernels, as compiled, run on the CPU in a functional wave
+"""The decode-only kernel, the per-launch mat-vec kernel, the chain's loop kernel and the general trellis' dequantize
+kernels, as compiled, run on the CPU in a functional wave
 model (`tests/wave_model.py`) against the oracle: every global access bounds-checked, loads completing late, registers and LDS full of garbage at the start, the
 sixteen waves of a workgroup interleaved at random.  What the GPU tests cannot show: an access outside the buffers, or
 a register used before its wait, is a test failure that names the instruction here and a dead process there.
@@ -41,6 +42,11 @@ def matvec_isa(tmp_path_factory):
 @pytest.fixture(scope="module")
 def lite_isa(tmp_path_factory):
     return compile_to_assembly(tmp_path_factory, "lite")
+
+
+@pytest.fixture(scope="module")
+def decompress_isa(tmp_path_factory):
+    return compile_to_assembly(tmp_path_factory, "decompress")
 
 
 def plan(shapes, addresses):
@@ -135,6 +141,48 @@ def test_the_model_reports_an_access_outside_the_buffers(matvec_isa, oracle):
         run_chain(matvec_isa, oracle, [(64, 2048)], 8, 0, blocks=[31], shorten=16)
 
 
+@pytest.mark.parametrize("m,n,S,mode", [(64, 2048, 8, 0), (33, 4096 + 768, 8, 1), (300, 64, 6, 0), (1024, 2048 + 64, 6, 1),
+                                        (2000, 1984, 8, 1), (7, 704, 8, 0), (5, 16384, 8, 1), (512, 6144, 6, 0)])
+def test_per_launch_kernel_matches_the_oracle(matvec_isa, oracle, m, n, S, mode):
+    """`matvec_kernel<S, MODE, 2, false>` (what `rptc_decompress_matvec_16_8_1` and its siblings launch), with the
+    geometry of `plan_matvec` in `csrc/matvec.hip`; the first and the last workgroup and one in between."""
+    rng = np.random.default_rng(m + n)
+    cb = (rng.standard_normal(2 << S) * 0.1).astype(np.float16)
+    comp = rng.integers(0, 256, m * n // 4, dtype=np.uint8)
+    x = (rng.standard_normal(n) * 0.5).astype(np.float16)
+    out = np.full(2 * m, 0xEE, dtype=np.uint8)
+    mem = wave_model.Memory()
+    c_at, cb_at, x_at, o_at = 0x7f40fffff000, 0x7f5000003400, 0x7f3ffff0fe00, 0x7f2ffffe0100     # the stream straddles 4 GiB
+    mem.add(c_at, comp, "stream")
+    mem.add(cb_at, cb.view(np.uint8).copy(), "codebook")
+    mem.add(x_at, x.view(np.uint8).copy(), "activations")
+    mem.add(o_at, out, "output")
+    rpb = 2 * ((m + 2 * CUS - 1) // (2 * CUS))
+    lt = (n & 2047) >> 6
+    rw_tail = 64 // lt if lt else 1
+    items_full = rpb // 2
+    items_tail = (rpb + rw_tail - 1) // rw_tail if lt else 0
+    magic = ((1 << 32) // items_full + 1) if items_full > 1 else 0
+    lds_bytes = 65536 + 2 * n + 4 * (n // 64) * rpb
+    assert lds_bytes <= 160 * 1024
+    grid = (m + rpb - 1) // rpb
+    blocks = sorted({0, grid // 2, grid - 1})
+    kernel = wave_model.Kernel(matvec_isa, "_ZN4rptc13matvec_kernelILi%dELi%dELi2ELb0EE" % (S, mode))
+    wave_model.Wave.vm_latency, wave_model.Wave.lgkm_latency = 400, 60
+    kernel.launch(mem, (grid,), 1024, [("ptr", c_at), ("ptr", cb_at), ("ptr", x_at), ("i32", m), ("i32", n), ("i32", rpb), ("i32", rw_tail),
+                                       ("i32", items_tail), ("u32", magic), ("ptr", o_at)], lds_bytes=lds_bytes,
+                  groups=[(b, 0, 0) for b in blocks], seed=m)
+    want = oracle.matvec(comp.view(np.uint32), cb, x, m, S, mode=mode)
+    got = out.view(np.float16).astype(np.float64)
+    touched = np.zeros(m, dtype=bool)
+    for b in blocks:
+        r0, r1 = b * rpb, min(m, (b + 1) * rpb)
+        touched[r0:r1] = True
+        err = np.abs(got[r0:r1] - want[r0:r1]).max() / (np.abs(want).max() + 1e-9)
+        assert err < 2e-3, f"workgroup {b}: rows {r0}..{r1 - 1} differ by {err:.3g} of the largest output"
+    assert (out.view(np.uint16)[~touched] == 0xEEEE).all()
+
+
 @pytest.mark.parametrize("L,S,R,V,rows,length", [(16, 9, 4, 2, 3, 1000), (16, 9, 4, 2, 3, 2048), (16, 9, 4, 2, 2, 1023),
                                                   (20, 13, 3, 2, 2, 515), (16, 8, 2, 3, 2, 300), (12, 6, 5, 1, 3, 77)])
 def test_lite_dequantize_kernels_match_the_oracle(lite_isa, oracle, L, S, R, V, rows, length):
@@ -172,3 +220,25 @@ def test_lite_dequantize_kernels_match_the_oracle(lite_isa, oracle, L, S, R, V, 
                            ("i32", history), ("i32", L - S), ("u32", (1 << S) - 1), ("i32", V)])
         want = np.stack([oracle.lite_dequantize(alphabet, L, S, R, symbols[r]) for r in range(rows)])
         assert np.array_equal(out.view(np.uint32), want.reshape(out.shape).view(np.uint32))
+
+
+@pytest.mark.parametrize("m,words_per_row,mode,grid", [(3, 128, 0, 1), (5, 256, 1, 2), (2, 384, 1, 3)])
+def test_decompress_kernel_matches_the_oracle(decompress_isa, oracle, m, words_per_row, mode, grid):
+    """`decompress_kernel<MODE>` as `rptc_decompress` launches it, with fewer workgroups than the rows need (the
+    kernel strides), bit for bit."""
+    rng = np.random.default_rng(m * words_per_row)
+    codebook = rng.integers(0, 65536, 65536, dtype=np.uint16)
+    stream = rng.integers(0, 1 << 32, (m, words_per_row), dtype=np.uint64).astype(np.uint32)
+    out = np.full((m, 16 * words_per_row), 0xEEEE, dtype=np.uint16)
+    mem = wave_model.Memory()
+    c_at, cb_at, o_at = 0x7f40fffff000, 0x7f5000003400, 0x7f2ffffe0100
+    mem.add(c_at, stream.view(np.uint8).reshape(-1), "stream")
+    mem.add(cb_at, codebook.view(np.uint8), "codebook")
+    mem.add(o_at, out.view(np.uint8).reshape(-1), "output")
+    groups = 2 * m * words_per_row
+    kernel = wave_model.Kernel(decompress_isa, "_ZN4rptc17decompress_kernelILi%dE" % mode)
+    wave_model.Wave.vm_latency, wave_model.Wave.lgkm_latency = 400, 60
+    kernel.launch(mem, (grid,), 1024, [("ptr", c_at), ("ptr", cb_at), ("ptr", o_at), ("u32", words_per_row), ("u32", groups)],
+                  lds_bytes=131072, seed=m)
+    want = oracle.decompress(stream.view(np.int32), codebook, mode=mode).view(np.uint16)
+    assert np.array_equal(out, want)

@@ -566,6 +566,10 @@ class Wave:
             self.ws(o[0], (S(o[1]) * S(o[2])) & 0xFFFFFFFF, 1)
         elif op == "s_mul_hi_u32":
             self.ws(o[0], (S(o[1]) * S(o[2])) >> 32, 1)
+        elif op == "s_mulk_i32":
+            v = int(o[1], 0)
+            if v & 0x8000 and v > 0: v -= 0x10000
+            self.ws(o[0], (S(o[0]) * v) & 0xFFFFFFFF, 1)
         elif op in ("s_and_b32", "s_or_b32", "s_xor_b32"):
             a, b = S(o[1]), S(o[2])
             r = a & b if op == "s_and_b32" else (a | b if op == "s_or_b32" else a ^ b)
@@ -654,6 +658,8 @@ class Wave:
         # ---------------------------------------------------------------- vector ALU
         elif op in ("v_mov_b32_e32", "v_mov_b32_e64"):
             self.wv(o[0], V(o[1]))
+        elif op in ("v_not_b32_e32", "v_not_b32_e64"):
+            self.wv(o[0], (~V(o[1]).astype(np.uint64) & np.uint64(0xFFFFFFFF)).astype(U32))
         elif op == "v_mov_b32_dpp":
             src, valid = self.dpp_src(V(o[1]), mods, None)
             self.wv(o[0], src, self.lanes() & valid)
@@ -845,6 +851,21 @@ class Wave:
             selm = S(o[3], 2)
             sel = np.array([(selm >> k) & 1 for k in range(64)], dtype=bool)
             self.wv(o[0], np.where(sel, V(o[2]), V(o[1])))
+        elif op == "v_cndmask_b32_sdwa":
+            # sub-dword operand selects (zero-extended); the whole destination register is written
+            def pick(val, how):
+                val = val.astype(np.uint64)
+                if how == "DWORD":
+                    return val
+                kind, idx = how.split("_")
+                width = 16 if kind == "WORD" else 8
+                return (val >> np.uint64(width * int(idx))) & np.uint64((1 << width) - 1)
+            if mods.get("dst_sel", "DWORD") != "DWORD" or "sext" in text:
+                raise Fault(f"operand selects of {op} not modelled ({self.who()})")
+            selm = S(o[3], 2)
+            sel = np.array([(selm >> k) & 1 for k in range(64)], dtype=bool)
+            a, b = pick(V(o[1]), mods.get("src0_sel", "DWORD")), pick(V(o[2]), mods.get("src1_sel", "DWORD"))
+            self.wv(o[0], np.where(sel, b, a).astype(U32))
         # ---------------------------------------------------------------- LDS
         elif op == "ds_read_b32":
             addr = V(o[1]).astype(np.int64) + int(mods.get("offset", "0"), 0)
@@ -858,6 +879,22 @@ class Wave:
                         if a + 4 > len(self.lds) * 4 or a % 4:
                             raise Fault(f"LDS read at {a:#x} ({who})")
                         self.v[i][k] = self.lds[a // 4]
+            i, _ = self.vreg_index(dst)
+            self.v[i][m] = 0xDEADBEEF
+            self.lgq.append((self.tick, fn))
+        elif op in ("ds_read_u16", "ds_read_u8"):
+            size = 2 if op == "ds_read_u16" else 1
+            addr = V(o[1]).astype(np.int64) + int(mods.get("offset", "0"), 0)
+            dst, m, who = o[0], self.lanes().copy(), self.who()
+
+            def fn(addr=addr, dst=dst, m=m, who=who, size=size):
+                i, _ = self.vreg_index(dst)
+                for k in range(64):
+                    if m[k]:
+                        a = int(addr[k])
+                        if a + size > len(self.lds) * 4 or a % size:
+                            raise Fault(f"LDS read at {a:#x} ({who})")
+                        self.v[i][k] = (int(self.lds[a // 4]) >> (8 * (a % 4))) & ((1 << (8 * size)) - 1)
             i, _ = self.vreg_index(dst)
             self.v[i][m] = 0xDEADBEEF
             self.lgq.append((self.tick, fn))
