@@ -1,5 +1,5 @@
-"""The decode-only kernel, the per-launch mat-vec kernel, the chain's loop kernel and the general trellis' dequantize
-kernels, as compiled, run on the CPU in a functional wave
+"""The decode-only kernel, the per-launch mat-vec kernel, the chain's loop kernel, the transposed mat-vec kernel and the
+general trellis' dequantize kernels, as compiled, run on the CPU in a functional wave
 model (`tests/wave_model.py`) against the oracle: every global access bounds-checked, loads completing late, registers and LDS full of garbage at the start, the
 sixteen waves of a workgroup interleaved at random.  What the GPU tests cannot show: an access outside the buffers, or
 a register used before its wait, is a test failure that names the instruction here and a dead process there.
@@ -47,6 +47,11 @@ def lite_isa(tmp_path_factory):
 @pytest.fixture(scope="module")
 def decompress_isa(tmp_path_factory):
     return compile_to_assembly(tmp_path_factory, "decompress")
+
+
+@pytest.fixture(scope="module")
+def matvec_t_isa(tmp_path_factory):
+    return compile_to_assembly(tmp_path_factory, "matvec_t")
 
 
 def plan(shapes, addresses):
@@ -242,3 +247,38 @@ def test_decompress_kernel_matches_the_oracle(decompress_isa, oracle, m, words_p
                   lds_bytes=131072, seed=m)
     want = oracle.decompress(stream.view(np.int32), codebook, mode=mode).view(np.uint16)
     assert np.array_equal(out, want)
+
+
+@pytest.mark.parametrize("m,n,L,mode,ksplit", [(100, 256, 16, 0, 1), (70, 512, 14, 1, 1), (64, 1024, 16, 1, 1), (64, 4096, 16, 1, 2),
+                                               (130, 8192, 14, 0, 3), (5, 64, 14, 0, 1)])
+def test_transposed_kernel_matches_the_oracle(matvec_t_isa, oracle, m, n, L, mode, ksplit):
+    """`matvec_t_kernel<L, MODE>` as `launch_matvec_t` (`csrc/matvec_t.hip`) launches it: `out +=`, one workgroup per 64
+    rows and, with `ksplit` > 1, several per row block that hand their partial sums over through memory (the model runs
+    the workgroups one after the other, so the last one finds every arrival and adds the parts up)."""
+    rng = np.random.default_rng(m + n + L)
+    codebook = (rng.standard_normal(1 << L) * 0.1).astype(np.float16)
+    cols = n // 64
+    stream = rng.integers(0, 1 << 32, 4 * cols * m, dtype=np.uint64).astype(np.uint32)
+    x = (rng.standard_normal(n) * 0.5).astype(np.float16)
+    before = (rng.standard_normal(m) * 0.1).astype(np.float16)
+    out = before.copy()
+    parts, arrived = np.zeros(4096 * 64, dtype=np.float32), np.zeros(4096, dtype=np.uint32)
+    mem = wave_model.Memory()
+    c_at, cb_at, x_at, o_at, p_at, a_at = 0x7f40fffff000, 0x7f5000003400, 0x7f3ffff0fe00, 0x7f2ffffe0100, 0x7f6000000000, 0x7f6100000000
+    mem.add(c_at, stream.view(np.uint8), "stream")
+    mem.add(cb_at, codebook.view(np.uint8).copy(), "codebook")
+    mem.add(x_at, x.view(np.uint8).copy(), "activations")
+    mem.add(o_at, out.view(np.uint8), "output")
+    mem.add(p_at, parts.view(np.uint8), "partial sums")
+    mem.add(a_at, arrived.view(np.uint8), "arrival counters")
+    row_blocks = (m + 63) // 64
+    lds_bytes = (2 << L) + 512 * 4 + (((cols + ksplit - 1) // ksplit) * 32 if mode == 0 else 0)
+    kernel = wave_model.Kernel(matvec_t_isa, "_ZN4rptc15matvec_t_kernelILi%dELi%dEE" % (L, mode))
+    wave_model.Wave.vm_latency, wave_model.Wave.lgkm_latency = 400, 60
+    kernel.launch(mem, (row_blocks * ksplit,), 512,
+                  [("ptr", c_at), ("ptr", cb_at), ("ptr", x_at), ("i32", m), ("i32", cols), ("i32", ksplit), ("ptr", o_at), ("ptr", p_at),
+                   ("ptr", a_at)], lds_bytes=lds_bytes, seed=m)
+    want = before.astype(np.float64) + oracle.matvec_t(stream, codebook, x, m, L, mode=mode)
+    err = np.abs(out.astype(np.float64) - want).max() / (np.abs(want).max() + 1e-9)
+    assert err < 3e-3
+    assert not arrived.any(), "an arrival counter was left non-zero"

@@ -566,6 +566,11 @@ class Wave:
             self.ws(o[0], (S(o[1]) * S(o[2])) & 0xFFFFFFFF, 1)
         elif op == "s_mul_hi_u32":
             self.ws(o[0], (S(o[1]) * S(o[2])) >> 32, 1)
+        elif op == "s_abs_i32":
+            a = S(o[1])
+            r = (0x100000000 - a) & 0xFFFFFFFF if a & 0x80000000 else a
+            setscc(r != 0)
+            self.ws(o[0], r, 1)
         elif op == "s_mulk_i32":
             v = int(o[1], 0)
             if v & 0x8000 and v > 0: v -= 0x10000
@@ -715,8 +720,12 @@ class Wave:
             m = self.lanes()
             self.v[d][m] = (r & np.uint64(0xFFFFFFFF)).astype(U32)[m]
             self.v[d + 1][m] = (r >> np.uint64(32)).astype(U32)[m]
-        elif op == "v_mad_u64_u32":
+        elif op in ("v_mad_u64_u32", "v_mad_i64_i32"):
             a, b = V(o[2]).astype(np.uint64), V(o[3]).astype(np.uint64)
+            if op == "v_mad_i64_i32":
+                # sign-extend both factors; the product and the sum wrap at 64 bits
+                a = np.where(a & np.uint64(0x80000000), a | np.uint64(0xFFFFFFFF00000000), a)
+                b = np.where(b & np.uint64(0x80000000), b | np.uint64(0xFFFFFFFF00000000), b)
             j, _ = self.vreg_index(o[4])
             if j is not None:
                 c = self.v[j].astype(np.uint64) | (self.v[j + 1].astype(np.uint64) << np.uint64(32))
@@ -769,9 +778,9 @@ class Wave:
                         out |= val << (8 * byte)
                     r[k] = out
             self.wv(o[0], r)
-        elif op in ("v_dot2c_f32_f16", "v_dot2_f32_f16"):
+        elif op in ("v_dot2c_f32_f16", "v_dot2c_f32_f16_e32", "v_dot2_f32_f16"):
             a, b = V(o[1]), V(o[2])
-            acc = f32(self.v[self.vreg_index(o[0])[0]].copy()) if op == "v_dot2c_f32_f16" else f32(V(o[3]))
+            acc = f32(self.v[self.vreg_index(o[0])[0]].copy()) if op.startswith("v_dot2c_") else f32(V(o[3]))
             al, ah = (a & 0xFFFF).astype(np.uint16).view(np.float16).astype(np.float32), (a >> 16).astype(np.uint16).view(np.float16).astype(np.float32)
             bl, bh = (b & 0xFFFF).astype(np.uint16).view(np.float16).astype(np.float32), (b >> 16).astype(np.uint16).view(np.float16).astype(np.float32)
             with np.errstate(all="ignore"):
@@ -810,6 +819,35 @@ class Wave:
             self.wv(o[0], as_u32(V(o[1]).astype(np.float32)))
         elif op == "v_cvt_f32_ubyte0_e32":
             self.wv(o[0], as_u32((V(o[1]) & 0xFF).astype(np.float32)))
+        elif op == "v_bfe_u32":
+            a, off, width = V(o[1]).astype(np.uint64), V(o[2]) & U32(31), V(o[3]) & U32(31)
+            r = (a >> off.astype(np.uint64)) & ((np.uint64(1) << width.astype(np.uint64)) - np.uint64(1))
+            self.wv(o[0], r.astype(U32))
+        elif op == "v_fma_mix_f32":
+            # a source is fp32, or (its op_sel_hi bit set) the fp16 in the half of the register that op_sel names
+            hi = [int(x) for x in mods.get("op_sel_hi", "[0,0,0]").strip("[]").split(",")]
+            lo = [int(x) for x in mods.get("op_sel", "[0,0,0]").strip("[]").split(",")]
+            if "neg" in text or "abs" in text or "|" in text or "clamp" in text:
+                raise Fault(f"modifiers of {op} not modelled ({self.who()})")
+            src = []
+            for q in range(3):
+                raw = V(o[1 + q])
+                if hi[q]:
+                    half = (raw >> U32(16)) if lo[q] else raw
+                    src.append((half & 0xFFFF).astype(np.uint16).view(np.float16).astype(np.float64))
+                else:
+                    src.append(f32(raw).astype(np.float64))
+            with np.errstate(all="ignore"):
+                self.wv(o[0], as_u32((src[0] * src[1] + src[2]).astype(np.float32)))
+        elif op in ("v_cvt_f32_f16_e32", "v_cvt_f32_f16_sdwa"):
+            src = V(o[1])
+            if op.endswith("_sdwa"):
+                how = mods.get("src0_sel", "DWORD")
+                if mods.get("dst_sel", "DWORD") != "DWORD" or how not in ("DWORD", "WORD_0", "WORD_1") or "sext" in text:
+                    raise Fault(f"operand selects of {op} not modelled ({self.who()})")
+                if how == "WORD_1":
+                    src = src >> U32(16)
+            self.wv(o[0], as_u32((src & 0xFFFF).astype(np.uint16).view(np.float16).astype(np.float32)))
         elif op == "v_cvt_f16_f32_e32":
             with np.errstate(all="ignore"):
                 h = f32(V(o[1])).astype(np.float16).view(np.uint16).astype(U32)
@@ -941,6 +979,22 @@ class Wave:
             for k in range(64):
                 if m[k]:
                     self.mem.read(int(addr[k]), 4 * n, who)
+            self.vmq.append((self.tick, fn))
+        elif op in ("global_load_ushort", "global_load_ubyte"):
+            size = 2 if op == "global_load_ushort" else 1
+            addr = self.global_addr(o[1], o[2] if len(o) > 2 else "off", mods)
+            dst, m, who = o[0], self.lanes().copy(), self.who()
+
+            def fn(addr=addr, dst=dst, m=m, who=who, size=size):
+                i, _ = self.vreg_index(dst)
+                for k in range(64):
+                    if m[k]:
+                        self.v[i][k] = int.from_bytes(self.mem.read(int(addr[k]), size, who), "little")
+            i, _ = self.vreg_index(dst)
+            self.v[i][m] = 0xBAD00000
+            for k in range(64):
+                if m[k]:
+                    self.mem.read(int(addr[k]), size, who)
             self.vmq.append((self.tick, fn))
         elif op == "global_load_lds_dword":
             addr = self.global_addr(o[0], o[1] if len(o) > 1 else "off", mods)
