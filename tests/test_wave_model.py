@@ -1,5 +1,6 @@
-"""The decode-only kernel, the per-launch mat-vec kernel, the chain's loop kernel, the transposed mat-vec kernel and the
-general trellis' dequantize kernels, as compiled, run on the CPU in a functional wave
+"""The decode-only kernel, the per-launch mat-vec kernel, the chain's loop kernel, the transposed mat-vec kernel, the batched
+kernel (matrix instructions, partial tiles handed over between workgroups) and the general trellis' dequantize kernels, as
+compiled, run on the CPU in a functional wave
 model (`tests/wave_model.py`) against the oracle: every global access bounds-checked, loads completing late, registers and LDS full of garbage at the start, the
 sixteen waves of a workgroup interleaved at random.  What the GPU tests cannot show: an access outside the buffers, or
 a register used before its wait, is a test failure that names the instruction here and a dead process there.
@@ -52,6 +53,11 @@ def decompress_isa(tmp_path_factory):
 @pytest.fixture(scope="module")
 def matvec_t_isa(tmp_path_factory):
     return compile_to_assembly(tmp_path_factory, "matvec_t")
+
+
+@pytest.fixture(scope="module")
+def matmul_isa(tmp_path_factory):
+    return compile_to_assembly(tmp_path_factory, "matmul")
 
 
 def plan(shapes, addresses):
@@ -282,3 +288,47 @@ def test_transposed_kernel_matches_the_oracle(matvec_t_isa, oracle, m, n, L, mod
     err = np.abs(out.astype(np.float64) - want).max() / (np.abs(want).max() + 1e-9)
     assert err < 3e-3
     assert not arrived.any(), "an arrival counter was left non-zero"
+
+
+@pytest.mark.parametrize("m,n,batch,S,mode", [(40, 2048 + 128, 5, 8, 0), (16, 2048, 16, 6, 1), (100, 704, 20, 8, 1), (33, 4096, 2, 6, 0)])
+def test_batched_kernel_matches_the_oracle(matmul_isa, oracle, m, n, batch, S, mode):
+    """`pack_x_kernel` and `matmul_kernel<S, MODE, PLANES, 2>` as `run_matmul` (`csrc/matmul.hip`) launches them: the
+    activations packed into the B operand's order, the arrival counters cleared whatever they held, one workgroup per
+    (row group, slab), the last workgroup of a row group to arrive adding the slabs' tiles up (the model runs the workgroups
+    one after the other).  One and two planes of 16 batch columns."""
+    rng = np.random.default_rng(m + n + batch)
+    codebook = (rng.standard_normal(2 << S) * 0.1).astype(np.float16)
+    stream = rng.integers(0, 256, m * n // 4, dtype=np.uint8)
+    x = (rng.standard_normal((batch, n)) * 0.5).astype(np.float16)
+    out = np.full((batch, m), np.nan, dtype=np.float16)
+    planes = 2 if batch > 16 else 1
+    slabs = n // 2048 + (1 if n % 2048 else 0)
+    total = (m + 15) // 16                                  # row blocks of 16 rows
+    groups = max(1, min(2 * CUS // slabs, total))
+    groups = max(groups, -(-total // (8 if planes == 1 else 6)))
+    max_rb = -(-total // groups)
+    xpack = np.zeros(planes * (n // 2) * 16, dtype=np.uint32)
+    partial = np.zeros(groups * slabs * max_rb * planes * 256, dtype=np.float32)
+    arrived = np.full(groups, 0xABCD, dtype=np.uint32)
+    mem = wave_model.Memory()
+    c_at, cb_at, x_at, o_at = 0x7f40fffff000, 0x7f5000003400, 0x7f3ffff0fe00, 0x7f2ffffe0100
+    xp_at, p_at, a_at = 0x7f6000000000, 0x7f6100000000, 0x7f6200000000
+    for at, data, name in ((c_at, stream, "stream"), (cb_at, codebook.view(np.uint8).copy(), "codebook"),
+                           (x_at, x.view(np.uint8).reshape(-1).copy(), "activations"), (o_at, out.view(np.uint8).reshape(-1), "output"),
+                           (xp_at, xpack.view(np.uint8), "packed activations"), (p_at, partial.view(np.uint8), "partial tiles"),
+                           (a_at, arrived.view(np.uint8), "arrival counters")):
+        mem.add(at, data, name)
+    wave_model.Wave.vm_latency, wave_model.Wave.lgkm_latency = 400, 60
+    pack = wave_model.Kernel(matmul_isa, "_ZN4rptc13pack_x_kernelE")
+    threads = max(planes * (n // 8) * 16, groups)
+    pack.launch(mem, ((threads + 255) // 256,), 256,
+                [("ptr", x_at), ("ptr", xp_at), ("ptr", a_at), ("i32", groups), ("i32", n), ("i32", batch), ("i32", planes)], seed=m)
+    mem.regions = [r for r in mem.regions if r[2] != "kernarg"]
+    kernel = wave_model.Kernel(matmul_isa, "_ZN4rptc13matmul_kernelILi%dELi%dELi%dELi2EE" % (S, mode, planes))
+    kernel.launch(mem, (groups * slabs,), 512,
+                  [("ptr", c_at), ("ptr", cb_at), ("ptr", xp_at), ("i32", m), ("i32", n), ("i32", total // groups), ("i32", total % groups),
+                   ("i32", 0), ("i32", max_rb), ("ptr", p_at), ("ptr", a_at), ("ptr", o_at), ("i32", batch)],
+                  lds_bytes=65536 + 8 * 2 * 256 * 4, seed=m)
+    want = np.stack([oracle.matvec(stream.view(np.uint32), codebook, x[b], m, S, mode=mode) for b in range(batch)])
+    err = np.abs(out.astype(np.float64) - want).max() / (np.abs(want).max() + 1e-9)
+    assert err < 2e-3

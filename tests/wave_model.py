@@ -602,6 +602,13 @@ class Wave:
             r = (sx(S(o[1])) >> (S(o[2]) & 31)) & 0xFFFFFFFF
             setscc(r != 0)
             self.ws(o[0], r, 1)
+        elif op == "s_lshr_b64":
+            r = S(o[1], 2) >> (S(o[2]) & 63)
+            setscc(r != 0)
+            self.ws(o[0], r, 2)
+        elif op in ("s_bitset0_b32", "s_bitset1_b32"):
+            bit = 1 << (S(o[1]) & 31)
+            self.ws(o[0], (S(o[0]) | bit) if op == "s_bitset1_b32" else (S(o[0]) & ~bit & 0xFFFFFFFF), 1)
         elif op == "s_lshl_b64":
             r = (S(o[1], 2) << (S(o[2]) & 63)) & MASK64
             setscc(r != 0)
@@ -620,6 +627,10 @@ class Wave:
                 c = a < b if "min" in op else a > b
             setscc(c)
             self.ws(o[0], a if c else b, 1)
+        elif op in ("s_cmp_eq_u64", "s_cmp_lg_u64"):
+            a = S(o[0], 2)
+            b = S(o[1], 2) if not re.match(r"^-?\d", o[1]) else int(o[1], 0) & MASK64
+            setscc((a == b) == (op == "s_cmp_eq_u64"))
         elif op.startswith("s_cmp_") or op.startswith("s_cmpk_"):
             a = S(o[0])
             b = S(o[1]) if op.startswith("s_cmp_") else int(o[1], 0) & 0xFFFFFFFF
@@ -714,7 +725,7 @@ class Wave:
             if j is not None:
                 c = self.v[j].astype(np.uint64) | (self.v[j + 1].astype(np.uint64) << np.uint64(32))
             else:
-                c = np.full(64, S(o[3], 2) if self.sreg_index(o[3])[0] is not None else int(o[3], 0), dtype=np.uint64)
+                c = np.full(64, S(o[3], 2) if self.sreg_index(o[3])[0] is not None else int(o[3], 0) & MASK64, dtype=np.uint64)
             r = (a << sh) + c
             d, _ = self.vreg_index(o[0])
             m = self.lanes()
@@ -749,6 +760,38 @@ class Wave:
                 if m[k]:
                     newvcc = (newvcc & ~(1 << k)) | (int(carry[k]) << k)
             self.vcc = newvcc
+        elif op == "v_or3_b32":
+            self.wv(o[0], V(o[1]) | V(o[2]) | V(o[3]))
+        elif op == "v_mfma_f32_16x16x32_f16":
+            # D[16 x 16] = A[16 x 32] B[32 x 16] + C, fp32.  Lane l = 16 g + i holds A[i][8 g .. 8 g + 7] (four registers of two
+            # halves) and, with j for i, B[8 g .. 8 g + 7][j]; register r of lane l = 16 q + j holds C and D [4 q + r][j].
+            # Every lane takes part whatever EXEC says.  The hardware's internal rounding is not modelled (sums in double).
+            if mods:
+                raise Fault(f"modifiers of {op} not modelled ({self.who()})")
+            def halves(tok):
+                i0, n = self.vreg_index(tok)
+                assert n == 4, tok
+                regs = np.stack([self.v[i0 + q] for q in range(4)], axis=1)                       # [lane][4]
+                h = np.stack([regs & U32(0xFFFF), regs >> U32(16)], axis=2).reshape(64, 8)       # [lane][8], low half first
+                return h.astype(np.uint16).view(np.float16).astype(np.float64)
+            ha, hb = halves(o[1]), halves(o[2])
+            A, B = np.zeros((16, 32)), np.zeros((32, 16))
+            for l in range(64):
+                A[l % 16, 8 * (l // 16):8 * (l // 16) + 8] = ha[l]
+                B[8 * (l // 16):8 * (l // 16) + 8, l % 16] = hb[l]
+            C = np.zeros((16, 16))
+            if self.vreg_index(o[3])[0] is not None:
+                c0, _ = self.vreg_index(o[3])
+                for l in range(64):
+                    for r in range(4):
+                        C[4 * (l // 16) + r, l % 16] = f32(self.v[c0 + r][l:l + 1])[0]
+            elif int(o[3], 0) != 0:
+                raise Fault(f"constant accumulator of {op} not modelled ({self.who()})")
+            with np.errstate(all="ignore"):
+                D = (A @ B + C).astype(np.float32)
+            d0, _ = self.vreg_index(o[0])
+            for r in range(4):
+                self.v[d0 + r] = as_u32(np.array([D[4 * (l // 16) + r, l % 16] for l in range(64)], dtype=np.float32))
         elif op in ("v_and_or_b32", "v_perm_b32", "v_alignbit_b32", "v_pk_mad_u16"):
             a, b, c = V(o[1]), V(o[2]), V(o[3])
             if op == "v_and_or_b32":
