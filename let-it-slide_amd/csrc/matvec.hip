@@ -920,6 +920,12 @@ __global__ __launch_bounds__(kMatvecThreads) void matvec_loop_kernel(
 #pragma unroll
         for (int u = 0; u < MAXI; u++) {
             if (w.it_begin + u >= w.it_end) break;
+            // A wave that is further along gives way to the ones behind it: left alone, the SIMD serves its oldest wave
+            // first and its youngest decodes its last element with nobody to share the vector ALU's idle cycles with.
+            if (u == 0) __builtin_amdgcn_s_setprio(3);
+            else if (u == 1) __builtin_amdgcn_s_setprio(2);
+            else if (u == 2) __builtin_amdgcn_s_setprio(1);
+            else __builtin_amdgcn_s_setprio(0);
             if (slab != cur_slab) {
                 cur_slab = slab;
                 if (slab < w.T) {
@@ -981,6 +987,7 @@ __global__ __launch_bounds__(kMatvecThreads) void matvec_loop_kernel(
                 sv = view(w, slab);
             }
         }
+        __builtin_amdgcn_s_setprio(3);
         if (k > 0) write_rows(prev, part0 + ((k - 1) & 1) * part_floats);
         if (has_next) {
             stage_x(sx0 + ((k + 1) & 1) * xslot_words, nxt.n8);
