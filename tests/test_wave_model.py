@@ -1,6 +1,6 @@
 """The decode-only kernel, the per-launch mat-vec kernel, the chain's loop kernel, the transposed mat-vec kernel, the batched
-kernel (matrix instructions, partial tiles handed over between workgroups) and the general trellis' dequantize kernels, as
-compiled, run on the CPU in a functional wave
+kernel (matrix instructions, partial tiles handed over between workgroups), the sign-Hadamard transform and the general
+trellis' dequantize kernels, as compiled, run on the CPU in a functional wave
 model (`tests/wave_model.py`) against the oracle: every global access bounds-checked, loads completing late, registers and LDS full of garbage at the start, the
 sixteen waves of a workgroup interleaved at random.  What the GPU tests cannot show: an access outside the buffers, or
 a register used before its wait, is a test failure that names the instruction here and a dead process there.
@@ -58,6 +58,11 @@ def matvec_t_isa(tmp_path_factory):
 @pytest.fixture(scope="module")
 def matmul_isa(tmp_path_factory):
     return compile_to_assembly(tmp_path_factory, "matmul")
+
+
+@pytest.fixture(scope="module")
+def hadamard_isa(tmp_path_factory):
+    return compile_to_assembly(tmp_path_factory, "hadamard")
 
 
 def plan(shapes, addresses):
@@ -330,5 +335,30 @@ def test_batched_kernel_matches_the_oracle(matmul_isa, oracle, m, n, batch, S, m
                    ("i32", 0), ("i32", max_rb), ("ptr", p_at), ("ptr", a_at), ("ptr", o_at), ("i32", batch)],
                   lds_bytes=65536 + 8 * 2 * 256 * 4, seed=m)
     want = np.stack([oracle.matvec(stream.view(np.uint32), codebook, x[b], m, S, mode=mode) for b in range(batch)])
+    err = np.abs(out.astype(np.float64) - want).max() / (np.abs(want).max() + 1e-9)
+    assert err < 2e-3
+
+
+@pytest.mark.parametrize("batch,n,block,inverse,misalign", [(2, 512, 256, 0, 0), (1, 1024, 1024, 1, 0), (3, 192, 64, 0, 2), (1, 12, 4, 1, 0),
+                                                            (1, 2048 + 512, 512, 0, 0)])
+def test_sign_hadamard_kernel_matches_the_oracle(hadamard_isa, oracle, batch, n, block, inverse, misalign):
+    """`sign_hadamard_kernel` as `rptc_sign_hadamard` launches it: one workgroup per block, 16-byte accesses where the
+    block and the three addresses allow them, two-byte ones otherwise."""
+    rng = np.random.default_rng(n + block)
+    x = rng.standard_normal((batch, n)).astype(np.float16)
+    signs = np.where(rng.integers(0, 2, n) == 1, 1.0, -1.0).astype(np.float16)
+    out = np.full((batch, n), np.nan, dtype=np.float16)
+    mem = wave_model.Memory()
+    x_at, s_at, o_at = 0x7f3ffff0fe00 + misalign, 0x7f5000003400, 0x7f2ffffe0100
+    mem.add(x_at, x.view(np.uint8).reshape(-1).copy(), "input")
+    mem.add(s_at, signs.view(np.uint8).copy(), "signs")
+    mem.add(o_at, out.view(np.uint8).reshape(-1), "output")
+    wide = 1 if block % 8 == 0 and misalign % 16 == 0 else 0
+    kernel = wave_model.Kernel(hadamard_isa, "_ZN4rptc20sign_hadamard_kernelE")
+    wave_model.Wave.vm_latency, wave_model.Wave.lgkm_latency = 400, 60
+    kernel.launch(mem, (batch * (n // block),), 256,
+                  [("ptr", x_at), ("ptr", s_at), ("ptr", o_at), ("i32", n), ("i32", block), ("i32", block.bit_length() - 1),
+                   ("i32", n // block), ("i32", inverse), ("i32", wide)], lds_bytes=(block + block // 32) * 4, seed=n)
+    want = oracle.sign_hadamard(x, signs, block, inverse=bool(inverse))
     err = np.abs(out.astype(np.float64) - want).max() / (np.abs(want).max() + 1e-9)
     assert err < 2e-3

@@ -566,6 +566,8 @@ class Wave:
             self.ws(o[0], (S(o[1]) * S(o[2])) & 0xFFFFFFFF, 1)
         elif op == "s_mul_hi_u32":
             self.ws(o[0], (S(o[1]) * S(o[2])) >> 32, 1)
+        elif op == "s_mul_hi_i32":
+            self.ws(o[0], ((sx(S(o[1])) * sx(S(o[2]))) >> 32) & 0xFFFFFFFF, 1)
         elif op == "s_abs_i32":
             a = S(o[1])
             r = (0x100000000 - a) & 0xFFFFFFFF if a & 0x80000000 else a
@@ -848,6 +850,20 @@ class Wave:
             with np.errstate(all="ignore"):
                 r = f32(V(o[1])) * f32(V(o[2])) + f32(V(o[3]))
             self.wv(o[0], as_u32(r))
+        elif op == "v_rsq_f32_e32":
+            with np.errstate(all="ignore"):
+                r = (np.float32(1.0) / np.sqrt(f32(V(o[1])).astype(np.float64))).astype(np.float32)
+            self.wv(o[0], as_u32(r))
+        elif op == "v_cvt_f16_f32_sdwa":
+            # dst_unused:UNUSED_PAD: the half that is not written becomes zero
+            if mods.get("src0_sel", "DWORD") != "DWORD" or mods.get("dst_unused", "UNUSED_PAD") != "UNUSED_PAD" or "sext" in text:
+                raise Fault(f"operand selects of {op} not modelled ({self.who()})")
+            with np.errstate(all="ignore"):
+                h = f32(V(o[1])).astype(np.float16).view(np.uint16).astype(U32)
+            where = mods.get("dst_sel", "DWORD")
+            if where not in ("DWORD", "WORD_0", "WORD_1"):
+                raise Fault(f"operand selects of {op} not modelled ({self.who()})")
+            self.wv(o[0], h << U32(16) if where == "WORD_1" else h)
         elif op == "v_rcp_iflag_f32_e32":
             with np.errstate(all="ignore"):
                 r = np.float32(1.0) / f32(V(o[1]))
@@ -860,6 +876,8 @@ class Wave:
             self.wv(o[0], r)
         elif op == "v_cvt_f32_u32_e32":
             self.wv(o[0], as_u32(V(o[1]).astype(np.float32)))
+        elif op == "v_cvt_f32_i32_e32":
+            self.wv(o[0], as_u32(V(o[1]).astype(np.int32).astype(np.float32)))
         elif op == "v_cvt_f32_ubyte0_e32":
             self.wv(o[0], as_u32((V(o[1]) & 0xFF).astype(np.float32)))
         elif op == "v_bfe_u32":
