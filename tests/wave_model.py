@@ -981,6 +981,20 @@ class Wave:
             i, _ = self.vreg_index(dst)
             self.v[i][m] = 0xDEADBEEF
             self.lgq.append((self.tick, fn))
+        elif op == "ds_bpermute_b32":
+            # lane k receives the data register of lane (address / 4) mod 64, or zero when that lane is switched off; the
+            # result arrives like an LDS read's (no LDS memory is touched)
+            src = (V(o[1]) >> U32(2)) & U32(63)
+            data, m, who, dst = V(o[2]).copy(), self.lanes().copy(), self.who(), o[0]
+
+            def fn(src=src, data=data, m=m, dst=dst):
+                i, _ = self.vreg_index(dst)
+                for k in range(64):
+                    if m[k]:
+                        self.v[i][k] = data[src[k]] if m[src[k]] else 0
+            i, _ = self.vreg_index(dst)
+            self.v[i][m] = 0xDEADBEEF
+            self.lgq.append((self.tick, fn))
         elif op in ("ds_read_u16", "ds_read_u8"):
             size = 2 if op == "ds_read_u16" else 1
             addr = V(o[1]).astype(np.int64) + int(mods.get("offset", "0"), 0)
