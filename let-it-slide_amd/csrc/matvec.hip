@@ -655,8 +655,17 @@ __device__ __forceinline__ void matvec_body(
             ccw[u] = cw[u];
         }
         if (base + kBatch < it_end) load_batch(base + kBatch);
+        if (total < 3 * kMatvecWaves) {
+            // equal shares: a wave that is further along gives way to the ones behind it, so that the four waves of a
+            // SIMD advance together instead of oldest first (the skewed shares above are the other answer to the same)
+            const int done = base - it_begin;
+            if (done == 0) __builtin_amdgcn_s_setprio(3);
+            else if (done == 1) __builtin_amdgcn_s_setprio(2);
+            else __builtin_amdgcn_s_setprio(1);
+        }
         decode_batch(cur, ccw, base);
     }
+    __builtin_amdgcn_s_setprio(3);
     __syncthreads();
     if constexpr (AFFINE) {
         // one pair per lane and sums across the lanes; the totals are the same for every lane
