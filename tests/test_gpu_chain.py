@@ -213,6 +213,26 @@ def test_chain_with_four_elements_a_wave(rk):
         assert torch.equal(out.view(torch.int16), ref.view(torch.int16))
 
 
+@pytest.mark.parametrize("seed", range(6))
+def test_chain_of_random_shapes(rk, seed):
+    """Eight independent layers of random shapes (any row count up to 3000, any multiple of 64 columns up to 12800: ragged
+    slabs of every width, row blocks that end early, layers with fewer rows than workgroups), S and carry mode by seed."""
+    rng = np.random.default_rng(1000 + seed)
+    S, mode = (6, 8)[seed & 1], (seed >> 1) & 1
+    cb = rand_half(2 << S, seed=40 + seed).cuda()
+    layers = []
+    for i in range(8):
+        m, n = int(rng.integers(1, 3001)), 64 * int(rng.integers(1, 201))
+        layers.append((rand_codes(m * n // 16, seed=1100 + 10 * seed + i).cuda(), rand_half(n, seed=1200 + 10 * seed + i).cuda(),
+                       torch.full((m,), float("nan"), dtype=torch.float16, device="cuda")))
+    chain = rk.MatvecChain(layers, cb)
+    chain.run(carry_mode=mode)
+    assert chain.status() == 0
+    for comp, x, out in layers:
+        assert not torch.isnan(out).any()
+        check_layer(rk, comp, cb, x, out, S, mode)
+
+
 def test_chain_gives_up_when_the_grid_cannot_arrive(rk):
     """A plan that expects one more workgroup than the grid has can never pass its grid-wide counter: with a small
     spin limit every wave gives up, the kernel ends by itself and the status says so.  (Forced from the host: the
