@@ -827,7 +827,8 @@ __global__ __launch_bounds__(kMatvecThreads) void matvec_loop_kernel(
         for (int u = 0; u < MAXI; u++) {
             const int row_first = idx * ld.rows_per_item;
             const int rows_here = min(ld.rows_per_item, w.rows - row_first);
-            const bool real = w.it_begin + u < w.it_end && rows_here > 0;
+            const bool mine = w.it_begin + u < w.it_end;
+            const bool real = mine && rows_here > 0;          // an item past the block's last row is the wave's, and empty
             const uint32_t elem = real ? ld.elem0 + (uint32_t)(w.row0 + row_first) * (uint32_t)ld.lanes : 0u;
             const uint32_t last = real ? (uint32_t)(rows_here * ld.lanes - 1) : 0u;
             const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<global_vec4>(at(w.comp + (size_t)elem * WORDS, 4u * WORDS * min((uint32_t)lane, last))));
@@ -841,7 +842,8 @@ __global__ __launch_bounds__(kMatvecThreads) void matvec_loop_kernel(
                     prev ? w.comp + (((size_t)(slab - 1) * w.m + w.row0 + row_first) * 32 + 31) * WORDS + WORDS - 1 : w.comp;
                 cw[u] = *reinterpret_cast<global_words>(at(row_base, (uint32_t)sub * (prev ? 4u * 32 * WORDS : 0u)));
             }
-            if (real && ++idx == ld.items) {
+            // the cursor moves past every item of the wave's, empty or not, as the decode's does
+            if (mine && ++idx == ld.items) {
                 idx = 0;
                 slab++;
                 ld = view(w, slab);

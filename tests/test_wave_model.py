@@ -141,6 +141,13 @@ def test_loop_kernel_on_mixed_shapes(matvec_isa, oracle):
     run_chain(matvec_isa, oracle, MIXED, 8, 1, blocks=[0, 16, 255])
 
 
+def test_loop_kernel_where_a_wave_holds_an_empty_item_in_front_of_a_real_one(matvec_isa, oracle):
+    """2546 rows are 254 blocks of ten and one of six: in that last block the items of rows 6 to 9 are empty, and the wave
+    that holds slab 0's last item (empty) and slab 1's first (rows 0 and 1) must move its load cursor past the empty one."""
+    run_chain(matvec_isa, oracle, [(2546, 7744)], 6, 0, blocks=[253, 254, 255])
+    run_chain(matvec_isa, oracle, [(2546, 7744), (2546, 7744)], 8, 1, blocks=[254])
+
+
 def test_loop_kernel_with_one_layer(matvec_isa, oracle):
     run_chain(matvec_isa, oracle, [(64, 2048)], 8, 0, blocks=[0, 31, 32])
 
