@@ -148,6 +148,18 @@ def test_loop_kernel_where_a_wave_holds_an_empty_item_in_front_of_a_real_one(mat
     run_chain(matvec_isa, oracle, [(2546, 7744), (2546, 7744)], 8, 1, blocks=[254])
 
 
+@pytest.mark.parametrize("seed", range(4))
+def test_loop_kernel_on_random_shapes(matvec_isa, oracle, seed):
+    """Four layers of random shapes; the first workgroup and, of every layer, the one that holds the end of its rows (where
+    a row block is partial and items are empty)."""
+    rng = np.random.default_rng(300 + seed)
+    shapes = [(int(rng.integers(1, 3001)), 64 * int(rng.integers(1, 121))) for _ in range(4)]
+    blocks = {0}
+    for m, _ in shapes:
+        blocks.add((m - 1) // (2 * ((m + 2 * CUS - 1) // (2 * CUS))))
+    run_chain(matvec_isa, oracle, shapes, (6, 8)[seed & 1], (seed >> 1) & 1, blocks=sorted(blocks), seed=seed)
+
+
 def test_loop_kernel_with_one_layer(matvec_isa, oracle):
     run_chain(matvec_isa, oracle, [(64, 2048)], 8, 0, blocks=[0, 31, 32])
 
