@@ -146,6 +146,9 @@ def test_loop_kernel_where_a_wave_holds_an_empty_item_in_front_of_a_real_one(mat
     that holds slab 0's last item (empty) and slab 1's first (rows 0 and 1) must move its load cursor past the empty one."""
     run_chain(matvec_isa, oracle, [(2546, 7744)], 6, 0, blocks=[253, 254, 255])
     run_chain(matvec_isa, oracle, [(2546, 7744), (2546, 7744)], 8, 1, blocks=[254])
+    # more of the kind (blocks of ten rows that end after 2, 7 and 8)
+    for (m, n), mode in (((2472, 10304), 0), ((2187, 8128), 1), ((2258, 8128), 0)):
+        run_chain(matvec_isa, oracle, [(m, n)], 8, mode, blocks=[(m - 1) // 10])
 
 
 @pytest.mark.parametrize("seed", range(4))
