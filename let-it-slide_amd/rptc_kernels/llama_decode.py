@@ -116,7 +116,7 @@ class QuantizedLlama(torch.nn.Module):
 
     # ---------------------------------------------------------------- fused one-token path
 
-    def decode_step(self, token, pos, fuse=True, half_logits=False, input_ready=False):
+    def decode_step(self, token, pos, fuse=True, half_logits=False, input_ready=False, after_layer=None):
         """token [1] long, pos [1] long, both on the device (read by the kernels, so a captured graph can be
         replayed with new values).  Returns the logits [1, vocab] (float; fp16 as the lm_head product leaves
         them with ``half_logits``).  ``input_ready``: the token's embedding row is already in the decoder's
@@ -124,6 +124,11 @@ class QuantizedLlama(torch.nn.Module):
 
         The position must be below ``shape.max_len``: it lives on the device, so it is not checked here
         (``greedy_decode`` checks its whole range up front; the kernels skip a position outside the caches).
+
+        ``after_layer``: called as ``after_layer(i)`` when layer i's launches have been queued (fused form only;
+        not inside a graph capture): the work buffers then hold, once the stream has been waited for, what that
+        layer's projections read and wrote (``_x2`` the residual stream it started from, ``_qkv``, ``_att``, ``_o``,
+        ``_x`` the residual stream after attention, ``_gu``, ``_down``).
 
         ``fuse`` (default): five launches per layer - the qkv and gate/up projections do the residual add and
         RMS norm in their prologue, the down projection the SiLU gate, and one kernel rotates q and k, appends
@@ -200,6 +205,8 @@ class QuantizedLlama(torch.nn.Module):
                 gemv_norm(blk.gate_up_proj, xb, self._o.data_ptr(), blk.norm2, xa, self._gu)
                 gemv_silu(blk.down_proj, self._gu, self._down)
                 delta = self._down.data_ptr()
+                if after_layer is not None:
+                    after_layer(i)
             ok(lib.rptc_add_rmsnorm(xa.data_ptr(), delta, self.final_norm.data_ptr(), xb.data_ptr(), self._h.data_ptr(), d,
                                     self.EPS, stream))
             logits = self._h.unsqueeze(0) @ self.lm_head.t()
