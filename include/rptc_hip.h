@@ -40,6 +40,7 @@ extern "C" {
 #define RPTC_ELIMIT (-5)     /* a size exceeds what the kernel's LDS staging can hold */
 #define RPTC_EDEVICE (-6)    /* the current device is not gfx950 */
 #define RPTC_EALIAS (-7)     /* an output buffer aliases an input the op still reads */
+#define RPTC_EDEPEND (-8)    /* a layer of a chain reads or overwrites what a layer of the chain writes */
 
 /* Library version, major*10000 + minor*100 + patch. */
 int rptc_version(void);
@@ -106,26 +107,26 @@ int rptc_decompress_matvec_20_8_1(const int32_t *compressed, const uint16_t *cod
 /*
  * A chain of the mat-vecs above in ONE launch: layer k computes out_k = W_k x_k for its own stream, activations
  * and output (the arithmetic of rptc_decompress_matvec_16_{S}_1, one codebook and one carry mode for the whole
- * chain; 2 bits per weight; n <= 16384).  No counterpart in the reference, whose ops are one launch per layer
- * (inference.cu:318-342).  The grid stays resident: the codebook table is built once, stream elements are
- * requested across layer boundaries, and a wave that has finished its share of a layer starts the next one.
- * Dependencies are found from the pointers: a layer whose activations overlap an earlier layer's output, or whose
- * output overlaps an earlier layer's activations or output, starts when every workgroup has finished the layers in
- * front of it (a grid-wide arrival counter); other layers overlap freely.  The result is the same, bit for bit,
- * as `count` separate launches in order would give, except that a row's slabs are added per slab first.
+ * chain; 2 bits per weight; n <= 16384, at most four stream elements of a layer per wave: m * n up to
+ * 2^26 on 256 compute units).  No counterpart in the reference, whose ops are one launch per layer
+ * (inference.cu:318-342).  The grid stays resident: the codebook table is built once and everything a layer reads
+ * is requested while the layer in front is decoded.  Each out_k is the same as a separate launch would give, up to
+ * the order of the fp32 sums of a row (fixed, so the bits repeat from run to run).
+ * The layers must not depend on each other: nothing orders a layer's reads behind another layer's writes.  A chain
+ * in which an `out` overlaps any layer's `x` or `compressed` (its own included) or another layer's `out` is refused
+ * with RPTC_EDEPEND; run such layers as separate calls on one stream, whose launch boundaries order them (a
+ * hand-over between dependent layers inside one launch measured slower than a launch boundary).  The codebook must
+ * not overlap any `out` either (not checked: it is passed at launch time).
  *
- *   rptc_chain_desc_bytes(...)     device bytes the caller provides for the chain's descriptors and item tables
+ *   rptc_chain_desc_bytes(...)     device bytes the caller provides for the chain's descriptors
  *                                  (< 0: a status; at most 65535 layers, each stream below 4 GiB)
  *   rptc_chain_plan(...)           checks the layers, writes the descriptors into device_desc (256-byte aligned
  *                                  device memory; copied on `stream`, which is waited for: a set-up call, not
- *                                  for stream capture) and fills *plan (host memory, opaque).  The plan and the
- *                                  descriptors stay valid until the caller frees device_desc; pointers and
+ *                                  for stream capture) and fills *plan (host memory, opaque).  RPTC_ELIMIT: a
+ *                                  layer does not fit the one-launch form; RPTC_EDEPEND: see above.  The plan and
+ *                                  the descriptors stay valid until the caller frees device_desc; pointers and
  *                                  sizes of the layers are fixed in them, the contents of the buffers are not.
- *   rptc_decompress_matvec_chain   one launch on `stream` (asynchronous unless ms != NULL); the same plan must
- *                                  not run twice at once (the arrival counters live behind its descriptors)
- *   rptc_chain_status              waits for `stream`, then *status = 0 when the last runs completed; bit 0: a
- *                                  bounded wait inside the kernel ran out (the kernel exits, outputs are
- *                                  incomplete); bit 1: an arrival counter is not zero (plan again to clear)
+ *   rptc_decompress_matvec_chain   one launch on `stream` (asynchronous unless ms != NULL)
  */
 typedef struct rptc_chain_layer {
     const int32_t *compressed;     /* the stream of rptc_decompress_matvec_16_{S}_1 for m x n */
@@ -141,7 +142,6 @@ int rptc_chain_plan(const rptc_chain_layer *layers, int64_t count, void *device_
                     rptc_chain_t *plan, void *stream);
 int rptc_decompress_matvec_chain(const rptc_chain_t *plan, const uint16_t *codebook, int S, int carry_mode,
                                  void *stream, float *ms);
-int rptc_chain_status(const rptc_chain_t *plan, int *status, void *stream);
 
 /*
  * Fused decode + mat-vec on the column-interleaved stream with a scalar 2^L codebook.

@@ -6,8 +6,10 @@ librptc_bench_aids.so two measurement aids bench.py times beside the mat-vec (an
 """
 import glob
 import os
+import re
 import subprocess
 import sys
+import tempfile
 from concurrent.futures import ThreadPoolExecutor
 
 HERE = os.path.dirname(os.path.abspath(__file__))
@@ -36,14 +38,57 @@ def _run(cmd, verbose):
     subprocess.run(cmd, check=True)
 
 
+def asm_blocks_left_waiting(assembly):
+    """The rule the hand-written blocks follow, checked on the assembly the compiler emits: a block of inline assembly
+    that issues LDS reads or global loads waits for them before it ends.  The data of such a request lands in its
+    register some time after the instruction; the compiler does not know that, and between two `asm` statements it is
+    free to copy or reuse that register, so a request and its wait must never sit in different statements.
+    Returns [(line number, instruction)] for every request that its own block does not wait for (empty = good)."""
+    bad = []
+    lgkm, vm, in_asm = [], [], False
+    for no, line in enumerate(assembly.split("\n"), 1):
+        t = line.strip()
+        if "#ASMSTART" in t:
+            in_asm, lgkm, vm = True, [], []
+        elif "#ASMEND" in t:
+            bad += lgkm + vm
+            in_asm = False
+        elif in_asm:
+            if re.match(r"ds_(read|bpermute|permute)", t):
+                lgkm.append((no, t))
+            elif re.match(r"(global|buffer|flat)_load", t):
+                vm.append((no, t))
+            elif t.startswith("s_waitcnt"):
+                k = re.search(r"lgkmcnt\((\d+)\)", t)
+                if k:
+                    lgkm = lgkm[len(lgkm) - int(k.group(1)):] if int(k.group(1)) else []
+                v = re.search(r"vmcnt\((\d+)\)", t)
+                if v:
+                    vm = vm[len(vm) - int(v.group(1)):] if int(v.group(1)) else []
+    return bad
+
+
+def check_assembly(src, verbose=False, extra=()):
+    """Compiles `src` to assembly with the library's flags and applies `asm_blocks_left_waiting`; raises on a hit."""
+    with tempfile.TemporaryDirectory() as tmp:
+        out = os.path.join(tmp, os.path.basename(src) + ".s")
+        _run(["hipcc", *FLAGS, *extra, "--cuda-device-only", "-S", src, "-o", out], verbose)
+        bad = asm_blocks_left_waiting(open(out).read())
+    if bad:
+        raise RuntimeError(f"{os.path.basename(src)}: an inline-assembly block ends with requests in flight: {bad[:3]}")
+
+
 def build(verbose=False, extra=()):
-    """Compiles every source (one hipcc per file, in parallel) and links the two libraries."""
+    """Compiles every source (one hipcc per file, in parallel), checks the emitted assembly of the sources that hold
+    hand-written request/wait sequences, and links the two libraries."""
     os.makedirs(OBJ, exist_ok=True)
     srcs = sources()
     objs = [os.path.join(OBJ, os.path.basename(s)[:-4] + ".o") for s in srcs]
     jobs = min(len(srcs), max(1, min(8, os.cpu_count() or 1)))
     with ThreadPoolExecutor(jobs) as pool:
         list(pool.map(lambda so: _run(["hipcc", *FLAGS, *extra, "-c", so[0], "-o", so[1]], verbose), zip(srcs, objs)))
+        with_asm = [s for s in srcs if re.search(r"\basm\b", open(s).read()) or "decode_asm.hpp" in open(s).read()]
+        list(pool.map(lambda s: check_assembly(s, verbose, extra), with_asm))
     _run(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs], verbose)
     _run(["hipcc", *FLAGS, *extra, "-shared", "-o", AIDS_LIB, os.path.join(HERE, "bench_aids", "probe.hip")], verbose)
     return LIB

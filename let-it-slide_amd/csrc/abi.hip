@@ -8,7 +8,6 @@ namespace rptc {
 
 int prepare_decompress();
 int prepare_matvec();
-int prepare_matvec_chain();
 int prepare_matvec_loop();
 int prepare_matvec_t(int device);
 int prepare_matmul(int device);
@@ -43,7 +42,6 @@ int device_info(DeviceInfo **out)
         if ((rc = (int)hipEventCreate(&d.ev_stop))) return rc;
         if ((rc = prepare_decompress())) return rc;
         if ((rc = prepare_matvec())) return rc;
-        if ((rc = prepare_matvec_chain())) return rc;
         if ((rc = prepare_matvec_loop())) return rc;
         if ((rc = prepare_matvec_t(dev))) return rc;
         if ((rc = prepare_matmul(dev))) return rc;
@@ -118,6 +116,7 @@ extern "C" const char *rptc_status_string(int status)
     case RPTC_ELIMIT: return "a size exceeds what the kernel supports";
     case RPTC_EDEVICE: return "the current device is not a gfx950 GPU";
     case RPTC_EALIAS: return "an output buffer aliases an input the op still reads";
+    case RPTC_EDEPEND: return "a layer of the chain reads or overwrites what a layer of the chain writes: run such layers as separate launches";
     default: break;
     }
     if (status > 0) return hipGetErrorString(static_cast<hipError_t>(status));

@@ -212,6 +212,31 @@ __device__ __forceinline__ uint4 silu_mul8(const uint4 gate, const uint4 up)
     return make_uint4(r[0], r[1], r[2], r[3]);
 }
 
+// A slab's 32 activation pairs of a lane from LDS: one address (XA) and 32 immediate offsets, 128 bytes (32 slots)
+// apart, into XR[0..31].  The reads and their wait are ONE asm statement (a register such a read writes holds
+// nothing until the wait; between two statements the compiler may copy or reuse it), and the outputs are
+// early-clobber: none may share the address register.
+#define RPTC_RELOAD_X32(XR, XA) \
+    asm volatile( \
+        "ds_read_b32 %0, %32 offset:0\n ds_read_b32 %1, %32 offset:128\n ds_read_b32 %2, %32 offset:256\n" \
+        "ds_read_b32 %3, %32 offset:384\n ds_read_b32 %4, %32 offset:512\n ds_read_b32 %5, %32 offset:640\n" \
+        "ds_read_b32 %6, %32 offset:768\n ds_read_b32 %7, %32 offset:896\n ds_read_b32 %8, %32 offset:1024\n" \
+        "ds_read_b32 %9, %32 offset:1152\n ds_read_b32 %10, %32 offset:1280\n ds_read_b32 %11, %32 offset:1408\n" \
+        "ds_read_b32 %12, %32 offset:1536\n ds_read_b32 %13, %32 offset:1664\n ds_read_b32 %14, %32 offset:1792\n" \
+        "ds_read_b32 %15, %32 offset:1920\n ds_read_b32 %16, %32 offset:2048\n ds_read_b32 %17, %32 offset:2176\n" \
+        "ds_read_b32 %18, %32 offset:2304\n ds_read_b32 %19, %32 offset:2432\n ds_read_b32 %20, %32 offset:2560\n" \
+        "ds_read_b32 %21, %32 offset:2688\n ds_read_b32 %22, %32 offset:2816\n ds_read_b32 %23, %32 offset:2944\n" \
+        "ds_read_b32 %24, %32 offset:3072\n ds_read_b32 %25, %32 offset:3200\n ds_read_b32 %26, %32 offset:3328\n" \
+        "ds_read_b32 %27, %32 offset:3456\n ds_read_b32 %28, %32 offset:3584\n ds_read_b32 %29, %32 offset:3712\n" \
+        "ds_read_b32 %30, %32 offset:3840\n ds_read_b32 %31, %32 offset:3968\n s_waitcnt lgkmcnt(0)\n" \
+        : "=&v"((XR)[0]), "=&v"((XR)[1]), "=&v"((XR)[2]), "=&v"((XR)[3]), "=&v"((XR)[4]), "=&v"((XR)[5]), "=&v"((XR)[6]), "=&v"((XR)[7]), \
+          "=&v"((XR)[8]), "=&v"((XR)[9]), "=&v"((XR)[10]), "=&v"((XR)[11]), "=&v"((XR)[12]), "=&v"((XR)[13]), "=&v"((XR)[14]), \
+          "=&v"((XR)[15]), "=&v"((XR)[16]), "=&v"((XR)[17]), "=&v"((XR)[18]), "=&v"((XR)[19]), "=&v"((XR)[20]), "=&v"((XR)[21]), \
+          "=&v"((XR)[22]), "=&v"((XR)[23]), "=&v"((XR)[24]), "=&v"((XR)[25]), "=&v"((XR)[26]), "=&v"((XR)[27]), "=&v"((XR)[28]), \
+          "=&v"((XR)[29]), "=&v"((XR)[30]), "=&v"((XR)[31]) \
+        : "v"(XA) \
+        : "memory");
+
 // COMPACT: partial sums per (row, full slab) and (row, ragged lane) instead of per (row, stream element)
 template <int S, int MODE, int BITS, int XMODE, bool COMPACT, bool AFFINE = false>
 __device__ __forceinline__ void matvec_body(
@@ -579,13 +604,12 @@ __device__ __forceinline__ void matvec_body(
                 // step q of element l multiplies pair slot(slab, q, l) (inference.cu:249)
                 const uint32_t *xp = sx + (slab < T ? 1024 * slab : 1024 * T) + l;
                 if (slab < T) {
-                    // one address and 32 immediate offsets (as inline assembly, or the compiler merges these
-                    // reads with those of the ragged slab and forms 31 addresses with vector adds)
+                    // One address and 32 immediate offsets (as inline assembly, or the compiler merges these reads with
+                    // those of the ragged slab and forms 31 addresses with vector adds).  The reads and their wait are
+                    // ONE statement: a register such a read writes holds nothing until the wait, and between two
+                    // statements the compiler may copy or reuse it.
                     const uint32_t xa = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(xp));
-#pragma unroll
-                    for (int q = 0; q < 32; q++)
-                        asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(xr[q]) : "v"(xa), "n"(128 * q));
-                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                    RPTC_RELOAD_X32(xr, xa);
                 } else {
 #pragma unroll
                     for (int q = 0; q < 32; q++) xr[q] = xp[q * sv.lanes];
@@ -955,25 +979,7 @@ __global__ __launch_bounds__(kMatvecThreads) void matvec_loop_kernel(
                     // that such a read writes holds nothing until the wait, and between two statements the compiler
                     // may copy or reuse it.  Early-clobber outputs: none may share the address register.
                     const uint32_t xa = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(xp));
-                    asm volatile(
-                        "ds_read_b32 %0, %32 offset:0\n ds_read_b32 %1, %32 offset:128\n ds_read_b32 %2, %32 offset:256\n"
-                        "ds_read_b32 %3, %32 offset:384\n ds_read_b32 %4, %32 offset:512\n ds_read_b32 %5, %32 offset:640\n"
-                        "ds_read_b32 %6, %32 offset:768\n ds_read_b32 %7, %32 offset:896\n ds_read_b32 %8, %32 offset:1024\n"
-                        "ds_read_b32 %9, %32 offset:1152\n ds_read_b32 %10, %32 offset:1280\n ds_read_b32 %11, %32 offset:1408\n"
-                        "ds_read_b32 %12, %32 offset:1536\n ds_read_b32 %13, %32 offset:1664\n ds_read_b32 %14, %32 offset:1792\n"
-                        "ds_read_b32 %15, %32 offset:1920\n ds_read_b32 %16, %32 offset:2048\n ds_read_b32 %17, %32 offset:2176\n"
-                        "ds_read_b32 %18, %32 offset:2304\n ds_read_b32 %19, %32 offset:2432\n ds_read_b32 %20, %32 offset:2560\n"
-                        "ds_read_b32 %21, %32 offset:2688\n ds_read_b32 %22, %32 offset:2816\n ds_read_b32 %23, %32 offset:2944\n"
-                        "ds_read_b32 %24, %32 offset:3072\n ds_read_b32 %25, %32 offset:3200\n ds_read_b32 %26, %32 offset:3328\n"
-                        "ds_read_b32 %27, %32 offset:3456\n ds_read_b32 %28, %32 offset:3584\n ds_read_b32 %29, %32 offset:3712\n"
-                        "ds_read_b32 %30, %32 offset:3840\n ds_read_b32 %31, %32 offset:3968\n s_waitcnt lgkmcnt(0)\n"
-                        : "=&v"(xr[0]), "=&v"(xr[1]), "=&v"(xr[2]), "=&v"(xr[3]), "=&v"(xr[4]), "=&v"(xr[5]), "=&v"(xr[6]), "=&v"(xr[7]),
-                          "=&v"(xr[8]), "=&v"(xr[9]), "=&v"(xr[10]), "=&v"(xr[11]), "=&v"(xr[12]), "=&v"(xr[13]), "=&v"(xr[14]),
-                          "=&v"(xr[15]), "=&v"(xr[16]), "=&v"(xr[17]), "=&v"(xr[18]), "=&v"(xr[19]), "=&v"(xr[20]), "=&v"(xr[21]),
-                          "=&v"(xr[22]), "=&v"(xr[23]), "=&v"(xr[24]), "=&v"(xr[25]), "=&v"(xr[26]), "=&v"(xr[27]), "=&v"(xr[28]),
-                          "=&v"(xr[29]), "=&v"(xr[30]), "=&v"(xr[31])
-                        : "v"(xa)
-                        : "memory");
+                    RPTC_RELOAD_X32(xr, xa);
                 } else {
 #pragma unroll
                     for (int q = 0; q < 32; q++) xr[q] = xp[q * sv.lanes];
@@ -1333,9 +1339,10 @@ int prepare_matvec_loop()
 }
 
 int matvec_loop_plan(const rptc_chain_layer *layers, int64_t count, int cus, LoopLayer *out, int *xslot_words,
-                     int *part_floats, int *lds_bytes, int *max_items)
+                     int *part_floats, int *lds_bytes, int *max_items, int *uniform)
 {
     int64_t n_max = 0, part_max = 0, items_max = 1;
+    *uniform = 1;
     for (int64_t k = 0; k < count; k++) {
         const rptc_chain_layer &u = layers[k];
         if (u.n > (int64_t)8 * kXRegs * kMatvecThreads) return RPTC_ELIMIT;      // a thread's two registers hold its share
@@ -1352,6 +1359,7 @@ int matvec_loop_plan(const rptc_chain_layer *layers, int64_t count, int cus, Loo
         d.items_tail = lt ? (d.rows_per_block + d.rw_tail - 1) / d.rw_tail : 0;
         d.full_magic = items_full > 1 ? (uint32_t)(((uint64_t)1 << 32) / (uint64_t)items_full) + 1u : 0u;
         d.same_shape_as_previous = k > 0 && layers[k - 1].m == u.m && layers[k - 1].n == u.n;
+        if (k > 0 && !d.same_shape_as_previous) *uniform = 0;
         // a wave keeps all its elements of a layer in registers: at most kLoopMaxItems of them
         const int64_t total = (u.n >> 11) * (int64_t)items_full + d.items_tail;
         const int64_t per_wave = (total + kMatvecWaves - 1) / kMatvecWaves;
@@ -1371,7 +1379,8 @@ int matvec_loop_plan(const rptc_chain_layer *layers, int64_t count, int cus, Loo
 }
 
 int matvec_loop_launch(const LoopLayer *device_layers, const uint32_t *codebook, int count, int xslot_words,
-                       int part_floats, int lds_bytes, int max_items, int grid, int S, int carry_mode, hipStream_t stream)
+                       int part_floats, int lds_bytes, int max_items, int uniform, int grid, int S, int carry_mode,
+                       hipStream_t stream)
 {
     if (max_items != 3 && max_items != 4) return RPTC_ESHAPE;
 #define RPTC_LOOP_GO(SS, MM)                                                                                          \

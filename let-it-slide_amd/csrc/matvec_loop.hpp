@@ -19,11 +19,13 @@ static_assert(sizeof(LoopLayer) == 64, "a descriptor is one 64-byte line");
 // Fills `out[count]` for a device of `cus` compute units.  Returns 0 when the kernel can run the chain (every layer's
 // activations fit a thread's two registers, a wave has at most four stream elements of a layer, two activation images and
 // two sets of partial sums fit in LDS beside the table), RPTC_ELIMIT when it cannot; the caller has checked pointers,
-// shapes and that no layer depends on another.  max_items: 3 or 4, the kernel variant that holds a wave's elements.
+// shapes and that no layer depends on another.  max_items: 3 or 4, the kernel variant that holds a wave's elements;
+// uniform: 1 when every layer has the shape of the first.
 int matvec_loop_plan(const rptc_chain_layer *layers, int64_t count, int cus, LoopLayer *out, int *xslot_words,
-                     int *part_floats, int *lds_bytes, int *max_items);
+                     int *part_floats, int *lds_bytes, int *max_items, int *uniform);
 // One launch over `count` layers whose descriptors are in device memory; returns hipGetLastError()'s value.
 int matvec_loop_launch(const LoopLayer *device_layers, const uint32_t *codebook, int count, int xslot_words,
-                       int part_floats, int lds_bytes, int max_items, int grid, int S, int carry_mode, hipStream_t stream);
+                       int part_floats, int lds_bytes, int max_items, int uniform, int grid, int S, int carry_mode,
+                       hipStream_t stream);
 
 }  // namespace rptc

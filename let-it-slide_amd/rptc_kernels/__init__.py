@@ -39,6 +39,9 @@ import torch
 
 AS_WRITTEN = 0
 CONTINUOUS = 1
+# statuses of include/rptc_hip.h that callers may want to tell apart
+ELIMIT = -5
+EDEPEND = -8
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(os.path.dirname(_HERE), "librptc_hip.so")
@@ -77,7 +80,6 @@ _SIGNATURES = {
     "rptc_chain_desc_bytes": ([ctypes.POINTER(ChainLayer), _I64], _I64),
     "rptc_chain_plan": ([ctypes.POINTER(ChainLayer), _I64, _VP, _I64, ctypes.POINTER(ChainPlan), _VP], _INT),
     "rptc_decompress_matvec_chain": ([ctypes.POINTER(ChainPlan), _VP, _INT, _INT, _VP, _FP], _INT),
-    "rptc_chain_status": ([ctypes.POINTER(ChainPlan), ctypes.POINTER(ctypes.c_int), _VP], _INT),
     "rptc_matvec_dense": ([_VP, _VP, _VP, _I64, _I64, _INT, _INT, _VP, _FP], _INT),
     "rptc_matvec_t_dense": ([_VP, _VP, _VP, _I64, _I64, _INT, _INT, _VP, _FP], _INT),
     "rptc_decompress_matmul": ([_VP, _VP, _VP, _VP, _I64, _I64, _I64, _INT, _INT, _VP, _FP], _INT),
@@ -670,12 +672,16 @@ def decompress_matvec_rmsnorm_affine(compressed, codebook, x_in, delta, weight, 
 
 
 class MatvecChain:
-    """A chain of ``decompress_matvec_16_{S}_1`` products in one launch (``rptc_decompress_matvec_chain``).
+    """A chain of ``decompress_matvec_16_{S}_1`` products (``rptc_decompress_matvec_chain``).
 
     ``layers`` is a sequence of ``(compressed, x, out)`` tensor triples (int32 stream, fp16 [n], fp16 [m]); the
     tensors are kept alive by the object and their addresses are fixed in the plan, their contents are read at
-    run time.  Dependencies between layers are found from the addresses (a layer that reads what an earlier one
-    writes waits for it).  One codebook and one carry mode serve the whole chain."""
+    run time.  One codebook and one carry mode serve the whole chain.
+
+    Layers that do not depend on each other run in ONE launch.  When the library refuses the one-launch form - a
+    layer reads or overwrites what another writes (``RPTC_EDEPEND``), or a layer is too large for it
+    (``RPTC_ELIMIT``) - ``run`` makes one ``decompress_matvec_16_{S}_1`` launch per layer on the current stream,
+    in order, which is what orders dependent layers; ``one_launch`` tells which of the two it is."""
 
     def __init__(self, layers, codebook):
         layers = list(layers)
@@ -707,28 +713,30 @@ class MatvecChain:
             base = (self.desc.data_ptr() + 255) & ~255
             self.plan = ChainPlan()
             stream = torch.cuda.current_stream().cuda_stream
-            _status(lib.rptc_chain_plan(arr, len(layers), base, need, ctypes.byref(self.plan), ctypes.c_void_p(stream)))
+            rc = lib.rptc_chain_plan(arr, len(layers), base, need, ctypes.byref(self.plan), ctypes.c_void_p(stream))
+        self.one_launch = rc == 0
+        if rc not in (0, EDEPEND, ELIMIT):
+            _status(rc)
 
     def run(self, carry_mode=None, timed=None):
-        """One launch on the current stream; returns elapsed ms (0.0 when not timed)."""
+        """Runs the chain on the current stream; returns elapsed ms (0.0 when not timed)."""
         ms = ctypes.c_float(0.0)
         mode = _carry_mode if carry_mode is None else carry_mode
+        want_ms = _timing if timed is None else timed
+        lib = library()
         with torch.cuda.device(self.codebook.device):
-            stream = torch.cuda.current_stream().cuda_stream
-            rc = library().rptc_decompress_matvec_chain(ctypes.byref(self.plan), self.codebook.data_ptr(), self.S, mode,
-                                                        ctypes.c_void_p(stream),
-                                                        ctypes.byref(ms) if (_timing if timed is None else timed) else None)
-        _status(rc)
-        return float(ms.value)
-
-    def status(self):
-        """Waits for the current stream; 0 when every run so far completed (bit 0: a bounded wait inside the kernel
-        ran out; bit 1: an arrival counter is not zero)."""
-        st = ctypes.c_int(-1)
-        with torch.cuda.device(self.codebook.device):
-            stream = torch.cuda.current_stream().cuda_stream
-            _status(library().rptc_chain_status(ctypes.byref(self.plan), ctypes.byref(st), ctypes.c_void_p(stream)))
-        return st.value
+            stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+            if self.one_launch:
+                _status(lib.rptc_decompress_matvec_chain(ctypes.byref(self.plan), self.codebook.data_ptr(), self.S, mode,
+                                                         stream, ctypes.byref(ms) if want_ms else None))
+                return float(ms.value)
+            fn = getattr(lib, f"rptc_decompress_matvec_16_{self.S}_1")
+            total = 0.0
+            for c, x, out in self.layers:
+                _status(fn(c.data_ptr(), self.codebook.data_ptr(), x.data_ptr(), out.data_ptr(), out.size(0), x.size(0),
+                           mode, stream, ctypes.byref(ms) if want_ms else None))
+                total += float(ms.value)
+        return total
 
 
 def matvec_bits_dense(compressed, codebook, out, bits):

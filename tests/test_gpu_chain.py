@@ -1,6 +1,7 @@
-"""rptc_decompress_matvec_chain on the GPU: a chain of fused decode + mat-vecs in one launch.  Every layer's output is
-held to the double-precision product of the bit-exact dense matrix (rel-L2 1e-3, the mat-vec's bar) on the input
-the chain itself fed it, to the per-launch kernel on the same input, and to itself from run to run (bit for bit)."""
+"""rptc_decompress_matvec_chain on the GPU: a chain of independent fused decode + mat-vecs in one launch.  Every layer's
+output is held to the double-precision product of the bit-exact dense matrix (rel-L2 1e-3, the mat-vec's bar) on its
+input, to the per-launch kernel on the same input, and to itself from run to run (bit for bit).  Chains with
+dependencies are refused by the library (RPTC_EDEPEND) and run by `MatvecChain` as one launch per layer."""
 import ctypes
 
 import numpy as np
@@ -70,7 +71,7 @@ def test_chain_of_independent_layers(rk, oracle, S, mode):
         layers.append((comp, x, out))
     chain = rk.MatvecChain(layers, cb)
     chain.run(carry_mode=mode)
-    assert chain.status() == 0
+    assert chain.one_launch
     first = [out.clone() for _, _, out in layers]
     for comp, x, out in layers:
         assert not torch.isnan(out).any()
@@ -92,15 +93,15 @@ def test_chain_of_independent_layers(rk, oracle, S, mode):
     for _, _, out in layers:
         out.fill_(float("nan"))
     chain.run(carry_mode=mode)
-    assert chain.status() == 0
+    assert chain.one_launch
     for (_, _, out), ref in zip(layers, first):
         assert torch.equal(out.view(torch.int16), ref.view(torch.int16))
 
 
 @pytest.mark.parametrize("mode", [0, 1])
 def test_chain_of_dependent_layers_at_the_llama_shapes(rk, mode):
-    """out of one layer is the next one's input (4096 -> 4096 -> 11008 -> 4096 -> 4096): every layer starts behind the
-    grid-wide counter.  Each layer is checked on the input the chain gave it."""
+    """out of one layer is the next one's input (4096 -> 4096 -> 11008 -> 4096 -> 4096): the library refuses the one-launch
+    form and the chain runs as a launch per layer, in order.  Each layer is checked on the input the chain gave it."""
     S = 8
     cb = (rand_half(2 << S, seed=6).float() * 0.02).half().cuda()       # keeps the activations in fp16 range
     dims = [4096, 4096, 11008, 4096, 4096]
@@ -110,11 +111,11 @@ def test_chain_of_dependent_layers_at_the_llama_shapes(rk, mode):
         n, m = dims[i], dims[i + 1]
         layers.append((rand_codes(m * n // 16, seed=300 + i).cuda(), bufs[i], bufs[i + 1]))
     chain = rk.MatvecChain(layers, cb)
+    assert not chain.one_launch
     for rep in range(3):
         for b in bufs[1:]:
             b.fill_(float("nan"))
         chain.run(carry_mode=mode)
-        assert chain.status() == 0
         for comp, x, out in layers:
             assert not torch.isnan(out).any()
             check_layer(rk, comp, cb, x, out, S, mode)
@@ -127,7 +128,8 @@ def test_chain_of_dependent_layers_at_the_llama_shapes(rk, mode):
 
 def test_chain_orders_layers_that_share_a_buffer(rk):
     """Two layers write the same output (the later one wins), and a third reads an input that an earlier one
-    overwrites afterwards (it must read the old contents): the plan finds the hazards from the addresses."""
+    overwrites afterwards (it must read the old contents): the plan finds the hazards from the addresses and the
+    layers run as launches in order."""
     S, m, n = 8, 1024, 2048
     cb = rand_half(2 << S, seed=8).cuda()
     c = [rand_codes(m * n // 16, seed=400 + i).cuda() for i in range(4)]
@@ -135,7 +137,9 @@ def test_chain_orders_layers_that_share_a_buffer(rk):
     shared = torch.zeros(m, dtype=torch.float16, device="cuda")
     a = torch.zeros(n, dtype=torch.float16, device="cuda")
     layers = [(c[0], x0, shared), (c[1], x1, shared)]
-    rk.MatvecChain(layers, cb).run()
+    chain = rk.MatvecChain(layers, cb)
+    assert not chain.one_launch
+    chain.run()
     y = torch.zeros(m, dtype=torch.float16, device="cuda")
     rk.decompress_matvec_16_8_1(c[1].reshape(1, m, 128), cb, x1, y)
     assert rel_l2(np_f16(shared), np_f16(y).astype(np.float64)) < REL_L2_TOL
@@ -154,9 +158,10 @@ def test_chain_orders_layers_that_share_a_buffer(rk):
     assert rel_l2(np_f16(a), np_f16(y1).astype(np.float64)) < REL_L2_TOL
 
 
-def test_long_chain_reuses_slots_and_counters(rk):
-    """200 layers over 8 streams (the three activation slots, two partial-sum buffers and their counters go round
-    many times), the headline shape included; outputs of layers with equal inputs are equal bit for bit."""
+def test_long_chain_at_the_headline_shape(rk):
+    """200 independent 4096 x 11008 layers over 8 streams and 3 activation vectors (the two activation images and the
+    two sets of partial sums of the loop go round many times); outputs of layers with equal inputs are equal bit for
+    bit."""
     S = 8
     cb = rand_half(2 << S, seed=12).cuda()
     m, n = 4096, 11008
@@ -166,7 +171,7 @@ def test_long_chain_reuses_slots_and_counters(rk):
     layers = [(comps[i % 8], xs[i % 3], outs[i]) for i in range(200)]
     chain = rk.MatvecChain(layers, cb)
     chain.run()
-    assert chain.status() == 0
+    assert chain.one_launch
     for i in range(24):
         check_layer(rk, comps[i % 8], cb, xs[i % 3], outs[i], S, 0)
     for i in range(24, 200):
@@ -187,7 +192,7 @@ def test_short_chains(rk, count):
     chain = rk.MatvecChain(layers, cb)
     for mode in (0, 1):
         chain.run(carry_mode=mode)
-        assert chain.status() == 0
+        assert chain.one_launch
         for comp, x, out in layers:
             assert not torch.isnan(out).any()
             check_layer(rk, comp, cb, x, out, S, mode)
@@ -204,7 +209,7 @@ def test_chain_with_four_elements_a_wave(rk):
                        torch.full((m,), float("nan"), dtype=torch.float16, device="cuda")))
     chain = rk.MatvecChain(layers, cb)
     chain.run(carry_mode=1)
-    assert chain.status() == 0
+    assert chain.one_launch
     first = [out.clone() for _, _, out in layers]
     for comp, x, out in layers:
         check_layer(rk, comp, cb, x, out, S, 1)
@@ -227,36 +232,10 @@ def test_chain_of_random_shapes(rk, seed):
                        torch.full((m,), float("nan"), dtype=torch.float16, device="cuda")))
     chain = rk.MatvecChain(layers, cb)
     chain.run(carry_mode=mode)
-    assert chain.status() == 0
+    assert chain.one_launch
     for comp, x, out in layers:
         assert not torch.isnan(out).any()
         check_layer(rk, comp, cb, x, out, S, mode)
-
-
-def test_chain_gives_up_when_the_grid_cannot_arrive(rk):
-    """A plan that expects one more workgroup than the grid has can never pass its grid-wide counter: with a small
-    spin limit every wave gives up, the kernel ends by itself and the status says so.  (Forced from the host: the
-    expected arrivals and the spin limit are fields of the plan.)"""
-    S, m, n = 8, 2048, 2048
-    cb = rand_half(2 << S, seed=13).cuda()
-    a = rand_half(n, seed=14).cuda()
-    b = torch.zeros(m, dtype=torch.float16, device="cuda")
-    c = torch.zeros(m, dtype=torch.float16, device="cuda")
-    comps = [rand_codes(m * n // 16, seed=800 + i).cuda() for i in range(2)]
-    chain = rk.MatvecChain([(comps[0], a, b), (comps[1], b, c)], cb)
-    words = (ctypes.c_uint32 * 20).from_buffer(chain.plan)
-    grid = words[5]
-    assert words[11] == grid                       # arrivals
-    words[11] = grid + 1
-    words[12] = 2000                               # spin limit
-    chain.run()
-    st = chain.status()                            # waits for the kernel: it must have ended
-    assert st & 1
-    # planned again, the chain runs to the end
-    chain = rk.MatvecChain([(comps[0], a, b), (comps[1], b, c)], cb)
-    chain.run()
-    assert chain.status() == 0
-    check_layer(rk, comps[1], cb, b, c, S, 0)
 
 
 def test_chain_rejects_bad_arguments(rk):
@@ -266,13 +245,58 @@ def test_chain_rejects_bad_arguments(rk):
           torch.zeros(64, dtype=torch.float16, device="cuda"))
     with pytest.raises(RuntimeError):
         rk.MatvecChain([], cb)
-    with pytest.raises(RuntimeError):                       # n too long for a thread's two registers
-        rk.MatvecChain([(torch.zeros(4 * 16448 // 16, dtype=torch.int32, device="cuda"),
-                         torch.zeros(16448, dtype=torch.float16, device="cuda"), torch.zeros(4, dtype=torch.float16, device="cuda"))], cb)
     chain = rk.MatvecChain([ok], cb)
+    assert chain.one_launch
     assert lib.rptc_decompress_matvec_chain(None, cb.data_ptr(), 8, 0, None, None) == -1
     assert lib.rptc_decompress_matvec_chain(ctypes.byref(chain.plan), cb.data_ptr(), 7, 0, None, None) == -2
     assert lib.rptc_decompress_matvec_chain(ctypes.byref(chain.plan), cb.data_ptr(), 8, 3, None, None) == -4
     blank = rk.ChainPlan()
     assert lib.rptc_decompress_matvec_chain(ctypes.byref(blank), cb.data_ptr(), 8, 0, None, None) == -2
     assert lib.rptc_chain_desc_bytes(None, 1) == -1
+
+
+def plan_status(rk, layers):
+    arr = (rk.ChainLayer * len(layers))()
+    for i, (c, x, out) in enumerate(layers):
+        arr[i] = rk.ChainLayer(c.data_ptr(), x.data_ptr(), out.data_ptr(), out.numel(), x.numel())
+    lib = rk.library()
+    need = lib.rptc_chain_desc_bytes(arr, len(layers))
+    assert need > 0
+    desc = torch.zeros(need + 256, dtype=torch.uint8, device="cuda")
+    plan = rk.ChainPlan()
+    return lib.rptc_chain_plan(arr, len(layers), (desc.data_ptr() + 255) & ~255, need, ctypes.byref(plan), None)
+
+
+def test_chain_plan_refuses_dependent_layers_and_layers_too_large(rk):
+    """The C ABI itself: RPTC_EDEPEND (-8) when an output overlaps anything a layer of the chain reads or another layer
+    writes, RPTC_ELIMIT (-5) when a layer does not fit the one-launch form; `MatvecChain` then launches per layer."""
+    m = n = 2048
+    comp = [torch.zeros(m * n // 16, dtype=torch.int32, device="cuda") for _ in range(2)]
+    a, b, c = (torch.zeros(n, dtype=torch.float16, device="cuda") for _ in range(3))
+    assert plan_status(rk, [(comp[0], a, b), (comp[1], a, c)]) == 0
+    assert plan_status(rk, [(comp[0], a, b), (comp[1], b, c)]) == -8           # read after write
+    assert plan_status(rk, [(comp[0], a, b), (comp[1], c, a)]) == -8           # write after read
+    assert plan_status(rk, [(comp[0], a, b), (comp[1], c, b)]) == -8           # write after write
+    assert plan_status(rk, [(comp[0], a, a)]) == -8                            # a layer's output is its own input
+    assert plan_status(rk, [(comp[0], a, comp[1].view(torch.float16)[:m]), (comp[1], a, c)]) == -8    # output inside a stream
+    half = b[:m // 2]
+    assert plan_status(rk, [(comp[0][: m // 2 * n // 16], a, half), (comp[1][: m // 2 * n // 16], a, b[m // 4: m // 4 + m // 2])]) == -8
+    # n too long for a thread's two activation registers; 16384 x 8192 has eight stream elements a wave
+    long_n = (torch.zeros(4 * 16448 // 16, dtype=torch.int32, device="cuda"), torch.zeros(16448, dtype=torch.float16, device="cuda"),
+              torch.zeros(4, dtype=torch.float16, device="cuda"))
+    assert plan_status(rk, [long_n]) == -5
+    big = (torch.zeros(16384 * 8192 // 16, dtype=torch.int32, device="cuda"), torch.zeros(8192, dtype=torch.float16, device="cuda"),
+           torch.zeros(16384, dtype=torch.float16, device="cuda"))
+    assert plan_status(rk, [big]) == -5
+
+
+def test_chain_too_large_for_one_launch_runs_as_launches(rk):
+    S, m, n = 8, 16384, 8192
+    cb = rand_half(2 << S, seed=31).cuda()
+    layers = [(rand_codes(m * n // 16, seed=940 + i).cuda(), rand_half(n, seed=950 + i).cuda(),
+               torch.full((m,), float("nan"), dtype=torch.float16, device="cuda")) for i in range(2)]
+    chain = rk.MatvecChain(layers, cb)
+    assert not chain.one_launch
+    chain.run(carry_mode=1)
+    for comp, x, out in layers:
+        check_layer(rk, comp, cb, x, out, S, 1)
