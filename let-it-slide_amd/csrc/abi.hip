@@ -9,6 +9,7 @@ namespace rptc {
 int prepare_decompress();
 int prepare_matvec();
 int prepare_matvec_loop();
+int prepare_matvec_steady();
 int prepare_matvec_t(int device);
 int prepare_matmul(int device);
 int prepare_hadamard();
@@ -43,6 +44,7 @@ int device_info(DeviceInfo **out)
         if ((rc = prepare_decompress())) return rc;
         if ((rc = prepare_matvec())) return rc;
         if ((rc = prepare_matvec_loop())) return rc;
+        if ((rc = prepare_matvec_steady())) return rc;
         if ((rc = prepare_matvec_t(dev))) return rc;
         if ((rc = prepare_matmul(dev))) return rc;
         if ((rc = prepare_hadamard())) return rc;

@@ -1379,8 +1379,7 @@ int matvec_loop_plan(const rptc_chain_layer *layers, int64_t count, int cus, Loo
 }
 
 int matvec_loop_launch(const LoopLayer *device_layers, const uint32_t *codebook, int count, int xslot_words,
-                       int part_floats, int lds_bytes, int max_items, int uniform, int grid, int S, int carry_mode,
-                       hipStream_t stream)
+                       int part_floats, int lds_bytes, int max_items, int grid, int S, int carry_mode, hipStream_t stream)
 {
     if (max_items != 3 && max_items != 4) return RPTC_ESHAPE;
 #define RPTC_LOOP_GO(SS, MM)                                                                                          \

@@ -26,7 +26,10 @@ constexpr uint64_t kChainMagic = 0x5250544343484E33ull;           // "RPTCCHN3"
 struct ChainPlanHost {            // what rptc_chain_t holds (see the header): written by rptc_chain_plan
     uint64_t magic;
     void *device_desc;
-    int32_t count, grid, lds_bytes, xslot_words, part_floats, max_items, uniform;
+    int32_t count, grid, lds_bytes, xslot_words, part_floats, max_items;
+    int32_t steady;               // every layer has one shape, and it fits the kernel of matvec_steady.hip: its geometry follows
+    int32_t m, n, rows_per_block, rw_tail, items_tail;
+    uint32_t full_magic;
     int32_t device;
 };
 static_assert(sizeof(ChainPlanHost) <= sizeof(rptc_chain_t), "the public struct holds the plan");
@@ -104,7 +107,9 @@ extern "C" int rptc_chain_plan(const rptc_chain_layer *layers, int64_t count, vo
     p.xslot_words = xslot_words;
     p.part_floats = part_floats;
     p.max_items = max_items;
-    p.uniform = uniform;
+    p.steady = uniform && matvec_steady_fits(image[0]) ? 1 : 0;
+    p.m = image[0].m, p.n = image[0].n, p.rows_per_block = image[0].rows_per_block;
+    p.rw_tail = image[0].rw_tail, p.items_tail = image[0].items_tail, p.full_magic = image[0].full_magic;
     p.device = dev->device;
     memset(plan, 0, sizeof(*plan));
     memcpy(plan, &p, sizeof(p));
@@ -129,8 +134,16 @@ extern "C" int rptc_decompress_matvec_chain(const rptc_chain_t *plan, const uint
     Timer t;
     rc = t.begin(dev, s, ms);
     if (rc) return rc;
-    rc = matvec_loop_launch(reinterpret_cast<const LoopLayer *>(p.device_desc), reinterpret_cast<const uint32_t *>(codebook),
-                            p.count, p.xslot_words, p.part_floats, p.lds_bytes, p.max_items, p.uniform, p.grid, S, carry_mode, s);
+    auto a_layers = reinterpret_cast<const LoopLayer *>(p.device_desc);
+    auto a_cb = reinterpret_cast<const uint32_t *>(codebook);
+    if (p.steady) {
+        LoopLayer shape{};
+        shape.m = p.m, shape.n = p.n, shape.rows_per_block = p.rows_per_block;
+        shape.rw_tail = p.rw_tail, shape.items_tail = p.items_tail, shape.full_magic = p.full_magic;
+        rc = matvec_steady_launch(a_layers, shape, a_cb, p.count, p.max_items, p.grid, S, carry_mode, s);
+    } else {
+        rc = matvec_loop_launch(a_layers, a_cb, p.count, p.xslot_words, p.part_floats, p.lds_bytes, p.max_items, p.grid, S, carry_mode, s);
+    }
     if (rc) return rc;
     return t.end();
 }

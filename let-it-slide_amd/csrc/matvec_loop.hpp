@@ -25,7 +25,12 @@ int matvec_loop_plan(const rptc_chain_layer *layers, int64_t count, int cus, Loo
                      int *part_floats, int *lds_bytes, int *max_items, int *uniform);
 // One launch over `count` layers whose descriptors are in device memory; returns hipGetLastError()'s value.
 int matvec_loop_launch(const LoopLayer *device_layers, const uint32_t *codebook, int count, int xslot_words,
-                       int part_floats, int lds_bytes, int max_items, int uniform, int grid, int S, int carry_mode,
-                       hipStream_t stream);
+                       int part_floats, int lds_bytes, int max_items, int grid, int S, int carry_mode, hipStream_t stream);
+
+// The same chain when every layer has the shape of `shape` and that shape fits the fixed LDS layout of the kernel of
+// matvec_steady.hip (`matvec_steady_fits`): the loop over layers as one hand-written block.
+bool matvec_steady_fits(const LoopLayer &shape);
+int matvec_steady_launch(const LoopLayer *device_layers, const LoopLayer &shape, const uint32_t *codebook, int count, int max_items,
+                         int grid, int S, int carry_mode, hipStream_t stream);
 
 }  // namespace rptc

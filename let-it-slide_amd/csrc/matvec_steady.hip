@@ -1,0 +1,539 @@
+// A chain of independent mat-vecs of ONE shape in one launch: the steady state of matvec.hip's loop kernel with the whole
+// per-layer loop written as one block of gfx950 assembly.
+//
+// Semantics per layer: rptc_kernels/csrc/rptc_kernels/inference.cu:189-277 of the reference (the op of matvec.hip).
+// The decomposition is the loop kernel's: one 16-wave workgroup per CU owns a block of rows and every slab of those rows;
+// a wave item is 64 consecutive stream elements; a wave keeps its (at most MAXI) elements of a layer in registers, asked
+// for a layer ahead; two activation images and two sets of partial sums take turns, ONE workgroup barrier a layer.
+// What is different: when all layers have one shape, everything about a wave's share that the loop kernel works out
+// again in every layer (element offsets, lane clamps, which lanes start a row, where the partial sums go, where the
+// activations are staged) is worked out once in front of the loop and kept in registers, and the loop body is written
+// by hand:
+//   * a layer costs a wave: one barrier, three scalar loads (the next layer's stream and activation pointers, the
+//     previous layer's output pointer), per element one 16-byte request, the decode block and one LDS store, one or two
+//     reloads of the 32 activation registers as sixteen two-dword LDS reads (an LDS read instruction costs the same for
+//     4 and for 8 bytes a lane), eight LDS stores for its share of the next activations;
+//   * requests and their waits are in one block, so a register with a request in flight is never the compiler's to
+//     touch, and the wait in front of a decode is for that element only (`s_waitcnt vmcnt(N)`, N fixed because every
+//     wave always makes the same number of requests a layer: a slot without an element asks for one cache line);
+//   * LDS layout with fixed strides so that which image / which set of partial sums a layer uses is an immediate
+//     offset (the loop is unrolled over the two parities): table [0, 64 KiB), images 32 KiB each, sets 16 KiB each;
+//     the ragged last slab sits in the image at the full slabs' stride (slot 32 q + l), so its reload is the same
+//     instruction sequence.
+// Every sum has a fixed order: outputs are bit-identical from run to run.
+#include "matvec_loop.hpp"
+#include "rptc_common.hpp"
+
+namespace rptc {
+
+constexpr int kStThreads = 1024, kStWaves = kStThreads / kWave;
+constexpr int kStTableBytes = 65536;                       // 256 rows x 64 lane copies of one half2
+constexpr int kStImageBytes = 32768;                       // one activation image: up to 8 slabs of 1024 slots
+constexpr int kStPartBytes = 16384;                        // one set of partial sums: rows_per_block * (n / 64) floats
+constexpr int kStPartBase = kStTableBytes + 2 * kStImageBytes;
+constexpr int kStLdsBytes = kStPartBase + 2 * kStPartBytes;
+static_assert(kStLdsBytes == kMaxLds, "the layout fills the LDS of a CU");
+constexpr int kStRowWaves = 8;                             // waves 0-7 add up the rows
+
+// ---- registers with fixed numbers: a request's 16 bytes are four consecutive registers, and an asm operand cannot
+// name one register of a tuple
+// stream elements of a wave: item u in v[80 + 4u : 83 + 4u]; next activations: v[72:75], v[76:79]
+// activation pairs of the slab being decoded: slot q in v(96 + q / 2) for even q, v(112 + (q - 1) / 2) for odd q, so
+// that slots q and q + 2 are neighbours and one ds_read2st64_b32 (two dwords 256 bytes apart) fills both
+#define ST_X0 "v96"
+#define ST_X2 "v97"
+#define ST_X4 "v98"
+#define ST_X6 "v99"
+#define ST_X8 "v100"
+#define ST_X10 "v101"
+#define ST_X12 "v102"
+#define ST_X14 "v103"
+#define ST_X16 "v104"
+#define ST_X18 "v105"
+#define ST_X20 "v106"
+#define ST_X22 "v107"
+#define ST_X24 "v108"
+#define ST_X26 "v109"
+#define ST_X28 "v110"
+#define ST_X30 "v111"
+#define ST_X1 "v112"
+#define ST_X3 "v113"
+#define ST_X5 "v114"
+#define ST_X7 "v115"
+#define ST_X9 "v116"
+#define ST_X11 "v117"
+#define ST_X13 "v118"
+#define ST_X15 "v119"
+#define ST_X17 "v120"
+#define ST_X19 "v121"
+#define ST_X21 "v122"
+#define ST_X23 "v123"
+#define ST_X25 "v124"
+#define ST_X27 "v125"
+#define ST_X29 "v126"
+#define ST_X31 "v127"
+
+#define ST_STR2(x) #x
+#define ST_STR(x) ST_STR2(x)
+
+// The 32 activation pairs of a lane for one slab: image P (0 / 1), XA = LDS address of the lane's slot 0 in image 0.
+// The wait covers the scalar loads made at the top of the layer as well (item 0 always reloads).
+#define ST_RD2(LO, HI, BASE, OFF, P)                                                                                  \
+    "ds_read2st64_b32 v[" #LO ":" #HI "], " BASE " offset0:" #P "*128+" #OFF " offset1:" #P "*128+" #OFF "+1\n"
+#define ST_RELOAD(XA, P)                                                                                              \
+    "v_add_u32 %[xb], 0x80, " XA "\n"                                                                                 \
+    ST_RD2(96, 97, XA, 0, P) ST_RD2(98, 99, XA, 2, P) ST_RD2(100, 101, XA, 4, P) ST_RD2(102, 103, XA, 6, P)           \
+    ST_RD2(104, 105, XA, 8, P) ST_RD2(106, 107, XA, 10, P) ST_RD2(108, 109, XA, 12, P) ST_RD2(110, 111, XA, 14, P)    \
+    ST_RD2(112, 113, "%[xb]", 0, P) ST_RD2(114, 115, "%[xb]", 2, P) ST_RD2(116, 117, "%[xb]", 4, P)                   \
+    ST_RD2(118, 119, "%[xb]", 6, P) ST_RD2(120, 121, "%[xb]", 8, P) ST_RD2(122, 123, "%[xb]", 10, P)                  \
+    ST_RD2(124, 125, "%[xb]", 12, P) ST_RD2(126, 127, "%[xb]", 14, P)                                                 \
+    "s_waitcnt lgkmcnt(0)\n"
+
+// ---- the decode block (decode_asm.hpp's schedule with named registers): per 8 steps 4 v_alignbit_b32 (none for shift
+// 0), 4 v_pk_mad_u16 (two window hashes each), 8 address ops, 8 gathers, 8 products; the gathers of 8 steps are in flight
+// while the products of the 8 before are formed
+#define ST_RDPAIR(G, TH, TL)                                  \
+    "v_perm_b32 " TH ", " G ", %[lane4], %[sel]\n"            \
+    "v_and_or_b32 " TL ", " G ", %[mask], %[lane4]\n"         \
+    "ds_read_b32 " TH ", " TH "\n"                            \
+    "ds_read_b32 " TL ", " TL "\n"
+#define ST_READS_A ST_RDPAIR("%[g0]", "%[t0]", "%[t1]") ST_RDPAIR("%[g1]", "%[t2]", "%[t3]") \
+                   ST_RDPAIR("%[g2]", "%[t4]", "%[t5]") ST_RDPAIR("%[g3]", "%[t6]", "%[t7]")
+#define ST_READS_B ST_RDPAIR("%[g0]", "%[u0]", "%[u1]") ST_RDPAIR("%[g1]", "%[u2]", "%[u3]") \
+                   ST_RDPAIR("%[g2]", "%[u4]", "%[u5]") ST_RDPAIR("%[g3]", "%[u6]", "%[u7]")
+#define ST_WINDOWS(SH, EX, EY, EZ, EW)                        \
+    "v_alignbit_b32 %[g0], %[cy], " EX ", " #SH "\n"          \
+    "v_alignbit_b32 %[g1], " EX ", " EY ", " #SH "\n"         \
+    "v_alignbit_b32 %[g2], " EY ", " EZ ", " #SH "\n"         \
+    "v_alignbit_b32 %[g3], " EZ ", " EW ", " #SH "\n"         \
+    "v_pk_mad_u16 %[g0], %[g0], %[g0], %[g0]\n"               \
+    "v_pk_mad_u16 %[g1], %[g1], %[g1], %[g1]\n"               \
+    "v_pk_mad_u16 %[g2], %[g2], %[g2], %[g2]\n"               \
+    "v_pk_mad_u16 %[g3], %[g3], %[g3], %[g3]\n"
+#define ST_WINDOWS0(EX, EY, EZ, EW)                           \
+    "v_pk_mad_u16 %[g0], " EX ", " EX ", " EX "\n"            \
+    "v_pk_mad_u16 %[g1], " EY ", " EY ", " EY "\n"            \
+    "v_pk_mad_u16 %[g2], " EZ ", " EZ ", " EZ "\n"            \
+    "v_pk_mad_u16 %[g3], " EW ", " EW ", " EW "\n"
+// window register g0 = {carry, x}: slots 28 + j (high window), j (low); g1 = {x, y}: 16 + j, 4 + j; g2 = {y, z}: 20 + j,
+// 8 + j; g3 = {z, w}: 24 + j, 12 + j, for shift 12 - 4 j (inference.cu:237-250)
+#define ST_DOTS_FIRST(T, XA, XB, XC, XD, XE, XF, XG, XH)      \
+    "v_dot2_f32_f16 %[a0], %[" T "0], " XA ", 0\n"            \
+    "v_dot2_f32_f16 %[a1], %[" T "1], " XB ", 0\n"            \
+    "v_dot2_f32_f16 %[a2], %[" T "2], " XC ", 0\n"            \
+    "v_dot2_f32_f16 %[a3], %[" T "3], " XD ", 0\n"            \
+    "v_dot2c_f32_f16 %[a0], %[" T "4], " XE "\n"              \
+    "v_dot2c_f32_f16 %[a1], %[" T "5], " XF "\n"              \
+    "v_dot2c_f32_f16 %[a2], %[" T "6], " XG "\n"              \
+    "v_dot2c_f32_f16 %[a3], %[" T "7], " XH "\n"
+#define ST_DOTS(T, XA, XB, XC, XD, XE, XF, XG, XH)            \
+    "v_dot2c_f32_f16 %[a0], %[" T "0], " XA "\n"              \
+    "v_dot2c_f32_f16 %[a1], %[" T "1], " XB "\n"              \
+    "v_dot2c_f32_f16 %[a2], %[" T "2], " XC "\n"              \
+    "v_dot2c_f32_f16 %[a3], %[" T "3], " XD "\n"              \
+    "v_dot2c_f32_f16 %[a0], %[" T "4], " XE "\n"              \
+    "v_dot2c_f32_f16 %[a1], %[" T "5], " XF "\n"              \
+    "v_dot2c_f32_f16 %[a2], %[" T "6], " XG "\n"              \
+    "v_dot2c_f32_f16 %[a3], %[" T "7], " XH "\n"
+// OWN: what a row's first lane takes for the 16 bits in front of its element (its own last word as written,
+// inference.cu:232; the word in front of the row, or zero in slab 0, in continuous mode); FIRST: the lanes that start a row
+#define ST_DECODE(EX, EY, EZ, EW, OWN, FIRST)                                                                         \
+    /* a DPP operand must not have been written by a vector op in the two instructions before */                     \
+    "s_nop 1\n"                                                                                                       \
+    "s_mov_b64 vcc, " FIRST "\n"                                                                                      \
+    "v_cndmask_b32_dpp %[cy], " EW ", " OWN ", vcc wave_shr:1 row_mask:0xf bank_mask:0xf bound_ctrl:1\n"              \
+    ST_WINDOWS(12, EX, EY, EZ, EW) ST_READS_A                                                                         \
+    ST_WINDOWS(8, EX, EY, EZ, EW) ST_READS_B                                                                          \
+    "s_waitcnt lgkmcnt(8)\n"                                                                                          \
+    ST_DOTS_FIRST("t", ST_X28, ST_X0, ST_X16, ST_X4, ST_X20, ST_X8, ST_X24, ST_X12)                                   \
+    ST_WINDOWS(4, EX, EY, EZ, EW) ST_READS_A                                                                          \
+    "s_waitcnt lgkmcnt(8)\n"                                                                                          \
+    ST_DOTS("u", ST_X29, ST_X1, ST_X17, ST_X5, ST_X21, ST_X9, ST_X25, ST_X13)                                         \
+    ST_WINDOWS0(EX, EY, EZ, EW) ST_READS_B                                                                            \
+    "s_waitcnt lgkmcnt(8)\n"                                                                                          \
+    ST_DOTS("t", ST_X30, ST_X2, ST_X18, ST_X6, ST_X22, ST_X10, ST_X26, ST_X14)                                        \
+    "s_waitcnt lgkmcnt(0)\n"                                                                                          \
+    ST_DOTS("u", ST_X31, ST_X3, ST_X19, ST_X7, ST_X23, ST_X11, ST_X27, ST_X15)
+
+// ---- one element of a layer.  U: which of the wave's elements; X, Y, Z, W / QUAD: its four registers; P: parity of
+// the layer; NEED: requests that may still be in flight when this element's has arrived.
+// Behind the last product the next layer's request for this slot goes out at once (three instructions between a dot
+// product and another kind of vector op that reads its result are needed anyway), then the four sums become one
+// and go to LDS under the mask of the lanes that hold an element of a row that exists.
+// A wave without a U-th element makes the request all the same (its offset register points at the first cache line of
+// the stream): every wave then has the same number of requests in flight, and the waits can be immediates.
+#define ST_ITEM_HEAD(U, P, NEED)                                                                                      \
+    "s_cmp_le_u32 %[nitems], " #U "\n"                                                                                \
+    "s_cbranch_scc1 7" #U "f\n"                                                                                       \
+    "s_setprio 3-" #U "\n"                                                                                            \
+    "s_bitcmp1_b32 %[rl], " #U "\n"                                                                                   \
+    "s_cbranch_scc0 5" #U "f\n"                                                                                       \
+    ST_RELOAD("%[xa" #U "]", P)                                                                                       \
+    "5" #U ":\n"                                                                                                      \
+    "s_waitcnt vmcnt(" #NEED ")\n"
+#define ST_ITEM_TAIL(U, P, REQUEST)                                                                                   \
+    REQUEST                                                                                                           \
+    "s_mov_b64 exec, %[keep" #U "]\n"                                                                                 \
+    "s_nop 0\n"                                                                                                       \
+    "v_add_f32 %[a0], %[a0], %[a1]\n"                                                                                 \
+    "v_add_f32 %[a2], %[a2], %[a3]\n"                                                                                 \
+    "v_add_f32 %[a0], %[a0], %[a2]\n"                                                                                 \
+    "ds_write_b32 %[pa" #U "], %[a0] offset:" #P "*16384\n"                                                           \
+    "s_mov_b64 exec, -1\n"                                                                                            \
+    "s_branch 8" #U "f\n"                                                                                             \
+    "7" #U ":\n"                                                                                                      \
+    REQUEST                                                                                                           \
+    "8" #U ":\n"
+#define ST_REQUEST_AW(U, QUAD) "global_load_dwordx4 " QUAD ", %[vo" #U "], %[cn] nt\n"
+#define ST_REQUEST_CT(U, QUAD) "global_load_dwordx4 " QUAD ", %[vo" #U "], %[cn] nt\n"                               \
+                               "global_load_dword %[cw" #U "], %[co" #U "], %[cn]\n"
+// as written (MODE 0): a row's first lane takes its own last word; continuous (MODE 1): the word in front of the row
+#define ST_ITEM_0(U, X, Y, Z, W, QUAD, P, NEED)                                                                       \
+    ST_ITEM_HEAD(U, P, NEED) ST_DECODE(X, Y, Z, W, W, "%[first" #U "]") ST_ITEM_TAIL(U, P, ST_REQUEST_AW(U, QUAD))
+#define ST_ITEM_1(U, X, Y, Z, W, QUAD, P, NEED)                                                                       \
+    ST_ITEM_HEAD(U, P, NEED) "v_and_b32 %[own], %[cm" #U "], %[cw" #U "]\n"                                           \
+    ST_DECODE(X, Y, Z, W, "%[own]", "%[first" #U "]") ST_ITEM_TAIL(U, P, ST_REQUEST_CT(U, QUAD))
+
+// ---- the rows of the layer in front: waves 0-7 add a row's n / 64 partial sums (lanes i, i + 64, i + 128, i + 192 in
+// that order, then across the lanes with DPP adds: rows of 16, row 0 into 1 and 2 into 3, rows 0-1 into 2-3), round
+// once to fp16 and lane 63 stores.  P: parity of the set that is read.
+#define ST_DPP_ADD(CTRL) "s_nop 1\n v_add_f32_dpp %[a0], %[a0], %[a0] " CTRL "\n"
+#define ST_ROWS(P)                                                                                                    \
+    "s_cmp_eq_u32 %[nr], 0\n"                                                                                         \
+    "s_cbranch_scc1 92f\n"                                                                                            \
+    "v_mov_b32 %[g0], %[rs]\n"                                                                                        \
+    "v_mov_b32 %[g1], %[oo]\n"                                                                                        \
+    "s_mov_b32 %[j], %[nr]\n"                                                                                         \
+    "91:\n"                                                                                                           \
+    "v_mov_b32 %[t0], 0\n v_mov_b32 %[t1], 0\n v_mov_b32 %[t2], 0\n v_mov_b32 %[t3], 0\n"                             \
+    "s_mov_b64 exec, %[rm0]\n ds_read_b32 %[t0], %[g0] offset:" #P "*16384\n"                                         \
+    "s_mov_b64 exec, %[rm1]\n ds_read_b32 %[t1], %[g0] offset:" #P "*16384+256\n"                                     \
+    "s_mov_b64 exec, %[rm2]\n ds_read_b32 %[t2], %[g0] offset:" #P "*16384+512\n"                                     \
+    "s_mov_b64 exec, %[rm3]\n ds_read_b32 %[t3], %[g0] offset:" #P "*16384+768\n"                                     \
+    "s_mov_b64 exec, -1\n"                                                                                            \
+    "s_waitcnt lgkmcnt(0)\n"                                                                                          \
+    "v_add_f32 %[a0], %[t0], %[t1]\n"                                                                                 \
+    "v_add_f32 %[a0], %[a0], %[t2]\n"                                                                                 \
+    "v_add_f32 %[a0], %[a0], %[t3]\n"                                                                                 \
+    ST_DPP_ADD("row_shr:1 row_mask:0xf bank_mask:0xf")                                                                \
+    ST_DPP_ADD("row_shr:2 row_mask:0xf bank_mask:0xf")                                                                \
+    ST_DPP_ADD("row_shr:4 row_mask:0xf bank_mask:0xf")                                                                \
+    ST_DPP_ADD("row_shr:8 row_mask:0xf bank_mask:0xf")                                                                \
+    ST_DPP_ADD("row_bcast:15 row_mask:0xa bank_mask:0xf")                                                             \
+    ST_DPP_ADD("row_bcast:31 row_mask:0xc bank_mask:0xf")                                                             \
+    "v_cvt_f16_f32 %[a0], %[a0]\n"                                                                                    \
+    "s_mov_b64 exec, %[l63]\n"                                                                                        \
+    "global_store_short %[g1], %[a0], %[op]\n"                                                                        \
+    "s_mov_b64 exec, -1\n"                                                                                            \
+    "v_add_u32 %[g0], %[rstep], %[g0]\n"                                                                              \
+    "v_add_u32 %[g1], 16, %[g1]\n"                                                                                    \
+    "s_sub_u32 %[j], %[j], 1\n"                                                                                       \
+    "s_cmp_lg_u32 %[j], 0\n"                                                                                          \
+    "s_cbranch_scc1 91b\n"                                                                                            \
+    "92:\n"
+
+// ---- a thread's share of the next layer's activations into image P (halves 8 idx .. 8 idx + 7 go to the four planes,
+// inference.cu:215-221; the addresses were worked out in front of the loop)
+#define ST_STAGE(P)                                                                                                   \
+    "s_mov_b64 exec, %[stm0]\n"                                                                                       \
+    "ds_write_b32 %[sa0], v72 offset:" #P "*32768\n ds_write_b32 %[sa1], v73 offset:" #P "*32768\n"                   \
+    "ds_write_b32 %[sa2], v74 offset:" #P "*32768\n ds_write_b32 %[sa3], v75 offset:" #P "*32768\n"                   \
+    "s_mov_b64 exec, %[stm1]\n"                                                                                       \
+    "ds_write_b32 %[sa4], v76 offset:" #P "*32768\n ds_write_b32 %[sa5], v77 offset:" #P "*32768\n"                   \
+    "ds_write_b32 %[sa6], v78 offset:" #P "*32768\n ds_write_b32 %[sa7], v79 offset:" #P "*32768\n"                   \
+    "s_mov_b64 exec, -1\n"
+
+// ---- the loop.  MODE: 0 as written, 1 continuous; LPI: requests per element (1; 2 continuous); M: elements a wave holds.
+// Requests in flight, oldest first, when element u's is waited for: u's own, the later elements' of this layer, the two
+// activation requests made at the top of this layer, the earlier elements' of the next layer: NEED = (M - 1) * LPI + 2
+// may stay in flight.  When the activations are staged the M * LPI element requests made behind them may stay in
+// flight (STW).  Stores of the rows phase sit in the same queue behind all of them: they only make a wait stricter.
+#define ST_POINTERS                                                                                                   \
+    /* the layer behind the one k counts (clamped to the last) and the layer in front of it (clamped to the first) */ \
+    "s_add_u32 %[kn], %[k], 1\n"                                                                                      \
+    "s_min_u32 %[kn], %[kn], %[last]\n"                                                                               \
+    "s_lshl_b32 %[kn], %[kn], 6\n"                                                                                    \
+    "s_load_dwordx2 %[cn], %[dc], %[kn]\n"                                                                            \
+    "s_load_dwordx2 %[xn], %[dx], %[kn]\n"                                                                            \
+    "s_max_u32 %[kn], %[k], 1\n"                                                                                      \
+    "s_sub_u32 %[kn], %[kn], 1\n"                                                                                     \
+    "s_lshl_b32 %[kn], %[kn], 6\n"                                                                                    \
+    "s_load_dwordx2 %[op], %[dq], %[kn]\n"
+#define ST_XREQUESTS                                                                                                  \
+    "global_load_dwordx4 v[72:75], %[xo0], %[xn]\n"                                                                   \
+    "global_load_dwordx4 v[76:79], %[xo1], %[xn]\n"
+
+#define ST_ITEMS_3(MODE, P, NEED)                                                                                     \
+    ST_ITEM_##MODE(0, "v80", "v81", "v82", "v83", "v[80:83]", P, NEED)                                                \
+    ST_ITEM_##MODE(1, "v84", "v85", "v86", "v87", "v[84:87]", P, NEED)                                                \
+    ST_ITEM_##MODE(2, "v88", "v89", "v90", "v91", "v[88:91]", P, NEED)
+#define ST_ITEMS_4(MODE, P, NEED) ST_ITEMS_3(MODE, P, NEED) ST_ITEM_##MODE(3, "v92", "v93", "v94", "v95", "v[92:95]", P, NEED)
+#define ST_REQUESTS_3(MODE) ST_REQUEST_##MODE(0, "v[80:83]") ST_REQUEST_##MODE(1, "v[84:87]") ST_REQUEST_##MODE(2, "v[88:91]")
+#define ST_REQUESTS_4(MODE) ST_REQUESTS_3(MODE) ST_REQUEST_##MODE(3, "v[92:95]")
+#define ST_REQUEST_0(U, QUAD) ST_REQUEST_AW(U, QUAD)
+#define ST_REQUEST_1(U, QUAD) ST_REQUEST_CT(U, QUAD)
+
+// layer k of parity P (Q the other one): on entry the pointers of layer k + 1 and of layer k - 1 have arrived, image P
+// holds layer k's activations and set Q layer k - 1's partial sums
+#define ST_LAYER(P, Q, MODE, M, NEED, STW)                                                                            \
+    ST_XREQUESTS                                                                                                      \
+    ST_ITEMS_##M(MODE, P, NEED)                                                                                       \
+    "s_setprio 3\n"                                                                                                   \
+    "s_waitcnt vmcnt(" #STW ")\n"                                                                                     \
+    ST_STAGE(Q)                                                                                                       \
+    "s_cmp_eq_u32 %[k], 0\n"                                                                                          \
+    "s_cbranch_scc1 93f\n"                                                                                            \
+    ST_ROWS(Q)                                                                                                        \
+    "93:\n"                                                                                                           \
+    "s_add_u32 %[k], %[k], 1\n"                                                                                       \
+    ST_POINTERS                                                                                                       \
+    "s_waitcnt lgkmcnt(0)\n"                                                                                          \
+    "s_barrier\n"
+
+#define ST_BODY(MODE, M, NEED, STW)                                                                                   \
+    "s_mov_b32 %[k], 0\n"                                                                                             \
+    "s_mov_b32 %[kn], 0\n"                                                                                            \
+    "s_load_dwordx2 %[cn], %[dc], %[kn]\n"                                                                            \
+    "s_load_dwordx2 %[xn], %[dx], %[kn]\n"                                                                            \
+    "s_waitcnt lgkmcnt(0)\n"                                                                                          \
+    ST_XREQUESTS                                                                                                      \
+    ST_REQUESTS_##M(MODE)                                                                                             \
+    "s_waitcnt vmcnt(" #STW ")\n"                                                                                     \
+    ST_STAGE(0)                                                                                                       \
+    ST_POINTERS                                                                                                       \
+    "s_waitcnt lgkmcnt(0)\n"                                                                                          \
+    "s_barrier\n"                                                                                                     \
+    "10:\n"                                                                                                           \
+    ST_LAYER(0, 1, MODE, M, NEED, STW)                                                                                \
+    "s_cmp_ge_u32 %[k], %[count]\n"                                                                                   \
+    "s_cbranch_scc1 11f\n"                                                                                            \
+    ST_LAYER(1, 0, MODE, M, NEED, STW)                                                                                \
+    "s_cmp_lt_u32 %[k], %[count]\n"                                                                                   \
+    "s_cbranch_scc1 10b\n"                                                                                            \
+    /* the last layer's rows: its partial sums are in set 1 (an even number of layers) or set 0 */                    \
+    ST_ROWS(1)                                                                                                        \
+    "s_branch 12f\n"                                                                                                  \
+    "11:\n"                                                                                                           \
+    ST_ROWS(0)                                                                                                        \
+    "12:\n"                                                                                                           \
+    "s_waitcnt vmcnt(0)\n"
+
+// what the loop reads and the registers it works in
+#define ST_OUT_COMMON                                                                                                 \
+    [a0] "=&v"(a0), [a1] "=&v"(a1), [a2] "=&v"(a2), [a3] "=&v"(a3), [cy] "=&v"(cy), [g0] "=&v"(g0), [g1] "=&v"(g1),  \
+    [g2] "=&v"(g2), [g3] "=&v"(g3), [t0] "=&v"(t0), [t1] "=&v"(t1), [t2] "=&v"(t2), [t3] "=&v"(t3), [t4] "=&v"(t4),  \
+    [t5] "=&v"(t5), [t6] "=&v"(t6), [t7] "=&v"(t7), [u0] "=&v"(u0), [u1] "=&v"(u1), [u2] "=&v"(u2), [u3] "=&v"(u3),  \
+    [u4] "=&v"(u4), [u5] "=&v"(u5), [u6] "=&v"(u6), [u7] "=&v"(u7), [xb] "=&v"(xb), [k] "=&s"(k), [kn] "=&s"(kn),    \
+    [j] "=&s"(j), [cn] "=&s"(cn), [xn] "=&s"(xn), [op] "=&s"(op)
+#define ST_IN_COMMON                                                                                                  \
+    [lane4] "v"(lane4), [mask] "s"(0xFF00u), [sel] "s"(0x0C0C0700u), [dc] "s"(dc), [dx] "s"(dx), [dq] "s"(dout),      \
+    [count] "s"(s_count), [last] "s"(s_count - 1), [nitems] "s"(s_nitems), [rl] "s"(rl), [xo0] "v"(xo[0]), [xo1] "v"(xo[1]),\
+    [sa0] "v"(sa[0]), [sa1] "v"(sa[1]), [sa2] "v"(sa[2]), [sa3] "v"(sa[3]), [sa4] "v"(sa[4]), [sa5] "v"(sa[5]),       \
+    [sa6] "v"(sa[6]), [sa7] "v"(sa[7]), [stm0] "s"(stm[0]), [stm1] "s"(stm[1]), [rs] "v"(rs), [oo] "v"(oo),           \
+    [rstep] "s"(s_rstep), [nr] "s"(s_nr), [rm0] "s"(rm[0]), [rm1] "s"(rm[1]), [rm2] "s"(rm[2]), [rm3] "s"(rm[3]),         \
+    [l63] "s"(0x8000000000000000ull)
+#define ST_IN_ITEM(U) [vo##U] "v"(vo[U]), [xa##U] "v"(xa[U]), [pa##U] "v"(pa[U]), [first##U] "s"(first[U]), [keep##U] "s"(keep[U])
+#define ST_IN_ITEM_CT(U) [co##U] "v"(co[U]), [cm##U] "s"(cm[U])
+#define ST_CLOBBERS                                                                                                   \
+    "memory", "vcc", "scc", "v72", "v73", "v74", "v75", "v76", "v77", "v78", "v79", "v80", "v81", "v82", "v83", "v84", "v85",   \
+    "v86", "v87", "v88", "v89", "v90", "v91", "v92", "v93", "v94", "v95", "v96", "v97", "v98", "v99", "v100", "v101", "v102",   \
+    "v103", "v104", "v105", "v106", "v107", "v108", "v109", "v110", "v111", "v112", "v113", "v114", "v115", "v116", "v117",     \
+    "v118", "v119", "v120", "v121", "v122", "v123", "v124", "v125", "v126", "v127"
+
+template <int S, int MODE, int MAXI>
+__global__ __launch_bounds__(kStThreads) void matvec_steady_kernel(
+    const LoopLayer *__restrict__ layers, const uint32_t *__restrict__ codebook, int count, int arg_m, int arg_n,
+    int rows_per_block, int rw_tail, int items_tail, uint32_t full_magic)
+{
+    static_assert(MAXI == 3 || MAXI == 4, "a wave holds three or four elements of a layer");
+    extern __shared__ uint32_t lds[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t lane4 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds)) + lane * 4;   // the table is at LDS address 0
+    const int m = arg_m, n = arg_n;
+    const int T = n >> 11, Lt = (n & 2047) >> 6, npr = n >> 6, n8 = n >> 3;
+    const int items_full = rows_per_block >> 1;
+    const int row0 = blockIdx.x * rows_per_block;
+    const int rows = min(rows_per_block, m - row0);
+
+    // the table: rows 16 wave .. 16 wave + 15 are this wave's to write (a row is 64 copies of one value; bit 7 of the row
+    // number is the sign that replaces the first value's, inference.cu:259-262)
+    constexpr int kRowsPerWave = 256 / kStWaves;
+    {
+        uint32_t cbv[kRowsPerWave];
+#pragma unroll
+        for (int i = 0; i < kRowsPerWave; i++) cbv[i] = codebook[(kRowsPerWave * wave + i) & ((1 << S) - 1)];
+        const uint32_t table_sign = (uint32_t)((kRowsPerWave * wave) >> 7) << 15;
+#pragma unroll
+        for (int i = 0; i < kRowsPerWave; i++) lds[(kRowsPerWave * wave + i) * 64 + lane] = (cbv[i] & 0xFFFF7FFFu) | table_sign;
+    }
+
+    // ---- this wave's elements of a layer (the same in every layer): equal shares, the first total % 16 waves one more
+    const int total = T * items_full + items_tail;
+    const int per_wave = (int)((uint32_t)total / kStWaves), extra = (int)((uint32_t)total % kStWaves);
+    const int it_begin = wave * per_wave + min(wave, extra);
+    const int nitems = per_wave + (wave < extra ? 1 : 0);                // at most MAXI: the host checks
+    uint32_t vo[MAXI], xa[MAXI], pa[MAXI], co[MAXI], cm[MAXI];
+    uint64_t first[MAXI], keep[MAXI];
+    uint32_t rl = 0;
+    int prev_slab = -1;
+#pragma unroll
+    for (int u = 0; u < MAXI; u++) {
+        const int it = it_begin + u;
+        const bool mine = u < nitems;
+        int slab = items_full == 1 ? it : (int)__umulhi((uint32_t)it, full_magic);
+        slab = min(slab, T);
+        const int idx = it - slab * items_full;
+        const bool full = slab < T;
+        const int lanes = full ? 32 : Lt, rpi = full ? 2 : rw_tail;
+        const int row_first = idx * rpi;
+        const int rows_here = mine ? min(rpi, rows - row_first) : 0;          // <= 0: an element past the block's last row
+        const bool real = rows_here > 0;
+        // lane -> (row inside the item, element inside the row); lanes past the last whole row of a ragged item idle on element 0
+        int sub, l;
+        if (full) {
+            sub = lane >> 5, l = lane & 31;
+        } else {
+            sub = lane / max(lanes, 1), l = lane - sub * lanes;
+            if (sub >= rpi) l = 0;
+        }
+        const uint32_t elem0 = (uint32_t)(full ? slab : T) * (uint32_t)m * 32u;
+        const uint32_t elem = real ? elem0 + (uint32_t)(row0 + row_first) * (uint32_t)lanes : 0u;
+        const uint32_t last = real ? (uint32_t)(rows_here * lanes - 1) : 0u;
+        vo[u] = 16u * (elem + min((uint32_t)lane, last));
+        xa[u] = (uint32_t)kStTableBytes + 4u * (uint32_t)(1024 * slab + l);
+        pa[u] = (uint32_t)kStPartBase + 4u * (uint32_t)((row_first + sub) * npr + 32 * slab + l);
+        first[u] = __builtin_amdgcn_ballot_w64(l == 0);
+        const int nact = max(rows_here, 0) * lanes;
+        keep[u] = nact >= 64 ? ~0ull : (1ull << nact) - 1ull;
+        if (mine && slab != prev_slab) rl |= 1u << u;
+        if (mine) prev_slab = slab;
+        // continuous mode: the word in front of a row is the last word of the row's lane 31 in the slab before
+        const bool prev = real && slab > 0;
+        const int sub_c = min(sub, max(rows_here, 1) - 1);
+        co[u] = prev ? 4u * ((((uint32_t)(slab - 1) * (uint32_t)m + (uint32_t)(row0 + row_first + sub_c)) * 32u + 31u) * 4u + 3u) : 0u;
+        cm[u] = prev ? ~0u : 0u;
+    }
+
+    // ---- a thread's share of a layer's activations: 16 bytes at 8 idx (two of them), whose four words are the pairs of
+    // slots i * n8 + idx (inference.cu:215-221); where each goes in an image (the ragged slab at the full slabs' stride)
+    uint32_t xo[2], sa[8];
+    uint64_t stm[2];
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+        const int idx = tid + u * kStThreads;
+        xo[u] = 16u * (uint32_t)min(idx, n8 - 1);
+        stm[u] = __builtin_amdgcn_ballot_w64(idx < n8);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int P = i * n8 + min(idx, n8 - 1);
+            int pos = P;
+            if (P >= 1024 * T) {
+                const int r = P - 1024 * T, q = r / max(Lt, 1);
+                pos = 1024 * T + 32 * q + (r - q * Lt);
+            }
+            sa[4 * u + i] = (uint32_t)kStTableBytes + 4u * (uint32_t)pos;
+        }
+    }
+
+    // ---- the rows: wave w < 8 adds rows w, w + 8, ... of the block
+    const uint32_t rs = (uint32_t)kStPartBase + 4u * (uint32_t)(wave * npr + lane);
+    const uint32_t oo = 2u * (uint32_t)(row0 + wave);
+    const uint32_t rstep = 4u * (uint32_t)(kStRowWaves * npr);
+    const uint32_t nr = wave < kStRowWaves && wave < rows ? (uint32_t)(rows - wave + kStRowWaves - 1) / kStRowWaves : 0u;
+    uint64_t rm[4];
+#pragma unroll
+    for (int c = 0; c < 4; c++) rm[c] = __builtin_amdgcn_ballot_w64(lane + 64 * c < npr);
+
+    const uint64_t dc = reinterpret_cast<uint64_t>(&layers[0].comp), dx = reinterpret_cast<uint64_t>(&layers[0].x),
+                   dout = reinterpret_cast<uint64_t>(&layers[0].out);
+    __syncthreads();                                          // the table is complete
+
+    // what the block takes in scalar registers is wave-uniform by construction; say so, so that every one of them is
+    // in a scalar register whatever the compiler's divergence analysis makes of the code above
+    auto uni = [](uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)v); };
+    auto uni64 = [&](uint64_t v) { return (uint64_t)uni((uint32_t)v) | ((uint64_t)uni((uint32_t)(v >> 32)) << 32); };
+    rl = uni(rl);
+    const uint32_t s_nitems = uni((uint32_t)nitems), s_nr = uni(nr), s_rstep = uni(rstep), s_count = uni((uint32_t)count);
+#pragma unroll
+    for (int u = 0; u < MAXI; u++) first[u] = uni64(first[u]), keep[u] = uni64(keep[u]), cm[u] = uni(cm[u]);
+#pragma unroll
+    for (int c = 0; c < 4; c++) rm[c] = uni64(rm[c]);
+    stm[0] = uni64(stm[0]), stm[1] = uni64(stm[1]);
+
+    uint32_t a0, a1, a2, a3, cy, g0, g1, g2, g3, t0, t1, t2, t3, t4, t5, t6, t7, u0, u1, u2, u3, u4, u5, u6, u7, xb, k, kn, j;
+    uint64_t cn, xn, op;
+    if constexpr (MODE == RPTC_AS_WRITTEN && MAXI == 3) {
+        asm volatile(ST_BODY(0, 3, 4, 3)
+                     : ST_OUT_COMMON
+                     : ST_IN_COMMON, ST_IN_ITEM(0), ST_IN_ITEM(1), ST_IN_ITEM(2)
+                     : ST_CLOBBERS);
+    } else if constexpr (MODE == RPTC_AS_WRITTEN) {
+        asm volatile(ST_BODY(0, 4, 5, 4)
+                     : ST_OUT_COMMON
+                     : ST_IN_COMMON, ST_IN_ITEM(0), ST_IN_ITEM(1), ST_IN_ITEM(2), ST_IN_ITEM(3)
+                     : ST_CLOBBERS);
+    } else if constexpr (MAXI == 3) {
+        uint32_t own, cw0 = 0, cw1 = 0, cw2 = 0;
+        asm volatile(ST_BODY(1, 3, 6, 6)
+                     : ST_OUT_COMMON, [own] "=&v"(own), [cw0] "+v"(cw0), [cw1] "+v"(cw1), [cw2] "+v"(cw2)
+                     : ST_IN_COMMON, ST_IN_ITEM(0), ST_IN_ITEM(1), ST_IN_ITEM(2), ST_IN_ITEM_CT(0), ST_IN_ITEM_CT(1), ST_IN_ITEM_CT(2)
+                     : ST_CLOBBERS);
+    } else {
+        uint32_t own, cw0 = 0, cw1 = 0, cw2 = 0, cw3 = 0;
+        asm volatile(ST_BODY(1, 4, 8, 8)
+                     : ST_OUT_COMMON, [own] "=&v"(own), [cw0] "+v"(cw0), [cw1] "+v"(cw1), [cw2] "+v"(cw2), [cw3] "+v"(cw3)
+                     : ST_IN_COMMON, ST_IN_ITEM(0), ST_IN_ITEM(1), ST_IN_ITEM(2), ST_IN_ITEM(3), ST_IN_ITEM_CT(0), ST_IN_ITEM_CT(1),
+                       ST_IN_ITEM_CT(2), ST_IN_ITEM_CT(3)
+                     : ST_CLOBBERS);
+    }
+}
+
+template <typename F>
+static int st_set_lds_limit(F *kernel)
+{
+    return (int)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds);
+}
+
+int prepare_matvec_steady()
+{
+    int rc;
+#define RPTC_SET_LIMITS(MAXI)                                                                    \
+    if ((rc = st_set_lds_limit(matvec_steady_kernel<6, RPTC_AS_WRITTEN, MAXI>))) return rc;        \
+    if ((rc = st_set_lds_limit(matvec_steady_kernel<6, RPTC_CONTINUOUS, MAXI>))) return rc;        \
+    if ((rc = st_set_lds_limit(matvec_steady_kernel<8, RPTC_AS_WRITTEN, MAXI>))) return rc;        \
+    if ((rc = st_set_lds_limit(matvec_steady_kernel<8, RPTC_CONTINUOUS, MAXI>))) return rc;
+    RPTC_SET_LIMITS(3)
+    RPTC_SET_LIMITS(4)
+#undef RPTC_SET_LIMITS
+    return 0;
+}
+
+bool matvec_steady_fits(const LoopLayer &d)
+{
+    const int T = d.n >> 11, lt = (d.n & 2047) >> 6;
+    return (T + (lt ? 1 : 0)) * 4096 <= kStImageBytes && (int64_t)d.rows_per_block * (d.n / 64) * 4 <= kStPartBytes;
+}
+
+int matvec_steady_launch(const LoopLayer *device_layers, const LoopLayer &shape, const uint32_t *codebook, int count, int max_items,
+                         int grid, int S, int carry_mode, hipStream_t stream)
+{
+    if (max_items != 3 && max_items != 4) return RPTC_ESHAPE;
+#define RPTC_ST_GO(SS, MM, II)                                                                                              \
+    hipLaunchKernelGGL((matvec_steady_kernel<SS, MM, II>), dim3(grid), dim3(kStThreads), kStLdsBytes, stream, device_layers, \
+                       codebook, count, shape.m, shape.n, shape.rows_per_block, shape.rw_tail, shape.items_tail, shape.full_magic)
+#define RPTC_ST_PICK(SS, MM)                     \
+    do {                                         \
+        if (max_items == 3) RPTC_ST_GO(SS, MM, 3); \
+        else RPTC_ST_GO(SS, MM, 4);              \
+    } while (0)
+    if (S == 6 && carry_mode == RPTC_AS_WRITTEN) RPTC_ST_PICK(6, RPTC_AS_WRITTEN);
+    else if (S == 6) RPTC_ST_PICK(6, RPTC_CONTINUOUS);
+    else if (carry_mode == RPTC_AS_WRITTEN) RPTC_ST_PICK(8, RPTC_AS_WRITTEN);
+    else RPTC_ST_PICK(8, RPTC_CONTINUOUS);
+#undef RPTC_ST_PICK
+#undef RPTC_ST_GO
+    return (int)hipGetLastError();
+}
+
+}  // namespace rptc

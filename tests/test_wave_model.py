@@ -384,3 +384,64 @@ def test_sign_hadamard_kernel_matches_the_oracle(hadamard_isa, oracle, batch, n,
     want = oracle.sign_hadamard(x, signs, block, inverse=bool(inverse))
     err = np.abs(out.astype(np.float64) - want).max() / (np.abs(want).max() + 1e-9)
     assert err < 2e-3
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# matvec_steady_kernel: the chain of equal layers whose loop is one block of hand-written assembly (csrc/matvec_steady.hip)
+
+@pytest.fixture(scope="module")
+def steady_isa(tmp_path_factory):
+    return compile_to_assembly(tmp_path_factory, "matvec_steady")
+
+
+def run_steady(isa, oracle, m, n, count, S, mode, blocks, seed=7, burst=8, latency=(400, 60)):
+    rng = np.random.default_rng(seed)
+    mem = wave_model.Memory()
+    cb = (rng.standard_normal(2 << S) * 0.1).astype(np.float16)
+    cb_at = 0x7f5000003400
+    mem.add(cb_at, cb.view(np.uint8).copy(), "codebook")
+    layers, addresses = [], []
+    for i in range(count):
+        comp_at = 0x7f4100000000 + (i << 33) - (4096 if i % 3 == 1 else -0x23456700)
+        x_at, out_at = 0x7f3ffff0fe00 + (i << 16), 0x7f2ffffe0100 + (i << 15)
+        comp = rng.integers(0, 256, m * n // 4, dtype=np.uint8)
+        x = (rng.standard_normal(n) * 0.5).astype(np.float16).view(np.uint8).copy()
+        out = np.full(2 * m, 0xEE, dtype=np.uint8)
+        mem.add(comp_at, comp, f"stream {i}")
+        mem.add(x_at, x, f"activations {i}")
+        mem.add(out_at, out, f"output {i}")
+        layers.append((comp, x, out))
+        addresses.append((comp_at, x_at, out_at))
+    desc, _, part_floats, _, maxi = plan([(m, n)] * count, addresses)
+    assert part_floats * 4 <= 16384 and ((n >> 11) + (1 if n & 2047 else 0)) * 4096 <= 32768, "outside the steady kernel's layout"
+    desc_at = 0x7f6000001000
+    mem.add(desc_at, desc, "descriptors")
+    rpb = 2 * ((m + 2 * CUS - 1) // (2 * CUS))
+    lt = (n & 2047) >> 6
+    rw_tail = 64 // lt if lt else 1
+    items_tail = (rpb + rw_tail - 1) // rw_tail if lt else 0
+    items_full = rpb // 2
+    magic = ((1 << 32) // items_full + 1) if items_full > 1 else 0
+    kernel = wave_model.Kernel(isa, "_ZN4rptc20matvec_steady_kernelILi%dELi%dELi%dE" % (S, mode, maxi))
+    wave_model.Wave.vm_latency, wave_model.Wave.lgkm_latency = latency
+    kernel.launch(mem, (CUS,), 1024, [("ptr", desc_at), ("ptr", cb_at), ("i32", count), ("i32", m), ("i32", n), ("i32", rpb),
+                                      ("i32", rw_tail), ("i32", items_tail), ("u32", magic)],
+                  lds_bytes=160 * 1024, groups=[(b, 0, 0) for b in blocks], seed=seed, burst=burst)
+    for i, (comp, x, out) in enumerate(layers):
+        want = oracle.matvec(comp.view(np.uint32), cb, x.view(np.float16), m, S, mode=mode)
+        got = out.view(np.float16).astype(np.float64)
+        touched = np.zeros(m, dtype=bool)
+        for b in blocks:
+            r0, r1 = b * rpb, min(m, (b + 1) * rpb)
+            if r0 >= r1:
+                continue
+            touched[r0:r1] = True
+            err = np.abs(got[r0:r1] - want[r0:r1]).max() / (np.abs(want).max() + 1e-9)
+            assert err < 2e-3, f"layer {i} ({m}x{n}), workgroup {b}: rows {r0}..{r1 - 1} differ by {err:.3g} of the layer's largest output"
+        assert (out.view(np.uint16)[~touched] == 0xEEEE).all(), f"layer {i}: a row outside the simulated workgroups was written"
+
+
+@pytest.mark.parametrize("m,n,count,S,mode", [(33, 4096 + 768, 3, 8, 0), (33, 4096 + 768, 2, 8, 1), (300, 64, 4, 6, 0),
+                                              (7, 704, 1, 6, 1), (512, 6144, 2, 8, 1), (1024, 2048 + 64, 5, 8, 0)])
+def test_steady_kernel_matches_the_oracle(steady_isa, oracle, m, n, count, S, mode):
+    run_steady(steady_isa, oracle, m, n, count, S, mode, blocks=sorted({0, 1, (m - 1) // (2 * ((m + 2 * CUS - 1) // (2 * CUS)))}))

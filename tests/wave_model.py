@@ -63,8 +63,21 @@ class Memory:
 ASM_LINES = set()
 
 
+E32_ALIASES = {"v_add_f32", "v_add_u32", "v_mov_b32", "v_and_b32", "v_or_b32", "v_xor_b32", "v_cvt_f16_f32", "v_sub_u32",
+               "v_mul_f32", "v_lshlrev_b32", "v_lshrrev_b32"}
+
+
+def _arith(text):
+    """`3-1`, `1*128+14+1`, `0*16384+256`: constant expressions the assembler folds (hand-written blocks use them for
+    offsets that depend on a macro parameter).  Anything else is returned as it is."""
+    if re.fullmatch(r"[0-9a-fA-Fx+*() -]+", text) and re.search(r"[+*-]", text.lstrip("-")) and not re.fullmatch(r"-?(0x)?[0-9a-fA-F]+", text):
+        return str(eval(text, {"__builtins__": {}}, {}))
+    return text
+
+
 def parse(path):
     insts, labels = [], {}
+    local_defs = {}          # numeric local labels ("10:"): number -> instruction indices where it is defined
     in_asm = False
     for ln, raw in enumerate(open(path).read().split("\n"), 1):
         if "#ASMSTART" in raw:
@@ -79,10 +92,15 @@ def parse(path):
             continue
         m = re.match(r"^([.\w$]+):", t)
         if m:
-            labels[m.group(1)] = len(insts)
+            if m.group(1).isdigit():
+                local_defs.setdefault(m.group(1), []).append(len(insts))
+            else:
+                labels[m.group(1)] = len(insts)
             continue
         parts = t.split(None, 1)
         op = parts[0]
+        if op in E32_ALIASES:                # hand-written blocks name the 32-bit encodings without their suffix
+            op += "_e32"
         rest = parts[1] if len(parts) > 1 else ""
         # split operands from modifiers
         ops, mods = [], {}
@@ -93,14 +111,26 @@ def parse(path):
             sub = tk.split()
             if not sub:
                 continue
-            flat.append(sub[0])
+            flat.append(_arith(sub[0]))
             for s in sub[1:]:
                 if ":" in s:
                     k, v = s.split(":", 1)
-                    mods[k] = v
+                    mods[k] = _arith(v)
                 else:
                     mods[s] = True
         insts.append((op, flat, mods, ln, t))
+    # references to numeric local labels: "10b" is the nearest definition at or before the instruction, "10f" the nearest after
+    for i, (op, flat, mods, ln, t) in enumerate(insts):
+        if (op == "s_branch" or op.startswith("s_cbranch")) and flat and re.fullmatch(r"\d+[bf]", flat[0]):
+            num, way = flat[0][:-1], flat[0][-1]
+            defs = local_defs.get(num, [])
+            cands = [d for d in defs if d <= i] if way == "b" else [d for d in defs if d > i]
+            if not cands:
+                raise Fault(f"line {ln}: no local label for {flat[0]}")
+            target = max(cands) if way == "b" else min(cands)
+            name = f".Llocal_{num}_{target}"
+            labels[name] = target
+            insts[i] = (op, [name] + flat[1:], mods, ln, t)
     return insts, labels
 
 
@@ -557,6 +587,10 @@ class Wave:
             r = S(o[1]) + S(o[2]) + self.scc
             setscc(r >> 32)
             self.ws(o[0], r & 0xFFFFFFFF, 1)
+        elif op == "s_sub_u32":
+            a, b = S(o[1]), S(o[2])
+            setscc(b > a)                         # borrow
+            self.ws(o[0], (a - b) & 0xFFFFFFFF, 1)
         elif op == "s_sub_i32":
             a, b = S(o[1]), S(o[2])
             r = (a - b) & 0xFFFFFFFF
@@ -621,6 +655,14 @@ class Wave:
             r = (a >> off) & ((1 << wid) - 1) if wid else 0
             setscc(r != 0)
             self.ws(o[0], r, 1)
+        elif op == "s_bfe_i32":
+            a, b = S(o[1]), S(o[2])
+            off, wid = b & 31, (b >> 16) & 0x7F
+            r = (a >> off) & ((1 << wid) - 1) if wid else 0
+            if wid and r & (1 << (wid - 1)):
+                r |= 0xFFFFFFFF & ~((1 << wid) - 1)          # sign-extended
+            setscc(r != 0)
+            self.ws(o[0], r, 1)
         elif op in ("s_min_i32", "s_min_u32", "s_max_u32", "s_max_i32"):
             a, b = S(o[1]), S(o[2])
             if op.endswith("i32"):
@@ -678,6 +720,12 @@ class Wave:
             self.wv(o[0], V(o[1]))
         elif op in ("v_not_b32_e32", "v_not_b32_e64"):
             self.wv(o[0], (~V(o[1]).astype(np.uint64) & np.uint64(0xFFFFFFFF)).astype(U32))
+        elif op == "v_bfrev_b32_e32":
+            a = V(o[1]).astype(np.uint64)
+            r = np.zeros(64, dtype=np.uint64)
+            for bit in range(32):
+                r |= ((a >> np.uint64(bit)) & np.uint64(1)) << np.uint64(31 - bit)
+            self.wv(o[0], r.astype(U32))
         elif op == "v_mov_b32_dpp":
             src, valid = self.dpp_src(V(o[1]), mods, None)
             self.wv(o[0], src, self.lanes() & valid)
@@ -715,6 +763,9 @@ class Wave:
             self.wv(o[0], (r & 0xFFFFFFFF).astype(U32))
         elif op == "v_lshl_add_u32":
             r = (V(o[1]).astype(np.uint64) << (V(o[2]).astype(np.uint64) & 31)) + V(o[3]).astype(np.uint64)
+            self.wv(o[0], (r & 0xFFFFFFFF).astype(U32))
+        elif op == "v_add_lshl_u32":
+            r = (V(o[1]).astype(np.uint64) + V(o[2]).astype(np.uint64)) << (V(o[3]).astype(np.uint64) & 31)
             self.wv(o[0], (r & 0xFFFFFFFF).astype(U32))
         elif op == "v_lshl_add_u64":
             i, _ = self.vreg_index(o[1])
@@ -1202,6 +1253,8 @@ class Wave:
             r = ~S(o[1]) & 0xFFFFFFFF
             setscc(r != 0)
             self.ws(o[0], r, 1)
+        elif op == "s_brev_b32":
+            self.ws(o[0], int(format(S(o[1]) & 0xFFFFFFFF, "032b")[::-1], 2), 1)
         elif op == "s_movk_i32":
             v = int(o[1], 0)
             if v & 0x8000 and v > 0: v -= 0x10000
