@@ -28,10 +28,21 @@ for p in (ROOT, os.path.join(ROOT, "let-it-slide_amd")):
 
 HBM_PEAK_GBS = 8000.0
 
-# HBM bytes per launch (per layer for the chain) measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on
-# `bench.py --pmc-probe` (scaled by a copy kernel of known size; the runs are summarised under profiles/).
-# Keyed by (launch kind, m, n, S); other workloads report null.
-MEASURED_TRAFFIC_BYTES = {("launch", 4096, 11008, 8): 11529600, ("chain", 4096, 11008, 8): 11248000}
+
+
+def measured_traffic(kernel, m, n):
+    """HBM bytes per launch (per layer for a chain kernel) of `kernel` on an m x n layer, as measured with
+    `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` on `bench.py --pmc-probe` and written down in
+    profiles/<kernel>_<m>x<n>.md (lines `traffic_bytes = N` and `measured_at = <commit>`).  The figure is a property of the
+    kernel that file names at that commit, not of this run: (None, None) when there is no such summary."""
+    import re
+    path = os.path.join(ROOT, "profiles", f"{kernel}_{m}x{n}.md")
+    if not os.path.exists(path):
+        return None, None
+    text = open(path).read()
+    t = re.search(r"^traffic_bytes\s*=\s*([\d,]+)", text, flags=re.M)
+    c = re.search(r"^measured_at\s*=\s*(\w+)", text, flags=re.M)
+    return (int(t.group(1).replace(",", "")) if t else None), (c.group(1) if c else None)
 
 
 def parse():
@@ -96,9 +107,13 @@ def evict_caches():
 
 
 def aids_library():
-    """librptc_bench_aids.so: an empty launch and a read-only kernel (measurement aids, not the product)."""
-    path = os.path.join(ROOT, "let-it-slide_amd", "librptc_bench_aids.so")
+    """bench_aids/librptc_bench_aids.so: an empty launch, read-only kernels, instruction issue rates (measurement aids,
+    not the product)."""
+    path = os.path.join(ROOT, "bench_aids", "librptc_bench_aids.so")
     lib = ctypes.CDLL(path)
+    lib.rptc_probe_read_chain.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_void_p,
+                                          ctypes.c_void_p]
+    lib.rptc_probe_lds.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
     lib.rptc_probe_empty.argtypes = [ctypes.c_int, ctypes.c_void_p]
     lib.rptc_probe_read.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p]
     lib.rptc_probe_valu.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
@@ -230,27 +245,34 @@ class Runner:
         return err
 
 
-def cpu_baseline(runner, min_seconds=8.0):
-    """The oracle's fused decode + mat-vec (fp32 accumulate, threads over rows) on the same
-    layer, repeated until it has run for min_seconds."""
+def cpu_baseline(runner, min_seconds=8.0, also_seconds=4.0):
+    """The oracle's fused decode + mat-vec (fp32 accumulate, threads over rows) on the same layer, repeated until it has
+    run for min_seconds; and, under "also", the same on the 4096 x 4096 layer (the single-layer configuration the
+    reference's own CPU path would run) for also_seconds."""
     import numpy as np
     from oracle import rptc_oracle
-    comp = runner.weights[0].cpu().numpy().view(np.uint32)
-    cb = runner.codebook.cpu().numpy()
-    x = runner.x.cpu().numpy()
     threads = rptc_oracle.num_threads()
-    rptc_oracle.matvec_f32(comp, cb, x, runner.m, runner.S)           # warm the caches and the thread pool
-    reps, t0 = 0, time.perf_counter()
-    while True:
-        rptc_oracle.matvec_f32(comp, cb, x, runner.m, runner.S)
-        reps += 1
-        dt = time.perf_counter() - t0
-        if dt >= min_seconds and reps >= 3:
-            break
-    gbs = runner.bytes * reps / dt / 1e9
-    return {"value": round(gbs, 4), "unit": "GB/s", "cores": threads, "kind": "port",
-            "sample": f"{reps} full passes of the same {runner.m}x{runner.n} layer, {dt:.1f} s of CPU work",
-            "ms_per_pass": round(dt / reps * 1e3, 3)}
+
+    def timed(comp, cb, x, m, n, S, seconds):
+        rptc_oracle.matvec_f32(comp, cb, x, m, S)                     # warm the caches and the thread pool
+        reps, t0 = 0, time.perf_counter()
+        while True:
+            rptc_oracle.matvec_f32(comp, cb, x, m, S)
+            reps += 1
+            dt = time.perf_counter() - t0
+            if dt >= seconds and reps >= 3:
+                break
+        return {"value": round(m * n // 4 * reps / dt / 1e9, 4), "unit": "GB/s", "cores": threads, "kind": "port",
+                "sample": f"{reps} full passes of the same {m}x{n} layer, {dt:.1f} s of CPU work", "ms_per_pass": round(dt / reps * 1e3, 3)}
+
+    cb = runner.codebook.cpu().numpy()
+    out = timed(runner.weights[0].cpu().numpy().view(np.uint32), cb, runner.x.cpu().numpy(), runner.m, runner.n, runner.S, min_seconds)
+    if (runner.m, runner.n) != (4096, 4096) and also_seconds > 0:
+        rng = np.random.default_rng(42)
+        comp = rng.integers(0, 1 << 32, 4096 * 4096 // 16, dtype=np.uint64).astype(np.uint32)
+        x = rng.standard_normal(4096).astype(np.float16)
+        out["also"] = {"4096x4096": timed(comp, cb, x, 4096, 4096, runner.S, also_seconds)}
+    return out
 
 
 MFMA_F16_PEAK_TFLOPS = 2516.6
@@ -515,12 +537,28 @@ def bench_valu_probe(a):
             t = e0.elapsed_time(e1) * 1e6 / (n_el * (threads // 256))      # ns per element and SIMD
             best = t if best is None or t < best else best
         decode[f"{threads // 256} waves a SIMD"] = round(best, 2)
+    # LDS read instructions, sixteen waves of a compute unit issuing them back to back
+    lds = {}
+    for kind, name in enumerate(["ds_read_b32", "ds_read2st64_b32", "ds_read_b64", "ds_read_b128"]):
+        best = None
+        n_it = 2000
+        for rep in range(4):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            rc = aids.rptc_probe_lds(kind, n_it, cus, None, ctypes.c_void_p(stream))
+            assert rc == 0, rc
+            e1.record()
+            torch.cuda.synchronize()
+            t = e0.elapsed_time(e1) * 1e6 / (n_it * 8 * 16)            # ns per instruction and compute unit (16 waves)
+            best = t if best is None or t < best else best
+        lds[name] = round(best, 4)
     fma = res["v_fma_f32"]
     rel = {k: round(v / fma, 3) for k, v in res.items()}
     per_element = 12 * res["v_alignbit_b32"] + 16 * res["v_pk_mad_u16"] + 16 * res["v_perm_b32"] + 16 * res["v_and_or_b32"] + 32 * res["v_dot2c_f32_f16"]
     print(json.dumps({"metric": "vector instruction issue time, ns per instruction and SIMD", "unit": "ns", "n_gpus": 1,
                       "config": {"waves_per_simd": 4, "instructions_per_wave": iters * 32}, "results": res,
-                      "relative_to_v_fma_f32": rel, "decode_block_ns_per_element_and_simd": decode,
+                      "relative_to_v_fma_f32": rel, "lds_read_ns_per_instruction_and_cu": lds,
+                      "decode_block_ns_per_element_and_simd": decode,
                       "decode_block_us_per_4096x11008_layer": round(12 * decode["4 waves a SIMD"] / 1e3, 3),
                       "decode_valu_us_per_4096x11008_layer": round(12 * per_element / 1e3, 3)}))
 
@@ -750,13 +788,16 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4),
-            "traffic": MEASURED_TRAFFIC_BYTES.get(("chain" if a.launch == "chain" else "launch", a.m, a.n, a.S)),
+            "traffic": None,
             "launch_us": round(launch_ms * 1e3, 3),
         },
     }
+    kernel = "matvec_steady_kernel" if a.launch == "chain" else "matvec_kernel"
+    line["roofline"]["traffic"], line["roofline"]["traffic_measured_at"] = measured_traffic(kernel, a.m, a.n)
     if per_launch is not None:
-        line["roofline"]["kernel"] = "matvec_loop_kernel (the form rptc_decompress_matvec_chain takes for independent layers): achieved = steps x compressed bytes / the one launch's duration; launch_us is per layer"
-        per_launch["traffic"] = MEASURED_TRAFFIC_BYTES.get(("launch", a.m, a.n, a.S))
+        line["roofline"]["kernel"] = ("matvec_steady_kernel (the form rptc_decompress_matvec_chain takes for independent layers of one shape): "
+                                      "achieved = steps x compressed bytes / the one launch's duration; launch_us is per layer")
+        per_launch["traffic"], per_launch["traffic_measured_at"] = measured_traffic("matvec_kernel", a.m, a.n)
         line["per_launch"] = per_launch
     # the floor of this workload on this machine, in the same launch pattern (graph replay over the
     # same rotating buffers): an empty launch, and a kernel that only reads the stream
@@ -792,6 +833,27 @@ def main():
         if aids.rptc_probe_read(w.data_ptr(), runner.bytes, None, ctypes.c_void_p(cs)):
             raise RuntimeError("rptc_probe_read failed")
 
+    def chain_read_us():
+        """The chain's pattern with nothing decoded: one persistent launch that reads every layer's stream."""
+        cus = torch.cuda.get_device_properties(0).multi_processor_count
+        if runner.bytes % (16 * cus):
+            return None
+        ptrs = torch.tensor([w.data_ptr() for w in runner.weights], dtype=torch.int64, device="cuda")
+        cs = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        best = None
+        for rep in range(3):
+            evict_caches()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            rc = aids.rptc_probe_read_chain(ptrs.data_ptr(), len(runner.weights), a.steps, runner.bytes, cus, None, cs)
+            e1.record()
+            torch.cuda.synchronize()
+            if rc:
+                return None
+            us = e0.elapsed_time(e1) / a.steps * 1e3
+            best = us if rep > 0 and (best is None or us < best) else best
+        return best
+
     if a.launch in ("graph", "chain"):
         empty_us, read_us = floor_us(call_empty), floor_us(call_read)
         line["roofline"]["floor"] = {
@@ -800,6 +862,13 @@ def main():
             "read_only_GBps": round(runner.bytes / read_us / 1e3, 1),
             "note": "same bytes, same graph-replayed launch pattern: an empty kernel, and a kernel that only reads the stream",
         }
+        if a.launch == "chain":
+            cr = chain_read_us()
+            if cr is not None:
+                line["roofline"]["floor"]["chain_read_only_us"] = round(cr, 3)
+                line["roofline"]["floor"]["chain_read_only_GBps"] = round(runner.bytes / cr / 1e3, 1)
+                line["roofline"]["floor"]["chain_note"] = ("one persistent launch, one workgroup per compute unit, that only reads the same layers "
+                                                           "(a layer ahead, 1 KiB per wave request): the memory floor of the chain's pattern")
     if a.extra_shapes:
         extra = {}
         for (m, n) in ((4096, 4096), (11008, 4096), (8192, 8192), (28672, 8192), (8192, 28672)):

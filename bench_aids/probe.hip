@@ -1,12 +1,14 @@
 // Measurement aids (librptc_bench_aids.so): what the machine does with no decode at all, for the
 // same bytes and the same launch pattern as the mat-vec.  bench.py times them beside the kernel it
 // grades, so that the roofline figure can be read against the floor of this workload size: the time
-// of an empty launch, and the time of a kernel that only reads the stream.  A library of its own:
-// nothing here is part of the product path or of its header.
+// of an empty launch, the time of a kernel that only reads the stream (one launch per layer, and as
+// one persistent launch over all layers, the chain's pattern), and the issue rates of the vector and
+// LDS instructions the decode is made of.  A library of its own, built beside bench.py: nothing here
+// is part of the product path or of its header.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
-#include "../csrc/decode_asm.hpp"
+#include "../let-it-slide_amd/csrc/decode_asm.hpp"
 
 namespace {
 
@@ -106,6 +108,88 @@ __global__ void probe_decode_kernel(int iters, uint32_t seed, uint32_t *sink)
     if (__builtin_bit_cast(uint32_t, acc) == 0x9E3779B9u && sink) sink[0] = 1u;
 }
 
+// The chain's read pattern with nothing decoded: one 1024-thread workgroup per compute unit stays for all `layers`;
+// workgroup b reads its 1/grid share of every layer (16-byte non-temporal loads, a wave's request 1 KiB contiguous),
+// the next layer's requests issued before the current layer's data is used, as the chain kernels do.
+__global__ __launch_bounds__(1024) void probe_read_chain_kernel(const uint64_t *__restrict__ layer_ptrs, int copies, int layers,
+                                                                 int per_group16, uint32_t *sink)
+{
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    const int tid = threadIdx.x;
+    uint32_t acc = 0;
+    u32x4 v[kPerThread], nv[kPerThread];
+    auto issue = [&](int k, u32x4 (&dst)[kPerThread]) {
+        const u32x4 *base = reinterpret_cast<const u32x4 *>(layer_ptrs[k % copies]) + (size_t)blockIdx.x * per_group16;
+#pragma unroll
+        for (int u = 0; u < kPerThread; u++) {
+            const int i = tid + u * 1024;
+            dst[u] = __builtin_nontemporal_load(base + (i < per_group16 ? i : 0));      // a thread past the share repeats element 0
+        }
+    };
+    issue(0, v);
+    for (int k = 0; k < layers; k++) {
+        if (k + 1 < layers) issue(k + 1, nv);
+#pragma unroll
+        for (int u = 0; u < kPerThread; u++) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+#pragma unroll
+        for (int u = 0; u < kPerThread; u++) v[u] = nv[u];
+    }
+    if (acc == 0x9E3779B9u && sink) sink[0] = acc;
+}
+
+// LDS read instructions, sixteen waves of a workgroup issuing eight of a kind and waiting, `iters` times.
+// KIND 0: ds_read_b32, every lane its own column of a row (the decode's gather); 1: ds_read2st64_b32 (two dwords
+// 256 bytes apart: the reload of the activation registers in the chain kernel); 2: ds_read_b64; 3: ds_read_b128
+template <int KIND>
+__global__ __launch_bounds__(1024) void probe_lds_kernel(int iters, uint32_t seed, uint32_t *sink)
+{
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+    extern __shared__ uint32_t probe_lds[];
+    const int lane = threadIdx.x & 63;
+    for (int i = threadIdx.x; i < 16384; i += 1024) probe_lds[i] = (uint32_t)i * 64u;
+    __syncthreads();
+    const uint32_t base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(probe_lds));
+    const uint32_t addr = base + lane * (KIND == 2 ? 8 : KIND == 3 ? 16 : 4);
+    uint32_t acc = seed;
+    for (int it = 0; it < iters; it++) {
+        if (KIND == 0) {
+            uint32_t t0, t1, t2, t3, t4, t5, t6, t7;
+            asm volatile(
+                "ds_read_b32 %0, %8 offset:0\n ds_read_b32 %1, %8 offset:256\n ds_read_b32 %2, %8 offset:512\n"
+                "ds_read_b32 %3, %8 offset:768\n ds_read_b32 %4, %8 offset:1024\n ds_read_b32 %5, %8 offset:1280\n"
+                "ds_read_b32 %6, %8 offset:1536\n ds_read_b32 %7, %8 offset:1792\n s_waitcnt lgkmcnt(0)\n"
+                : "=&v"(t0), "=&v"(t1), "=&v"(t2), "=&v"(t3), "=&v"(t4), "=&v"(t5), "=&v"(t6), "=&v"(t7) : "v"(addr) : "memory");
+            acc ^= t0 ^ t1 ^ t2 ^ t3 ^ t4 ^ t5 ^ t6 ^ t7;
+        } else if (KIND == 1 || KIND == 2) {
+            u32x2 t0, t1, t2, t3, t4, t5, t6, t7;
+            if (KIND == 1)
+                asm volatile(
+                    "ds_read2st64_b32 %0, %8 offset0:0 offset1:1\n ds_read2st64_b32 %1, %8 offset0:2 offset1:3\n"
+                    "ds_read2st64_b32 %2, %8 offset0:4 offset1:5\n ds_read2st64_b32 %3, %8 offset0:6 offset1:7\n"
+                    "ds_read2st64_b32 %4, %8 offset0:8 offset1:9\n ds_read2st64_b32 %5, %8 offset0:10 offset1:11\n"
+                    "ds_read2st64_b32 %6, %8 offset0:12 offset1:13\n ds_read2st64_b32 %7, %8 offset0:14 offset1:15\n s_waitcnt lgkmcnt(0)\n"
+                    : "=&v"(t0), "=&v"(t1), "=&v"(t2), "=&v"(t3), "=&v"(t4), "=&v"(t5), "=&v"(t6), "=&v"(t7) : "v"(addr) : "memory");
+            else
+                asm volatile(
+                    "ds_read_b64 %0, %8 offset:0\n ds_read_b64 %1, %8 offset:512\n ds_read_b64 %2, %8 offset:1024\n"
+                    "ds_read_b64 %3, %8 offset:1536\n ds_read_b64 %4, %8 offset:2048\n ds_read_b64 %5, %8 offset:2560\n"
+                    "ds_read_b64 %6, %8 offset:3072\n ds_read_b64 %7, %8 offset:3584\n s_waitcnt lgkmcnt(0)\n"
+                    : "=&v"(t0), "=&v"(t1), "=&v"(t2), "=&v"(t3), "=&v"(t4), "=&v"(t5), "=&v"(t6), "=&v"(t7) : "v"(addr) : "memory");
+            acc ^= t0.x ^ t1.y ^ t2.x ^ t3.y ^ t4.x ^ t5.y ^ t6.x ^ t7.y;
+        } else {
+            u32x4 t0, t1, t2, t3, t4, t5, t6, t7;
+            asm volatile(
+                "ds_read_b128 %0, %8 offset:0\n ds_read_b128 %1, %8 offset:1024\n ds_read_b128 %2, %8 offset:2048\n"
+                "ds_read_b128 %3, %8 offset:3072\n ds_read_b128 %4, %8 offset:4096\n ds_read_b128 %5, %8 offset:5120\n"
+                "ds_read_b128 %6, %8 offset:6144\n ds_read_b128 %7, %8 offset:7168\n s_waitcnt lgkmcnt(0)\n"
+                : "=&v"(t0), "=&v"(t1), "=&v"(t2), "=&v"(t3), "=&v"(t4), "=&v"(t5), "=&v"(t6), "=&v"(t7) : "v"(addr) : "memory");
+            acc ^= t0.x ^ t1.y ^ t2.z ^ t3.w ^ t4.x ^ t5.y ^ t6.z ^ t7.w;
+        }
+    }
+    if (acc == 0x9E3779B9u && sink) sink[0] = acc;
+}
+
 }  // namespace
 
 // `iters` elements decoded by every wave of `workgroups` workgroups of `threads` threads (64..1024: 1 to 4 waves a SIMD)
@@ -166,5 +250,47 @@ extern "C" int rptc_probe_read(const void *data, int64_t bytes, void *sink, void
     if (grid >= ((size_t)1 << 31)) return -5;
     hipLaunchKernelGGL(probe_read_kernel, dim3((unsigned)grid), dim3(1024), 0, static_cast<hipStream_t>(stream),
                        static_cast<const uint32_t *>(data), static_cast<uint32_t *>(sink), total16);
+    return (int)hipGetLastError();
+}
+
+// `layers` layers of `layer_bytes` each (a multiple of 16 * workgroups; layer k is layer_ptrs[k % copies], device pointers
+// in device memory), read by `workgroups` resident workgroups in one launch; nothing is written
+extern "C" int rptc_probe_read_chain(const void *layer_ptrs, int copies, int layers, int64_t layer_bytes, int workgroups, void *sink,
+                                     void *stream)
+{
+    if (!layer_ptrs) return -1;
+    if (copies < 1 || layers < 1 || workgroups < 1 || layer_bytes < 16 || layer_bytes % (16 * (int64_t)workgroups) != 0) return -2;
+    const int64_t per_group16 = layer_bytes / 16 / workgroups;
+    if (per_group16 > 1024 * kPerThread) return -5;
+    hipLaunchKernelGGL(probe_read_chain_kernel, dim3(workgroups), dim3(1024), 0, static_cast<hipStream_t>(stream),
+                       static_cast<const uint64_t *>(layer_ptrs), copies, layers, (int)per_group16, static_cast<uint32_t *>(sink));
+    return (int)hipGetLastError();
+}
+
+// `iters` rounds of 8 LDS read instructions of one kind in every wave of `workgroups` 1024-thread workgroups;
+// kind: 0 ds_read_b32, 1 ds_read2st64_b32, 2 ds_read_b64, 3 ds_read_b128
+extern "C" int rptc_probe_lds(int kind, int iters, int workgroups, void *sink, void *stream)
+{
+    if (kind < 0 || kind > 3 || iters < 1 || workgroups < 1) return -2;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    uint32_t *out = static_cast<uint32_t *>(sink);
+    static bool allowed = false;
+    if (!allowed) {
+        int rc = 0;
+        rc = rc ? rc : (int)hipFuncSetAttribute(reinterpret_cast<const void *>(probe_lds_kernel<0>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        rc = rc ? rc : (int)hipFuncSetAttribute(reinterpret_cast<const void *>(probe_lds_kernel<1>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        rc = rc ? rc : (int)hipFuncSetAttribute(reinterpret_cast<const void *>(probe_lds_kernel<2>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        rc = rc ? rc : (int)hipFuncSetAttribute(reinterpret_cast<const void *>(probe_lds_kernel<3>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (rc) return rc;
+        allowed = true;
+    }
+#define RPTC_PROBE_GO(K) hipLaunchKernelGGL(probe_lds_kernel<K>, dim3(workgroups), dim3(1024), 100 * 1024, s, iters, 12345u, out)
+    switch (kind) {
+    case 0: RPTC_PROBE_GO(0); break;
+    case 1: RPTC_PROBE_GO(1); break;
+    case 2: RPTC_PROBE_GO(2); break;
+    default: RPTC_PROBE_GO(3); break;
+    }
+#undef RPTC_PROBE_GO
     return (int)hipGetLastError();
 }

@@ -1,8 +1,9 @@
 """Build the gfx950 libraries in-tree with hipcc.
 
 librptc_hip.so        the C-ABI library of kernels (include/rptc_hip.h), from csrc/*.hip
-librptc_bench_aids.so two measurement aids bench.py times beside the mat-vec (an empty launch, a
-                      kernel that only reads); kept out of the product library and its header
+../bench_aids/librptc_bench_aids.so
+                      measurement aids bench.py times beside the mat-vec (an empty launch, kernels that only read,
+                      instruction issue rates); beside bench.py, out of the product library, its header and its folder
 """
 import glob
 import os
@@ -16,7 +17,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "librptc_hip.so")
-AIDS_LIB = os.path.join(HERE, "librptc_bench_aids.so")
+AIDS_DIR = os.path.join(os.path.dirname(HERE), "bench_aids")
+AIDS_LIB = os.path.join(AIDS_DIR, "librptc_bench_aids.so")
 
 FLAGS = [
     "-O3", "-std=c++17", "--offload-arch=gfx950", "-fPIC",
@@ -90,7 +92,7 @@ def build(verbose=False, extra=()):
         with_asm = [s for s in srcs if re.search(r"\basm\b", open(s).read()) or "decode_asm.hpp" in open(s).read()]
         list(pool.map(lambda s: check_assembly(s, verbose, extra), with_asm))
     _run(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs], verbose)
-    _run(["hipcc", *FLAGS, *extra, "-shared", "-o", AIDS_LIB, os.path.join(HERE, "bench_aids", "probe.hip")], verbose)
+    _run(["hipcc", *FLAGS, *extra, "-shared", "-o", AIDS_LIB, os.path.join(AIDS_DIR, "probe.hip")], verbose)
     return LIB
 
 
