@@ -165,32 +165,44 @@ def dequantize_symbols(symbols, codebook, S=8, bits=2):
 
 
 def factorize(W, iterations=64):
-    """The reference's row/column factorisation W = b_out + b_in + s_out * s_in * N, transliterated from
-    quantize_hf.py:77-117 (jax.numpy -> torch, statement for statement, so that the iteration is the same):
-    64 rounds of alternately re-estimating the biases (means of the scaled residual) and the scales (RMS of
-    the residual), each followed by the balancing step that keeps the two biases' means and the two scales'
-    geometric means equal.  W float [out, in] on any device.  Returns (b_out [out, 1], b_in [1, in],
-    s_out [out, 1], s_in [1, in], N [out, in]); N has row and column RMS close to 1."""
+    """Row/column conditioning of a weight in front of the search: W = b_out + b_in + s_out * s_in * N with N close to
+    zero mean and unit RMS along every row and every column (the model the reference's quantizer fits,
+    quantize_hf.py:77-117, and reconstructs with at quantize_hf.py:167).
+
+    It is a fixed point of four conditions, imposed in turn (``iterations`` rounds, as many as the reference runs):
+      * every row of (W - b_out - b_in) / s_in sums to zero        -> b_out is the 1/s_in-weighted row mean of W - b_in
+      * every column of (W - b_out - b_in) / s_out sums to zero    -> b_in likewise, over rows, with weights 1/s_out
+      * every row of (W - b_out - b_in) / s_in has mean square s_out^2, every column of (W - b_out - b_in) / s_out
+        has mean square s_in^2
+    and two gauges that the model leaves free: a constant can move between b_out and b_in (fixed by giving them equal
+    means) and a factor between s_out and s_in (fixed by giving them equal geometric means).
+    W float [out, in] on any device.  Returns (b_out [out, 1], b_in [1, in], s_out [out, 1], s_in [1, in], N [out, in])."""
     W = torch.as_tensor(W).to(torch.float32)
-    out_features, in_features = W.shape
-    b_out = torch.zeros((out_features, 1), dtype=torch.float32, device=W.device)
-    b_in = torch.zeros((1, in_features), dtype=torch.float32, device=W.device)
-    s_out = torch.ones_like(b_out)
-    s_in = torch.ones_like(b_in)
+    rows, cols = W.shape
+    bias = [W.new_zeros((rows, 1)), W.new_zeros((1, cols))]          # [per row, per column]
+    scale = [W.new_ones((rows, 1)), W.new_ones((1, cols))]
+
+    def weighted_mean(A, w, dim):
+        # sum(A * w) / sum(w) along dim, w broadcast along the other axis
+        return (A * w).mean(dim=dim, keepdim=True) / w.mean()
+
+    def root_mean_square(A, dim):
+        return A.square().mean(dim=dim, keepdim=True).sqrt()
+
     for _ in range(iterations):
-        nb_out = ((W - b_in) / s_in).mean(dim=1, keepdim=True) / (1 / s_in).mean()
-        nb_in = ((W - nb_out) / s_out).mean(dim=0, keepdim=True) / (1 / s_out).mean()
-        balancer = (nb_in.mean() - nb_out.mean()) / 2
-        nb_out = nb_out + balancer
-        nb_in = nb_in - balancer
-        ns_out = (((W - nb_out - nb_in) / s_in) ** 2).mean(dim=1, keepdim=True).sqrt()
-        ns_in = (((W - nb_out - nb_in) / ns_out) ** 2).mean(dim=0, keepdim=True).sqrt()
-        balancer = torch.exp((ns_in.log().mean() - ns_out.log().mean()) / 2)
-        ns_out = ns_out * balancer
-        ns_in = ns_in / balancer
-        b_out, b_in, s_out, s_in = nb_out, nb_in, ns_out, ns_in
-    N = (W - b_out - b_in) / s_out / s_in
-    return b_out, b_in, s_out, s_in, N
+        # biases: rows against the current column side, then columns against the new rows; then the gauge
+        bias[0] = weighted_mean(W - bias[1], 1 / scale[1], dim=1)
+        bias[1] = weighted_mean(W - bias[0], 1 / scale[0], dim=0)
+        shift = (bias[1].mean() - bias[0].mean()) / 2
+        bias[0], bias[1] = bias[0] + shift, bias[1] - shift
+        # scales on the residual of the new biases, rows first; then the gauge
+        R = W - bias[0] - bias[1]
+        scale[0] = root_mean_square(R / scale[1], dim=1)
+        scale[1] = root_mean_square(R / scale[0], dim=0)
+        ratio = torch.exp((scale[1].log().mean() - scale[0].log().mean()) / 2)
+        scale[0], scale[1] = scale[0] * ratio, scale[1] / ratio
+    N = (W - bias[0] - bias[1]) / scale[0] / scale[1]
+    return bias[0], bias[1], scale[0], scale[1], N
 
 
 def quantile_alphabet(values, L=16, seed=0):
