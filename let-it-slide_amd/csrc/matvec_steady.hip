@@ -77,19 +77,10 @@ constexpr int kStRowWaves = 8;
 #define ST_STR(x) ST_STR2(x)
 
 // The 32 activation pairs of a lane for one slab: image P (0 / 1), XA = LDS address of the lane's slot 0 in image 0.
-// The wait covers the scalar loads made at the top of the layer as well (item 0 always reloads).
 #define ST_RD2(LO, HI, BASE, OFF, P)                                                                                  \
     "ds_read2st64_b32 v[" #LO ":" #HI "], " BASE " offset0:" #P "*128+" #OFF " offset1:" #P "*128+" #OFF "+1\n"
 // LDS reads complete in order and the decode block's first wait (at most 8 reads in flight, its own) comes before its
 // first product, which is the first instruction to read an activation register: the reload needs no wait of its own
-#ifdef ST_WAIT_AFTER_RELOAD
-#define ST_RELOAD_WAIT "s_waitcnt lgkmcnt(0)\n"
-#else
-#define ST_RELOAD_WAIT ""
-#endif
-#ifdef ST_NO_RELOAD
-#define ST_RELOAD(XA, P) "s_waitcnt lgkmcnt(0)\n"
-#else
 #define ST_RELOAD(XA, P)                                                                                              \
     "v_add_u32 %[xb], 0x80, " XA "\n"                                                                                 \
     ST_RD2(96, 97, XA, 0, P) ST_RD2(98, 99, XA, 2, P) ST_RD2(100, 101, XA, 4, P) ST_RD2(102, 103, XA, 6, P)           \
@@ -97,37 +88,20 @@ constexpr int kStRowWaves = 8;
     ST_RD2(112, 113, "%[xb]", 0, P) ST_RD2(114, 115, "%[xb]", 2, P) ST_RD2(116, 117, "%[xb]", 4, P)                   \
     ST_RD2(118, 119, "%[xb]", 6, P) ST_RD2(120, 121, "%[xb]", 8, P) ST_RD2(122, 123, "%[xb]", 10, P)                  \
     ST_RD2(124, 125, "%[xb]", 12, P) ST_RD2(126, 127, "%[xb]", 14, P)                                                 \
-    ST_RELOAD_WAIT
-#endif
+    ""
 
 // ---- the decode block (decode_asm.hpp's schedule with named registers): per 8 steps 4 v_alignbit_b32 (none for shift
 // 0), 4 v_pk_mad_u16 (two window hashes each), 8 address ops, 8 gathers, 8 products; the gathers of 8 steps are in flight
 // while the products of the 8 before are formed
-#if defined(ST_NO_GATHER)
-#define ST_RDPAIR(G, TH, TL)                                  \
-    "v_perm_b32 " TH ", " G ", %[lane4], %[sel]\n"            \
-    "v_and_or_b32 " TL ", " G ", %[mask], %[lane4]\n"
-#elif defined(ST_NO_VALU)
-#define ST_RDPAIR(G, TH, TL)                                  \
-    "ds_read_b32 " TH ", %[lane4]\n"                          \
-    "ds_read_b32 " TL ", %[lane4] offset:256\n"
-#else
 #define ST_RDPAIR(G, TH, TL)                                  \
     "v_perm_b32 " TH ", " G ", %[lane4], %[sel]\n"            \
     "v_and_or_b32 " TL ", " G ", %[mask], %[lane4]\n"         \
     "ds_read_b32 " TH ", " TH "\n"                            \
     "ds_read_b32 " TL ", " TL "\n"
-#endif
 #define ST_READS_A ST_RDPAIR("%[g0]", "%[t0]", "%[t1]") ST_RDPAIR("%[g1]", "%[t2]", "%[t3]") \
                    ST_RDPAIR("%[g2]", "%[t4]", "%[t5]") ST_RDPAIR("%[g3]", "%[t6]", "%[t7]")
 #define ST_READS_B ST_RDPAIR("%[g0]", "%[u0]", "%[u1]") ST_RDPAIR("%[g1]", "%[u2]", "%[u3]") \
                    ST_RDPAIR("%[g2]", "%[u4]", "%[u5]") ST_RDPAIR("%[g3]", "%[u6]", "%[u7]")
-#ifdef ST_NO_VALU
-#define ST_WINDOWS(SH, EX, EY, EZ, EW) ""
-#define ST_WINDOWS0(EX, EY, EZ, EW) ""
-#define ST_DOTS_FIRST(T, XA, XB, XC, XD, XE, XF, XG, XH) "v_mov_b32 %[a0], %[" T "0]\n v_mov_b32 %[a1], %[" T "1]\n v_mov_b32 %[a2], %[" T "2]\n v_mov_b32 %[a3], %[" T "7]\n"
-#define ST_DOTS(T, XA, XB, XC, XD, XE, XF, XG, XH) "v_mov_b32 %[a0], %[" T "7]\n"
-#else
 #define ST_WINDOWS(SH, EX, EY, EZ, EW)                        \
     "v_alignbit_b32 %[g0], %[cy], " EX ", " #SH "\n"          \
     "v_alignbit_b32 %[g1], " EX ", " EY ", " #SH "\n"         \
@@ -162,12 +136,8 @@ constexpr int kStRowWaves = 8;
     "v_dot2c_f32_f16 %[a1], %[" T "5], " XF "\n"              \
     "v_dot2c_f32_f16 %[a2], %[" T "6], " XG "\n"              \
     "v_dot2c_f32_f16 %[a3], %[" T "7], " XH "\n"
-#endif
 // OWN: what a row's first lane takes for the 16 bits in front of its element (its own last word as written,
 // inference.cu:232; the word in front of the row, or zero in slab 0, in continuous mode); FIRST: the lanes that start a row
-#ifdef ST_NO_DECODE
-#define ST_DECODE(EX, EY, EZ, EW, OWN, FIRST) "v_mov_b32 %[a0], " EX "\n v_mov_b32 %[a1], " EY "\n v_mov_b32 %[a2], " EZ "\n v_mov_b32 %[a3], " EW "\n"
-#else
 #define ST_DECODE(EX, EY, EZ, EW, OWN, FIRST)                                                                         \
     /* a DPP operand must not have been written by a vector op in the two instructions before */                     \
     "s_nop 1\n"                                                                                                       \
@@ -185,7 +155,6 @@ constexpr int kStRowWaves = 8;
     ST_DOTS("t", ST_X30, ST_X2, ST_X18, ST_X6, ST_X22, ST_X10, ST_X26, ST_X14)                                        \
     "s_waitcnt lgkmcnt(0)\n"                                                                                          \
     ST_DOTS("u", ST_X31, ST_X3, ST_X19, ST_X7, ST_X23, ST_X11, ST_X27, ST_X15)
-#endif
 
 // ---- one element of a layer.  U: which of the wave's elements; X, Y, Z, W / QUAD: its four registers; P: parity of
 // the layer; NEED: requests that may still be in flight when this element's has arrived.
@@ -216,27 +185,20 @@ constexpr int kStRowWaves = 8;
     "7" #U ":\n"                                                                                                      \
     REQUEST                                                                                                           \
     "8" #U ":\n"
-#ifdef ST_NO_STREAM
-#define ST_REQUEST_AW(U, QUAD) "s_nop 0\n"
-#else
 #define ST_REQUEST_AW(U, QUAD) "global_load_dwordx4 " QUAD ", %[vo" #U "], %[cn] nt\n"
-#endif
 #define ST_REQUEST_CT(U, QUAD) "global_load_dwordx4 " QUAD ", %[vo" #U "], %[cn] nt\n"                               \
                                "global_load_dword %[cw" #U "], %[co" #U "], %[cn]\n"
 // as written (MODE 0): a row's first lane takes its own last word; continuous (MODE 1): the word in front of the row
-#define ST_ITEM_0(U, X, Y, Z, W, QUAD, P, NEED)                                                                       \
-    ST_ITEM_HEAD(U, P, NEED) ST_DECODE(X, Y, Z, W, W, "%[first" #U "]") ST_ITEM_TAIL(U, P, ST_REQUEST_AW(U, QUAD))
-#define ST_ITEM_1(U, X, Y, Z, W, QUAD, P, NEED)                                                                       \
+#define ST_ITEM_0(U, X, Y, Z, W, P, NEED, REQUEST)                                                                    \
+    ST_ITEM_HEAD(U, P, NEED) ST_DECODE(X, Y, Z, W, W, "%[first" #U "]") ST_ITEM_TAIL(U, P, REQUEST)
+#define ST_ITEM_1(U, X, Y, Z, W, P, NEED, REQUEST)                                                                    \
     ST_ITEM_HEAD(U, P, NEED) "v_and_b32 %[own], %[cm" #U "], %[cw" #U "]\n"                                           \
-    ST_DECODE(X, Y, Z, W, "%[own]", "%[first" #U "]") ST_ITEM_TAIL(U, P, ST_REQUEST_CT(U, QUAD))
+    ST_DECODE(X, Y, Z, W, "%[own]", "%[first" #U "]") ST_ITEM_TAIL(U, P, REQUEST)
 
 // ---- the rows of the layer in front: a wave adds a row's n / 64 partial sums (lanes i, i + 64, i + 128, i + 192 in
 // that order, then across the lanes with DPP adds: rows of 16, row 0 into 1 and 2 into 3, rows 0-1 into 2-3), round
 // once to fp16 and lane 63 stores.  P: parity of the set that is read.
 #define ST_DPP_ADD(CTRL) "s_nop 1\n v_add_f32_dpp %[a0], %[a0], %[a0] " CTRL "\n"
-#ifdef ST_NO_ROWS
-#define ST_ROWS(P) ""
-#else
 #define ST_ROWS(P)                                                                                                    \
     "s_cmp_eq_u32 %[nr], 0\n"                                                                                         \
     "s_cbranch_scc1 92f\n"                                                                                            \
@@ -270,13 +232,9 @@ constexpr int kStRowWaves = 8;
     "s_cmp_lg_u32 %[j], 0\n"                                                                                          \
     "s_cbranch_scc1 91b\n"                                                                                            \
     "92:\n"
-#endif
 
 // ---- a thread's share of the next layer's activations into image P (halves 8 idx .. 8 idx + 7 go to the four planes,
 // inference.cu:215-221; the addresses were worked out in front of the loop)
-#ifdef ST_NO_STAGE
-#define ST_STAGE(P) ""
-#else
 #define ST_STAGE(P)                                                                                                   \
     "s_mov_b64 exec, %[stm0]\n"                                                                                       \
     "ds_write_b32 %[sa0], v72 offset:" #P "*32768\n ds_write_b32 %[sa1], v73 offset:" #P "*32768\n"                   \
@@ -285,12 +243,6 @@ constexpr int kStRowWaves = 8;
     "ds_write_b32 %[sa4], v76 offset:" #P "*32768\n ds_write_b32 %[sa5], v77 offset:" #P "*32768\n"                   \
     "ds_write_b32 %[sa6], v78 offset:" #P "*32768\n ds_write_b32 %[sa7], v79 offset:" #P "*32768\n"                   \
     "s_mov_b64 exec, -1\n"
-#endif
-#ifdef ST_NO_BARRIER
-#define ST_BARRIER ""
-#else
-#define ST_BARRIER "s_barrier\n"
-#endif
 
 // ---- the loop.  MODE: 0 as written, 1 continuous; LPI: requests per element (1; 2 continuous); M: elements a wave holds.
 // Requests in flight, oldest first, when element u's is waited for: u's own, the later elements' of this layer, the two
@@ -314,19 +266,19 @@ constexpr int kStRowWaves = 8;
 
 // The next layer's activations are staged behind the first element: their requests went out at the top of the layer,
 // and only the first element's next request has been made since (LPI requests may stay in flight).
-#ifdef ST_LATE_STAGE
-#define ST_EARLY_STAGE(Q, LPI) ""
-#define ST_END_STAGE(Q, STW) "s_waitcnt vmcnt(" #STW ")\n" ST_STAGE(Q)
-#else
 #define ST_EARLY_STAGE(Q, LPI) "s_waitcnt vmcnt(" #LPI ")\n" ST_STAGE(Q)
-#define ST_END_STAGE(Q, STW) ""
-#endif
 #define ST_ITEMS_3(MODE, P, Q, NEED, LPI)                                                                             \
-    ST_ITEM_##MODE(0, "v80", "v81", "v82", "v83", "v[80:83]", P, NEED)                                                \
+    ST_ITEM_##MODE(0, "v80", "v81", "v82", "v83", P, NEED, ST_REQUEST_##MODE(0, "v[80:83]"))                          \
     ST_EARLY_STAGE(Q, LPI)                                                                                            \
-    ST_ITEM_##MODE(1, "v84", "v85", "v86", "v87", "v[84:87]", P, NEED)                                                \
-    ST_ITEM_##MODE(2, "v88", "v89", "v90", "v91", "v[88:91]", P, NEED)
-#define ST_ITEMS_4(MODE, P, Q, NEED, LPI) ST_ITEMS_3(MODE, P, Q, NEED, LPI) ST_ITEM_##MODE(3, "v92", "v93", "v94", "v95", "v[92:95]", P, NEED)
+    ST_ITEM_##MODE(1, "v84", "v85", "v86", "v87", P, NEED, ST_REQUEST_##MODE(1, "v[84:87]"))                          \
+    ST_ITEM_##MODE(2, "v88", "v89", "v90", "v91", P, NEED, ST_REQUEST_##MODE(2, "v[88:91]"))
+#define ST_ITEMS_4(MODE, P, Q, NEED, LPI)                                                                             \
+    ST_ITEMS_3(MODE, P, Q, NEED, LPI) ST_ITEM_##MODE(3, "v92", "v93", "v94", "v95", P, NEED, ST_REQUEST_##MODE(3, "v[92:95]"))
+// the chain's last layer: nothing is requested any more, and everything requested has been waited for (vmcnt(63) waits for nothing)
+#define ST_LAST_ITEMS_3(MODE, P)                                                                                      \
+    ST_ITEM_##MODE(0, "v80", "v81", "v82", "v83", P, 63, "") ST_ITEM_##MODE(1, "v84", "v85", "v86", "v87", P, 63, "")  \
+    ST_ITEM_##MODE(2, "v88", "v89", "v90", "v91", P, 63, "")
+#define ST_LAST_ITEMS_4(MODE, P) ST_LAST_ITEMS_3(MODE, P) ST_ITEM_##MODE(3, "v92", "v93", "v94", "v95", P, 63, "")
 #define ST_REQUESTS_3(MODE) ST_REQUEST_##MODE(0, "v[80:83]") ST_REQUEST_##MODE(1, "v[84:87]") ST_REQUEST_##MODE(2, "v[88:91]")
 #define ST_REQUESTS_4(MODE) ST_REQUESTS_3(MODE) ST_REQUEST_##MODE(3, "v[92:95]")
 #define ST_REQUEST_0(U, QUAD) ST_REQUEST_AW(U, QUAD)
@@ -338,7 +290,6 @@ constexpr int kStRowWaves = 8;
     ST_XREQUESTS                                                                                                      \
     ST_ITEMS_##M(MODE, P, Q, NEED, LPI)                                                                               \
     "s_setprio 3\n"                                                                                                   \
-    ST_END_STAGE(Q, STW)                                                                                              \
     "s_cmp_eq_u32 %[k], 0\n"                                                                                          \
     "s_cbranch_scc1 93f\n"                                                                                            \
     ST_ROWS(Q)                                                                                                        \
@@ -346,9 +297,25 @@ constexpr int kStRowWaves = 8;
     "s_add_u32 %[k], %[k], 1\n"                                                                                       \
     ST_POINTERS                                                                                                       \
     "s_waitcnt lgkmcnt(0)\n"                                                                                          \
-    ST_BARRIER
+    "s_barrier\n"
 
-#define ST_BODY(MODE, M, NEED, STW, LPI)                                                                                   \
+// the last layer, of parity P: no requests (there is no layer behind it to ask for), the rows of the layer in front, then
+// its own rows behind one more barrier
+#define ST_LAST_LAYER(P, Q, MODE, M)                                                                                  \
+    "s_waitcnt vmcnt(0)\n"                                                                                            \
+    ST_LAST_ITEMS_##M(MODE, P)                                                                                        \
+    "s_setprio 3\n"                                                                                                   \
+    "s_cmp_eq_u32 %[k], 0\n"                                                                                          \
+    "s_cbranch_scc1 93f\n"                                                                                            \
+    ST_ROWS(Q)                                                                                                        \
+    "93:\n"                                                                                                           \
+    "s_add_u32 %[k], %[k], 1\n"                                                                                       \
+    ST_POINTERS                                                                                                       \
+    "s_waitcnt lgkmcnt(0)\n"                                                                                          \
+    "s_barrier\n"                                                                                                     \
+    ST_ROWS(P)
+
+#define ST_BODY(MODE, M, NEED, STW, LPI)                                                                              \
     "s_mov_b32 %[k], 0\n"                                                                                             \
     "s_mov_b32 %[kn], 0\n"                                                                                            \
     "s_load_dwordx2 %[cn], %[dc], %[kn]\n"                                                                            \
@@ -361,18 +328,21 @@ constexpr int kStRowWaves = 8;
     ST_POINTERS                                                                                                       \
     "s_waitcnt lgkmcnt(0)\n"                                                                                          \
     "s_barrier\n"                                                                                                     \
-    "10:\n"                                                                                                           \
-    ST_LAYER(0, 1, MODE, M, NEED, STW, LPI)                                                                                \
-    "s_cmp_ge_u32 %[k], %[count]\n"                                                                                   \
+    /* layers 0 .. count - 2 ask for the layer behind them while they decode; the last one (k == last) does not */    \
+    "s_cmp_eq_u32 %[k], %[last]\n"                                                                                    \
     "s_cbranch_scc1 11f\n"                                                                                            \
-    ST_LAYER(1, 0, MODE, M, NEED, STW, LPI)                                                                                \
-    "s_cmp_lt_u32 %[k], %[count]\n"                                                                                   \
+    "10:\n"                                                                                                           \
+    ST_LAYER(0, 1, MODE, M, NEED, STW, LPI)                                                                           \
+    "s_cmp_eq_u32 %[k], %[last]\n"                                                                                    \
+    "s_cbranch_scc1 13f\n"                                                                                            \
+    ST_LAYER(1, 0, MODE, M, NEED, STW, LPI)                                                                           \
+    "s_cmp_lg_u32 %[k], %[last]\n"                                                                                    \
     "s_cbranch_scc1 10b\n"                                                                                            \
-    /* the last layer's rows: its partial sums are in set 1 (an even number of layers) or set 0 */                    \
-    ST_ROWS(1)                                                                                                        \
-    "s_branch 12f\n"                                                                                                  \
     "11:\n"                                                                                                           \
-    ST_ROWS(0)                                                                                                        \
+    ST_LAST_LAYER(0, 1, MODE, M)                                                                                      \
+    "s_branch 12f\n"                                                                                                  \
+    "13:\n"                                                                                                           \
+    ST_LAST_LAYER(1, 0, MODE, M)                                                                                      \
     "12:\n"                                                                                                           \
     "s_waitcnt vmcnt(0)\n"
 
@@ -496,11 +466,7 @@ __global__ __launch_bounds__(kStThreads) void matvec_steady_kernel(
 
     // ---- the rows: added up by the waves that hold the fewest elements (all sixteen when the shares are equal), the
     // i-th of them taking rows i, i + their number, ...
-#ifdef ST_OLD_ROWS
-    const int first_row_wave = 0, row_waves = kStRowWaves;
-#else
     const int first_row_wave = extra, row_waves = kStWaves - extra;
-#endif
     const int ri = wave - first_row_wave;
     const uint32_t rs = (uint32_t)kStPartBase + 4u * (uint32_t)(max(ri, 0) * npr + lane);
     const uint32_t oo = 2u * (uint32_t)(row0 + max(ri, 0));
