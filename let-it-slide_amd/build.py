@@ -70,14 +70,59 @@ def asm_blocks_left_waiting(assembly):
     return bad
 
 
+def handoff_violations(assembly):
+    """The hand-off of partial results between workgroups (`publishing()` .. `published()`, `arrive()`, `merging()` ..
+    `merged()` in csrc/rptc_common.hpp) replaces release / acquire fences by three properties of the emitted code, checked
+    here on the markers those functions leave in the assembly: every global store of a publishing region and every global
+    load of a merging region is an sc1 one (written through to / read from the level all XCDs share); `published()`'s
+    `s_waitcnt vmcnt(0)` is there; and a workgroup barrier stands between it and the arrival's atomic add.
+    Returns [(line number, text, what is wrong)] (empty = good)."""
+    bad = []
+    state = None                  # None, "publishing", "waiting" (published, barrier not yet seen), "merging"
+    lines = assembly.split("\n")
+    for no, line in enumerate(lines, 1):
+        t = line.strip()
+        if t.startswith("; rptc-handoff: publishing"):
+            state = "publishing"
+        elif t.startswith("; rptc-handoff: published"):
+            nxt = next((x.strip() for x in lines[no:no + 3] if x.strip() and not x.strip().startswith(";")), "")
+            if not (nxt.startswith("s_waitcnt") and "vmcnt(0)" in nxt):
+                bad.append((no, t, "no s_waitcnt vmcnt(0) behind published()"))
+            state = "waiting"
+        elif t.startswith("; rptc-handoff: merging"):
+            state = "merging"
+        elif t.startswith("; rptc-handoff: merged"):
+            state = None
+        elif t.startswith(".Lfunc_end"):
+            state = None
+        elif state == "publishing" and re.match(r"(global|flat|buffer)_store", t) and " sc1" not in t:
+            bad.append((no, t, "a store of a publishing region without sc1"))
+        elif state == "merging" and re.match(r"(global|flat|buffer)_load", t) and " sc1" not in t:
+            bad.append((no, t, "a load of a merging region without sc1"))
+        elif state == "waiting":
+            if t.startswith("s_barrier"):
+                state = None
+            elif re.match(r"(global|flat|buffer)_atomic", t):
+                bad.append((no, t, "the arrival is counted without a barrier behind published()"))
+                state = None
+    return bad
+
+
 def check_assembly(src, verbose=False, extra=()):
-    """Compiles `src` to assembly with the library's flags and applies `asm_blocks_left_waiting`; raises on a hit."""
+    """Compiles `src` to assembly with the library's flags and applies `asm_blocks_left_waiting` and
+    `handoff_violations`; raises on a hit."""
     with tempfile.TemporaryDirectory() as tmp:
         out = os.path.join(tmp, os.path.basename(src) + ".s")
         _run(["hipcc", *FLAGS, *extra, "--cuda-device-only", "-S", src, "-o", out], verbose)
-        bad = asm_blocks_left_waiting(open(out).read())
+        text = open(out).read()
+    bad = asm_blocks_left_waiting(text)
     if bad:
         raise RuntimeError(f"{os.path.basename(src)}: an inline-assembly block ends with requests in flight: {bad[:3]}")
+    bad = handoff_violations(text)
+    if bad:
+        raise RuntimeError(f"{os.path.basename(src)}: the hand-off between workgroups is not what rptc_common.hpp says: {bad[:3]}")
+    if "arrive(" in open(src).read() and "rptc-handoff: published" not in text:
+        raise RuntimeError(f"{os.path.basename(src)}: arrive() without the markers of a hand-off in the assembly")
 
 
 def build(verbose=False, extra=()):

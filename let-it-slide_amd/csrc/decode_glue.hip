@@ -341,6 +341,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(
 
     // publish the piece, count the arrival, and let the last workgroup of the head merge
     float *mine = parts + (size_t)blockIdx.x * kAttnPartStride;
+    publishing();
     if (tid < hd) __hip_atomic_store(&mine[tid], y, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     if (tid == 0) {
         __hip_atomic_store(&mine[256], mx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -361,6 +362,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(
     const float *head_parts = parts + (size_t)h * splits * kAttnPartStride;
     constexpr int kMaxSplits = 16;
     float pm[kMaxSplits], pl[kMaxSplits], pa[kMaxSplits];
+    merging();
 #pragma unroll
     for (int i = 0; i < kMaxSplits; i++) {
         pm[i] = -INFINITY;
@@ -372,6 +374,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(
             pa[i] = __hip_atomic_load(&pp[tid], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
+    merged();
     float M = pm[0];                             // piece 0 is never empty
 #pragma unroll
     for (int i = 1; i < kMaxSplits; i++) M = fmaxf(M, pm[i]);

@@ -299,6 +299,7 @@ __global__ __launch_bounds__(kMmThreads) __attribute__((amdgpu_waves_per_eu(4, 4
             for (int w = 0; w < waves_used; w++) y += buf[(w * PLANES + p) * 256 + vl];
             // device-coherent store (written through the XCD's L2): visible to the workgroup on
             // another XCD that adds the slabs, without flushing a whole cache
+            publishing();
             __hip_atomic_store(&my_partial[rb * (PLANES * 256) + tid], y, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
         if (kPartBuffers == 1) __syncthreads();                   // the one buffer is free again
@@ -326,6 +327,7 @@ __global__ __launch_bounds__(kMmThreads) __attribute__((amdgpu_waves_per_eu(4, 4
     for (int k = 0; k < kPerThread; k++) y[k] = 0.f;
     for (int sl0 = 0; sl0 < slabs; sl0 += 4) {
         float v[kPerThread][4];
+        merging();
 #pragma unroll
         for (int k = 0; k < kPerThread; k++)
 #pragma unroll
@@ -336,6 +338,7 @@ __global__ __launch_bounds__(kMmThreads) __attribute__((amdgpu_waves_per_eu(4, 4
                     v[k][u] = __hip_atomic_load(&grp_partial[(size_t)(sl0 + u) * tile_stride + t], __ATOMIC_RELAXED,
                                                 __HIP_MEMORY_SCOPE_AGENT);
             }
+        merged();
 #pragma unroll
         for (int k = 0; k < kPerThread; k++)
 #pragma unroll

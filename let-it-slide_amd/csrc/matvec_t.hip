@@ -162,6 +162,7 @@ __global__ __launch_bounds__(kTThreads) void matvec_t_kernel(
         return;
     }
     // (the hand-off between workgroups: see published() / arrive() in rptc_common.hpp)
+    publishing();
     if (tid < kWave) __hip_atomic_store(&parts[(size_t)blockIdx.x * kWave + tid], y, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     published();
     __syncthreads();
@@ -175,11 +176,13 @@ __global__ __launch_bounds__(kTThreads) void matvec_t_kernel(
     __syncthreads();
     if (!*flag || tid >= kWave || !valid) return;
     float p[kTMaxSplit];
+    merging();
 #pragma unroll
     for (int i = 0; i < kTMaxSplit; i++)
         p[i] = i < ksplit ? __hip_atomic_load(&parts[((size_t)rb * ksplit + i) * kWave + tid], __ATOMIC_RELAXED,
                                               __HIP_MEMORY_SCOPE_AGENT)
                           : 0.f;
+    merged();
     float total = 0.f;
 #pragma unroll
     for (int i = 0; i < kTMaxSplit; i++) total += p[i];

@@ -135,7 +135,7 @@ __device__ __forceinline__ float half_wave_sum(float v)
 }
 
 // Hand-off of partial results between workgroups (which may run on different XCDs, each with an L2 of its own).
-// The producing threads write their results with agent-scope stores (`__hip_atomic_store(..., __ATOMIC_RELAXED,
+// Between publishing() and published() the producing threads write their results with agent-scope stores (`__hip_atomic_store(..., __ATOMIC_RELAXED,
 // __HIP_MEMORY_SCOPE_AGENT)`: global_store ... sc1, written through to the level all XCDs share), then call
 // published() and meet at a workgroup barrier; one thread then counts the arrival with arrive().  The workgroup
 // that sees the last arrival reads the others' results with agent-scope loads (global_load ... sc1, which do not
@@ -150,7 +150,14 @@ __device__ __forceinline__ float half_wave_sum(float v)
 // buffer_inv sc1), which nothing here needs (no plain store is part of the hand-off) and which costs 15-25 us per
 // launch, measured on the transposed mat-vec (4096 x 4096: 27 us with the fences, 8 us without) and on the batched
 // product (batch 16 on 4096 x 11008: 67 us against 15 us).
-__device__ __forceinline__ void published() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+// The three markers are assembler comments: build.py reads them back from the emitted assembly and fails the build when
+// a store between publishing() and published() or a load between merging() and merged() is not an sc1 one, or when
+// the wait of published() is not followed by a barrier before the arrival is counted (`handoff_violations`).  Their
+// "memory" clobbers keep the compiler from moving a store or load across them.
+__device__ __forceinline__ void publishing() { asm volatile("; rptc-handoff: publishing" ::: "memory"); }
+__device__ __forceinline__ void published() { asm volatile("; rptc-handoff: published\n\ts_waitcnt vmcnt(0)" ::: "memory"); }
+__device__ __forceinline__ void merging() { asm volatile("; rptc-handoff: merging" ::: "memory"); }
+__device__ __forceinline__ void merged() { asm volatile("; rptc-handoff: merged" ::: "memory"); }
 __device__ __forceinline__ uint32_t arrive(uint32_t *counter)
 {
     return __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

@@ -63,3 +63,32 @@ def test_the_checker_sees_a_block_that_ends_with_reads_in_flight():
 	;;#ASMEND
 """
     assert [t for _, t in check(partial)] == ["ds_read_b32 v51, v14 offset:128"]
+
+
+@pytest.mark.skipif(shutil.which("hipcc") is None, reason="needs hipcc")
+@pytest.mark.parametrize("source", ["matvec_t.hip", "decode_glue.hip"])
+def test_handoffs_between_workgroups_are_what_the_source_says(source):
+    """Partial results that one workgroup writes and another adds up (csrc/rptc_common.hpp: publishing / published /
+    arrive / merging / merged): sc1 stores, the wait, a barrier in front of the arrival's atomic, sc1 loads."""
+    _build_module().check_assembly(os.path.join(PKG, "csrc", source))
+
+
+def test_the_handoff_checker_sees_a_plain_store_a_plain_load_and_a_missing_barrier():
+    check = _build_module().handoff_violations
+    good = """
+	; rptc-handoff: publishing
+	global_store_dword v2, v4, s[6:7] sc1
+	; rptc-handoff: published
+	s_waitcnt vmcnt(0)
+	s_barrier
+	global_atomic_add v1, v1, v3, s[6:7] sc0
+	; rptc-handoff: merging
+	global_load_dword v2, v[6:7], off sc1
+	; rptc-handoff: merged
+	global_load_dword v9, v[6:7], off
+"""
+    assert check(good) == []
+    assert [w for _, _, w in check(good.replace("v4, s[6:7] sc1", "v4, s[6:7]"))] == ["a store of a publishing region without sc1"]
+    assert [w for _, _, w in check(good.replace("off sc1", "off"))] == ["a load of a merging region without sc1"]
+    assert [w for _, _, w in check(good.replace("\ts_barrier\n", ""))] == ["the arrival is counted without a barrier behind published()"]
+    assert [w for _, _, w in check(good.replace("\ts_waitcnt vmcnt(0)\n", ""))] == ["no s_waitcnt vmcnt(0) behind published()"]
