@@ -40,6 +40,7 @@ constexpr int kStRowWaves = 8;
 // stream elements of a wave: item u in v[80 + 4u : 83 + 4u]; next activations: v[72:75], v[76:79]
 // activation pairs of the slab being decoded: slot q in v(96 + q / 2) for even q, v(112 + (q - 1) / 2) for odd q, so
 // that slots q and q + 2 are neighbours and one ds_read2st64_b32 (two dwords 256 bytes apart) fills both
+#ifndef ST_MFMA
 #define ST_X0 "v96"
 #define ST_X2 "v97"
 #define ST_X4 "v98"
@@ -73,10 +74,16 @@ constexpr int kStRowWaves = 8;
 #define ST_X29 "v126"
 #define ST_X31 "v127"
 
+#else
+// With the products on the matrix unit (ST_MFMA) an operand is a PAIR of registers: the two windows of one window register
+// (slots hi, lo) sit side by side, pair 4 j + i in v[96 + 8 j + 2 i : +1] for shift group j and window register i
+#define ST_XP(J, I) "v[96+8*" #J "+2*" #I ":96+8*" #J "+2*" #I "+1]"
+#endif
 #define ST_STR2(x) #x
 #define ST_STR(x) ST_STR2(x)
 
 // The 32 activation pairs of a lane for one slab: image P (0 / 1), XA = LDS address of the lane's slot 0 in image 0.
+#ifndef ST_MFMA
 #define ST_RD2(LO, HI, BASE, OFF, P)                                                                                  \
     "ds_read2st64_b32 v[" #LO ":" #HI "], " BASE " offset0:" #P "*128+" #OFF " offset1:" #P "*128+" #OFF "+1\n"
 // LDS reads complete in order and the decode block's first wait (at most 8 reads in flight, its own) comes before its
@@ -90,9 +97,23 @@ constexpr int kStRowWaves = 8;
     ST_RD2(124, 125, "%[xb]", 12, P) ST_RD2(126, 127, "%[xb]", 14, P)                                                 \
     ""
 
+#else
+// pair (slot hi, slot lo) of a window register: both slots have the shift group's parity, so both are whole
+// 256-byte units away from the base of that parity (XA for even slots, XA + 128 for odd ones)
+#define ST_RDP(J, I, BASE, OHI, OLO, P)                                                                               \
+    "ds_read2st64_b32 " ST_XP(J, I) ", " BASE " offset0:" #P "*128+" #OHI " offset1:" #P "*128+" #OLO "\n"
+#define ST_RELOAD(XA, P)                                                                                              \
+    "v_add_u32 %[xb], 0x80, " XA "\n"                                                                                 \
+    ST_RDP(0, 0, XA, 14, 0, P) ST_RDP(0, 1, XA, 8, 2, P) ST_RDP(0, 2, XA, 10, 4, P) ST_RDP(0, 3, XA, 12, 6, P)        \
+    ST_RDP(1, 0, "%[xb]", 14, 0, P) ST_RDP(1, 1, "%[xb]", 8, 2, P) ST_RDP(1, 2, "%[xb]", 10, 4, P) ST_RDP(1, 3, "%[xb]", 12, 6, P) \
+    ST_RDP(2, 0, XA, 15, 1, P) ST_RDP(2, 1, XA, 9, 3, P) ST_RDP(2, 2, XA, 11, 5, P) ST_RDP(2, 3, XA, 13, 7, P)        \
+    ST_RDP(3, 0, "%[xb]", 15, 1, P) ST_RDP(3, 1, "%[xb]", 9, 3, P) ST_RDP(3, 2, "%[xb]", 11, 5, P) ST_RDP(3, 3, "%[xb]", 13, 7, P)
+
+#endif
 // ---- the decode block (decode_asm.hpp's schedule with named registers): per 8 steps 4 v_alignbit_b32 (none for shift
 // 0), 4 v_pk_mad_u16 (two window hashes each), 8 address ops, 8 gathers, 8 products; the gathers of 8 steps are in flight
 // while the products of the 8 before are formed
+#ifndef ST_MFMA
 #define ST_RDPAIR(G, TH, TL)                                  \
     "v_perm_b32 " TH ", " G ", %[lane4], %[sel]\n"            \
     "v_and_or_b32 " TL ", " G ", %[mask], %[lane4]\n"         \
@@ -156,6 +177,72 @@ constexpr int kStRowWaves = 8;
     "s_waitcnt lgkmcnt(0)\n"                                                                                          \
     ST_DOTS("u", ST_X31, ST_X3, ST_X19, ST_X7, ST_X23, ST_X11, ST_X27, ST_X15)
 
+#else
+// The products on the matrix unit: v_mfma_f32_4x4x4_16b_f16 multiplies, in every group of four lanes, the 4 x 4 matrix
+// whose row i is lane i's A operand (four halves: the two gathered pairs of one window register) by the one whose
+// column j is lane j's B operand (the activation pairs of the same two slots), so the diagonal of the result, element
+// (i, i), in register i of lane i, is lane i's own four products added to what was there.  Sixteen of them replace the
+// element's 32 two-term dot products, run beside the vector ALU, and cost it one issue slot each.  The gathered pairs
+// land in fixed register pairs (v[56:63], v[64:71]: a matrix operand is an aligned pair), the sum in v[52:55].
+// Distances the hardware does not interlock: two instructions between a matrix instruction and the next one that
+// accumulates into its result; five before anything else reads the result.
+#define ST_RDPAIR(G, TH, TL)                                  \
+    "v_perm_b32 " TH ", " G ", %[lane4], %[sel]\n"            \
+    "v_and_or_b32 " TL ", " G ", %[mask], %[lane4]\n"         \
+    "ds_read_b32 " TH ", " TH "\n"                            \
+    "ds_read_b32 " TL ", " TL "\n"
+#define ST_READS_A ST_RDPAIR("%[g0]", "v56", "v57") ST_RDPAIR("%[g1]", "v58", "v59") \
+                   ST_RDPAIR("%[g2]", "v60", "v61") ST_RDPAIR("%[g3]", "v62", "v63")
+#define ST_READS_B ST_RDPAIR("%[g0]", "v64", "v65") ST_RDPAIR("%[g1]", "v66", "v67") \
+                   ST_RDPAIR("%[g2]", "v68", "v69") ST_RDPAIR("%[g3]", "v70", "v71")
+#define ST_MM(A, J, I, C) "v_mfma_f32_4x4x4_16b_f16 v[52:55], " A ", " ST_XP(J, I) ", " C "\n"
+#define ST_DECODE(EX, EY, EZ, EW, OWN, FIRST)                                                                         \
+    /* a DPP operand must not have been written by a vector op in the two instructions before */                     \
+    "s_nop 1\n"                                                                                                       \
+    "s_mov_b64 vcc, " FIRST "\n"                                                                                      \
+    "v_cndmask_b32_dpp %[cy], " EW ", " OWN ", vcc wave_shr:1 row_mask:0xf bank_mask:0xf bound_ctrl:1\n"              \
+    /* shift 12 */                                                                                                    \
+    "v_alignbit_b32 %[g0], %[cy], " EX ", 12\n v_alignbit_b32 %[g1], " EX ", " EY ", 12\n"                            \
+    "v_alignbit_b32 %[g2], " EY ", " EZ ", 12\n v_alignbit_b32 %[g3], " EZ ", " EW ", 12\n"                           \
+    "v_pk_mad_u16 %[g0], %[g0], %[g0], %[g0]\n v_pk_mad_u16 %[g1], %[g1], %[g1], %[g1]\n"                             \
+    "v_pk_mad_u16 %[g2], %[g2], %[g2], %[g2]\n v_pk_mad_u16 %[g3], %[g3], %[g3], %[g3]\n"                             \
+    ST_READS_A                                                                                                        \
+    /* shift 8 */                                                                                                     \
+    "v_alignbit_b32 %[g0], %[cy], " EX ", 8\n v_alignbit_b32 %[g1], " EX ", " EY ", 8\n"                              \
+    "v_alignbit_b32 %[g2], " EY ", " EZ ", 8\n v_alignbit_b32 %[g3], " EZ ", " EW ", 8\n"                             \
+    "v_pk_mad_u16 %[g0], %[g0], %[g0], %[g0]\n v_pk_mad_u16 %[g1], %[g1], %[g1], %[g1]\n"                             \
+    "v_pk_mad_u16 %[g2], %[g2], %[g2], %[g2]\n v_pk_mad_u16 %[g3], %[g3], %[g3], %[g3]\n"                             \
+    ST_READS_B                                                                                                        \
+    "s_waitcnt lgkmcnt(8)\n"                                                                                          \
+    /* products of shift 12 between the windows of shift 4 */                                                         \
+    ST_MM("v[56:57]", 0, 0, "0")                                                                                      \
+    "v_alignbit_b32 %[g0], %[cy], " EX ", 4\n v_alignbit_b32 %[g1], " EX ", " EY ", 4\n"                              \
+    ST_MM("v[58:59]", 0, 1, "v[52:55]")                                                                               \
+    "v_alignbit_b32 %[g2], " EY ", " EZ ", 4\n v_alignbit_b32 %[g3], " EZ ", " EW ", 4\n"                             \
+    ST_MM("v[60:61]", 0, 2, "v[52:55]")                                                                               \
+    "v_pk_mad_u16 %[g0], %[g0], %[g0], %[g0]\n v_pk_mad_u16 %[g1], %[g1], %[g1], %[g1]\n"                             \
+    ST_MM("v[62:63]", 0, 3, "v[52:55]")                                                                               \
+    "v_pk_mad_u16 %[g2], %[g2], %[g2], %[g2]\n v_pk_mad_u16 %[g3], %[g3], %[g3], %[g3]\n"                             \
+    ST_READS_A                                                                                                        \
+    "s_waitcnt lgkmcnt(8)\n"                                                                                          \
+    /* products of shift 8 between the hashes of shift 0 (the words as they are) */                                   \
+    ST_MM("v[64:65]", 1, 0, "v[52:55]")                                                                               \
+    "v_pk_mad_u16 %[g0], " EX ", " EX ", " EX "\n v_pk_mad_u16 %[g1], " EY ", " EY ", " EY "\n"                       \
+    ST_MM("v[66:67]", 1, 1, "v[52:55]")                                                                               \
+    "v_pk_mad_u16 %[g2], " EZ ", " EZ ", " EZ "\n v_pk_mad_u16 %[g3], " EW ", " EW ", " EW "\n"                       \
+    ST_MM("v[68:69]", 1, 2, "v[52:55]")                                                                               \
+    "s_nop 1\n"                                                                                                       \
+    ST_MM("v[70:71]", 1, 3, "v[52:55]")                                                                               \
+    ST_READS_B                                                                                                        \
+    "s_waitcnt lgkmcnt(8)\n"                                                                                          \
+    ST_MM("v[56:57]", 2, 0, "v[52:55]") "s_nop 1\n" ST_MM("v[58:59]", 2, 1, "v[52:55]") "s_nop 1\n"                   \
+    ST_MM("v[60:61]", 2, 2, "v[52:55]") "s_nop 1\n" ST_MM("v[62:63]", 2, 3, "v[52:55]")                               \
+    "s_waitcnt lgkmcnt(0)\n"                                                                                          \
+    "s_nop 0\n"                                                                                                       \
+    ST_MM("v[64:65]", 3, 0, "v[52:55]") "s_nop 1\n" ST_MM("v[66:67]", 3, 1, "v[52:55]") "s_nop 1\n"                   \
+    ST_MM("v[68:69]", 3, 2, "v[52:55]") "s_nop 1\n" ST_MM("v[70:71]", 3, 3, "v[52:55]")
+
+#endif
 // ---- one element of a layer.  U: which of the wave's elements; X, Y, Z, W / QUAD: its four registers; P: parity of
 // the layer; NEED: requests that may still be in flight when this element's has arrived.
 // Behind the last product the next layer's request for this slot goes out at once (three instructions between a dot
@@ -172,13 +259,27 @@ constexpr int kStRowWaves = 8;
     ST_RELOAD("%[xa" #U "]", P)                                                                                       \
     "5" #U ":\n"                                                                                                      \
     "s_waitcnt vmcnt(" #NEED ")\n"
-#define ST_ITEM_TAIL(U, P, REQUEST)                                                                                   \
-    REQUEST                                                                                                           \
+#ifndef ST_MFMA
+#define ST_ELEMENT_SUM(U)                                                                                             \
     "s_mov_b64 exec, %[keep" #U "]\n"                                                                                 \
     "s_nop 0\n"                                                                                                       \
     "v_add_f32 %[a0], %[a0], %[a1]\n"                                                                                 \
     "v_add_f32 %[a2], %[a2], %[a3]\n"                                                                                 \
-    "v_add_f32 %[a0], %[a0], %[a2]\n"                                                                                 \
+    "v_add_f32 %[a0], %[a0], %[a2]\n"
+#else
+// the lane's sum is register (lane % 4) of the matrix result: two selects by the lane number's bit 0, one by bit 1
+#define ST_ELEMENT_SUM(U)                                                                                             \
+    /* five instructions' distance from the last matrix instruction, whether or not a request stands in between */   \
+    "s_mov_b64 vcc, %[odd]\n"                                                                                         \
+    "s_mov_b64 exec, %[keep" #U "]\n"                                                                                 \
+    "s_nop 2\n"                                                                                                       \
+    "v_cndmask_b32 %[a0], v52, v53, vcc\n"                                                                            \
+    "v_cndmask_b32 %[a1], v54, v55, vcc\n"                                                                            \
+    "v_cndmask_b32_e64 %[a0], %[a0], %[a1], %[upper]\n"
+#endif
+#define ST_ITEM_TAIL(U, P, REQUEST)                                                                                   \
+    REQUEST                                                                                                           \
+    ST_ELEMENT_SUM(U)                                                                                                 \
     "ds_write_b32 %[pa" #U "], %[a0] offset:" #P "*16384\n"                                                           \
     "s_mov_b64 exec, -1\n"                                                                                            \
     "s_branch 8" #U "f\n"                                                                                             \
@@ -347,14 +448,27 @@ constexpr int kStRowWaves = 8;
     "s_waitcnt vmcnt(0)\n"
 
 // what the loop reads and the registers it works in
+#ifndef ST_MFMA
 #define ST_OUT_COMMON                                                                                                 \
     [a0] "=&v"(a0), [a1] "=&v"(a1), [a2] "=&v"(a2), [a3] "=&v"(a3), [cy] "=&v"(cy), [g0] "=&v"(g0), [g1] "=&v"(g1),  \
     [g2] "=&v"(g2), [g3] "=&v"(g3), [t0] "=&v"(t0), [t1] "=&v"(t1), [t2] "=&v"(t2), [t3] "=&v"(t3), [t4] "=&v"(t4),  \
     [t5] "=&v"(t5), [t6] "=&v"(t6), [t7] "=&v"(t7), [u0] "=&v"(u0), [u1] "=&v"(u1), [u2] "=&v"(u2), [u3] "=&v"(u3),  \
     [u4] "=&v"(u4), [u5] "=&v"(u5), [u6] "=&v"(u6), [u7] "=&v"(u7), [xb] "=&v"(xb), [k] "=&s"(k), [kn] "=&s"(kn),    \
     [j] "=&s"(j), [cn] "=&s"(cn), [xn] "=&s"(xn), [op] "=&s"(op)
+#define ST_IN_SUM [mask] "s"(0xFF00u)
+#define ST_CLOBBERS_SUM "memory"
+#else
+#define ST_OUT_COMMON                                                                                                 \
+    [a0] "=&v"(a0), [a1] "=&v"(a1), [cy] "=&v"(cy), [g0] "=&v"(g0), [g1] "=&v"(g1), [g2] "=&v"(g2), [g3] "=&v"(g3),  \
+    [t0] "=&v"(t0), [t1] "=&v"(t1), [t2] "=&v"(t2), [t3] "=&v"(t3), [xb] "=&v"(xb), [k] "=&s"(k), [kn] "=&s"(kn),    \
+    [j] "=&s"(j), [cn] "=&s"(cn), [xn] "=&s"(xn), [op] "=&s"(op)
+#define ST_IN_SUM [mask] "s"(0xFF00u), [odd] "s"(0xAAAAAAAAAAAAAAAAull), [upper] "s"(0xCCCCCCCCCCCCCCCCull)
+#define ST_CLOBBERS_SUM                                                                                               \
+    "memory", "v52", "v53", "v54", "v55", "v56", "v57", "v58", "v59", "v60", "v61", "v62", "v63", "v64", "v65", "v66", "v67",   \
+    "v68", "v69", "v70", "v71"
+#endif
 #define ST_IN_COMMON                                                                                                  \
-    [lane4] "v"(lane4), [mask] "s"(0xFF00u), [sel] "s"(0x0C0C0700u), [dc] "s"(dc), [dx] "s"(dx), [dq] "s"(dout),      \
+    [lane4] "v"(lane4), ST_IN_SUM, [sel] "s"(0x0C0C0700u), [dc] "s"(dc), [dx] "s"(dx), [dq] "s"(dout),      \
     [count] "s"(s_count), [last] "s"(s_count - 1), [nitems] "s"(s_nitems), [rl] "s"(rl), [xo0] "v"(xo[0]), [xo1] "v"(xo[1]),\
     [sa0] "v"(sa[0]), [sa1] "v"(sa[1]), [sa2] "v"(sa[2]), [sa3] "v"(sa[3]), [sa4] "v"(sa[4]), [sa5] "v"(sa[5]),       \
     [sa6] "v"(sa[6]), [sa7] "v"(sa[7]), [stm0] "s"(stm[0]), [stm1] "s"(stm[1]), [rs] "v"(rs), [oo] "v"(oo),           \
@@ -363,7 +477,7 @@ constexpr int kStRowWaves = 8;
 #define ST_IN_ITEM(U) [vo##U] "v"(vo[U]), [xa##U] "v"(xa[U]), [pa##U] "v"(pa[U]), [first##U] "s"(first[U]), [keep##U] "s"(keep[U])
 #define ST_IN_ITEM_CT(U) [co##U] "v"(co[U]), [cm##U] "s"(cm[U])
 #define ST_CLOBBERS                                                                                                   \
-    "memory", "vcc", "scc", "v72", "v73", "v74", "v75", "v76", "v77", "v78", "v79", "v80", "v81", "v82", "v83", "v84", "v85",   \
+    ST_CLOBBERS_SUM, "vcc", "scc", "v72", "v73", "v74", "v75", "v76", "v77", "v78", "v79", "v80", "v81", "v82", "v83", "v84", "v85",   \
     "v86", "v87", "v88", "v89", "v90", "v91", "v92", "v93", "v94", "v95", "v96", "v97", "v98", "v99", "v100", "v101", "v102",   \
     "v103", "v104", "v105", "v106", "v107", "v108", "v109", "v110", "v111", "v112", "v113", "v114", "v115", "v116", "v117",     \
     "v118", "v119", "v120", "v121", "v122", "v123", "v124", "v125", "v126", "v127"

@@ -63,13 +63,17 @@ class Memory:
 ASM_LINES = set()
 
 
-E32_ALIASES = {"v_add_f32", "v_add_u32", "v_mov_b32", "v_and_b32", "v_or_b32", "v_xor_b32", "v_cvt_f16_f32", "v_sub_u32",
+E32_ALIASES = {"v_cndmask_b32", "v_add_f32", "v_add_u32", "v_mov_b32", "v_and_b32", "v_or_b32", "v_xor_b32", "v_cvt_f16_f32", "v_sub_u32",
                "v_mul_f32", "v_lshlrev_b32", "v_lshrrev_b32"}
 
 
 def _arith(text):
-    """`3-1`, `1*128+14+1`, `0*16384+256`: constant expressions the assembler folds (hand-written blocks use them for
-    offsets that depend on a macro parameter).  Anything else is returned as it is."""
+    """`3-1`, `1*128+14+1`, `0*16384+256`, `v[96+8*1+2*3:96+8*1+2*3+1]`: constant expressions the assembler folds
+    (hand-written blocks use them for offsets and register numbers that depend on a macro parameter).  Anything else is
+    returned as it is."""
+    m = re.fullmatch(r"([vsa])\[([0-9+* -]+):([0-9+* -]+)\]", text)
+    if m:
+        return "%s[%d:%d]" % (m.group(1), eval(m.group(2), {"__builtins__": {}}, {}), eval(m.group(3), {"__builtins__": {}}, {}))
     if re.fullmatch(r"[0-9a-fA-Fx+*() -]+", text) and re.search(r"[+*-]", text.lstrip("-")) and not re.fullmatch(r"-?(0x)?[0-9a-fA-F]+", text):
         return str(eval(text, {"__builtins__": {}}, {}))
     return text
@@ -221,7 +225,9 @@ def inst_info(inst):
             for t in o[1:]: vuse |= _regs(t, "v")
         else:
             for t in o: vuse |= _regs(t, "v")
-    info = dict(kind=kind, sdef=sdef, vdef=vdef, suse=suse, vuse=vuse, op=op, ln=ln, text=text,
+    mfma_passes = {"v_mfma_f32_4x4x4_16b_f16": 2, "v_mfma_f32_16x16x32_f16": 5}.get(op, 0)    # (passes + 3 = the distance hipcc keeps: 5 and 8)
+    info = dict(kind=kind, sdef=sdef, vdef=vdef, suse=suse, vuse=vuse, op=op, ln=ln, text=text, mfma=mfma_passes,
+                srcc=(_regs(o[3], "v") if mfma_passes and len(o) > 3 else set()),
                 dpp=any(k in mods for k in ("row_shr", "row_shl", "row_ror", "quad_perm", "row_bcast", "wave_shr", "wave_shl", "row_mirror", "row_half_mirror", "row_newbcast")) or "_dpp" in op,
                 trans=op.startswith(TRANS), lds_dma=("_lds_" in op or (kind == "vmem" and "lds" in mods)),
                 rwlane=bool(re.match(r"v_(readlane|writelane)", op)), readlane=bool(re.match(r"v_(readlane|readfirstlane)", op)),
@@ -244,8 +250,20 @@ class Wave:
             HAZARDS[key][0] += 1
         for after, prev in reversed(hist):
             between = now - after
-            if between >= 5:
+            if between >= 12:
                 break
+            # matrix instructions (what the compiler puts between such pairs on gfx950: 2 wait states between a matrix
+            # instruction and one that accumulates into its result, passes + 3 before anything else reads the result, 2
+            # between a vector instruction that writes a register and a matrix instruction that reads it)
+            if prev["mfma"]:
+                if cur["mfma"] and between < 2 and prev["vdef"] & cur["srcc"]:
+                    hit("matrix result -> accumulated into by the next matrix instruction (2)", prev)
+                elif not cur["mfma"] and between < prev["mfma"] + 3 and cur["kind"] in ("valu", "vmem", "lds") and prev["vdef"] & (cur["vuse"] | cur["vdef"]):
+                    hit("matrix result -> read or overwritten by another instruction (passes + 3)", prev)
+            elif prev["kind"] == "valu" and cur["mfma"] and between < 2 and prev["vdef"] & cur["vuse"]:
+                hit("VALU writes VGPR -> matrix instruction reads it (2)", prev)
+            if between >= 5:
+                continue
             pv = prev["kind"] == "valu"
             if pv and cur["kind"] == "vmem" and prev["sdef"] & cur["suse"]:
                 hit("VALU writes SGPR -> VMEM reads it (5)", prev)
@@ -278,7 +296,7 @@ class Wave:
             except Exception: step = 1
         self.wstate = now + step
         hist.append((self.wstate, cur))
-        if len(hist) > 8:
+        if len(hist) > 16:
             del hist[0]
 
     def __init__(self, wg, wid, insts, labels, mem, lds, kernarg, wg_id, rng):
@@ -845,6 +863,33 @@ class Wave:
             d0, _ = self.vreg_index(o[0])
             for r in range(4):
                 self.v[d0 + r] = as_u32(np.array([D[4 * (l // 16) + r, l % 16] for l in range(64)], dtype=np.float32))
+        elif op == "v_mfma_f32_4x4x4_16b_f16":
+            # Sixteen independent 4 x 4 x 4 products: block b = lanes 4 b .. 4 b + 3.  Lane 4 b + i holds A_b[i][0 .. 3] (two
+            # registers of two halves) and, with j for i, B_b[0 .. 3][j]; register r of lane 4 b + j holds C and D [r][j].
+            # Every lane takes part whatever EXEC says; sums in double, rounded once to fp32.
+            if mods:
+                raise Fault(f"modifiers of {op} not modelled ({self.who()})")
+            def halves4(tok):
+                i0, n = self.vreg_index(tok)
+                assert n == 2, tok
+                regs = np.stack([self.v[i0 + q] for q in range(2)], axis=1)                       # [lane][2]
+                h = np.stack([regs & U32(0xFFFF), regs >> U32(16)], axis=2).reshape(64, 4)       # [lane][4], low half first
+                return h.astype(np.uint16).view(np.float16).astype(np.float64)
+            ha, hb = halves4(o[1]), halves4(o[2])
+            c0 = self.vreg_index(o[3])[0]
+            if c0 is None and int(o[3], 0) != 0:
+                raise Fault(f"constant accumulator of {op} not modelled ({self.who()})")
+            d0, nd = self.vreg_index(o[0])
+            assert nd == 4, o[0]
+            out = np.zeros((4, 64), dtype=np.float32)
+            with np.errstate(all="ignore"):
+                for l in range(64):
+                    b, j = l // 4, l % 4
+                    for r in range(4):
+                        acc = float(f32(self.v[c0 + r][l:l + 1])[0]) if c0 is not None else 0.0
+                        out[r, l] = np.float32(acc + float(np.dot(ha[4 * b + r], hb[4 * b + j])))
+            for r in range(4):
+                self.v[d0 + r] = as_u32(out[r])
         elif op in ("v_and_or_b32", "v_perm_b32", "v_alignbit_b32", "v_pk_mad_u16"):
             a, b, c = V(o[1]), V(o[2]), V(o[3])
             if op == "v_and_or_b32":
