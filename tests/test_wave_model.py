@@ -23,14 +23,14 @@ PKG = os.path.join(ROOT, "let-it-slide_amd")
 CUS = 256                        # the grid the planner makes on the target: one workgroup per compute unit
 
 
-def compile_to_assembly(tmp_path_factory, name):
+def compile_to_assembly(tmp_path_factory, name, extra=()):
     if shutil.which("hipcc") is None:
         pytest.skip("hipcc not found")
     spec = importlib.util.spec_from_file_location("rptc_build", os.path.join(PKG, "build.py"))
     mod = importlib.util.module_from_spec(spec)
     spec.loader.exec_module(mod)
     out = str(tmp_path_factory.mktemp("isa") / (name + ".s"))
-    subprocess.run(["hipcc", *mod.FLAGS, "--cuda-device-only", "-S", os.path.join(PKG, "csrc", name + ".hip"), "-o", out],
+    subprocess.run(["hipcc", *mod.FLAGS, *extra, "--cuda-device-only", "-S", os.path.join(PKG, "csrc", name + ".hip"), "-o", out],
                    check=True, capture_output=True)
     return out
 
@@ -445,3 +445,52 @@ def run_steady(isa, oracle, m, n, count, S, mode, blocks, seed=7, burst=8, laten
                                               (7, 704, 1, 6, 1), (512, 6144, 2, 8, 1), (1024, 2048 + 64, 5, 8, 0)])
 def test_steady_kernel_matches_the_oracle(steady_isa, oracle, m, n, count, S, mode):
     run_steady(steady_isa, oracle, m, n, count, S, mode, blocks=sorted({0, 1, (m - 1) // (2 * ((m + 2 * CUS - 1) // (2 * CUS)))}))
+
+
+def steady_fits(m, n):
+    rpb = 2 * ((m + 2 * CUS - 1) // (2 * CUS))
+    lt = (n & 2047) >> 6
+    rw_tail = 64 // lt if lt else 1
+    total = (n >> 11) * (rpb // 2) + ((rpb + rw_tail - 1) // rw_tail if lt else 0)
+    return (-(-total // 16) <= 4 and rpb * (n // 64) * 4 <= 16384 and ((n >> 11) + (1 if lt else 0)) * 4096 <= 32768 and n <= 16384)
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_steady_kernel_on_random_shapes(steady_isa, oracle, seed):
+    """Chains of one random shape (any row count up to 3000, any multiple of 64 columns up to 12800 that the kernel's
+    fixed LDS layout holds): the first workgroup, one in the middle and the one that holds the end of the rows, where a
+    row block is partial and elements are empty; S and carry mode by seed."""
+    rng = np.random.default_rng(700 + seed)
+    while True:
+        m, n = int(rng.integers(1, 3001)), 64 * int(rng.integers(1, 201))
+        if steady_fits(m, n):
+            break
+    rpb = 2 * ((m + 2 * CUS - 1) // (2 * CUS))
+    last = (m - 1) // rpb
+    run_steady(steady_isa, oracle, m, n, int(rng.integers(1, 5)), (6, 8)[seed & 1], (seed >> 1) & 1, blocks=sorted({0, last // 2, last}), seed=seed)
+
+
+def test_steady_kernel_with_four_elements_a_wave_and_at_its_limits(steady_isa, oracle):
+    """8192 x 8192: 64 elements a workgroup and layer, four a wave, the set of partial sums full (32 rows x 128);
+    16384 columns: the activation image full; a single row; 64 columns."""
+    run_steady(steady_isa, oracle, 8192, 8192, 2, 8, 1, blocks=[0, 255])
+    run_steady(steady_isa, oracle, 5, 16384, 2, 8, 0, blocks=[0, 1, 2])
+    run_steady(steady_isa, oracle, 1, 64, 3, 6, 1, blocks=[0])
+    run_steady(steady_isa, oracle, 4096, 11008, 2, 8, 0, blocks=[0, 255])
+
+
+@pytest.mark.parametrize("burst,latency", [(10 ** 6, (400, 60)), (8, (3000, 300)), (8, (40, 10))])
+def test_steady_kernel_under_other_interleavings_and_latencies(steady_isa, oracle, burst, latency):
+    """Every wave running until it blocks; memory that answers very late; memory that answers at once."""
+    run_steady(steady_isa, oracle, 33, 4096 + 768, 3, 8, 1, blocks=[0, 16], seed=11, burst=burst, latency=latency)
+
+
+@pytest.fixture(scope="module")
+def steady_mfma_isa(tmp_path_factory):
+    return compile_to_assembly(tmp_path_factory, "matvec_steady", extra=("-DST_MFMA",))
+
+
+@pytest.mark.parametrize("m,n,count,S,mode", [(33, 4096 + 768, 3, 8, 0), (300, 64, 2, 6, 1), (1024, 2048 + 64, 3, 8, 1), (8192, 8192, 2, 8, 0)])
+def test_steady_kernel_with_the_products_on_the_matrix_unit(steady_mfma_isa, oracle, m, n, count, S, mode):
+    """The -DST_MFMA build of the same kernel (v_mfma_f32_4x4x4_16b_f16 in place of the two-term dot products)."""
+    run_steady(steady_mfma_isa, oracle, m, n, count, S, mode, blocks=sorted({0, (m - 1) // (2 * ((m + 2 * CUS - 1) // (2 * CUS)))}))
