@@ -71,6 +71,46 @@ __global__ __launch_bounds__(256) void pack_x_kernel(const uint4 *__restrict__ x
     dst[(size_t)n8 * 48] = v.w;
 }
 
+// The packed image of the row-owner kernel below: the four activation pairs that one MFMA's B operand takes from a lane
+// are 16 consecutive bytes.  Step q = 4k + j of lane-of-row l in slab t (slot 1024 t + q * lanes + l, `lanes` elements a
+// row in that slab) goes to dword ((((32 t + l) * 8 + 2 j + h) * 16 + b) * 4 + p) of its plane, b the batch column, with
+// (h, p) = (0, 0..3) for k = 7, 0, 4, 1 and (1, 0..3) for k = 5, 2, 6, 3: the order in which the steps of an element meet
+// the slots (inference.cu:237-250).  A ragged last slab is padded with zeros to a multiple of four lanes-of-row.
+// Thread (idx, b) reads the 16 bytes x[b][8 idx .. 8 idx + 7] (slots i * (n/8) + idx, i = 0..3) as pack_x_kernel does;
+// the threads behind them write the padding.
+__device__ __forceinline__ size_t mm_tuple_position(int slot, int n, int b)
+{
+    const int T = n >> 11, Lt = (n & 2047) >> 6;
+    const int t = slot >> 10 < T ? slot >> 10 : T;
+    const int lanes = t < T ? 32 : Lt;
+    const int r = slot - (t << 10), q = r / lanes, l = r - q * lanes;
+    const int k = q >> 2, j = q & 3;
+    // k:     0  1  2  3  4  5  6  7
+    // half:  0  0  1  1  0  1  1  0
+    // pos:   1  3  1  3  2  0  2  0
+    const int h = (0x6C >> k) & 1, pos = (0x22DD >> (2 * k)) & 3;     // two bits of position per k, k = 0 lowest
+    return ((((size_t)(32 * t + l) * 8 + 2 * j + h) * 16 + b) << 2) + pos;
+}
+
+__global__ __launch_bounds__(256) void pack_x_tuples_kernel(const uint4 *__restrict__ x, uint32_t *__restrict__ xp, int n, int batch)
+{
+    const int t = blockIdx.x * 256 + threadIdx.x;
+    const int n8 = n >> 3, b = t & 15, idx = t >> 4;
+    if (idx < n8) {
+        const uint4 v = b < batch ? x[(size_t)b * n8 + idx] : make_uint4(0, 0, 0, 0);
+        xp[mm_tuple_position(idx, n, b)] = v.x;
+        xp[mm_tuple_position(n8 + idx, n, b)] = v.y;
+        xp[mm_tuple_position(2 * n8 + idx, n, b)] = v.z;
+        xp[mm_tuple_position(3 * n8 + idx, n, b)] = v.w;
+        return;
+    }
+    // the lanes-of-row Lt .. 4 * ceil(Lt / 4) - 1 of the ragged slab: 512 dwords each
+    const int T = n >> 11, Lt = (n & 2047) >> 6;
+    const int pad = (t - n8 * 16) * 4;                                   // four dwords a thread
+    if (pad < (((Lt + 3) & ~3) - Lt) * 512)
+        *reinterpret_cast<uint4 *>(xp + (size_t)(32 * T + Lt) * 512 + pad) = make_uint4(0, 0, 0, 0);
+}
+
 template <int S>
 __device__ __forceinline__ uint32_t mm_table_value(const uint32_t *__restrict__ codebook, int b)
 {
@@ -354,6 +394,170 @@ __global__ __launch_bounds__(kMmThreads) __attribute__((amdgpu_waves_per_eu(4, 4
     }
 }
 
+// ---------------------------------------------------------------- the row-owner form (2 bits, batch <= 16)
+// A workgroup of 16 waves owns TILES blocks of 16 rows over the whole width, so nothing leaves the workgroup but the
+// finished fp16 outputs: no partial tiles in memory, no arrival counters, no second pass.  The price is the one named
+// above: every workgroup reads the whole packed activation image (from L2), 8 KiB for every 64 stream elements it
+// decodes, so its first-level cache moves 352 KiB of activations for 44 KiB of stream on a 16 x 11008 share.
+//   * a wave takes the (slab, group of four lanes-of-row) pairs w, w + 16, ... of the row; the 32 activation registers of
+//     a pair serve its TILES row blocks.  They are refilled for the wave's next pair a quarter at a time, each quarter
+//     as soon as the last row block has used it, so one set of 32 registers is enough.
+//   * a wave's MFMA accumulators run over all its pairs; the 16 waves' tiles are added in LDS in wave order once.
+constexpr int kMrThreads = 1024;
+constexpr int kMrWaves = kMrThreads / kWave;
+constexpr int kMrMaxTiles = 3;
+
+template <int S, int MODE, int TILES>
+__global__ __launch_bounds__(kMrThreads) void matmul_rows_kernel(const uint32_t *__restrict__ comp32,
+                                                                 const uint32_t *__restrict__ codebook,
+                                                                 const uint32_t *__restrict__ xp32, uint16_t *__restrict__ out,
+                                                                 int m, int n, int batch)
+{
+    extern __shared__ uint32_t lds[];
+    float *part = reinterpret_cast<float *>(lds + kMmTableBytes / 4);    // [wave][tile][v][lane]
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int i = lane & 15, g = lane >> 4;
+    const uint32_t lane4 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds)) + lane * 4;
+    const int T = n >> 11, Lt = (n & 2047) >> 6;
+    const int pairs = 8 * T + ((Lt + 3) >> 2);                    // (slab, four lanes-of-row) pairs of a row
+    const int row0 = blockIdx.x * (16 * TILES);
+
+    constexpr int kTableRowsPerWave = 256 / kMrWaves;
+    uint32_t table_values[kTableRowsPerWave];
+#pragma unroll
+    for (int r = 0; r < kTableRowsPerWave; r++) table_values[r] = mm_table_value<S>(codebook, kTableRowsPerWave * w + r);
+
+    // what a pair's loads need: where its slab starts, how many elements a row has there, this lane's lane-of-row
+    struct Pair {
+        int slab, lanes, l;
+        bool has_l;
+    };
+    auto pair_of = [&](int sq) {
+        Pair p;
+        p.slab = sq < 8 * T ? sq >> 3 : T;
+        p.lanes = sq < 8 * T ? 32 : Lt;
+        p.l = 4 * (sq - 8 * p.slab) + g;
+        p.has_l = p.l < p.lanes;
+        return p;
+    };
+    // this lane's element of row block t and the word in front of it (as in matmul_kernel: a lane with nothing to decode
+    // reads element 0, and its products meet zero activations or land in rows that are never stored)
+    auto load_element = [&](const Pair &p, int t, uint4 &e, uint32_t &carry) {
+        const int row = row0 + 16 * t + i;
+        const bool valid = p.has_l && row < m;
+        const size_t ei = valid ? (size_t)p.slab * m * 32 + (size_t)row * p.lanes + p.l : 0;
+        size_t ci = ei * 4 + 3;
+        if (p.l > 0 && valid) ci = ei * 4 - 1;
+        else if (MODE == RPTC_CONTINUOUS && p.slab > 0 && valid) ci = (((size_t)(p.slab - 1) * m + row) * 32 + 31) * 4 + 3;
+        e = reinterpret_cast<const uint4 *>(comp32)[ei];
+        carry = comp32[ci];
+    };
+    // the B operands of the two MFMAs of quarter j (steps 4k + j): 16 bytes each in the packed image, and zeros for a
+    // lane past the end of a ragged row (pack_x_tuples_kernel pads), so no lane needs a predicate here
+    auto load_quarter = [&](const Pair &p, int j, v4u32 (&xb)[8]) {
+        const v4u32 *xq = reinterpret_cast<const v4u32 *>(xp32) + ((size_t)(32 * p.slab + p.l) * 8 + 2 * j) * 16 + i;
+        xb[2 * j] = xq[0];
+        xb[2 * j + 1] = xq[16];
+    };
+    // One pair's share of the product for every row block: quarter by quarter (the windows of a quarter come straight
+    // from the element's words, so the order of the quarters is free), and behind each quarter the next pair's
+    // activations for it when there is a next pair (`more` is a constant where this is expanded).
+    auto consume = [&](const Pair &p, const Pair &next, bool more, v4u32 (&xb)[8], const uint4 (&e)[TILES],
+                       const uint32_t (&carry)[TILES], v4f32 (&d)[TILES]) {
+        const bool no_carry = MODE == RPTC_CONTINUOUS && p.slab == 0 && p.l == 0;    // the stream starts here
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint32_t sh = 12 - 4 * j;
+#pragma unroll
+            for (int t = 0; t < TILES; t++) {
+                const uint32_t cw = no_carry ? 0u : carry[t];
+                const uint32_t gc = j == 3 ? e[t].x : alignbit(cw, e[t].x, sh);        // steps (7,j) and (0,j)
+                const uint32_t gx = j == 3 ? e[t].y : alignbit(e[t].x, e[t].y, sh);    // (4,j), (1,j)
+                const uint32_t gy = j == 3 ? e[t].z : alignbit(e[t].y, e[t].z, sh);    // (5,j), (2,j)
+                const uint32_t gz = j == 3 ? e[t].w : alignbit(e[t].z, e[t].w, sh);    // (6,j), (3,j)
+                // one accumulator: the second MFMA waits for the first, with the second half's decode between them
+                uint32_t w0, w1, w2, w3, w4, w5, w6, w7;
+                gather2(gc, lane4, w0, w1);
+                gather2(gx, lane4, w2, w3);
+                const v4u32 a0 = {w0, w1, w2, w3};
+                d[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8f16, a0), __builtin_bit_cast(v8f16, xb[2 * j]), d[t], 0, 0, 0);
+                gather2(gy, lane4, w4, w5);
+                gather2(gz, lane4, w6, w7);
+                const v4u32 a1 = {w4, w5, w6, w7};
+                d[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8f16, a1), __builtin_bit_cast(v8f16, xb[2 * j + 1]), d[t], 0, 0, 0);
+            }
+            if (more) load_quarter(next, j, xb);                  // this quarter is free: the next pair's goes in
+        }
+    };
+
+    int sq = w;
+    Pair cur = pair_of(sq < pairs ? sq : 0);
+    v4u32 xb[8];
+    uint4 e[TILES];
+    uint32_t carry[TILES];
+    if (sq < pairs) {
+#pragma unroll
+        for (int t = 0; t < TILES; t++) load_element(cur, t, e[t], carry[t]);
+#pragma unroll
+        for (int j = 0; j < 4; j++) load_quarter(cur, j, xb);
+    }
+#pragma unroll
+    for (int r = 0; r < kTableRowsPerWave; r++) lds[(kTableRowsPerWave * w + r) * 64 + lane] = table_values[r];
+    __syncthreads();                                              // the table is complete
+
+    v4f32 d[TILES];
+#pragma unroll
+    for (int t = 0; t < TILES; t++) d[t] = v4f32{0.f, 0.f, 0.f, 0.f};
+    if (sq < pairs) {
+        // every pair but the wave's last with the next pair's requests among the work, then the last without (one
+        // loop with the requests under a condition would make every wait count as if they had not been made)
+        while (sq + kMrWaves < pairs) {
+            const Pair next = pair_of(sq + kMrWaves);
+            uint4 en[TILES];
+            uint32_t cn[TILES];
+#pragma unroll
+            for (int t = 0; t < TILES; t++) load_element(next, t, en[t], cn[t]);
+            consume(cur, next, true, xb, e, carry, d);
+#pragma unroll
+            for (int t = 0; t < TILES; t++) e[t] = en[t], carry[t] = cn[t];
+            cur = next;
+            sq += kMrWaves;
+        }
+        consume(cur, cur, false, xb, e, carry, d);
+    }
+
+    // tile element (row 4*(lane/16) + v, batch column lane%16) sits in register v of lane `lane`
+#pragma unroll
+    for (int t = 0; t < TILES; t++)
+#pragma unroll
+        for (int v = 0; v < 4; v++) part[((w * TILES + t) * 4 + v) * 64 + lane] = d[t][v];
+    __syncthreads();
+    if (tid < TILES * 256) {
+        const int t = tid >> 8, vl = tid & 255;
+        float y = 0.f;
+#pragma unroll
+        for (int k = 0; k < kMrWaves; k++) y += part[(k * TILES + t) * 256 + vl];      // wave order
+        const int ln = vl & 63, v = vl >> 6;
+        const int b = ln & 15, row = row0 + 16 * t + 4 * (ln >> 4) + v;
+        if (b < batch && row < m) out[(size_t)b * m + row] = float_to_half_bits(y);
+    }
+}
+
+template <int S, int MODE>
+static void launch_matmul_rows(const uint32_t *comp, const uint32_t *cb, const uint32_t *xpack, uint16_t *out, int m, int n,
+                               int batch, int cus, hipStream_t s)
+{
+    const int total = (m + 15) / 16;
+    int tiles = (total + cus - 1) / cus;                          // one workgroup per CU where the row blocks allow
+    if (tiles > kMrMaxTiles) tiles = kMrMaxTiles;
+    const int grid = (total + tiles - 1) / tiles;
+    const int lds_bytes = kMmTableBytes + kMrWaves * tiles * 256 * 4;
+    if (tiles == 1) hipLaunchKernelGGL((matmul_rows_kernel<S, MODE, 1>), dim3(grid), dim3(kMrThreads), lds_bytes, s, comp, cb, xpack, out, m, n, batch);
+    else if (tiles == 2) hipLaunchKernelGGL((matmul_rows_kernel<S, MODE, 2>), dim3(grid), dim3(kMrThreads), lds_bytes, s, comp, cb, xpack, out, m, n, batch);
+    else hipLaunchKernelGGL((matmul_rows_kernel<S, MODE, 3>), dim3(grid), dim3(kMrThreads), lds_bytes, s, comp, cb, xpack, out, m, n, batch);
+}
+
 struct MmScratch {
     uint32_t *xpack;
     float *partial;
@@ -384,6 +588,15 @@ int prepare_matmul(int device)
     RPTC_MM_ALLOW(1, 4)
     RPTC_MM_ALLOW(2, 4)
 #undef RPTC_MM_ALLOW
+#define RPTC_MR_ALLOW(TILES)                                                                \
+    if ((rc = mm_allow_lds(matmul_rows_kernel<6, RPTC_AS_WRITTEN, TILES>))) return rc;     \
+    if ((rc = mm_allow_lds(matmul_rows_kernel<6, RPTC_CONTINUOUS, TILES>))) return rc;     \
+    if ((rc = mm_allow_lds(matmul_rows_kernel<8, RPTC_AS_WRITTEN, TILES>))) return rc;     \
+    if ((rc = mm_allow_lds(matmul_rows_kernel<8, RPTC_CONTINUOUS, TILES>))) return rc;
+    RPTC_MR_ALLOW(1)
+    RPTC_MR_ALLOW(2)
+    RPTC_MR_ALLOW(3)
+#undef RPTC_MR_ALLOW
     // the device addresses of the static scratch arrays (the symbols themselves are not device addresses)
     MmScratch &sc = g_mm[device];
     if ((rc = (int)hipGetSymbolAddress(reinterpret_cast<void **>(&sc.xpack), HIP_SYMBOL(g_xpack)))) return rc;
@@ -470,7 +683,7 @@ static int plan_matmul(const void *compressed, const void *codebook, const void 
     p->counters = p->groups < kMmMaxGroups ? p->groups : kMmMaxGroups;
     const int total = ((int)m + 15) / 16;
     const int max_rb = (total + p->groups - 1) / p->groups;
-    p->xpack_words = (int64_t)p->planes * (n / 2) * 16;
+    p->xpack_words = (int64_t)p->planes * (n / 2) * 16 + 3 * 512;     // and the padding of a ragged slab in the row-owner form's image
     p->partial_floats = (int64_t)p->groups * p->slabs * max_rb * p->planes * 256;
     return 0;
 }
@@ -485,6 +698,19 @@ static int run_matmul(const int32_t *compressed, const uint16_t *codebook, const
     if (rc) return rc;
     auto a_comp = reinterpret_cast<const uint32_t *>(compressed);
     auto a_cb = reinterpret_cast<const uint32_t *>(codebook);
+#ifdef RPTC_MM_ROWS
+    if (bits == 2 && batch <= 16) {
+        // the row-owner form: its own packed image (B operands as 16-byte tuples, the ragged slab padded), no counters
+        const int threads = (int)(n / 8) * 16 + 3 * 512 / 4;
+        hipLaunchKernelGGL(pack_x_tuples_kernel, dim3((threads + 255) / 256), dim3(256), 0, s, reinterpret_cast<const uint4 *>(x), sc.xpack,
+                           (int)n, (int)batch);
+        if (S == 6 && carry_mode == RPTC_AS_WRITTEN) launch_matmul_rows<6, RPTC_AS_WRITTEN>(a_comp, a_cb, sc.xpack, out, (int)m, (int)n, (int)batch, dev->cus, s);
+        if (S == 6 && carry_mode == RPTC_CONTINUOUS) launch_matmul_rows<6, RPTC_CONTINUOUS>(a_comp, a_cb, sc.xpack, out, (int)m, (int)n, (int)batch, dev->cus, s);
+        if (S == 8 && carry_mode == RPTC_AS_WRITTEN) launch_matmul_rows<8, RPTC_AS_WRITTEN>(a_comp, a_cb, sc.xpack, out, (int)m, (int)n, (int)batch, dev->cus, s);
+        if (S == 8 && carry_mode == RPTC_CONTINUOUS) launch_matmul_rows<8, RPTC_CONTINUOUS>(a_comp, a_cb, sc.xpack, out, (int)m, (int)n, (int)batch, dev->cus, s);
+        return t.end();
+    }
+#endif
     const int total = p.planes * (int)(n / 8) * 16;
     const int pack_threads = total > p.counters ? total : p.counters;
     hipLaunchKernelGGL(pack_x_kernel, dim3((pack_threads + 255) / 256), dim3(256), 0, s, reinterpret_cast<const uint4 *>(x), sc.xpack, sc.arrived,

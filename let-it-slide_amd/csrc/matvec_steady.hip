@@ -33,7 +33,6 @@ constexpr int kStPartBytes = 16384;                        // one set of partial
 constexpr int kStPartBase = kStTableBytes + 2 * kStImageBytes;
 constexpr int kStLdsBytes = kStPartBase + 2 * kStPartBytes;
 static_assert(kStLdsBytes == kMaxLds, "the layout fills the LDS of a CU");
-constexpr int kStRowWaves = 8;
 
 // ---- registers with fixed numbers: a request's 16 bytes are four consecutive registers, and an asm operand cannot
 // name one register of a tuple

@@ -361,6 +361,40 @@ def test_batched_kernel_matches_the_oracle(matmul_isa, oracle, m, n, batch, S, m
     assert err < 2e-3
 
 
+@pytest.mark.parametrize("m,n,batch,S,mode,tiles", [(16, 2048 + 768, 16, 8, 0, 1), (40, 4096 + 64 * 5, 5, 6, 1, 3), (30, 64 * 3, 16, 8, 1, 2),
+                                                        (48, 2048 * 3, 9, 8, 0, 1), (20, 2048 + 64 * 30, 3, 6, 0, 2)])
+def test_row_owner_batched_kernel_matches_the_oracle(matmul_isa, oracle, m, n, batch, S, mode, tiles):
+    """`pack_x_tuples_kernel` and `matmul_rows_kernel<S, MODE, TILES>` (`csrc/matmul.hip`): the activations packed as the
+    16-byte B operands of the MFMAs with a ragged slab padded by zeros, one workgroup per `tiles` blocks of 16 rows over
+    the whole width, a wave's accumulators running over its (slab, four lanes-of-row) pairs.  Ragged widths that are and
+    are not a multiple of four lanes-of-row, fewer pairs than waves, more than two pairs a wave, rows past m."""
+    rng = np.random.default_rng(m + n + batch)
+    codebook = (rng.standard_normal(2 << S) * 0.1).astype(np.float16)
+    stream = rng.integers(0, 256, m * n // 4, dtype=np.uint8)
+    x = (rng.standard_normal((batch, n)) * 0.5).astype(np.float16)
+    out = np.full((batch, m), np.nan, dtype=np.float16)
+    T, Lt = n // 2048, n % 2048 // 64
+    xpack = np.full((32 * T + (Lt + 3) // 4 * 4) * 512, 0x7E007E00, dtype=np.uint32)        # NaNs wherever nothing is written
+    mem = wave_model.Memory()
+    c_at, cb_at, x_at, o_at, xp_at = 0x7f40fffff000, 0x7f5000003400, 0x7f3ffff0fe00, 0x7f2ffffe0100, 0x7f6000000000
+    for at, data, name in ((c_at, stream, "stream"), (cb_at, codebook.view(np.uint8).copy(), "codebook"),
+                           (x_at, x.view(np.uint8).reshape(-1).copy(), "activations"), (o_at, out.view(np.uint8).reshape(-1), "output"),
+                           (xp_at, xpack.view(np.uint8), "packed activations")):
+        mem.add(at, data, name)
+    wave_model.Wave.vm_latency, wave_model.Wave.lgkm_latency = 400, 60
+    pack = wave_model.Kernel(matmul_isa, "_ZN4rptc20pack_x_tuples_kernelE")
+    pack.launch(mem, (((n // 8) * 16 + 384 + 255) // 256,), 256, [("ptr", x_at), ("ptr", xp_at), ("i32", n), ("i32", batch)], seed=m)
+    mem.regions = [r for r in mem.regions if r[2] != "kernarg"]
+    kernel = wave_model.Kernel(matmul_isa, "_ZN4rptc18matmul_rows_kernelILi%dELi%dELi%dEE" % (S, mode, tiles))
+    total = (m + 15) // 16
+    kernel.launch(mem, (-(-total // tiles),), 1024,
+                  [("ptr", c_at), ("ptr", cb_at), ("ptr", xp_at), ("ptr", o_at), ("i32", m), ("i32", n), ("i32", batch)],
+                  lds_bytes=65536 + 16 * tiles * 1024, seed=m)
+    want = np.stack([oracle.matvec(stream.view(np.uint32), codebook, x[b], m, S, mode=mode) for b in range(batch)])
+    err = np.abs(out.astype(np.float64) - want).max() / (np.abs(want).max() + 1e-9)
+    assert err < 2e-3
+
+
 @pytest.mark.parametrize("batch,n,block,inverse,misalign", [(2, 512, 256, 0, 0), (1, 1024, 1024, 1, 0), (3, 192, 64, 0, 2), (1, 12, 4, 1, 0),
                                                             (1, 2048 + 512, 512, 0, 0)])
 def test_sign_hadamard_kernel_matches_the_oracle(hadamard_isa, oracle, batch, n, block, inverse, misalign):

@@ -1061,6 +1061,18 @@ class Wave:
             sel = np.array([(selm >> k) & 1 for k in range(64)], dtype=bool)
             a, b = pick(V(o[1]), mods.get("src0_sel", "DWORD")), pick(V(o[2]), mods.get("src1_sel", "DWORD"))
             self.wv(o[0], np.where(sel, b, a).astype(U32))
+        elif op == "v_lshlrev_b32_sdwa":
+            # dst = src1 << src0[4:0], each source after its sub-dword select (zero-extended); whole destination written
+            def pick(val, how):
+                if how == "DWORD":
+                    return val.astype(np.uint64)
+                kind, idx = how.split("_")
+                width = 16 if kind == "WORD" else 8
+                return (val.astype(np.uint64) >> np.uint64(width * int(idx))) & np.uint64((1 << width) - 1)
+            if mods.get("dst_sel", "DWORD") != "DWORD" or mods.get("dst_unused", "UNUSED_PAD") != "UNUSED_PAD" or "sext" in text:
+                raise Fault(f"operand selects of {op} not modelled ({self.who()})")
+            count, val = pick(V(o[1]), mods.get("src0_sel", "DWORD")), pick(V(o[2]), mods.get("src1_sel", "DWORD"))
+            self.wv(o[0], ((val << (count & np.uint64(31))) & np.uint64(0xFFFFFFFF)).astype(U32))
         # ---------------------------------------------------------------- LDS
         elif op == "ds_read_b32":
             addr = V(o[1]).astype(np.int64) + int(mods.get("offset", "0"), 0)
