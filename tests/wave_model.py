@@ -1142,7 +1142,11 @@ class Wave:
                         self.lds_write32(int(addr[k]) + o1, int(d1[k]), who)
             self.lgq.append((self.tick, fn))
         # ---------------------------------------------------------------- global memory
-        elif op in ("global_load_dwordx4", "global_load_dword", "global_load_dwordx2", "global_load_dwordx3"):
+        elif op in ("global_load_dwordx4", "global_load_dword", "global_load_dwordx2", "global_load_dwordx3",
+                    "flat_load_dwordx4", "flat_load_dword", "flat_load_dwordx2", "flat_load_dwordx3"):
+            # a flat load whose address is in global memory is a global load that counts in both counters
+            if op.startswith("flat_"):
+                self.lgq.append((self.tick, lambda: None))
             n = {"4": 4, "2": 2, "3": 3}.get(op[-1], 1)
             addr = self.global_addr(o[1], o[2] if len(o) > 2 else "off", mods)
             dst, m, who = o[0], self.lanes().copy(), self.who()
