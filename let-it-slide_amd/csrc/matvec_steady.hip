@@ -78,6 +78,13 @@ static_assert(kStLdsBytes == kMaxLds, "the layout fills the LDS of a CU");
 // (slots hi, lo) sit side by side, pair 4 j + i in v[96 + 8 j + 2 i : +1] for shift group j and window register i
 #define ST_XP(J, I) "v[96+8*" #J "+2*" #I ":96+8*" #J "+2*" #I "+1]"
 #endif
+// a wave's priority at the instruction arbiter: highest in front of its first element and in the rows, lower with
+// every element it has behind it, so that the waves of a SIMD drift apart instead of queueing at the same unit
+#ifndef ST_NOPRIO
+#define ST_PRIO(X) "s_setprio " X "\n"
+#else
+#define ST_PRIO(X) ""
+#endif
 #define ST_STR2(x) #x
 #define ST_STR(x) ST_STR2(x)
 
@@ -158,6 +165,49 @@ static_assert(kStLdsBytes == kMaxLds, "the layout fills the LDS of a CU");
     "v_dot2c_f32_f16 %[a3], %[" T "7], " XH "\n"
 // OWN: what a row's first lane takes for the 16 bits in front of its element (its own last word as written,
 // inference.cu:232; the word in front of the row, or zero in slab 0, in continuous mode); FIRST: the lanes that start a row
+#ifdef ST_ROLL
+// The same work as a rolling pipeline: sixteen gathers stay in flight; a step waits for the oldest two, forms their two
+// products and puts the next window register's two gathers in their place, so a gather has eight steps' time to return
+// instead of the time of one group of eight.
+#define ST_STEP_FIRST(G, TH, TL, AH, AL, XH, XL)              \
+    "s_waitcnt lgkmcnt(14)\n"                                 \
+    "v_dot2_f32_f16 " AH ", " TH ", " XH ", 0\n"              \
+    "v_dot2_f32_f16 " AL ", " TL ", " XL ", 0\n"              \
+    ST_RDPAIR(G, TH, TL)
+#define ST_STEP(G, TH, TL, AH, AL, XH, XL)                    \
+    "s_waitcnt lgkmcnt(14)\n"                                 \
+    "v_dot2c_f32_f16 " AH ", " TH ", " XH "\n"                \
+    "v_dot2c_f32_f16 " AL ", " TL ", " XL "\n"                \
+    ST_RDPAIR(G, TH, TL)
+#define ST_DRAIN(N, TH, TL, AH, AL, XH, XL)                   \
+    "s_waitcnt lgkmcnt(" #N ")\n"                             \
+    "v_dot2c_f32_f16 " AH ", " TH ", " XH "\n"                \
+    "v_dot2c_f32_f16 " AL ", " TL ", " XL "\n"
+#define ST_DECODE(EX, EY, EZ, EW, OWN, FIRST)                                                                         \
+    "s_nop 1\n"                                                                                                       \
+    "s_mov_b64 vcc, " FIRST "\n"                                                                                      \
+    "v_cndmask_b32_dpp %[cy], " EW ", " OWN ", vcc wave_shr:1 row_mask:0xf bank_mask:0xf bound_ctrl:1\n"              \
+    ST_WINDOWS(12, EX, EY, EZ, EW) ST_READS_A                                                                         \
+    ST_WINDOWS(8, EX, EY, EZ, EW) ST_READS_B                                                                          \
+    ST_WINDOWS(4, EX, EY, EZ, EW)                                                                                     \
+    ST_STEP_FIRST("%[g0]", "%[t0]", "%[t1]", "%[a0]", "%[a1]", ST_X28, ST_X0)                                         \
+    ST_STEP_FIRST("%[g1]", "%[t2]", "%[t3]", "%[a2]", "%[a3]", ST_X16, ST_X4)                                         \
+    ST_STEP("%[g2]", "%[t4]", "%[t5]", "%[a0]", "%[a1]", ST_X20, ST_X8)                                               \
+    ST_STEP("%[g3]", "%[t6]", "%[t7]", "%[a2]", "%[a3]", ST_X24, ST_X12)                                              \
+    ST_WINDOWS0(EX, EY, EZ, EW)                                                                                       \
+    ST_STEP("%[g0]", "%[u0]", "%[u1]", "%[a0]", "%[a1]", ST_X29, ST_X1)                                               \
+    ST_STEP("%[g1]", "%[u2]", "%[u3]", "%[a2]", "%[a3]", ST_X17, ST_X5)                                               \
+    ST_STEP("%[g2]", "%[u4]", "%[u5]", "%[a0]", "%[a1]", ST_X21, ST_X9)                                               \
+    ST_STEP("%[g3]", "%[u6]", "%[u7]", "%[a2]", "%[a3]", ST_X25, ST_X13)                                              \
+    ST_DRAIN(14, "%[t0]", "%[t1]", "%[a0]", "%[a1]", ST_X30, ST_X2)                                                   \
+    ST_DRAIN(12, "%[t2]", "%[t3]", "%[a2]", "%[a3]", ST_X18, ST_X6)                                                   \
+    ST_DRAIN(10, "%[t4]", "%[t5]", "%[a0]", "%[a1]", ST_X22, ST_X10)                                                  \
+    ST_DRAIN(8, "%[t6]", "%[t7]", "%[a2]", "%[a3]", ST_X26, ST_X14)                                                   \
+    ST_DRAIN(6, "%[u0]", "%[u1]", "%[a0]", "%[a1]", ST_X31, ST_X3)                                                    \
+    ST_DRAIN(4, "%[u2]", "%[u3]", "%[a2]", "%[a3]", ST_X19, ST_X7)                                                    \
+    ST_DRAIN(2, "%[u4]", "%[u5]", "%[a0]", "%[a1]", ST_X23, ST_X11)                                                   \
+    ST_DRAIN(0, "%[u6]", "%[u7]", "%[a2]", "%[a3]", ST_X27, ST_X15)
+#else
 #define ST_DECODE(EX, EY, EZ, EW, OWN, FIRST)                                                                         \
     /* a DPP operand must not have been written by a vector op in the two instructions before */                     \
     "s_nop 1\n"                                                                                                       \
@@ -175,6 +225,7 @@ static_assert(kStLdsBytes == kMaxLds, "the layout fills the LDS of a CU");
     ST_DOTS("t", ST_X30, ST_X2, ST_X18, ST_X6, ST_X22, ST_X10, ST_X26, ST_X14)                                        \
     "s_waitcnt lgkmcnt(0)\n"                                                                                          \
     ST_DOTS("u", ST_X31, ST_X3, ST_X19, ST_X7, ST_X23, ST_X11, ST_X27, ST_X15)
+#endif
 
 #else
 // The products on the matrix unit: v_mfma_f32_4x4x4_16b_f16 multiplies, in every group of four lanes, the 4 x 4 matrix
@@ -252,7 +303,7 @@ static_assert(kStLdsBytes == kMaxLds, "the layout fills the LDS of a CU");
 #define ST_ITEM_HEAD(U, P, NEED)                                                                                      \
     "s_cmp_le_u32 %[nitems], " #U "\n"                                                                                \
     "s_cbranch_scc1 7" #U "f\n"                                                                                       \
-    "s_setprio 3-" #U "\n"                                                                                            \
+    ST_PRIO("3-" #U)                                                                                                  \
     "s_bitcmp1_b32 %[rl], " #U "\n"                                                                                   \
     "s_cbranch_scc0 5" #U "f\n"                                                                                       \
     ST_RELOAD("%[xa" #U "]", P)                                                                                       \
@@ -389,7 +440,7 @@ static_assert(kStLdsBytes == kMaxLds, "the layout fills the LDS of a CU");
 #define ST_LAYER(P, Q, MODE, M, NEED, STW, LPI)                                                                       \
     ST_XREQUESTS                                                                                                      \
     ST_ITEMS_##M(MODE, P, Q, NEED, LPI)                                                                               \
-    "s_setprio 3\n"                                                                                                   \
+    ST_PRIO("3")                                                                                                      \
     "s_cmp_eq_u32 %[k], 0\n"                                                                                          \
     "s_cbranch_scc1 93f\n"                                                                                            \
     ST_ROWS(Q)                                                                                                        \
@@ -404,7 +455,7 @@ static_assert(kStLdsBytes == kMaxLds, "the layout fills the LDS of a CU");
 #define ST_LAST_LAYER(P, Q, MODE, M)                                                                                  \
     "s_waitcnt vmcnt(0)\n"                                                                                            \
     ST_LAST_ITEMS_##M(MODE, P)                                                                                        \
-    "s_setprio 3\n"                                                                                                   \
+    ST_PRIO("3")                                                                                                      \
     "s_cmp_eq_u32 %[k], 0\n"                                                                                          \
     "s_cbranch_scc1 93f\n"                                                                                            \
     ST_ROWS(Q)                                                                                                        \

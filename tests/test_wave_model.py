@@ -528,3 +528,14 @@ def steady_mfma_isa(tmp_path_factory):
 def test_steady_kernel_with_the_products_on_the_matrix_unit(steady_mfma_isa, oracle, m, n, count, S, mode):
     """The -DST_MFMA build of the same kernel (v_mfma_f32_4x4x4_16b_f16 in place of the two-term dot products)."""
     run_steady(steady_mfma_isa, oracle, m, n, count, S, mode, blocks=sorted({0, (m - 1) // (2 * ((m + 2 * CUS - 1) // (2 * CUS)))}))
+
+
+@pytest.fixture(scope="module")
+def steady_roll_isa(tmp_path_factory):
+    return compile_to_assembly(tmp_path_factory, "matvec_steady", extra=("-DST_ROLL",))
+
+
+@pytest.mark.parametrize("m,n,count,S,mode", [(33, 4096 + 768, 3, 8, 0), (300, 64, 2, 6, 1), (1024, 2048 + 64, 3, 8, 1), (8192, 8192, 2, 8, 0)])
+def test_steady_kernel_with_the_decode_as_a_rolling_pipeline(steady_roll_isa, oracle, m, n, count, S, mode):
+    """The -DST_ROLL build of the same kernel (sixteen gathers kept in flight, two products and two new gathers a step)."""
+    run_steady(steady_roll_isa, oracle, m, n, count, S, mode, blocks=sorted({0, (m - 1) // (2 * ((m + 2 * CUS - 1) // (2 * CUS)))}))
