@@ -367,6 +367,23 @@ int rptc_viterbi_scalar(const float *targets, const float *weights, int64_t weig
                         const uint16_t *alphabet, int L, void *scratch, uint8_t *symbols, int32_t *end_state,
                         float *cost, int64_t rows, int64_t steps, void *stream, float *ms);
 
+/*
+ * The search of the reference's rptc_lite.py (quantize, rptc_lite.py:19-60) for the trellis that
+ * rptc_lite_dequantize decodes: rho[0] = 0 at the start, per step the cheapest of the 2^R predecessors of every
+ * state (first index on ties, as argmin picks), plus sum_v importance[t][v] * (samples[t][v] - alphabet[index_fn(
+ * state)][v])^2 in fp32; the cheapest end state is traced back.  symbols[t] is the reference's `quantized[t]`,
+ * cost its `expected_loss`.  Built for the parameters the reference's own driver uses (rptc_lite.py:134-139):
+ * L = 16, R = 4, V = 2, and any S <= 9; other parameters return RPTC_ELIMIT.
+ *   samples     float [rows][steps][2]
+ *   importance  NULL (all ones), or float [.][steps][2]: row r reads importance + r * importance_row_stride
+ *               (0 = one set for all rows)
+ *   alphabet    float [2^S][2];  scratch rptc_viterbi_scratch_bytes(rows, steps) bytes of device memory
+ *   symbols     uint8 [rows][steps], values 0..15;  end_state int32 [rows];  cost float [rows]
+ */
+int rptc_lite_viterbi(const float *samples, const float *importance, int64_t importance_row_stride,
+                      const float *alphabet, int L, int S, int R, int V, void *scratch, uint8_t *symbols,
+                      int32_t *end_state, float *cost, int64_t rows, int64_t steps, void *stream, float *ms);
+
 #ifdef __cplusplus
 }
 #endif

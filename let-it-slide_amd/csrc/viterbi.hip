@@ -235,6 +235,129 @@ __global__ __launch_bounds__(kVitThreads) void viterbi_pairs_kernel(
     }
 }
 
+// The same search on the trellis of the reference's rptc_lite.py (quantize, rptc_lite.py:19-60) for L = 16, R = 4, V = 2,
+// the parameters its own driver uses (rptc_lite.py:134-139): state s' emits alphabet[index_fn(s')] (rptc_lite.py:12-16,27-29),
+// a row of an fp32 alphabet of 2^S pairs, S <= 9, and a step costs sum_v importance[t][v] * (samples[t][v] - value)^2
+// (rptc_lite.py:39).  Structure of viterbi_pairs_kernel<., 4, .>; what differs is the loss table: up to 512 distinct
+// values a step instead of 256, so a row has 16 copies a step parity (128 bytes a row, 64 KiB in all) and a gather meets
+// another lane's in the same bank about every second time; and a state's row number needs 9 bits, so the codes are 16-bit
+// halves (the row's byte offset, ready to be or-ed with the copy's offset), two a register.
+template <bool WEIGHTED>
+__global__ __launch_bounds__(kVitThreads) void viterbi_lite_kernel(
+    const float *__restrict__ targets, const float *__restrict__ weights, int64_t weights_row_stride,
+    const float *__restrict__ alphabet, int S, uint16_t *__restrict__ back, int32_t *__restrict__ end_state,
+    float *__restrict__ cost, int steps)
+{
+    extern __shared__ float lds[];
+    constexpr int kCopies = 16, kRow = 2 * kCopies;     // floats in a table row: 16 copies for even steps, 16 for odd
+    float *loss = lds;                                  // [512][2][16], at LDS address 0 (see viterbi_pairs_kernel)
+    float *best = lds + kVitLossFloats;                 // [2][4096]
+    float *red_v = best + 2 * kVitGroups;               // [1024]
+    int *red_i = reinterpret_cast<int *>(red_v + kVitThreads);
+    static_assert(512 * kRow == kVitLossFloats, "the table takes the room of the pair search's");
+
+    const int j = threadIdx.x, copy = j & (kCopies - 1);
+    const int64_t row = blockIdx.x;
+    const uint32_t loss_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(loss));
+
+    float rho[64];
+    uint32_t code[32];                                  // half r % 2 of code[r / 2]: 128 * index_fn(state of register r)
+#pragma unroll
+    for (int r = 0; r < 64; r++) {
+        const uint32_t st = vit_state<4>(r, j);
+        uint32_t x = st * (2u * st + 1u);               // index_fn: only bits below 16 reach the result when L = 16
+        x ^= x >> (16 - S);
+        const uint32_t c = (x & ((1u << S) - 1u)) * (kRow * 4u);
+        if (r & 1) code[r >> 1] |= c << 16;
+        else code[r >> 1] = c;
+        rho[r] = (st == 0) ? 0.f : INFINITY;
+    }
+    const uint32_t copy4 = loss_base + 4u * (uint32_t)copy;
+
+    // the table row this thread fills: two threads a row, 8 copies each
+    const int e_mine = (j >> 1) & ((1 << S) - 1);
+    const float w0 = alphabet[2 * e_mine], w1 = alphabet[2 * e_mine + 1];
+    float4 *loss_mine = reinterpret_cast<float4 *>(loss + e_mine * kRow + (j & 1) * 8);
+
+    const float *tg = targets + row * steps * 2;
+    const float *wt = WEIGHTED ? weights + row * weights_row_stride : nullptr;
+    uint16_t *back_row = back + row * steps * (int64_t)kVitThreads;
+    float x0 = tg[0], x1 = tg[1], c0 = WEIGHTED ? wt[0] : 1.f, c1 = WEIGHTED ? wt[1] : 1.f;
+    for (int t = 0; t < steps; t++) {
+        const int tn = t + 1 < steps ? t + 1 : t;
+        const float nx0 = tg[2 * tn], nx1 = tg[2 * tn + 1];
+        const float nc0 = WEIGHTED ? wt[2 * tn] : 1.f, nc1 = WEIGHTED ? wt[2 * tn + 1] : 1.f;
+
+        const float l = WEIGHTED ? pair_loss_weighted(x0, x1, w0, w1, c0, c1) : pair_loss(x0, x1, w0, w1);
+        const float4 l4 = make_float4(l, l, l, l);
+        float4 *lm = loss_mine + (t & 1) * (kCopies / 4);
+        lm[0] = l4;
+        lm[1] = l4;
+
+        float *bw = best + (t & 1) * kVitGroups;
+        const uint32_t copy4_t = copy4 + (uint32_t)(t & 1) * (kCopies * 4u);
+        auto loss_of = [&](int r) {
+            const uint32_t off = (r & 1) ? (code[r >> 1] >> 16) | copy4_t : and_or(code[r >> 1], 0xFFFFu, copy4_t);
+            return __builtin_bit_cast(float, lds_read_abs(off));
+        };
+        uint32_t nib = 0;
+#pragma unroll
+        for (int gi = 0; gi < 4; gi++) {
+            float m = rho[16 * gi];
+            uint32_t arg = 0;
+#pragma unroll
+            for (int d = 1; d < 16; d++) {
+                const bool lt = rho[16 * gi + d] < m;          // the first minimum wins (argmin, rptc_lite.py:34)
+                m = lt ? rho[16 * gi + d] : m;
+                arg = lt ? (uint32_t)d : arg;
+            }
+            bw[4 * j + gi] = m;
+            nib |= arg << (4 * gi);
+        }
+        back_row[(int64_t)t * kVitThreads + j] = (uint16_t)nib;
+        __syncthreads();
+#pragma unroll
+        for (int d = 0; d < 16; d++) {
+            const float b = bw[(d << 8) | (j >> 2)];
+#pragma unroll
+            for (int gi = 0; gi < 4; gi++) rho[16 * gi + d] = b + loss_of(16 * gi + d);
+            if ((d & 1) == 1) __builtin_amdgcn_sched_barrier(0);
+        }
+        x0 = nx0, x1 = nx1, c0 = nc0, c1 = nc1;
+    }
+
+    // cheapest end state, the lowest index among equals (argmin, rptc_lite.py:52)
+    float mv = rho[0];
+    int mi = (int)vit_state<4>(0, j);
+#pragma unroll
+    for (int a = 0; a < 64; a++) {
+        const int r = 16 * (a & 3) + (a >> 2);
+        const float v = rho[r];
+        if (v < mv) {
+            mv = v;
+            mi = (int)vit_state<4>(r, j);
+        }
+    }
+    red_v[j] = mv;
+    red_i[j] = mi;
+    __syncthreads();
+    for (int width = kVitThreads / 2; width > 0; width >>= 1) {
+        if (j < width) {
+            const float ov = red_v[j + width];
+            const int oi = red_i[j + width];
+            if (ov < red_v[j] || (ov == red_v[j] && oi < red_i[j])) {
+                red_v[j] = ov;
+                red_i[j] = oi;
+            }
+        }
+        __syncthreads();
+    }
+    if (j == 0) {
+        end_state[row] = red_i[0];
+        cost[row] = red_v[0];
+    }
+}
+
 // x - (fp16 in the low / high half of v) in one op: x * 1.0 + (-half), the product exact, so the
 // result is the correctly rounded difference.  Written as asm also because the conversion alone
 // does not change from step to step: the compiler would convert all values once and keep them as
@@ -434,6 +557,8 @@ int prepare_viterbi()
     RPTC_VIT_ALLOW(6)
     RPTC_VIT_ALLOW(8)
 #undef RPTC_VIT_ALLOW
+    if ((rc = vit_allow_lds(viterbi_lite_kernel<false>))) return rc;
+    if ((rc = vit_allow_lds(viterbi_lite_kernel<true>))) return rc;
     return 0;
 }
 
@@ -537,4 +662,34 @@ extern "C" int rptc_viterbi_pairs(const float *targets, const float *weights, in
 {
     return rptc_viterbi_pairs_bits(targets, weights, weights_row_stride, codebook, scratch, symbols, end_state, cost, rows,
                                    steps, S, 2, stream, ms);
+}
+
+
+extern "C" int rptc_lite_viterbi(const float *samples, const float *importance, int64_t importance_row_stride,
+                                 const float *alphabet, int L, int S, int R, int V, void *scratch, uint8_t *symbols,
+                                 int32_t *end_state, float *cost, int64_t rows, int64_t steps, void *stream, float *ms)
+{
+    if (!samples || !alphabet || !scratch || !symbols || !end_state || !cost) return RPTC_ENULL;
+    if (L < 1 || S < 1 || S > L || R < 1 || R > L || V < 1) return RPTC_ESHAPE;
+    if (L != 16 || R != 4 || V != 2 || S > 9) return RPTC_ELIMIT;          // the search kernel's trellis
+    if (rows < 1 || steps < 1 || importance_row_stride < 0) return RPTC_ESHAPE;
+    if (importance && importance_row_stride != 0 && importance_row_stride < 2 * steps) return RPTC_ESHAPE;
+    if (rows >= ((int64_t)1 << 24) || steps >= ((int64_t)1 << 24)) return RPTC_ELIMIT;
+    DeviceInfo *dev;
+    int rc = device_info(&dev);
+    if (rc) return rc;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    Timer t;
+    rc = t.begin(dev, s, ms);
+    if (rc) return rc;
+    uint16_t *back = static_cast<uint16_t *>(scratch);
+    if (importance)
+        hipLaunchKernelGGL(viterbi_lite_kernel<true>, dim3((unsigned)rows), dim3(kVitThreads), kVitLdsBytes, s, samples, importance,
+                           importance_row_stride, alphabet, S, back, end_state, cost, (int)steps);
+    else
+        hipLaunchKernelGGL(viterbi_lite_kernel<false>, dim3((unsigned)rows), dim3(kVitThreads), kVitLdsBytes, s, samples, importance,
+                           importance_row_stride, alphabet, S, back, end_state, cost, (int)steps);
+    hipLaunchKernelGGL(viterbi_trace_kernel<4>, dim3((unsigned)((rows + 63) / 64)), dim3(64), 0, s, back, end_state, symbols, (int)rows,
+                       (int)steps);
+    return t.end();
 }

@@ -27,7 +27,8 @@ the matrix cores), ``decompress_matvec_bits`` (2, 3, 4 bits per weight), ``decom
 ``decompress_matvec_affine`` / ``_silu_affine`` / ``_rmsnorm_affine`` (with the row/column scales and biases of
 the reference's factorisation, quantize_hf.py:167, applied inside the kernel),
 ``sign_hadamard``, ``viterbi_pairs`` and ``viterbi_scalar`` (the quantizer's trellis search, rptc.py:13-71,
-as kernels: for the hashed pair stream and for the reference's own scalar trellis).
+as kernels: for the hashed pair stream and for the reference's own scalar trellis), ``lite_dequantize`` and
+``lite_quantize`` (rptc_lite.py's decoder and search).
 Sub-modules: ``packing`` (symbols -> streams), ``quantize`` (the quantizer around that search),
 ``linear`` (``QuantizedLinear``, ``patch_model``), ``llama_decode`` (a Llama-shaped decode loop),
 ``eval_ppl`` (perplexity on a token file).
@@ -91,6 +92,7 @@ _SIGNATURES = {
     "rptc_viterbi_scalar_scratch_bytes": ([_I64, _I64], _I64),
     "rptc_viterbi_scalar": ([_VP, _VP, _I64, _VP, _INT, _VP, _VP, _VP, _VP, _I64, _I64, _VP, _FP], _INT),
     "rptc_viterbi_pairs": ([_VP, _VP, _I64, _VP, _VP, _VP, _VP, _VP, _I64, _I64, _INT, _VP, _FP], _INT),
+    "rptc_lite_viterbi": ([_VP, _VP, _I64, _VP, _INT, _INT, _INT, _INT, _VP, _VP, _VP, _VP, _I64, _I64, _VP, _FP], _INT),
     "rptc_viterbi_pairs_bits": ([_VP, _VP, _I64, _VP, _VP, _VP, _VP, _VP, _I64, _I64, _INT, _INT, _VP, _FP], _INT),
     "rptc_lite_dequantize": ([_VP, _INT, _INT, _INT, _INT, _VP, _I64, _I64, _VP, _VP, _FP], _INT),
     "rptc_sign_hadamard": ([_VP, _VP, _VP, _I64, _I64, _I64, _INT, _VP, _FP], _INT),
@@ -436,6 +438,49 @@ def lite_dequantize(alphabet, L, S, R, quantized, timed=None):
                                             ctypes.c_void_p(stream), ctypes.byref(ms) if (_timing if timed is None else timed) else None)
     _status(rc)
     return out, float(ms.value)
+
+
+def lite_quantize(alphabet, L, S, R, importance, samples):
+    """``rptc_lite.quantize(alphabet, L, S, R, importance, samples)`` (rptc_lite.py:19-60): the symbol sequence whose
+    ``lite_dequantize`` is closest to ``samples`` under the per-value ``importance``, by exact Viterbi search.
+
+    alphabet: float32 [2^S, 2]; samples, importance: float32 [length, 2], or [rows, length, 2] with every row a sequence
+    of its own (importance may be None for all ones, or [length, 2] for one set shared by all rows).  Built for
+    L = 16, R = 4, V = 2, S <= 9 (the parameters of the reference's own driver); other parameters raise.
+    Returns (quantized int32 [length] or [rows, length], expected_loss float32 scalar or [rows])."""
+    _check_input(alphabet, "alphabet")
+    _check_input(samples, "samples")
+    _check(alphabet.dtype == torch.float32 and alphabet.dim() == 2, "alphabet must be float32 [2^S, V]")
+    _check(samples.dtype == torch.float32 and samples.dim() in (2, 3), "samples must be float32 [length, V] or [rows, length, V]")
+    _check(1 <= S <= L and 1 <= R <= L, "1 <= S <= L and 1 <= R <= L")
+    _check(alphabet.size(0) == 1 << S, "alphabet.size(0) == 1 << S")
+    V = alphabet.size(1)
+    _check(samples.size(-1) == V, "samples.size(-1) == alphabet.size(1)")
+    single = samples.dim() == 2
+    rows, steps = (1, samples.size(0)) if single else (samples.size(0), samples.size(1))
+    _check(rows >= 1 and steps >= 1, "rows >= 1 and length >= 1")
+    stride = 0
+    if importance is not None:
+        _check_input(importance, "importance")
+        _check(importance.dtype == torch.float32, "importance must be float32")
+        _check(tuple(importance.shape) in ((steps, V), (rows, steps, V)), "importance must have the shape of samples, or [length, V]")
+        stride = 0 if importance.dim() == 2 else V * steps
+    device = samples.device
+    _check(alphabet.device == device, "all tensors must be on the same device")
+    lib = library()
+    with torch.cuda.device(device):
+        scratch = torch.empty(max(lib.rptc_viterbi_scratch_bytes(rows, steps), 16), dtype=torch.uint8, device=device)
+        symbols = torch.empty((rows, steps), dtype=torch.uint8, device=device)
+        end_state = torch.empty(rows, dtype=torch.int32, device=device)
+        cost = torch.empty(rows, dtype=torch.float32, device=device)
+        stream = torch.cuda.current_stream().cuda_stream
+        rc = lib.rptc_lite_viterbi(samples.data_ptr(), importance.data_ptr() if importance is not None else None, stride,
+                                   alphabet.data_ptr(), L, S, R, V, scratch.data_ptr(), symbols.data_ptr(), end_state.data_ptr(),
+                                   cost.data_ptr(), rows, steps, ctypes.c_void_p(stream), None)
+        _status(rc)
+        torch.cuda.current_stream().synchronize()     # scratch is freed on return
+    quantized = symbols.to(torch.int32)
+    return (quantized[0], cost[0]) if single else (quantized, cost)
 
 
 def viterbi_pairs(targets, codebook, weights=None, bits=2):

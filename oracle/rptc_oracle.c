@@ -34,6 +34,9 @@
  *                         (bits above L never reach the index: tested), so the
  *                         output equals alphabet[index of the last L stream
  *                         bits] over sequences that wrap the register
+ *   (lite_quantize of rptc_oracle.py = orc_viterbi over the table alphabet[orc_lite_index_fn(state)]: every symbol
+ *                         sequence of small trellises decoded by orc_lite_dequantize, none cheaper than the returned
+ *                         cost and the returned sequence has that cost)
  *   orc_viterbi           exhaustive enumeration of every symbol sequence on
  *                         trellises small enough for it (optimal cost, and the
  *                         returned path has that cost); the tie rules are

@@ -208,6 +208,18 @@ def lite_dequantize(alphabet, L, S, R, symbols):
     return out
 
 
+def lite_quantize(alphabet, L, S, R, importance, samples):
+    """rptc_lite.py:19-60: the search over the 2^L states whose values are alphabet[index_fn(state)] (the reference's
+    `permuted_alphabet`, rptc_lite.py:27-29), R stream bits a step, cost sum_v importance * (samples - value)^2
+    (rptc_lite.py:39); orc_viterbi is the same recursion and trace back (its tie rules are argmin's first index, as
+    rptc_lite.py:34,52 use it).  alphabet float32 [2^S, V]; samples float32 [length, V]; importance the same shape or
+    None (all ones).  Returns (quantized int32 [length], expected_loss float32)."""
+    alphabet = np.ascontiguousarray(alphabet, dtype=np.float32)
+    table = alphabet[[lite_index_fn(s, L, S) for s in range(1 << L)]]
+    symbols, cost, _ = viterbi(table, R, samples, importance)
+    return symbols, cost
+
+
 def dense_matvec(W, x):
     """float64 y = W x from float16 W [m, n] and x [n] or [B, n]."""
     Wb = _u16(W)

@@ -411,6 +411,47 @@ def test_lite_dequantize_window(oracle):
         assert np.array_equal(got[t], alphabet[_index_fn_python(state, L, S)])
 
 
+# ------------------------------------------------------------------ rptc_lite.py:19-60 (the search)
+
+@pytest.mark.parametrize("L,S,R,V,steps,weighted", [(6, 3, 2, 2, 5, False), (6, 4, 3, 2, 4, True), (4, 2, 1, 1, 9, True), (8, 5, 4, 2, 3, False),
+                                                     (5, 5, 2, 3, 5, True)])
+def test_lite_quantize_finds_the_cheapest_sequence(oracle, L, S, R, V, steps, weighted):
+    """Every symbol sequence of a small trellis, decoded by the decoder's own restatement (rptc_lite.py:63-73) and priced
+    as rptc_lite.py:39 prices a step: none is cheaper than what the search returns, the returned sequence has that price,
+    and among the cheapest sequences it is the one the recursion's first-index tie rule picks whenever the optimum is
+    unique (random floats: it is)."""
+    import itertools
+    g = rng(100 * L + steps)
+    alphabet = g.standard_normal((1 << S, V)).astype(np.float32)
+    samples = g.standard_normal((steps, V)).astype(np.float32)
+    importance = (g.random((steps, V)) + 0.25).astype(np.float32) if weighted else None
+    got, cost = oracle.lite_quantize(alphabet, L, S, R, importance, samples)
+    w = importance if weighted else np.ones((steps, V), dtype=np.float32)
+
+    def price(seq):
+        out = oracle.lite_dequantize(alphabet, L, S, R, np.array(seq, dtype=np.int32))
+        return float((w.astype(np.float64) * (samples.astype(np.float64) - out) ** 2).sum())
+    prices = {seq: price(seq) for seq in itertools.product(range(1 << R), repeat=steps)}
+    best = min(prices, key=prices.get)
+    assert abs(prices[best] - float(cost)) <= 1e-5 * max(1.0, prices[best])
+    assert abs(price(tuple(int(v) for v in got)) - float(cost)) <= 1e-5 * max(1.0, float(cost))
+    ranked = sorted(prices.values())
+    if ranked[1] - ranked[0] > 1e-4:
+        assert tuple(int(v) for v in got) == best
+
+
+def test_lite_quantize_starts_from_state_zero_and_breaks_ties_low(oracle):
+    """rho[0] = 0 and infinity elsewhere at the start (rptc_lite.py:42-43): the first symbols shift into a zero register.
+    With an alphabet of equal rows every sequence costs the same; argmin's first index (rptc_lite.py:34 for a step,
+    :52 for the end state) then gives the all-zero sequence."""
+    L, S, R, V = 6, 3, 2, 2
+    alphabet = np.full((1 << S, V), 0.5, dtype=np.float32)
+    samples = rng(5).standard_normal((7, V)).astype(np.float32)
+    got, cost = oracle.lite_quantize(alphabet, L, S, R, None, samples)
+    assert not got.any()
+    assert abs(float(cost) - float(((samples - 0.5) ** 2).sum())) < 1e-4
+
+
 # ------------------------------------------------------------------ sign-Hadamard transform (no reference counterpart)
 
 @pytest.mark.parametrize("P", [2, 64, 256, 1024])

@@ -539,3 +539,48 @@ def steady_roll_isa(tmp_path_factory):
 def test_steady_kernel_with_the_decode_as_a_rolling_pipeline(steady_roll_isa, oracle, m, n, count, S, mode):
     """The -DST_ROLL build of the same kernel (sixteen gathers kept in flight, two products and two new gathers a step)."""
     run_steady(steady_roll_isa, oracle, m, n, count, S, mode, blocks=sorted({0, (m - 1) // (2 * ((m + 2 * CUS - 1) // (2 * CUS)))}))
+
+
+@pytest.fixture(scope="module")
+def viterbi_isa(tmp_path_factory):
+    return compile_to_assembly(tmp_path_factory, "viterbi")
+
+
+@pytest.mark.parametrize("S,steps,weighted", [(9, 3, False), (7, 2, True)])
+def test_lite_search_kernel_matches_the_oracle(viterbi_isa, oracle, S, steps, weighted):
+    """`viterbi_lite_kernel` and `viterbi_trace_kernel<4>` as `rptc_lite_viterbi` launches them (`csrc/viterbi.hip`): a few
+    steps of the search over the 65536 states of rptc_lite.py's trellis at L = 16, R = 4, V = 2 against the oracle's
+    `lite_quantize`: the same symbols, end state and cost to the bit (every sum is fp32 in the same order)."""
+    rng = np.random.default_rng(S + steps)
+    alphabet = rng.standard_normal((1 << S, 2)).astype(np.float32)
+    samples = rng.standard_normal((steps, 2)).astype(np.float32)
+    importance = (rng.random((steps, 2)) + 0.25).astype(np.float32) if weighted else None
+    back = np.full(steps * 1024, 0xABCD, dtype=np.uint16)
+    symbols = np.full(steps, 0xEE, dtype=np.uint8)
+    end_state = np.full(1, -1, dtype=np.int32)
+    cost = np.full(1, np.nan, dtype=np.float32)
+    mem = wave_model.Memory()
+    t_at, w_at, a_at, b_at, s_at, e_at, c_at = (0x7f4000000000, 0x7f4100000000, 0x7f4200000000, 0x7f4300000000, 0x7f4400000000,
+                                                0x7f4500000000, 0x7f4600000000)
+    mem.add(t_at, samples.view(np.uint8).reshape(-1).copy(), "samples")
+    if weighted:
+        mem.add(w_at, importance.view(np.uint8).reshape(-1).copy(), "importance")
+    mem.add(a_at, alphabet.view(np.uint8).reshape(-1).copy(), "alphabet")
+    mem.add(b_at, back.view(np.uint8), "back pointers")
+    mem.add(s_at, symbols, "symbols")
+    mem.add(e_at, end_state.view(np.uint8), "end state")
+    mem.add(c_at, cost.view(np.uint8), "cost")
+    wave_model.Wave.vm_latency, wave_model.Wave.lgkm_latency = 400, 60
+    search = wave_model.Kernel(viterbi_isa, "_ZN4rptc19viterbi_lite_kernelILb%dEE" % (1 if weighted else 0))
+    search.launch(mem, (1,), 1024, [("ptr", t_at), ("ptr", w_at if weighted else 0), ("i64", 0), ("ptr", a_at), ("i32", S), ("ptr", b_at),
+                                    ("ptr", e_at), ("ptr", c_at), ("i32", steps)], lds_bytes=(256 * 64 + 2 * 4096) * 4 + 2 * 1024 * 4, seed=S)
+    mem.regions = [r for r in mem.regions if r[2] != "kernarg"]
+    trace = wave_model.Kernel(viterbi_isa, "_ZN4rptc20viterbi_trace_kernelILi4EE")
+    trace.launch(mem, (1,), 64, [("ptr", b_at), ("ptr", e_at), ("ptr", s_at), ("i32", 1), ("i32", steps)], seed=S)
+    want_symbols, want_cost = oracle.lite_quantize(alphabet, 16, S, 4, importance, samples)
+    assert np.array_equal(symbols.astype(np.int32), want_symbols)
+    assert cost.view(np.uint32)[0] == np.float32(want_cost).view(np.uint32)
+    state = 0
+    for v in want_symbols:
+        state = ((state << 4) | int(v)) & 0xFFFF
+    assert int(end_state[0]) == state

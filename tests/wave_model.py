@@ -634,9 +634,10 @@ class Wave:
             r = a & b if op == "s_and_b32" else (a | b if op == "s_or_b32" else a ^ b)
             setscc(r != 0)
             self.ws(o[0], r, 1)
-        elif op in ("s_and_b64", "s_or_b64", "s_xor_b64", "s_andn2_b64"):
+        elif op in ("s_and_b64", "s_or_b64", "s_xor_b64", "s_andn2_b64", "s_orn2_b64"):
             a, b = S(o[1], 2), S(o[2], 2)
-            r = {"s_and_b64": a & b, "s_or_b64": a | b, "s_xor_b64": a ^ b, "s_andn2_b64": a & ~b & MASK64}[op]
+            r = {"s_and_b64": a & b, "s_or_b64": a | b, "s_xor_b64": a ^ b, "s_andn2_b64": a & ~b & MASK64,
+                 "s_orn2_b64": (a | ~b) & MASK64}[op]
             setscc(r != 0)
             self.ws(o[0], r, 2)
         elif op == "s_and_saveexec_b64":
@@ -833,6 +834,22 @@ class Wave:
             self.vcc = newvcc
         elif op == "v_or3_b32":
             self.wv(o[0], V(o[1]) | V(o[2]) | V(o[3]))
+        elif op in ("v_bitop3_b32", "v_bitop3_b16"):
+            # every result bit is the truth table's entry for the three source bits (source 0 the most significant of the
+            # index).  The 16-bit form is taken to write the low half and keep the high one; a use of the high half of
+            # its result would show which the hardware does, and none is modelled.
+            if "op_sel" in mods:
+                raise Fault(f"operand selects of {op} not modelled ({self.who()})")
+            tt = int(mods["bitop3"], 0)
+            a, b, c = V(o[1]), V(o[2]), V(o[3])
+            r = np.zeros(64, dtype=U32)
+            for idx in range(8):
+                if (tt >> idx) & 1:
+                    r |= (a if idx & 4 else ~a) & (b if idx & 2 else ~b) & (c if idx & 1 else ~c)
+            if op.endswith("b16"):
+                i, _ = self.vreg_index(o[0])
+                r = (r & U32(0xFFFF)) | (self.v[i] & U32(0xFFFF0000))
+            self.wv(o[0], r)
         elif op == "v_mfma_f32_16x16x32_f16":
             # D[16 x 16] = A[16 x 32] B[32 x 16] + C, fp32.  Lane l = 16 g + i holds A[i][8 g .. 8 g + 7] (four registers of two
             # halves) and, with j for i, B[8 g .. 8 g + 7][j]; register r of lane l = 16 q + j holds C and D [4 q + r][j].
@@ -1039,7 +1056,13 @@ class Wave:
             else:
                 A, B = A.astype(np.int64), B.astype(np.int64)
             with np.errstate(all="ignore"):
-                c = {"eq": A == B, "ne": A != B, "gt": A > B, "ge": A >= B, "lt": A < B, "le": A <= B}[kind]
+                table = {"eq": A == B, "ne": A != B, "gt": A > B, "ge": A >= B, "lt": A < B, "le": A <= B}
+                if ty == "f32":
+                    # the negated forms are true when an operand is not a number; lg is "less or greater"
+                    table.update({"nlt": ~(A < B), "ngt": ~(A > B), "nge": ~(A >= B), "nle": ~(A <= B), "neq": ~(A == B),
+                                  "lg": (A < B) | (A > B), "nlg": ~((A < B) | (A > B)), "o": ~(np.isnan(A) | np.isnan(B)),
+                                  "u": np.isnan(A) | np.isnan(B)})
+                c = table[kind]
             val = self.mask_to_int(c & self.lanes())
             self.ws(dst, val, 2)
         elif op in ("v_cndmask_b32_e32", "v_cndmask_b32_e64"):
@@ -1061,8 +1084,8 @@ class Wave:
             sel = np.array([(selm >> k) & 1 for k in range(64)], dtype=bool)
             a, b = pick(V(o[1]), mods.get("src0_sel", "DWORD")), pick(V(o[2]), mods.get("src1_sel", "DWORD"))
             self.wv(o[0], np.where(sel, b, a).astype(U32))
-        elif op == "v_lshlrev_b32_sdwa":
-            # dst = src1 << src0[4:0], each source after its sub-dword select (zero-extended); whole destination written
+        elif op in ("v_lshlrev_b32_sdwa", "v_lshrrev_b32_sdwa", "v_or_b32_sdwa", "v_and_b32_sdwa", "v_xor_b32_sdwa", "v_add_u32_sdwa"):
+            # a two-operand op whose sources go through a sub-dword select first (zero-extended); whole destination written
             def pick(val, how):
                 if how == "DWORD":
                     return val.astype(np.uint64)
@@ -1071,8 +1094,15 @@ class Wave:
                 return (val.astype(np.uint64) >> np.uint64(width * int(idx))) & np.uint64((1 << width) - 1)
             if mods.get("dst_sel", "DWORD") != "DWORD" or mods.get("dst_unused", "UNUSED_PAD") != "UNUSED_PAD" or "sext" in text:
                 raise Fault(f"operand selects of {op} not modelled ({self.who()})")
-            count, val = pick(V(o[1]), mods.get("src0_sel", "DWORD")), pick(V(o[2]), mods.get("src1_sel", "DWORD"))
-            self.wv(o[0], ((val << (count & np.uint64(31))) & np.uint64(0xFFFFFFFF)).astype(U32))
+            x, y = pick(V(o[1]), mods.get("src0_sel", "DWORD")), pick(V(o[2]), mods.get("src1_sel", "DWORD"))
+            base = op[:-5]
+            if base == "v_lshlrev_b32": r = y << (x & np.uint64(31))          # the count is source 0
+            elif base == "v_lshrrev_b32": r = y >> (x & np.uint64(31))
+            elif base == "v_or_b32": r = x | y
+            elif base == "v_and_b32": r = x & y
+            elif base == "v_xor_b32": r = x ^ y
+            else: r = x + y
+            self.wv(o[0], (r & np.uint64(0xFFFFFFFF)).astype(U32))
         # ---------------------------------------------------------------- LDS
         elif op == "ds_read_b32":
             addr = V(o[1]).astype(np.int64) + int(mods.get("offset", "0"), 0)
