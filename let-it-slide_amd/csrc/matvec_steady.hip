@@ -21,6 +21,10 @@
 //     the ragged last slab sits in the image at the full slabs' stride (slot 32 q + l), so its reload is the same
 //     instruction sequence.
 // Every sum has a fixed order: outputs are bit-identical from run to run.
+//
+// Compile-time switches, all off in the library's build (each is a variant to be timed against it; every one passes the
+// same tests in the CPU wave model): ST_MFMA, the element's products on the matrix unit instead of 32 two-term dot
+// products; ST_ROLL, the decode block as a rolling pipeline of sixteen gathers; ST_NOPRIO, no s_setprio.
 #include "matvec_loop.hpp"
 #include "rptc_common.hpp"
 
