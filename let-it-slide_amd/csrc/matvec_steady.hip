@@ -250,6 +250,39 @@ static_assert(kStLdsBytes == kMaxLds, "the layout fills the LDS of a CU");
 #define ST_READS_B ST_RDPAIR("%[g0]", "v64", "v65") ST_RDPAIR("%[g1]", "v66", "v67") \
                    ST_RDPAIR("%[g2]", "v68", "v69") ST_RDPAIR("%[g3]", "v70", "v71")
 #define ST_MM(A, J, I, C) "v_mfma_f32_4x4x4_16b_f16 v[52:55], " A ", " ST_XP(J, I) ", " C "\n"
+#ifdef ST_ROLL
+// the rolling form (see the dot-product build above): a step waits for the oldest two gathers, multiplies them and
+// puts the next window register's two gathers in their registers
+#define ST_STEP(G, TH, TL, J, I, C)                           \
+    "s_waitcnt lgkmcnt(14)\n"                                 \
+    ST_MM("v[" TH ":" TL "]", J, I, C)                        \
+    ST_RDPAIR(G, "v" TH, "v" TL)
+#define ST_DRAIN(N, TH, TL, J, I)                             \
+    "s_nop 0\n"                                               \
+    "s_waitcnt lgkmcnt(" #N ")\n"                             \
+    ST_MM("v[" TH ":" TL "]", J, I, "v[52:55]")
+#define ST_WIN(SH, EX, EY, EZ, EW)                                                                                    \
+    "v_alignbit_b32 %[g0], %[cy], " EX ", " #SH "\n v_alignbit_b32 %[g1], " EX ", " EY ", " #SH "\n"                  \
+    "v_alignbit_b32 %[g2], " EY ", " EZ ", " #SH "\n v_alignbit_b32 %[g3], " EZ ", " EW ", " #SH "\n"                 \
+    "v_pk_mad_u16 %[g0], %[g0], %[g0], %[g0]\n v_pk_mad_u16 %[g1], %[g1], %[g1], %[g1]\n"                             \
+    "v_pk_mad_u16 %[g2], %[g2], %[g2], %[g2]\n v_pk_mad_u16 %[g3], %[g3], %[g3], %[g3]\n"
+#define ST_DECODE(EX, EY, EZ, EW, OWN, FIRST)                                                                         \
+    "s_nop 1\n"                                                                                                       \
+    "s_mov_b64 vcc, " FIRST "\n"                                                                                      \
+    "v_cndmask_b32_dpp %[cy], " EW ", " OWN ", vcc wave_shr:1 row_mask:0xf bank_mask:0xf bound_ctrl:1\n"              \
+    ST_WIN(12, EX, EY, EZ, EW) ST_READS_A                                                                             \
+    ST_WIN(8, EX, EY, EZ, EW) ST_READS_B                                                                              \
+    ST_WIN(4, EX, EY, EZ, EW)                                                                                         \
+    ST_STEP("%[g0]", "56", "57", 0, 0, "0") ST_STEP("%[g1]", "58", "59", 0, 1, "v[52:55]")                            \
+    ST_STEP("%[g2]", "60", "61", 0, 2, "v[52:55]") ST_STEP("%[g3]", "62", "63", 0, 3, "v[52:55]")                     \
+    "v_pk_mad_u16 %[g0], " EX ", " EX ", " EX "\n v_pk_mad_u16 %[g1], " EY ", " EY ", " EY "\n"                       \
+    "v_pk_mad_u16 %[g2], " EZ ", " EZ ", " EZ "\n v_pk_mad_u16 %[g3], " EW ", " EW ", " EW "\n"                       \
+    ST_STEP("%[g0]", "64", "65", 1, 0, "v[52:55]") ST_STEP("%[g1]", "66", "67", 1, 1, "v[52:55]")                     \
+    ST_STEP("%[g2]", "68", "69", 1, 2, "v[52:55]") ST_STEP("%[g3]", "70", "71", 1, 3, "v[52:55]")                     \
+    ST_DRAIN(14, "56", "57", 2, 0) ST_DRAIN(12, "58", "59", 2, 1) ST_DRAIN(10, "60", "61", 2, 2)                      \
+    ST_DRAIN(8, "62", "63", 2, 3) ST_DRAIN(6, "64", "65", 3, 0) ST_DRAIN(4, "66", "67", 3, 1)                         \
+    ST_DRAIN(2, "68", "69", 3, 2) ST_DRAIN(0, "70", "71", 3, 3)
+#else
 #define ST_DECODE(EX, EY, EZ, EW, OWN, FIRST)                                                                         \
     /* a DPP operand must not have been written by a vector op in the two instructions before */                     \
     "s_nop 1\n"                                                                                                       \
@@ -295,6 +328,7 @@ static_assert(kStLdsBytes == kMaxLds, "the layout fills the LDS of a CU");
     "s_nop 0\n"                                                                                                       \
     ST_MM("v[64:65]", 3, 0, "v[52:55]") "s_nop 1\n" ST_MM("v[66:67]", 3, 1, "v[52:55]") "s_nop 1\n"                   \
     ST_MM("v[68:69]", 3, 2, "v[52:55]") "s_nop 1\n" ST_MM("v[70:71]", 3, 3, "v[52:55]")
+#endif
 
 #endif
 // ---- one element of a layer.  U: which of the wave's elements; X, Y, Z, W / QUAD: its four registers; P: parity of

@@ -584,3 +584,13 @@ def test_lite_search_kernel_matches_the_oracle(viterbi_isa, oracle, S, steps, we
     for v in want_symbols:
         state = ((state << 4) | int(v)) & 0xFFFF
     assert int(end_state[0]) == state
+
+
+@pytest.fixture(scope="module")
+def steady_mfma_roll_isa(tmp_path_factory):
+    return compile_to_assembly(tmp_path_factory, "matvec_steady", extra=("-DST_MFMA", "-DST_ROLL"))
+
+
+@pytest.mark.parametrize("m,n,count,S,mode", [(33, 4096 + 768, 3, 8, 0), (300, 64, 2, 6, 1), (1024, 2048 + 64, 3, 8, 1), (8192, 8192, 2, 8, 0)])
+def test_steady_kernel_with_both_the_matrix_unit_and_the_rolling_pipeline(steady_mfma_roll_isa, oracle, m, n, count, S, mode):
+    run_steady(steady_mfma_roll_isa, oracle, m, n, count, S, mode, blocks=sorted({0, (m - 1) // (2 * ((m + 2 * CUS - 1) // (2 * CUS)))}))
