@@ -594,3 +594,42 @@ def steady_mfma_roll_isa(tmp_path_factory):
 @pytest.mark.parametrize("m,n,count,S,mode", [(33, 4096 + 768, 3, 8, 0), (300, 64, 2, 6, 1), (1024, 2048 + 64, 3, 8, 1), (8192, 8192, 2, 8, 0)])
 def test_steady_kernel_with_both_the_matrix_unit_and_the_rolling_pipeline(steady_mfma_roll_isa, oracle, m, n, count, S, mode):
     run_steady(steady_mfma_roll_isa, oracle, m, n, count, S, mode, blocks=sorted({0, (m - 1) // (2 * ((m + 2 * CUS - 1) // (2 * CUS)))}))
+
+
+@pytest.mark.parametrize("S,bits,steps,weighted", [(8, 2, 3, False), (6, 2, 2, True), (8, 3, 2, False), (6, 3, 2, True)])
+def test_pair_search_kernel_matches_the_oracle(viterbi_isa, oracle, S, bits, steps, weighted):
+    """`viterbi_pairs_kernel<S, 2 bits, WEIGHTED>` and `viterbi_trace_kernel` (`csrc/viterbi.hip`) for a few steps of one
+    row against `orc_viterbi` over the table of pairs the states decode to: symbols, end state and cost to the bit.  (The
+    8-bits-a-step kernels keep a few registers in scratch memory, which the model does not have: they are GPU tests only.)"""
+    import torch
+    from rptc_kernels import quantize
+    rng = np.random.default_rng(10 * S + bits)
+    cb = rng.standard_normal(2 << S).astype(np.float16)
+    targets = (0.7 * rng.standard_normal((steps, 2))).astype(np.float32)
+    weights = rng.uniform(0.25, 4.0, (steps, 2)).astype(np.float32) if weighted else None
+    table = quantize.decode_table(torch.from_numpy(cb), S).numpy()          # the same states at every width; a step shifts 2 * bits in
+    back = np.full(steps * 1024, 0xABCD, dtype=np.uint16)
+    symbols = np.full(steps, 0xEE, dtype=np.uint8)
+    end_state = np.full(1, -1, dtype=np.int32)
+    cost = np.full(1, np.nan, dtype=np.float32)
+    mem = wave_model.Memory()
+    t_at, w_at, a_at, b_at, s_at, e_at, c_at = (0x7f4000000000, 0x7f4100000000, 0x7f4200000000, 0x7f4300000000, 0x7f4400000000,
+                                                0x7f4500000000, 0x7f4600000000)
+    mem.add(t_at, targets.view(np.uint8).reshape(-1).copy(), "targets")
+    if weighted:
+        mem.add(w_at, weights.view(np.uint8).reshape(-1).copy(), "weights")
+    mem.add(a_at, cb.view(np.uint8).copy(), "codebook")
+    mem.add(b_at, back.view(np.uint8), "back pointers")
+    mem.add(s_at, symbols, "symbols")
+    mem.add(e_at, end_state.view(np.uint8), "end state")
+    mem.add(c_at, cost.view(np.uint8), "cost")
+    wave_model.Wave.vm_latency, wave_model.Wave.lgkm_latency = 400, 60
+    search = wave_model.Kernel(viterbi_isa, "_ZN4rptc20viterbi_pairs_kernelILi%dELi%dELb%dEE" % (S, 2 * bits, 1 if weighted else 0))
+    search.launch(mem, (1,), 1024, [("ptr", t_at), ("ptr", w_at if weighted else 0), ("i64", 0), ("ptr", a_at), ("ptr", b_at), ("ptr", e_at),
+                                    ("ptr", c_at), ("i32", steps)], lds_bytes=(256 * 64 + 2 * 4096) * 4 + 2 * 1024 * 4, seed=S)
+    mem.regions = [r for r in mem.regions if r[2] != "kernarg"]
+    trace = wave_model.Kernel(viterbi_isa, "_ZN4rptc20viterbi_trace_kernelILi%dEE" % (2 * bits))
+    trace.launch(mem, (1,), 64, [("ptr", b_at), ("ptr", e_at), ("ptr", s_at), ("i32", 1), ("i32", steps)], seed=S)
+    want_symbols, want_cost, want_end = oracle.viterbi(table, 2 * bits, targets, weights)
+    assert np.array_equal(symbols.astype(np.int32), want_symbols)
+    assert cost.view(np.uint32)[0] == np.float32(want_cost).view(np.uint32) and int(end_state[0]) == want_end

@@ -1013,8 +1013,14 @@ class Wave:
                     src.append(f32(raw).astype(np.float64))
             with np.errstate(all="ignore"):
                 self.wv(o[0], as_u32((src[0] * src[1] + src[2]).astype(np.float32)))
-        elif op in ("v_cvt_f32_f16_e32", "v_cvt_f32_f16_sdwa"):
-            src = V(o[1])
+        elif op in ("v_cvt_f32_f16_e32", "v_cvt_f32_f16_sdwa", "v_cvt_f32_f16_e64"):
+            tok = o[1]
+            absolute, negate = "|" in tok, tok.startswith("-")
+            src = V(tok.strip("-|"))
+            if absolute:
+                src = src & U32(0x7FFF)
+            if negate:
+                src = src ^ U32(0x8000)
             if op.endswith("_sdwa"):
                 how = mods.get("src0_sel", "DWORD")
                 if mods.get("dst_sel", "DWORD") != "DWORD" or how not in ("DWORD", "WORD_0", "WORD_1") or "sext" in text:
@@ -1084,15 +1090,18 @@ class Wave:
             sel = np.array([(selm >> k) & 1 for k in range(64)], dtype=bool)
             a, b = pick(V(o[1]), mods.get("src0_sel", "DWORD")), pick(V(o[2]), mods.get("src1_sel", "DWORD"))
             self.wv(o[0], np.where(sel, b, a).astype(U32))
-        elif op in ("v_lshlrev_b32_sdwa", "v_lshrrev_b32_sdwa", "v_or_b32_sdwa", "v_and_b32_sdwa", "v_xor_b32_sdwa", "v_add_u32_sdwa"):
-            # a two-operand op whose sources go through a sub-dword select first (zero-extended); whole destination written
+        elif op in ("v_lshlrev_b32_sdwa", "v_lshrrev_b32_sdwa", "v_or_b32_sdwa", "v_and_b32_sdwa", "v_xor_b32_sdwa", "v_add_u32_sdwa",
+                    "v_mul_u32_u24_sdwa"):
+            # a two-operand op whose sources go through a sub-dword select first (zero-extended) and whose result goes to
+            # the selected part of the destination, the rest zero (UNUSED_PAD) or kept (UNUSED_PRESERVE)
             def pick(val, how):
                 if how == "DWORD":
                     return val.astype(np.uint64)
                 kind, idx = how.split("_")
                 width = 16 if kind == "WORD" else 8
                 return (val.astype(np.uint64) >> np.uint64(width * int(idx))) & np.uint64((1 << width) - 1)
-            if mods.get("dst_sel", "DWORD") != "DWORD" or mods.get("dst_unused", "UNUSED_PAD") != "UNUSED_PAD" or "sext" in text:
+            unused = mods.get("dst_unused", "UNUSED_PAD")
+            if unused not in ("UNUSED_PAD", "UNUSED_PRESERVE") or "sext" in text:
                 raise Fault(f"operand selects of {op} not modelled ({self.who()})")
             x, y = pick(V(o[1]), mods.get("src0_sel", "DWORD")), pick(V(o[2]), mods.get("src1_sel", "DWORD"))
             base = op[:-5]
@@ -1101,8 +1110,19 @@ class Wave:
             elif base == "v_or_b32": r = x | y
             elif base == "v_and_b32": r = x & y
             elif base == "v_xor_b32": r = x ^ y
+            elif base == "v_mul_u32_u24": r = (x & np.uint64(0xFFFFFF)) * (y & np.uint64(0xFFFFFF))
             else: r = x + y
-            self.wv(o[0], (r & np.uint64(0xFFFFFFFF)).astype(U32))
+            r = r & np.uint64(0xFFFFFFFF)
+            where = mods.get("dst_sel", "DWORD")
+            if where != "DWORD":
+                kind, idx = where.split("_")
+                width = 16 if kind == "WORD" else 8
+                field = np.uint64(((1 << width) - 1) << (width * int(idx)))
+                r = (r << np.uint64(width * int(idx))) & field
+                if unused == "UNUSED_PRESERVE":
+                    i, _ = self.vreg_index(o[0])
+                    r = r | (self.v[i].astype(np.uint64) & ~field & np.uint64(0xFFFFFFFF))
+            self.wv(o[0], r.astype(U32))
         # ---------------------------------------------------------------- LDS
         elif op == "ds_read_b32":
             addr = V(o[1]).astype(np.int64) + int(mods.get("offset", "0"), 0)
@@ -1382,6 +1402,9 @@ class Wave:
             x = self.v64(o[2])
             sh = V(o[1]).astype(np.uint64) & np.uint64(63)
             self.wv64(o[0], (x >> sh) if op == "v_lshrrev_b64" else (x.view(np.int64) >> sh.astype(np.int64)).view(np.uint64))
+        elif op == "v_mad_u32_u24":
+            r = (V(o[1]).astype(np.uint64) & np.uint64(0xFFFFFF)) * (V(o[2]).astype(np.uint64) & np.uint64(0xFFFFFF)) + V(o[3]).astype(np.uint64)
+            self.wv(o[0], (r & np.uint64(0xFFFFFFFF)).astype(U32))
         elif op == "v_mul_lo_u32":
             self.wv(o[0], ((V(o[1]).astype(np.uint64) * V(o[2]).astype(np.uint64)) & np.uint64(0xFFFFFFFF)).astype(U32))
         elif op == "v_mul_hi_u32":
