@@ -633,3 +633,83 @@ def test_pair_search_kernel_matches_the_oracle(viterbi_isa, oracle, S, bits, ste
     want_symbols, want_cost, want_end = oracle.viterbi(table, 2 * bits, targets, weights)
     assert np.array_equal(symbols.astype(np.int32), want_symbols)
     assert cost.view(np.uint32)[0] == np.float32(want_cost).view(np.uint32) and int(end_state[0]) == want_end
+
+
+@pytest.fixture(scope="module")
+def glue_isa(tmp_path_factory):
+    return compile_to_assembly(tmp_path_factory, "decode_glue")
+
+
+def _matvec_geometry(m, n):
+    rpb = 2 * ((m + 2 * CUS - 1) // (2 * CUS))
+    lt = (n & 2047) >> 6
+    rw_tail = 64 // lt if lt else 1
+    items_full = rpb // 2
+    items_tail = (rpb + rw_tail - 1) // rw_tail if lt else 0
+    magic = ((1 << 32) // items_full + 1) if items_full > 1 else 0
+    return rpb, rw_tail, items_tail, magic, 65536 + 2 * n + 4 * (n // 64) * rpb
+
+
+@pytest.mark.parametrize("prologue,m,n,mode", [("silu", 40, 2048 + 320, 0), ("rmsnorm", 70, 4096, 1), ("rmsnorm", 33, 64 * 7, 0)])
+def test_fused_prologue_kernels_equal_the_separate_kernels(matvec_isa, glue_isa, prologue, m, n, mode):
+    """`matvec_fused_kernel` with the SiLU gate or the residual add + RMS norm in its prologue (`csrc/matvec.hip`) against
+    the stand-alone element-wise kernel (`csrc/decode_glue.hip`) followed by the plain mat-vec kernel, all three run in the
+    model: the same output bits (the prologue repeats the stand-alone kernel's roundings; the residual stream the norm
+    form writes back is compared as well), and no access outside the buffers."""
+    S = 8
+    rng = np.random.default_rng(m + n)
+    cb = (rng.standard_normal(2 << S) * 0.1).astype(np.float16)
+    comp = rng.integers(0, 256, m * n // 4, dtype=np.uint8)
+    rpb, rw_tail, items_tail, magic, lds_plain = _matvec_geometry(m, n)
+    grid = (m + rpb - 1) // rpb
+    wave_model.Wave.vm_latency, wave_model.Wave.lgkm_latency = 400, 60
+    c_at, cb_at, x_at, x2_at, w_at, xo_at, h_at, o_at, o2_at = (0x7f40fffff000, 0x7f5000003400, 0x7f3ffff0fe00, 0x7f3000000000, 0x7f3100000000,
+                                                               0x7f3200000000, 0x7f3300000000, 0x7f2ffffe0100, 0x7f2e00000000)
+    out_fused = np.full(2 * m, 0xEE, dtype=np.uint8)
+    out_plain = np.full(2 * m, 0xEE, dtype=np.uint8)
+    mem = wave_model.Memory()
+    mem.add(c_at, comp, "stream")
+    mem.add(cb_at, cb.view(np.uint8).copy(), "codebook")
+    mem.add(o_at, out_fused, "output of the fused kernel")
+    mem.add(o2_at, out_plain, "output of the plain kernel")
+    common = [("ptr", c_at), ("ptr", cb_at), ("ptr", x_at), ("i32", m), ("i32", n), ("i32", rpb), ("i32", rw_tail), ("i32", items_tail), ("u32", magic)]
+
+    def forget_kernargs():
+        mem.regions = [r for r in mem.regions if r[2] != "kernarg"]
+    if prologue == "silu":
+        gu = (rng.standard_normal(2 * n) * 1.5).astype(np.float16)
+        h = np.full(2 * n, 0xEE, dtype=np.uint8)
+        mem.add(x_at, gu.view(np.uint8).copy(), "gate and up")
+        mem.add(h_at, h, "gated activations")
+        wave_model.Kernel(glue_isa, "_ZN4rptc15silu_mul_kernelE").launch(mem, ((n + 255) // 256,), 256, [("ptr", x_at), ("ptr", h_at), ("i32", n)], seed=1)
+        forget_kernargs()
+        fused = wave_model.Kernel(matvec_isa, "_ZN4rptc19matvec_fused_kernelILi%dELi%dELi1ELb0EE" % (S, mode))
+        fused.launch(mem, (grid,), 1024, common + [("ptr", 0), ("ptr", o_at), ("ptr", 0), ("ptr", 0), ("f32", 0.0), ("i32", 0)],
+                     lds_bytes=lds_plain, seed=m)
+    else:
+        x_in = (rng.standard_normal(n) * 1.2).astype(np.float16)
+        delta = (rng.standard_normal(n) * 0.3).astype(np.float16)
+        weight = (1.0 + 0.1 * rng.standard_normal(n)).astype(np.float16)
+        res_a = np.full(2 * n, 0xEE, dtype=np.uint8)
+        res_b = np.full(2 * n, 0xEE, dtype=np.uint8)
+        h = np.full(2 * n, 0xEE, dtype=np.uint8)
+        mem.add(x_at, x_in.view(np.uint8).copy(), "residual stream in")
+        mem.add(x2_at, delta.view(np.uint8).copy(), "delta")
+        mem.add(w_at, weight.view(np.uint8).copy(), "norm weight")
+        mem.add(xo_at, res_a, "residual stream out (stand-alone)")
+        mem.add(0x7f3400000000, res_b, "residual stream out (fused)")
+        mem.add(h_at, h, "normed activations")
+        eps = 1e-5
+        wave_model.Kernel(glue_isa, "_ZN4rptc18add_rmsnorm_kernelE").launch(
+            mem, (1,), 1024, [("ptr", x_at), ("ptr", x2_at), ("ptr", w_at), ("ptr", xo_at), ("ptr", h_at), ("i32", n), ("f32", eps)], seed=1)
+        forget_kernargs()
+        fused = wave_model.Kernel(matvec_isa, "_ZN4rptc19matvec_fused_kernelILi%dELi%dELi2ELb0EE" % (S, mode))
+        fused.launch(mem, (grid,), 1024, common + [("ptr", x2_at), ("ptr", o_at), ("ptr", w_at), ("ptr", 0x7f3400000000), ("f32", eps), ("i32", 0)],
+                     lds_bytes=lds_plain + 48 * 4, seed=m)
+        assert np.array_equal(res_a, res_b), "the residual stream written back differs"
+    forget_kernargs()
+    plain = wave_model.Kernel(matvec_isa, "_ZN4rptc13matvec_kernelILi%dELi%dELi2ELb0EE" % (S, mode))
+    plain.launch(mem, (grid,), 1024, [("ptr", c_at), ("ptr", cb_at), ("ptr", h_at), ("i32", m), ("i32", n), ("i32", rpb), ("i32", rw_tail),
+                                      ("i32", items_tail), ("u32", magic), ("ptr", o2_at)], lds_bytes=lds_plain, seed=m)
+    assert np.array_equal(out_fused, out_plain)
+    assert np.isfinite(out_fused.view(np.float16).astype(np.float32)).all()

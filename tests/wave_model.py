@@ -959,9 +959,14 @@ class Wave:
             sel = np.array([(S(o[3], 2) >> k) & 1 for k in range(64)], dtype=bool)
             r = np.where(sel, V(o[2]), src0)
             self.wv(o[0], r, self.lanes() & valid)
-        elif op == "v_fma_f32":
+        elif op == "v_fmac_f32_e32":
             with np.errstate(all="ignore"):
-                r = f32(V(o[1])) * f32(V(o[2])) + f32(V(o[3]))
+                r = (f32(V(o[1])).astype(np.float64) * f32(V(o[2])).astype(np.float64) + f32(V(o[0])).astype(np.float64)).astype(np.float32)
+            self.wv(o[0], as_u32(r))
+        elif op == "v_fma_f32":
+            # one rounding: the product of two fp32 values is exact in double
+            with np.errstate(all="ignore"):
+                r = (f32(V(o[1])).astype(np.float64) * f32(V(o[2])).astype(np.float64) + f32(V(o[3])).astype(np.float64)).astype(np.float32)
             self.wv(o[0], as_u32(r))
         elif op == "v_rsq_f32_e32":
             with np.errstate(all="ignore"):
@@ -977,6 +982,38 @@ class Wave:
             if where not in ("DWORD", "WORD_0", "WORD_1"):
                 raise Fault(f"operand selects of {op} not modelled ({self.who()})")
             self.wv(o[0], h << U32(16) if where == "WORD_1" else h)
+        elif op in ("v_exp_f32_e32", "v_rcp_f32_e32", "v_log_f32_e32", "v_sqrt_f32_e32"):
+            # the hardware's approximations are within an ulp of these; kernels that must agree bit for bit run the same
+            # instruction on the same input on both sides, which the model reproduces
+            with np.errstate(all="ignore"):
+                x = f32(V(o[1])).astype(np.float64)
+                r = {"v_exp_f32_e32": np.exp2, "v_rcp_f32_e32": lambda v: 1.0 / v, "v_log_f32_e32": np.log2, "v_sqrt_f32_e32": np.sqrt}[op](x)
+                r = r.astype(np.float32)
+            self.wv(o[0], as_u32(r))
+        elif op == "v_div_scale_f32":
+            # the operand (numerator or denominator) as it is and VCC = 0: true for operands far from the ends of the
+            # exponent range, which is checked (the scaled cases are not modelled)
+            src0 = f32(V(o[2]))
+            mag = np.abs(np.concatenate([f32(V(o[2])), f32(V(o[3])), f32(V(o[4]))]).astype(np.float64))
+            live = np.concatenate([self.lanes()] * 3)
+            if ((mag[live] != 0) & ((mag[live] < 1e-30) | (mag[live] > 1e30))).any():
+                raise Fault(f"{op}: operands that need scaling are not modelled ({self.who()})")
+            self.wv(o[0], as_u32(src0))
+            old = S(o[1], 2)
+            for k in range(64):
+                if self.lanes()[k]:
+                    old &= ~(1 << k)
+            self.ws(o[1], old, 2)
+        elif op == "v_div_fmas_f32":
+            with np.errstate(all="ignore"):
+                r = (f32(V(o[1])).astype(np.float64) * f32(V(o[2])).astype(np.float64) + f32(V(o[3])).astype(np.float64)).astype(np.float32)
+            self.wv(o[0], as_u32(r))
+        elif op == "v_div_fixup_f32":
+            q, den, num = f32(V(o[1])), f32(V(o[2])), f32(V(o[3]))
+            with np.errstate(all="ignore"):
+                exact = (num.astype(np.float64) / den.astype(np.float64)).astype(np.float32)
+            special = ~np.isfinite(q) | (den == 0) | ~np.isfinite(den) | ~np.isfinite(num)
+            self.wv(o[0], as_u32(np.where(special, exact, q)))
         elif op == "v_rcp_iflag_f32_e32":
             with np.errstate(all="ignore"):
                 r = np.float32(1.0) / f32(V(o[1]))
@@ -997,6 +1034,62 @@ class Wave:
             a, off, width = V(o[1]).astype(np.uint64), V(o[2]) & U32(31), V(o[3]) & U32(31)
             r = (a >> off.astype(np.uint64)) & ((np.uint64(1) << width.astype(np.uint64)) - np.uint64(1))
             self.wv(o[0], r.astype(U32))
+        elif op in ("v_lshrrev_b16_e32", "v_lshlrev_b16_e32", "v_add_u16_e32", "v_sub_u16_e32", "v_subrev_u16_e32", "v_mul_lo_u16_e32",
+                    "v_max_u16_e32", "v_min_u16_e32"):
+            # 16-bit integer ops on the low halves; the high half of the destination becomes zero (gfx9)
+            a, b = (V(o[1]) & 0xFFFF).astype(np.int64), (V(o[2]) & 0xFFFF).astype(np.int64)
+            r = {"v_lshrrev_b16_e32": lambda: b >> (a & 15), "v_lshlrev_b16_e32": lambda: b << (a & 15), "v_add_u16_e32": lambda: a + b,
+                 "v_sub_u16_e32": lambda: a - b, "v_subrev_u16_e32": lambda: b - a, "v_mul_lo_u16_e32": lambda: a * b,
+                 "v_max_u16_e32": lambda: np.maximum(a, b), "v_min_u16_e32": lambda: np.minimum(a, b)}[op]()
+            self.wv(o[0], (r & 0xFFFF).astype(U32))
+        elif op in ("v_mul_f16_e32", "v_add_f16_e32", "v_sub_f16_e32", "v_subrev_f16_e32", "v_max_f16_e32", "v_min_f16_e32"):
+            # the low halves; the high half of the destination becomes zero (gfx9: 16-bit vector ops clear it)
+            a = (V(o[1]) & 0xFFFF).astype(np.uint16).view(np.float16).astype(np.float64)
+            b = (V(o[2]) & 0xFFFF).astype(np.uint16).view(np.float16).astype(np.float64)
+            with np.errstate(all="ignore"):
+                r = {"v_mul_f16_e32": a * b, "v_add_f16_e32": a + b, "v_sub_f16_e32": a - b, "v_subrev_f16_e32": b - a,
+                     "v_max_f16_e32": np.maximum(a, b), "v_min_f16_e32": np.minimum(a, b)}[op]
+            self.wv(o[0], r.astype(np.float16).view(np.uint16).astype(U32))
+        elif op in ("v_pk_mul_f16", "v_pk_add_f16", "v_pk_fma_f16"):
+            if mods:
+                raise Fault(f"modifiers of {op} not modelled ({self.who()})")
+            def halves(tok):
+                raw = V(tok)
+                return ((raw & 0xFFFF).astype(np.uint16).view(np.float16).astype(np.float64),
+                        (raw >> U32(16)).astype(np.uint16).view(np.float16).astype(np.float64))
+            (al, ah), (bl, bh) = halves(o[1]), halves(o[2])
+            with np.errstate(all="ignore"):
+                if op == "v_pk_mul_f16": rl, rh = al * bl, ah * bh
+                elif op == "v_pk_add_f16": rl, rh = al + bl, ah + bh
+                else:
+                    cl, ch = halves(o[3])
+                    rl, rh = al * bl + cl, ah * bh + ch
+            self.wv(o[0], rl.astype(np.float16).view(np.uint16).astype(U32) | (rh.astype(np.float16).view(np.uint16).astype(U32) << U32(16)))
+        elif op == "v_cvt_pk_f16_f32":
+            # two fp32 values rounded to nearest even into the halves of one register (gfx950)
+            with np.errstate(all="ignore"):
+                lo16 = f32(V(o[1])).astype(np.float16).view(np.uint16).astype(U32)
+                hi16 = f32(V(o[2])).astype(np.float16).view(np.uint16).astype(U32)
+            self.wv(o[0], lo16 | (hi16 << U32(16)))
+        elif op in ("v_fma_mixlo_f16", "v_fma_mixhi_f16"):
+            # as v_fma_mix_f32, the result rounded once to fp16 and written to one half of the destination (the other kept)
+            hi = [int(x) for x in mods.get("op_sel_hi", "[0,0,0]").strip("[]").split(",")]
+            lo = [int(x) for x in mods.get("op_sel", "[0,0,0]").strip("[]").split(",")]
+            if "neg" in text or "abs" in text or "|" in text or "clamp" in text:
+                raise Fault(f"modifiers of {op} not modelled ({self.who()})")
+            src = []
+            for q in range(3):
+                raw = V(o[1 + q])
+                if hi[q]:
+                    half = (raw >> U32(16)) if lo[q] else raw
+                    src.append((half & 0xFFFF).astype(np.uint16).view(np.float16).astype(np.float64))
+                else:
+                    src.append(f32(raw).astype(np.float64))
+            with np.errstate(all="ignore"):
+                h = (src[0] * src[1] + src[2]).astype(np.float16).view(np.uint16).astype(U32)
+            i, _ = self.vreg_index(o[0])
+            old_v = self.v[i]
+            self.wv(o[0], (old_v & U32(0xFFFF0000)) | h if op == "v_fma_mixlo_f16" else (old_v & U32(0xFFFF)) | (h << U32(16)))
         elif op == "v_fma_mix_f32":
             # a source is fp32, or (its op_sel_hi bit set) the fp16 in the half of the register that op_sel names
             hi = [int(x) for x in mods.get("op_sel_hi", "[0,0,0]").strip("[]").split(",")]
@@ -1044,7 +1137,9 @@ class Wave:
                 r[k] = (bin(bits).count("1") + int(base[k])) & 0xFFFFFFFF
             self.wv(o[0], r)
         elif op.startswith("v_cmp_"):
-            m = re.match(r"v_cmp_(\w+?)_(u32|i32|f32|i64|u64)_(e32|e64)", op)
+            m = re.match(r"v_cmp_(\w+?)_(u32|i32|f32|i64|u64|u16|i16)_(e32|e64)", op)
+            if not m:
+                raise Fault(f"instruction not modelled: {op} ({self.who()})")
             kind, ty, enc = m.group(1), m.group(2), m.group(3)
             dst, a, b = (o[0], o[1], o[2])
             if ty in ("i64", "u64"):
@@ -1057,6 +1152,10 @@ class Wave:
                 pass
             elif ty == "i32":
                 A, B = A.view(np.int32).astype(np.int64), B.view(np.int32).astype(np.int64)
+            elif ty == "u16":
+                A, B = (A & 0xFFFF).astype(np.int64), (B & 0xFFFF).astype(np.int64)
+            elif ty == "i16":
+                A, B = (A & 0xFFFF).astype(np.uint16).view(np.int16).astype(np.int64), (B & 0xFFFF).astype(np.uint16).view(np.int16).astype(np.int64)
             elif ty == "f32":
                 A, B = f32(A), f32(B)
             else:
