@@ -713,3 +713,70 @@ def test_fused_prologue_kernels_equal_the_separate_kernels(matvec_isa, glue_isa,
                                       ("i32", items_tail), ("u32", magic), ("ptr", o2_at)], lds_bytes=lds_plain, seed=m)
     assert np.array_equal(out_fused, out_plain)
     assert np.isfinite(out_fused.view(np.float16).astype(np.float32)).all()
+
+
+def _rope_reference(x, cos_row, sin_row):
+    """The rotation of decode_glue.hip's rope_pair: products and sums in fp16, each rounded once."""
+    a, b = x[0::2].astype(np.float16), x[1::2].astype(np.float16)
+    c, s = cos_row.astype(np.float16), sin_row.astype(np.float16)
+    out = np.empty_like(x)
+    out[0::2] = (a * c).astype(np.float16) - (b * s).astype(np.float16)
+    out[1::2] = (a * s).astype(np.float16) + (b * c).astype(np.float16)
+    return out
+
+
+@pytest.mark.parametrize("rope,heads,hd,max_len,pos,splits", [(False, 3, 64, 96, 50, 3), (True, 2, 128, 64, 37, 4), (False, 2, 32, 48, 0, 2),
+                                                               (True, 1, 64, 32, 31, 2)])
+def test_attention_kernel_matches_a_softmax_in_double(glue_isa, rope, heads, hd, max_len, pos, splits):
+    """`attn_decode_kernel<ROPE>` (`csrc/decode_glue.hip`) as `rptc_attn_decode` / `rptc_rope_attn_decode` launch it: a head's
+    keys cut into pieces, one workgroup each, the last to arrive merging them (the model runs the workgroups one after the
+    other); with ROPE the rotation of q and k and the append to the caches happen inside.  Against softmax attention in
+    double over positions 0..pos; the caches outside row pos untouched; the arrival counters left at zero."""
+    rng = np.random.default_rng(heads * 1000 + pos)
+    d = heads * hd
+    k_cache = (rng.standard_normal((heads, max_len, hd)) * 0.5).astype(np.float16)
+    v_cache = (rng.standard_normal((heads, max_len, hd)) * 0.5).astype(np.float16)
+    cos_t = np.cos(rng.random((max_len, hd // 2)) * 6.28).astype(np.float16)
+    sin_t = np.sin(rng.random((max_len, hd // 2)) * 6.28).astype(np.float16)
+    qkv = (rng.standard_normal(3 * d) * 0.7).astype(np.float16)
+    k_before, v_before = k_cache.copy(), v_cache.copy()
+    if rope:
+        q_eff = np.concatenate([_rope_reference(qkv[h * hd:(h + 1) * hd], cos_t[pos], sin_t[pos]) for h in range(heads)])
+        for h in range(heads):
+            k_before[h, pos] = _rope_reference(qkv[d + h * hd:d + (h + 1) * hd], cos_t[pos], sin_t[pos])
+            v_before[h, pos] = qkv[2 * d + h * hd:2 * d + (h + 1) * hd]
+        q_in = qkv
+    else:
+        q_eff = qkv[:d]
+        q_in = qkv[:d].copy()
+    out = np.full(d, np.nan, dtype=np.float16)
+    parts = np.full(heads * splits * 258, np.nan, dtype=np.float32)
+    arrived = np.zeros(heads, dtype=np.uint32)
+    position = np.array([pos], dtype=np.int64)
+    mem = wave_model.Memory()
+    at = {name: 0x7f4000000000 + i * 0x100000000 for i, name in enumerate(("pos", "q", "k", "v", "cos", "sin", "out", "parts", "arrived"))}
+    mem.add(at["pos"], position.view(np.uint8), "position")
+    mem.add(at["q"], q_in.view(np.uint8).copy(), "query")
+    mem.add(at["k"], k_cache.view(np.uint8).reshape(-1), "key cache")
+    mem.add(at["v"], v_cache.view(np.uint8).reshape(-1), "value cache")
+    mem.add(at["cos"], cos_t.view(np.uint8).reshape(-1).copy(), "cosines")
+    mem.add(at["sin"], sin_t.view(np.uint8).reshape(-1).copy(), "sines")
+    mem.add(at["out"], out.view(np.uint8), "output")
+    mem.add(at["parts"], parts.view(np.uint8), "pieces")
+    mem.add(at["arrived"], arrived.view(np.uint8), "arrival counters")
+    wave_model.Wave.vm_latency, wave_model.Wave.lgkm_latency = 400, 60
+    kernel = wave_model.Kernel(glue_isa, "_ZN4rptc18attn_decode_kernelILb%dEE" % (1 if rope else 0))
+    kernel.launch(mem, (heads * splits,), 256,
+                  [("ptr", at["pos"]), ("ptr", at["q"]), ("ptr", at["k"]), ("ptr", at["v"]), ("i32", heads), ("i32", hd), ("i32", max_len),
+                   ("i32", splits), ("ptr", at["cos"]), ("ptr", at["sin"]), ("ptr", at["out"]), ("ptr", at["parts"]), ("ptr", at["arrived"])],
+                  lds_bytes=(16 + 2048) * 4 + hd * 6, seed=pos + 1)
+    assert np.array_equal(k_cache.view(np.uint16), k_before.view(np.uint16)) and np.array_equal(v_cache.view(np.uint16), v_before.view(np.uint16))
+    assert not arrived.any()
+    for h in range(heads):
+        q = q_eff[h * hd:(h + 1) * hd].astype(np.float64)
+        keys, values = k_before[h, :pos + 1].astype(np.float64), v_before[h, :pos + 1].astype(np.float64)
+        scores = keys @ q / np.sqrt(hd)
+        w = np.exp(scores - scores.max())
+        want = (w / w.sum()) @ values
+        got = out[h * hd:(h + 1) * hd].astype(np.float64)
+        assert np.abs(got - want).max() < 4e-3 * max(1.0, np.abs(want).max()), h

@@ -525,6 +525,16 @@ class Wave:
             elif "quad_perm" in mods:
                 qp = [int(x) for x in mods["quad_perm"].strip("[]").split(",")]
                 srcl = (lane & ~3) + qp[lane & 3]
+            elif "row_mirror" in mods:
+                srcl = row * 16 + (15 - idx)
+            elif "row_half_mirror" in mods:
+                srcl = row * 16 + (idx & 8) + (7 - (idx & 7))
+            elif "row_shl" in mods:
+                k = int(mods["row_shl"])
+                if idx + k <= 15:
+                    srcl = lane + k
+            elif "row_ror" in mods:
+                srcl = row * 16 + ((idx - int(mods["row_ror"])) & 15)
             else:
                 raise Fault(f"DPP control not modelled: {mods} ({self.who()})")
             if srcl is not None and (self.exec >> srcl) & 1:
@@ -832,6 +842,10 @@ class Wave:
                 if m[k]:
                     newvcc = (newvcc & ~(1 << k)) | (int(carry[k]) << k)
             self.vcc = newvcc
+        elif op == "v_bfi_b32":
+            # bits of source 1 where source 0 has ones, of source 2 elsewhere
+            mask = V(o[1])
+            self.wv(o[0], (mask & V(o[2])) | (~mask & V(o[3])))
         elif op == "v_or3_b32":
             self.wv(o[0], V(o[1]) | V(o[2]) | V(o[3]))
         elif op in ("v_bitop3_b32", "v_bitop3_b16"):
@@ -959,6 +973,13 @@ class Wave:
             sel = np.array([(S(o[3], 2) >> k) & 1 for k in range(64)], dtype=bool)
             r = np.where(sel, V(o[2]), src0)
             self.wv(o[0], r, self.lanes() & valid)
+        elif op in ("v_max_f32_e32", "v_min_f32_e32", "v_max3_f32", "v_min3_f32", "v_max_f32_e64", "v_min_f32_e64"):
+            # IEEE maxNum / minNum: a number wins over a NaN
+            fn = np.fmax if "max" in op else np.fmin
+            r = fn(f32(V(o[1])), f32(V(o[2])))
+            if "3" in op.split("_")[1]:
+                r = fn(r, f32(V(o[3])))
+            self.wv(o[0], as_u32(r.astype(np.float32)))
         elif op == "v_fmac_f32_e32":
             with np.errstate(all="ignore"):
                 r = (f32(V(o[1])).astype(np.float64) * f32(V(o[2])).astype(np.float64) + f32(V(o[0])).astype(np.float64)).astype(np.float32)
@@ -1051,19 +1072,26 @@ class Wave:
                      "v_max_f16_e32": np.maximum(a, b), "v_min_f16_e32": np.minimum(a, b)}[op]
             self.wv(o[0], r.astype(np.float16).view(np.uint16).astype(U32))
         elif op in ("v_pk_mul_f16", "v_pk_add_f16", "v_pk_fma_f16"):
-            if mods:
+            # op_sel[i]: the half of source i that feeds the low result; op_sel_hi[i]: the one that feeds the high result
+            nsrc = 3 if op == "v_pk_fma_f16" else 2
+            if "clamp" in mods:
                 raise Fault(f"modifiers of {op} not modelled ({self.who()})")
+            neg_lo = [int(x) for x in mods.get("neg_lo", "[0,0,0]").strip("[]").split(",")] + [0, 0, 0]
+            neg_hi = [int(x) for x in mods.get("neg_hi", "[0,0,0]").strip("[]").split(",")] + [0, 0, 0]
+            sel_lo = [int(x) for x in mods.get("op_sel", "[0,0,0]").strip("[]").split(",")] + [0, 0, 0]
+            sel_hi = [int(x) for x in mods.get("op_sel_hi", "[1,1,1]").strip("[]").split(",")] + [1, 1, 1]
+
             def halves(tok):
                 raw = V(tok)
                 return ((raw & 0xFFFF).astype(np.uint16).view(np.float16).astype(np.float64),
                         (raw >> U32(16)).astype(np.uint16).view(np.float16).astype(np.float64))
-            (al, ah), (bl, bh) = halves(o[1]), halves(o[2])
+            src = [halves(o[1 + q]) for q in range(nsrc)]
+            lo = [src[q][sel_lo[q]] * (-1.0 if neg_lo[q] else 1.0) for q in range(nsrc)]
+            hi = [src[q][sel_hi[q]] * (-1.0 if neg_hi[q] else 1.0) for q in range(nsrc)]
             with np.errstate(all="ignore"):
-                if op == "v_pk_mul_f16": rl, rh = al * bl, ah * bh
-                elif op == "v_pk_add_f16": rl, rh = al + bl, ah + bh
-                else:
-                    cl, ch = halves(o[3])
-                    rl, rh = al * bl + cl, ah * bh + ch
+                if op == "v_pk_mul_f16": rl, rh = lo[0] * lo[1], hi[0] * hi[1]
+                elif op == "v_pk_add_f16": rl, rh = lo[0] + lo[1], hi[0] + hi[1]
+                else: rl, rh = lo[0] * lo[1] + lo[2], hi[0] * hi[1] + hi[2]
             self.wv(o[0], rl.astype(np.float16).view(np.uint16).astype(U32) | (rh.astype(np.float16).view(np.uint16).astype(U32) << U32(16)))
         elif op == "v_cvt_pk_f16_f32":
             # two fp32 values rounded to nearest even into the halves of one register (gfx950)
