@@ -780,3 +780,75 @@ def test_attention_kernel_matches_a_softmax_in_double(glue_isa, rope, heads, hd,
         want = (w / w.sum()) @ values
         got = out[h * hd:(h + 1) * hd].astype(np.float64)
         assert np.abs(got - want).max() < 4e-3 * max(1.0, np.abs(want).max()), h
+
+
+@pytest.mark.parametrize("vocab,d,ties", [(32000, 128, False), (1003, 64, True), (7, 8, False)])
+def test_greedy_hand_over_kernel(glue_isa, vocab, d, ties):
+    """`greedy_next_kernel` (`csrc/decode_glue.hip`): the first maximum of the logits (a vocabulary that is no multiple of
+    eight included, and equal maxima), appended to the output list, its embedding row copied, index and position moved on."""
+    rng = np.random.default_rng(vocab)
+    logits = rng.standard_normal(vocab).astype(np.float16)
+    if ties:
+        top = np.float16(logits.astype(np.float32).max() + 1)
+        logits[[900, 333, 1002]] = top
+    embed = rng.standard_normal((vocab, d)).astype(np.float16)
+    token = np.array([-1], dtype=np.int64)
+    out_list = np.full(8, -1, dtype=np.int64)
+    out_index = np.array([3], dtype=np.int64)
+    pos = np.array([41], dtype=np.int64)
+    x = np.full(d, np.nan, dtype=np.float16)
+    mem = wave_model.Memory()
+    at = {name: 0x7f4000000000 + i * 0x100000000 for i, name in enumerate(("logits", "embed", "token", "list", "index", "pos", "x"))}
+    mem.add(at["logits"], logits.view(np.uint8).copy(), "logits")
+    mem.add(at["embed"], embed.view(np.uint8).reshape(-1).copy(), "embedding")
+    mem.add(at["token"], token.view(np.uint8), "token")
+    mem.add(at["list"], out_list.view(np.uint8), "output list")
+    mem.add(at["index"], out_index.view(np.uint8), "output index")
+    mem.add(at["pos"], pos.view(np.uint8), "position")
+    mem.add(at["x"], x.view(np.uint8), "next input")
+    wave_model.Wave.vm_latency, wave_model.Wave.lgkm_latency = 400, 60
+    kernel = wave_model.Kernel(glue_isa, "_ZN4rptc18greedy_next_kernelE")
+    kernel.launch(mem, (1,), 1024, [("ptr", at["logits"]), ("i32", vocab), ("ptr", at["embed"]), ("i32", d), ("ptr", at["token"]), ("ptr", at["list"]),
+                                    ("ptr", at["index"]), ("ptr", at["pos"]), ("ptr", at["x"])], seed=vocab)
+    want = int(np.argmax(logits.astype(np.float32)))
+    assert int(token[0]) == want and int(out_list[3]) == want and int(out_index[0]) == 4 and int(pos[0]) == 42
+    assert (out_list[[0, 1, 2, 4, 5, 6, 7]] == -1).all()
+    assert np.array_equal(x.view(np.uint16), embed[want].view(np.uint16))
+
+
+@pytest.mark.parametrize("heads,hd,max_len,pos", [(3, 64, 20, 7), (2, 128, 5, 4), (2, 32, 9, 9)])
+def test_rope_and_cache_kernel(glue_isa, heads, hd, max_len, pos):
+    """`rope_cache_kernel` (`csrc/decode_glue.hip`): q rotated, k rotated into its cache row, v copied into its, bit for bit
+    against the same fp16 arithmetic; a position outside the caches writes nothing."""
+    rng = np.random.default_rng(heads + pos)
+    d = heads * hd
+    qkv = (rng.standard_normal(3 * d) * 0.7).astype(np.float16)
+    cos_t = np.cos(rng.random((max_len, hd // 2)) * 6.28).astype(np.float16)
+    sin_t = np.sin(rng.random((max_len, hd // 2)) * 6.28).astype(np.float16)
+    k_cache = rng.standard_normal((heads, max_len, hd)).astype(np.float16)
+    v_cache = rng.standard_normal((heads, max_len, hd)).astype(np.float16)
+    k_want, v_want = k_cache.copy(), v_cache.copy()
+    q_out = np.full(d, np.nan, dtype=np.float16)
+    q_want = q_out.copy()
+    if pos < max_len:
+        q_want = np.concatenate([_rope_reference(qkv[h * hd:(h + 1) * hd], cos_t[pos], sin_t[pos]) for h in range(heads)])
+        for h in range(heads):
+            k_want[h, pos] = _rope_reference(qkv[d + h * hd:d + (h + 1) * hd], cos_t[pos], sin_t[pos])
+            v_want[h, pos] = qkv[2 * d + h * hd:2 * d + (h + 1) * hd]
+    position = np.array([pos], dtype=np.int64)
+    mem = wave_model.Memory()
+    at = {name: 0x7f4000000000 + i * 0x100000000 for i, name in enumerate(("qkv", "cos", "sin", "pos", "q", "k", "v"))}
+    mem.add(at["qkv"], qkv.view(np.uint8).copy(), "projection output")
+    mem.add(at["cos"], cos_t.view(np.uint8).reshape(-1).copy(), "cosines")
+    mem.add(at["sin"], sin_t.view(np.uint8).reshape(-1).copy(), "sines")
+    mem.add(at["pos"], position.view(np.uint8), "position")
+    mem.add(at["q"], q_out.view(np.uint8), "rotated query")
+    mem.add(at["k"], k_cache.view(np.uint8).reshape(-1), "key cache")
+    mem.add(at["v"], v_cache.view(np.uint8).reshape(-1), "value cache")
+    wave_model.Wave.vm_latency, wave_model.Wave.lgkm_latency = 400, 60
+    kernel = wave_model.Kernel(glue_isa, "_ZN4rptc17rope_cache_kernelE")
+    kernel.launch(mem, ((heads * hd // 2 + 255) // 256,), 256,
+                  [("ptr", at["qkv"]), ("ptr", at["cos"]), ("ptr", at["sin"]), ("ptr", at["pos"]), ("ptr", at["q"]), ("ptr", at["k"]), ("ptr", at["v"]),
+                   ("i32", heads), ("i32", hd), ("i32", max_len)], seed=pos)
+    assert np.array_equal(q_out.view(np.uint16), q_want.view(np.uint16))
+    assert np.array_equal(k_cache.view(np.uint16), k_want.view(np.uint16)) and np.array_equal(v_cache.view(np.uint16), v_want.view(np.uint16))

@@ -146,6 +146,12 @@ def f32(a):
     return a.view(np.float32)
 
 
+def f16_bits(a):
+    """float array -> fp16 bit patterns in uint32 (round to nearest even; garbage lanes may overflow: no warnings)"""
+    with np.errstate(all="ignore"):
+        return np.asarray(a).astype(np.float16).view(np.uint16).astype(U32)
+
+
 def as_u32(a):
     return np.asarray(a, dtype=np.float32).view(U32)
 
@@ -1070,7 +1076,7 @@ class Wave:
             with np.errstate(all="ignore"):
                 r = {"v_mul_f16_e32": a * b, "v_add_f16_e32": a + b, "v_sub_f16_e32": a - b, "v_subrev_f16_e32": b - a,
                      "v_max_f16_e32": np.maximum(a, b), "v_min_f16_e32": np.minimum(a, b)}[op]
-            self.wv(o[0], r.astype(np.float16).view(np.uint16).astype(U32))
+            self.wv(o[0], f16_bits(r))
         elif op in ("v_pk_mul_f16", "v_pk_add_f16", "v_pk_fma_f16"):
             # op_sel[i]: the half of source i that feeds the low result; op_sel_hi[i]: the one that feeds the high result
             nsrc = 3 if op == "v_pk_fma_f16" else 2
@@ -1086,13 +1092,16 @@ class Wave:
                 return ((raw & 0xFFFF).astype(np.uint16).view(np.float16).astype(np.float64),
                         (raw >> U32(16)).astype(np.uint16).view(np.float16).astype(np.float64))
             src = [halves(o[1 + q]) for q in range(nsrc)]
-            lo = [src[q][sel_lo[q]] * (-1.0 if neg_lo[q] else 1.0) for q in range(nsrc)]
-            hi = [src[q][sel_hi[q]] * (-1.0 if neg_hi[q] else 1.0) for q in range(nsrc)]
+            with np.errstate(all="ignore"):
+                lo = [src[q][sel_lo[q]] * (-1.0 if neg_lo[q] else 1.0) for q in range(nsrc)]
+                hi = [src[q][sel_hi[q]] * (-1.0 if neg_hi[q] else 1.0) for q in range(nsrc)]
             with np.errstate(all="ignore"):
                 if op == "v_pk_mul_f16": rl, rh = lo[0] * lo[1], hi[0] * hi[1]
                 elif op == "v_pk_add_f16": rl, rh = lo[0] + lo[1], hi[0] + hi[1]
                 else: rl, rh = lo[0] * lo[1] + lo[2], hi[0] * hi[1] + hi[2]
-            self.wv(o[0], rl.astype(np.float16).view(np.uint16).astype(U32) | (rh.astype(np.float16).view(np.uint16).astype(U32) << U32(16)))
+            self.wv(o[0], f16_bits(rl) | (f16_bits(rh) << U32(16)))
+        elif op == "v_pack_b32_f16":
+            self.wv(o[0], (V(o[1]) & U32(0xFFFF)) | ((V(o[2]) & U32(0xFFFF)) << U32(16)))
         elif op == "v_cvt_pk_f16_f32":
             # two fp32 values rounded to nearest even into the halves of one register (gfx950)
             with np.errstate(all="ignore"):
@@ -1218,7 +1227,7 @@ class Wave:
             a, b = pick(V(o[1]), mods.get("src0_sel", "DWORD")), pick(V(o[2]), mods.get("src1_sel", "DWORD"))
             self.wv(o[0], np.where(sel, b, a).astype(U32))
         elif op in ("v_lshlrev_b32_sdwa", "v_lshrrev_b32_sdwa", "v_or_b32_sdwa", "v_and_b32_sdwa", "v_xor_b32_sdwa", "v_add_u32_sdwa",
-                    "v_mul_u32_u24_sdwa"):
+                    "v_mul_u32_u24_sdwa", "v_mul_f16_sdwa", "v_add_f16_sdwa", "v_sub_f16_sdwa"):
             # a two-operand op whose sources go through a sub-dword select first (zero-extended) and whose result goes to
             # the selected part of the destination, the rest zero (UNUSED_PAD) or kept (UNUSED_PRESERVE)
             def pick(val, how):
@@ -1238,6 +1247,12 @@ class Wave:
             elif base == "v_and_b32": r = x & y
             elif base == "v_xor_b32": r = x ^ y
             elif base == "v_mul_u32_u24": r = (x & np.uint64(0xFFFFFF)) * (y & np.uint64(0xFFFFFF))
+            elif base in ("v_mul_f16", "v_add_f16", "v_sub_f16"):
+                hx = (x & np.uint64(0xFFFF)).astype(np.uint16).view(np.float16).astype(np.float64)
+                hy = (y & np.uint64(0xFFFF)).astype(np.uint16).view(np.float16).astype(np.float64)
+                with np.errstate(all="ignore"):
+                    hr = hx * hy if base == "v_mul_f16" else hx + hy if base == "v_add_f16" else hx - hy
+                r = f16_bits(hr).astype(np.uint64)
             else: r = x + y
             r = r & np.uint64(0xFFFFFFFF)
             where = mods.get("dst_sel", "DWORD")
@@ -1655,7 +1670,8 @@ class Kernel:
         GARBAGE = garbage
         rng = random.Random(seed)
         total = 0
-        lds_words = max(lds_bytes // 4, 16)
+        # the kernel's static LDS (its `__shared__` variables) comes first, the launch's dynamic LDS behind it
+        lds_words = max((self.desc.get("group_segment_fixed_size", 0) + lds_bytes) // 4, 16)
         waves = (block + 63) // 64
         todo = groups if groups is not None else [(x, y, z) for z in range(grid[2]) for y in range(grid[1]) for x in range(grid[0])]
         for (gx, gy, gz) in todo:
