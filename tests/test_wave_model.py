@@ -852,3 +852,58 @@ def test_rope_and_cache_kernel(glue_isa, heads, hd, max_len, pos):
                    ("i32", heads), ("i32", hd), ("i32", max_len)], seed=pos)
     assert np.array_equal(q_out.view(np.uint16), q_want.view(np.uint16))
     assert np.array_equal(k_cache.view(np.uint16), k_want.view(np.uint16)) and np.array_equal(v_cache.view(np.uint16), v_want.view(np.uint16))
+
+
+@pytest.mark.parametrize("m,n,mode,which", [(40, 2048 + 320, 0, "all"), (70, 4096, 1, "all"), (33, 64 * 7, 0, "none"), (20, 1024, 1, "out")])
+def test_affine_kernel_applies_the_factorisation(matvec_isa, oracle, m, n, mode, which):
+    """`matvec_affine_kernel<S, MODE, plain>` (`csrc/matvec.hip`): y = s_out * (W (s_in * a)) + b_out * sum(a) + b_in . a with
+    the factorisation's four vectors (quantize_hf.py:167), any of them absent; against the same in double on the decoded
+    matrix; with none of them the output bits are the plain kernel's."""
+    S = 8
+    rng = np.random.default_rng(m + n)
+    cb = (rng.standard_normal(2 << S) * 0.1).astype(np.float16)
+    comp = rng.integers(0, 256, m * n // 4, dtype=np.uint8)
+    x = (rng.standard_normal(n) * 0.5).astype(np.float16)
+    si = (rng.random(n) + 0.5).astype(np.float16) if which == "all" else None
+    bi = (rng.standard_normal(n) * 0.02).astype(np.float16) if which == "all" else None
+    so = (rng.random(m) + 0.5).astype(np.float16) if which in ("all", "out") else None
+    bo = (rng.standard_normal(m) * 0.02).astype(np.float16) if which in ("all", "out") else None
+    rpb, rw_tail, items_tail, magic, lds_plain = _matvec_geometry(m, n)
+    grid = (m + rpb - 1) // rpb
+    out = np.full(2 * m, 0xEE, dtype=np.uint8)
+    mem = wave_model.Memory()
+    at = {name: 0x7f4000000000 + i * 0x100000000 + 0x100 for i, name in enumerate(("comp", "cb", "x", "si", "bi", "so", "bo", "out", "plain"))}
+    mem.add(at["comp"], comp, "stream")
+    mem.add(at["cb"], cb.view(np.uint8).copy(), "codebook")
+    mem.add(at["x"], x.view(np.uint8).copy(), "activations")
+    for name, vec in (("si", si), ("bi", bi), ("so", so), ("bo", bo)):
+        if vec is not None:
+            mem.add(at[name], vec.view(np.uint8).copy(), name)
+    mem.add(at["out"], out, "output")
+    wave_model.Wave.vm_latency, wave_model.Wave.lgkm_latency = 400, 60
+    ptr = lambda name, vec: ("ptr", at[name] if vec is not None else 0)
+    kernel = wave_model.Kernel(matvec_isa, "_ZN4rptc20matvec_affine_kernelILi%dELi%dELi0EE" % (S, mode))
+    kernel.launch(mem, (grid,), 1024,
+                  [("ptr", at["comp"]), ("ptr", at["cb"]), ("ptr", at["x"]), ("i32", m), ("i32", n), ("i32", rpb), ("i32", rw_tail), ("i32", items_tail),
+                   ("u32", magic), ("ptr", 0), ("ptr", at["out"]), ("ptr", 0), ("ptr", 0), ("f32", 0.0), ptr("si", si), ptr("bi", bi), ptr("so", so),
+                   ptr("bo", bo)], lds_bytes=lds_plain + 48 * 4, seed=m)
+    W = oracle.matvec_dense(comp.view(np.uint32), cb, m, n, S, mode=mode).astype(np.float64)
+    a64 = x.astype(np.float64)
+    xs = (x * si).astype(np.float16).astype(np.float64) if si is not None else a64
+    want = W @ xs
+    if so is not None:
+        want = want * so.astype(np.float64)
+    if bo is not None:
+        want = want + bo.astype(np.float64) * a64.sum()
+    if bi is not None:
+        want = want + (bi.astype(np.float64) * a64).sum()
+    got = out.view(np.float16).astype(np.float64)
+    assert np.linalg.norm(got - want) / np.linalg.norm(want) < 1e-3
+    if which == "none":
+        plain_out = np.full(2 * m, 0xEE, dtype=np.uint8)
+        mem.add(at["plain"], plain_out, "output of the plain kernel")
+        mem.regions = [r for r in mem.regions if r[2] != "kernarg"]
+        plain = wave_model.Kernel(matvec_isa, "_ZN4rptc13matvec_kernelILi%dELi%dELi2ELb0EE" % (S, mode))
+        plain.launch(mem, (grid,), 1024, [("ptr", at["comp"]), ("ptr", at["cb"]), ("ptr", at["x"]), ("i32", m), ("i32", n), ("i32", rpb), ("i32", rw_tail),
+                                          ("i32", items_tail), ("u32", magic), ("ptr", at["plain"])], lds_bytes=lds_plain, seed=m)
+        assert np.array_equal(out, plain_out)

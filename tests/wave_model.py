@@ -1707,7 +1707,8 @@ class Kernel:
                 for _ in range(rng.randint(1, burst)):
                     if w.done or w.at_barrier:
                         break
-                    w.step()
+                    with np.errstate(all="ignore"):          # lanes that hold garbage overflow and divide by zero
+                        w.step()
                     steps += 1
                 if steps > max_steps:
                     raise Fault("step limit: " + "; ".join(f"w{x.wid}@{x.insts[x.pc][3]}" for x in ws if not x.done))
