@@ -907,3 +907,100 @@ def test_affine_kernel_applies_the_factorisation(matvec_isa, oracle, m, n, mode,
         plain.launch(mem, (grid,), 1024, [("ptr", at["comp"]), ("ptr", at["cb"]), ("ptr", at["x"]), ("i32", m), ("i32", n), ("i32", rpb), ("i32", rw_tail),
                                           ("i32", items_tail), ("u32", magic), ("ptr", at["plain"])], lds_bytes=lds_plain, seed=m)
         assert np.array_equal(out, plain_out)
+
+
+@pytest.mark.parametrize("bits,m,n,S,mode", [(3, 40, 2048 + 320, 8, 0), (4, 33, 4096, 6, 1), (3, 20, 64 * 5, 6, 1), (4, 70, 2048 + 64, 8, 0)])
+def test_per_launch_kernel_at_3_and_4_bits(matvec_isa, oracle, bits, m, n, S, mode):
+    """`matvec_kernel<S, MODE, BITS, false>` for the 3- and 4-bit streams (`rptc_decompress_matvec_bits`) against the dense
+    matrix the oracle decodes from the same stream (`orc_bits_dense`) times the activations in double."""
+    rng = np.random.default_rng(bits * 100 + m)
+    cb = (rng.standard_normal(2 << S) * 0.1).astype(np.float16)
+    comp = rng.integers(0, 256, m * n * bits // 8, dtype=np.uint8)
+    x = (rng.standard_normal(n) * 0.5).astype(np.float16)
+    out = np.full(2 * m, 0xEE, dtype=np.uint8)
+    rpb, rw_tail, items_tail, magic, lds_bytes = _matvec_geometry(m, n)
+    grid = (m + rpb - 1) // rpb
+    mem = wave_model.Memory()
+    c_at, cb_at, x_at, o_at = 0x7f40fffff000, 0x7f5000003400, 0x7f3ffff0fe00, 0x7f2ffffe0100
+    mem.add(c_at, comp, "stream")
+    mem.add(cb_at, cb.view(np.uint8).copy(), "codebook")
+    mem.add(x_at, x.view(np.uint8).copy(), "activations")
+    mem.add(o_at, out, "output")
+    wave_model.Wave.vm_latency, wave_model.Wave.lgkm_latency = 400, 60
+    kernel = wave_model.Kernel(matvec_isa, "_ZN4rptc13matvec_kernelILi%dELi%dELi%dELb0EE" % (S, mode, bits))
+    kernel.launch(mem, (grid,), 1024, [("ptr", c_at), ("ptr", cb_at), ("ptr", x_at), ("i32", m), ("i32", n), ("i32", rpb), ("i32", rw_tail),
+                                       ("i32", items_tail), ("u32", magic), ("ptr", o_at)], lds_bytes=lds_bytes, seed=m)
+    W = oracle.bits_dense(comp.view(np.uint32), cb, m, n, S, bits, mode=mode).astype(np.float64)
+    want = W @ x.astype(np.float64)
+    got = out.view(np.float16).astype(np.float64)
+    assert np.abs(got - want).max() / (np.abs(want).max() + 1e-9) < 2e-3
+
+
+@pytest.mark.parametrize("bits,m,n,S,mode", [(2, 10, 2048 + 320, 8, 0), (2, 7, 64 * 3, 6, 1), (3, 9, 2048 + 64, 8, 1), (4, 5, 4096, 6, 0)])
+def test_dense_export_kernels_are_bit_exact(matvec_isa, oracle, bits, m, n, S, mode):
+    """`matvec_dense_kernel` / `bits_dense_kernel` (`csrc/matvec.hip`), one launch a slab as the library launches them:
+    the fp16 matrix a stream stands for, bit for bit against the oracle's."""
+    rng = np.random.default_rng(bits * 10 + m)
+    cb = rng.standard_normal(2 << S).astype(np.float16)
+    comp = rng.integers(0, 256, m * n * bits // 8, dtype=np.uint8)
+    W = np.full(m * n, 0xEEEE, dtype=np.uint16)
+    mem = wave_model.Memory()
+    c_at, cb_at, w_at = 0x7f40fffff000, 0x7f5000003400, 0x7f2ffffe0100
+    mem.add(c_at, comp, "stream")
+    mem.add(cb_at, cb.view(np.uint8).copy(), "codebook")
+    mem.add(w_at, W.view(np.uint8), "dense matrix")
+    wave_model.Wave.vm_latency, wave_model.Wave.lgkm_latency = 400, 60
+    name = "_ZN4rptc19matvec_dense_kernelILi%dELi%dEE" % (S, mode) if bits == 2 else "_ZN4rptc17bits_dense_kernelILi%dELi%dELi%dEE" % (S, mode, bits)
+    kernel = wave_model.Kernel(matvec_isa, name)
+    T, lt = n >> 11, (n & 2047) >> 6
+    for slab in range(T + (1 if lt else 0)):
+        elems = m * (32 if slab < T else lt)
+        kernel.launch(mem, ((elems + 255) // 256,), 256, [("ptr", c_at), ("ptr", cb_at), ("ptr", w_at), ("i32", m), ("i32", n), ("i32", slab),
+                                                         ("i32", elems)], seed=slab + 1)
+        mem.regions = [r for r in mem.regions if r[2] != "kernarg"]
+    want = (oracle.matvec_dense(comp.view(np.uint32), cb, m, n, S, mode=mode) if bits == 2 else
+            oracle.bits_dense(comp.view(np.uint32), cb, m, n, S, bits, mode=mode))
+    assert np.array_equal(W.reshape(m, n), want.view(np.uint16))
+
+
+@pytest.mark.parametrize("m,n,block,mode", [(40, 2048 + 256, 256, 0), (33, 1024, 1024, 1), (20, 64 * 6, 128, 0)])
+def test_hadamard_prologue_kernel_equals_the_two_kernels(matvec_isa, hadamard_isa, m, n, block, mode):
+    """`matvec_fused_kernel` with the sign-Hadamard transform of the activations in its prologue
+    (`rptc_decompress_matvec_hadamard`) against `sign_hadamard_kernel` followed by the plain mat-vec kernel, all in the
+    model: the same output bits."""
+    S = 8
+    rng = np.random.default_rng(m + n)
+    cb = (rng.standard_normal(2 << S) * 0.1).astype(np.float16)
+    comp = rng.integers(0, 256, m * n // 4, dtype=np.uint8)
+    x = rng.standard_normal(n).astype(np.float16)
+    signs = np.where(rng.integers(0, 2, n) == 1, 1.0, -1.0).astype(np.float16)
+    rpb, rw_tail, items_tail, magic, lds_plain = _matvec_geometry(m, n)
+    grid = (m + rpb - 1) // rpb
+    h = np.full(2 * n, 0xEE, dtype=np.uint8)
+    out_fused = np.full(2 * m, 0xEE, dtype=np.uint8)
+    out_plain = np.full(2 * m, 0xEE, dtype=np.uint8)
+    mem = wave_model.Memory()
+    c_at, cb_at, x_at, s_at, h_at, o_at, o2_at = (0x7f40fffff000, 0x7f5000003400, 0x7f3ffff0fe00, 0x7f3000000000, 0x7f3300000000, 0x7f2ffffe0100,
+                                                  0x7f2e00000000)
+    mem.add(c_at, comp, "stream")
+    mem.add(cb_at, cb.view(np.uint8).copy(), "codebook")
+    mem.add(x_at, x.view(np.uint8).copy(), "activations")
+    mem.add(s_at, signs.view(np.uint8).copy(), "signs")
+    mem.add(h_at, h, "transformed activations")
+    mem.add(o_at, out_fused, "output of the fused kernel")
+    mem.add(o2_at, out_plain, "output of the plain kernel")
+    wave_model.Wave.vm_latency, wave_model.Wave.lgkm_latency = 400, 60
+    log_p = block.bit_length() - 1
+    wave_model.Kernel(hadamard_isa, "_ZN4rptc20sign_hadamard_kernelE").launch(
+        mem, (n // block,), 256, [("ptr", x_at), ("ptr", s_at), ("ptr", h_at), ("i32", n), ("i32", block), ("i32", log_p), ("i32", n // block),
+                                  ("i32", 0), ("i32", 1 if block % 8 == 0 else 0)], lds_bytes=(block + block // 32) * 4, seed=n)
+    mem.regions = [r for r in mem.regions if r[2] != "kernarg"]
+    common = [("ptr", c_at), ("ptr", cb_at), ("ptr", x_at), ("i32", m), ("i32", n), ("i32", rpb), ("i32", rw_tail), ("i32", items_tail), ("u32", magic)]
+    fused = wave_model.Kernel(matvec_isa, "_ZN4rptc19matvec_fused_kernelILi%dELi%dELi3ELb0EE" % (S, mode))
+    fused.launch(mem, (grid,), 1024, common + [("ptr", s_at), ("ptr", o_at), ("ptr", 0), ("ptr", 0), ("f32", 0.0), ("i32", log_p)],
+                 lds_bytes=lds_plain + (n + n // 32 + 1) * 4, seed=m)
+    mem.regions = [r for r in mem.regions if r[2] != "kernarg"]
+    plain = wave_model.Kernel(matvec_isa, "_ZN4rptc13matvec_kernelILi%dELi%dELi2ELb0EE" % (S, mode))
+    plain.launch(mem, (grid,), 1024, [("ptr", c_at), ("ptr", cb_at), ("ptr", h_at), ("i32", m), ("i32", n), ("i32", rpb), ("i32", rw_tail),
+                                      ("i32", items_tail), ("u32", magic), ("ptr", o2_at)], lds_bytes=lds_plain, seed=m)
+    assert np.array_equal(out_fused, out_plain)
