@@ -1004,3 +1004,132 @@ def test_hadamard_prologue_kernel_equals_the_two_kernels(matvec_isa, hadamard_is
     plain.launch(mem, (grid,), 1024, [("ptr", c_at), ("ptr", cb_at), ("ptr", h_at), ("i32", m), ("i32", n), ("i32", rpb), ("i32", rw_tail),
                                       ("i32", items_tail), ("u32", magic), ("ptr", o2_at)], lds_bytes=lds_plain, seed=m)
     assert np.array_equal(out_fused, out_plain)
+
+
+def test_per_launch_kernel_with_compact_sums_on_long_rows(matvec_isa, oracle):
+    """`matvec_kernel<S, MODE, 2, true>`: rows so long (n = 28672) that one partial sum per row and 64 columns does not fit
+    beside the table and the activations; the lanes of a full slab are added first and a row keeps one sum per slab."""
+    m, n, S, mode = 8192, 28672, 8, 0
+    rng = np.random.default_rng(5)
+    cb = (rng.standard_normal(2 << S) * 0.1).astype(np.float16)
+    comp = rng.integers(0, 256, m * n // 4, dtype=np.uint8)
+    x = (rng.standard_normal(n) * 0.5).astype(np.float16)
+    out = np.full(2 * m, 0xEE, dtype=np.uint8)
+    rpb, rw_tail, items_tail, magic, lds_wide = _matvec_geometry(m, n)
+    assert lds_wide > 160 * 1024                                    # which is why the library picks the compact form here
+    lds_bytes = 65536 + 2 * n + 4 * ((n >> 11) + ((n & 2047) >> 6)) * rpb
+    grid = (m + rpb - 1) // rpb
+    mem = wave_model.Memory()
+    c_at, cb_at, x_at, o_at = 0x7f40fffff000, 0x7f5000003400, 0x7f3ffff0fe00, 0x7f2ffffe0100
+    mem.add(c_at, comp, "stream")
+    mem.add(cb_at, cb.view(np.uint8).copy(), "codebook")
+    mem.add(x_at, x.view(np.uint8).copy(), "activations")
+    mem.add(o_at, out, "output")
+    wave_model.Wave.vm_latency, wave_model.Wave.lgkm_latency = 400, 60
+    blocks = [0, grid - 1]
+    kernel = wave_model.Kernel(matvec_isa, "_ZN4rptc13matvec_kernelILi%dELi%dELi2ELb1EE" % (S, mode))
+    kernel.launch(mem, (grid,), 1024, [("ptr", c_at), ("ptr", cb_at), ("ptr", x_at), ("i32", m), ("i32", n), ("i32", rpb), ("i32", rw_tail),
+                                       ("i32", items_tail), ("u32", magic), ("ptr", o_at)], lds_bytes=lds_bytes,
+                  groups=[(b, 0, 0) for b in blocks], seed=3)
+    want = oracle.matvec(comp.view(np.uint32), cb, x, m, S, mode=mode)
+    got = out.view(np.float16).astype(np.float64)
+    for b in blocks:
+        r0, r1 = b * rpb, min(m, (b + 1) * rpb)
+        assert np.abs(got[r0:r1] - want[r0:r1]).max() / (np.abs(want).max() + 1e-9) < 2e-3
+
+
+@pytest.mark.parametrize("m,n,L,mode", [(70, 192, 16, 0), (300, 128, 14, 1), (5, 64, 16, 1)])
+def test_transposed_dense_export_is_bit_exact(matvec_t_isa, oracle, m, n, L, mode):
+    """`matvec_t_dense_kernel<L, MODE>` (`csrc/matvec_t.hip`), a two-dimensional grid (row blocks x columns of 64)."""
+    rng = np.random.default_rng(m + n + L)
+    cb = rng.standard_normal(1 << L).astype(np.float16)
+    comp = rng.integers(0, 256, m * n // 4, dtype=np.uint8)
+    W = np.full(m * n, 0xEEEE, dtype=np.uint16)
+    mem = wave_model.Memory()
+    c_at, cb_at, w_at = 0x7f40fffff000, 0x7f5000003400, 0x7f2ffffe0100
+    mem.add(c_at, comp, "stream")
+    mem.add(cb_at, cb.view(np.uint8).copy(), "codebook")
+    mem.add(w_at, W.view(np.uint8), "dense matrix")
+    wave_model.Wave.vm_latency, wave_model.Wave.lgkm_latency = 400, 60
+    kernel = wave_model.Kernel(matvec_t_isa, "_ZN4rptc21matvec_t_dense_kernelILi%dELi%dEE" % (L, mode))
+    kernel.launch(mem, ((m + 255) // 256, n // 64), 256, [("ptr", c_at), ("ptr", cb_at), ("ptr", w_at), ("i32", m), ("i32", n // 64)], seed=m)
+    want = oracle.matvec_t_dense(comp.view(np.uint32), cb, m, n, L, mode=mode)
+    assert np.array_equal(W.reshape(m, n), want.view(np.uint16))
+
+
+@pytest.mark.parametrize("L,steps,weighted", [(14, 3, False), (16, 2, True)])
+def test_scalar_search_kernel_matches_the_oracle(viterbi_isa, oracle, L, steps, weighted):
+    """`viterbi_scalar_kernel<L, WEIGHTED>` and its trace kernel (`csrc/viterbi.hip`): the reference's own trellis (2 bits and
+    one alphabet value a step) for a few steps against `orc_viterbi`, to the bit."""
+    rng = np.random.default_rng(L + steps)
+    alphabet = rng.standard_normal(1 << L).astype(np.float16)
+    targets = (0.7 * rng.standard_normal(steps)).astype(np.float32)
+    weights = rng.uniform(0.25, 4.0, steps).astype(np.float32) if weighted else None
+    back = np.full(steps * 1024, 0xABCDABCD, dtype=np.uint32)
+    symbols = np.full(steps, 0xEE, dtype=np.uint8)
+    end_state = np.full(1, -1, dtype=np.int32)
+    cost = np.full(1, np.nan, dtype=np.float32)
+    mem = wave_model.Memory()
+    t_at, w_at, a_at, b_at, s_at, e_at, c_at = (0x7f4000000000, 0x7f4100000000, 0x7f4200000000, 0x7f4300000000, 0x7f4400000000,
+                                                0x7f4500000000, 0x7f4600000000)
+    mem.add(t_at, targets.view(np.uint8).copy(), "targets")
+    if weighted:
+        mem.add(w_at, weights.view(np.uint8).copy(), "weights")
+    mem.add(a_at, alphabet.view(np.uint8).copy(), "alphabet")
+    mem.add(b_at, back.view(np.uint8), "back pointers")
+    mem.add(s_at, symbols, "symbols")
+    mem.add(e_at, end_state.view(np.uint8), "end state")
+    mem.add(c_at, cost.view(np.uint8), "cost")
+    wave_model.Wave.vm_latency, wave_model.Wave.lgkm_latency = 400, 60
+    search = wave_model.Kernel(viterbi_isa, "_ZN4rptc21viterbi_scalar_kernelILi%dELb%dEE" % (L, 1 if weighted else 0))
+    search.launch(mem, (1,), 1024, [("ptr", t_at), ("ptr", w_at if weighted else 0), ("i64", 0), ("ptr", a_at), ("ptr", b_at), ("ptr", e_at),
+                                    ("ptr", c_at), ("i32", steps)], lds_bytes=2 * ((1 << L) // 4) * 4 + 2 * 1024 * 4, seed=L)
+    mem.regions = [r for r in mem.regions if r[2] != "kernarg"]
+    trace = wave_model.Kernel(viterbi_isa, "_ZN4rptc27viterbi_scalar_trace_kernelILi%dEE" % L)
+    trace.launch(mem, (1,), 64, [("ptr", b_at), ("ptr", e_at), ("ptr", s_at), ("i32", 1), ("i32", steps)], seed=L)
+    want_symbols, want_cost, want_end = oracle.viterbi(alphabet.astype(np.float32), 2, targets, weights)
+    assert np.array_equal(symbols.astype(np.int32), want_symbols)
+    assert cost.view(np.uint32)[0] == np.float32(want_cost).view(np.uint32) and int(end_state[0]) == want_end
+
+
+@pytest.mark.parametrize("bits,m,n,batch,S,mode", [(3, 40, 2048 + 128, 5, 8, 0), (4, 100, 704, 20, 6, 1), (4, 16, 2048, 16, 8, 1), (3, 33, 4096, 18, 6, 0)])
+def test_batched_kernel_at_3_and_4_bits(matmul_isa, oracle, bits, m, n, batch, S, mode):
+    """`matmul_kernel<S, MODE, PLANES, BITS>` for the 3- and 4-bit streams (an element is 2 * BITS words; fewer row blocks a
+    workgroup) behind `pack_x_kernel`, against the dense matrix the oracle decodes times the activations."""
+    rng = np.random.default_rng(m + n + batch + bits)
+    codebook = (rng.standard_normal(2 << S) * 0.1).astype(np.float16)
+    stream = rng.integers(0, 256, m * n * bits // 8, dtype=np.uint8)
+    x = (rng.standard_normal((batch, n)) * 0.5).astype(np.float16)
+    out = np.full((batch, m), np.nan, dtype=np.float16)
+    planes = 2 if batch > 16 else 1
+    slabs = n // 2048 + (1 if n % 2048 else 0)
+    total = (m + 15) // 16
+    groups = max(1, min(2 * CUS // slabs, total))
+    groups = max(groups, -(-total // (6 if planes == 1 else 3)))
+    max_rb = -(-total // groups)
+    xpack = np.zeros(planes * (n // 2) * 16 + 1536, dtype=np.uint32)
+    partial = np.zeros(groups * slabs * max_rb * planes * 256, dtype=np.float32)
+    arrived = np.full(groups, 0xABCD, dtype=np.uint32)
+    mem = wave_model.Memory()
+    c_at, cb_at, x_at, o_at = 0x7f40fffff000, 0x7f5000003400, 0x7f3ffff0fe00, 0x7f2ffffe0100
+    xp_at, p_at, a_at = 0x7f6000000000, 0x7f6100000000, 0x7f6200000000
+    for at, data, name in ((c_at, stream, "stream"), (cb_at, codebook.view(np.uint8).copy(), "codebook"),
+                           (x_at, x.view(np.uint8).reshape(-1).copy(), "activations"), (o_at, out.view(np.uint8).reshape(-1), "output"),
+                           (xp_at, xpack.view(np.uint8), "packed activations"), (p_at, partial.view(np.uint8), "partial tiles"),
+                           (a_at, arrived.view(np.uint8), "arrival counters")):
+        mem.add(at, data, name)
+    wave_model.Wave.vm_latency, wave_model.Wave.lgkm_latency = 400, 60
+    pack = wave_model.Kernel(matmul_isa, "_ZN4rptc13pack_x_kernelE")
+    threads = max(planes * (n // 8) * 16, groups)
+    pack.launch(mem, ((threads + 255) // 256,), 256,
+                [("ptr", x_at), ("ptr", xp_at), ("ptr", a_at), ("i32", groups), ("i32", n), ("i32", batch), ("i32", planes)], seed=m)
+    mem.regions = [r for r in mem.regions if r[2] != "kernarg"]
+    kernel = wave_model.Kernel(matmul_isa, "_ZN4rptc13matmul_kernelILi%dELi%dELi%dELi%dEE" % (S, mode, planes, bits))
+    kernel.launch(mem, (groups * slabs,), 512,
+                  [("ptr", c_at), ("ptr", cb_at), ("ptr", xp_at), ("i32", m), ("i32", n), ("i32", total // groups), ("i32", total % groups),
+                   ("i32", 0), ("i32", max_rb), ("ptr", p_at), ("ptr", a_at), ("ptr", o_at), ("i32", batch)],
+                  lds_bytes=65536 + 8 * 2 * 256 * 4, seed=m)
+    W = oracle.bits_dense(stream.view(np.uint32), codebook, m, n, S, bits, mode=mode).astype(np.float64)
+    want = x.astype(np.float64) @ W.T
+    assert np.abs(out.astype(np.float64) - want).max() / (np.abs(want).max() + 1e-9) < 2e-3
+    assert not arrived.any()

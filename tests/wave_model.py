@@ -1112,16 +1112,24 @@ class Wave:
             # as v_fma_mix_f32, the result rounded once to fp16 and written to one half of the destination (the other kept)
             hi = [int(x) for x in mods.get("op_sel_hi", "[0,0,0]").strip("[]").split(",")]
             lo = [int(x) for x in mods.get("op_sel", "[0,0,0]").strip("[]").split(",")]
-            if "neg" in text or "abs" in text or "|" in text or "clamp" in text:
+            if "neg_" in text or "clamp" in text:
                 raise Fault(f"modifiers of {op} not modelled ({self.who()})")
             src = []
             for q in range(3):
-                raw = V(o[1 + q])
+                tok = o[1 + q].strip()
+                negate = tok.startswith("-") and tok[1:2] in ("v", "s", "|")
+                tok = tok[1:] if negate else tok
+                absolute = tok.startswith("|") and tok.endswith("|")
+                tok = tok[1:-1] if absolute else tok
+                raw = V(tok)
                 if hi[q]:
                     half = (raw >> U32(16)) if lo[q] else raw
-                    src.append((half & 0xFFFF).astype(np.uint16).view(np.float16).astype(np.float64))
+                    val = (half & 0xFFFF).astype(np.uint16).view(np.float16).astype(np.float64)
                 else:
-                    src.append(f32(raw).astype(np.float64))
+                    val = f32(raw).astype(np.float64)
+                # the modifiers act on the value the selects picked (the sign of the half, not bit 31 of the register)
+                val = np.abs(val) if absolute else val
+                src.append(-val if negate else val)
             with np.errstate(all="ignore"):
                 h = (src[0] * src[1] + src[2]).astype(np.float16).view(np.uint16).astype(U32)
             i, _ = self.vreg_index(o[0])
@@ -1131,16 +1139,24 @@ class Wave:
             # a source is fp32, or (its op_sel_hi bit set) the fp16 in the half of the register that op_sel names
             hi = [int(x) for x in mods.get("op_sel_hi", "[0,0,0]").strip("[]").split(",")]
             lo = [int(x) for x in mods.get("op_sel", "[0,0,0]").strip("[]").split(",")]
-            if "neg" in text or "abs" in text or "|" in text or "clamp" in text:
+            if "neg_" in text or "clamp" in text:
                 raise Fault(f"modifiers of {op} not modelled ({self.who()})")
             src = []
             for q in range(3):
-                raw = V(o[1 + q])
+                tok = o[1 + q].strip()
+                negate = tok.startswith("-") and tok[1:2] in ("v", "s", "|")
+                tok = tok[1:] if negate else tok
+                absolute = tok.startswith("|") and tok.endswith("|")
+                tok = tok[1:-1] if absolute else tok
+                raw = V(tok)
                 if hi[q]:
                     half = (raw >> U32(16)) if lo[q] else raw
-                    src.append((half & 0xFFFF).astype(np.uint16).view(np.float16).astype(np.float64))
+                    val = (half & 0xFFFF).astype(np.uint16).view(np.float16).astype(np.float64)
                 else:
-                    src.append(f32(raw).astype(np.float64))
+                    val = f32(raw).astype(np.float64)
+                # the modifiers act on the value the selects picked (the sign of the half, not bit 31 of the register)
+                val = np.abs(val) if absolute else val
+                src.append(-val if negate else val)
             with np.errstate(all="ignore"):
                 self.wv(o[0], as_u32((src[0] * src[1] + src[2]).astype(np.float32)))
         elif op in ("v_cvt_f32_f16_e32", "v_cvt_f32_f16_sdwa", "v_cvt_f32_f16_e64"):
