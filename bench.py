@@ -194,8 +194,8 @@ class Runner:
         return t1 - t0, ev0.elapsed_time(ev1)
 
     def chain_run(self, steps, warmup):
-        """`steps` layers (step k = weight copy k % copies, an output of its own per step: two layers that write one
-        buffer would be ordered by the chain, behind a grid-wide counter) as ONE chain launch.
+        """`steps` layers (step k = weight copy k % copies, an output of its own per step: layers that write one buffer
+        depend on each other, and such a chain is run as separate launches) as ONE chain launch.
         Returns (wall seconds, event milliseconds, rel-L2 of the last layer's output against the dense product)."""
         torch = self.torch
         import rptc_kernels
