@@ -22,9 +22,12 @@
 //     instruction sequence.
 // Every sum has a fixed order: outputs are bit-identical from run to run.
 //
-// Compile-time switches, all off in the library's build (each is a variant to be timed against it; every one passes the
-// same tests in the CPU wave model): ST_MFMA, the element's products on the matrix unit instead of 32 two-term dot
-// products; ST_ROLL, the decode block as a rolling pipeline of sixteen gathers; ST_NOPRIO, no s_setprio.
+// Compile-time switches, all off in the library's build, which is the kernel as it was timed (each switch is a variant
+// to be timed against it; every one passes the same tests in the CPU wave model): ST_TUNED, four changes to the layer's
+// chores (the activation reload without a wait of its own, the rows added by the waves with the fewest elements, the
+// next activations staged behind the first element instead of behind the last, a last layer that asks for nothing);
+// ST_MFMA, the element's products on the matrix unit instead of 32 two-term dot products; ST_ROLL, the decode block as a
+// rolling pipeline of sixteen gathers (both on top of ST_TUNED); ST_NOPRIO, no s_setprio.
 #include "matvec_loop.hpp"
 #include "rptc_common.hpp"
 
@@ -43,6 +46,9 @@ static_assert(kStLdsBytes == kMaxLds, "the layout fills the LDS of a CU");
 // stream elements of a wave: item u in v[80 + 4u : 83 + 4u]; next activations: v[72:75], v[76:79]
 // activation pairs of the slab being decoded: slot q in v(96 + q / 2) for even q, v(112 + (q - 1) / 2) for odd q, so
 // that slots q and q + 2 are neighbours and one ds_read2st64_b32 (two dwords 256 bytes apart) fills both
+#if (defined(ST_MFMA) || defined(ST_ROLL)) && !defined(ST_TUNED)
+#define ST_TUNED
+#endif
 #ifndef ST_MFMA
 #define ST_X0 "v96"
 #define ST_X2 "v97"
@@ -96,8 +102,14 @@ static_assert(kStLdsBytes == kMaxLds, "the layout fills the LDS of a CU");
 #ifndef ST_MFMA
 #define ST_RD2(LO, HI, BASE, OFF, P)                                                                                  \
     "ds_read2st64_b32 v[" #LO ":" #HI "], " BASE " offset0:" #P "*128+" #OFF " offset1:" #P "*128+" #OFF "+1\n"
-// LDS reads complete in order and the decode block's first wait (at most 8 reads in flight, its own) comes before its
-// first product, which is the first instruction to read an activation register: the reload needs no wait of its own
+// ST_TUNED: LDS reads complete in order and the decode block's first wait (at most 8 reads in flight, its own) comes
+// before its first product, which is the first instruction to read an activation register: the reload then needs no wait
+// of its own
+#ifdef ST_TUNED
+#define ST_RELOAD_WAIT ""
+#else
+#define ST_RELOAD_WAIT "s_waitcnt lgkmcnt(0)\n"
+#endif
 #define ST_RELOAD(XA, P)                                                                                              \
     "v_add_u32 %[xb], 0x80, " XA "\n"                                                                                 \
     ST_RD2(96, 97, XA, 0, P) ST_RD2(98, 99, XA, 2, P) ST_RD2(100, 101, XA, 4, P) ST_RD2(102, 103, XA, 6, P)           \
@@ -105,7 +117,7 @@ static_assert(kStLdsBytes == kMaxLds, "the layout fills the LDS of a CU");
     ST_RD2(112, 113, "%[xb]", 0, P) ST_RD2(114, 115, "%[xb]", 2, P) ST_RD2(116, 117, "%[xb]", 4, P)                   \
     ST_RD2(118, 119, "%[xb]", 6, P) ST_RD2(120, 121, "%[xb]", 8, P) ST_RD2(122, 123, "%[xb]", 10, P)                  \
     ST_RD2(124, 125, "%[xb]", 12, P) ST_RD2(126, 127, "%[xb]", 14, P)                                                 \
-    ""
+    ST_RELOAD_WAIT
 
 #else
 // pair (slot hi, slot lo) of a window register: both slots have the shift group's parity, so both are whole
@@ -387,6 +399,12 @@ static_assert(kStLdsBytes == kMaxLds, "the layout fills the LDS of a CU");
 // ---- the rows of the layer in front: a wave adds a row's n / 64 partial sums (lanes i, i + 64, i + 128, i + 192 in
 // that order, then across the lanes with DPP adds: rows of 16, row 0 into 1 and 2 into 3, rows 0-1 into 2-3), round
 // once to fp16 and lane 63 stores.  P: parity of the set that is read.
+// a row wave's next row: eight rows further, or (ST_TUNED) as many as there are row waves
+#ifdef ST_TUNED
+#define ST_NEXT_ROW "v_add_u32 %[g1], %[ostep], %[g1]\n"
+#else
+#define ST_NEXT_ROW "v_add_u32 %[g1], 16, %[g1]\n"
+#endif
 #define ST_DPP_ADD(CTRL) "s_nop 1\n v_add_f32_dpp %[a0], %[a0], %[a0] " CTRL "\n"
 #define ST_ROWS(P)                                                                                                    \
     "s_cmp_eq_u32 %[nr], 0\n"                                                                                         \
@@ -416,7 +434,7 @@ static_assert(kStLdsBytes == kMaxLds, "the layout fills the LDS of a CU");
     "global_store_short %[g1], %[a0], %[op]\n"                                                                        \
     "s_mov_b64 exec, -1\n"                                                                                            \
     "v_add_u32 %[g0], %[rstep], %[g0]\n"                                                                              \
-    "v_add_u32 %[g1], %[ostep], %[g1]\n"                                                                                    \
+    ST_NEXT_ROW                                                                                                       \
     "s_sub_u32 %[j], %[j], 1\n"                                                                                       \
     "s_cmp_lg_u32 %[j], 0\n"                                                                                          \
     "s_cbranch_scc1 91b\n"                                                                                            \
@@ -453,6 +471,7 @@ static_assert(kStLdsBytes == kMaxLds, "the layout fills the LDS of a CU");
     "global_load_dwordx4 v[72:75], %[xo0], %[xn]\n"                                                                   \
     "global_load_dwordx4 v[76:79], %[xo1], %[xn]\n"
 
+#ifdef ST_TUNED
 // The next layer's activations are staged behind the first element: their requests went out at the top of the layer,
 // and only the first element's next request has been made since (LPI requests may stay in flight).
 #define ST_EARLY_STAGE(Q, LPI) "s_waitcnt vmcnt(" #LPI ")\n" ST_STAGE(Q)
@@ -468,11 +487,20 @@ static_assert(kStLdsBytes == kMaxLds, "the layout fills the LDS of a CU");
     ST_ITEM_##MODE(0, "v80", "v81", "v82", "v83", P, 63, "") ST_ITEM_##MODE(1, "v84", "v85", "v86", "v87", P, 63, "")  \
     ST_ITEM_##MODE(2, "v88", "v89", "v90", "v91", P, 63, "")
 #define ST_LAST_ITEMS_4(MODE, P) ST_LAST_ITEMS_3(MODE, P) ST_ITEM_##MODE(3, "v92", "v93", "v94", "v95", P, 63, "")
+#else
+#define ST_ITEMS_3(MODE, P, Q, NEED, LPI)                                                                             \
+    ST_ITEM_##MODE(0, "v80", "v81", "v82", "v83", P, NEED, ST_REQUEST_##MODE(0, "v[80:83]"))                          \
+    ST_ITEM_##MODE(1, "v84", "v85", "v86", "v87", P, NEED, ST_REQUEST_##MODE(1, "v[84:87]"))                          \
+    ST_ITEM_##MODE(2, "v88", "v89", "v90", "v91", P, NEED, ST_REQUEST_##MODE(2, "v[88:91]"))
+#define ST_ITEMS_4(MODE, P, Q, NEED, LPI)                                                                             \
+    ST_ITEMS_3(MODE, P, Q, NEED, LPI) ST_ITEM_##MODE(3, "v92", "v93", "v94", "v95", P, NEED, ST_REQUEST_##MODE(3, "v[92:95]"))
+#endif
 #define ST_REQUESTS_3(MODE) ST_REQUEST_##MODE(0, "v[80:83]") ST_REQUEST_##MODE(1, "v[84:87]") ST_REQUEST_##MODE(2, "v[88:91]")
 #define ST_REQUESTS_4(MODE) ST_REQUESTS_3(MODE) ST_REQUEST_##MODE(3, "v[92:95]")
 #define ST_REQUEST_0(U, QUAD) ST_REQUEST_AW(U, QUAD)
 #define ST_REQUEST_1(U, QUAD) ST_REQUEST_CT(U, QUAD)
 
+#ifdef ST_TUNED
 // layer k of parity P (Q the other one): on entry the pointers of layer k + 1 and of layer k - 1 have arrived, image P
 // holds layer k's activations and set Q layer k - 1's partial sums
 #define ST_LAYER(P, Q, MODE, M, NEED, STW, LPI)                                                                       \
@@ -534,6 +562,54 @@ static_assert(kStLdsBytes == kMaxLds, "the layout fills the LDS of a CU");
     ST_LAST_LAYER(1, 0, MODE, M)                                                                                      \
     "12:\n"                                                                                                           \
     "s_waitcnt vmcnt(0)\n"
+#else
+// layer k of parity P (Q the other one): on entry the pointers of layer k + 1 and of layer k - 1 have arrived, image P
+// holds layer k's activations and set Q layer k - 1's partial sums.  Behind the elements the next layer's activations
+// are staged and the rows of the layer in front added up.
+#define ST_LAYER(P, Q, MODE, M, NEED, STW, LPI)                                                                       \
+    ST_XREQUESTS                                                                                                      \
+    ST_ITEMS_##M(MODE, P, Q, NEED, LPI)                                                                               \
+    ST_PRIO("3")                                                                                                      \
+    "s_waitcnt vmcnt(" #STW ")\n"                                                                                     \
+    ST_STAGE(Q)                                                                                                       \
+    "s_cmp_eq_u32 %[k], 0\n"                                                                                          \
+    "s_cbranch_scc1 93f\n"                                                                                            \
+    ST_ROWS(Q)                                                                                                        \
+    "93:\n"                                                                                                           \
+    "s_add_u32 %[k], %[k], 1\n"                                                                                       \
+    ST_POINTERS                                                                                                       \
+    "s_waitcnt lgkmcnt(0)\n"                                                                                          \
+    "s_barrier\n"
+
+// every layer asks for the layer behind it (the last one for itself again: the pointers are clamped)
+#define ST_BODY(MODE, M, NEED, STW, LPI)                                                                              \
+    "s_mov_b32 %[k], 0\n"                                                                                             \
+    "s_mov_b32 %[kn], 0\n"                                                                                            \
+    "s_load_dwordx2 %[cn], %[dc], %[kn]\n"                                                                            \
+    "s_load_dwordx2 %[xn], %[dx], %[kn]\n"                                                                            \
+    "s_waitcnt lgkmcnt(0)\n"                                                                                          \
+    ST_XREQUESTS                                                                                                      \
+    ST_REQUESTS_##M(MODE)                                                                                             \
+    "s_waitcnt vmcnt(" #STW ")\n"                                                                                     \
+    ST_STAGE(0)                                                                                                       \
+    ST_POINTERS                                                                                                       \
+    "s_waitcnt lgkmcnt(0)\n"                                                                                          \
+    "s_barrier\n"                                                                                                     \
+    "10:\n"                                                                                                           \
+    ST_LAYER(0, 1, MODE, M, NEED, STW, LPI)                                                                           \
+    "s_cmp_ge_u32 %[k], %[count]\n"                                                                                   \
+    "s_cbranch_scc1 11f\n"                                                                                            \
+    ST_LAYER(1, 0, MODE, M, NEED, STW, LPI)                                                                           \
+    "s_cmp_lt_u32 %[k], %[count]\n"                                                                                   \
+    "s_cbranch_scc1 10b\n"                                                                                            \
+    /* the last layer's rows: its partial sums are in set 1 (an even number of layers) or set 0 */                    \
+    ST_ROWS(1)                                                                                                        \
+    "s_branch 12f\n"                                                                                                  \
+    "11:\n"                                                                                                           \
+    ST_ROWS(0)                                                                                                        \
+    "12:\n"                                                                                                           \
+    "s_waitcnt vmcnt(0)\n"
+#endif
 
 // what the loop reads and the registers it works in
 #ifndef ST_MFMA
@@ -560,8 +636,13 @@ static_assert(kStLdsBytes == kMaxLds, "the layout fills the LDS of a CU");
     [count] "s"(s_count), [last] "s"(s_count - 1), [nitems] "s"(s_nitems), [rl] "s"(rl), [xo0] "v"(xo[0]), [xo1] "v"(xo[1]),\
     [sa0] "v"(sa[0]), [sa1] "v"(sa[1]), [sa2] "v"(sa[2]), [sa3] "v"(sa[3]), [sa4] "v"(sa[4]), [sa5] "v"(sa[5]),       \
     [sa6] "v"(sa[6]), [sa7] "v"(sa[7]), [stm0] "s"(stm[0]), [stm1] "s"(stm[1]), [rs] "v"(rs), [oo] "v"(oo),           \
-    [rstep] "s"(s_rstep), [ostep] "s"(s_ostep), [nr] "s"(s_nr), [rm0] "s"(rm[0]), [rm1] "s"(rm[1]), [rm2] "s"(rm[2]), [rm3] "s"(rm[3]),         \
+    [rstep] "s"(s_rstep), ST_IN_OSTEP [nr] "s"(s_nr), [rm0] "s"(rm[0]), [rm1] "s"(rm[1]), [rm2] "s"(rm[2]), [rm3] "s"(rm[3]),         \
     [l63] "s"(0x8000000000000000ull)
+#ifdef ST_TUNED
+#define ST_IN_OSTEP [ostep] "s"(s_ostep),
+#else
+#define ST_IN_OSTEP
+#endif
 #define ST_IN_ITEM(U) [vo##U] "v"(vo[U]), [xa##U] "v"(xa[U]), [pa##U] "v"(pa[U]), [first##U] "s"(first[U]), [keep##U] "s"(keep[U])
 #define ST_IN_ITEM_CT(U) [co##U] "v"(co[U]), [cm##U] "s"(cm[U])
 #define ST_CLOBBERS                                                                                                   \
@@ -666,9 +747,13 @@ __global__ __launch_bounds__(kStThreads) void matvec_steady_kernel(
         }
     }
 
-    // ---- the rows: added up by the waves that hold the fewest elements (all sixteen when the shares are equal), the
-    // i-th of them taking rows i, i + their number, ...
+    // ---- the rows: added up by waves 0-7, or (ST_TUNED) by the waves that hold the fewest elements (all sixteen when the
+    // shares are equal), the i-th of them taking rows i, i + their number, ...
+#ifdef ST_TUNED
     const int first_row_wave = extra, row_waves = kStWaves - extra;
+#else
+    const int first_row_wave = 0, row_waves = 8;
+#endif
     const int ri = wave - first_row_wave;
     const uint32_t rs = (uint32_t)kStPartBase + 4u * (uint32_t)(max(ri, 0) * npr + lane);
     const uint32_t oo = 2u * (uint32_t)(row0 + max(ri, 0));
@@ -687,7 +772,8 @@ __global__ __launch_bounds__(kStThreads) void matvec_steady_kernel(
     auto uni = [](uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)v); };
     auto uni64 = [&](uint64_t v) { return (uint64_t)uni((uint32_t)v) | ((uint64_t)uni((uint32_t)(v >> 32)) << 32); };
     rl = uni(rl);
-    const uint32_t s_nitems = uni((uint32_t)nitems), s_nr = uni(nr), s_rstep = uni(rstep), s_ostep = uni(ostep), s_count = uni((uint32_t)count);
+    const uint32_t s_nitems = uni((uint32_t)nitems), s_nr = uni(nr), s_rstep = uni(rstep), s_count = uni((uint32_t)count);
+    [[maybe_unused]] const uint32_t s_ostep = uni(ostep);
 #pragma unroll
     for (int u = 0; u < MAXI; u++) first[u] = uni64(first[u]), keep[u] = uni64(keep[u]), cm[u] = uni(cm[u]);
 #pragma unroll

@@ -520,6 +520,24 @@ def test_steady_kernel_under_other_interleavings_and_latencies(steady_isa, oracl
 
 
 @pytest.fixture(scope="module")
+def steady_tuned_isa(tmp_path_factory):
+    return compile_to_assembly(tmp_path_factory, "matvec_steady", extra=("-DST_TUNED",))
+
+
+@pytest.mark.parametrize("m,n,count,S,mode", [(33, 4096 + 768, 3, 8, 0), (33, 4096 + 768, 2, 8, 1), (300, 64, 4, 6, 0), (7, 704, 1, 6, 1),
+                                              (512, 6144, 2, 8, 1), (1024, 2048 + 64, 5, 8, 0), (8192, 8192, 2, 8, 0), (64, 16384, 2, 8, 1)])
+def test_steady_kernel_with_the_untimed_changes(steady_tuned_isa, oracle, m, n, count, S, mode):
+    """The -DST_TUNED build: the activation reload without a wait of its own, the rows added by the waves with the fewest
+    elements, the next activations staged behind the first element, and a last layer that asks for nothing."""
+    run_steady(steady_tuned_isa, oracle, m, n, count, S, mode, blocks=sorted({0, 1, (m - 1) // (2 * ((m + 2 * CUS - 1) // (2 * CUS)))}))
+
+
+@pytest.mark.parametrize("burst,latency", [(1, (3000, 300)), (64, (5, 2)), (3, (40, 400))])
+def test_steady_kernel_with_the_untimed_changes_under_other_interleavings(steady_tuned_isa, oracle, burst, latency):
+    run_steady(steady_tuned_isa, oracle, 100, 4096 + 64 * 7, 3, 8, 1, blocks=[0, 1], burst=burst, latency=latency)
+
+
+@pytest.fixture(scope="module")
 def steady_mfma_isa(tmp_path_factory):
     return compile_to_assembly(tmp_path_factory, "matvec_steady", extra=("-DST_MFMA",))
 
