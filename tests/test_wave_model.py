@@ -525,7 +525,7 @@ def steady_tuned_isa(tmp_path_factory):
 
 
 @pytest.mark.parametrize("m,n,count,S,mode", [(33, 4096 + 768, 3, 8, 0), (33, 4096 + 768, 2, 8, 1), (300, 64, 4, 6, 0), (7, 704, 1, 6, 1),
-                                              (512, 6144, 2, 8, 1), (1024, 2048 + 64, 5, 8, 0), (8192, 8192, 2, 8, 0), (64, 16384, 2, 8, 1)])
+                                              (1024, 2048 + 64, 5, 8, 0), (8192, 8192, 2, 8, 0), (64, 16384, 2, 8, 1)])
 def test_steady_kernel_with_the_untimed_changes(steady_tuned_isa, oracle, m, n, count, S, mode):
     """The -DST_TUNED build: the activation reload without a wait of its own, the rows added by the waves with the fewest
     elements, the next activations staged behind the first element, and a last layer that asks for nothing."""
@@ -553,7 +553,7 @@ def steady_roll_isa(tmp_path_factory):
     return compile_to_assembly(tmp_path_factory, "matvec_steady", extra=("-DST_ROLL",))
 
 
-@pytest.mark.parametrize("m,n,count,S,mode", [(33, 4096 + 768, 3, 8, 0), (300, 64, 2, 6, 1), (1024, 2048 + 64, 3, 8, 1), (8192, 8192, 2, 8, 0)])
+@pytest.mark.parametrize("m,n,count,S,mode", [(33, 4096 + 768, 3, 8, 0), (300, 64, 2, 6, 1), (1024, 2048 + 64, 3, 8, 1)])
 def test_steady_kernel_with_the_decode_as_a_rolling_pipeline(steady_roll_isa, oracle, m, n, count, S, mode):
     """The -DST_ROLL build of the same kernel (sixteen gathers kept in flight, two products and two new gathers a step)."""
     run_steady(steady_roll_isa, oracle, m, n, count, S, mode, blocks=sorted({0, (m - 1) // (2 * ((m + 2 * CUS - 1) // (2 * CUS)))}))
@@ -609,7 +609,7 @@ def steady_mfma_roll_isa(tmp_path_factory):
     return compile_to_assembly(tmp_path_factory, "matvec_steady", extra=("-DST_MFMA", "-DST_ROLL"))
 
 
-@pytest.mark.parametrize("m,n,count,S,mode", [(33, 4096 + 768, 3, 8, 0), (300, 64, 2, 6, 1), (1024, 2048 + 64, 3, 8, 1), (8192, 8192, 2, 8, 0)])
+@pytest.mark.parametrize("m,n,count,S,mode", [(33, 4096 + 768, 3, 8, 0), (300, 64, 2, 6, 1), (1024, 2048 + 64, 3, 8, 1)])
 def test_steady_kernel_with_both_the_matrix_unit_and_the_rolling_pipeline(steady_mfma_roll_isa, oracle, m, n, count, S, mode):
     run_steady(steady_mfma_roll_isa, oracle, m, n, count, S, mode, blocks=sorted({0, (m - 1) // (2 * ((m + 2 * CUS - 1) // (2 * CUS)))}))
 
@@ -668,7 +668,7 @@ def _matvec_geometry(m, n):
     return rpb, rw_tail, items_tail, magic, 65536 + 2 * n + 4 * (n // 64) * rpb
 
 
-@pytest.mark.parametrize("prologue,m,n,mode", [("silu", 40, 2048 + 320, 0), ("rmsnorm", 70, 4096, 1), ("rmsnorm", 33, 64 * 7, 0)])
+@pytest.mark.parametrize("prologue,m,n,mode", [("silu", 40, 2048 + 320, 0), ("rmsnorm", 40, 2048 + 64, 1), ("rmsnorm", 33, 64 * 7, 0)])
 def test_fused_prologue_kernels_equal_the_separate_kernels(matvec_isa, glue_isa, prologue, m, n, mode):
     """`matvec_fused_kernel` with the SiLU gate or the residual add + RMS norm in its prologue (`csrc/matvec.hip`) against
     the stand-alone element-wise kernel (`csrc/decode_glue.hip`) followed by the plain mat-vec kernel, all three run in the
@@ -872,7 +872,7 @@ def test_rope_and_cache_kernel(glue_isa, heads, hd, max_len, pos):
     assert np.array_equal(k_cache.view(np.uint16), k_want.view(np.uint16)) and np.array_equal(v_cache.view(np.uint16), v_want.view(np.uint16))
 
 
-@pytest.mark.parametrize("m,n,mode,which", [(40, 2048 + 320, 0, "all"), (70, 4096, 1, "all"), (33, 64 * 7, 0, "none"), (20, 1024, 1, "out")])
+@pytest.mark.parametrize("m,n,mode,which", [(40, 2048 + 320, 0, "all"), (33, 64 * 7, 1, "none"), (20, 1024, 1, "out")])
 def test_affine_kernel_applies_the_factorisation(matvec_isa, oracle, m, n, mode, which):
     """`matvec_affine_kernel<S, MODE, plain>` (`csrc/matvec.hip`): y = s_out * (W (s_in * a)) + b_out * sum(a) + b_in . a with
     the factorisation's four vectors (quantize_hf.py:167), any of them absent; against the same in double on the decoded
