@@ -110,3 +110,19 @@ def test_carry_mode_and_timing_switches():
         rptc_kernels.set_carry_mode(3)
     prev = rptc_kernels.set_timing(False)
     rptc_kernels.set_timing(prev)
+
+
+def test_bench_aids_library_exports_what_bench_binds():
+    """`bench.py` binds the measurement aids by name when it starts: a missing symbol would end the benchmark before its
+    first line.  (Loading the library and setting argument types touches no device.)"""
+    import importlib.util
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    path = os.path.join(root, "bench_aids", "librptc_bench_aids.so")
+    if not os.path.exists(path):
+        pytest.skip("bench_aids/librptc_bench_aids.so is not built")
+    spec = importlib.util.spec_from_file_location("bench_for_test", os.path.join(root, "bench.py"))
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    lib = bench.aids_library()
+    for name in ("rptc_probe_empty", "rptc_probe_read", "rptc_probe_read_chain", "rptc_probe_lds", "rptc_probe_valu", "rptc_probe_decode"):
+        assert hasattr(lib, name)
