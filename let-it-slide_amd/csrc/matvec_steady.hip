@@ -49,6 +49,13 @@ static_assert(kStLdsBytes == kMaxLds, "the layout fills the LDS of a CU");
 #if (defined(ST_MFMA) || defined(ST_ROLL)) && !defined(ST_TUNED)
 #define ST_TUNED
 #endif
+// ST_TUNED is three switches that can be timed one by one: the reload's wait, who adds the rows, and the order of a
+// layer's chores (staging behind the first element, a last layer that asks for nothing)
+#ifdef ST_TUNED
+#define ST_T_RELOAD
+#define ST_T_ROWS
+#define ST_T_FLOW
+#endif
 #ifndef ST_MFMA
 #define ST_X0 "v96"
 #define ST_X2 "v97"
@@ -102,10 +109,10 @@ static_assert(kStLdsBytes == kMaxLds, "the layout fills the LDS of a CU");
 #ifndef ST_MFMA
 #define ST_RD2(LO, HI, BASE, OFF, P)                                                                                  \
     "ds_read2st64_b32 v[" #LO ":" #HI "], " BASE " offset0:" #P "*128+" #OFF " offset1:" #P "*128+" #OFF "+1\n"
-// ST_TUNED: LDS reads complete in order and the decode block's first wait (at most 8 reads in flight, its own) comes
+// ST_T_RELOAD: LDS reads complete in order and the decode block's first wait (at most 8 reads in flight, its own) comes
 // before its first product, which is the first instruction to read an activation register: the reload then needs no wait
 // of its own
-#ifdef ST_TUNED
+#ifdef ST_T_RELOAD
 #define ST_RELOAD_WAIT ""
 #else
 #define ST_RELOAD_WAIT "s_waitcnt lgkmcnt(0)\n"
@@ -399,8 +406,8 @@ static_assert(kStLdsBytes == kMaxLds, "the layout fills the LDS of a CU");
 // ---- the rows of the layer in front: a wave adds a row's n / 64 partial sums (lanes i, i + 64, i + 128, i + 192 in
 // that order, then across the lanes with DPP adds: rows of 16, row 0 into 1 and 2 into 3, rows 0-1 into 2-3), round
 // once to fp16 and lane 63 stores.  P: parity of the set that is read.
-// a row wave's next row: eight rows further, or (ST_TUNED) as many as there are row waves
-#ifdef ST_TUNED
+// a row wave's next row: eight rows further, or (ST_T_ROWS) as many as there are row waves
+#ifdef ST_T_ROWS
 #define ST_NEXT_ROW "v_add_u32 %[g1], %[ostep], %[g1]\n"
 #else
 #define ST_NEXT_ROW "v_add_u32 %[g1], 16, %[g1]\n"
@@ -471,7 +478,7 @@ static_assert(kStLdsBytes == kMaxLds, "the layout fills the LDS of a CU");
     "global_load_dwordx4 v[72:75], %[xo0], %[xn]\n"                                                                   \
     "global_load_dwordx4 v[76:79], %[xo1], %[xn]\n"
 
-#ifdef ST_TUNED
+#ifdef ST_T_FLOW
 // The next layer's activations are staged behind the first element: their requests went out at the top of the layer,
 // and only the first element's next request has been made since (LPI requests may stay in flight).
 #define ST_EARLY_STAGE(Q, LPI) "s_waitcnt vmcnt(" #LPI ")\n" ST_STAGE(Q)
@@ -500,7 +507,7 @@ static_assert(kStLdsBytes == kMaxLds, "the layout fills the LDS of a CU");
 #define ST_REQUEST_0(U, QUAD) ST_REQUEST_AW(U, QUAD)
 #define ST_REQUEST_1(U, QUAD) ST_REQUEST_CT(U, QUAD)
 
-#ifdef ST_TUNED
+#ifdef ST_T_FLOW
 // layer k of parity P (Q the other one): on entry the pointers of layer k + 1 and of layer k - 1 have arrived, image P
 // holds layer k's activations and set Q layer k - 1's partial sums
 #define ST_LAYER(P, Q, MODE, M, NEED, STW, LPI)                                                                       \
@@ -638,7 +645,7 @@ static_assert(kStLdsBytes == kMaxLds, "the layout fills the LDS of a CU");
     [sa6] "v"(sa[6]), [sa7] "v"(sa[7]), [stm0] "s"(stm[0]), [stm1] "s"(stm[1]), [rs] "v"(rs), [oo] "v"(oo),           \
     [rstep] "s"(s_rstep), ST_IN_OSTEP [nr] "s"(s_nr), [rm0] "s"(rm[0]), [rm1] "s"(rm[1]), [rm2] "s"(rm[2]), [rm3] "s"(rm[3]),         \
     [l63] "s"(0x8000000000000000ull)
-#ifdef ST_TUNED
+#ifdef ST_T_ROWS
 #define ST_IN_OSTEP [ostep] "s"(s_ostep),
 #else
 #define ST_IN_OSTEP
@@ -747,9 +754,9 @@ __global__ __launch_bounds__(kStThreads) void matvec_steady_kernel(
         }
     }
 
-    // ---- the rows: added up by waves 0-7, or (ST_TUNED) by the waves that hold the fewest elements (all sixteen when the
+    // ---- the rows: added up by waves 0-7, or (ST_T_ROWS) by the waves that hold the fewest elements (all sixteen when the
     // shares are equal), the i-th of them taking rows i, i + their number, ...
-#ifdef ST_TUNED
+#ifdef ST_T_ROWS
     const int first_row_wave = extra, row_waves = kStWaves - extra;
 #else
     const int first_row_wave = 0, row_waves = 8;
