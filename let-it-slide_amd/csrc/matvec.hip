@@ -1127,6 +1127,14 @@ static int launch_matvec(const int32_t *compressed, const uint16_t *codebook, co
             else RPTC_LAUNCH(RPTC_CONTINUOUS, true);
             return t.end();
         }
+#ifdef RPTC_MV_ONE
+        // the same layer through the chain kernel's hand-written body (an experiment until it is timed)
+        if (matvec_one_fits(a.n, a.rows_per_block, a.items_tail)) {
+            rc = matvec_one_launch(a_comp, a_cb, a_x, out, a.m, a.n, a.rows_per_block, a.rw_tail, a.items_tail, a.full_magic, grid, S,
+                                   carry_mode, s);
+            return rc ? rc : t.end();
+        }
+#endif
     }
     if (carry_mode == RPTC_AS_WRITTEN) RPTC_LAUNCH(RPTC_AS_WRITTEN, false);
     else RPTC_LAUNCH(RPTC_CONTINUOUS, false);

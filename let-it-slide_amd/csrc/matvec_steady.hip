@@ -815,11 +815,252 @@ __global__ __launch_bounds__(kStThreads) void matvec_steady_kernel(
     }
 }
 
+#ifndef ST_MFMA
+// ---------------------------------------------------------------- one layer per launch with the same hand-written body
+// (behind -DRPTC_MV_ONE in matvec.hip's launcher until it is timed).  The launch is the per-launch op's
+// (rptc_decompress_matvec_16_{S}_1: one layer, no descriptors); what it takes from the chain kernel is the decode of a
+// wave's elements with everything about them worked out in front, the activation reload as two-dword reads and the
+// rows as a counted loop - the per-launch kernel's own element loop spends 86 scalar and 146 vector instructions an
+// element where this body spends 14 and 105.  The prologue is written for a short way to the first request: the
+// activation and stream requests go out first (ordinary loads: the compiler waits for them in front of the block),
+// the table and the rest of the geometry while they are on their way; the ragged slab's lane numbers and slots come
+// from a multiplication (a 16-bit reciprocal of the ragged row's length from the host) instead of a division.
+#define ST_ONE_ITEM_0(U) ST_ITEM_0(U, "%[e" #U "x]", "%[e" #U "y]", "%[e" #U "z]", "%[e" #U "w]", 0, 63, "")
+#define ST_ONE_ITEM_1(U) ST_ITEM_1(U, "%[e" #U "x]", "%[e" #U "y]", "%[e" #U "z]", "%[e" #U "w]", 0, 63, "")
+#define ST_ONE_ITEMS_3(MODE) ST_ONE_ITEM_##MODE(0) ST_ONE_ITEM_##MODE(1) ST_ONE_ITEM_##MODE(2)
+#define ST_ONE_ITEMS_4(MODE) ST_ONE_ITEMS_3(MODE) ST_ONE_ITEM_##MODE(3)
+#define ST_ONE_BODY(MODE, M)                                                                                          \
+    "s_waitcnt lgkmcnt(0)\n"                                                                                          \
+    "s_barrier\n"                                                                                                     \
+    ST_ONE_ITEMS_##M(MODE)                                                                                            \
+    ST_PRIO("3")                                                                                                      \
+    "s_waitcnt lgkmcnt(0)\n"                                                                                          \
+    "s_barrier\n"                                                                                                     \
+    ST_ROWS(0)                                                                                                        \
+    "s_waitcnt vmcnt(0)\n"
+#define ST_ONE_OUT                                                                                                    \
+    [a0] "=&v"(a0), [a1] "=&v"(a1), [a2] "=&v"(a2), [a3] "=&v"(a3), [cy] "=&v"(cy), [g0] "=&v"(g0), [g1] "=&v"(g1),  \
+    [g2] "=&v"(g2), [g3] "=&v"(g3), [t0] "=&v"(t0), [t1] "=&v"(t1), [t2] "=&v"(t2), [t3] "=&v"(t3), [t4] "=&v"(t4),  \
+    [t5] "=&v"(t5), [t6] "=&v"(t6), [t7] "=&v"(t7), [u0] "=&v"(u0), [u1] "=&v"(u1), [u2] "=&v"(u2), [u3] "=&v"(u3),  \
+    [u4] "=&v"(u4), [u5] "=&v"(u5), [u6] "=&v"(u6), [u7] "=&v"(u7), [xb] "=&v"(xb), [j] "=&s"(j)
+#define ST_ONE_IN                                                                                                     \
+    [lane4] "v"(lane4), [mask] "s"(0xFF00u), [sel] "s"(0x0C0C0700u), [nitems] "s"(s_nitems), [rl] "s"(rl), [rs] "v"(rs), \
+    [oo] "v"(oo), [rstep] "s"(s_rstep), ST_IN_OSTEP [nr] "s"(s_nr), [rm0] "s"(rm[0]), [rm1] "s"(rm[1]), [rm2] "s"(rm[2]), \
+    [rm3] "s"(rm[3]), [l63] "s"(0x8000000000000000ull), [op] "s"(out_address)
+#define ST_ONE_IN_ITEM(U)                                                                                             \
+    [xa##U] "v"(xa[U]), [pa##U] "v"(pa[U]), [first##U] "s"(first[U]), [keep##U] "s"(keep[U]), [e##U##x] "v"(e[U].x),  \
+    [e##U##y] "v"(e[U].y), [e##U##z] "v"(e[U].z), [e##U##w] "v"(e[U].w)
+#define ST_ONE_IN_ITEM_CT(U) [cw##U] "v"(cw[U]), [cm##U] "s"(cm[U])
+#define ST_ONE_CLOBBERS                                                                                               \
+    "memory", "vcc", "scc", "v96", "v97", "v98", "v99", "v100", "v101", "v102", "v103", "v104", "v105", "v106", "v107", \
+    "v108", "v109", "v110", "v111", "v112", "v113", "v114", "v115", "v116", "v117", "v118", "v119", "v120", "v121", "v122", \
+    "v123", "v124", "v125", "v126", "v127"
+
+template <int S, int MODE, int MAXI>
+__global__ __launch_bounds__(kStThreads) void matvec_one_kernel(
+    const uint4 *__restrict__ comp, const uint32_t *__restrict__ codebook, const uint4 *__restrict__ x, int arg_m, int arg_n,
+    int rows_per_block, int rw_tail, int items_tail, uint32_t full_magic, uint32_t tail_magic, uint16_t *__restrict__ out)
+{
+    static_assert(MAXI == 3 || MAXI == 4, "a wave holds three or four elements");
+    extern __shared__ uint32_t lds[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t lane4 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds)) + lane * 4;   // the table is at LDS address 0
+    const int m = arg_m, n = arg_n;
+    const int T = n >> 11, Lt = (n & 2047) >> 6, npr = n >> 6, n8 = n >> 3;
+    const int items_full = rows_per_block >> 1;
+    const int row0 = blockIdx.x * rows_per_block;
+    const int rows = min(rows_per_block, m - row0);
+
+    // ---- requests first: a thread's share of the activations (16 bytes at 8 idx, two of them) ...
+    const int i0 = tid, i1 = tid + kStThreads;
+    const uint4 xv0 = x[min(i0, n8 - 1)], xv1 = x[min(i1, n8 - 1)];
+    // ... and this wave's elements: equal shares, the first total % 16 waves one more.  Lane -> (row inside the item,
+    // element inside the row): two rows of 32 in a full slab; in the ragged slab lane / Lt rows of Lt, the quotient from
+    // the host's reciprocal (exact for lane < 64); lanes past the item's last whole row idle on element 0
+    const int total = T * items_full + items_tail;
+    const int per_wave = (int)((uint32_t)total / kStWaves), extra = (int)((uint32_t)total % kStWaves);
+    const int it_begin = wave * per_wave + min(wave, extra);
+    const int nitems = per_wave + (wave < extra ? 1 : 0);                // at most MAXI: the host checks
+    const int sub_full = lane >> 5, l_full = lane & 31;
+    int sub_tail = (int)(((uint32_t)lane * tail_magic) >> 16), l_tail = lane - sub_tail * Lt;
+    if (sub_tail >= rw_tail) l_tail = 0;
+    uint4 e[MAXI];
+    uint32_t cw[MAXI], cm[MAXI], xa[MAXI], pa[MAXI];
+    uint64_t first[MAXI], keep[MAXI];
+    uint32_t rl = 0;
+    int prev_slab = -1;
+    const uint64_t first_tail = __builtin_amdgcn_ballot_w64(l_tail == 0);
+#pragma unroll
+    for (int u = 0; u < MAXI; u++) {
+        const int it = it_begin + u;
+        const bool mine = u < nitems;
+        int slab = items_full == 1 ? it : (int)__umulhi((uint32_t)it, full_magic);
+        slab = min(slab, T);
+        const int idx = it - slab * items_full;
+        const bool full = slab < T;
+        const int lanes = full ? 32 : Lt, rpi = full ? 2 : rw_tail;
+        const int sub = full ? sub_full : sub_tail, l = full ? l_full : l_tail;
+        const int row_first = idx * rpi;
+        const int rows_here = mine ? min(rpi, rows - row_first) : 0;          // <= 0: an element past the block's last row
+        const bool real = rows_here > 0;
+        const uint32_t elem0 = (uint32_t)slab * (uint32_t)m * 32u;
+        const uint32_t elem = real ? elem0 + (uint32_t)(row0 + row_first) * (uint32_t)lanes : 0u;
+        const uint32_t last = real ? (uint32_t)(rows_here * lanes - 1) : 0u;
+        {
+            typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+            const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(comp) + (elem + min((uint32_t)lane, last)));
+            e[u] = make_uint4(v.x, v.y, v.z, v.w);
+        }
+        if constexpr (MODE == RPTC_CONTINUOUS) {
+            // the word in front of a row: the last word of the row's lane 31 in the slab before
+            const bool prev = real && slab > 0;
+            const int sub_c = min(sub, max(rows_here, 1) - 1);
+            const uint32_t co = prev ? (((uint32_t)(slab - 1) * (uint32_t)m + (uint32_t)(row0 + row_first + sub_c)) * 32u + 31u) * 4u + 3u : 0u;
+            cw[u] = reinterpret_cast<const uint32_t *>(comp)[co];
+            cm[u] = prev ? ~0u : 0u;
+        } else {
+            cw[u] = cm[u] = 0u;
+        }
+        xa[u] = (uint32_t)kStTableBytes + 4u * (uint32_t)(1024 * slab + l);
+        pa[u] = (uint32_t)kStPartBase + 4u * (uint32_t)((row_first + sub) * npr + 32 * slab + l);
+        first[u] = full ? 0x0000000100000001ull : first_tail;
+        const int nact = max(rows_here, 0) * lanes;
+        keep[u] = nact >= 64 ? ~0ull : (1ull << nact) - 1ull;
+        if (mine && slab != prev_slab) rl |= 1u << u;
+        if (mine) prev_slab = slab;
+    }
+
+    // ---- the table: rows 16 wave .. 16 wave + 15 are this wave's to write (as in the chain kernel)
+    constexpr int kRowsPerWave = 256 / kStWaves;
+    {
+        uint32_t cbv[kRowsPerWave];
+#pragma unroll
+        for (int i = 0; i < kRowsPerWave; i++) cbv[i] = codebook[(kRowsPerWave * wave + i) & ((1 << S) - 1)];
+        const uint32_t table_sign = (uint32_t)((kRowsPerWave * wave) >> 7) << 15;
+#pragma unroll
+        for (int i = 0; i < kRowsPerWave; i++) lds[(kRowsPerWave * wave + i) * 64 + lane] = (cbv[i] & 0xFFFF7FFFu) | table_sign;
+    }
+
+    // ---- the activations into the image (slot i * n8 + idx for word i of the 16 bytes at 8 idx, inference.cu:215-221;
+    // the ragged slab at the full slabs' stride: slot 32 q + l for its q-th step's lane l)
+    {
+        uint32_t *image = lds + kStTableBytes / 4;
+        auto place = [&](int P, uint32_t v) {
+            int pos = P;
+            if (P >= 1024 * T) {
+                const int r = P - 1024 * T, q = (int)(((uint32_t)r * tail_magic) >> 16);
+                pos = 1024 * T + 32 * q + (r - q * Lt);
+            }
+            image[pos] = v;
+        };
+        if (i0 < n8) {
+            place(i0, xv0.x), place(n8 + i0, xv0.y), place(2 * n8 + i0, xv0.z), place(3 * n8 + i0, xv0.w);
+        }
+        if (i1 < n8) {
+            place(i1, xv1.x), place(n8 + i1, xv1.y), place(2 * n8 + i1, xv1.z), place(3 * n8 + i1, xv1.w);
+        }
+    }
+
+    // ---- the rows (as in the chain kernel)
+#ifdef ST_T_ROWS
+    const int first_row_wave = extra, row_waves = kStWaves - extra;
+#else
+    const int first_row_wave = 0, row_waves = 8;
+#endif
+    const int ri = wave - first_row_wave;
+    const uint32_t rs = (uint32_t)kStPartBase + 4u * (uint32_t)(max(ri, 0) * npr + lane);
+    const uint32_t oo = 2u * (uint32_t)(row0 + max(ri, 0));
+    const uint32_t rstep = 4u * (uint32_t)(row_waves * npr), ostep = 2u * (uint32_t)row_waves;
+    const uint32_t nr = ri >= 0 && ri < row_waves && ri < rows ? (uint32_t)(rows - ri + row_waves - 1) / (uint32_t)row_waves : 0u;
+    uint64_t rm[4];
+#pragma unroll
+    for (int c = 0; c < 4; c++) rm[c] = __builtin_amdgcn_ballot_w64(lane + 64 * c < npr);
+
+    auto uni = [](uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)v); };
+    auto uni64 = [&](uint64_t v) { return (uint64_t)uni((uint32_t)v) | ((uint64_t)uni((uint32_t)(v >> 32)) << 32); };
+    rl = uni(rl);
+    const uint32_t s_nitems = uni((uint32_t)nitems), s_nr = uni(nr), s_rstep = uni(rstep);
+    [[maybe_unused]] const uint32_t s_ostep = uni(ostep);
+#pragma unroll
+    for (int u = 0; u < MAXI; u++) first[u] = uni64(first[u]), keep[u] = uni64(keep[u]), cm[u] = uni(cm[u]);
+#pragma unroll
+    for (int c = 0; c < 4; c++) rm[c] = uni64(rm[c]);
+    const uint64_t out_address = uni64(reinterpret_cast<uint64_t>(out));
+
+    uint32_t a0, a1, a2, a3, cy, g0, g1, g2, g3, t0, t1, t2, t3, t4, t5, t6, t7, u0, u1, u2, u3, u4, u5, u6, u7, xb, j;
+    if constexpr (MODE == RPTC_AS_WRITTEN && MAXI == 3) {
+        asm volatile(ST_ONE_BODY(0, 3) : ST_ONE_OUT : ST_ONE_IN, ST_ONE_IN_ITEM(0), ST_ONE_IN_ITEM(1), ST_ONE_IN_ITEM(2) : ST_ONE_CLOBBERS);
+    } else if constexpr (MODE == RPTC_AS_WRITTEN) {
+        asm volatile(ST_ONE_BODY(0, 4)
+                     : ST_ONE_OUT
+                     : ST_ONE_IN, ST_ONE_IN_ITEM(0), ST_ONE_IN_ITEM(1), ST_ONE_IN_ITEM(2), ST_ONE_IN_ITEM(3)
+                     : ST_ONE_CLOBBERS);
+    } else if constexpr (MAXI == 3) {
+        uint32_t own;
+        asm volatile(ST_ONE_BODY(1, 3)
+                     : ST_ONE_OUT, [own] "=&v"(own)
+                     : ST_ONE_IN, ST_ONE_IN_ITEM(0), ST_ONE_IN_ITEM(1), ST_ONE_IN_ITEM(2), ST_ONE_IN_ITEM_CT(0), ST_ONE_IN_ITEM_CT(1),
+                       ST_ONE_IN_ITEM_CT(2)
+                     : ST_ONE_CLOBBERS);
+    } else {
+        uint32_t own;
+        asm volatile(ST_ONE_BODY(1, 4)
+                     : ST_ONE_OUT, [own] "=&v"(own)
+                     : ST_ONE_IN, ST_ONE_IN_ITEM(0), ST_ONE_IN_ITEM(1), ST_ONE_IN_ITEM(2), ST_ONE_IN_ITEM(3), ST_ONE_IN_ITEM_CT(0),
+                       ST_ONE_IN_ITEM_CT(1), ST_ONE_IN_ITEM_CT(2), ST_ONE_IN_ITEM_CT(3)
+                     : ST_ONE_CLOBBERS);
+    }
+}
+#endif
+
 template <typename F>
 static int st_set_lds_limit(F *kernel)
 {
     return (int)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds);
 }
+
+#ifndef ST_MFMA
+bool matvec_one_fits(int n, int rows_per_block, int items_tail)
+{
+    const int T = n >> 11, lt = (n & 2047) >> 6;
+    const int total = T * (rows_per_block >> 1) + items_tail;
+    return (T + (lt ? 1 : 0)) * 4096 <= kStImageBytes && (int64_t)rows_per_block * (n / 64) * 4 <= kStPartBytes &&
+           (total + kStWaves - 1) / kStWaves <= 4;
+}
+
+int matvec_one_launch(const uint32_t *comp, const uint32_t *codebook, const uint4 *x, uint16_t *out, int m, int n,
+                      int rows_per_block, int rw_tail, int items_tail, uint32_t full_magic, int grid, int S, int carry_mode,
+                      hipStream_t stream)
+{
+    const int T = n >> 11, lt = (n & 2047) >> 6;
+    const int total = T * (rows_per_block >> 1) + items_tail;
+    const int max_items = (total + kStWaves - 1) / kStWaves <= 3 ? 3 : 4;
+    const uint32_t tail_magic = lt ? 65536u / (uint32_t)lt + 1u : 0u;       // (v * magic) >> 16 == v / lt for v < 1024
+    auto a_comp = reinterpret_cast<const uint4 *>(comp);
+#define RPTC_ONE_GO(SS, MM, II)                                                                                      \
+    hipLaunchKernelGGL((matvec_one_kernel<SS, MM, II>), dim3(grid), dim3(kStThreads), kStLdsBytes, stream, a_comp,    \
+                       codebook, x, m, n, rows_per_block, rw_tail, items_tail, full_magic, tail_magic, out)
+#define RPTC_ONE_PICK(SS, MM)                     \
+    do {                                          \
+        if (max_items == 3) RPTC_ONE_GO(SS, MM, 3); \
+        else RPTC_ONE_GO(SS, MM, 4);              \
+    } while (0)
+    if (S == 6 && carry_mode == RPTC_AS_WRITTEN) RPTC_ONE_PICK(6, RPTC_AS_WRITTEN);
+    else if (S == 6) RPTC_ONE_PICK(6, RPTC_CONTINUOUS);
+    else if (carry_mode == RPTC_AS_WRITTEN) RPTC_ONE_PICK(8, RPTC_AS_WRITTEN);
+    else RPTC_ONE_PICK(8, RPTC_CONTINUOUS);
+#undef RPTC_ONE_PICK
+#undef RPTC_ONE_GO
+    return (int)hipGetLastError();
+}
+#else
+bool matvec_one_fits(int, int, int) { return false; }
+int matvec_one_launch(const uint32_t *, const uint32_t *, const uint4 *, uint16_t *, int, int, int, int, int, uint32_t, int, int, int, hipStream_t)
+{
+    return RPTC_ESHAPE;
+}
+#endif
 
 int prepare_matvec_steady()
 {
@@ -832,6 +1073,16 @@ int prepare_matvec_steady()
     RPTC_SET_LIMITS(3)
     RPTC_SET_LIMITS(4)
 #undef RPTC_SET_LIMITS
+#ifndef ST_MFMA
+#define RPTC_SET_LIMITS(MAXI)                                                                 \
+    if ((rc = st_set_lds_limit(matvec_one_kernel<6, RPTC_AS_WRITTEN, MAXI>))) return rc;        \
+    if ((rc = st_set_lds_limit(matvec_one_kernel<6, RPTC_CONTINUOUS, MAXI>))) return rc;        \
+    if ((rc = st_set_lds_limit(matvec_one_kernel<8, RPTC_AS_WRITTEN, MAXI>))) return rc;        \
+    if ((rc = st_set_lds_limit(matvec_one_kernel<8, RPTC_CONTINUOUS, MAXI>))) return rc;
+    RPTC_SET_LIMITS(3)
+    RPTC_SET_LIMITS(4)
+#undef RPTC_SET_LIMITS
+#endif
     return 0;
 }
 

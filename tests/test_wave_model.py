@@ -1151,3 +1151,53 @@ def test_batched_kernel_at_3_and_4_bits(matmul_isa, oracle, bits, m, n, batch, S
     want = x.astype(np.float64) @ W.T
     assert np.abs(out.astype(np.float64) - want).max() / (np.abs(want).max() + 1e-9) < 2e-3
     assert not arrived.any()
+
+
+def run_one_layer(isa, oracle, m, n, S, mode, blocks, seed=7, burst=8, latency=(400, 60)):
+    """`matvec_one_kernel<S, MODE, MAXI>` (`csrc/matvec_steady.hip`) as `matvec_one_launch` launches it: the per-launch op's
+    arguments plus the reciprocal of the ragged row's length, the chain kernel's fixed LDS layout."""
+    rng = np.random.default_rng(seed + m + n)
+    cb = (rng.standard_normal(2 << S) * 0.1).astype(np.float16)
+    comp = rng.integers(0, 256, m * n // 4, dtype=np.uint8)
+    x = (rng.standard_normal(n) * 0.5).astype(np.float16)
+    out = np.full(2 * m, 0xEE, dtype=np.uint8)
+    rpb, rw_tail, items_tail, magic, _ = _matvec_geometry(m, n)
+    T, lt = n >> 11, (n & 2047) >> 6
+    total = T * (rpb // 2) + items_tail
+    per_wave = -(-total // 16)
+    assert (T + (1 if lt else 0)) * 4096 <= 32768 and rpb * (n // 64) * 4 <= 16384 and per_wave <= 4
+    tail_magic = 65536 // lt + 1 if lt else 0
+    grid = (m + rpb - 1) // rpb
+    mem = wave_model.Memory()
+    c_at, cb_at, x_at, o_at = 0x7f40fffff000, 0x7f5000003400, 0x7f3ffff0fe00, 0x7f2ffffe0100
+    mem.add(c_at, comp, "stream")
+    mem.add(cb_at, cb.view(np.uint8).copy(), "codebook")
+    mem.add(x_at, x.view(np.uint8).copy(), "activations")
+    mem.add(o_at, out, "output")
+    wave_model.Wave.vm_latency, wave_model.Wave.lgkm_latency = latency
+    kernel = wave_model.Kernel(isa, "_ZN4rptc17matvec_one_kernelILi%dELi%dELi%dEE" % (S, mode, 3 if per_wave <= 3 else 4))
+    blocks = sorted({b for b in blocks if b < grid})
+    kernel.launch(mem, (grid,), 1024, [("ptr", c_at), ("ptr", cb_at), ("ptr", x_at), ("i32", m), ("i32", n), ("i32", rpb), ("i32", rw_tail),
+                                       ("i32", items_tail), ("u32", magic), ("u32", tail_magic), ("ptr", o_at)], lds_bytes=160 * 1024,
+                  groups=[(b, 0, 0) for b in blocks], seed=seed, burst=burst)
+    want = oracle.matvec(comp.view(np.uint32), cb, x, m, S, mode=mode)
+    got = out.view(np.float16).astype(np.float64)
+    touched = np.zeros(m, dtype=bool)
+    for b in blocks:
+        r0, r1 = b * rpb, min(m, (b + 1) * rpb)
+        touched[r0:r1] = True
+        err = np.abs(got[r0:r1] - want[r0:r1]).max() / (np.abs(want).max() + 1e-9)
+        assert err < 2e-3, f"workgroup {b}: rows {r0}..{r1 - 1} differ by {err:.3g} of the largest output"
+    assert (out.view(np.uint16)[~touched] == 0xEEEE).all()
+
+
+@pytest.mark.parametrize("m,n,S,mode", [(33, 4096 + 768, 8, 0), (33, 4096 + 768, 6, 1), (300, 64, 6, 0), (7, 704, 8, 1), (4096, 11008, 8, 0),
+                                        (11008, 4096, 8, 1), (8192, 8192, 8, 0), (64, 16384, 6, 1), (1000, 2048 + 64 * 31, 8, 1)])
+def test_one_layer_kernel_matches_the_oracle(steady_isa, oracle, m, n, S, mode):
+    rpb = 2 * ((m + 2 * CUS - 1) // (2 * CUS))
+    run_one_layer(steady_isa, oracle, m, n, S, mode, blocks=[0, 1, (m - 1) // rpb])
+
+
+@pytest.mark.parametrize("burst,latency", [(1, (3000, 300)), (64, (5, 2))])
+def test_one_layer_kernel_under_other_interleavings(steady_isa, oracle, burst, latency):
+    run_one_layer(steady_isa, oracle, 100, 4096 + 64 * 7, 8, 1, blocks=[0, 3], burst=burst, latency=latency)
