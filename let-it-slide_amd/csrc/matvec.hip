@@ -203,15 +203,6 @@ __device__ __forceinline__ uint4 pack8(const Halves8 &r)
 
 __device__ __forceinline__ float round_half(float v) { return half_bits_to_float(float_to_half_bits(v)); }
 
-__device__ __forceinline__ uint4 silu_mul8(const uint4 gate, const uint4 up)
-{
-    const uint32_t g[4] = {gate.x, gate.y, gate.z, gate.w}, u[4] = {up.x, up.y, up.z, up.w};
-    uint32_t r[4];
-#pragma unroll
-    for (int i = 0; i < 4; i++) r[i] = silu_mul_pair(g[i], u[i]);
-    return make_uint4(r[0], r[1], r[2], r[3]);
-}
-
 // A slab's 32 activation pairs of a lane from LDS: one address (XA) and 32 immediate offsets, 128 bytes (32 slots)
 // apart, into XR[0..31].  The reads and their wait are ONE asm statement (a register such a read writes holds
 // nothing until the wait; between two statements the compiler may copy or reuse it), and the outputs are
@@ -1131,7 +1122,7 @@ static int launch_matvec(const int32_t *compressed, const uint16_t *codebook, co
         // the same layer through the chain kernel's hand-written body (an experiment until it is timed)
         if (matvec_one_fits(a.n, a.rows_per_block, a.items_tail)) {
             rc = matvec_one_launch(a_comp, a_cb, a_x, out, a.m, a.n, a.rows_per_block, a.rw_tail, a.items_tail, a.full_magic, grid, S,
-                                   carry_mode, s);
+                                   carry_mode, false, s);
             return rc ? rc : t.end();
         }
 #endif
@@ -1177,6 +1168,13 @@ static int launch_matvec_fused(const int32_t *compressed, const uint16_t *codebo
             else RPTC_LAUNCH(RPTC_CONTINUOUS, true);
             return t.end();
         }
+#ifdef RPTC_MV_ONE
+        if (matvec_one_fits(a.n, a.rows_per_block, a.items_tail)) {
+            rc = matvec_one_launch(a_comp, a_cb, a_x, out, a.m, a.n, a.rows_per_block, a.rw_tail, a.items_tail, a.full_magic, grid, S,
+                                   carry_mode, true, s);
+            return rc ? rc : t.end();
+        }
+#endif
     }
     if (carry_mode == RPTC_AS_WRITTEN) RPTC_LAUNCH(RPTC_AS_WRITTEN, false);
     else RPTC_LAUNCH(RPTC_CONTINUOUS, false);

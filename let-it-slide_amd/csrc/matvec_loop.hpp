@@ -35,10 +35,10 @@ int matvec_steady_launch(const LoopLayer *device_layers, const LoopLayer &shape,
 
 // One layer per launch with the chain kernel's hand-written body (matvec_steady.hip): whether a layer of width n whose
 // workgroups own rows_per_block rows fits its fixed LDS layout and its four elements a wave, and the launch (the
-// arguments of the per-launch kernel).
+// arguments of the per-launch kernel; silu: x is [gate | up] and the activations are silu(gate) * up).
 bool matvec_one_fits(int n, int rows_per_block, int items_tail);
 int matvec_one_launch(const uint32_t *comp, const uint32_t *codebook, const uint4 *x, uint16_t *out, int m, int n,
                       int rows_per_block, int rw_tail, int items_tail, uint32_t full_magic, int grid, int S, int carry_mode,
-                      hipStream_t stream);
+                      bool silu, hipStream_t stream);
 
 }  // namespace rptc

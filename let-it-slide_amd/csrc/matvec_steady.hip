@@ -856,7 +856,9 @@ __global__ __launch_bounds__(kStThreads) void matvec_steady_kernel(
     "v108", "v109", "v110", "v111", "v112", "v113", "v114", "v115", "v116", "v117", "v118", "v119", "v120", "v121", "v122", \
     "v123", "v124", "v125", "v126", "v127"
 
-template <int S, int MODE, int MAXI>
+// SILU: x is [gate | up], 2n halves, and the activations are silu(gate) * up (the down projection of a decoder layer, as
+// rptc_decompress_matvec_silu), the same roundings as the stand-alone kernel
+template <int S, int MODE, int MAXI, bool SILU>
 __global__ __launch_bounds__(kStThreads) void matvec_one_kernel(
     const uint4 *__restrict__ comp, const uint32_t *__restrict__ codebook, const uint4 *__restrict__ x, int arg_m, int arg_n,
     int rows_per_block, int rw_tail, int items_tail, uint32_t full_magic, uint32_t tail_magic, uint16_t *__restrict__ out)
@@ -874,7 +876,9 @@ __global__ __launch_bounds__(kStThreads) void matvec_one_kernel(
 
     // ---- requests first: a thread's share of the activations (16 bytes at 8 idx, two of them) ...
     const int i0 = tid, i1 = tid + kStThreads;
-    const uint4 xv0 = x[min(i0, n8 - 1)], xv1 = x[min(i1, n8 - 1)];
+    uint4 xv0 = x[min(i0, n8 - 1)], xv1 = x[min(i1, n8 - 1)];
+    uint4 up0, up1;
+    if constexpr (SILU) up0 = x[n8 + min(i0, n8 - 1)], up1 = x[n8 + min(i1, n8 - 1)];
     // ... and this wave's elements: equal shares, the first total % 16 waves one more.  Lane -> (row inside the item,
     // element inside the row): two rows of 32 in a full slab; in the ragged slab lane / Lt rows of Lt, the quotient from
     // the host's reciprocal (exact for lane < 64); lanes past the item's last whole row idle on element 0
@@ -942,6 +946,7 @@ __global__ __launch_bounds__(kStThreads) void matvec_one_kernel(
         for (int i = 0; i < kRowsPerWave; i++) lds[(kRowsPerWave * wave + i) * 64 + lane] = (cbv[i] & 0xFFFF7FFFu) | table_sign;
     }
 
+    if constexpr (SILU) xv0 = silu_mul8(xv0, up0), xv1 = silu_mul8(xv1, up1);
     // ---- the activations into the image (slot i * n8 + idx for word i of the 16 bytes at 8 idx, inference.cu:215-221;
     // the ragged slab at the full slabs' stride: slot 32 q + l for its q-th step's lane l)
     {
@@ -1031,20 +1036,22 @@ bool matvec_one_fits(int n, int rows_per_block, int items_tail)
 
 int matvec_one_launch(const uint32_t *comp, const uint32_t *codebook, const uint4 *x, uint16_t *out, int m, int n,
                       int rows_per_block, int rw_tail, int items_tail, uint32_t full_magic, int grid, int S, int carry_mode,
-                      hipStream_t stream)
+                      bool silu, hipStream_t stream)
 {
     const int T = n >> 11, lt = (n & 2047) >> 6;
     const int total = T * (rows_per_block >> 1) + items_tail;
     const int max_items = (total + kStWaves - 1) / kStWaves <= 3 ? 3 : 4;
     const uint32_t tail_magic = lt ? 65536u / (uint32_t)lt + 1u : 0u;       // (v * magic) >> 16 == v / lt for v < 1024
     auto a_comp = reinterpret_cast<const uint4 *>(comp);
-#define RPTC_ONE_GO(SS, MM, II)                                                                                      \
-    hipLaunchKernelGGL((matvec_one_kernel<SS, MM, II>), dim3(grid), dim3(kStThreads), kStLdsBytes, stream, a_comp,    \
+#define RPTC_ONE_GO(SS, MM, II, GG)                                                                                  \
+    hipLaunchKernelGGL((matvec_one_kernel<SS, MM, II, GG>), dim3(grid), dim3(kStThreads), kStLdsBytes, stream, a_comp, \
                        codebook, x, m, n, rows_per_block, rw_tail, items_tail, full_magic, tail_magic, out)
-#define RPTC_ONE_PICK(SS, MM)                     \
-    do {                                          \
-        if (max_items == 3) RPTC_ONE_GO(SS, MM, 3); \
-        else RPTC_ONE_GO(SS, MM, 4);              \
+#define RPTC_ONE_PICK(SS, MM)                                 \
+    do {                                                      \
+        if (max_items == 3 && silu) RPTC_ONE_GO(SS, MM, 3, true);  \
+        else if (max_items == 3) RPTC_ONE_GO(SS, MM, 3, false);    \
+        else if (silu) RPTC_ONE_GO(SS, MM, 4, true);               \
+        else RPTC_ONE_GO(SS, MM, 4, false);                        \
     } while (0)
     if (S == 6 && carry_mode == RPTC_AS_WRITTEN) RPTC_ONE_PICK(6, RPTC_AS_WRITTEN);
     else if (S == 6) RPTC_ONE_PICK(6, RPTC_CONTINUOUS);
@@ -1056,7 +1063,7 @@ int matvec_one_launch(const uint32_t *comp, const uint32_t *codebook, const uint
 }
 #else
 bool matvec_one_fits(int, int, int) { return false; }
-int matvec_one_launch(const uint32_t *, const uint32_t *, const uint4 *, uint16_t *, int, int, int, int, int, uint32_t, int, int, int, hipStream_t)
+int matvec_one_launch(const uint32_t *, const uint32_t *, const uint4 *, uint16_t *, int, int, int, int, int, uint32_t, int, int, int, bool, hipStream_t)
 {
     return RPTC_ESHAPE;
 }
@@ -1074,13 +1081,15 @@ int prepare_matvec_steady()
     RPTC_SET_LIMITS(4)
 #undef RPTC_SET_LIMITS
 #ifndef ST_MFMA
-#define RPTC_SET_LIMITS(MAXI)                                                                 \
-    if ((rc = st_set_lds_limit(matvec_one_kernel<6, RPTC_AS_WRITTEN, MAXI>))) return rc;        \
-    if ((rc = st_set_lds_limit(matvec_one_kernel<6, RPTC_CONTINUOUS, MAXI>))) return rc;        \
-    if ((rc = st_set_lds_limit(matvec_one_kernel<8, RPTC_AS_WRITTEN, MAXI>))) return rc;        \
-    if ((rc = st_set_lds_limit(matvec_one_kernel<8, RPTC_CONTINUOUS, MAXI>))) return rc;
-    RPTC_SET_LIMITS(3)
-    RPTC_SET_LIMITS(4)
+#define RPTC_SET_LIMITS(MAXI, GG)                                                             \
+    if ((rc = st_set_lds_limit(matvec_one_kernel<6, RPTC_AS_WRITTEN, MAXI, GG>))) return rc;    \
+    if ((rc = st_set_lds_limit(matvec_one_kernel<6, RPTC_CONTINUOUS, MAXI, GG>))) return rc;    \
+    if ((rc = st_set_lds_limit(matvec_one_kernel<8, RPTC_AS_WRITTEN, MAXI, GG>))) return rc;    \
+    if ((rc = st_set_lds_limit(matvec_one_kernel<8, RPTC_CONTINUOUS, MAXI, GG>))) return rc;
+    RPTC_SET_LIMITS(3, false)
+    RPTC_SET_LIMITS(4, false)
+    RPTC_SET_LIMITS(3, true)
+    RPTC_SET_LIMITS(4, true)
 #undef RPTC_SET_LIMITS
 #endif
     return 0;

@@ -200,6 +200,16 @@ __device__ __forceinline__ uint32_t silu_mul_pair(uint32_t gate, uint32_t up)
     sg.y = (_Float16)(g1 * __builtin_amdgcn_rcpf(1.f + e1));
     return __builtin_bit_cast(uint32_t, sg * __builtin_bit_cast(half2_t, up));
 }
+
+// the same for the eight halves of 16 bytes
+__device__ __forceinline__ uint4 silu_mul8(const uint4 gate, const uint4 up)
+{
+    const uint32_t g[4] = {gate.x, gate.y, gate.z, gate.w}, u[4] = {up.x, up.y, up.z, up.w};
+    uint32_t r[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) r[i] = silu_mul_pair(g[i], u[i]);
+    return make_uint4(r[0], r[1], r[2], r[3]);
+}
 #endif
 
 }  // namespace rptc

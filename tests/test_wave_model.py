@@ -1153,13 +1153,20 @@ def test_batched_kernel_at_3_and_4_bits(matmul_isa, oracle, bits, m, n, batch, S
     assert not arrived.any()
 
 
-def run_one_layer(isa, oracle, m, n, S, mode, blocks, seed=7, burst=8, latency=(400, 60)):
+def run_one_layer(isa, oracle, m, n, S, mode, blocks, seed=7, burst=8, latency=(400, 60), silu=False):
     """`matvec_one_kernel<S, MODE, MAXI>` (`csrc/matvec_steady.hip`) as `matvec_one_launch` launches it: the per-launch op's
     arguments plus the reciprocal of the ragged row's length, the chain kernel's fixed LDS layout."""
     rng = np.random.default_rng(seed + m + n)
     cb = (rng.standard_normal(2 << S) * 0.1).astype(np.float16)
     comp = rng.integers(0, 256, m * n // 4, dtype=np.uint8)
     x = (rng.standard_normal(n) * 0.5).astype(np.float16)
+    x_in = x
+    if silu:
+        # [gate | up]: the activations are silu(gate) * up, the gate rounded to fp16 before the product (csrc/rptc_common.hpp)
+        gate, up = (rng.standard_normal(n) * 1.5).astype(np.float16), (rng.standard_normal(n) * 0.5).astype(np.float16)
+        g32 = gate.astype(np.float32)
+        x = ((g32 / (1.0 + np.exp(-g32))).astype(np.float16) * up).astype(np.float16)
+        x_in = np.concatenate([gate, up])
     out = np.full(2 * m, 0xEE, dtype=np.uint8)
     rpb, rw_tail, items_tail, magic, _ = _matvec_geometry(m, n)
     T, lt = n >> 11, (n & 2047) >> 6
@@ -1172,10 +1179,10 @@ def run_one_layer(isa, oracle, m, n, S, mode, blocks, seed=7, burst=8, latency=(
     c_at, cb_at, x_at, o_at = 0x7f40fffff000, 0x7f5000003400, 0x7f3ffff0fe00, 0x7f2ffffe0100
     mem.add(c_at, comp, "stream")
     mem.add(cb_at, cb.view(np.uint8).copy(), "codebook")
-    mem.add(x_at, x.view(np.uint8).copy(), "activations")
+    mem.add(x_at, x_in.view(np.uint8).copy(), "activations")
     mem.add(o_at, out, "output")
     wave_model.Wave.vm_latency, wave_model.Wave.lgkm_latency = latency
-    kernel = wave_model.Kernel(isa, "_ZN4rptc17matvec_one_kernelILi%dELi%dELi%dEE" % (S, mode, 3 if per_wave <= 3 else 4))
+    kernel = wave_model.Kernel(isa, "_ZN4rptc17matvec_one_kernelILi%dELi%dELi%dELb%dEE" % (S, mode, 3 if per_wave <= 3 else 4, 1 if silu else 0))
     blocks = sorted({b for b in blocks if b < grid})
     kernel.launch(mem, (grid,), 1024, [("ptr", c_at), ("ptr", cb_at), ("ptr", x_at), ("i32", m), ("i32", n), ("i32", rpb), ("i32", rw_tail),
                                        ("i32", items_tail), ("u32", magic), ("u32", tail_magic), ("ptr", o_at)], lds_bytes=160 * 1024,
@@ -1201,3 +1208,9 @@ def test_one_layer_kernel_matches_the_oracle(steady_isa, oracle, m, n, S, mode):
 @pytest.mark.parametrize("burst,latency", [(1, (3000, 300)), (64, (5, 2))])
 def test_one_layer_kernel_under_other_interleavings(steady_isa, oracle, burst, latency):
     run_one_layer(steady_isa, oracle, 100, 4096 + 64 * 7, 8, 1, blocks=[0, 3], burst=burst, latency=latency)
+
+
+@pytest.mark.parametrize("m,n,S,mode", [(40, 2048 + 320, 8, 0), (4096, 11008, 8, 1), (300, 64, 6, 0)])
+def test_one_layer_kernel_with_the_silu_gate_in_front(steady_isa, oracle, m, n, S, mode):
+    rpb = 2 * ((m + 2 * CUS - 1) // (2 * CUS))
+    run_one_layer(steady_isa, oracle, m, n, S, mode, blocks=[0, (m - 1) // rpb], silu=True)
