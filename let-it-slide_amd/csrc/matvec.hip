@@ -1122,7 +1122,7 @@ static int launch_matvec(const int32_t *compressed, const uint16_t *codebook, co
         // the same layer through the chain kernel's hand-written body (an experiment until it is timed)
         if (matvec_one_fits(a.n, a.rows_per_block, a.items_tail)) {
             rc = matvec_one_launch(a_comp, a_cb, a_x, out, a.m, a.n, a.rows_per_block, a.rw_tail, a.items_tail, a.full_magic, grid, S,
-                                   carry_mode, false, s);
+                                   carry_mode, 0, nullptr, nullptr, nullptr, 0.f, s);
             return rc ? rc : t.end();
         }
 #endif
@@ -1171,11 +1171,20 @@ static int launch_matvec_fused(const int32_t *compressed, const uint16_t *codebo
 #ifdef RPTC_MV_ONE
         if (matvec_one_fits(a.n, a.rows_per_block, a.items_tail)) {
             rc = matvec_one_launch(a_comp, a_cb, a_x, out, a.m, a.n, a.rows_per_block, a.rw_tail, a.items_tail, a.full_magic, grid, S,
-                                   carry_mode, true, s);
+                                   carry_mode, 1, nullptr, nullptr, nullptr, 0.f, s);
             return rc ? rc : t.end();
         }
 #endif
     }
+#ifdef RPTC_MV_ONE
+    if constexpr (XMODE == kXAddRmsNorm) {
+        if (matvec_one_fits(a.n, a.rows_per_block, a.items_tail)) {
+            rc = matvec_one_launch(a_comp, a_cb, a_x, out, a.m, a.n, a.rows_per_block, a.rw_tail, a.items_tail, a.full_magic, grid, S,
+                                   carry_mode, 2, a_x2, a_w, a_xo, eps, s);
+            return rc ? rc : t.end();
+        }
+    }
+#endif
     if (carry_mode == RPTC_AS_WRITTEN) RPTC_LAUNCH(RPTC_AS_WRITTEN, false);
     else RPTC_LAUNCH(RPTC_CONTINUOUS, false);
 #undef RPTC_LAUNCH

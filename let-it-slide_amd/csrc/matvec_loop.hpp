@@ -35,10 +35,11 @@ int matvec_steady_launch(const LoopLayer *device_layers, const LoopLayer &shape,
 
 // One layer per launch with the chain kernel's hand-written body (matvec_steady.hip): whether a layer of width n whose
 // workgroups own rows_per_block rows fits its fixed LDS layout and its four elements a wave, and the launch (the
-// arguments of the per-launch kernel; silu: x is [gate | up] and the activations are silu(gate) * up).
+// arguments of the per-launch kernel).  prologue: 0 none; 1 x is [gate | up] and the activations are silu(gate) * up;
+// 2 the activations are the RMS norm of x + delta (delta may be null) times norm_w, and x + delta goes to x_out.
 bool matvec_one_fits(int n, int rows_per_block, int items_tail);
 int matvec_one_launch(const uint32_t *comp, const uint32_t *codebook, const uint4 *x, uint16_t *out, int m, int n,
                       int rows_per_block, int rw_tail, int items_tail, uint32_t full_magic, int grid, int S, int carry_mode,
-                      bool silu, hipStream_t stream);
+                      int prologue, const uint4 *delta, const uint4 *norm_w, uint4 *x_out, float eps, hipStream_t stream);
 
 }  // namespace rptc

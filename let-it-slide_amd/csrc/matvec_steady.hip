@@ -856,12 +856,16 @@ __global__ __launch_bounds__(kStThreads) void matvec_steady_kernel(
     "v108", "v109", "v110", "v111", "v112", "v113", "v114", "v115", "v116", "v117", "v118", "v119", "v120", "v121", "v122", \
     "v123", "v124", "v125", "v126", "v127"
 
-// SILU: x is [gate | up], 2n halves, and the activations are silu(gate) * up (the down projection of a decoder layer, as
-// rptc_decompress_matvec_silu), the same roundings as the stand-alone kernel
-template <int S, int MODE, int MAXI, bool SILU>
+// XMODE 1: x is [gate | up], 2n halves, and the activations are silu(gate) * up (the down projection of a decoder layer, as
+// rptc_decompress_matvec_silu).  XMODE 2: the activations are the RMS norm of x + delta times norm_w, and workgroup 0
+// writes x + delta to x_out (as rptc_decompress_matvec_rmsnorm; delta may be null).  The same operations in the same
+// order as matvec.hip's prologues, so the same bits.
+constexpr int kOnePlain = 0, kOneSilu = 1, kOneNorm = 2;
+template <int S, int MODE, int MAXI, int XMODE>
 __global__ __launch_bounds__(kStThreads) void matvec_one_kernel(
     const uint4 *__restrict__ comp, const uint32_t *__restrict__ codebook, const uint4 *__restrict__ x, int arg_m, int arg_n,
-    int rows_per_block, int rw_tail, int items_tail, uint32_t full_magic, uint32_t tail_magic, uint16_t *__restrict__ out)
+    int rows_per_block, int rw_tail, int items_tail, uint32_t full_magic, uint32_t tail_magic, uint16_t *__restrict__ out,
+    const uint4 *delta, const uint4 *__restrict__ norm_w, uint4 *x_out, float eps)
 {
     static_assert(MAXI == 3 || MAXI == 4, "a wave holds three or four elements");
     extern __shared__ uint32_t lds[];
@@ -877,8 +881,12 @@ __global__ __launch_bounds__(kStThreads) void matvec_one_kernel(
     // ---- requests first: a thread's share of the activations (16 bytes at 8 idx, two of them) ...
     const int i0 = tid, i1 = tid + kStThreads;
     uint4 xv0 = x[min(i0, n8 - 1)], xv1 = x[min(i1, n8 - 1)];
-    uint4 up0, up1;
-    if constexpr (SILU) up0 = x[n8 + min(i0, n8 - 1)], up1 = x[n8 + min(i1, n8 - 1)];
+    uint4 second0 = make_uint4(0, 0, 0, 0), second1 = second0, weight0 = second0, weight1 = second0;
+    if constexpr (XMODE == kOneSilu) second0 = x[n8 + min(i0, n8 - 1)], second1 = x[n8 + min(i1, n8 - 1)];
+    if constexpr (XMODE == kOneNorm) {
+        if (delta) second0 = delta[min(i0, n8 - 1)], second1 = delta[min(i1, n8 - 1)];
+        weight0 = norm_w[min(i0, n8 - 1)], weight1 = norm_w[min(i1, n8 - 1)];
+    }
     // ... and this wave's elements: equal shares, the first total % 16 waves one more.  Lane -> (row inside the item,
     // element inside the row): two rows of 32 in a full slab; in the ragged slab lane / Lt rows of Lt, the quotient from
     // the host's reciprocal (exact for lane < 64); lanes past the item's last whole row idle on element 0
@@ -946,7 +954,51 @@ __global__ __launch_bounds__(kStThreads) void matvec_one_kernel(
         for (int i = 0; i < kRowsPerWave; i++) lds[(kRowsPerWave * wave + i) * 64 + lane] = (cbv[i] & 0xFFFF7FFFu) | table_sign;
     }
 
-    if constexpr (SILU) xv0 = silu_mul8(xv0, up0), xv1 = silu_mul8(xv1, up1);
+    if constexpr (XMODE == kOneSilu) xv0 = silu_mul8(xv0, second0), xv1 = silu_mul8(xv1, second1);
+    if constexpr (XMODE == kOneNorm) {
+        // as matvec.hip's prologue: packed fp16 residual add, squares as two-term dot products with an fp32 sum, the sum
+        // over the workgroup in a fixed order (a wave's lanes, then the sixteen waves), each half scaled and rounded
+        // once, a packed fp16 multiply by the weight.  A thread past the end of the vector adds nothing.
+        float *red = reinterpret_cast<float *>(lds + kStPartBase / 4);       // free until the elements' sums go there
+        uint32_t r[2][4];
+        float ss = 0.f;
+        const uint4 xin[2] = {xv0, xv1}, din[2] = {second0, second1}, win[2] = {weight0, weight1};
+        const int idx_of[2] = {i0, i1};
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+            const bool inside = idx_of[u] < n8;
+            const uint32_t xw[4] = {xin[u].x, xin[u].y, xin[u].z, xin[u].w}, dw[4] = {din[u].x, din[u].y, din[u].z, din[u].w};
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                r[u][i] = delta ? __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, xw[i]) + __builtin_bit_cast(half2_t, dw[i])) : xw[i];
+                if (!inside) r[u][i] = 0u;
+                ss = dot2(r[u][i], r[u][i], ss);
+            }
+            if (blockIdx.x == 0 && inside) x_out[idx_of[u]] = make_uint4(r[u][0], r[u][1], r[u][2], r[u][3]);
+        }
+        ss = wave_sum(ss);
+        if (lane == 63) red[wave] = ss;
+        __syncthreads();
+        float total_ss = wave_sum(lane < kStWaves ? red[lane] : 0.f);
+        total_ss = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, total_ss), 63));
+        const float inv = rsqrtf(total_ss / (float)n + eps);
+        uint4 hv[2];
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+            const uint32_t ww[4] = {win[u].x, win[u].y, win[u].z, win[u].w};
+            uint32_t h[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const half2_t rv = __builtin_bit_cast(half2_t, r[u][i]);
+                half2_t sv;
+                sv.x = (_Float16)((float)rv.x * inv);
+                sv.y = (_Float16)((float)rv.y * inv);
+                h[i] = __builtin_bit_cast(uint32_t, sv * __builtin_bit_cast(half2_t, ww[i]));
+            }
+            hv[u] = make_uint4(h[0], h[1], h[2], h[3]);
+        }
+        xv0 = hv[0], xv1 = hv[1];
+    }
     // ---- the activations into the image (slot i * n8 + idx for word i of the 16 bytes at 8 idx, inference.cu:215-221;
     // the ragged slab at the full slabs' stride: slot 32 q + l for its q-th step's lane l)
     {
@@ -1036,34 +1088,40 @@ bool matvec_one_fits(int n, int rows_per_block, int items_tail)
 
 int matvec_one_launch(const uint32_t *comp, const uint32_t *codebook, const uint4 *x, uint16_t *out, int m, int n,
                       int rows_per_block, int rw_tail, int items_tail, uint32_t full_magic, int grid, int S, int carry_mode,
-                      bool silu, hipStream_t stream)
+                      int prologue, const uint4 *delta, const uint4 *norm_w, uint4 *x_out, float eps, hipStream_t stream)
 {
     const int T = n >> 11, lt = (n & 2047) >> 6;
     const int total = T * (rows_per_block >> 1) + items_tail;
     const int max_items = (total + kStWaves - 1) / kStWaves <= 3 ? 3 : 4;
     const uint32_t tail_magic = lt ? 65536u / (uint32_t)lt + 1u : 0u;       // (v * magic) >> 16 == v / lt for v < 1024
     auto a_comp = reinterpret_cast<const uint4 *>(comp);
-#define RPTC_ONE_GO(SS, MM, II, GG)                                                                                  \
-    hipLaunchKernelGGL((matvec_one_kernel<SS, MM, II, GG>), dim3(grid), dim3(kStThreads), kStLdsBytes, stream, a_comp, \
-                       codebook, x, m, n, rows_per_block, rw_tail, items_tail, full_magic, tail_magic, out)
-#define RPTC_ONE_PICK(SS, MM)                                 \
-    do {                                                      \
-        if (max_items == 3 && silu) RPTC_ONE_GO(SS, MM, 3, true);  \
-        else if (max_items == 3) RPTC_ONE_GO(SS, MM, 3, false);    \
-        else if (silu) RPTC_ONE_GO(SS, MM, 4, true);               \
-        else RPTC_ONE_GO(SS, MM, 4, false);                        \
+#define RPTC_ONE_GO(SS, MM, II, XX)                                                                                  \
+    hipLaunchKernelGGL((matvec_one_kernel<SS, MM, II, XX>), dim3(grid), dim3(kStThreads), kStLdsBytes, stream, a_comp, \
+                       codebook, x, m, n, rows_per_block, rw_tail, items_tail, full_magic, tail_magic, out, delta, norm_w, x_out, eps)
+#define RPTC_ONE_PICK_X(SS, MM, II)                             \
+    do {                                                        \
+        if (prologue == kOneSilu) RPTC_ONE_GO(SS, MM, II, kOneSilu);      \
+        else if (prologue == kOneNorm) RPTC_ONE_GO(SS, MM, II, kOneNorm); \
+        else RPTC_ONE_GO(SS, MM, II, kOnePlain);                          \
+    } while (0)
+#define RPTC_ONE_PICK(SS, MM)                        \
+    do {                                             \
+        if (max_items == 3) RPTC_ONE_PICK_X(SS, MM, 3); \
+        else RPTC_ONE_PICK_X(SS, MM, 4);             \
     } while (0)
     if (S == 6 && carry_mode == RPTC_AS_WRITTEN) RPTC_ONE_PICK(6, RPTC_AS_WRITTEN);
     else if (S == 6) RPTC_ONE_PICK(6, RPTC_CONTINUOUS);
     else if (carry_mode == RPTC_AS_WRITTEN) RPTC_ONE_PICK(8, RPTC_AS_WRITTEN);
     else RPTC_ONE_PICK(8, RPTC_CONTINUOUS);
 #undef RPTC_ONE_PICK
+#undef RPTC_ONE_PICK_X
 #undef RPTC_ONE_GO
     return (int)hipGetLastError();
 }
 #else
 bool matvec_one_fits(int, int, int) { return false; }
-int matvec_one_launch(const uint32_t *, const uint32_t *, const uint4 *, uint16_t *, int, int, int, int, int, uint32_t, int, int, int, bool, hipStream_t)
+int matvec_one_launch(const uint32_t *, const uint32_t *, const uint4 *, uint16_t *, int, int, int, int, int, uint32_t, int, int, int, int,
+                      const uint4 *, const uint4 *, uint4 *, float, hipStream_t)
 {
     return RPTC_ESHAPE;
 }
@@ -1086,10 +1144,12 @@ int prepare_matvec_steady()
     if ((rc = st_set_lds_limit(matvec_one_kernel<6, RPTC_CONTINUOUS, MAXI, GG>))) return rc;    \
     if ((rc = st_set_lds_limit(matvec_one_kernel<8, RPTC_AS_WRITTEN, MAXI, GG>))) return rc;    \
     if ((rc = st_set_lds_limit(matvec_one_kernel<8, RPTC_CONTINUOUS, MAXI, GG>))) return rc;
-    RPTC_SET_LIMITS(3, false)
-    RPTC_SET_LIMITS(4, false)
-    RPTC_SET_LIMITS(3, true)
-    RPTC_SET_LIMITS(4, true)
+    RPTC_SET_LIMITS(3, kOnePlain)
+    RPTC_SET_LIMITS(4, kOnePlain)
+    RPTC_SET_LIMITS(3, kOneSilu)
+    RPTC_SET_LIMITS(4, kOneSilu)
+    RPTC_SET_LIMITS(3, kOneNorm)
+    RPTC_SET_LIMITS(4, kOneNorm)
 #undef RPTC_SET_LIMITS
 #endif
     return 0;

@@ -1182,10 +1182,11 @@ def run_one_layer(isa, oracle, m, n, S, mode, blocks, seed=7, burst=8, latency=(
     mem.add(x_at, x_in.view(np.uint8).copy(), "activations")
     mem.add(o_at, out, "output")
     wave_model.Wave.vm_latency, wave_model.Wave.lgkm_latency = latency
-    kernel = wave_model.Kernel(isa, "_ZN4rptc17matvec_one_kernelILi%dELi%dELi%dELb%dEE" % (S, mode, 3 if per_wave <= 3 else 4, 1 if silu else 0))
+    kernel = wave_model.Kernel(isa, "_ZN4rptc17matvec_one_kernelILi%dELi%dELi%dELi%dEE" % (S, mode, 3 if per_wave <= 3 else 4, 1 if silu else 0))
     blocks = sorted({b for b in blocks if b < grid})
     kernel.launch(mem, (grid,), 1024, [("ptr", c_at), ("ptr", cb_at), ("ptr", x_at), ("i32", m), ("i32", n), ("i32", rpb), ("i32", rw_tail),
-                                       ("i32", items_tail), ("u32", magic), ("u32", tail_magic), ("ptr", o_at)], lds_bytes=160 * 1024,
+                                       ("i32", items_tail), ("u32", magic), ("u32", tail_magic), ("ptr", o_at), ("ptr", 0), ("ptr", 0),
+                                       ("ptr", 0), ("f32", 0.0)], lds_bytes=160 * 1024,
                   groups=[(b, 0, 0) for b in blocks], seed=seed, burst=burst)
     want = oracle.matvec(comp.view(np.uint32), cb, x, m, S, mode=mode)
     got = out.view(np.float16).astype(np.float64)
@@ -1214,3 +1215,77 @@ def test_one_layer_kernel_under_other_interleavings(steady_isa, oracle, burst, l
 def test_one_layer_kernel_with_the_silu_gate_in_front(steady_isa, oracle, m, n, S, mode):
     rpb = 2 * ((m + 2 * CUS - 1) // (2 * CUS))
     run_one_layer(steady_isa, oracle, m, n, S, mode, blocks=[0, (m - 1) // rpb], silu=True)
+
+
+@pytest.mark.parametrize("m,n,S,mode", [(4096, 11008, 8, 0), (33, 4096 + 768, 6, 1)])
+def test_one_layer_kernel_has_the_per_launch_kernels_bits(matvec_isa, steady_isa, m, n, S, mode):
+    """Both kernels add an element's four sums, a row's partial sums and the lanes of the row's wave in the same order, so
+    routing the op through the other kernel changes no output bit."""
+    rng = np.random.default_rng(3)
+    cb = (rng.standard_normal(2 << S) * 0.1).astype(np.float16)
+    comp = rng.integers(0, 256, m * n // 4, dtype=np.uint8)
+    x = (rng.standard_normal(n) * 0.5).astype(np.float16)
+    rpb, rw_tail, items_tail, magic, lds_plain = _matvec_geometry(m, n)
+    lt = (n & 2047) >> 6
+    per_wave = -(-((n >> 11) * (rpb // 2) + items_tail) // 16)
+    grid = (m + rpb - 1) // rpb
+    outs = []
+    for one in (True, False):
+        out = np.full(2 * m, 0xEE, dtype=np.uint8)
+        mem = wave_model.Memory()
+        c_at, cb_at, x_at, o_at = 0x7f40fffff000, 0x7f5000003400, 0x7f3ffff0fe00, 0x7f2ffffe0100
+        for at, data, name in ((c_at, comp, "stream"), (cb_at, cb.view(np.uint8).copy(), "codebook"), (x_at, x.view(np.uint8).copy(), "activations"),
+                               (o_at, out, "output")):
+            mem.add(at, data, name)
+        wave_model.Wave.vm_latency, wave_model.Wave.lgkm_latency = 400, 60
+        head = [("ptr", c_at), ("ptr", cb_at), ("ptr", x_at), ("i32", m), ("i32", n), ("i32", rpb), ("i32", rw_tail), ("i32", items_tail), ("u32", magic)]
+        if one:
+            kernel = wave_model.Kernel(steady_isa, "_ZN4rptc17matvec_one_kernelILi%dELi%dELi%dELi0EE" % (S, mode, 3 if per_wave <= 3 else 4))
+            kernel.launch(mem, (grid,), 1024, head + [("u32", 65536 // lt + 1 if lt else 0), ("ptr", o_at), ("ptr", 0), ("ptr", 0), ("ptr", 0), ("f32", 0.0)],
+                          lds_bytes=160 * 1024, groups=[(0, 0, 0)], seed=1)
+        else:
+            kernel = wave_model.Kernel(matvec_isa, "_ZN4rptc13matvec_kernelILi%dELi%dELi2ELb0EE" % (S, mode))
+            kernel.launch(mem, (grid,), 1024, head + [("ptr", o_at)], lds_bytes=lds_plain, groups=[(0, 0, 0)], seed=1)
+        outs.append(out)
+    assert np.array_equal(outs[0], outs[1]) and (outs[0][:2 * min(rpb, m)] != 0xEE).any()
+
+
+@pytest.mark.parametrize("m,n,S,mode,with_delta", [(40, 2048 + 320, 8, 0, True), (12288, 4096, 8, 1, True), (33, 64 * 7, 6, 0, False)])
+def test_one_layer_kernel_with_the_norm_in_front_has_the_fused_kernels_bits(matvec_isa, steady_isa, m, n, S, mode, with_delta):
+    """The XMODE 2 form (residual add + RMS norm in the prologue) against `matvec_fused_kernel` with the same prologue:
+    the same output bits and the same residual stream written back."""
+    rng = np.random.default_rng(m + n)
+    cb = (rng.standard_normal(2 << S) * 0.1).astype(np.float16)
+    comp = rng.integers(0, 256, m * n // 4, dtype=np.uint8)
+    x_in = (rng.standard_normal(n) * 1.2).astype(np.float16)
+    delta = (rng.standard_normal(n) * 0.3).astype(np.float16)
+    weight = (1.0 + 0.1 * rng.standard_normal(n)).astype(np.float16)
+    rpb, rw_tail, items_tail, magic, lds_plain = _matvec_geometry(m, n)
+    lt = (n & 2047) >> 6
+    per_wave = -(-((n >> 11) * (rpb // 2) + items_tail) // 16)
+    grid = (m + rpb - 1) // rpb
+    results = []
+    for one in (True, False):
+        out = np.full(2 * m, 0xEE, dtype=np.uint8)
+        res = np.full(2 * n, 0xEE, dtype=np.uint8)
+        mem = wave_model.Memory()
+        c_at, cb_at, x_at, d_at, w_at, r_at, o_at = (0x7f40fffff000, 0x7f5000003400, 0x7f3ffff0fe00, 0x7f3000000000, 0x7f3100000000, 0x7f3200000000,
+                                                     0x7f2ffffe0100)
+        for at, data, name in ((c_at, comp, "stream"), (cb_at, cb.view(np.uint8).copy(), "codebook"), (x_at, x_in.view(np.uint8).copy(), "residual in"),
+                               (d_at, delta.view(np.uint8).copy(), "delta"), (w_at, weight.view(np.uint8).copy(), "norm weight"),
+                               (r_at, res, "residual out"), (o_at, out, "output")):
+            mem.add(at, data, name)
+        wave_model.Wave.vm_latency, wave_model.Wave.lgkm_latency = 400, 60
+        head = [("ptr", c_at), ("ptr", cb_at), ("ptr", x_at), ("i32", m), ("i32", n), ("i32", rpb), ("i32", rw_tail), ("i32", items_tail), ("u32", magic)]
+        dptr = ("ptr", d_at if with_delta else 0)
+        if one:
+            kernel = wave_model.Kernel(steady_isa, "_ZN4rptc17matvec_one_kernelILi%dELi%dELi%dELi2EE" % (S, mode, 3 if per_wave <= 3 else 4))
+            kernel.launch(mem, (grid,), 1024, head + [("u32", 65536 // lt + 1 if lt else 0), ("ptr", o_at), dptr, ("ptr", w_at), ("ptr", r_at), ("f32", 1e-5)],
+                          lds_bytes=160 * 1024, groups=[(0, 0, 0)], seed=1)
+        else:
+            kernel = wave_model.Kernel(matvec_isa, "_ZN4rptc19matvec_fused_kernelILi%dELi%dELi2ELb0EE" % (S, mode))
+            kernel.launch(mem, (grid,), 1024, head + [dptr, ("ptr", o_at), ("ptr", w_at), ("ptr", r_at), ("f32", 1e-5), ("i32", 0)],
+                          lds_bytes=lds_plain + 48 * 4, groups=[(0, 0, 0)], seed=1)
+        results.append((out, res))
+    assert np.array_equal(results[0][0], results[1][0]) and np.array_equal(results[0][1], results[1][1])
+    assert (results[0][1] != 0xEE).any() and (results[0][0][:2 * min(rpb, m)] != 0xEE).any()
