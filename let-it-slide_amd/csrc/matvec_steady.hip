@@ -102,6 +102,12 @@ static_assert(kStLdsBytes == kMaxLds, "the layout fills the LDS of a CU");
 #else
 #define ST_PRIO(X) ""
 #endif
+#define ST_PRIO_OF_0 ST_PRIO("3")
+#define ST_PRIO_OF_1 ST_PRIO("2")
+#define ST_PRIO_OF_2 ST_PRIO("1")
+#define ST_PRIO_OF_3 ST_PRIO("0")
+#define ST_PRIO_OF_4 ST_PRIO("0")
+#define ST_PRIO_OF_5 ST_PRIO("0")
 #define ST_STR2(x) #x
 #define ST_STR(x) ST_STR2(x)
 
@@ -360,7 +366,7 @@ static_assert(kStLdsBytes == kMaxLds, "the layout fills the LDS of a CU");
 #define ST_ITEM_HEAD(U, P, NEED)                                                                                      \
     "s_cmp_le_u32 %[nitems], " #U "\n"                                                                                \
     "s_cbranch_scc1 7" #U "f\n"                                                                                       \
-    ST_PRIO("3-" #U)                                                                                                  \
+    ST_PRIO_OF_##U                                                                                                    \
     "s_bitcmp1_b32 %[rl], " #U "\n"                                                                                   \
     "s_cbranch_scc0 5" #U "f\n"                                                                                       \
     ST_RELOAD("%[xa" #U "]", P)                                                                                       \
@@ -829,6 +835,7 @@ __global__ __launch_bounds__(kStThreads) void matvec_steady_kernel(
 #define ST_ONE_ITEM_1(U) ST_ITEM_1(U, "%[e" #U "x]", "%[e" #U "y]", "%[e" #U "z]", "%[e" #U "w]", 0, 63, "")
 #define ST_ONE_ITEMS_3(MODE) ST_ONE_ITEM_##MODE(0) ST_ONE_ITEM_##MODE(1) ST_ONE_ITEM_##MODE(2)
 #define ST_ONE_ITEMS_4(MODE) ST_ONE_ITEMS_3(MODE) ST_ONE_ITEM_##MODE(3)
+#define ST_ONE_ITEMS_6(MODE) ST_ONE_ITEMS_4(MODE) ST_ONE_ITEM_##MODE(4) ST_ONE_ITEM_##MODE(5)
 #define ST_ONE_BODY(MODE, M)                                                                                          \
     "s_waitcnt lgkmcnt(0)\n"                                                                                          \
     "s_barrier\n"                                                                                                     \
@@ -867,7 +874,7 @@ __global__ __launch_bounds__(kStThreads) void matvec_one_kernel(
     int rows_per_block, int rw_tail, int items_tail, uint32_t full_magic, uint32_t tail_magic, uint16_t *__restrict__ out,
     const uint4 *delta, const uint4 *__restrict__ norm_w, uint4 *x_out, float eps)
 {
-    static_assert(MAXI == 3 || MAXI == 4, "a wave holds three or four elements");
+    static_assert(MAXI == 3 || MAXI == 4 || MAXI == 6, "a wave holds up to three, four or six elements");
     extern __shared__ uint32_t lds[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -877,6 +884,9 @@ __global__ __launch_bounds__(kStThreads) void matvec_one_kernel(
     const int items_full = rows_per_block >> 1;
     const int row0 = blockIdx.x * rows_per_block;
     const int rows = min(rows_per_block, m - row0);
+    // one layer needs one activation image and one set of partial sums: the set starts where the chain kernel keeps
+    // its second image and has 64 KiB
+    constexpr int kOnePartBase = kStTableBytes + kStImageBytes;
 
     // ---- requests first: a thread's share of the activations (16 bytes at 8 idx, two of them) ...
     const int i0 = tid, i1 = tid + kStThreads;
@@ -935,7 +945,7 @@ __global__ __launch_bounds__(kStThreads) void matvec_one_kernel(
             cw[u] = cm[u] = 0u;
         }
         xa[u] = (uint32_t)kStTableBytes + 4u * (uint32_t)(1024 * slab + l);
-        pa[u] = (uint32_t)kStPartBase + 4u * (uint32_t)((row_first + sub) * npr + 32 * slab + l);
+        pa[u] = (uint32_t)kOnePartBase + 4u * (uint32_t)((row_first + sub) * npr + 32 * slab + l);
         first[u] = full ? 0x0000000100000001ull : first_tail;
         const int nact = max(rows_here, 0) * lanes;
         keep[u] = nact >= 64 ? ~0ull : (1ull << nact) - 1ull;
@@ -959,7 +969,7 @@ __global__ __launch_bounds__(kStThreads) void matvec_one_kernel(
         // as matvec.hip's prologue: packed fp16 residual add, squares as two-term dot products with an fp32 sum, the sum
         // over the workgroup in a fixed order (a wave's lanes, then the sixteen waves), each half scaled and rounded
         // once, a packed fp16 multiply by the weight.  A thread past the end of the vector adds nothing.
-        float *red = reinterpret_cast<float *>(lds + kStPartBase / 4);       // free until the elements' sums go there
+        float *red = reinterpret_cast<float *>(lds + kOnePartBase / 4);       // free until the elements' sums go there
         uint32_t r[2][4];
         float ss = 0.f;
         const uint4 xin[2] = {xv0, xv1}, din[2] = {second0, second1}, win[2] = {weight0, weight1};
@@ -1026,7 +1036,7 @@ __global__ __launch_bounds__(kStThreads) void matvec_one_kernel(
     const int first_row_wave = 0, row_waves = 8;
 #endif
     const int ri = wave - first_row_wave;
-    const uint32_t rs = (uint32_t)kStPartBase + 4u * (uint32_t)(max(ri, 0) * npr + lane);
+    const uint32_t rs = (uint32_t)kOnePartBase + 4u * (uint32_t)(max(ri, 0) * npr + lane);
     const uint32_t oo = 2u * (uint32_t)(row0 + max(ri, 0));
     const uint32_t rstep = 4u * (uint32_t)(row_waves * npr), ostep = 2u * (uint32_t)row_waves;
     const uint32_t nr = ri >= 0 && ri < row_waves && ri < rows ? (uint32_t)(rows - ri + row_waves - 1) / (uint32_t)row_waves : 0u;
@@ -1048,10 +1058,23 @@ __global__ __launch_bounds__(kStThreads) void matvec_one_kernel(
     uint32_t a0, a1, a2, a3, cy, g0, g1, g2, g3, t0, t1, t2, t3, t4, t5, t6, t7, u0, u1, u2, u3, u4, u5, u6, u7, xb, j;
     if constexpr (MODE == RPTC_AS_WRITTEN && MAXI == 3) {
         asm volatile(ST_ONE_BODY(0, 3) : ST_ONE_OUT : ST_ONE_IN, ST_ONE_IN_ITEM(0), ST_ONE_IN_ITEM(1), ST_ONE_IN_ITEM(2) : ST_ONE_CLOBBERS);
-    } else if constexpr (MODE == RPTC_AS_WRITTEN) {
+    } else if constexpr (MODE == RPTC_AS_WRITTEN && MAXI == 4) {
         asm volatile(ST_ONE_BODY(0, 4)
                      : ST_ONE_OUT
                      : ST_ONE_IN, ST_ONE_IN_ITEM(0), ST_ONE_IN_ITEM(1), ST_ONE_IN_ITEM(2), ST_ONE_IN_ITEM(3)
+                     : ST_ONE_CLOBBERS);
+    } else if constexpr (MODE == RPTC_AS_WRITTEN && MAXI == 6) {
+        asm volatile(ST_ONE_BODY(0, 6)
+                     : ST_ONE_OUT
+                     : ST_ONE_IN, ST_ONE_IN_ITEM(0), ST_ONE_IN_ITEM(1), ST_ONE_IN_ITEM(2), ST_ONE_IN_ITEM(3), ST_ONE_IN_ITEM(4), ST_ONE_IN_ITEM(5)
+                     : ST_ONE_CLOBBERS);
+    } else if constexpr (MAXI == 6) {
+        uint32_t own;
+        asm volatile(ST_ONE_BODY(1, 6)
+                     : ST_ONE_OUT, [own] "=&v"(own)
+                     : ST_ONE_IN, ST_ONE_IN_ITEM(0), ST_ONE_IN_ITEM(1), ST_ONE_IN_ITEM(2), ST_ONE_IN_ITEM(3), ST_ONE_IN_ITEM(4), ST_ONE_IN_ITEM(5),
+                       ST_ONE_IN_ITEM_CT(0), ST_ONE_IN_ITEM_CT(1), ST_ONE_IN_ITEM_CT(2), ST_ONE_IN_ITEM_CT(3), ST_ONE_IN_ITEM_CT(4),
+                       ST_ONE_IN_ITEM_CT(5)
                      : ST_ONE_CLOBBERS);
     } else if constexpr (MAXI == 3) {
         uint32_t own;
@@ -1082,8 +1105,8 @@ bool matvec_one_fits(int n, int rows_per_block, int items_tail)
 {
     const int T = n >> 11, lt = (n & 2047) >> 6;
     const int total = T * (rows_per_block >> 1) + items_tail;
-    return (T + (lt ? 1 : 0)) * 4096 <= kStImageBytes && (int64_t)rows_per_block * (n / 64) * 4 <= kStPartBytes &&
-           (total + kStWaves - 1) / kStWaves <= 4;
+    return (T + (lt ? 1 : 0)) * 4096 <= kStImageBytes && (int64_t)rows_per_block * (n / 64) * 4 <= kStImageBytes + 2 * kStPartBytes &&
+           (total + kStWaves - 1) / kStWaves <= 6;
 }
 
 int matvec_one_launch(const uint32_t *comp, const uint32_t *codebook, const uint4 *x, uint16_t *out, int m, int n,
@@ -1092,7 +1115,7 @@ int matvec_one_launch(const uint32_t *comp, const uint32_t *codebook, const uint
 {
     const int T = n >> 11, lt = (n & 2047) >> 6;
     const int total = T * (rows_per_block >> 1) + items_tail;
-    const int max_items = (total + kStWaves - 1) / kStWaves <= 3 ? 3 : 4;
+    const int per_wave = (total + kStWaves - 1) / kStWaves, max_items = per_wave <= 3 ? 3 : per_wave <= 4 ? 4 : 6;
     const uint32_t tail_magic = lt ? 65536u / (uint32_t)lt + 1u : 0u;       // (v * magic) >> 16 == v / lt for v < 1024
     auto a_comp = reinterpret_cast<const uint4 *>(comp);
 #define RPTC_ONE_GO(SS, MM, II, XX)                                                                                  \
@@ -1107,7 +1130,8 @@ int matvec_one_launch(const uint32_t *comp, const uint32_t *codebook, const uint
 #define RPTC_ONE_PICK(SS, MM)                        \
     do {                                             \
         if (max_items == 3) RPTC_ONE_PICK_X(SS, MM, 3); \
-        else RPTC_ONE_PICK_X(SS, MM, 4);             \
+        else if (max_items == 4) RPTC_ONE_PICK_X(SS, MM, 4); \
+        else RPTC_ONE_PICK_X(SS, MM, 6);             \
     } while (0)
     if (S == 6 && carry_mode == RPTC_AS_WRITTEN) RPTC_ONE_PICK(6, RPTC_AS_WRITTEN);
     else if (S == 6) RPTC_ONE_PICK(6, RPTC_CONTINUOUS);
@@ -1150,6 +1174,9 @@ int prepare_matvec_steady()
     RPTC_SET_LIMITS(4, kOneSilu)
     RPTC_SET_LIMITS(3, kOneNorm)
     RPTC_SET_LIMITS(4, kOneNorm)
+    RPTC_SET_LIMITS(6, kOnePlain)
+    RPTC_SET_LIMITS(6, kOneSilu)
+    RPTC_SET_LIMITS(6, kOneNorm)
 #undef RPTC_SET_LIMITS
 #endif
     return 0;

@@ -1172,7 +1172,7 @@ def run_one_layer(isa, oracle, m, n, S, mode, blocks, seed=7, burst=8, latency=(
     T, lt = n >> 11, (n & 2047) >> 6
     total = T * (rpb // 2) + items_tail
     per_wave = -(-total // 16)
-    assert (T + (1 if lt else 0)) * 4096 <= 32768 and rpb * (n // 64) * 4 <= 16384 and per_wave <= 4
+    assert (T + (1 if lt else 0)) * 4096 <= 32768 and rpb * (n // 64) * 4 <= 65536 and per_wave <= 6
     tail_magic = 65536 // lt + 1 if lt else 0
     grid = (m + rpb - 1) // rpb
     mem = wave_model.Memory()
@@ -1182,7 +1182,7 @@ def run_one_layer(isa, oracle, m, n, S, mode, blocks, seed=7, burst=8, latency=(
     mem.add(x_at, x_in.view(np.uint8).copy(), "activations")
     mem.add(o_at, out, "output")
     wave_model.Wave.vm_latency, wave_model.Wave.lgkm_latency = latency
-    kernel = wave_model.Kernel(isa, "_ZN4rptc17matvec_one_kernelILi%dELi%dELi%dELi%dEE" % (S, mode, 3 if per_wave <= 3 else 4, 1 if silu else 0))
+    kernel = wave_model.Kernel(isa, "_ZN4rptc17matvec_one_kernelILi%dELi%dELi%dELi%dEE" % (S, mode, 3 if per_wave <= 3 else 4 if per_wave <= 4 else 6, 1 if silu else 0))
     blocks = sorted({b for b in blocks if b < grid})
     kernel.launch(mem, (grid,), 1024, [("ptr", c_at), ("ptr", cb_at), ("ptr", x_at), ("i32", m), ("i32", n), ("i32", rpb), ("i32", rw_tail),
                                        ("i32", items_tail), ("u32", magic), ("u32", tail_magic), ("ptr", o_at), ("ptr", 0), ("ptr", 0),
@@ -1200,7 +1200,8 @@ def run_one_layer(isa, oracle, m, n, S, mode, blocks, seed=7, burst=8, latency=(
 
 
 @pytest.mark.parametrize("m,n,S,mode", [(33, 4096 + 768, 8, 0), (33, 4096 + 768, 6, 1), (300, 64, 6, 0), (7, 704, 8, 1), (4096, 11008, 8, 0),
-                                        (11008, 4096, 8, 1), (8192, 8192, 8, 0), (64, 16384, 6, 1), (1000, 2048 + 64 * 31, 8, 1)])
+                                        (11008, 4096, 8, 1), (8192, 8192, 8, 0), (64, 16384, 6, 1), (1000, 2048 + 64 * 31, 8, 1),
+                                        (22016, 4096, 8, 0), (22016, 4096, 6, 1), (12288, 4096, 8, 1), (40000, 2048 + 192, 8, 1)])
 def test_one_layer_kernel_matches_the_oracle(steady_isa, oracle, m, n, S, mode):
     rpb = 2 * ((m + 2 * CUS - 1) // (2 * CUS))
     run_one_layer(steady_isa, oracle, m, n, S, mode, blocks=[0, 1, (m - 1) // rpb])
@@ -1217,7 +1218,7 @@ def test_one_layer_kernel_with_the_silu_gate_in_front(steady_isa, oracle, m, n, 
     run_one_layer(steady_isa, oracle, m, n, S, mode, blocks=[0, (m - 1) // rpb], silu=True)
 
 
-@pytest.mark.parametrize("m,n,S,mode", [(4096, 11008, 8, 0), (33, 4096 + 768, 6, 1)])
+@pytest.mark.parametrize("m,n,S,mode", [(4096, 11008, 8, 0), (33, 4096 + 768, 6, 1), (22016, 4096, 8, 1)])
 def test_one_layer_kernel_has_the_per_launch_kernels_bits(matvec_isa, steady_isa, m, n, S, mode):
     """Both kernels add an element's four sums, a row's partial sums and the lanes of the row's wave in the same order, so
     routing the op through the other kernel changes no output bit."""
@@ -1240,7 +1241,7 @@ def test_one_layer_kernel_has_the_per_launch_kernels_bits(matvec_isa, steady_isa
         wave_model.Wave.vm_latency, wave_model.Wave.lgkm_latency = 400, 60
         head = [("ptr", c_at), ("ptr", cb_at), ("ptr", x_at), ("i32", m), ("i32", n), ("i32", rpb), ("i32", rw_tail), ("i32", items_tail), ("u32", magic)]
         if one:
-            kernel = wave_model.Kernel(steady_isa, "_ZN4rptc17matvec_one_kernelILi%dELi%dELi%dELi0EE" % (S, mode, 3 if per_wave <= 3 else 4))
+            kernel = wave_model.Kernel(steady_isa, "_ZN4rptc17matvec_one_kernelILi%dELi%dELi%dELi0EE" % (S, mode, 3 if per_wave <= 3 else 4 if per_wave <= 4 else 6))
             kernel.launch(mem, (grid,), 1024, head + [("u32", 65536 // lt + 1 if lt else 0), ("ptr", o_at), ("ptr", 0), ("ptr", 0), ("ptr", 0), ("f32", 0.0)],
                           lds_bytes=160 * 1024, groups=[(0, 0, 0)], seed=1)
         else:
@@ -1250,7 +1251,8 @@ def test_one_layer_kernel_has_the_per_launch_kernels_bits(matvec_isa, steady_isa
     assert np.array_equal(outs[0], outs[1]) and (outs[0][:2 * min(rpb, m)] != 0xEE).any()
 
 
-@pytest.mark.parametrize("m,n,S,mode,with_delta", [(40, 2048 + 320, 8, 0, True), (12288, 4096, 8, 1, True), (33, 64 * 7, 6, 0, False)])
+@pytest.mark.parametrize("m,n,S,mode,with_delta", [(40, 2048 + 320, 8, 0, True), (12288, 4096, 8, 1, True), (33, 64 * 7, 6, 0, False),
+                                                   (22016, 4096, 8, 1, True)])
 def test_one_layer_kernel_with_the_norm_in_front_has_the_fused_kernels_bits(matvec_isa, steady_isa, m, n, S, mode, with_delta):
     """The XMODE 2 form (residual add + RMS norm in the prologue) against `matvec_fused_kernel` with the same prologue:
     the same output bits and the same residual stream written back."""
@@ -1279,7 +1281,7 @@ def test_one_layer_kernel_with_the_norm_in_front_has_the_fused_kernels_bits(matv
         head = [("ptr", c_at), ("ptr", cb_at), ("ptr", x_at), ("i32", m), ("i32", n), ("i32", rpb), ("i32", rw_tail), ("i32", items_tail), ("u32", magic)]
         dptr = ("ptr", d_at if with_delta else 0)
         if one:
-            kernel = wave_model.Kernel(steady_isa, "_ZN4rptc17matvec_one_kernelILi%dELi%dELi%dELi2EE" % (S, mode, 3 if per_wave <= 3 else 4))
+            kernel = wave_model.Kernel(steady_isa, "_ZN4rptc17matvec_one_kernelILi%dELi%dELi%dELi2EE" % (S, mode, 3 if per_wave <= 3 else 4 if per_wave <= 4 else 6))
             kernel.launch(mem, (grid,), 1024, head + [("u32", 65536 // lt + 1 if lt else 0), ("ptr", o_at), dptr, ("ptr", w_at), ("ptr", r_at), ("f32", 1e-5)],
                           lds_bytes=160 * 1024, groups=[(0, 0, 0)], seed=1)
         else:
