@@ -1291,3 +1291,44 @@ def test_one_layer_kernel_with_the_norm_in_front_has_the_fused_kernels_bits(matv
         results.append((out, res))
     assert np.array_equal(results[0][0], results[1][0]) and np.array_equal(results[0][1], results[1][1])
     assert (results[0][1] != 0xEE).any() and (results[0][0][:2 * min(rpb, m)] != 0xEE).any()
+
+
+# ------------------------------------------------------------------------------------------------
+# bench_aids/probe.hip: the read-only kernels whose times bench.py prints as the memory floor
+
+@pytest.fixture(scope="module")
+def probe_isa(tmp_path_factory):
+    if shutil.which("hipcc") is None:
+        pytest.skip("hipcc not found")
+    out = str(tmp_path_factory.mktemp("isa") / "probe.s")
+    subprocess.run(["hipcc", "-O3", "-std=c++17", "--offload-arch=gfx950", "-I", os.path.join(PKG, "csrc"), "--cuda-device-only", "-S",
+                    os.path.join(os.path.dirname(PKG), "bench_aids", "probe.hip"), "-o", out], check=True, capture_output=True)
+    return out
+
+
+@pytest.mark.parametrize("copies,layers,per_group16,grid", [(3, 5, 2752, 4), (1, 1, 7, 3), (2, 4, 3072, 2)])
+def test_read_only_chain_probe_stays_inside_its_layers(probe_isa, copies, layers, per_group16, grid):
+    """`probe_read_chain_kernel` reads workgroup b's share of every layer and nothing else: the buffers have no slack, so a
+    request one element past a layer or the pointer table fails the model's bounds check; nothing is stored."""
+    rng = np.random.default_rng(copies + layers)
+    mem = wave_model.Memory()
+    ptrs = np.zeros(copies, dtype=np.uint64)
+    for c in range(copies):
+        at = 0x7f4100000000 + (c << 32) + 0x100 * c
+        ptrs[c] = at
+        mem.add(at, rng.integers(0, 256, 16 * per_group16 * grid, dtype=np.uint8), f"layer {c}")
+    p_at = 0x7f2000000000
+    mem.add(p_at, ptrs.view(np.uint8).copy(), "layer pointers")
+    wave_model.Wave.vm_latency, wave_model.Wave.lgkm_latency = 400, 60
+    kernel = wave_model.Kernel(probe_isa, "_ZN12_GLOBAL__N_123probe_read_chain_kernelEPKmiiiPj")
+    kernel.launch(mem, (grid,), 1024, [("ptr", p_at), ("i32", copies), ("i32", layers), ("i32", per_group16), ("ptr", 0)],
+                  lds_bytes=0, groups=[(0, 0, 0), (grid - 1, 0, 0)], seed=2)
+
+
+def test_read_only_probe_stays_inside_its_buffer(probe_isa):
+    total16 = 2 * 3072 + 1000
+    mem = wave_model.Memory()
+    at = 0x7f4100000000
+    mem.add(at, np.arange(16 * total16, dtype=np.uint32).astype(np.uint8), "stream")
+    kernel = wave_model.Kernel(probe_isa, "_ZN12_GLOBAL__N_117probe_read_kernelEPKjPjm")
+    kernel.launch(mem, (3,), 1024, [("ptr", at), ("ptr", 0), ("u64", total16)], lds_bytes=0, groups=[(0, 0, 0), (2, 0, 0)], seed=2)
