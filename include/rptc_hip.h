@@ -372,17 +372,22 @@ int rptc_viterbi_scalar(const float *targets, const float *weights, int64_t weig
  * rptc_lite_dequantize decodes: rho[0] = 0 at the start, per step the cheapest of the 2^R predecessors of every
  * state (first index on ties, as argmin picks), plus sum_v importance[t][v] * (samples[t][v] - alphabet[index_fn(
  * state)][v])^2 in fp32; the cheapest end state is traced back.  symbols[t] is the reference's `quantized[t]`,
- * cost its `expected_loss`.  Built for the parameters the reference's own driver uses (rptc_lite.py:134-139):
- * L = 16, R = 4, V = 2, and any S <= 9; other parameters return RPTC_ELIMIT.
- *   samples     float [rows][steps][2]
- *   importance  NULL (all ones), or float [.][steps][2]: row r reads importance + r * importance_row_stride
+ * cost its `expected_loss`.  Any 1 <= S <= L <= 20, R <= min(L, 8), V <= 4 (RPTC_ELIMIT beyond); the parameters the
+ * reference's own driver uses (rptc_lite.py:134-139: L = 16, R = 4, V = 2, S <= 9) have a kernel of their own that
+ * keeps the path costs in registers, the others a plain one that keeps them in the scratch.
+ *   samples     float [rows][steps][V]
+ *   importance  NULL (all ones), or float [.][steps][V]: row r reads importance + r * importance_row_stride
  *               (0 = one set for all rows)
- *   alphabet    float [2^S][2];  scratch rptc_viterbi_scratch_bytes(rows, steps) bytes of device memory
- *   symbols     uint8 [rows][steps], values 0..15;  end_state int32 [rows];  cost float [rows]
+ *   alphabet    float [2^S][V];  scratch rptc_lite_viterbi_scratch_bytes(L, R, rows, steps) bytes of device memory
+ *   symbols     uint8 [rows][steps], values below 2^R;  end_state int32 [rows];  cost float [rows]
  */
 int rptc_lite_viterbi(const float *samples, const float *importance, int64_t importance_row_stride,
                       const float *alphabet, int L, int S, int R, int V, void *scratch, uint8_t *symbols,
                       int32_t *end_state, float *cost, int64_t rows, int64_t steps, void *stream, float *ms);
+
+/* Bytes of scratch rptc_lite_viterbi needs (back pointers of every step, and the path costs where they are not held
+ * in registers); 0 for parameters it does not take.  No counterpart in the reference, which lets jax allocate. */
+int64_t rptc_lite_viterbi_scratch_bytes(int L, int R, int64_t rows, int64_t steps);
 
 #ifdef __cplusplus
 }

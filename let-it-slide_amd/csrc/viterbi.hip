@@ -506,6 +506,129 @@ __global__ __launch_bounds__(64) void viterbi_scalar_trace_kernel(const uint32_t
     }
 }
 
+// The search of rptc_lite.py:19-60 for any other (L, S, R, V) the reference's function takes, within L <= 20, R <= 8,
+// V <= 4: one workgroup a row, the 2^L path costs and the 2^(L-R) group minima in the caller's scratch (global memory that
+// stays in the L2: the costs of L = 16 alone are 256 KiB, more than the LDS), two barriers a step.  A step is the
+// reference's: minimum and first arg-minimum over the 2^R predecessors (d << (L - R)) | p of each group p
+// (rptc_lite.py:33-34, the back pointer; a byte here, R bits packed into int32 words there), then
+// cost[s] = minimum[s >> R] + sum_v importance[t][v] * (samples[t][v] - alphabet[index_fn(s)][v])^2 (rptc_lite.py:39-40),
+// every sum fp32 in that order.  Not tuned: the trellis the reference's driver uses has the kernel above.
+struct LiteGeneralScratch {
+    int64_t row_floats;      // floats a row: 2^L costs, then 2^(L-R) minima
+    int64_t back_offset;     // byte offset of the back pointers ([row][step][2^(L-R)] bytes) in the scratch
+};
+
+__host__ __device__ inline LiteGeneralScratch lite_general_scratch(int L, int R, int64_t rows)
+{
+    LiteGeneralScratch g;
+    g.row_floats = ((int64_t)1 << L) + ((int64_t)1 << (L - R));
+    g.back_offset = (rows * g.row_floats * 4 + 255) / 256 * 256;
+    return g;
+}
+
+template <bool WEIGHTED>
+__global__ __launch_bounds__(kVitThreads) void viterbi_lite_general_kernel(
+    const float *__restrict__ targets, const float *__restrict__ weights, int64_t weights_row_stride,
+    const float *__restrict__ alphabet, int L, int S, int R, int V, float *work, uint8_t *back,
+    int32_t *__restrict__ end_state, float *__restrict__ cost, int steps)
+{
+    __shared__ float red_v[kVitThreads];
+    __shared__ int red_i[kVitThreads];
+    const int j = threadIdx.x;
+    const int64_t row = blockIdx.x;
+    const int states = 1 << L, groups = 1 << (L - R), fan = 1 << R;
+    float *rho = work + row * ((int64_t)states + groups);
+    float *best = rho + states;
+    uint8_t *back_row = back + row * steps * (int64_t)groups;
+    const float *tg = targets + row * steps * V;
+    const float *wt = WEIGHTED ? weights + row * weights_row_stride : nullptr;
+
+    for (int s = j; s < states; s += kVitThreads) rho[s] = s == 0 ? 0.f : INFINITY;      // rptc_lite.py:43-44
+    __syncthreads();
+    for (int t = 0; t < steps; t++) {
+        for (int p = j; p < groups; p += kVitThreads) {
+            float m = rho[p];
+            int arg = 0;
+            for (int d = 1; d < fan; d++) {
+                const float v = rho[(d << (L - R)) | p];
+                if (v < m) {                            // the first minimum wins (argmin)
+                    m = v;
+                    arg = d;
+                }
+            }
+            best[p] = m;
+            back_row[(int64_t)t * groups + p] = (uint8_t)arg;
+        }
+        __syncthreads();
+        float x[4], c[4];
+        for (int v = 0; v < 4; v++) {
+            x[v] = v < V ? tg[(int64_t)t * V + v] : 0.f;
+            c[v] = (WEIGHTED && v < V) ? wt[(int64_t)t * V + v] : 1.f;
+        }
+        for (int s = j; s < states; s += kVitThreads) {
+            uint32_t h = (uint32_t)s * (2u * (uint32_t)s + 1u);        // index_fn, rptc_lite.py:12-16 (bits below L decide)
+            h ^= h >> (L - S);
+            const float *a = alphabet + (int64_t)(h & ((1u << S) - 1u)) * V;
+            float loss = 0.f;
+            for (int v = 0; v < V; v++) {
+                const float d = x[v] - a[v];
+                float sq = d * d;
+                if (WEIGHTED) sq = c[v] * sq;
+                loss = v == 0 ? sq : loss + sq;
+            }
+            rho[s] = best[s >> R] + loss;
+        }
+        __syncthreads();
+    }
+
+    // cheapest end state, the lowest index among equals (argmin, rptc_lite.py:52)
+    float mv = INFINITY;
+    int mi = 0x7FFFFFFF;
+    for (int s = j; s < states; s += kVitThreads) {
+        const float v = rho[s];
+        if (v < mv || mi == 0x7FFFFFFF) {
+            mv = v;
+            mi = s;
+        }
+    }
+    red_v[j] = mv;
+    red_i[j] = mi;
+    __syncthreads();
+    for (int width = kVitThreads / 2; width > 0; width >>= 1) {
+        if (j < width) {
+            const float ov = red_v[j + width];
+            const int oi = red_i[j + width];
+            if (ov < red_v[j] || (ov == red_v[j] && oi < red_i[j])) {
+                red_v[j] = ov;
+                red_i[j] = oi;
+            }
+        }
+        __syncthreads();
+    }
+    if (j == 0) {
+        end_state[row] = red_i[0];
+        cost[row] = red_v[0];
+    }
+}
+
+// one thread a row walks the general search's back pointers from the end state (rptc_lite.py:47-55)
+__global__ __launch_bounds__(64) void viterbi_lite_general_trace_kernel(const uint8_t *__restrict__ back,
+                                                                        const int32_t *__restrict__ end_state,
+                                                                        uint8_t *__restrict__ symbols, int L, int R, int rows, int steps)
+{
+    const int row = blockIdx.x * 64 + threadIdx.x;
+    if (row >= rows) return;
+    const int64_t groups = (int64_t)1 << (L - R);
+    const uint8_t *back_row = back + (int64_t)row * steps * groups;
+    uint8_t *sym = symbols + (int64_t)row * steps;
+    uint32_t state = (uint32_t)end_state[row];
+    for (int t = steps - 1; t >= 0; t--) {
+        sym[t] = (uint8_t)(state & ((1u << R) - 1u));
+        const uint32_t p = state >> R;
+        state = ((uint32_t)back_row[(int64_t)t * groups + p] << (L - R)) | p;
+    }
+}
+
 // one thread per row walks the back pointers from the end state (rptc.py:60-65)
 template <int STEP>
 __global__ __launch_bounds__(64) void viterbi_trace_kernel(const uint16_t *__restrict__ back,
@@ -665,15 +788,22 @@ extern "C" int rptc_viterbi_pairs(const float *targets, const float *weights, in
 }
 
 
+extern "C" int64_t rptc_lite_viterbi_scratch_bytes(int L, int R, int64_t rows, int64_t steps)
+{
+    if (L < 1 || L > 20 || R < 1 || R > L || R > 8 || rows < 1 || steps < 1) return 0;
+    if (L == 16 && R == 4) return rptc_viterbi_scratch_bytes(rows, steps);
+    return lite_general_scratch(L, R, rows).back_offset + rows * steps * ((int64_t)1 << (L - R));
+}
+
 extern "C" int rptc_lite_viterbi(const float *samples, const float *importance, int64_t importance_row_stride,
                                  const float *alphabet, int L, int S, int R, int V, void *scratch, uint8_t *symbols,
                                  int32_t *end_state, float *cost, int64_t rows, int64_t steps, void *stream, float *ms)
 {
     if (!samples || !alphabet || !scratch || !symbols || !end_state || !cost) return RPTC_ENULL;
     if (L < 1 || S < 1 || S > L || R < 1 || R > L || V < 1) return RPTC_ESHAPE;
-    if (L != 16 || R != 4 || V != 2 || S > 9) return RPTC_ELIMIT;          // the search kernel's trellis
+    if (L > 20 || R > 8 || V > 4) return RPTC_ELIMIT;
     if (rows < 1 || steps < 1 || importance_row_stride < 0) return RPTC_ESHAPE;
-    if (importance && importance_row_stride != 0 && importance_row_stride < 2 * steps) return RPTC_ESHAPE;
+    if (importance && importance_row_stride != 0 && importance_row_stride < V * steps) return RPTC_ESHAPE;
     if (rows >= ((int64_t)1 << 24) || steps >= ((int64_t)1 << 24)) return RPTC_ELIMIT;
     DeviceInfo *dev;
     int rc = device_info(&dev);
@@ -682,14 +812,27 @@ extern "C" int rptc_lite_viterbi(const float *samples, const float *importance, 
     Timer t;
     rc = t.begin(dev, s, ms);
     if (rc) return rc;
-    uint16_t *back = static_cast<uint16_t *>(scratch);
+    if (L == 16 && R == 4 && V == 2 && S <= 9) {        // the trellis of the reference's driver: the register-resident kernel
+        uint16_t *back = static_cast<uint16_t *>(scratch);
+        if (importance)
+            hipLaunchKernelGGL(viterbi_lite_kernel<true>, dim3((unsigned)rows), dim3(kVitThreads), kVitLdsBytes, s, samples, importance,
+                               importance_row_stride, alphabet, S, back, end_state, cost, (int)steps);
+        else
+            hipLaunchKernelGGL(viterbi_lite_kernel<false>, dim3((unsigned)rows), dim3(kVitThreads), kVitLdsBytes, s, samples, importance,
+                               importance_row_stride, alphabet, S, back, end_state, cost, (int)steps);
+        hipLaunchKernelGGL(viterbi_trace_kernel<4>, dim3((unsigned)((rows + 63) / 64)), dim3(64), 0, s, back, end_state, symbols, (int)rows,
+                           (int)steps);
+        return t.end();
+    }
+    float *work = static_cast<float *>(scratch);
+    uint8_t *back = static_cast<uint8_t *>(scratch) + lite_general_scratch(L, R, rows).back_offset;
     if (importance)
-        hipLaunchKernelGGL(viterbi_lite_kernel<true>, dim3((unsigned)rows), dim3(kVitThreads), kVitLdsBytes, s, samples, importance,
-                           importance_row_stride, alphabet, S, back, end_state, cost, (int)steps);
+        hipLaunchKernelGGL(viterbi_lite_general_kernel<true>, dim3((unsigned)rows), dim3(kVitThreads), 0, s, samples, importance,
+                           importance_row_stride, alphabet, L, S, R, V, work, back, end_state, cost, (int)steps);
     else
-        hipLaunchKernelGGL(viterbi_lite_kernel<false>, dim3((unsigned)rows), dim3(kVitThreads), kVitLdsBytes, s, samples, importance,
-                           importance_row_stride, alphabet, S, back, end_state, cost, (int)steps);
-    hipLaunchKernelGGL(viterbi_trace_kernel<4>, dim3((unsigned)((rows + 63) / 64)), dim3(64), 0, s, back, end_state, symbols, (int)rows,
-                       (int)steps);
+        hipLaunchKernelGGL(viterbi_lite_general_kernel<false>, dim3((unsigned)rows), dim3(kVitThreads), 0, s, samples, importance,
+                           importance_row_stride, alphabet, L, S, R, V, work, back, end_state, cost, (int)steps);
+    hipLaunchKernelGGL(viterbi_lite_general_trace_kernel, dim3((unsigned)((rows + 63) / 64)), dim3(64), 0, s, back, end_state, symbols, L, R,
+                       (int)rows, (int)steps);
     return t.end();
 }

@@ -92,6 +92,7 @@ _SIGNATURES = {
     "rptc_viterbi_scalar_scratch_bytes": ([_I64, _I64], _I64),
     "rptc_viterbi_scalar": ([_VP, _VP, _I64, _VP, _INT, _VP, _VP, _VP, _VP, _I64, _I64, _VP, _FP], _INT),
     "rptc_viterbi_pairs": ([_VP, _VP, _I64, _VP, _VP, _VP, _VP, _VP, _I64, _I64, _INT, _VP, _FP], _INT),
+    "rptc_lite_viterbi_scratch_bytes": ([_INT, _INT, _I64, _I64], _I64),
     "rptc_lite_viterbi": ([_VP, _VP, _I64, _VP, _INT, _INT, _INT, _INT, _VP, _VP, _VP, _VP, _I64, _I64, _VP, _FP], _INT),
     "rptc_viterbi_pairs_bits": ([_VP, _VP, _I64, _VP, _VP, _VP, _VP, _VP, _I64, _I64, _INT, _INT, _VP, _FP], _INT),
     "rptc_lite_dequantize": ([_VP, _INT, _INT, _INT, _INT, _VP, _I64, _I64, _VP, _VP, _FP], _INT),
@@ -444,10 +445,10 @@ def lite_quantize(alphabet, L, S, R, importance, samples):
     """``rptc_lite.quantize(alphabet, L, S, R, importance, samples)`` (rptc_lite.py:19-60): the symbol sequence whose
     ``lite_dequantize`` is closest to ``samples`` under the per-value ``importance``, by exact Viterbi search.
 
-    alphabet: float32 [2^S, 2]; samples, importance: float32 [length, 2], or [rows, length, 2] with every row a sequence
-    of its own (importance may be None for all ones, or [length, 2] for one set shared by all rows).  Built for
-    L = 16, R = 4, V = 2, S <= 9 (the parameters of the reference's own driver); other parameters raise.
-    Returns (quantized int32 [length] or [rows, length], expected_loss float32 scalar or [rows])."""
+    alphabet: float32 [2^S, V]; samples, importance: float32 [length, V], or [rows, length, V] with every row a sequence
+    of its own (importance may be None for all ones, or [length, V] for one set shared by all rows).  Takes
+    S <= L <= 20, R <= 8, V <= 4; L = 16, R = 4, V = 2, S <= 9 (the parameters of the reference's own driver) run the
+    fast kernel.  Returns (quantized int32 [length] or [rows, length], expected_loss float32 scalar or [rows])."""
     _check_input(alphabet, "alphabet")
     _check_input(samples, "samples")
     _check(alphabet.dtype == torch.float32 and alphabet.dim() == 2, "alphabet must be float32 [2^S, V]")
@@ -469,7 +470,7 @@ def lite_quantize(alphabet, L, S, R, importance, samples):
     _check(alphabet.device == device, "all tensors must be on the same device")
     lib = library()
     with torch.cuda.device(device):
-        scratch = torch.empty(max(lib.rptc_viterbi_scratch_bytes(rows, steps), 16), dtype=torch.uint8, device=device)
+        scratch = torch.empty(max(lib.rptc_lite_viterbi_scratch_bytes(L, R, rows, steps), 16), dtype=torch.uint8, device=device)
         symbols = torch.empty((rows, steps), dtype=torch.uint8, device=device)
         end_state = torch.empty(rows, dtype=torch.int32, device=device)
         cost = torch.empty(rows, dtype=torch.float32, device=device)

@@ -67,15 +67,44 @@ def test_lite_quantize_of_one_sequence_and_the_reference_length(rk, oracle):
     assert 0.06 < float(cost) / (T * V) < 0.12
 
 
-def test_lite_quantize_rejects_what_the_kernel_is_not_built_for(rk):
+@pytest.mark.parametrize("L,S,R,V,rows,steps,weights", [(16, 10, 4, 2, 2, 9, "own"), (16, 9, 2, 2, 1, 12, "none"), (12, 8, 4, 3, 3, 40, "shared"),
+                                                         (8, 8, 8, 1, 2, 5, "own"), (14, 6, 1, 4, 1, 33, "none"), (20, 9, 4, 2, 1, 3, "own"),
+                                                         (4, 2, 2, 2, 5, 100, "shared")])
+def test_lite_quantize_with_other_parameters_equals_the_oracle(rk, oracle, L, S, R, V, rows, steps, weights):
+    """Parameters other than the reference driver's go through the plain kernel (path costs in the scratch buffer): the
+    same symbols and cost as the CPU restatement, bit for bit, and the decoder's output of the symbols has that price."""
+    g = np.random.default_rng(1000 * L + 10 * R + V)
+    alphabet = g.standard_normal((1 << S, V)).astype(np.float32)
+    samples = g.standard_normal((rows, steps, V)).astype(np.float32)
+    imp = None
+    if weights == "own":
+        imp = (g.random((rows, steps, V)) + 0.25).astype(np.float32)
+    elif weights == "shared":
+        imp = (g.random((steps, V)) + 0.25).astype(np.float32)
+    a = torch.from_numpy(alphabet).cuda()
+    q, cost = rk.lite_quantize(a, L, S, R, None if imp is None else torch.from_numpy(imp).cuda(), torch.from_numpy(samples).cuda())
+    assert q.shape == (rows, steps) and q.dtype == torch.int32 and cost.shape == (rows,)
+    for r in range(rows):
+        w = None if imp is None else (imp if imp.ndim == 2 else imp[r])
+        want_q, want_cost = oracle.lite_quantize(alphabet, L, S, R, w, samples[r])
+        assert np.array_equal(q[r].cpu().numpy(), want_q), (r, L, S, R, V)
+        assert cost[r].cpu().numpy().view(np.uint32) == np.float32(want_cost).view(np.uint32)
+    deq, _ = rk.lite_dequantize(a, L, S, R, q)
+    ww = np.ones_like(samples) if imp is None else np.broadcast_to(imp, samples.shape)
+    price = (ww.astype(np.float64) * (samples.astype(np.float64) - deq.cpu().numpy().reshape(samples.shape)) ** 2).sum(axis=(1, 2))
+    assert np.allclose(price, cost.cpu().numpy(), rtol=1e-4, atol=1e-5)
+
+
+def test_lite_quantize_rejects_what_the_kernels_are_not_built_for(rk):
     a = torch.zeros((512, 2), dtype=torch.float32, device="cuda")
     x = torch.zeros((8, 2), dtype=torch.float32, device="cuda")
     with pytest.raises(RuntimeError, match="status -5"):
-        rk.lite_quantize(a, 20, 9, 4, None, x)                  # L
+        rk.lite_quantize(torch.zeros((2, 2), dtype=torch.float32, device="cuda"), 21, 1, 4, None, x)      # L
     with pytest.raises(RuntimeError, match="status -5"):
-        rk.lite_quantize(a, 16, 9, 2, None, x)                  # R
+        rk.lite_quantize(a, 16, 9, 16, None, x)                 # R
     with pytest.raises(RuntimeError, match="status -5"):
-        rk.lite_quantize(torch.zeros((1024, 2), dtype=torch.float32, device="cuda"), 16, 10, 4, None, x)     # S
+        rk.lite_quantize(torch.zeros((512, 5), dtype=torch.float32, device="cuda"), 16, 9, 4, None,
+                         torch.zeros((8, 5), dtype=torch.float32, device="cuda"))                          # V
     with pytest.raises(RuntimeError):
         rk.lite_quantize(a, 16, 8, 4, None, x)                  # alphabet.size(0) != 1 << S
     with pytest.raises(RuntimeError):

@@ -604,6 +604,54 @@ def test_lite_search_kernel_matches_the_oracle(viterbi_isa, oracle, S, steps, we
     assert int(end_state[0]) == state
 
 
+@pytest.mark.parametrize("L,S,R,V,rows,steps,weighted", [(8, 5, 2, 2, 2, 9, False), (6, 6, 1, 3, 1, 14, True), (12, 9, 4, 2, 1, 4, True),
+                                                         (10, 4, 8, 1, 1, 3, False), (3, 2, 3, 4, 3, 5, True), (13, 7, 2, 2, 1, 2, False)])
+def test_general_lite_search_kernel_matches_the_oracle(viterbi_isa, oracle, L, S, R, V, rows, steps, weighted):
+    """`viterbi_lite_general_kernel` and its trace kernel as `rptc_lite_viterbi` launches them for parameters other than the
+    reference driver's: path costs, group minima and back pointers in a scratch buffer of exactly the size
+    `rptc_lite_viterbi_scratch_bytes` states (anything beyond it fails the model's bounds check); symbols and cost equal
+    the oracle's `lite_quantize` to the bit, every row's importance set is its own.  The waves of the workgroup hand the
+    path costs to each other through global memory across `__syncthreads()` (see `barrier_orders_memory`)."""
+    rng = np.random.default_rng(100 * L + 10 * R + V)
+    alphabet = rng.standard_normal((1 << S, V)).astype(np.float32)
+    samples = rng.standard_normal((rows, steps, V)).astype(np.float32)
+    importance = (rng.random((rows, steps, V)) + 0.25).astype(np.float32) if weighted else None
+    states, groups = 1 << L, 1 << (L - R)
+    back_offset = (rows * (states + groups) * 4 + 255) // 256 * 256
+    scratch = np.full(back_offset + rows * steps * groups, 0xAB, dtype=np.uint8)
+    symbols = np.full(rows * steps, 0xEE, dtype=np.uint8)
+    end_state = np.full(rows, -1, dtype=np.int32)
+    cost = np.full(rows, np.nan, dtype=np.float32)
+    mem = wave_model.Memory()
+    t_at, w_at, a_at, b_at, s_at, e_at, c_at = (0x7f4000000000, 0x7f4100000000, 0x7f4200000000, 0x7f4300000000, 0x7f4400000000,
+                                                0x7f4500000000, 0x7f4600000000)
+    mem.add(t_at, samples.view(np.uint8).reshape(-1).copy(), "samples")
+    if weighted:
+        mem.add(w_at, importance.view(np.uint8).reshape(-1).copy(), "importance")
+    mem.add(a_at, alphabet.view(np.uint8).reshape(-1).copy(), "alphabet")
+    mem.add(b_at, scratch, "scratch")
+    mem.add(s_at, symbols, "symbols")
+    mem.add(e_at, end_state.view(np.uint8), "end state")
+    mem.add(c_at, cost.view(np.uint8), "cost")
+    wave_model.Wave.vm_latency, wave_model.Wave.lgkm_latency = 400, 60
+    search = wave_model.Kernel(viterbi_isa, "_ZN4rptc27viterbi_lite_general_kernelILb%dEE" % (1 if weighted else 0))
+    search.launch(mem, (rows,), 1024, [("ptr", t_at), ("ptr", w_at if weighted else 0), ("i64", V * steps if weighted else 0), ("ptr", a_at),
+                                       ("i32", L), ("i32", S), ("i32", R), ("i32", V), ("ptr", b_at), ("ptr", b_at + back_offset),
+                                       ("ptr", e_at), ("ptr", c_at), ("i32", steps)], lds_bytes=0, seed=L, barrier_orders_memory=True)
+    mem.regions = [r for r in mem.regions if r[2] != "kernarg"]
+    trace = wave_model.Kernel(viterbi_isa, "_ZN4rptc33viterbi_lite_general_trace_kernelE")
+    trace.launch(mem, (1,), 64, [("ptr", b_at + back_offset), ("ptr", e_at), ("ptr", s_at), ("i32", L), ("i32", R), ("i32", rows), ("i32", steps)],
+                 seed=L)
+    for r in range(rows):
+        want_symbols, want_cost = oracle.lite_quantize(alphabet, L, S, R, importance[r] if weighted else None, samples[r])
+        assert np.array_equal(symbols[r * steps:(r + 1) * steps].astype(np.int32), want_symbols), r
+        assert cost.view(np.uint32)[r] == np.float32(want_cost).view(np.uint32), r
+        state = 0
+        for v in want_symbols:
+            state = ((state << R) | int(v)) & (states - 1)
+        assert int(end_state[r]) == state
+
+
 @pytest.fixture(scope="module")
 def steady_mfma_roll_isa(tmp_path_factory):
     return compile_to_assembly(tmp_path_factory, "matvec_steady", extra=("-DST_MFMA", "-DST_ROLL"))

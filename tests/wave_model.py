@@ -67,6 +67,10 @@ E32_ALIASES = {"v_cndmask_b32", "v_add_f32", "v_add_u32", "v_mov_b32", "v_and_b3
                "v_mul_f32", "v_lshlrev_b32", "v_lshrrev_b32"}
 
 
+INT_E64_AS_E32 = {"v_add_u32", "v_sub_u32", "v_subrev_u32", "v_and_b32", "v_or_b32", "v_xor_b32", "v_lshlrev_b32", "v_lshrrev_b32",
+                  "v_ashrrev_i32", "v_min_u32", "v_max_u32", "v_mul_u32_u24", "v_mul_i32_i24"}
+
+
 def _arith(text):
     """`3-1`, `1*128+14+1`, `0*16384+256`, `v[96+8*1+2*3:96+8*1+2*3+1]`: constant expressions the assembler folds
     (hand-written blocks use them for offsets and register numbers that depend on a macro parameter).  Anything else is
@@ -105,6 +109,8 @@ def parse(path):
         op = parts[0]
         if op in E32_ALIASES:                # hand-written blocks name the 32-bit encodings without their suffix
             op += "_e32"
+        if op.endswith("_e64") and op[:-4] in INT_E64_AS_E32:      # the long encoding of an integer op: other operand kinds, same result
+            op = op[:-4] + "_e32"
         rest = parts[1] if len(parts) > 1 else ""
         # split operands from modifiers
         ops, mods = [], {}
@@ -1671,10 +1677,18 @@ class Kernel:
         return bytes(buf)
 
     def launch(self, mem, grid, block, args, lds_bytes=0, seed=1, groups=None, max_steps=50_000_000, garbage=True,
-               kernarg_at=0x7e0000001000, burst=8):
+               kernarg_at=0x7e0000001000, burst=8, barrier_orders_memory=False):
         """Runs the workgroups `groups` (default: the whole grid) one after the other; `args` is a list of (kind, value)
         with kind in ptr, i64, u64, i32, u32, f32; `burst` bounds how many instructions a wave runs before another
-        is picked (a large value lets every wave run until it blocks).  Returns the number of instructions executed."""
+        is picked (a large value lets every wave run until it blocks).  Returns the number of instructions executed.
+
+        `barrier_orders_memory`: the vector memory operations of a workgroup's waves pass through their compute unit's
+        one memory pipeline in the order they were issued, so a load issued behind a barrier sees a store issued in front
+        of it by another wave of the workgroup without any wait for the store; the compiler's workgroup-scope fence
+        (`__syncthreads()`) relies on that and emits no `vmcnt` wait.  The model's memory operations complete late and
+        wave by wave, which is stricter; with this flag every queued operation of the workgroup completes when a barrier
+        opens.  For kernels whose waves hand data to each other through global memory; not for hand-overs between
+        workgroups, which need the wait."""
         grid = tuple(grid) + (1,) * (3 - len(grid))
         ka = self.kernarg(args, grid, block)
         mem.add(kernarg_at, np.frombuffer(ka, dtype=np.uint8).copy(), "kernarg")
@@ -1718,6 +1732,8 @@ class Kernel:
                         break
                     for w in ws:
                         w.at_barrier = False
+                        if barrier_orders_memory:
+                            w.force_vm(0)
                     continue
                 w = rng.choice(live)
                 for _ in range(rng.randint(1, burst)):
