@@ -1624,8 +1624,24 @@ class Kernel:
         k.launch(mem, grid=(256,), block=1024, args=[("ptr", address), ("i32", 3), ...], lds_bytes=98304, groups=[(0, 0, 0)])
     """
 
+    _files = {}          # path -> (mtime, lines, parsed metadata): an assembly file is read and its metadata parsed once
+
+    @classmethod
+    def _file(cls, path):
+        import yaml
+        mtime = os.path.getmtime(path)
+        hit = cls._files.get(path)
+        if hit is None or hit[0] != mtime:
+            text = open(path).read().split("\n")
+            y0 = next(i for i, l in enumerate(text) if l.strip() == ".amdgpu_metadata")
+            y1 = next(i for i, l in enumerate(text) if l.strip() == ".end_amdgpu_metadata")
+            loader = getattr(yaml, "CSafeLoader", yaml.SafeLoader)
+            hit = (mtime, text, yaml.load("\n".join(text[y0 + 1:y1]), Loader=loader))
+            cls._files[path] = hit
+        return hit[1], hit[2]
+
     def __init__(self, path, symbol_prefix):
-        text = open(path).read().split("\n")
+        text, meta = self._file(path)
         start = next(i for i, l in enumerate(text) if l.startswith(symbol_prefix) and re.match(r"^[\w$.]+:", l))
         self.symbol = text[start].split(":")[0]
         end = next(i for i in range(start, len(text)) if text[i].startswith(".Lfunc_end"))
@@ -1647,10 +1663,6 @@ class Kernel:
             k, v = l.split()
             self.desc[k[len(".amdhsa_"):]] = int(v, 0)
         # argument offsets from the metadata
-        import yaml
-        y0 = next(i for i, l in enumerate(text) if l.strip() == ".amdgpu_metadata")
-        y1 = next(i for i, l in enumerate(text) if l.strip() == ".end_amdgpu_metadata")
-        meta = yaml.safe_load("\n".join(text[y0 + 1:y1]))
         entry = next(k for k in meta["amdhsa.kernels"] if k[".name"] == self.symbol)
         self.args = [{k[1:]: str(v) for k, v in a.items()} for a in entry[".args"]]
         self.kernarg_size = self.desc["kernarg_size"]
