@@ -92,3 +92,15 @@ def test_the_handoff_checker_sees_a_plain_store_a_plain_load_and_a_missing_barri
     assert [w for _, _, w in check(good.replace("off sc1", "off"))] == ["a load of a merging region without sc1"]
     assert [w for _, _, w in check(good.replace("\ts_barrier\n", ""))] == ["the arrival is counted without a barrier behind published()"]
     assert [w for _, _, w in check(good.replace("\ts_waitcnt vmcnt(0)\n", ""))] == ["no s_waitcnt vmcnt(0) behind published()"]
+
+
+@pytest.mark.skipif(shutil.which("hipcc") is None, reason="needs hipcc")
+@pytest.mark.parametrize("source,switch", [("matvec.hip", "-DRPTC_MV_ONE"), ("matmul.hip", "-DRPTC_MM_ROWS"), ("matvec_steady.hip", "-DST_TUNED"),
+                                           ("matvec_steady.hip", "-DST_MFMA"), ("matvec_steady.hip", "-DST_ROLL")])
+def test_host_code_behind_the_build_switches_still_compiles(source, switch):
+    """The untimed variants are off in the library's build; their host-side routing must not rot meanwhile (the device code
+    of each is compiled and run by the wave-model tests)."""
+    import subprocess
+    r = subprocess.run(["hipcc", "-std=c++17", "--offload-arch=gfx950", "--cuda-host-only", "-fsyntax-only", "-Wall", "-Wno-unused-function",
+                        switch, os.path.join(PKG, "csrc", source)], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
