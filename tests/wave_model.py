@@ -18,6 +18,7 @@ mistakes visible and attributable:
 Only the instructions that the compiled kernels use are modelled; an unknown one raises `Fault("instruction not
 modelled")`.  Timing is not modelled at all.  `Kernel` reads a kernel's descriptor and argument layout from the same
 assembly file and launches it the way the runtime does (kernarg segment, workgroup ids, lane ids)."""
+import functools
 import os
 import random
 import re
@@ -32,6 +33,25 @@ MASK64 = (1 << 64) - 1
 
 class Fault(Exception):
     pass
+
+
+@functools.lru_cache(maxsize=None)
+def _reg_index(kind, tok):
+    """(first register, count) of `v7`, `s[4:5]`, ...; (None, 0) for anything else"""
+    m = re.match(r"^%s(\d+)$" % kind, tok)
+    if m:
+        return int(m.group(1)), 1
+    m = re.match(r"^%s\[(\d+):(\d+)\]$" % kind, tok)
+    if m:
+        return int(m.group(1)), int(m.group(2)) - int(m.group(1)) + 1
+    return None, 0
+
+
+@functools.lru_cache(maxsize=4096)
+def _lanes_of(exec_mask):
+    out = np.array([(exec_mask >> k) & 1 for k in range(64)], dtype=bool)
+    out.flags.writeable = False
+    return out
 
 
 class Memory:
@@ -346,22 +366,10 @@ class Wave:
         return f"wg {self.wg} wave {self.wid} line {ln}: {t}"
 
     def sreg_index(self, tok):
-        m = re.match(r"^s(\d+)$", tok)
-        if m:
-            return int(m.group(1)), 1
-        m = re.match(r"^s\[(\d+):(\d+)\]$", tok)
-        if m:
-            return int(m.group(1)), int(m.group(2)) - int(m.group(1)) + 1
-        return None, 0
+        return _reg_index("s", tok)
 
     def vreg_index(self, tok):
-        m = re.match(r"^v(\d+)$", tok)
-        if m:
-            return int(m.group(1)), 1
-        m = re.match(r"^v\[(\d+):(\d+)\]$", tok)
-        if m:
-            return int(m.group(1)), int(m.group(2)) - int(m.group(1)) + 1
-        return None, 0
+        return _reg_index("v", tok)
 
     def rs(self, tok, width=1):
         """scalar source -> python int (width 1 or 2 dwords)"""
@@ -467,7 +475,7 @@ class Wave:
         self.v[d + 1][m] = (val >> np.uint64(32)).astype(U32)[m]
 
     def lanes(self):
-        return np.array([(self.exec >> k) & 1 for k in range(64)], dtype=bool)
+        return _lanes_of(self.exec)
 
     def wv(self, tok, val, mask=None):
         i, n = self.vreg_index(tok)
