@@ -99,6 +99,16 @@ def test_c_abi_rejects_bad_arguments_before_touching_a_device():
     assert lib.rptc_viterbi_scalar(16, None, 0, 16, 15, 16, 16, 16, 16, 4, 64, None, None) == -2     # L
     assert lib.rptc_viterbi_scalar(16, None, 0, None, 16, 16, 16, 16, 16, 4, 64, None, None) == -1   # no alphabet
     assert lib.rptc_viterbi_scalar_scratch_bytes(4, 64) == 4 * 64 * 4096
+    # the rptc_lite search: limits of both of its kernels, and the scratch each asks for
+    assert lib.rptc_lite_viterbi(16, None, 0, 16, 16, 9, 4, 2, None, 16, 16, 16, 4, 64, None, None) == -1    # no scratch
+    assert lib.rptc_lite_viterbi(16, None, 0, 16, 16, 17, 4, 2, 16, 16, 16, 16, 4, 64, None, None) == -2     # S > L
+    assert lib.rptc_lite_viterbi(16, None, 0, 16, 21, 9, 4, 2, 16, 16, 16, 16, 4, 64, None, None) == -5      # L
+    assert lib.rptc_lite_viterbi(16, None, 0, 16, 16, 9, 16, 2, 16, 16, 16, 16, 4, 64, None, None) == -5     # R
+    assert lib.rptc_lite_viterbi(16, None, 0, 16, 16, 9, 4, 5, 16, 16, 16, 16, 4, 64, None, None) == -5      # V
+    assert lib.rptc_lite_viterbi(16, 16, 100, 16, 12, 9, 4, 2, 16, 16, 16, 16, 4, 64, None, None) == -2      # importance stride < V * steps
+    assert lib.rptc_lite_viterbi_scratch_bytes(16, 4, 4, 64) == 4 * 64 * 2048
+    assert lib.rptc_lite_viterbi_scratch_bytes(12, 2, 3, 10) == (3 * (4096 + 1024) * 4 + 255) // 256 * 256 + 3 * 10 * 1024
+    assert lib.rptc_lite_viterbi_scratch_bytes(21, 4, 1, 1) == 0 and lib.rptc_lite_viterbi_scratch_bytes(16, 16, 1, 1) == 0
 
 
 def test_carry_mode_and_timing_switches():
