@@ -395,6 +395,17 @@ def test_row_owner_batched_kernel_matches_the_oracle(matmul_isa, oracle, m, n, b
     assert err < 2e-3
 
 
+@pytest.mark.parametrize("seed", range(3))
+def test_row_owner_batched_kernel_on_random_shapes(matmul_isa, oracle, seed):
+    import random
+    rnd = random.Random(300 + seed)
+    for _ in range(3):
+        n = 64 * rnd.choice([1, 2, 3, 4, 5, 31, 32, 33, 35, 36, 47, 64, 65, 66, 96, 127, 128])
+        m = rnd.choice([1, 2, 15, 16, 17, 31, 33, 48, 50, 64, 80])
+        test_row_owner_batched_kernel_matches_the_oracle(matmul_isa, oracle, m, n, rnd.randint(1, 16), rnd.choice([6, 8]), rnd.choice([0, 1]),
+                                                         rnd.choice([1, 2, 3]))
+
+
 @pytest.mark.parametrize("batch,n,block,inverse,misalign", [(2, 512, 256, 0, 0), (1, 1024, 1024, 1, 0), (3, 192, 64, 0, 2), (1, 12, 4, 1, 0),
                                                             (1, 2048 + 512, 512, 0, 0)])
 def test_sign_hadamard_kernel_matches_the_oracle(hadamard_isa, oracle, batch, n, block, inverse, misalign):
@@ -1253,6 +1264,29 @@ def run_one_layer(isa, oracle, m, n, S, mode, blocks, seed=7, burst=8, latency=(
 def test_one_layer_kernel_matches_the_oracle(steady_isa, oracle, m, n, S, mode):
     rpb = 2 * ((m + 2 * CUS - 1) // (2 * CUS))
     run_one_layer(steady_isa, oracle, m, n, S, mode, blocks=[0, 1, (m - 1) // rpb])
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_one_layer_kernel_on_random_shapes(steady_isa, oracle, seed):
+    """Shapes drawn from ragged and full widths and from row counts around the grid's multiples, whatever fits the
+    kernel's LDS layout and six elements a wave; first, last and one other workgroup; S, carry mode, the SiLU form, the
+    interleaving and the memory latency by seed."""
+    import random
+    rnd = random.Random(900 + seed)
+    done = 0
+    while done < 3:
+        n = 64 * rnd.choice([1, 2, 5, 31, 32, 33, 47, 64, 65, 96, 127, 128, 160, 172, 200, 255, 256])
+        m = rnd.choice([1, 2, 3, 17, 100, 511, 512, 513, 1000, 4096, 5000, 11008, 12288, 22016, 30000, 44000])
+        rpb, rw_tail, items_tail, magic, _ = _matvec_geometry(m, n)
+        T, lt = n >> 11, (n & 2047) >> 6
+        per_wave = -(-(T * (rpb // 2) + items_tail) // 16)
+        if not ((T + (1 if lt else 0)) * 4096 <= 32768 and rpb * (n // 64) * 4 <= 65536 and per_wave <= 6):
+            continue
+        grid = (m + rpb - 1) // rpb
+        run_one_layer(steady_isa, oracle, m, n, rnd.choice([6, 8]), rnd.choice([0, 1]), blocks=sorted({0, grid - 1, rnd.randrange(grid)}),
+                      seed=rnd.randrange(1000), burst=rnd.choice([1, 8, 64]), latency=rnd.choice([(400, 60), (3000, 300), (5, 2)]),
+                      silu=rnd.random() < 0.3)
+        done += 1
 
 
 @pytest.mark.parametrize("burst,latency", [(1, (3000, 300)), (64, (5, 2))])
