@@ -727,12 +727,16 @@ def _matvec_geometry(m, n):
     return rpb, rw_tail, items_tail, magic, 65536 + 2 * n + 4 * (n // 64) * rpb
 
 
-@pytest.mark.parametrize("prologue,m,n,mode", [("silu", 40, 2048 + 320, 0), ("rmsnorm", 40, 2048 + 64, 1), ("rmsnorm", 33, 64 * 7, 0)])
+@pytest.mark.parametrize("prologue,m,n,mode", [("silu", 40, 2048 + 320, 0), ("rmsnorm", 40, 2048 + 64, 1), ("rmsnorm", 33, 64 * 7, 0),
+                                               ("rmsnorm", 40, 6144, 1), ("rmsnorm", 2, 11008, 1), ("silu", 2, 8192, 1)])
 def test_fused_prologue_kernels_equal_the_separate_kernels(matvec_isa, glue_isa, prologue, m, n, mode):
     """`matvec_fused_kernel` with the SiLU gate or the residual add + RMS norm in its prologue (`csrc/matvec.hip`) against
     the stand-alone element-wise kernel (`csrc/decode_glue.hip`) followed by the plain mat-vec kernel, all three run in the
-    model: the same output bits (the prologue repeats the stand-alone kernel's roundings; the residual stream the norm
-    form writes back is compared as well), and no access outside the buffers."""
+    model, and no access outside the buffers.  SiLU: the same output bits (the prologue repeats the stand-alone kernel's
+    roundings).  Norm: the residual stream written back has the same bits; the sum of squares is added in another order
+    (eight neighbours a thread and two-term dot products against one element a thread and step), so the scale can differ
+    in its last fp32 bit, a few activations in their last fp16 bit and a few outputs with them (2 x 11008 is such a case; so
+    is 511 x 6144): outputs within fp16 rounding of each other."""
     S = 8
     rng = np.random.default_rng(m + n)
     cb = (rng.standard_normal(2 << S) * 0.1).astype(np.float16)
@@ -788,8 +792,12 @@ def test_fused_prologue_kernels_equal_the_separate_kernels(matvec_isa, glue_isa,
     plain = wave_model.Kernel(matvec_isa, "_ZN4rptc13matvec_kernelILi%dELi%dELi2ELb0EE" % (S, mode))
     plain.launch(mem, (grid,), 1024, [("ptr", c_at), ("ptr", cb_at), ("ptr", h_at), ("i32", m), ("i32", n), ("i32", rpb), ("i32", rw_tail),
                                       ("i32", items_tail), ("u32", magic), ("ptr", o2_at)], lds_bytes=lds_plain, seed=m)
-    assert np.array_equal(out_fused, out_plain)
-    assert np.isfinite(out_fused.view(np.float16).astype(np.float32)).all()
+    got, want = out_fused.view(np.float16).astype(np.float64), out_plain.view(np.float16).astype(np.float64)
+    assert np.isfinite(got).all()
+    if prologue == "silu":
+        assert np.array_equal(out_fused, out_plain)
+    else:
+        assert np.abs(got - want).max() <= 2e-3 * np.abs(want).max()
 
 
 def _rope_reference(x, cos_row, sin_row):
