@@ -735,8 +735,8 @@ def test_fused_prologue_kernels_equal_the_separate_kernels(matvec_isa, glue_isa,
     model, and no access outside the buffers.  SiLU: the same output bits (the prologue repeats the stand-alone kernel's
     roundings).  Norm: the residual stream written back has the same bits; the sum of squares is added in another order
     (eight neighbours a thread and two-term dot products against one element a thread and step), so the scale can differ
-    in its last fp32 bit, a few activations in their last fp16 bit and a few outputs with them (2 x 11008 is such a case; so
-    is 511 x 6144): outputs within fp16 rounding of each other."""
+    in its last fp32 bit, a few activations in their last fp16 bit and a few outputs with them (rarely: 511 x 6144 with these
+    inputs is such a case, the ones here are not): outputs within fp16 rounding of each other."""
     S = 8
     rng = np.random.default_rng(m + n)
     cb = (rng.standard_normal(2 << S) * 0.1).astype(np.float16)

@@ -1123,7 +1123,8 @@ class Wave:
                 hi16 = f32(V(o[2])).astype(np.float16).view(np.uint16).astype(U32)
             self.wv(o[0], lo16 | (hi16 << U32(16)))
         elif op in ("v_fma_mixlo_f16", "v_fma_mixhi_f16"):
-            # as v_fma_mix_f32, the result rounded once to fp16 and written to one half of the destination (the other kept)
+            # as v_fma_mix_f32 (the sum rounded to fp32), that result then rounded to fp16 and written to one half of the
+            # destination (the other kept): the compiler emits it for a half(a * b) with fp32 a and b, which rounds twice
             hi = [int(x) for x in mods.get("op_sel_hi", "[0,0,0]").strip("[]").split(",")]
             lo = [int(x) for x in mods.get("op_sel", "[0,0,0]").strip("[]").split(",")]
             if "neg_" in text or "clamp" in text:
@@ -1145,7 +1146,7 @@ class Wave:
                 val = np.abs(val) if absolute else val
                 src.append(-val if negate else val)
             with np.errstate(all="ignore"):
-                h = (src[0] * src[1] + src[2]).astype(np.float16).view(np.uint16).astype(U32)
+                h = (src[0] * src[1] + src[2]).astype(np.float32).astype(np.float16).view(np.uint16).astype(U32)
             i, _ = self.vreg_index(o[0])
             old_v = self.v[i]
             self.wv(o[0], (old_v & U32(0xFFFF0000)) | h if op == "v_fma_mixlo_f16" else (old_v & U32(0xFFFF)) | (h << U32(16)))
